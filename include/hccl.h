@@ -1,0 +1,156 @@
+/*
+ * C ABI of the MI355X loopback data plane.
+ *
+ * The five collective entry points have the signatures of the reference's public
+ * header (reference include/hccl.h) so that a caller built against that header links
+ * against this library unchanged.  `aclrtStream` carries a hipStream_t; every buffer
+ * is a device pointer in the HBM of the one GPU; count / displacement arrays are host
+ * arrays of uint64_t in elements and are copied during the call.
+ *
+ * A "world" is a rankSize-N loopback communicator: N HcclComm handles in one process
+ * whose send/recv buffers are separate HBM allocations of the same GPU.  One
+ * collective is N calls (one per rank, identical count / type / op); the call that
+ * completes the set launches ONE fused kernel that performs every rank's share of
+ * the work and orders every rank's stream after it.
+ *
+ * Calling conventions (two are supported):
+ *   - one host thread per rank (the reference's examples/02_collectives pattern):
+ *     each call blocks on the host until all N ranks have called, then returns with
+ *     the work enqueued behind the caller's stream;
+ *   - one host thread driving all ranks: bracket the N calls with HcclGroupStart() /
+ *     HcclGroupEnd(); calls inside a group never block.
+ */
+#ifndef HCCL_AMD_HCCL_H_
+#define HCCL_AMD_HCCL_H_
+
+#include "hccl_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Collectives (the drop-in boundary)
+ * ---------------------------------------------------------------------------------------- */
+
+/*
+ * recvBuf[i] = sendBuf_0[i] (+) sendBuf_1[i] (+) ... over all ranks, for i in [0, count),
+ * written to every rank's recvBuf.  Replaces reference include/hccl.h:36-38
+ * (implementation src/ops/all_reduce/all_reduce.cc:23).  In-place (sendBuf == recvBuf)
+ * is allowed.  count == 0 succeeds without touching anything.
+ */
+HcclResult HcclAllReduce(void* sendBuf, void* recvBuf, uint64_t count, HcclDataType dataType, HcclReduceOp op,
+                         HcclComm comm, aclrtStream stream);
+
+/*
+ * Rank k's recvBuf[0, recvCount) = reduction over ranks t of sendBuf_t[k*recvCount + i].
+ * Replaces reference include/hccl.h:69-71 (src/ops/reduce_scatter/reduce_scatter.cc:24).
+ */
+HcclResult HcclReduceScatter(void* sendBuf, void* recvBuf, uint64_t recvCount, HcclDataType dataType,
+                             HcclReduceOp op, HcclComm comm, aclrtStream stream);
+
+/*
+ * Every rank's recvBuf[r*sendCount + i] = sendBuf_r[i].
+ * Replaces reference include/hccl.h:123-124 (src/ops/all_gather/all_gather.cc:23).
+ */
+HcclResult HcclAllGather(void* sendBuf, void* recvBuf, uint64_t sendCount, HcclDataType dataType, HcclComm comm,
+                         aclrtStream stream);
+
+/*
+ * Every rank's recvBuf[recvDispls[r] + i] = sendBuf_r[i], i in [0, recvCounts[r]).
+ * recvCounts / recvDispls: host uint64_t[rankSize], elements.  Intervals may be unordered
+ * and have holes but must not overlap.  Replaces reference include/hccl.h:141-143
+ * (src/ops/all_gather_v/all_gather_v.cc:23).
+ */
+HcclResult HcclAllGatherV(void* sendBuf, uint64_t sendCount, void* recvBuf, const void* recvCounts,
+                          const void* recvDispls, HcclDataType dataType, HcclComm comm, aclrtStream stream);
+
+/*
+ * Rank i's recvBuf[rdispls_i[j] + e] = sendBuf_j[sdispls_j[i] + e], e in [0, sendCounts_j[i]),
+ * with recvCounts_i[j] == sendCounts_j[i].  All four arrays: host uint64_t[rankSize], elements.
+ * Replaces reference include/hccl.h:215-217 (src/ops/all_to_all_v/all_to_all_v.cc:85).
+ */
+HcclResult HcclAlltoAllV(const void* sendBuf, const void* sendCounts, const void* sdispls, HcclDataType sendType,
+                         const void* recvBuf, const void* recvCounts, const void* rdispls, HcclDataType recvType,
+                         HcclComm comm, aclrtStream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Communicator lifecycle.  In the reference these live in the separate HCOMM library and
+ * are only called (examples/02_collectives/01_allreduce/main.cc:76,101,123;
+ * docs/en/user_guide/api_comm_impl.md:169-190; src/ops/all_reduce/all_reduce.cc:121-125).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Creates ndev communicators of one loopback world; comms[r] has rank r.  `devices` may be
+ * NULL; when given, every entry must name the same GPU (peer buffers share one HBM). */
+HcclResult HcclCommInitAll(uint32_t ndev, int32_t* devices, HcclComm* comms);
+
+/* Fills rootInfo with a fresh world identity to hand to HcclCommInitRootInfo. */
+HcclResult HcclGetRootInfo(HcclRootInfo* rootInfo);
+
+/* Joins rank `rank` of the nRanks-rank world named by rootInfo (same process). */
+HcclResult HcclCommInitRootInfo(uint32_t nRanks, const HcclRootInfo* rootInfo, uint32_t rank, HcclComm* comm);
+
+HcclResult HcclCommDestroy(HcclComm comm);
+HcclResult HcclGetRankSize(HcclComm comm, uint32_t* rankSize);
+HcclResult HcclGetRankId(HcclComm comm, uint32_t* rank);
+const char* HcclGetErrorString(HcclResult code);
+
+/* Calls between Start and End on the calling thread are queued without blocking. */
+HcclResult HcclGroupStart(void);
+HcclResult HcclGroupEnd(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Algorithm choice.  The reference picks an algorithm with its selector and the HCCL_ALGO
+ * environment variable (src/common/alg_parse.cc); here it is an explicit per-world knob
+ * because the algorithm fixes the association order of the reduction.
+ * ---------------------------------------------------------------------------------------- */
+typedef enum {
+    HCCL_AMD_OP_ALL_REDUCE = 0,
+    HCCL_AMD_OP_REDUCE_SCATTER = 1,
+    HCCL_AMD_OP_COUNT
+} HcclAmdOpKind;
+
+typedef enum {
+    /* AllReduce: (((x0+x1)+x2)...+x_{N-1}), the mesh one-shot / two-shot / host-reduce order
+     * (reference ins_temp_all_reduce_mesh_1D_one_shot.cc:223-239,
+     * ins_temp_all_reduce_aicpu_reduce_nhr.cc:272-285).
+     * ReduceScatter: rank k starts from its own slice then adds ranks ascending, skipping k
+     * (reference ins_temp_reduce_scatter_mesh_1D.cc:203-237). */
+    HCCL_AMD_ALGO_MESH = 0,
+    /* Alias kept for the reference's naming: "ring" AllReduce on the host-reduce path folds
+     * in rank order like MESH; "ring" ReduceScatter uses the NHR step tree. */
+    HCCL_AMD_ALGO_RING = 1,
+    /* Recursive halving-doubling with pre-fold of non-power-of-two ranks
+     * (reference template_utils.cc:117-307, ins_temp_reduce_scatter_rhd.cc). */
+    HCCL_AMD_ALGO_RHD = 2,
+    /* Non-uniform hierarchical ring step tree (reference ins_temp_reduce_scatter_nhr.cc:458-506). */
+    HCCL_AMD_ALGO_NHR = 3,
+    /* Power-of-two block fold used when results must not depend on arrival order
+     * (reference ins_temp_reduce_scatter_order_preserved_group.cc:306-409). */
+    HCCL_AMD_ALGO_ORDER_PRESERVED = 4,
+    /* Vector-core mesh order: chunk c of a rank's output starts at peer c and wraps upward
+     * (reference aiv_reduce_scatter_mesh_1d.h:23-71). ReduceScatter only. */
+    HCCL_AMD_ALGO_AIV_MESH = 5,
+    HCCL_AMD_ALGO_COUNT
+} HcclAmdAlgo;
+
+/* Sets the algorithm every later call of `op` on comm's world uses.  Also settable before
+ * world creation through HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr". */
+HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo);
+HcclResult HcclAmdGetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo* algo);
+
+/*
+ * Host-only view of the reduction plan: writes the fold program the kernel would run for
+ * segment `segment` of (op, algo, rankSize) into `out` (at most `cap` bytes) and its length
+ * into *len.  Program bytes: 0x00-0x3F = fold rank r into the accumulator of the current
+ * nesting level (the first operand of a level initialises it); 0x80 = open a nested level;
+ * 0x81 = close it and fold its value (as the incoming operand) into the parent level;
+ * 0xC0|n (n in 1..8) = the next n bytes are ranks folded in that order.  No GPU needed.
+ */
+HcclResult HcclAmdGetFoldProgram(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t segment,
+                                 uint8_t* out, uint32_t cap, uint32_t* len, uint32_t* segmentCount);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HCCL_AMD_HCCL_H_ */

@@ -1,0 +1,1467 @@
+/*
+ * CPU oracle for the loopback data plane -- see hccl_oracle.h.  TEST INFRASTRUCTURE ONLY:
+ * nothing under hccl_amd/ may link, load or call this file.
+ *
+ * "wrapper.cc" below is the reference file
+ *   src/ops/op_common/algorithm/template/wrapper/alg_data_trans_wrapper.cc
+ * and "template_utils.cc" is
+ *   src/ops/op_common/algorithm/template/template_utils.cc.
+ *
+ * Parity status per function group:
+ *   pinned   : orc_fp16_to_fp32 / orc_fp32_to_fp16 (exhaustive numpy float16 tables + NaN /
+ *              boundary known answers), orc_aicpu_reduce (closed forms: modular integer
+ *              arithmetic, single IEEE operations, enumerated +-0 / NaN / tie cases), the RHD /
+ *              NHR step geometry (hand tables and invariants of the reference's unit tests),
+ *              every executor's association order (brute force on tiny inputs against the
+ *              order written in the reference's templates and worked examples), copies and
+ *              packs (index-map brute force).
+ *   unpinned : int16 and bf16 pairwise arithmetic and fp16 SUM/MAX/MIN on the device path
+ *              (the reference computes them in libhcomm / DMA hardware that is not in its
+ *              tree and no reference test holds a numeric answer).  Rules used: int16 wraps
+ *              like int8 / int32; bf16 follows the fp16 host pattern; ORC_ACC_FP32 is the
+ *              fp32-accumulated result the kernels are compared against.
+ */
+#include "hccl_oracle.h"
+
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---------------------------------------------------------------------------------------------
+ * dtype table (reference src/ops/op_common/inc/alg_param.h:55-73)
+ * ------------------------------------------------------------------------------------------- */
+size_t orc_dtype_size(int dtype)
+{
+    static const size_t sizes[18] = {1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16, 2, 1, 1, 1, 1};
+    if (dtype < 0 || dtype >= 18) {
+        return 0;
+    }
+    return sizes[dtype];
+}
+
+static uint32_t f2u(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, sizeof(u));
+    return u;
+}
+
+static float u2f(uint32_t u)
+{
+    float f;
+    memcpy(&f, &u, sizeof(f));
+    return f;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * a2: fp16 <-> fp32 (wrapper.cc:1082-1235)
+ * ------------------------------------------------------------------------------------------- */
+
+/* wrapper.cc:1082-1152.  Zero keeps its sign; subnormals are renormalised; Inf / NaN keep the
+ * 10 mantissa bits in the top of the fp32 mantissa. */
+float orc_fp16_to_fp32(uint16_t h)
+{
+    uint32_t sign = ((uint32_t)h >> 15) & 1u;
+    uint32_t exponent = ((uint32_t)h >> 10) & 0x1Fu;
+    uint32_t mantissa = (uint32_t)h & 0x3FFu;
+    if (exponent == 0) {
+        if (mantissa == 0) {
+            return u2f(sign << 31);
+        }
+        int shift = 0;
+        while ((mantissa & 0x400u) == 0) {
+            mantissa <<= 1;
+            shift++;
+        }
+        mantissa &= 0x3FFu;
+        int32_t e32 = 127 - 15 + 1 - shift;
+        if (e32 <= 0) {
+            return u2f(sign << 31);
+        }
+        return u2f((sign << 31) | ((uint32_t)e32 << 23) | (mantissa << 13));
+    }
+    if (exponent == 0x1Fu) {
+        return u2f((sign << 31) | (0xFFu << 23) | (mantissa << 13));
+    }
+    return u2f((sign << 31) | ((exponent + 112u) << 23) | (mantissa << 13));
+}
+
+/* wrapper.cc:1158-1179: fp32 normal that lands in the fp16 subnormal range; round to nearest
+ * even on the shifted-out bits; a carry out of the mantissa becomes the smallest normal. */
+static uint16_t fp32_denorm_to_fp16(uint32_t sign, uint32_t mantissa, int32_t e16)
+{
+    if (e16 < -10) {
+        return (uint16_t)(sign << 15);
+    }
+    mantissa |= 0x800000u;
+    int32_t shift = 14 - e16;
+    uint32_t roundBit = (mantissa >> (shift - 1)) & 1u;
+    uint32_t sticky = (mantissa & ((1u << (shift - 1)) - 1u)) != 0;
+    uint16_t m16 = (uint16_t)(mantissa >> shift);
+    m16 = (uint16_t)(m16 + (roundBit && (sticky || (m16 & 1u))));
+    if (m16 & 0x400u) {
+        return (uint16_t)((sign << 15) | (1u << 10));
+    }
+    return (uint16_t)((sign << 15) | m16);
+}
+
+/* wrapper.cc:1181-1235.  fp32 zero / subnormal -> signed zero; Inf -> Inf; NaN keeps the top
+ * 10 mantissa bits, forced to 1 if they are all zero; overflow saturates to Inf; otherwise
+ * round to nearest even with carry into the exponent. */
+uint16_t orc_fp32_to_fp16(float f)
+{
+    uint32_t bits = f2u(f);
+    uint32_t sign = (bits >> 31) & 1u;
+    uint32_t exponent = (bits >> 23) & 0xFFu;
+    uint32_t mantissa = bits & 0x7FFFFFu;
+    if (exponent == 0) {
+        return (uint16_t)(sign << 15);
+    }
+    if (exponent == 0xFFu) {
+        if (mantissa == 0) {
+            return (uint16_t)((sign << 15) | 0x7C00u);
+        }
+        uint16_t m16 = (uint16_t)(mantissa >> 13);
+        if (m16 == 0) {
+            m16 = 1;
+        }
+        return (uint16_t)((sign << 15) | 0x7C00u | m16);
+    }
+    int32_t e16 = (int32_t)exponent - 127 + 15;
+    if (e16 >= 31) {
+        return (uint16_t)((sign << 15) | 0x7C00u);
+    }
+    if (e16 <= 0) {
+        return fp32_denorm_to_fp16(sign, mantissa, e16);
+    }
+    uint32_t discarded = mantissa & 0x1FFFu;
+    uint16_t m16 = (uint16_t)(mantissa >> 13);
+    uint32_t roundBit = (discarded >> 12) & 1u;
+    uint32_t sticky = (discarded & 0xFFFu) != 0;
+    m16 = (uint16_t)(m16 + (roundBit && (sticky || (m16 & 1u))));
+    if (m16 == 0x400u) {
+        m16 = 0;
+        e16++;
+    }
+    if (e16 >= 31) {
+        return (uint16_t)((sign << 15) | 0x7C00u);
+    }
+    return (uint16_t)((sign << 15) | ((uint32_t)e16 << 10) | m16);
+}
+
+/* bf16: no reference host path (parity unpinned). */
+float orc_bf16_to_fp32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+uint16_t orc_fp32_to_bf16(float f)
+{
+    uint32_t u = f2u(f);
+    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu) != 0) {
+        return (uint16_t)((u >> 16) | 0x0040u);
+    }
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+void orc_fp16_to_fp32_n(const uint16_t* in, float* out, uint64_t n)
+{
+    for (uint64_t i = 0; i < n; ++i) out[i] = orc_fp16_to_fp32(in[i]);
+}
+
+void orc_fp32_to_fp16_n(const float* in, uint16_t* out, uint64_t n)
+{
+    for (uint64_t i = 0; i < n; ++i) out[i] = orc_fp32_to_fp16(in[i]);
+}
+
+void orc_bf16_to_fp32_n(const uint16_t* in, float* out, uint64_t n)
+{
+    for (uint64_t i = 0; i < n; ++i) out[i] = orc_bf16_to_fp32(in[i]);
+}
+
+void orc_fp32_to_bf16_n(const float* in, uint16_t* out, uint64_t n)
+{
+    for (uint64_t i = 0; i < n; ++i) out[i] = orc_fp32_to_bf16(in[i]);
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * a1: AicpuReduceTemplate<T> (wrapper.cc:1319-1358): dst[i] = src[i] (+) dst[i]
+ *   SUM  : src + dst            (integers wrap; written with unsigned arithmetic)
+ *   PROD : int8 via uint8 multiply, int32 via uint32 multiply, otherwise src * dst (wraps)
+ *   MAX  : std::max(src, dst) == (src < dst) ? dst : src   -> ties / unordered return src
+ *   MIN  : std::min(src, dst) == (dst < src) ? dst : src   -> ties / unordered return src
+ * ------------------------------------------------------------------------------------------- */
+#define DEFINE_INT_PAIR(NAME, T, UT)                                                      \
+    static void NAME(T* dst, const T* src, uint64_t n, int op)                            \
+    {                                                                                     \
+        uint64_t i;                                                                       \
+        switch (op) {                                                                     \
+            case ORC_SUM:                                                                 \
+                for (i = 0; i < n; ++i) dst[i] = (T)(UT)((UT)src[i] + (UT)dst[i]);        \
+                break;                                                                    \
+            case ORC_PROD:                                                                \
+                for (i = 0; i < n; ++i) dst[i] = (T)(UT)((UT)src[i] * (UT)dst[i]);        \
+                break;                                                                    \
+            case ORC_MAX:                                                                 \
+                for (i = 0; i < n; ++i) dst[i] = (src[i] < dst[i]) ? dst[i] : src[i];     \
+                break;                                                                    \
+            default:                                                                      \
+                for (i = 0; i < n; ++i) dst[i] = (dst[i] < src[i]) ? dst[i] : src[i];     \
+                break;                                                                    \
+        }                                                                                 \
+    }
+
+#define DEFINE_FP_PAIR(NAME, T)                                                           \
+    static void NAME(T* dst, const T* src, uint64_t n, int op)                            \
+    {                                                                                     \
+        uint64_t i;                                                                       \
+        switch (op) {                                                                     \
+            case ORC_SUM:                                                                 \
+                for (i = 0; i < n; ++i) dst[i] = src[i] + dst[i];                         \
+                break;                                                                    \
+            case ORC_PROD:                                                                \
+                for (i = 0; i < n; ++i) dst[i] = src[i] * dst[i];                         \
+                break;                                                                    \
+            case ORC_MAX:                                                                 \
+                for (i = 0; i < n; ++i) dst[i] = (src[i] < dst[i]) ? dst[i] : src[i];     \
+                break;                                                                    \
+            default:                                                                      \
+                for (i = 0; i < n; ++i) dst[i] = (dst[i] < src[i]) ? dst[i] : src[i];     \
+                break;                                                                    \
+        }                                                                                 \
+    }
+
+DEFINE_INT_PAIR(pair_i8, int8_t, uint8_t)
+DEFINE_INT_PAIR(pair_i16, int16_t, uint16_t)
+DEFINE_INT_PAIR(pair_i32, int32_t, uint32_t)
+DEFINE_INT_PAIR(pair_i64, int64_t, uint64_t)
+DEFINE_INT_PAIR(pair_u64, uint64_t, uint64_t)
+DEFINE_FP_PAIR(pair_f32, float)
+DEFINE_FP_PAIR(pair_f64, double)
+
+static float fp32_op(float s, float d, int op)
+{
+    switch (op) {
+        case ORC_SUM:
+            return s + d;
+        case ORC_PROD:
+            return s * d;
+        case ORC_MAX:
+            return (s < d) ? d : s;
+        default:
+            return (d < s) ? d : s;
+    }
+}
+
+/* AicpuReduceFp16 (wrapper.cc:1237-1257): widen both, fp32 op, narrow the result. */
+static void pair_f16(uint16_t* dst, const uint16_t* src, uint64_t n, int op)
+{
+    for (uint64_t i = 0; i < n; ++i) {
+        dst[i] = orc_fp32_to_fp16(fp32_op(orc_fp16_to_fp32(src[i]), orc_fp16_to_fp32(dst[i]), op));
+    }
+}
+
+/* bf16 by analogy with the fp16 host pattern (parity unpinned). */
+static void pair_bf16(uint16_t* dst, const uint16_t* src, uint64_t n, int op)
+{
+    for (uint64_t i = 0; i < n; ++i) {
+        dst[i] = orc_fp32_to_bf16(fp32_op(orc_bf16_to_fp32(src[i]), orc_bf16_to_fp32(dst[i]), op));
+    }
+}
+
+int orc_pair_reduce(void* dst, const void* src, uint64_t count, int dtype, int op)
+{
+    if (op < ORC_SUM || op > ORC_MIN) {
+        return ORC_E_INTERNAL;
+    }
+    switch (dtype) {
+        case ORC_INT8:
+            pair_i8((int8_t*)dst, (const int8_t*)src, count, op);
+            return ORC_OK;
+        case ORC_INT16:
+            pair_i16((int16_t*)dst, (const int16_t*)src, count, op);
+            return ORC_OK;
+        case ORC_INT32:
+            pair_i32((int32_t*)dst, (const int32_t*)src, count, op);
+            return ORC_OK;
+        case ORC_INT64:
+            pair_i64((int64_t*)dst, (const int64_t*)src, count, op);
+            return ORC_OK;
+        case ORC_UINT64:
+            pair_u64((uint64_t*)dst, (const uint64_t*)src, count, op);
+            return ORC_OK;
+        case ORC_FP16:
+            pair_f16((uint16_t*)dst, (const uint16_t*)src, count, op);
+            return ORC_OK;
+        case ORC_BF16:
+            pair_bf16((uint16_t*)dst, (const uint16_t*)src, count, op);
+            return ORC_OK;
+        case ORC_FP32:
+            pair_f32((float*)dst, (const float*)src, count, op);
+            return ORC_OK;
+        case ORC_FP64:
+            pair_f64((double*)dst, (const double*)src, count, op);
+            return ORC_OK;
+        default:
+            return ORC_E_INTERNAL;
+    }
+}
+
+/* AicpuReduce (wrapper.cc:1259-1316). */
+int orc_aicpu_reduce(void* dst, uint64_t dstBytes, const void* src, uint64_t srcBytes, int dtype, int op)
+{
+    if (dstBytes != srcBytes) {
+        return ORC_E_INTERNAL;
+    }
+    switch (dtype) {
+        case ORC_INT8:
+        case ORC_INT32:
+        case ORC_FP16:
+        case ORC_FP32:
+        case ORC_INT64:
+        case ORC_UINT64:
+        case ORC_FP64:
+            return orc_pair_reduce(dst, src, dstBytes / orc_dtype_size(dtype), dtype, op);
+        default:
+            return ORC_E_INTERNAL;
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Accumulation domain shared by the executors
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+    int dtype, op, accF32;
+    size_t esz, asz;
+} red_t;
+
+/* Admission follows reference op_common.cc:4323-4413 (CheckDataType / CheckReduceOp). */
+static int red_init(red_t* r, int dtype, int op, int accMode)
+{
+    switch (dtype) {
+        case ORC_INT8:
+        case ORC_INT16:
+        case ORC_INT32:
+        case ORC_INT64:
+        case ORC_UINT64:
+        case ORC_FP16:
+        case ORC_FP32:
+        case ORC_FP64:
+        case ORC_BF16:
+            break;
+        default:
+            return ORC_E_NOT_SUPPORT;
+    }
+    if (op < ORC_SUM || op > ORC_MIN) {
+        return ORC_E_PARA;
+    }
+    if (op == ORC_PROD && (dtype == ORC_INT16 || dtype == ORC_BF16)) {
+        return ORC_E_NOT_SUPPORT;
+    }
+    r->dtype = dtype;
+    r->op = op;
+    r->esz = orc_dtype_size(dtype);
+    r->accF32 = (accMode == ORC_ACC_FP32) && (dtype == ORC_FP16 || dtype == ORC_BF16) && op == ORC_SUM;
+    r->asz = r->accF32 ? sizeof(float) : r->esz;
+    return ORC_OK;
+}
+
+static void red_widen(const red_t* r, const void* in, void* acc, uint64_t n)
+{
+    if (!r->accF32) {
+        memcpy(acc, in, n * r->esz);
+        return;
+    }
+    const uint16_t* h = (const uint16_t*)in;
+    float* a = (float*)acc;
+    if (r->dtype == ORC_FP16) {
+        for (uint64_t i = 0; i < n; ++i) a[i] = orc_fp16_to_fp32(h[i]);
+    } else {
+        for (uint64_t i = 0; i < n; ++i) a[i] = orc_bf16_to_fp32(h[i]);
+    }
+}
+
+static void red_narrow(const red_t* r, const void* acc, void* out, uint64_t n)
+{
+    if (!r->accF32) {
+        memcpy(out, acc, n * r->esz);
+        return;
+    }
+    const float* a = (const float*)acc;
+    uint16_t* h = (uint16_t*)out;
+    if (r->dtype == ORC_FP16) {
+        for (uint64_t i = 0; i < n; ++i) h[i] = orc_fp32_to_fp16(a[i]);
+    } else {
+        for (uint64_t i = 0; i < n; ++i) h[i] = orc_fp32_to_bf16(a[i]);
+    }
+}
+
+/* dst = src (+) dst, both in the accumulation domain. */
+static void red_pair(const red_t* r, void* dst, const void* src, uint64_t n)
+{
+    if (r->accF32) {
+        pair_f32((float*)dst, (const float*)src, n, ORC_SUM);
+    } else {
+        orc_pair_reduce(dst, src, n, r->dtype, r->op);
+    }
+}
+
+/* dst (accumulation domain) = widen(src in storage) (+) dst, without a staging copy. */
+static void red_pair_from_storage(const red_t* r, void* dst, const void* src, uint64_t n, void* tmp)
+{
+    if (r->accF32) {
+        red_widen(r, src, tmp, n);
+        red_pair(r, dst, tmp, n);
+    } else {
+        orc_pair_reduce(dst, src, n, r->dtype, r->op);
+    }
+}
+
+static const uint8_t* cbytes(const void* p) { return (const uint8_t*)p; }
+static uint8_t* bytes(void* p) { return (uint8_t*)p; }
+
+/* ---------------------------------------------------------------------------------------------
+ * a16: slice geometry
+ * ------------------------------------------------------------------------------------------- */
+uint64_t orc_round_up(uint64_t dividend, uint64_t divisor)
+{
+    if (divisor == 0) {
+        return dividend;
+    }
+    return dividend / divisor + ((dividend % divisor != 0) ? 1 : 0);
+}
+
+uint32_t orc_nhr_step_num(uint32_t rankSize)
+{
+    uint32_t n = 0;
+    for (uint32_t t = rankSize - 1; t != 0; t >>= 1) n++;
+    return n;
+}
+
+uint32_t orc_rhd_step_num(uint32_t rankSize)
+{
+    uint32_t n = 0;
+    for (uint32_t t = rankSize; t > 1; t >>= 1) n++;
+    return n;
+}
+
+/* r = p - 2^floor(log2 p) (template_utils.cc:53-63). */
+static uint32_t rhd_pair_num(uint32_t p)
+{
+    if (p == 0) {
+        return 0;
+    }
+    uint32_t hp = 1;
+    while (hp <= p / 2) hp *= 2;
+    return p - hp;
+}
+
+static int rhd_rep_is_low(uint32_t r, uint32_t root)
+{
+    return (root == ORC_INVALID_RANK || root >= 2 * r) ? 1 : (root < r);
+}
+
+static uint32_t rhd_unit_start_impl(uint32_t r, uint32_t j)
+{
+    if (j < r) {
+        return 2 * j;
+    }
+    if (j < 2 * r) {
+        return 2 * (j - r) + 1;
+    }
+    return j;
+}
+
+uint32_t orc_rhd_unit_start_of_rank(uint32_t p, uint32_t j)
+{
+    if (p == 0 || j >= p) {
+        return ORC_INVALID_RANK;
+    }
+    return rhd_unit_start_impl(rhd_pair_num(p), j);
+}
+
+uint32_t orc_rhd_alg_rank_of_virtual(uint32_t p, uint32_t root, uint32_t v)
+{
+    if (p == 0) {
+        return ORC_INVALID_RANK;
+    }
+    uint32_t r = rhd_pair_num(p);
+    uint32_t P = p - r;
+    if (v >= P) {
+        return ORC_INVALID_RANK;
+    }
+    if (v >= r) {
+        return v + r;
+    }
+    return rhd_rep_is_low(r, root) ? v : v + r;
+}
+
+uint32_t orc_rhd_owner_of_unit(uint32_t p, uint32_t unit)
+{
+    uint32_t r = rhd_pair_num(p);
+    if (unit >= 2 * r) {
+        return unit;
+    }
+    return unit / 2 + ((unit % 2 == 0) ? 0 : r);
+}
+
+int orc_rhd_part1(uint32_t p, uint32_t j, uint32_t root, orc_rhd_part1_t* info)
+{
+    if (p == 0 || j >= p) {
+        return ORC_E_PARA;
+    }
+    if (root != ORC_INVALID_RANK && root >= p) {
+        return ORC_E_PARA;
+    }
+    memset(info, 0, sizeof(*info));
+    uint32_t r = rhd_pair_num(p);
+    info->r = r;
+    info->isPowerOfTwo = (r == 0);
+    info->effectiveRankSize = p - r;
+    info->virtualRank = (j < 2 * r) ? (j % r) : (j - r);
+    info->inPart1 = (j < 2 * r);
+    if (info->inPart1) {
+        uint32_t t = j % r;
+        int low = j < r;
+        info->pairedAlgRank = low ? (t + r) : t;
+        int repLow = rhd_rep_is_low(r, root);
+        info->isRepresentative = repLow ? low : !low;
+        if (info->isRepresentative) {
+            info->unitStart = 2 * t;
+            info->unitCount = 2;
+        } else {
+            info->unitStart = orc_rhd_unit_start_of_rank(p, j);
+            info->unitCount = 1;
+        }
+    } else {
+        info->pairedAlgRank = ORC_INVALID_RANK;
+        info->isRepresentative = 0;
+        info->unitStart = j;
+        info->unitCount = 1;
+    }
+    return ORC_OK;
+}
+
+static uint32_t unit_start_of_virtual(uint32_t r, uint32_t a) { return (a < r) ? 2 * a : a + r; }
+static uint32_t unit_end_of_virtual(uint32_t r, uint32_t b) { return (b <= r) ? 2 * b : b + r; }
+
+static int rhd_info_ok(const orc_rhd_part1_t* info)
+{
+    uint32_t P = info->effectiveRankSize;
+    if (P == 0 || info->virtualRank >= P) {
+        return 0;
+    }
+    if ((P & (P - 1)) != 0 || info->r >= P) {
+        return 0;
+    }
+    return 1;
+}
+
+int orc_rhd_rs_steps(const orc_rhd_part1_t* info, orc_rhd_step_t* steps, uint32_t* nSteps)
+{
+    *nSteps = 0;
+    if (!rhd_info_ok(info)) {
+        return ORC_E_PARA;
+    }
+    uint32_t v = info->virtualRank, P = info->effectiveRankSize, r = info->r;
+    uint32_t n = orc_rhd_step_num(P);
+    for (uint32_t k = 0; k < n; ++k) {
+        uint32_t dist = P >> (k + 1);
+        uint32_t peer = v ^ dist;
+        uint32_t peerBase = peer & ~(dist - 1);
+        uint32_t myBase = v & ~(dist - 1);
+        orc_rhd_step_t* s = &steps[k];
+        s->step = k;
+        s->peer = peer;
+        s->nSlices = dist;
+        s->txSegStart = unit_start_of_virtual(r, peerBase);
+        s->txSegEnd = unit_end_of_virtual(r, peerBase + dist);
+        s->rxSegStart = unit_start_of_virtual(r, myBase);
+        s->rxSegEnd = unit_end_of_virtual(r, myBase + dist);
+    }
+    *nSteps = n;
+    return ORC_OK;
+}
+
+int orc_rhd_ag_steps(const orc_rhd_part1_t* info, orc_rhd_step_t* steps, uint32_t* nSteps)
+{
+    *nSteps = 0;
+    if (!rhd_info_ok(info)) {
+        return ORC_E_PARA;
+    }
+    uint32_t v = info->virtualRank, P = info->effectiveRankSize, r = info->r;
+    uint32_t n = orc_rhd_step_num(P);
+    for (uint32_t k = 0; k < n; ++k) {
+        uint32_t dist = 1u << k;
+        uint32_t held = v & ~(dist - 1);
+        uint32_t rx = held ^ dist;
+        orc_rhd_step_t* s = &steps[k];
+        s->step = k;
+        s->peer = v ^ dist;
+        s->nSlices = dist;
+        s->txSegStart = unit_start_of_virtual(r, held);
+        s->txSegEnd = unit_end_of_virtual(r, held + dist);
+        s->rxSegStart = unit_start_of_virtual(r, rx);
+        s->rxSegEnd = unit_end_of_virtual(r, rx + dist);
+    }
+    *nSteps = n;
+    return ORC_OK;
+}
+
+int orc_rhd_prepost(const orc_rhd_part1_t* info, orc_rhd_step_t* pre, orc_rhd_step_t* post, int preFull,
+                    int postFull)
+{
+    memset(pre, 0, sizeof(*pre));
+    memset(post, 0, sizeof(*post));
+    uint32_t P = info->effectiveRankSize;
+    if ((P & (P - 1)) != 0 || info->r >= P) {
+        return ORC_E_PARA;
+    }
+    if (!info->inPart1) {
+        pre->peer = ORC_INVALID_RANK;
+        post->peer = ORC_INVALID_RANK;
+        return ORC_OK;
+    }
+    uint32_t p = P + info->r;
+    if (info->pairedAlgRank >= p || (!info->isRepresentative && info->unitStart >= p)) {
+        return ORC_E_PARA;
+    }
+    uint32_t segStart = info->isRepresentative ? orc_rhd_unit_start_of_rank(p, info->pairedAlgRank) : info->unitStart;
+    uint32_t segEnd = segStart + 1;
+    uint32_t preS = preFull ? 0 : segStart, preE = preFull ? p : segEnd, preN = preFull ? p : 1;
+    uint32_t postS = postFull ? 0 : segStart, postE = postFull ? p : segEnd, postN = postFull ? p : 1;
+    pre->peer = info->pairedAlgRank;
+    post->peer = info->pairedAlgRank;
+    pre->nSlices = preN;
+    post->nSlices = postN;
+    if (info->isRepresentative) {
+        pre->rxSegStart = preS;
+        pre->rxSegEnd = preE;
+        post->txSegStart = postS;
+        post->txSegEnd = postE;
+    } else {
+        pre->txSegStart = preS;
+        pre->txSegEnd = preE;
+        post->rxSegStart = postS;
+        post->rxSegEnd = postE;
+    }
+    return ORC_OK;
+}
+
+void orc_rhd_seg_bytes_uniform(uint32_t us, uint32_t ue, uint64_t sliceSize, uint64_t tailSize, uint32_t tailUnit,
+                               uint64_t* offset, uint64_t* len)
+{
+    *offset = 0;
+    *len = 0;
+    if (us >= ue) {
+        return;
+    }
+    *offset = (uint64_t)us * sliceSize;
+    uint64_t tailLen = (tailSize == 0) ? sliceSize : tailSize;
+    int includesTail = ue > tailUnit;
+    uint32_t normal = ue - us - (includesTail ? 1 : 0);
+    *len = (uint64_t)normal * sliceSize + (includesTail ? tailLen : 0);
+}
+
+uint64_t orc_rhd_select_loop_count(uint64_t remaining, uint64_t maxCountPerLoop, uint64_t rankAlign)
+{
+    uint64_t count = remaining < maxCountPerLoop ? remaining : maxCountPerLoop;
+    return count >= rankAlign ? count / rankAlign * rankAlign : count;
+}
+
+int orc_nhr_step_info(uint32_t n, uint32_t me, uint32_t step, uint32_t* toRank, uint32_t* fromRank,
+                      uint32_t* nSlices, uint32_t* tx, uint32_t* rx)
+{
+    if (n == 0 || me >= n || step >= orc_nhr_step_num(n)) {
+        return ORC_E_PARA;
+    }
+    uint32_t delta = 1u << step;
+    uint32_t sendTo = (me + n - delta % n) % n;
+    uint32_t recvFrom = (me + delta) % n;
+    uint32_t cnt = (n - 1 + (1u << step)) / (1u << (step + 1));
+    uint32_t dIdx = (1u << (step + 1)) % n;
+    uint32_t t = sendTo, x = me;
+    for (uint32_t i = 0; i < cnt; ++i) {
+        tx[i] = t;
+        rx[i] = x;
+        t = (t + n - dIdx) % n;
+        x = (x + n - dIdx) % n;
+    }
+    *toRank = sendTo;
+    *fromRank = recvFrom;
+    *nSlices = cnt;
+    return ORC_OK;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * a6 / a7: AllReduce in rank order.  Scratch slot r holds rank r's input; slot 0 accumulates
+ * slots 1..N-1 ascending; slot 0 is copied to every output (one_shot.cc:223-239,
+ * aicpu_reduce_nhr.cc:272-285).
+ * ------------------------------------------------------------------------------------------- */
+static int all_reduce_mesh_range(uint32_t n, const void* const* in, void* const* out, uint64_t first, uint64_t count,
+                                 const red_t* r)
+{
+    if (count == 0) {
+        return ORC_OK;
+    }
+    void* acc = malloc(count * r->asz);
+    void* tmp = r->accF32 ? malloc(count * r->asz) : NULL;
+    if (!acc || (r->accF32 && !tmp)) {
+        free(acc);
+        free(tmp);
+        return ORC_E_INTERNAL;
+    }
+    red_widen(r, cbytes(in[0]) + first * r->esz, acc, count);
+    for (uint32_t k = 1; k < n; ++k) {
+        red_pair_from_storage(r, acc, cbytes(in[k]) + first * r->esz, count, tmp);
+    }
+    for (uint32_t k = 0; k < n; ++k) {
+        red_narrow(r, acc, bytes(out[k]) + first * r->esz, count);
+    }
+    free(acc);
+    free(tmp);
+    return ORC_OK;
+}
+
+int orc_all_reduce_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                        int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    return all_reduce_mesh_range(n, in, out, 0, count, &r);
+}
+
+/* a8: slice k = [k*ceil(count/n), min(count, (k+1)*ceil(count/n))) is reduced by rank k in rank
+ * order, then gathered (two_shot.cc:178-210, 326-360). */
+int orc_all_reduce_two_shot(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                            int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    uint64_t sliceCount = orc_round_up(count, n);
+    uint64_t off = 0;
+    for (uint32_t k = 0; k < n; ++k) {
+        uint64_t cur = (count - off > sliceCount) ? sliceCount : count - off;
+        rc = all_reduce_mesh_range(n, in, out, off, cur, &r);
+        if (rc != ORC_OK) {
+            return rc;
+        }
+        off += cur;
+    }
+    return ORC_OK;
+}
+
+/* a9: rank k: out = in_k[k]; for t = 0..N-1, t != k: out = in_t[k] (+) out. */
+static int reduce_scatter_mesh_range(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount,
+                                     uint64_t first, uint64_t count, const red_t* r)
+{
+    if (count == 0) {
+        return ORC_OK;
+    }
+    void* acc = malloc(count * r->asz);
+    void* tmp = r->accF32 ? malloc(count * r->asz) : NULL;
+    if (!acc || (r->accF32 && !tmp)) {
+        free(acc);
+        free(tmp);
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t k = 0; k < n; ++k) {
+        uint64_t base = ((uint64_t)k * recvCount + first) * r->esz;
+        red_widen(r, cbytes(in[k]) + base, acc, count);
+        for (uint32_t t = 0; t < n; ++t) {
+            if (t != k) {
+                red_pair_from_storage(r, acc, cbytes(in[t]) + base, count, tmp);
+            }
+        }
+        red_narrow(r, acc, bytes(out[k]) + first * r->esz, count);
+    }
+    free(acc);
+    free(tmp);
+    return ORC_OK;
+}
+
+int orc_reduce_scatter_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                            int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    return reduce_scatter_mesh_range(n, in, out, recvCount, 0, recvCount, &r);
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Per-rank scratch used by the step-driven executors: scratch[rank][slot][elem].
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+    uint32_t n;
+    uint64_t slotElems;
+    size_t asz;
+    uint8_t* mem;
+} scratch_t;
+
+static int scratch_alloc(scratch_t* s, uint32_t n, uint64_t slotElems, size_t asz)
+{
+    s->n = n;
+    s->slotElems = slotElems;
+    s->asz = asz;
+    uint64_t total = (uint64_t)n * n * slotElems * asz;
+    s->mem = (uint8_t*)malloc(total ? total : 1);
+    return s->mem ? ORC_OK : ORC_E_INTERNAL;
+}
+
+static uint8_t* scratch_at(const scratch_t* s, uint32_t rank, uint32_t slot)
+{
+    return s->mem + ((uint64_t)rank * s->n + slot) * s->slotElems * s->asz;
+}
+
+/* a10: NHR reduce-scatter.  Slot i of a rank's scratch starts as its input slice i; in step s
+ * rank m write-reduces its slots txSliceIdxs into the same slots of rank (m - 2^s) mod N
+ * (receiver's value is dst, incoming is src; reduce_scatter_nhr.cc:316-447).  After the last
+ * step rank m's slot m is its output (:268-312). */
+static int nhr_reduce_scatter_scratch(const red_t* r, scratch_t* sc)
+{
+    uint32_t n = sc->n;
+    uint32_t steps = orc_nhr_step_num(n);
+    uint32_t* tx = (uint32_t*)malloc(sizeof(uint32_t) * n * 2);
+    uint32_t* rx = tx + n;
+    uint8_t* dirty = (uint8_t*)malloc((size_t)n * n);
+    if (!tx || !dirty) {
+        free(tx);
+        free(dirty);
+        return ORC_E_INTERNAL;
+    }
+    int rc = ORC_OK;
+    for (uint32_t s = 0; s < steps && rc == ORC_OK; ++s) {
+        /* A slot written in this step must not also be read in it (sends and receives of one step run
+         * concurrently in the reference). */
+        memset(dirty, 0, (size_t)n * n);
+        for (uint32_t m = 0; m < n; ++m) {
+            uint32_t to, from, cnt;
+            orc_nhr_step_info(n, m, s, &to, &from, &cnt, tx, rx);
+            for (uint32_t i = 0; i < cnt; ++i) dirty[to * n + tx[i]] = 1;
+        }
+        for (uint32_t m = 0; m < n && rc == ORC_OK; ++m) {
+            uint32_t to, from, cnt;
+            orc_nhr_step_info(n, m, s, &to, &from, &cnt, tx, rx);
+            for (uint32_t i = 0; i < cnt; ++i) {
+                if (dirty[m * n + tx[i]]) {
+                    rc = ORC_E_INTERNAL;
+                    break;
+                }
+                red_pair(r, scratch_at(sc, to, tx[i]), scratch_at(sc, m, tx[i]), sc->slotElems);
+            }
+        }
+    }
+    free(tx);
+    free(dirty);
+    return rc;
+}
+
+int orc_reduce_scatter_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                           int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (recvCount == 0) {
+        return ORC_OK;
+    }
+    scratch_t sc;
+    if (scratch_alloc(&sc, n, recvCount, r.asz) != ORC_OK) {
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t m = 0; m < n; ++m) {
+        for (uint32_t i = 0; i < n; ++i) {
+            red_widen(&r, cbytes(in[m]) + (uint64_t)i * recvCount * r.esz, scratch_at(&sc, m, i), recvCount);
+        }
+    }
+    rc = nhr_reduce_scatter_scratch(&r, &sc);
+    if (rc == ORC_OK) {
+        for (uint32_t m = 0; m < n; ++m) red_narrow(&r, scratch_at(&sc, m, m), out[m], recvCount);
+    }
+    free(sc.mem);
+    return rc;
+}
+
+int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                       int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (count == 0) {
+        return ORC_OK;
+    }
+    uint64_t slice = orc_round_up(count, n);
+    scratch_t sc;
+    if (scratch_alloc(&sc, n, slice, r.asz) != ORC_OK) {
+        return ORC_E_INTERNAL;
+    }
+    memset(sc.mem, 0, (uint64_t)n * n * slice * r.asz);
+    for (uint32_t m = 0; m < n; ++m) {
+        for (uint32_t i = 0; i < n; ++i) {
+            uint64_t off = (uint64_t)i * slice;
+            uint64_t cur = off >= count ? 0 : (count - off > slice ? slice : count - off);
+            red_widen(&r, cbytes(in[m]) + off * r.esz, scratch_at(&sc, m, i), cur);
+        }
+    }
+    rc = nhr_reduce_scatter_scratch(&r, &sc);
+    if (rc == ORC_OK) {
+        for (uint32_t i = 0; i < n; ++i) {
+            uint64_t off = (uint64_t)i * slice;
+            uint64_t cur = off >= count ? 0 : (count - off > slice ? slice : count - off);
+            for (uint32_t m = 0; m < n; ++m) red_narrow(&r, scratch_at(&sc, i, i), bytes(out[m]) + off * r.esz, cur);
+        }
+    }
+    free(sc.mem);
+    return rc;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * a11: RHD.  One "frame" = p units of `unit` elements per rank.
+ *   mirror : input slice i of every rank goes to slot sigma(i)            (rhd.cc:365-410)
+ *   PRE    : merged rank t+r write-reduces all p slots into representative t (:412-476)
+ *   MAIN   : step k, dist = P>>(k+1): virtual rank v write-reduces its tx segment into the
+ *            same slots of v^dist; receiver's value is dst                (:478-564)
+ *   POST   : representative writes the merged rank's slot back             (:566-629)
+ * ------------------------------------------------------------------------------------------- */
+static int rhd_rs_frame(const red_t* r, scratch_t* sc, int skipPost)
+{
+    uint32_t p = sc->n;
+    orc_rhd_part1_t info;
+    orc_rhd_step_t steps[32];
+    uint32_t nSteps;
+    /* PRE (FULL segment [0,p)) */
+    for (uint32_t j = 0; j < p; ++j) {
+        orc_rhd_part1(p, j, ORC_INVALID_RANK, &info);
+        if (info.inPart1 && !info.isRepresentative) {
+            orc_rhd_step_t pre, post;
+            if (orc_rhd_prepost(&info, &pre, &post, 1, 0) != ORC_OK) {
+                return ORC_E_INTERNAL;
+            }
+            for (uint32_t u = pre.txSegStart; u < pre.txSegEnd; ++u) {
+                red_pair(r, scratch_at(sc, pre.peer, u), scratch_at(sc, j, u), sc->slotElems);
+            }
+        }
+    }
+    /* MAIN: tx and rx segments of a step are disjoint, so in-place per step is exact. */
+    uint32_t P = p - rhd_pair_num(p);
+    uint32_t total = orc_rhd_step_num(P);
+    for (uint32_t k = 0; k < total; ++k) {
+        for (uint32_t v = 0; v < P; ++v) {
+            uint32_t phys = orc_rhd_alg_rank_of_virtual(p, ORC_INVALID_RANK, v);
+            orc_rhd_part1(p, phys, ORC_INVALID_RANK, &info);
+            if (orc_rhd_rs_steps(&info, steps, &nSteps) != ORC_OK) {
+                return ORC_E_INTERNAL;
+            }
+            uint32_t peerPhys = orc_rhd_alg_rank_of_virtual(p, ORC_INVALID_RANK, steps[k].peer);
+            for (uint32_t u = steps[k].txSegStart; u < steps[k].txSegEnd; ++u) {
+                red_pair(r, scratch_at(sc, peerPhys, u), scratch_at(sc, phys, u), sc->slotElems);
+            }
+        }
+    }
+    /* POST (SHARE segment) */
+    if (!skipPost) {
+        for (uint32_t j = 0; j < p; ++j) {
+            orc_rhd_part1(p, j, ORC_INVALID_RANK, &info);
+            if (info.inPart1 && info.isRepresentative) {
+                orc_rhd_step_t pre, post;
+                if (orc_rhd_prepost(&info, &pre, &post, 1, 0) != ORC_OK) {
+                    return ORC_E_INTERNAL;
+                }
+                for (uint32_t u = post.txSegStart; u < post.txSegEnd; ++u) {
+                    memcpy(scratch_at(sc, post.peer, u), scratch_at(sc, j, u), sc->slotElems * sc->asz);
+                }
+            }
+        }
+    }
+    return ORC_OK;
+}
+
+int orc_reduce_scatter_rhd(uint32_t p, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                           int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (recvCount == 0) {
+        return ORC_OK;
+    }
+    scratch_t sc;
+    if (scratch_alloc(&sc, p, recvCount, r.asz) != ORC_OK) {
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t j = 0; j < p; ++j) {
+        for (uint32_t i = 0; i < p; ++i) {
+            red_widen(&r, cbytes(in[j]) + (uint64_t)i * recvCount * r.esz,
+                      scratch_at(&sc, j, orc_rhd_unit_start_of_rank(p, i)), recvCount);
+        }
+    }
+    rc = rhd_rs_frame(&r, &sc, 0);
+    if (rc == ORC_OK) {
+        for (uint32_t j = 0; j < p; ++j) {
+            red_narrow(&r, scratch_at(&sc, j, orc_rhd_unit_start_of_rank(p, j)), out[j], recvCount);
+        }
+    }
+    free(sc.mem);
+    return rc;
+}
+
+/* AG-RHD with PRE skipped and POST = FULL over a grid indexed by owner rank
+ * (all_gather_rhd.cc:355-365 owner map; template_utils.cc:211-249 steps). */
+static int rhd_ag_frame(scratch_t* grid)
+{
+    uint32_t p = grid->n;
+    uint32_t P = p - rhd_pair_num(p);
+    uint32_t total = orc_rhd_step_num(P);
+    orc_rhd_part1_t info;
+    orc_rhd_step_t steps[32];
+    uint32_t nSteps;
+    size_t slotBytes = grid->slotElems * grid->asz;
+    for (uint32_t k = 0; k < total; ++k) {
+        for (uint32_t v = 0; v < P; ++v) {
+            uint32_t phys = orc_rhd_alg_rank_of_virtual(p, ORC_INVALID_RANK, v);
+            orc_rhd_part1(p, phys, ORC_INVALID_RANK, &info);
+            if (orc_rhd_ag_steps(&info, steps, &nSteps) != ORC_OK) {
+                return ORC_E_INTERNAL;
+            }
+            uint32_t peerPhys = orc_rhd_alg_rank_of_virtual(p, ORC_INVALID_RANK, steps[k].peer);
+            for (uint32_t u = steps[k].txSegStart; u < steps[k].txSegEnd; ++u) {
+                uint32_t owner = orc_rhd_owner_of_unit(p, u);
+                memcpy(scratch_at(grid, peerPhys, owner), scratch_at(grid, phys, owner), slotBytes);
+            }
+        }
+    }
+    for (uint32_t j = 0; j < p; ++j) {
+        orc_rhd_part1(p, j, ORC_INVALID_RANK, &info);
+        if (info.inPart1 && info.isRepresentative) {
+            orc_rhd_step_t pre, post;
+            if (orc_rhd_prepost(&info, &pre, &post, 0, 1) != ORC_OK) {
+                return ORC_E_INTERNAL;
+            }
+            for (uint32_t u = post.txSegStart; u < post.txSegEnd; ++u) {
+                uint32_t owner = orc_rhd_owner_of_unit(p, u);
+                memcpy(scratch_at(grid, post.peer, owner), scratch_at(grid, j, owner), slotBytes);
+            }
+        }
+    }
+    return ORC_OK;
+}
+
+/* AllReduce over a flat p-rank RHD level: per loop the aligned prefix is split into p uniform
+ * units; a final remainder shorter than p is staged into a p-element tile whose unused lanes
+ * duplicate valid input (rhd_tail.h:98-165; executor_aicpu.cc:684-759). */
+int orc_all_reduce_rhd(uint32_t p, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                       int accMode, uint64_t maxCountPerLoop)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (maxCountPerLoop == 0) {
+        maxCountPerLoop = UINT64_MAX / 2;
+    }
+    maxCountPerLoop = maxCountPerLoop / p * p;
+    if (maxCountPerLoop == 0) {
+        return ORC_E_INTERNAL;
+    }
+    uint8_t* tile = (uint8_t*)malloc((size_t)p * p * r.esz);
+    uint8_t* result = (uint8_t*)malloc((count ? count : 1) * r.esz * p);
+    if (!tile || !result) {
+        free(tile);
+        free(result);
+        return ORC_E_INTERNAL;
+    }
+    uint64_t processed = 0;
+    while (processed < count && rc == ORC_OK) {
+        uint64_t valid = orc_rhd_select_loop_count(count - processed, maxCountPerLoop, p);
+        uint64_t curr = valid > p ? valid : p;
+        int padded = valid != curr;
+        uint64_t unit = curr / p;
+        scratch_t sc, grid;
+        if (scratch_alloc(&sc, p, unit, r.asz) != ORC_OK) {
+            rc = ORC_E_INTERNAL;
+            break;
+        }
+        if (scratch_alloc(&grid, p, unit, r.asz) != ORC_OK) {
+            free(sc.mem);
+            rc = ORC_E_INTERNAL;
+            break;
+        }
+        for (uint32_t j = 0; j < p; ++j) {
+            const uint8_t* src = cbytes(in[j]) + processed * r.esz;
+            if (padded) {
+                uint8_t* t = tile + (size_t)j * p * r.esz;
+                memcpy(t, src, valid * r.esz);
+                uint64_t filled = valid;
+                while (filled < p) {
+                    uint64_t c = filled < p - filled ? filled : p - filled;
+                    memcpy(t + filled * r.esz, t, c * r.esz);
+                    filled += c;
+                }
+                src = t;
+            }
+            for (uint32_t i = 0; i < p; ++i) {
+                red_widen(&r, src + (uint64_t)i * unit * r.esz, scratch_at(&sc, j, orc_rhd_unit_start_of_rank(p, i)),
+                          unit);
+            }
+        }
+        rc = rhd_rs_frame(&r, &sc, 1);
+        if (rc == ORC_OK) {
+            size_t slotBytes = unit * r.asz;
+            memset(grid.mem, 0, (uint64_t)p * p * slotBytes);
+            for (uint32_t j = 0; j < p; ++j) {
+                orc_rhd_part1_t info;
+                orc_rhd_part1(p, j, ORC_INVALID_RANK, &info);
+                if (info.inPart1 && !info.isRepresentative) {
+                    continue; /* merged ranks skip the final copy when POST is skipped */
+                }
+                memcpy(scratch_at(&grid, j, j), scratch_at(&sc, j, orc_rhd_unit_start_of_rank(p, j)), slotBytes);
+                if (info.inPart1 && info.isRepresentative) {
+                    /* bridge: merged party's final slot 2t+1 -> owner slot t+r (rhd_tail.h:33-53) */
+                    memcpy(scratch_at(&grid, j, info.pairedAlgRank), scratch_at(&sc, j, info.unitStart + 1),
+                           slotBytes);
+                }
+            }
+            rc = rhd_ag_frame(&grid);
+        }
+        if (rc == ORC_OK) {
+            for (uint32_t j = 0; j < p; ++j) {
+                uint8_t* dst = result + ((uint64_t)j * count + processed) * r.esz;
+                if (padded) {
+                    uint8_t* t = tile + (size_t)j * p * r.esz;
+                    for (uint32_t i = 0; i < p; ++i) red_narrow(&r, scratch_at(&grid, j, i), t + (size_t)i * r.esz, 1);
+                    memcpy(dst, t, valid * r.esz);
+                } else {
+                    for (uint32_t i = 0; i < p; ++i) {
+                        red_narrow(&r, scratch_at(&grid, j, i), dst + (uint64_t)i * unit * r.esz, unit);
+                    }
+                }
+            }
+        }
+        free(sc.mem);
+        free(grid.mem);
+        processed += valid;
+    }
+    if (rc == ORC_OK) {
+        for (uint32_t j = 0; j < p; ++j) memcpy(out[j], result + (uint64_t)j * count * r.esz, count * r.esz);
+    }
+    free(tile);
+    free(result);
+    return rc;
+}
+
+/* a12: while blocks > 1: M = largest power of two < blocks; for src = M..blocks-1:
+ * slot[src % M] = slot[src] (+) slot[src % M]; blocks = M.  Block v is rank v's contribution. */
+static uint32_t largest_pow2_less_than(uint32_t v)
+{
+    if (v <= 1) {
+        return 0;
+    }
+    uint32_t p = 1;
+    while (p * 2 < v) p *= 2;
+    return p;
+}
+
+static int order_preserved_fold(const red_t* r, uint32_t n, const void* const* in, uint64_t srcElemOff,
+                                uint64_t count, void* accOut /* count * asz */)
+{
+    uint8_t* slots = (uint8_t*)malloc((uint64_t)n * count * r->asz);
+    if (!slots) {
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t v = 0; v < n; ++v) {
+        red_widen(r, cbytes(in[v]) + srcElemOff * r->esz, slots + (uint64_t)v * count * r->asz, count);
+    }
+    uint32_t remaining = n;
+    while (remaining > 1) {
+        uint32_t M = largest_pow2_less_than(remaining);
+        if (M == 0) {
+            break;
+        }
+        for (uint32_t src = M; src < remaining; ++src) {
+            red_pair(r, slots + (uint64_t)(src % M) * count * r->asz, slots + (uint64_t)src * count * r->asz, count);
+        }
+        remaining = M;
+    }
+    memcpy(accOut, slots, count * r->asz);
+    free(slots);
+    return ORC_OK;
+}
+
+int orc_reduce_scatter_order_preserved(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount,
+                                       int dtype, int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK || recvCount == 0) {
+        return rc;
+    }
+    void* acc = malloc(recvCount * r.asz);
+    if (!acc) {
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t k = 0; k < n && rc == ORC_OK; ++k) {
+        rc = order_preserved_fold(&r, n, in, (uint64_t)k * recvCount, recvCount, acc);
+        if (rc == ORC_OK) {
+            red_narrow(&r, acc, out[k], recvCount);
+        }
+    }
+    free(acc);
+    return rc;
+}
+
+int orc_all_reduce_order_preserved(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype,
+                                   int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK || count == 0) {
+        return rc;
+    }
+    void* acc = malloc(count * r.asz);
+    if (!acc) {
+        return ORC_E_INTERNAL;
+    }
+    rc = order_preserved_fold(&r, n, in, 0, count, acc);
+    if (rc == ORC_OK) {
+        for (uint32_t k = 0; k < n; ++k) red_narrow(&r, acc, out[k], count);
+    }
+    free(acc);
+    return rc;
+}
+
+/* Vector-core mesh: rank k's output is cut into N chunks of recvCount / N elements (the last takes
+ * the remainder); chunk c = copy of peer c's slice, then peers c+1, c+2, ... (mod N) folded in. */
+int orc_reduce_scatter_aiv_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                                int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK || recvCount == 0) {
+        return rc;
+    }
+    uint64_t per = recvCount / n;
+    void* acc = malloc(recvCount * r.asz);
+    void* tmp = malloc(recvCount * r.asz);
+    if (!acc || !tmp) {
+        free(acc);
+        free(tmp);
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t k = 0; k < n; ++k) {
+        for (uint32_t c = 0; c < n; ++c) {
+            uint64_t off = (uint64_t)c * per;
+            uint64_t cnt = (c == n - 1) ? recvCount - per * (n - 1) : per;
+            if (cnt == 0) {
+                continue;
+            }
+            for (uint32_t i = 0; i < n; ++i) {
+                uint32_t peer = (i + c) % n;
+                const uint8_t* src = cbytes(in[peer]) + ((uint64_t)k * recvCount + off) * r.esz;
+                if (i == 0) {
+                    red_widen(&r, src, acc, cnt);
+                } else {
+                    red_pair_from_storage(&r, acc, src, cnt, tmp);
+                }
+            }
+            red_narrow(&r, acc, bytes(out[k]) + off * r.esz, cnt);
+        }
+    }
+    free(acc);
+    free(tmp);
+    return ORC_OK;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * a13 / a14 / a15: copies
+ * ------------------------------------------------------------------------------------------- */
+static int copy_dtype_ok(int dtype)
+{
+    /* Non-reduce ops reject only int128 and invalid values (op_common.cc:4349-4364). */
+    return orc_dtype_size(dtype) != 0 && dtype != 12 && dtype != 13;
+}
+
+int orc_all_gather(uint32_t n, const void* const* in, void* const* out, uint64_t sendCount, int dtype)
+{
+    if (!copy_dtype_ok(dtype)) {
+        return ORC_E_NOT_SUPPORT;
+    }
+    size_t esz = orc_dtype_size(dtype);
+    /* Gather into a temporary first so that an output aliasing an input stays well defined. */
+    uint8_t* all = (uint8_t*)malloc((uint64_t)n * sendCount * esz + 1);
+    if (!all) {
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t r = 0; r < n; ++r) memcpy(all + (uint64_t)r * sendCount * esz, in[r], sendCount * esz);
+    for (uint32_t r = 0; r < n; ++r) memcpy(out[r], all, (uint64_t)n * sendCount * esz);
+    free(all);
+    return ORC_OK;
+}
+
+int orc_all_gather_v(uint32_t n, const void* const* in, void* const* out, const uint64_t* counts,
+                     const uint64_t* displs, int dtype)
+{
+    if (!copy_dtype_ok(dtype)) {
+        return ORC_E_NOT_SUPPORT;
+    }
+    size_t esz = orc_dtype_size(dtype);
+    /* Non-empty intervals must not overlap (all_gather_v.cc:200-240). */
+    for (uint32_t a = 0; a < n; ++a) {
+        if (counts[a] == 0) continue;
+        if (displs[a] + counts[a] < displs[a]) return ORC_E_PARA;
+        for (uint32_t b = a + 1; b < n; ++b) {
+            if (counts[b] == 0) continue;
+            if (displs[a] < displs[b] + counts[b] && displs[b] < displs[a] + counts[a]) return ORC_E_PARA;
+        }
+    }
+    for (uint32_t dst = 0; dst < n; ++dst) {
+        for (uint32_t src = 0; src < n; ++src) {
+            memcpy(bytes(out[dst]) + displs[src] * esz, in[src], counts[src] * esz);
+        }
+    }
+    return ORC_OK;
+}
+
+int orc_all_to_all_v(uint32_t n, const void* const* in, void* const* out, const uint64_t* sendCounts,
+                     const uint64_t* sdispls, const uint64_t* recvCounts, const uint64_t* rdispls, int dtype)
+{
+    if (!copy_dtype_ok(dtype)) {
+        return ORC_E_NOT_SUPPORT;
+    }
+    size_t esz = orc_dtype_size(dtype);
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t j = 0; j < n; ++j) {
+            if (recvCounts[(uint64_t)i * n + j] != sendCounts[(uint64_t)j * n + i]) {
+                return ORC_E_PARA;
+            }
+        }
+    }
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t j = 0; j < n; ++j) {
+            uint64_t cnt = sendCounts[(uint64_t)j * n + i];
+            memcpy(bytes(out[i]) + rdispls[(uint64_t)i * n + j] * esz, cbytes(in[j]) + sdispls[(uint64_t)j * n + i] * esz,
+                   cnt * esz);
+        }
+    }
+    return ORC_OK;
+}
+
+/* a5: LocalCopySlices (wrapper.cc:930-997).  Zero-size slices are skipped; a slice whose source and
+ * destination both continue the pending run is merged into it; the pending run is issued when the
+ * next slice does not continue it or at the last slice. */
+uint32_t orc_local_copy_slices(uint32_t nSlices, const uint64_t* srcOff, const uint64_t* dstOff,
+                               const uint64_t* sizes, uint64_t* copies)
+{
+    if (nSlices == 0) {
+        return 0;
+    }
+    uint32_t issued = 0;
+    uint64_t curSrc = srcOff[0], curDst = dstOff[0], curSize = sizes[0];
+    for (uint32_t i = 0; i < nSlices; ++i) {
+        if (sizes[i] == 0) {
+            continue;
+        }
+        if (i == nSlices - 1) {
+            copies[issued * 3 + 0] = curSrc;
+            copies[issued * 3 + 1] = curDst;
+            copies[issued * 3 + 2] = curSize;
+            issued++;
+        } else if (srcOff[i + 1] == curSrc + curSize && dstOff[i + 1] == curDst + curSize) {
+            curSize += sizes[i + 1];
+        } else {
+            copies[issued * 3 + 0] = curSrc;
+            copies[issued * 3 + 1] = curDst;
+            copies[issued * 3 + 2] = curSize;
+            issued++;
+            curSrc = srcOff[i + 1];
+            curDst = dstOff[i + 1];
+            curSize = sizes[i + 1];
+        }
+    }
+    return issued;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * "All cores" CPU baseline: static split of the element range over threads.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+    int isRs;
+    uint32_t n;
+    const void* const* in;
+    void* const* out;
+    uint64_t recvCount, first, count;
+    const red_t* r;
+    int rc;
+} mt_job_t;
+
+static void* mt_worker(void* arg)
+{
+    mt_job_t* j = (mt_job_t*)arg;
+    if (j->isRs) {
+        j->rc = reduce_scatter_mesh_range(j->n, j->in, j->out, j->recvCount, j->first, j->count, j->r);
+    } else {
+        j->rc = all_reduce_mesh_range(j->n, j->in, j->out, j->first, j->count, j->r);
+    }
+    return NULL;
+}
+
+static int run_mt(int isRs, uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                  int accMode, uint32_t nThreads)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (nThreads == 0) {
+        nThreads = 1;
+    }
+    pthread_t* th = (pthread_t*)malloc(sizeof(pthread_t) * nThreads);
+    mt_job_t* jobs = (mt_job_t*)malloc(sizeof(mt_job_t) * nThreads);
+    uint64_t per = (count + nThreads - 1) / nThreads;
+    uint32_t started = 0;
+    for (uint32_t t = 0; t < nThreads; ++t) {
+        uint64_t first = (uint64_t)t * per;
+        if (first >= count) {
+            break;
+        }
+        mt_job_t j = {isRs, n, in, out, count, first, (count - first < per) ? count - first : per, &r, ORC_OK};
+        jobs[t] = j;
+        pthread_create(&th[t], NULL, mt_worker, &jobs[t]);
+        started++;
+    }
+    for (uint32_t t = 0; t < started; ++t) {
+        pthread_join(th[t], NULL);
+        if (jobs[t].rc != ORC_OK) {
+            rc = jobs[t].rc;
+        }
+    }
+    free(th);
+    free(jobs);
+    return rc;
+}
+
+int orc_reduce_scatter_mesh_mt(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                               int op, int accMode, uint32_t nThreads)
+{
+    return run_mt(1, n, in, out, recvCount, dtype, op, accMode, nThreads);
+}
+
+int orc_all_reduce_mesh_mt(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                           int accMode, uint32_t nThreads)
+{
+    return run_mt(0, n, in, out, count, dtype, op, accMode, nThreads);
+}

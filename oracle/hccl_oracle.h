@@ -1,0 +1,161 @@
+/*
+ * CPU oracle for the loopback data plane.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This is a plain-C restatement of what the reference computes on the path
+ * "local reduce / slice copy / displacement pack-unpack" of its ring, mesh and
+ * recursive-halving-doubling executors.  Only tests/, __graft_entry__.smoke() and the
+ * cpu_baseline leg of bench.py may load it; the shipped library never links or calls it.
+ *
+ * Every function names the reference lines it follows.  Where the reference's own
+ * arithmetic is not in its tree (device DMA reduce for int16 / bf16 / fp16-SUM lives in the
+ * separate HCOMM library) the function says "parity unpinned" and states the rule used.
+ *
+ * Reference build status: the host-reduce arithmetic sits in
+ * src/ops/op_common/algorithm/template/wrapper/alg_data_trans_wrapper.cc, a translation
+ * unit that includes HCOMM / CANN headers which are not part of the reference tree, so it
+ * cannot be compiled from its own sources here (no oracle/_ref).  The restatement is pinned
+ * instead by IEEE-754 / two's-complement closed forms, exhaustive numpy float16 tables,
+ * brute force on tiny inputs and the step tables held by the reference's unit tests.
+ */
+#ifndef HCCL_ORACLE_H_
+#define HCCL_ORACLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Same numeric values as HcclDataType / HcclReduceOp / HcclResult. */
+enum {
+    ORC_INT8 = 0, ORC_INT16 = 1, ORC_INT32 = 2, ORC_FP16 = 3, ORC_FP32 = 4, ORC_INT64 = 5, ORC_UINT64 = 6,
+    ORC_UINT8 = 7, ORC_UINT16 = 8, ORC_UINT32 = 9, ORC_FP64 = 10, ORC_BF16 = 11
+};
+enum { ORC_SUM = 0, ORC_PROD = 1, ORC_MAX = 2, ORC_MIN = 3 };
+enum { ORC_OK = 0, ORC_E_PARA = 1, ORC_E_PTR = 2, ORC_E_INTERNAL = 4, ORC_E_NOT_SUPPORT = 5 };
+
+/* How fp16 / bf16 SUM chains accumulate.
+ *   ORC_ACC_STEP : every pairwise step widens to fp32, adds, and narrows again -- the
+ *                  reference's host pattern (AicpuReduceFp16, wrapper.cc:1237-1257).
+ *   ORC_ACC_FP32 : operands are widened once, the whole chain runs in fp32 in the
+ *                  algorithm's order, one round-to-nearest-even narrowing at the end.
+ *                  This is the rule the GPU kernels implement for fp16 / bf16 SUM (the
+ *                  reference's device DMA reduce for these is not in its tree: parity
+ *                  unpinned; accepted tolerance is 1 ulp against this mode).
+ * PROD / MAX / MIN and every non-half type behave identically in both modes except fp16
+ * PROD, which always narrows after every step (it only exists on the host path). */
+enum { ORC_ACC_STEP = 0, ORC_ACC_FP32 = 1 };
+
+size_t orc_dtype_size(int dtype);
+
+/* --- a2: half conversions (wrapper.cc:1082-1235) ------------------------------------- */
+float orc_fp16_to_fp32(uint16_t h);
+uint16_t orc_fp32_to_fp16(float f);
+/* bf16 has no host path in the reference (parity unpinned): widen = bits << 16; narrow =
+ * round-to-nearest-even on the upper 16 bits, NaN keeps sign and payload top bits with the
+ * quiet bit forced. */
+float orc_bf16_to_fp32(uint16_t h);
+uint16_t orc_fp32_to_bf16(float f);
+/* Array forms of the four conversions (same functions applied element by element). */
+void orc_fp16_to_fp32_n(const uint16_t* in, float* out, uint64_t n);
+void orc_fp32_to_fp16_n(const float* in, uint16_t* out, uint64_t n);
+void orc_bf16_to_fp32_n(const uint16_t* in, float* out, uint64_t n);
+void orc_fp32_to_bf16_n(const float* in, uint16_t* out, uint64_t n);
+
+/* --- a1/a3: dst[i] = src[i] (+) dst[i] ------------------------------------------------ */
+/* Strict restatement of AicpuReduce (wrapper.cc:1259-1316): byte sizes, E_INTERNAL on a size
+ * mismatch or on a type outside {int8,int32,fp16,fp32,int64,uint64,fp64}. */
+int orc_aicpu_reduce(void* dst, uint64_t dstBytes, const void* src, uint64_t srcBytes, int dtype, int op);
+/* Same plus int16 (modular, like int8/int32) and bf16 (fp16 pattern): "by analogy". */
+int orc_pair_reduce(void* dst, const void* src, uint64_t count, int dtype, int op);
+
+/* --- a16 / a10 / a11: step geometry (template_utils.cc:32-362) ------------------------ */
+#define ORC_INVALID_RANK 0xFFFFFFFFu
+typedef struct {
+    uint32_t r, effectiveRankSize, virtualRank, inPart1, isRepresentative, pairedAlgRank, unitStart, unitCount,
+        isPowerOfTwo;
+} orc_rhd_part1_t;
+typedef struct {
+    uint32_t step, peer, nSlices, txSegStart, txSegEnd, rxSegStart, rxSegEnd;
+} orc_rhd_step_t;
+
+uint64_t orc_round_up(uint64_t dividend, uint64_t divisor);       /* template_utils.h:766 */
+uint32_t orc_nhr_step_num(uint32_t rankSize);                      /* template_utils.cc:32 */
+uint32_t orc_rhd_step_num(uint32_t rankSize);                      /* :42 */
+uint32_t orc_rhd_unit_start_of_rank(uint32_t p, uint32_t algRank); /* :93 (sigma) */
+uint32_t orc_rhd_alg_rank_of_virtual(uint32_t p, uint32_t root, uint32_t v); /* :101 */
+uint32_t orc_rhd_owner_of_unit(uint32_t p, uint32_t unit); /* ins_temp_all_gather_rhd.cc:355-365 */
+int orc_rhd_part1(uint32_t p, uint32_t algRank, uint32_t root, orc_rhd_part1_t* info);     /* :117 */
+int orc_rhd_rs_steps(const orc_rhd_part1_t* info, orc_rhd_step_t* steps, uint32_t* nSteps); /* :170 */
+int orc_rhd_ag_steps(const orc_rhd_part1_t* info, orc_rhd_step_t* steps, uint32_t* nSteps); /* :211 */
+int orc_rhd_prepost(const orc_rhd_part1_t* info, orc_rhd_step_t* pre, orc_rhd_step_t* post, int preFull,
+                    int postFull);                                                           /* :251 */
+void orc_rhd_seg_bytes_uniform(uint32_t unitStart, uint32_t unitEnd, uint64_t sliceSize, uint64_t tailSize,
+                               uint32_t tailUnit, uint64_t* offset, uint64_t* len);          /* :310 */
+/* ins_v2_all_reduce_sequence_rhd_tail.h:98-113 */
+uint64_t orc_rhd_select_loop_count(uint64_t remaining, uint64_t maxCountPerLoop, uint64_t rankAlign);
+/* ins_temp_reduce_scatter_nhr.cc:458-506; tx/rx arrays need rankSize entries. */
+int orc_nhr_step_info(uint32_t rankSize, uint32_t algRank, uint32_t step, uint32_t* toRank, uint32_t* fromRank,
+                      uint32_t* nSlices, uint32_t* txSliceIdxs, uint32_t* rxSliceIdxs);
+
+/* --- collectives over N loopback ranks ------------------------------------------------
+ * in[r] / out[r] are rank r's send / recv buffers (host memory).  accMode is ORC_ACC_*.  */
+
+/* a6/a7/a8: (((x0+x1)+x2)...): one-shot (one_shot.cc:203-242) / host NHR (aicpu_reduce_nhr.cc:266-288). */
+int orc_all_reduce_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                        int accMode);
+/* a8: two-shot slicing (two_shot.cc:178-210, 326-360) then gather; same values as one-shot. */
+int orc_all_reduce_two_shot(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                            int accMode);
+/* a11: RS-RHD (skip POST) + bridge + AG-RHD (skip PRE), looped per rhd_tail.h; maxCountPerLoop 0 = unbounded. */
+int orc_all_reduce_rhd(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                       int accMode, uint64_t maxCountPerLoop);
+/* a9: own slice first, then ranks ascending (reduce_scatter_mesh_1D.cc:203-237). */
+int orc_reduce_scatter_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                            int op, int accMode);
+/* a10: write-reduce steps of reduce_scatter_nhr.cc:316-447. */
+int orc_reduce_scatter_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                           int op, int accMode);
+/* a11: mirror / PRE / MAIN / POST of reduce_scatter_rhd.cc:192-245. */
+int orc_reduce_scatter_rhd(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                           int op, int accMode);
+/* a12: power-of-two block fold (order_preserved_group.cc:306-409). */
+int orc_reduce_scatter_order_preserved(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount,
+                                       int dtype, int op, int accMode);
+int orc_all_reduce_order_preserved(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype,
+                                   int op, int accMode);
+/* vector-core mesh order (aiv_reduce_scatter_mesh_1d.h:23-71). */
+int orc_reduce_scatter_aiv_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                                int op, int accMode);
+/* AllReduce whose every element follows the NHR reduce-scatter tree of its slice
+ * (slices of ceil(count/n) elements), then gather. */
+int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                       int accMode);
+
+/* a13: all_gather_mesh_1D.cc:249-423. */
+int orc_all_gather(uint32_t n, const void* const* in, void* const* out, uint64_t sendCount, int dtype);
+/* a14: all_gather_v_mesh_1D.cc:242-310; counts/displs are the (identical) per-rank arrays. */
+int orc_all_gather_v(uint32_t n, const void* const* in, void* const* out, const uint64_t* recvCounts,
+                     const uint64_t* recvDispls, int dtype);
+/* a15: all_to_all_v_mesh_1D.cc:229-246, 459-611.  The four tables are n x n row-major,
+ * row r = rank r's argument array. */
+int orc_all_to_all_v(uint32_t n, const void* const* in, void* const* out, const uint64_t* sendCounts,
+                     const uint64_t* sdispls, const uint64_t* recvCounts, const uint64_t* rdispls, int dtype);
+
+/* a5: LocalCopySlices merge rule (wrapper.cc:930-997): returns how many copies are issued
+ * for slices (offset,size) over one base address; copies[] gets (srcOff,dstOff,size) triples. */
+uint32_t orc_local_copy_slices(uint32_t nSlices, const uint64_t* srcOff, const uint64_t* dstOff,
+                               const uint64_t* sizes, uint64_t* copies);
+
+/* Multi-threaded variants used only for the "all cores" CPU baseline: the element range is
+ * split statically over nThreads. */
+int orc_reduce_scatter_mesh_mt(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                               int op, int accMode, uint32_t nThreads);
+int orc_all_reduce_mesh_mt(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                           int accMode, uint32_t nThreads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HCCL_ORACLE_H_ */

@@ -1,0 +1,439 @@
+"""Pins the association order and data movement of every executor the oracle restates
+(rows a5-a15), by brute force on small inputs against the order written in the reference's
+templates, its worked examples, and independent closed forms.
+
+fp32 inputs span ~12 decades so that a different association order changes low bits in most
+elements; MAX / MIN inputs are drawn from {+0, -0, NaNs with distinct payloads, 1} so that a swapped
+src / dst role changes the result.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "rhd_nhr_tables.json")))
+I8, I16, I32, F16, F32, I64, U64, F64, BF16 = 0, 1, 2, 3, 4, 5, 6, 10, 11
+SUM, PROD, MAX, MIN = range(4)
+
+
+def wide_f32(rng, n, count):
+    return [(rng.standard_normal(count) * 10.0 ** rng.integers(-6, 6, count)).astype(np.float32) for _ in range(n)]
+
+
+def tricky_f32(rng, n, count):
+    pool = np.array([0x00000000, 0x80000000, 0x7FC00001, 0x7FC00002, 0xFFC00003, 0x3F800000, 0xBF800000],
+                    dtype=np.uint32)
+    return [pool[rng.integers(0, pool.size, count)].view(np.float32).copy() for _ in range(n)]
+
+
+def f32_op(src, dst, op):
+    """dst <- src (+) dst with the reference's operand roles."""
+    with np.errstate(all="ignore"):
+        if op == SUM:
+            return src + dst
+        if op == PROD:
+            return src * dst
+        if op == MAX:
+            return np.where(src < dst, dst, src)
+        return np.where(dst < src, dst, src)
+
+
+def bits_equal_nan_class(a, b):
+    """Bit-exact except that arithmetic NaNs only need to be NaN on both sides."""
+    a32, b32 = a.view(np.uint32), b.view(np.uint32)
+    both_nan = np.isnan(a) & np.isnan(b)
+    return np.array_equal(a32[~both_nan], b32[~both_nan]) and np.array_equal(np.isnan(a), np.isnan(b))
+
+
+def outs_like(ins, count=None):
+    return [np.zeros(ins[0].size if count is None else count, dtype=ins[0].dtype) for _ in ins]
+
+
+# ---------------------------------------------------------------------------------------------
+# AllReduce in rank order (a6, a7, a8)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1, 2, 3, 8, 16])
+@pytest.mark.parametrize("algo", ["mesh", "two_shot"])
+def test_all_reduce_rank_order_fp32(orc, n, algo):
+    rng = np.random.default_rng(n)
+    count = 1031
+    ins = wide_f32(rng, n, count)
+    outs = outs_like(ins)
+    assert orc.all_reduce(ins, outs, count, F32, SUM, algo=algo) == 0
+    acc = ins[0].copy()
+    for r in range(1, n):
+        acc = ins[r] + acc
+    for o in outs:
+        assert np.array_equal(o.view(np.uint32), acc.view(np.uint32))
+    if n >= 8:   # the check discriminates: pairwise-tree order gives different bits
+        tree = [x.copy() for x in ins]
+        while len(tree) > 1:
+            tree = [tree[i] + tree[i + 1] for i in range(0, len(tree), 2)]
+        assert np.count_nonzero(tree[0] != acc) > count // 10
+
+
+@pytest.mark.parametrize("op", [MAX, MIN])
+def test_all_reduce_rank_order_roles(orc, op):
+    rng = np.random.default_rng(3)
+    n, count = 5, 4096
+    ins = tricky_f32(rng, n, count)
+    outs = outs_like(ins)
+    assert orc.all_reduce(ins, outs, count, F32, op) == 0
+    acc = ins[0].copy()
+    for r in range(1, n):
+        acc = f32_op(ins[r], acc, op)
+    assert np.array_equal(outs[0].view(np.uint32), acc.view(np.uint32))
+    # swapping the roles is observable on this input
+    swapped = ins[0].copy()
+    for r in range(1, n):
+        swapped = f32_op(swapped, ins[r], op)
+    assert np.count_nonzero(swapped.view(np.uint32) != acc.view(np.uint32)) > 100
+
+
+def test_all_reduce_in_place(orc):
+    rng = np.random.default_rng(4)
+    ins = [rng.integers(-100, 100, 257, dtype=np.int32) for _ in range(4)]
+    want = sum(x.astype(np.int64) for x in ins).astype(np.int32)
+    assert orc.all_reduce(ins, ins, 257, I32, SUM) == 0
+    for x in ins:
+        assert np.array_equal(x, want)
+
+
+# ---------------------------------------------------------------------------------------------
+# ReduceScatter orders (a9, a10, a12, vector-core mesh)
+# ---------------------------------------------------------------------------------------------
+def rs_expected(ins, n, c, k, leaf_order):
+    """Left fold over leaf_order of rank t's slice k."""
+    acc = ins[leaf_order[0]][k * c:(k + 1) * c].copy()
+    for t in leaf_order[1:]:
+        acc = ins[t][k * c:(k + 1) * c] + acc
+    return acc
+
+
+@pytest.mark.parametrize("n", [1, 2, 5, 8])
+def test_reduce_scatter_mesh_own_rank_first(orc, n):
+    rng = np.random.default_rng(10 + n)
+    c = 333
+    ins = wide_f32(rng, n, n * c)
+    outs = outs_like(ins, c)
+    assert orc.reduce_scatter(ins, outs, c, F32, SUM, algo="mesh") == 0
+    for k in range(n):
+        order = [k] + [t for t in range(n) if t != k]
+        assert np.array_equal(outs[k].view(np.uint32), rs_expected(ins, n, c, k, order).view(np.uint32))
+    if n == 8:
+        plain = rs_expected(ins, n, c, 5, list(range(n)))
+        assert np.count_nonzero(plain != outs[5]) > c // 10
+
+
+def test_reduce_scatter_nhr_tree_n8(orc):
+    """Slice k ends as ((x_k+x_k+1)+(x_k+2+x_k+3)) + ((x_k+4+x_k+5)+(x_k+6+x_k+7)), indices mod 8,
+    the receiver's partial being dst at every step."""
+    rng = np.random.default_rng(21)
+    n, c = 8, 257
+    ins = wide_f32(rng, n, n * c)
+    outs = outs_like(ins, c)
+    assert orc.reduce_scatter(ins, outs, c, F32, SUM, algo="nhr") == 0
+    for k in range(n):
+        x = [ins[(k + i) % n][k * c:(k + 1) * c] for i in range(n)]
+        a = (x[1] + x[0])
+        b = (x[3] + x[2])
+        cc = (x[5] + x[4])
+        d = (x[7] + x[6])
+        want = (((d + cc)) + (b + a))
+        assert np.array_equal(outs[k].view(np.uint32), want.view(np.uint32)), k
+
+
+def test_reduce_scatter_nhr_roles_n4(orc):
+    """N=4 from the reference's hand table: step 0 rank m receives slices {m, m-2} from m+1; step 1 slice m
+    from m+2.  Slice k at rank k: step0 acc = x_{k+1} (+) x_k ; rank k+2 holds x_{k+3} (+) x_{k+2};
+    step1 acc = (x_{k+3} (+) x_{k+2}) (+) acc."""
+    rng = np.random.default_rng(22)
+    n, c = 4, 512
+    ins = tricky_f32(rng, n, n * c)
+    for op in (MAX, MIN):
+        outs = outs_like(ins, c)
+        assert orc.reduce_scatter(ins, outs, c, F32, op, algo="nhr") == 0
+        for k in range(n):
+            x = [ins[(k + i) % n][k * c:(k + 1) * c] for i in range(n)]
+            own = f32_op(x[1], x[0], op)
+            far = f32_op(x[3], x[2], op)
+            want = f32_op(far, own, op)
+            assert np.array_equal(outs[k].view(np.uint32), want.view(np.uint32))
+
+
+def test_order_preserved_six_block_example(orc):
+    """The worked example in the reference's own comment: E->A, F->B, C->(AE), D->(BF), (BFD)->(AEC)."""
+    rng = np.random.default_rng(30)
+    n, c = 6, 300
+    ins = wide_f32(rng, n, n * c)
+    outs = outs_like(ins, c)
+    assert orc.reduce_scatter(ins, outs, c, F32, SUM, algo="order_preserved") == 0
+    for k in range(n):
+        slot = [ins[t][k * c:(k + 1) * c].copy() for t in range(n)]
+        for src, dst in GOLD["order_preserved_six_blocks"]["steps"]:
+            slot[dst] = slot[src] + slot[dst]
+        assert np.array_equal(outs[k].view(np.uint32), slot[0].view(np.uint32))
+
+
+def test_order_preserved_n8_tree(orc):
+    rng = np.random.default_rng(31)
+    n, count = 8, 999
+    x = wide_f32(rng, n, count)
+    outs = outs_like(x)
+    assert orc.all_reduce(x, outs, count, F32, SUM, algo="order_preserved") == 0
+    want = ((x[4] + x[0]) + (x[6] + x[2])) + ((x[5] + x[1]) + (x[7] + x[3]))
+    # association: ((x0+x4)+(x2+x6)) + ((x1+x5)+(x3+x7)); fp add is commutative bit for bit
+    assert np.array_equal(outs[3].view(np.uint32), want.view(np.uint32))
+
+
+def test_aiv_mesh_chunk_rotation(orc):
+    rng = np.random.default_rng(40)
+    n, c = 4, 103     # 103 = 4*25 + 3: the last chunk takes the remainder
+    ins = wide_f32(rng, n, n * c)
+    outs = outs_like(ins, c)
+    assert orc.reduce_scatter(ins, outs, c, F32, SUM, algo="aiv_mesh") == 0
+    per = c // n
+    for k in range(n):
+        for ch in range(n):
+            lo = ch * per
+            hi = c if ch == n - 1 else lo + per
+            acc = ins[ch][k * c + lo:k * c + hi].copy()
+            for i in range(1, n):
+                acc = ins[(ch + i) % n][k * c + lo:k * c + hi] + acc
+            assert np.array_equal(outs[k][lo:hi].view(np.uint32), acc.view(np.uint32))
+
+
+# ---------------------------------------------------------------------------------------------
+# RHD (a11): message-passing simulation vs an independent recursive closed form
+# ---------------------------------------------------------------------------------------------
+def rhd_tree(x, p, i, op):
+    """Value of data unit i after RHD: holder f folds, at halving step k, the partial of f ^ (P >> (k+1))
+    (incoming = src) into its own (dst); virtual rank v < r starts from x[v+r] (+) x[v]."""
+    hp = 1
+    while hp <= p // 2:
+        hp *= 2
+    r, P = p - hp, hp
+    K = P.bit_length() - 1
+    f = i if i < r else i - r
+
+    def leaf(v):
+        return f32_op(x[v + r], x[v], op) if v < r else x[v + r]
+
+    def held(k, v):
+        if k < 0:
+            return leaf(v)
+        dist = P >> (k + 1)
+        return f32_op(held(k - 1, v ^ dist), held(k - 1, v), op)
+
+    return held(K - 1, f)
+
+
+def test_rhd_p6_worked_example(orc):
+    rng = np.random.default_rng(50)
+    p, c = 6, 200
+    ins = wide_f32(rng, p, p * c)
+    outs = outs_like(ins, c)
+    assert orc.reduce_scatter(ins, outs, c, F32, SUM, algo="rhd") == 0
+    for k in range(p):
+        x = [ins[t][k * c:(k + 1) * c] for t in range(p)]
+        want = ((x[0] + x[2]) + x[4]) + ((x[1] + x[3]) + x[5])
+        assert np.array_equal(outs[k].view(np.uint32), want.view(np.uint32)), k
+
+
+@pytest.mark.parametrize("p", [2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17])
+@pytest.mark.parametrize("op", [SUM, MAX, MIN])
+def test_rhd_reduce_scatter_matches_closed_form(orc, p, op):
+    rng = np.random.default_rng(100 * p + op)
+    c = 64
+    ins = wide_f32(rng, p, p * c) if op == SUM else tricky_f32(rng, p, p * c)
+    outs = outs_like(ins, c)
+    assert orc.reduce_scatter(ins, outs, c, F32, op, algo="rhd") == 0
+    for k in range(p):
+        x = [ins[t][k * c:(k + 1) * c] for t in range(p)]
+        assert bits_equal_nan_class(outs[k], rhd_tree(x, p, k, op)), (p, k)
+
+
+@pytest.mark.parametrize("p,count", [(6, 6 * 40), (6, 6 * 40 + 5), (5, 3), (3, 100), (12, 1000), (7, 7), (8, 64)])
+@pytest.mark.parametrize("op", [SUM, MAX])
+def test_rhd_all_reduce_units_and_tail(orc, p, count, op):
+    rng = np.random.default_rng(p * 7 + count)
+    ins = wide_f32(rng, p, count) if op == SUM else tricky_f32(rng, p, count)
+    outs = outs_like(ins)
+    assert orc.all_reduce(ins, outs, count, F32, op, algo="rhd") == 0
+    unit = count // p
+    want = np.zeros(count, dtype=np.float32)
+    for i in range(p):
+        lo, hi = i * unit, (i + 1) * unit
+        want[lo:hi] = rhd_tree([x[lo:hi] for x in ins], p, i, op)
+    for e in range(unit * p, count):       # padded tail: element e sits alone in unit e - unit*p
+        want[e:e + 1] = rhd_tree([x[e:e + 1] for x in ins], p, e - unit * p, op)
+    for o in outs:
+        assert bits_equal_nan_class(o, want)
+
+
+def test_rhd_all_reduce_loop_bound_changes_only_roles(orc):
+    """A bounded staging buffer re-cuts the units per loop; integer results cannot depend on it."""
+    rng = np.random.default_rng(60)
+    p, count = 6, 1000
+    ins = [rng.integers(-2 ** 31, 2 ** 31 - 1, count, dtype=np.int32) for _ in range(p)]
+    a, b = outs_like(ins), outs_like(ins)
+    assert orc.all_reduce(ins, a, count, I32, SUM, algo="rhd") == 0
+    assert orc.all_reduce(ins, b, count, I32, SUM, algo="rhd", max_count_per_loop=120) == 0
+    want = np.sum(np.stack(ins).astype(np.int64), axis=0).astype(np.int32)
+    assert np.array_equal(a[0], want) and np.array_equal(b[5], want)
+
+
+# ---------------------------------------------------------------------------------------------
+# Every algorithm uses every rank exactly once; integer results are order independent
+# ---------------------------------------------------------------------------------------------
+AR_ALGOS = ["mesh", "two_shot", "rhd", "nhr", "order_preserved"]
+RS_ALGOS = ["mesh", "nhr", "rhd", "order_preserved", "aiv_mesh"]
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 6, 7, 8, 16, 33, 64])
+def test_every_rank_contributes_once(orc, n):
+    count = 2 * n + 3
+    ins = [np.full(count, np.uint64(1) << np.uint64(r), dtype=np.uint64) for r in range(n)]
+    full = np.uint64((1 << n) - 1)
+    for algo in AR_ALGOS:
+        outs = outs_like(ins)
+        assert orc.all_reduce(ins, outs, count, U64, SUM, algo=algo) == 0, algo
+        for o in outs:
+            assert np.all(o == full), (algo, n)
+    c = 7
+    ins = [np.full(n * c, np.uint64(1) << np.uint64(r), dtype=np.uint64) for r in range(n)]
+    for algo in RS_ALGOS:
+        outs = outs_like(ins, c)
+        assert orc.reduce_scatter(ins, outs, c, U64, SUM, algo=algo) == 0, algo
+        for o in outs:
+            assert np.all(o == full), (algo, n)
+
+
+@pytest.mark.parametrize("dtype,npdt", [(I8, np.int8), (I16, np.int16), (I32, np.int32), (I64, np.int64)])
+def test_integer_results_match_modular_closed_form(orc, dtype, npdt):
+    rng = np.random.default_rng(int(dtype) + 70)
+    n, count = 6, 1234
+    info = np.iinfo(npdt)
+    ins = [rng.integers(info.min, info.max, count, dtype=npdt, endpoint=True) for _ in range(n)]
+    stack = np.stack(ins).astype(object)
+    bits = info.bits
+    for op in (SUM, PROD, MAX, MIN):
+        if op == PROD and dtype == I16:
+            continue
+        if op == SUM:
+            want = [sum(int(v) for v in col) for col in stack.T]
+        elif op == PROD:
+            want = []
+            for col in stack.T:
+                acc = 1
+                for v in col:
+                    acc *= int(v)
+                want.append(acc)
+        elif op == MAX:
+            want = [max(int(v) for v in col) for col in stack.T]
+        else:
+            want = [min(int(v) for v in col) for col in stack.T]
+        want = np.array([w % (1 << bits) for w in want], dtype=object)
+        for algo in AR_ALGOS:
+            outs = outs_like(ins)
+            assert orc.all_reduce(ins, outs, count, dtype, op, algo=algo) == 0
+            got = np.array([int(v) % (1 << bits) for v in outs[n - 1]], dtype=object)
+            assert np.array_equal(got, want), (algo, op)
+
+
+def test_half_accumulation_modes(orc):
+    """ACC_FP32: one rounding at the end; ACC_STEP: the host pattern rounds after every pair."""
+    rng = np.random.default_rng(80)
+    n, count = 8, 5000
+    f = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]
+    for dtype, narrow, widen in ((F16, lambda a: a.astype(np.float16).view(np.uint16),
+                                  lambda h: h.view(np.float16).astype(np.float32)),
+                                 (BF16, orc.np_fp32_to_bf16_bits, orc.bf16_bits_to_fp32)):
+        ins = [narrow(x) for x in f]
+        w = [widen(h) for h in ins]
+        outs = outs_like(ins)
+        assert orc.all_reduce(ins, outs, count, dtype, SUM, acc=orc.ACC_FP32) == 0
+        acc = w[0].copy()
+        for r in range(1, n):
+            acc = w[r] + acc
+        assert np.array_equal(outs[0], narrow(acc))
+        assert orc.all_reduce(ins, outs, count, dtype, SUM, acc=orc.ACC_STEP) == 0
+        acc = w[0].copy()
+        for r in range(1, n):
+            acc = widen(narrow(w[r] + acc))
+        assert np.array_equal(outs[0], narrow(acc))
+        # fp32 accumulation is within 1 ulp of the exactly-rounded sum
+        exact = narrow(np.sum(np.stack(w).astype(np.float64), axis=0).astype(np.float32))
+        assert orc.all_reduce(ins, outs, count, dtype, SUM, acc=orc.ACC_FP32) == 0
+        d = np.abs(outs[0].astype(np.int32) - exact.astype(np.int32))
+        same_sign = (outs[0] >> 15) == (exact >> 15)
+        assert np.all(d[same_sign] <= 1)
+
+
+def test_admission(orc):
+    a = [np.zeros(8, dtype=np.uint16) for _ in range(2)]
+    o = outs_like(a)
+    assert orc.all_reduce(a, o, 8, 7, SUM) == 5         # uint8 cannot be reduced
+    assert orc.all_reduce(a, o, 8, I16, PROD) == 5      # PROD not defined for int16
+    assert orc.all_reduce(a, o, 8, BF16, PROD) == 5
+    assert orc.all_reduce(a, o, 8, BF16, MAX) == 0
+    assert orc.all_reduce(a, o, 0, F16, SUM) == 0
+
+
+# ---------------------------------------------------------------------------------------------
+# Copies (a13, a14, a15): index maps on distinct byte patterns
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1, 2, 3, 8])
+def test_all_gather_index_map(orc, n):
+    c = 37
+    ins = [(np.arange(c, dtype=np.uint16) + 1000 * r).astype(np.uint16) for r in range(n)]
+    outs = [np.zeros(n * c, dtype=np.uint16) for _ in range(n)]
+    assert orc.all_gather(ins, outs, c, F16) == 0
+    for o in outs:
+        for r in range(n):
+            assert np.array_equal(o[r * c:(r + 1) * c], ins[r])
+
+
+def test_all_gather_v_unordered_with_holes(orc):
+    n = 4
+    counts = [5, 0, 9, 3]
+    displs = [20, 7, 0, 11]            # unordered, holes at [9,11) and [14,20)
+    ins = [np.full(max(c, 1), 10 + r, dtype=np.int32) for r, c in enumerate(counts)]
+    outs = [np.full(25, -1, dtype=np.int32) for _ in range(n)]
+    assert orc.all_gather_v(ins, outs, counts, displs, I32) == 0
+    want = np.full(25, -1, dtype=np.int32)
+    want[20:25], want[0:9], want[11:14] = 10, 12, 13
+    for o in outs:
+        assert np.array_equal(o, want)
+    assert orc.all_gather_v(ins, outs, [5, 5, 0, 0], [0, 4, 0, 0], I32) == 1   # overlap
+
+
+@pytest.mark.parametrize("n", [2, 3, 8])
+def test_all_to_all_v_index_map(orc, n):
+    rng = np.random.default_rng(n)
+    send_counts = rng.integers(0, 6, size=(n, n)).astype(np.uint64)
+    recv_counts = send_counts.T.copy()
+    # displacements with gaps, in shuffled block order
+    sdispls = np.zeros((n, n), dtype=np.uint64)
+    rdispls = np.zeros((n, n), dtype=np.uint64)
+    for r in range(n):
+        for tab, cnts in ((sdispls, send_counts), (rdispls, recv_counts)):
+            off = 1
+            for j in rng.permutation(n):
+                tab[r, j] = off
+                off += int(cnts[r, j]) + int(rng.integers(0, 3))
+    in_sz = int((sdispls + send_counts).max()) + 2
+    out_sz = int((rdispls + recv_counts).max()) + 2
+    ins = [(np.arange(in_sz, dtype=np.int64) + 10_000 * r) for r in range(n)]
+    outs = [np.full(out_sz, -7, dtype=np.int64) for _ in range(n)]
+    assert orc.all_to_all_v(ins, outs, send_counts, sdispls, recv_counts, rdispls, I64) == 0
+    for i in range(n):
+        want = np.full(out_sz, -7, dtype=np.int64)
+        for j in range(n):
+            c = int(send_counts[j, i])
+            want[int(rdispls[i, j]):int(rdispls[i, j]) + c] = ins[j][int(sdispls[j, i]):int(sdispls[j, i]) + c]
+        assert np.array_equal(outs[i], want)
+    bad = recv_counts.copy()
+    bad[0, 1] += 1
+    assert orc.all_to_all_v(ins, outs, send_counts, sdispls, bad, rdispls, I64) == 1

@@ -1,0 +1,244 @@
+"""Pins the oracle's step geometry (rows a10, a11, a16) against the hand tables and invariants held by
+the reference's own unit tests (tests/golden/rhd_nhr_tables.json lists the source lines)."""
+import json
+import os
+
+import pytest
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "rhd_nhr_tables.json")))
+INVALID = 0xFFFFFFFF
+
+
+def _largest_pow2_le(p):
+    hp = 1
+    while hp <= p // 2:
+        hp *= 2
+    return hp
+
+
+def _info_for_virtual(orc, p, v):
+    r = p - _largest_pow2_le(p)
+    carrier = v if v < r else v + r
+    rc, info = orc.rhd_part1(p, carrier)
+    assert rc == 0 and info.virtualRank == v
+    return info
+
+
+def test_step_counts(orc):
+    for n, want in GOLD["rhd_step_num"]:
+        assert orc.lib().orc_rhd_step_num(n) == want
+    for n in range(1, 70):
+        steps, covered = 0, 1
+        while covered < n:
+            covered <<= 1
+            steps += 1
+        assert orc.lib().orc_nhr_step_num(n) == steps
+
+
+def test_round_up(orc):
+    assert orc.lib().orc_round_up(10, 4) == 3
+    assert orc.lib().orc_round_up(8, 4) == 2
+    assert orc.lib().orc_round_up(0, 4) == 0
+    assert orc.lib().orc_round_up(7, 0) == 7
+
+
+def test_rs_and_ag_segment_tables_p8(orc):
+    for key, fn in (("rs_segment_formula_p8", orc.rhd_rs_steps), ("ag_segment_formula_p8", orc.rhd_ag_steps)):
+        for v, k, peer, txs, txe, rxs, rxe in GOLD[key]["rows"]:
+            rc, steps = fn(_info_for_virtual(orc, 8, v))
+            assert rc == 0 and len(steps) == 3
+            s = steps[k]
+            assert (s.step, s.peer, s.txSegStart, s.txSegEnd, s.rxSegStart, s.rxSegEnd) == (k, peer, txs, txe, rxs, rxe)
+            assert s.nSlices == ((8 >> (k + 1)) if key.startswith("rs") else (1 << k))
+
+
+def test_seg_bytes_uniform_table(orc):
+    for us, ue, ss, ts, tu, off, ln in GOLD["seg_bytes_uniform"]["rows"]:
+        assert orc.rhd_seg_bytes_uniform(us, ue, ss, ts, tu) == (off, ln)
+
+
+def test_unit_start_sentinels_and_sigma(orc):
+    for p, j, want in GOLD["unit_start_of_rank"]:
+        assert orc.lib().orc_rhd_unit_start_of_rank(p, j) == want
+    for p in (5, 6, 7, 13):
+        r = p - _largest_pow2_le(p)
+        starts = sorted(orc.lib().orc_rhd_unit_start_of_rank(p, j) for j in range(p))
+        assert starts == list(range(p))                      # sigma is a permutation
+        for t in range(r):                                   # pair members sit next to each other
+            assert orc.lib().orc_rhd_unit_start_of_rank(p, t) == 2 * t
+            assert orc.lib().orc_rhd_unit_start_of_rank(p, t + r) == 2 * t + 1
+        for u in range(p):                                   # owner map inverts sigma
+            assert orc.lib().orc_rhd_unit_start_of_rank(p, orc.lib().orc_rhd_owner_of_unit(p, u)) == u
+
+
+def test_part1_partition(orc):
+    for p in (2, 4, 8, 16):
+        for j in range(p):
+            rc, i = orc.rhd_part1(p, j)
+            assert rc == 0 and i.isPowerOfTwo and i.r == 0 and i.effectiveRankSize == p and not i.inPart1
+            assert i.pairedAlgRank == INVALID and i.virtualRank == j and i.unitStart == j and i.unitCount == 1
+    for p in (5, 6, 7, 9, 13):
+        r = p - _largest_pow2_le(p)
+        for j in range(p):
+            rc, i = orc.rhd_part1(p, j)
+            assert rc == 0 and i.r == r and not i.isPowerOfTwo and i.effectiveRankSize == p - r
+            assert bool(i.inPart1) == (j < 2 * r)
+            assert i.virtualRank == ((j % r) if j < 2 * r else j - r)
+            assert bool(i.isRepresentative) == (j < r)
+
+
+def test_part1_roles_follow_root(orc):
+    for p in (5, 7, 9, 13):
+        r = p - _largest_pow2_le(p)
+        for root in range(p):
+            rep_low = (root < r) if root < 2 * r else True
+            for j in range(p):
+                rc, i = orc.rhd_part1(p, j, root)
+                assert rc == 0
+                if j >= 2 * r:
+                    assert not i.inPart1 and i.unitStart == j and i.unitCount == 1
+                    continue
+                low, t = j < r, j % r
+                assert i.pairedAlgRank == (t + r if low else t)
+                assert bool(i.isRepresentative) == (low if rep_low else not low)
+                if i.isRepresentative:
+                    assert (i.unitStart, i.unitCount) == (2 * t, 2)
+                else:
+                    assert (i.unitStart, i.unitCount) == (2 * t if low else 2 * t + 1, 1)
+            for v in range(p - r):
+                carrier = orc.lib().orc_rhd_alg_rank_of_virtual(p, root, v)
+                rc, ci = orc.rhd_part1(p, carrier, root)
+                assert ci.virtualRank == v
+                assert ci.isRepresentative if v < r else carrier == v + r
+
+
+def test_part1_validation(orc):
+    assert orc.rhd_part1(0, 0)[0] == 1
+    assert orc.rhd_part1(4, 4, 0)[0] == 1
+    assert orc.rhd_part1(4, 0, 4)[0] == 1
+    rc, i = orc.rhd_part1(1, 0)
+    assert rc == 0 and i.isPowerOfTwo and i.effectiveRankSize == 1
+    assert orc.lib().orc_rhd_alg_rank_of_virtual(0, INVALID, 0) == INVALID
+    assert orc.lib().orc_rhd_alg_rank_of_virtual(5, INVALID, 4) == INVALID
+
+
+def test_prepost_seg_modes_p5(orc):
+    for j, pre_full, post_full, pre_w, post_w in GOLD["prepost_seg_mode_p5"]["rows"]:
+        rc, info = orc.rhd_part1(5, j)
+        rc, pre, post = orc.rhd_prepost(info, pre_full, post_full)
+        assert rc == 0
+        assert [pre.nSlices, pre.txSegStart, pre.txSegEnd, pre.rxSegStart, pre.rxSegEnd] == pre_w
+        assert [post.nSlices, post.txSegStart, post.txSegEnd, post.rxSegStart, post.rxSegEnd] == post_w
+    for p in (2, 4, 8, 16):   # powers of two: both steps empty
+        for j in range(p):
+            rc, info = orc.rhd_part1(p, j)
+            rc, pre, post = orc.rhd_prepost(info, True, True)
+            assert rc == 0 and pre.nSlices == 0 and post.nSlices == 0 and pre.peer == INVALID
+
+
+@pytest.mark.parametrize("p", [2, 3, 4, 5, 6, 7, 9, 17, 32, 48, 64])
+def test_rs_steps_deliver_every_contribution_once(orc, p):
+    """Counting simulation: every rank contributes +1 to every unit; after PRE(FULL) and the MAIN
+    steps each unit holds exactly p at its owner (the invariant of the reference's RsFinalState)."""
+    r = p - _largest_pow2_le(p)
+    P = p - r
+    L = orc.lib()
+    hold = [[1] * p for _ in range(p)]
+    for t in range(r):
+        rc, minfo = orc.rhd_part1(p, t + r)
+        rc, pre, post = orc.rhd_prepost(minfo, True, False)
+        assert pre.peer == t and (pre.txSegStart, pre.txSegEnd) == (0, p)
+        for u in range(p):
+            hold[t][u] += hold[t + r][u]
+            hold[t + r][u] = 0
+    steps = [orc.rhd_rs_steps(_info_for_virtual(orc, p, v))[1] for v in range(P)]
+    n_steps = L.orc_rhd_step_num(P)
+    for k in range(n_steps):
+        sent = [[0] * p for _ in range(p)]
+        for v in range(P):
+            s, phys = steps[v][k], L.orc_rhd_alg_rank_of_virtual(p, INVALID, v)
+            ps = steps[s.peer][k]   # mirror: my tx is the peer's rx
+            assert ps.peer == v and (ps.rxSegStart, ps.rxSegEnd) == (s.txSegStart, s.txSegEnd)
+            for u in range(s.txSegStart, s.txSegEnd):
+                sent[phys][u], hold[phys][u] = hold[phys][u], 0
+        for v in range(P):
+            s, phys = steps[v][k], L.orc_rhd_alg_rank_of_virtual(p, INVALID, v)
+            peer = L.orc_rhd_alg_rank_of_virtual(p, INVALID, s.peer)
+            for u in range(s.rxSegStart, s.rxSegEnd):
+                hold[phys][u] += sent[peer][u]
+    for u in range(p):
+        v = u // 2 if u < 2 * r else u - r
+        assert hold[L.orc_rhd_alg_rank_of_virtual(p, INVALID, v)][u] == p
+
+
+@pytest.mark.parametrize("p", [2, 3, 5, 6, 7, 9, 17, 32])
+def test_ag_steps_mirror_rs_steps(orc, p):
+    r = p - _largest_pow2_le(p)
+    P = p - r
+    n = orc.lib().orc_rhd_step_num(P)
+    for v in range(P):
+        info = _info_for_virtual(orc, p, v)
+        rs, ag = orc.rhd_rs_steps(info)[1], orc.rhd_ag_steps(info)[1]
+        for k in range(n):
+            a, s = ag[k], rs[n - 1 - k]
+            assert a.peer == s.peer
+            assert (a.txSegStart, a.txSegEnd, a.rxSegStart, a.rxSegEnd) == (s.rxSegStart, s.rxSegEnd, s.txSegStart, s.txSegEnd)
+
+
+def test_step_validation(orc):
+    import oracle
+    info = oracle.RhdPart1()
+    assert orc.rhd_rs_steps(info)[0] == 1
+    info.effectiveRankSize, info.r, info.virtualRank = 4, 0, 4
+    assert orc.rhd_rs_steps(info)[0] == 1 and orc.rhd_ag_steps(info)[0] == 1
+    info.effectiveRankSize, info.r, info.virtualRank = 6, 1, 5
+    assert orc.rhd_rs_steps(info)[0] == 1
+    info.effectiveRankSize, info.r, info.virtualRank = 4, 4, 0
+    assert orc.rhd_rs_steps(info)[0] == 1
+
+
+def test_nhr_hand_table_and_totals(orc):
+    for row in GOLD["nhr_steps_n4_rank0"]:
+        rc, to, frm, tx, rx = orc.nhr_step_info(4, 0, row["step"])
+        assert rc == 0 and (to, frm, tx, rx) == (row["toRank"], row["fromRank"], row["tx"], row["rx"])
+    for n in (1, 2, 3, 4, 5, 6, 8, 9, 16, 33, 64):
+        steps = orc.lib().orc_nhr_step_num(n)
+        for me in range(n):
+            total = 0
+            for s in range(steps):
+                rc, to, frm, tx, rx = orc.nhr_step_info(n, me, s)
+                assert rc == 0 and to < n and frm < n and all(i < n for i in tx + rx)
+                total += len(tx)
+            assert total == n - 1
+
+
+def test_rhd_tail_loop_plan(orc):
+    g = GOLD["rhd_tail_one_mib_72_ranks"]
+    sel = orc.lib().orc_rhd_select_loop_count
+    processed, tail = 0, 0
+    while processed < g["totalCount"]:
+        c = sel(g["totalCount"] - processed, g["maxCountPerLoop"], g["rankAlign"])
+        if c < g["rankAlign"]:
+            tail = c
+        processed += c
+    assert processed == g["totalCount"] and tail == g["tailCount"]
+    for ranks in (2, 3, 6, 12, 16, 24, 72):       # every element processed exactly once
+        cap = 3 * ranks
+        for total in range(0, 300):
+            done = 0
+            while done < total:
+                c = sel(total - done, cap, ranks)
+                assert 0 < c <= cap
+                assert c == total - done if c < ranks else c % ranks == 0
+                done += c
+            assert done == total
+
+
+def test_local_copy_slices_merges_contiguous_runs(orc):
+    # three contiguous slices then a gap then one more: two copies
+    got = orc.local_copy_slices([0, 16, 32, 100], [64, 80, 96, 400], [16, 16, 16, 8])
+    assert got == [(0, 64, 48), (100, 400, 8)]
+    # source contiguous but destination not: no merge
+    got = orc.local_copy_slices([0, 16], [0, 32], [16, 16])
+    assert got == [(0, 0, 16), (16, 32, 16)]
+    assert orc.local_copy_slices([5], [9], [7]) == [(5, 9, 7)]
