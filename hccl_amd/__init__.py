@@ -1,0 +1,296 @@
+"""ctypes bindings of libhccl_amd.so, shaped like the reference's hccl4py.ops
+(reference experimental/eco_system/python/hccl4py/ops.py:48-80): every collective takes
+``(hccl_comm, send_buf, recv_buf, count, data_type, reduce_op, stream)`` with element counts and
+device pointers, returns the HcclResult code and raises :class:`HcclError` when it is not zero.
+
+The library is loaded from ``hccl_amd/libhccl_amd.so`` (built by ``make -C hccl_amd/csrc``).  There
+is no fallback: if the shared object is missing the import of any collective fails loudly.
+"""
+import ctypes
+import enum
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhccl_amd.so")
+MAX_RANKS = 64
+
+
+class HcclDataType(enum.IntEnum):
+    INT8 = 0
+    INT16 = 1
+    INT32 = 2
+    FP16 = 3
+    FP32 = 4
+    INT64 = 5
+    UINT64 = 6
+    UINT8 = 7
+    UINT16 = 8
+    UINT32 = 9
+    FP64 = 10
+    BFP16 = 11
+    INT128 = 12
+    HIF8 = 14
+    FP8E4M3 = 15
+    FP8E5M2 = 16
+    FP8E8M0 = 17
+    RESERVED = 255
+
+
+class HcclReduceOp(enum.IntEnum):
+    SUM = 0
+    PROD = 1
+    MAX = 2
+    MIN = 3
+    RESERVED = 4
+
+
+class HcclResult(enum.IntEnum):
+    SUCCESS = 0
+    E_PARA = 1
+    E_PTR = 2
+    E_MEMORY = 3
+    E_INTERNAL = 4
+    E_NOT_SUPPORT = 5
+    E_TIMEOUT = 9
+    E_RUNTIME = 15
+
+
+class Algo(enum.IntEnum):
+    MESH = 0
+    RING = 1
+    RHD = 2
+    NHR = 3
+    ORDER_PRESERVED = 4
+    AIV_MESH = 5
+
+
+class OpKind(enum.IntEnum):
+    ALL_REDUCE = 0
+    REDUCE_SCATTER = 1
+
+
+DTYPE_SIZE = {0: 1, 1: 2, 2: 4, 3: 2, 4: 4, 5: 8, 6: 8, 7: 1, 8: 2, 9: 4, 10: 8, 11: 2, 12: 16, 14: 1, 15: 1,
+              16: 1, 17: 1}
+
+
+class HcclError(RuntimeError):
+    def __init__(self, code, where):
+        self.code = int(code)
+        super().__init__("%s failed with HcclResult %d (%s)" % (where, self.code, error_string(self.code)))
+
+
+def build(jobs=8):
+    """Compiles the gfx950 kernels and the host layer into libhccl_amd.so."""
+    subprocess.check_call(["make", "-s", "-C", os.path.join(_HERE, "csrc"), "-j%d" % jobs])
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """Loads libhccl_amd.so; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("%s is missing: run `make -C hccl_amd/csrc` (or hccl_amd.build()) first" % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    vp, u64, u32, i32 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_int
+    L.HcclAllReduce.argtypes = [vp, vp, u64, i32, i32, vp, vp]
+    L.HcclReduceScatter.argtypes = [vp, vp, u64, i32, i32, vp, vp]
+    L.HcclAllGather.argtypes = [vp, vp, u64, i32, vp, vp]
+    L.HcclAllGatherV.argtypes = [vp, u64, vp, vp, vp, i32, vp, vp]
+    L.HcclAlltoAllV.argtypes = [vp, vp, vp, i32, vp, vp, vp, i32, vp, vp]
+    L.HcclCommInitAll.argtypes = [u32, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(vp)]
+    L.HcclGetRootInfo.argtypes = [vp]
+    L.HcclCommInitRootInfo.argtypes = [u32, vp, u32, ctypes.POINTER(vp)]
+    L.HcclCommDestroy.argtypes = [vp]
+    L.HcclGetRankSize.argtypes = [vp, ctypes.POINTER(u32)]
+    L.HcclGetRankId.argtypes = [vp, ctypes.POINTER(u32)]
+    L.HcclGetErrorString.argtypes = [i32]
+    L.HcclGetErrorString.restype = ctypes.c_char_p
+    L.HcclGroupStart.argtypes = []
+    L.HcclGroupEnd.argtypes = []
+    L.HcclAmdSetAlgo.argtypes = [vp, i32, i32]
+    L.HcclAmdGetAlgo.argtypes = [vp, i32, ctypes.POINTER(i32)]
+    L.HcclAmdGetFoldProgram.argtypes = [i32, i32, u32, u32, vp, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
+    for name in ("HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV",
+                 "HcclCommInitAll", "HcclGetRootInfo", "HcclCommInitRootInfo", "HcclCommDestroy", "HcclGetRankSize",
+                 "HcclGetRankId", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
+                 "HcclAmdGetFoldProgram"):
+        getattr(L, name).restype = ctypes.c_int
+    _lib = L
+    return L
+
+
+def error_string(code):
+    return lib().HcclGetErrorString(int(code)).decode()
+
+
+def check(code, where):
+    if int(code) != 0:
+        raise HcclError(code, where)
+    return int(code)
+
+
+def _as_ptr(buf):
+    """Accepts None, an int address, a ctypes pointer, or anything with data_ptr() (torch tensors)."""
+    if buf is None:
+        return None
+    if hasattr(buf, "data_ptr"):
+        return ctypes.c_void_p(buf.data_ptr())
+    if isinstance(buf, int):
+        return ctypes.c_void_p(buf)
+    return ctypes.cast(buf, ctypes.c_void_p)
+
+
+def _as_stream(stream):
+    if stream is None:
+        return None
+    if hasattr(stream, "cuda_stream"):
+        return ctypes.c_void_p(stream.cuda_stream)
+    return ctypes.c_void_p(int(stream))
+
+
+def u64_array(values):
+    """Builds the host uint64 array the V-collectives take; pass the result to skip per-call conversion."""
+    vals = [int(v) for v in values]
+    return (ctypes.c_uint64 * len(vals))(*vals)
+
+
+def _u64_array(values, n):
+    if isinstance(values, ctypes.Array) and values._type_ is ctypes.c_uint64:
+        if len(values) != n:
+            raise ValueError("expected %d entries, got %d" % (n, len(values)))
+        return values
+    vals = [int(v) for v in values]
+    if len(vals) != n:
+        raise ValueError("expected %d entries, got %d" % (n, len(vals)))
+    return (ctypes.c_uint64 * n)(*vals)
+
+
+# ---- lifecycle ------------------------------------------------------------------------------------
+def comm_init_all(ndev, devices=None):
+    """Creates the ``ndev`` communicators of one loopback world; element r has rank r."""
+    comms = (ctypes.c_void_p * ndev)()
+    dev = None
+    if devices is not None:
+        dev = (ctypes.c_int32 * ndev)(*devices)
+    check(lib().HcclCommInitAll(ndev, dev, comms), "HcclCommInitAll")
+    return [ctypes.c_void_p(c) for c in comms]
+
+
+def get_root_info():
+    buf = ctypes.create_string_buffer(4108)
+    check(lib().HcclGetRootInfo(buf), "HcclGetRootInfo")
+    return buf
+
+
+def comm_init_root_info(n_ranks, root_info, rank):
+    comm = ctypes.c_void_p()
+    check(lib().HcclCommInitRootInfo(n_ranks, root_info, rank, ctypes.byref(comm)), "HcclCommInitRootInfo")
+    return comm
+
+
+def comm_destroy(hccl_comm):
+    return check(lib().HcclCommDestroy(hccl_comm), "HcclCommDestroy")
+
+
+def get_rank_size(hccl_comm):
+    v = ctypes.c_uint32()
+    check(lib().HcclGetRankSize(hccl_comm, ctypes.byref(v)), "HcclGetRankSize")
+    return v.value
+
+
+def get_rank_id(hccl_comm):
+    v = ctypes.c_uint32()
+    check(lib().HcclGetRankId(hccl_comm, ctypes.byref(v)), "HcclGetRankId")
+    return v.value
+
+
+def group_start():
+    return check(lib().HcclGroupStart(), "HcclGroupStart")
+
+
+def group_end():
+    return check(lib().HcclGroupEnd(), "HcclGroupEnd")
+
+
+class group:
+    """``with hccl_amd.group():`` -- queue the per-rank calls of one host thread without blocking."""
+
+    def __enter__(self):
+        group_start()
+        return self
+
+    def __exit__(self, *exc):
+        group_end()
+        return False
+
+
+def set_algo(hccl_comm, op_kind, algo):
+    return check(lib().HcclAmdSetAlgo(hccl_comm, int(op_kind), int(algo)), "HcclAmdSetAlgo")
+
+
+def get_algo(hccl_comm, op_kind):
+    v = ctypes.c_int()
+    check(lib().HcclAmdGetAlgo(hccl_comm, int(op_kind), ctypes.byref(v)), "HcclAmdGetAlgo")
+    return Algo(v.value)
+
+
+def fold_programs(op_kind, algo, rank_size):
+    """Host-only: the byte programs (one per segment) that fix the reduction order."""
+    L = lib()
+    out = []
+    seg, count = 0, 1
+    while seg < count:
+        buf = (ctypes.c_uint8 * 512)()
+        ln, cnt = ctypes.c_uint32(), ctypes.c_uint32()
+        check(L.HcclAmdGetFoldProgram(int(op_kind), int(algo), rank_size, seg, buf, 512, ctypes.byref(ln),
+                                      ctypes.byref(cnt)), "HcclAmdGetFoldProgram")
+        count = cnt.value
+        out.append(bytes(buf[:ln.value]))
+        seg += 1
+    return out
+
+
+# ---- collectives (names and argument order of hccl4py.ops) ----------------------------------------
+def all_reduce(hccl_comm, send_buf, recv_buf, count, data_type=HcclDataType.FP32, reduce_op=HcclReduceOp.SUM,
+               stream=None):
+    code = lib().HcclAllReduce(_as_ptr(send_buf), _as_ptr(recv_buf), ctypes.c_uint64(count), int(data_type),
+                               int(reduce_op), hccl_comm, _as_stream(stream))
+    return check(code, "HcclAllReduce")
+
+
+def reduce_scatter(hccl_comm, send_buf, recv_buf, recv_count, data_type=HcclDataType.FP32,
+                   reduce_op=HcclReduceOp.SUM, stream=None):
+    code = lib().HcclReduceScatter(_as_ptr(send_buf), _as_ptr(recv_buf), ctypes.c_uint64(recv_count), int(data_type),
+                                   int(reduce_op), hccl_comm, _as_stream(stream))
+    return check(code, "HcclReduceScatter")
+
+
+def all_gather(hccl_comm, send_buf, recv_buf, send_count, data_type=HcclDataType.FP32, stream=None):
+    code = lib().HcclAllGather(_as_ptr(send_buf), _as_ptr(recv_buf), ctypes.c_uint64(send_count), int(data_type),
+                               hccl_comm, _as_stream(stream))
+    return check(code, "HcclAllGather")
+
+
+def all_gather_v(hccl_comm, send_buf, send_count, recv_buf, recv_counts, recv_displs,
+                 data_type=HcclDataType.FP32, stream=None):
+    n = get_rank_size(hccl_comm)
+    counts = _u64_array(recv_counts, n)
+    displs = _u64_array(recv_displs, n)
+    code = lib().HcclAllGatherV(_as_ptr(send_buf), ctypes.c_uint64(send_count), _as_ptr(recv_buf), counts, displs,
+                                int(data_type), hccl_comm, _as_stream(stream))
+    return check(code, "HcclAllGatherV")
+
+
+def all_to_all_v(hccl_comm, send_buf, send_counts, sdispls, send_type, recv_buf, recv_counts, rdispls, recv_type,
+                 stream=None):
+    n = get_rank_size(hccl_comm)
+    code = lib().HcclAlltoAllV(_as_ptr(send_buf), _u64_array(send_counts, n), _u64_array(sdispls, n), int(send_type),
+                               _as_ptr(recv_buf), _u64_array(recv_counts, n), _u64_array(rdispls, n), int(recv_type),
+                               hccl_comm, _as_stream(stream))
+    return check(code, "HcclAlltoAllV")

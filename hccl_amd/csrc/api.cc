@@ -1,0 +1,1233 @@
+// Host layer of the loopback data plane: the C ABI of include/hccl.h over HIP streams.
+//
+// What the reference spreads over op entry / selector / executor / template / wrapper
+// (src/ops/<op>/<op>.cc -> op_common.cc Selector + HcclExecOp -> executor -> template ->
+// alg_data_trans_wrapper.cc) collapses here to: argument checks with the reference's return codes,
+// a rendezvous of the N per-rank calls, and one fused kernel launch per collective.
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <condition_variable>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "dataplane.h"
+#include "fold_plan.h"
+#include "hccl.h"
+
+namespace hccl_amd {
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// Logging: HCCL_AMD_LOG_LEVEL = 0 (silent), 1 (errors, default), 2 (info).
+// ---------------------------------------------------------------------------------------------
+int LogLevel()
+{
+    static int level = [] {
+        const char* s = getenv("HCCL_AMD_LOG_LEVEL");
+        return s ? atoi(s) : 1;
+    }();
+    return level;
+}
+
+void Log(int level, const char* fmt, ...)
+{
+    if (level > LogLevel()) {
+        return;
+    }
+    va_list ap;
+    va_start(ap, fmt);
+    fprintf(stderr, level == 1 ? "[hccl_amd][ERROR] " : "[hccl_amd][INFO] ");
+    vfprintf(stderr, fmt, ap);
+    fputc('\n', stderr);
+    va_end(ap);
+}
+
+#define HIP_OK(expr)                                                                          \
+    do {                                                                                      \
+        hipError_t e_ = (expr);                                                               \
+        if (e_ != hipSuccess) {                                                               \
+            Log(1, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
+            return HCCL_E_RUNTIME;                                                            \
+        }                                                                                     \
+    } while (0)
+
+// Element sizes, indexed by HcclDataType (reference src/ops/op_common/inc/alg_param.h:55-73).
+uint32_t DataTypeSize(HcclDataType t)
+{
+    static const uint32_t sizes[18] = {1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16, 2, 1, 1, 1, 1};
+    int v = static_cast<int>(t);
+    return (v >= 0 && v < 18) ? sizes[v] : 0;
+}
+
+bool IsValidDataType(HcclDataType t)
+{
+    int v = static_cast<int>(t);
+    return v >= 0 && v <= 17 && v != 13;   // 13 is a reserved gap, 255 is RESERVED
+}
+
+// Reference op_common.cc:4311-4321.
+HcclResult CheckCount(uint64_t count)
+{
+    if (count > HCCL_SYS_MAX_COUNT) {
+        Log(1, "count %llu exceeds the supported maximum %llu", (unsigned long long)count,
+            (unsigned long long)HCCL_SYS_MAX_COUNT);
+        return HCCL_E_PARA;
+    }
+    return HCCL_SUCCESS;
+}
+
+// Reference op_common.cc:4323-4364.
+HcclResult CheckDataType(HcclDataType t, bool needReduce)
+{
+    bool notValid = !IsValidDataType(t);
+    if (needReduce) {
+        switch (t) {
+            case HCCL_DATA_TYPE_UINT8:
+            case HCCL_DATA_TYPE_UINT16:
+            case HCCL_DATA_TYPE_UINT32:
+            case HCCL_DATA_TYPE_INT128:
+            case HCCL_DATA_TYPE_HIF8:
+            case HCCL_DATA_TYPE_FP8E4M3:
+            case HCCL_DATA_TYPE_FP8E5M2:
+            case HCCL_DATA_TYPE_FP8E8M0:
+                notValid = true;
+                break;
+            default:
+                break;
+        }
+    } else if (t == HCCL_DATA_TYPE_INT128) {
+        notValid = true;
+    }
+    if (notValid) {
+        Log(1, "data type %d is not supported (%s)", static_cast<int>(t), needReduce ? "reduce" : "copy");
+        return HCCL_E_NOT_SUPPORT;
+    }
+    return HCCL_SUCCESS;
+}
+
+// Reference op_common.cc:4392-4413: PROD exists for int8, int32, int64, uint64, fp16, fp32, fp64 only.
+HcclResult CheckReduceOp(HcclDataType t, HcclReduceOp op)
+{
+    if (static_cast<int>(op) < 0 || static_cast<int>(op) >= static_cast<int>(HCCL_REDUCE_RESERVED)) {
+        Log(1, "reduce op %d is invalid", static_cast<int>(op));
+        return HCCL_E_PARA;
+    }
+    if (op == HCCL_REDUCE_PROD) {
+        switch (t) {
+            case HCCL_DATA_TYPE_INT8:
+            case HCCL_DATA_TYPE_INT32:
+            case HCCL_DATA_TYPE_INT64:
+            case HCCL_DATA_TYPE_UINT64:
+            case HCCL_DATA_TYPE_FP16:
+            case HCCL_DATA_TYPE_FP32:
+            case HCCL_DATA_TYPE_FP64:
+                break;
+            default:
+                Log(1, "PROD is not supported for data type %d", static_cast<int>(t));
+                return HCCL_E_NOT_SUPPORT;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// ---------------------------------------------------------------------------------------------
+// World, communicators, pending collectives
+// ---------------------------------------------------------------------------------------------
+enum class OpType { ALL_REDUCE, REDUCE_SCATTER, ALL_GATHER, ALL_GATHER_V, ALL_TO_ALL_V };
+
+const char* OpName(OpType t)
+{
+    switch (t) {
+        case OpType::ALL_REDUCE: return "AllReduce";
+        case OpType::REDUCE_SCATTER: return "ReduceScatter";
+        case OpType::ALL_GATHER: return "AllGather";
+        case OpType::ALL_GATHER_V: return "AllGatherV";
+        default: return "AlltoAllV";
+    }
+}
+
+struct RankArgs {
+    const void* send = nullptr;
+    void* recv = nullptr;
+    hipStream_t stream = nullptr;
+    bool arrived = false;
+    std::vector<uint64_t> var;   // AllGatherV: counts | displs ; AlltoAllV: sendCounts | recvCounts | sdispls | rdispls
+};
+
+struct PendingOp {
+    OpType type;
+    HcclDataType dtype;
+    HcclReduceOp op = HCCL_REDUCE_RESERVED;
+    uint64_t count = 0;
+    uint32_t arrived = 0;
+    bool done = false;
+    HcclResult result = HCCL_SUCCESS;
+    std::vector<RankArgs> ranks;
+};
+
+struct DevicePlan {
+    uint8_t* dev = nullptr;
+    uint32_t nProg = 0;
+    bool segmentsAreSubs = false;
+};
+
+constexpr uint32_t kMagic = 0x48434C41u;   // "HCLA"
+constexpr int kStagingSlots = 4;
+
+struct World;
+struct Comm {
+    uint32_t magic = kMagic;
+    World* world = nullptr;
+    uint32_t rank = 0;
+    bool destroyed = false;
+};
+
+struct World {
+    std::mutex mu;
+    std::condition_variable cv;
+    uint64_t id = 0;
+    uint32_t n = 0;
+    int device = 0;
+    uint32_t joined = 0;
+    uint32_t destroyed = 0;
+    std::vector<std::unique_ptr<Comm>> comms;
+    HcclAmdAlgo algo[HCCL_AMD_OP_COUNT] = {HCCL_AMD_ALGO_MESH, HCCL_AMD_ALGO_MESH};
+    std::deque<std::shared_ptr<PendingOp>> pending;
+    uint64_t baseSeq = 0;
+    uint64_t nextSeq[kMaxRanks] = {};
+    std::map<uint32_t, DevicePlan> plans;
+    std::vector<hipEvent_t> eventPool;
+    hipEvent_t doneEvent = nullptr;
+    // AlltoAllV tables
+    uint8_t* a2aDev = nullptr;
+    uint64_t* a2aHost[kStagingSlots] = {};
+    hipEvent_t a2aSlotFree[kStagingSlots] = {};
+    bool a2aSlotUsed[kStagingSlots] = {};
+    uint32_t a2aNext = 0;
+    uint32_t reduceBlocks = 2048;
+    uint32_t copyBlocks = 2048;
+
+    ~World()
+    {
+        for (auto& kv : plans) {
+            if (kv.second.dev) (void)hipFree(kv.second.dev);
+        }
+        for (hipEvent_t e : eventPool) (void)hipEventDestroy(e);
+        if (doneEvent) (void)hipEventDestroy(doneEvent);
+        if (a2aDev) (void)hipFree(a2aDev);
+        for (int s = 0; s < kStagingSlots; ++s) {
+            if (a2aHost[s]) (void)hipHostFree(a2aHost[s]);
+            if (a2aSlotFree[s]) (void)hipEventDestroy(a2aSlotFree[s]);
+        }
+    }
+};
+
+std::mutex g_registryMu;
+std::map<uint64_t, std::unique_ptr<World>> g_worlds;
+uint64_t g_nextWorldId = 1;
+thread_local int t_groupDepth = 0;
+
+uint32_t EnvU32(const char* name, uint32_t dflt)
+{
+    const char* s = getenv(name);
+    if (!s || !*s) {
+        return dflt;
+    }
+    long v = atol(s);
+    return v > 0 ? static_cast<uint32_t>(v) : dflt;
+}
+
+bool ParseAlgoName(const std::string& s, HcclAmdAlgo* algo)
+{
+    static const struct { const char* name; HcclAmdAlgo algo; } table[] = {
+        {"mesh", HCCL_AMD_ALGO_MESH}, {"ring", HCCL_AMD_ALGO_RING}, {"rhd", HCCL_AMD_ALGO_RHD},
+        {"nhr", HCCL_AMD_ALGO_NHR}, {"order_preserved", HCCL_AMD_ALGO_ORDER_PRESERVED},
+        {"aiv_mesh", HCCL_AMD_ALGO_AIV_MESH}};
+    for (const auto& e : table) {
+        if (s == e.name) {
+            *algo = e.algo;
+            return true;
+        }
+    }
+    return false;
+}
+
+// HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr"
+void ApplyAlgoEnv(World* w)
+{
+    const char* env = getenv("HCCL_AMD_ALGO");
+    if (!env) {
+        return;
+    }
+    std::string s(env);
+    size_t pos = 0;
+    while (pos < s.size()) {
+        size_t end = s.find(';', pos);
+        if (end == std::string::npos) end = s.size();
+        std::string item = s.substr(pos, end - pos);
+        size_t eq = item.find('=');
+        if (eq != std::string::npos) {
+            std::string key = item.substr(0, eq), val = item.substr(eq + 1);
+            HcclAmdAlgo a;
+            if (ParseAlgoName(val, &a)) {
+                if (key == "allreduce" && a != HCCL_AMD_ALGO_AIV_MESH) w->algo[HCCL_AMD_OP_ALL_REDUCE] = a;
+                if (key == "reducescatter") w->algo[HCCL_AMD_OP_REDUCE_SCATTER] = a;
+            } else {
+                Log(1, "HCCL_AMD_ALGO: unknown algorithm '%s'", val.c_str());
+            }
+        }
+        pos = end + 1;
+    }
+}
+
+std::unique_ptr<World> NewWorld(uint32_t n)
+{
+    auto w = std::make_unique<World>();
+    w->n = n;
+    w->comms.resize(n);
+    if (hipGetDevice(&w->device) != hipSuccess) {
+        w->device = 0;
+    }
+    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 2048);
+    w->copyBlocks = EnvU32("HCCL_AMD_COPY_BLOCKS", 2048);
+    ApplyAlgoEnv(w.get());
+    return w;
+}
+
+Comm* AsComm(HcclComm h)
+{
+    Comm* c = static_cast<Comm*>(h);
+    if (c == nullptr || c->magic != kMagic || c->destroyed || c->world == nullptr) {
+        return nullptr;
+    }
+    return c;
+}
+
+// Reference src/common/param_check.cc:153-162.
+HcclResult CheckUserRank(const Comm* c)
+{
+    if (c->rank >= c->world->n) {
+        Log(1, "rank %u is out of range [0, %u)", c->rank, c->world->n);
+        return HCCL_E_PARA;
+    }
+    return HCCL_SUCCESS;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Device resources
+// ---------------------------------------------------------------------------------------------
+HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DevicePlan* out)
+{
+    uint32_t key = static_cast<uint32_t>(kind) * 64 + static_cast<uint32_t>(algo);
+    auto it = w->plans.find(key);
+    if (it != w->plans.end()) {
+        *out = it->second;
+        return HCCL_SUCCESS;
+    }
+    FoldPlan plan;
+    HcclResult rc = BuildFoldPlan(kind, algo, w->n, &plan);
+    if (rc != HCCL_SUCCESS) {
+        return rc;
+    }
+    std::vector<uint8_t> image(plan.programs.size() * kProgStride, kTokEnd);
+    for (size_t s = 0; s < plan.programs.size(); ++s) {
+        memcpy(image.data() + s * kProgStride, plan.programs[s].data(), plan.programs[s].size());
+    }
+    DevicePlan dp;
+    dp.nProg = static_cast<uint32_t>(plan.programs.size());
+    dp.segmentsAreSubs = plan.segmentsAreSubs;
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&dp.dev), image.size()));
+    HIP_OK(hipMemcpy(dp.dev, image.data(), image.size(), hipMemcpyHostToDevice));
+    w->plans[key] = dp;
+    *out = dp;
+    return HCCL_SUCCESS;
+}
+
+HcclResult TakeEvent(World* w, hipEvent_t* ev)
+{
+    if (!w->eventPool.empty()) {
+        *ev = w->eventPool.back();
+        w->eventPool.pop_back();
+        return HCCL_SUCCESS;
+    }
+    HIP_OK(hipEventCreateWithFlags(ev, hipEventDisableTiming));
+    return HCCL_SUCCESS;
+}
+
+size_t A2aTableBytes(uint32_t n) { return static_cast<size_t>(n) * n * sizeof(uint64_t); }
+
+// Device bytes of one slot: three u64 tables, rowStart (n + 1) and segEnd (n * n) as u32, 256-byte padded.
+size_t A2aSlotBytes(uint32_t n)
+{
+    size_t bytes = 3 * A2aTableBytes(n) + (static_cast<size_t>(n) * n + n + 1) * sizeof(uint32_t);
+    return (bytes + 255) & ~static_cast<size_t>(255);
+}
+
+// Calls may be in flight on different streams, so each of the kStagingSlots calls owns its own host
+// staging area and device tables until the event recorded behind its copy kernel has fired.
+HcclResult EnsureA2aBuffers(World* w)
+{
+    if (w->a2aDev != nullptr) {
+        return HCCL_SUCCESS;
+    }
+    size_t tab = A2aTableBytes(w->n);
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&w->a2aDev), kStagingSlots * A2aSlotBytes(w->n)));
+    for (int s = 0; s < kStagingSlots; ++s) {
+        HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&w->a2aHost[s]), 3 * tab, hipHostMallocDefault));
+        HIP_OK(hipEventCreateWithFlags(&w->a2aSlotFree[s], hipEventDisableTiming));
+    }
+    return HCCL_SUCCESS;
+}
+
+uint32_t AlignUnitOf(uint64_t bits)
+{
+    uint32_t low = static_cast<uint32_t>(bits) | 16u;
+    return low & (0u - low);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Launches.  `s` is the stream the fused kernel runs on.
+// ---------------------------------------------------------------------------------------------
+uint32_t BlocksPerSub(const World* w, uint64_t subLen, uint32_t esz, uint64_t nSubTotal)
+{
+    uint64_t vecs = (subLen * esz + 15) / 16;
+    uint64_t maxUseful = (vecs + 255) / 256;
+    if (maxUseful == 0) maxUseful = 1;
+    uint64_t want = (w->reduceBlocks + nSubTotal - 1) / nSubTotal;
+    if (want == 0) want = 1;
+    return static_cast<uint32_t>(want < maxUseful ? want : maxUseful);
+}
+
+HcclResult LaunchOneReduce(World* w, ReduceArgs& a, HcclDataType dtype, HcclReduceOp op, hipStream_t s)
+{
+    uint32_t esz = DataTypeSize(dtype);
+    uint64_t bits = 0;
+    uint32_t nSrc = w->n;
+    for (uint32_t r = 0; r < nSrc; ++r) bits |= reinterpret_cast<uint64_t>(a.src[r]);
+    if (a.dstOwn) {
+        for (uint32_t g = 0; g < a.nGroup; ++g) bits |= reinterpret_cast<uint64_t>(a.dst[g]);
+    } else {
+        for (uint32_t d = 0; d < a.nDst; ++d) bits |= reinterpret_cast<uint64_t>(a.dst[d]);
+    }
+    if (a.nGroup > 1) bits |= a.srcGroupStride * esz | a.dstGroupStride * esz;
+    if (a.nSub > 1) bits |= a.subLen * esz;
+    a.vecOk = (bits & 15u) == 0 ? 1u : 0u;
+    uint64_t subs = static_cast<uint64_t>(a.nGroup) * a.nSub;
+    uint64_t longest = a.groupLen;   // the last sub-segment takes what the others leave
+    if (a.nSub > 1) {
+        uint64_t before = a.subLen * (a.nSub - 1);
+        uint64_t last = a.groupLen > before ? a.groupLen - before : 0;
+        longest = last > a.subLen ? last : a.subLen;
+    }
+    a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs);
+    uint64_t blocks = subs * a.blocksPerSub;
+    if (blocks == 0 || blocks > 0x7FFFFFFFull) {
+        return HCCL_E_INTERNAL;
+    }
+    HIP_OK(LaunchReduce(a, dtype, op, static_cast<uint32_t>(blocks), s));
+    return HCCL_SUCCESS;
+}
+
+HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    HcclAmdAlgo algo = w->algo[HCCL_AMD_OP_ALL_REDUCE];
+    DevicePlan plan;
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_ALL_REDUCE, algo, &plan);
+    if (rc != HCCL_SUCCESS) {
+        return rc;
+    }
+    const uint32_t esz = DataTypeSize(p.dtype);
+    ReduceArgs a{};
+    for (uint32_t r = 0; r < n; ++r) {
+        a.src[r] = p.ranks[r].send;
+        a.dst[r] = p.ranks[r].recv;
+    }
+    a.prog = plan.dev;
+    a.nDst = n;
+    a.dstOwn = 0;
+    a.nGroup = 1;
+    if (plan.nProg == 1) {
+        a.total = a.groupLen = a.subLen = p.count;
+        a.nSub = 1;
+        return LaunchOneReduce(w, a, p.dtype, p.op, s);
+    }
+    a.nSub = n;
+    a.progSubStride = 1;
+    if (algo == HCCL_AMD_ALGO_RHD) {
+        // Aligned prefix in n uniform units, then a remainder shorter than n with one element per unit
+        // (reference ins_v2_all_reduce_sequence_rhd_tail.h:98-113, staging buffer taken as unbounded).
+        uint64_t unit = p.count / n;
+        uint64_t prefix = unit * n;
+        if (unit > 0) {
+            a.total = a.groupLen = prefix;
+            a.subLen = unit;
+            rc = LaunchOneReduce(w, a, p.dtype, p.op, s);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+        }
+        if (p.count > prefix) {
+            for (uint32_t r = 0; r < n; ++r) {
+                a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + prefix * esz;
+                a.dst[r] = static_cast<uint8_t*>(p.ranks[r].recv) + prefix * esz;
+            }
+            a.total = a.groupLen = p.count - prefix;
+            a.subLen = 1;
+            return LaunchOneReduce(w, a, p.dtype, p.op, s);
+        }
+        return HCCL_SUCCESS;
+    }
+    // NHR: slices of ceil(count / n) elements (reference two_shot.cc:184 slicing rule).
+    a.total = a.groupLen = p.count;
+    a.subLen = (p.count + n - 1) / n;
+    return LaunchOneReduce(w, a, p.dtype, p.op, s);
+}
+
+HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    HcclAmdAlgo algo = w->algo[HCCL_AMD_OP_REDUCE_SCATTER];
+    DevicePlan plan;
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, algo, &plan);
+    if (rc != HCCL_SUCCESS) {
+        return rc;
+    }
+    ReduceArgs a{};
+    for (uint32_t r = 0; r < n; ++r) {
+        a.src[r] = p.ranks[r].send;
+        a.dst[r] = p.ranks[r].recv;
+    }
+    a.prog = plan.dev;
+    a.nDst = 1;
+    a.dstOwn = 1;
+    a.nGroup = n;
+    a.groupLen = p.count;                  // input slice stride = recvCount (reference
+    a.srcGroupStride = p.count;            // ins_v2_reduce_scatter_sole_executor.cc:260)
+    a.total = static_cast<uint64_t>(n) * p.count;
+    if (plan.segmentsAreSubs && plan.nProg > 1) {
+        a.nSub = n;                        // vector-core mesh: output cut into n chunks
+        a.subLen = p.count / n;
+        a.progSubStride = 1;
+    } else {
+        a.nSub = 1;
+        a.subLen = p.count;
+        a.progGroupStride = plan.nProg > 1 ? 1 : 0;
+    }
+    return LaunchOneReduce(w, a, p.dtype, p.op, s);
+}
+
+HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
+{
+    (void)w;
+    uint64_t bits = 0;
+    for (uint32_t d = 0; d < b.nDst; ++d) bits |= reinterpret_cast<uint64_t>(b.dst[d]);
+    b.unit = AlignUnitOf(bits);
+    HIP_OK(LaunchBcastCopy(b, s));
+    return HCCL_SUCCESS;
+}
+
+HcclResult RunAllGather(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    const uint64_t esz = DataTypeSize(p.dtype);
+    BcastCopyArgs b{};
+    b.nSeg = n;
+    b.nDst = n;
+    for (uint32_t r = 0; r < n; ++r) {
+        b.src[r] = p.ranks[r].send;
+        b.dst[r] = p.ranks[r].recv;
+        b.len[r] = p.count * esz;
+        b.dstOff[r] = static_cast<uint64_t>(r) * p.count * esz;   // reference all_gather_mesh_1D.cc:298-380
+    }
+    return RunBcast(w, b, s);
+}
+
+HcclResult RunAllGatherV(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    const uint64_t esz = DataTypeSize(p.dtype);
+    const std::vector<uint64_t>& ref = p.ranks[0].var;   // counts | displs | sendCount
+    for (uint32_t r = 0; r < n; ++r) {
+        const std::vector<uint64_t>& v = p.ranks[r].var;
+        if (memcmp(v.data(), ref.data(), 2 * n * sizeof(uint64_t)) != 0) {
+            Log(1, "AllGatherV: rank %u passed recvCounts / recvDispls that differ from rank 0", r);
+            return HCCL_E_PARA;
+        }
+        if (v[2 * n] != ref[r]) {
+            Log(1, "AllGatherV: rank %u sendCount %llu != recvCounts[%u] %llu", r, (unsigned long long)v[2 * n], r,
+                (unsigned long long)ref[r]);
+            return HCCL_E_PARA;
+        }
+    }
+    BcastCopyArgs b{};
+    b.nSeg = n;
+    b.nDst = n;
+    for (uint32_t r = 0; r < n; ++r) {
+        b.src[r] = p.ranks[r].send;
+        b.dst[r] = p.ranks[r].recv;
+        b.len[r] = ref[r] * esz;
+        b.dstOff[r] = ref[n + r] * esz;   // reference all_gather_v_mesh_1D.cc:242-310
+    }
+    return RunBcast(w, b, s);
+}
+
+HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    const uint32_t esz = DataTypeSize(p.dtype);
+    // rank r's var = sendCounts | recvCounts | sdispls | rdispls (reference all_to_all_v.cc:617-643)
+    uint64_t tiles = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t j = 0; j < n; ++j) {
+            uint64_t sent = p.ranks[j].var[i];
+            uint64_t expected = p.ranks[i].var[n + j];
+            if (sent != expected) {
+                Log(1, "AlltoAllV: rank %u recvCounts[%u]=%llu but rank %u sendCounts[%u]=%llu", i, j,
+                    (unsigned long long)expected, j, i, (unsigned long long)sent);
+                return HCCL_E_PARA;
+            }
+            tiles += (sent * esz + kCopyTileBytes - 1) / kCopyTileBytes;
+        }
+    }
+    if (tiles == 0) {
+        return HCCL_SUCCESS;
+    }
+    if (tiles > 0xFFFFFFF0ull) {
+        return HCCL_E_PARA;
+    }
+    HcclResult rc = EnsureA2aBuffers(w);
+    if (rc != HCCL_SUCCESS) {
+        return rc;
+    }
+    const uint32_t slot = w->a2aNext;
+    w->a2aNext = (w->a2aNext + 1) % kStagingSlots;
+    if (w->a2aSlotUsed[slot]) {
+        HIP_OK(hipEventSynchronize(w->a2aSlotFree[slot]));   // the call that last used this slot has finished
+    }
+    uint8_t* dev = w->a2aDev + slot * A2aSlotBytes(n);
+    const size_t tab = A2aTableBytes(n);
+    uint64_t* host = w->a2aHost[slot];
+    uint64_t* hCnt = host;
+    uint64_t* hSd = host + static_cast<size_t>(n) * n;
+    uint64_t* hRd = host + 2 * static_cast<size_t>(n) * n;
+    for (uint32_t r = 0; r < n; ++r) {
+        const uint64_t* v = p.ranks[r].var.data();
+        memcpy(hCnt + static_cast<size_t>(r) * n, v, n * sizeof(uint64_t));
+        memcpy(hSd + static_cast<size_t>(r) * n, v + 2 * n, n * sizeof(uint64_t));
+        memcpy(hRd + static_cast<size_t>(r) * n, v + 3 * n, n * sizeof(uint64_t));
+    }
+    HIP_OK(hipMemcpyAsync(dev, host, 3 * tab, hipMemcpyHostToDevice, s));
+
+    A2aArgs a{};
+    for (uint32_t r = 0; r < n; ++r) {
+        a.send[r] = p.ranks[r].send;
+        a.recv[r] = p.ranks[r].recv;
+    }
+    a.cnt = reinterpret_cast<const uint64_t*>(dev);
+    a.sdis = reinterpret_cast<const uint64_t*>(dev + tab);
+    a.rdis = reinterpret_cast<const uint64_t*>(dev + 2 * tab);
+    a.rowStart = reinterpret_cast<uint32_t*>(dev + 3 * tab);
+    a.segEnd = a.rowStart + (n + 1);
+    a.n = n;
+    a.esz = esz;
+    HIP_OK(LaunchA2aPlan(a, s));
+    uint32_t blocks = tiles < w->copyBlocks ? static_cast<uint32_t>(tiles) : w->copyBlocks;
+    HIP_OK(LaunchA2aCopy(a, blocks, s));
+    HIP_OK(hipEventRecord(w->a2aSlotFree[slot], s));
+    w->a2aSlotUsed[slot] = true;
+    return HCCL_SUCCESS;
+}
+
+// rankSize == 1: a plain copy, nothing when in place (reference op_common.cc:4458-4522).
+HcclResult RunSingleRank(World* w, PendingOp& p, hipStream_t s)
+{
+    const RankArgs& r = p.ranks[0];
+    if (r.send == r.recv) {
+        return HCCL_SUCCESS;
+    }
+    const uint64_t esz = DataTypeSize(p.dtype);
+    uint64_t len = p.count * esz;
+    uint64_t dstOff = 0;
+    if (p.type == OpType::ALL_GATHER_V) {
+        len = r.var[0] * esz;
+        dstOff = r.var[1] * esz;
+    } else if (p.type == OpType::ALL_TO_ALL_V) {
+        len = r.var[0] * esz;   // sendCounts[0], copied from the start of sendBuf to the start of recvBuf
+    }
+    if (len == 0) {
+        return HCCL_SUCCESS;
+    }
+    BcastCopyArgs b{};
+    b.nSeg = 1;
+    b.nDst = 1;
+    b.src[0] = r.send;
+    b.dst[0] = r.recv;
+    b.len[0] = len;
+    b.dstOff[0] = dstOff;
+    return RunBcast(w, b, s);
+}
+
+HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
+{
+    hipStream_t s = p.ranks[launcher].stream;
+    // Order the fused kernel after everything queued so far on the other ranks' streams (a superset of
+    // what each rank had queued when it called).  Ranks that share the launch stream need nothing.
+    std::vector<hipEvent_t> used;
+    for (uint32_t r = 0; r < w->n; ++r) {
+        if (p.ranks[r].stream == s) {
+            continue;
+        }
+        bool seen = false;
+        for (uint32_t q = 0; q < r; ++q) {
+            seen = seen || p.ranks[q].stream == p.ranks[r].stream;
+        }
+        if (seen) {
+            continue;
+        }
+        hipEvent_t ev;
+        HcclResult erc = TakeEvent(w, &ev);
+        if (erc != HCCL_SUCCESS) {
+            return erc;
+        }
+        used.push_back(ev);
+        HIP_OK(hipEventRecord(ev, p.ranks[r].stream));
+        HIP_OK(hipStreamWaitEvent(s, ev, 0));
+    }
+    HcclResult rc;
+    if (w->n == 1) {
+        rc = RunSingleRank(w, p, s);
+    } else {
+        switch (p.type) {
+            case OpType::ALL_REDUCE: rc = RunAllReduce(w, p, s); break;
+            case OpType::REDUCE_SCATTER: rc = RunReduceScatter(w, p, s); break;
+            case OpType::ALL_GATHER: rc = RunAllGather(w, p, s); break;
+            case OpType::ALL_GATHER_V: rc = RunAllGatherV(w, p, s); break;
+            default: rc = RunAlltoAllV(w, p, s); break;
+        }
+    }
+    // Order every other rank's stream after the fused kernel.
+    bool others = false;
+    for (uint32_t r = 0; r < w->n; ++r) {
+        others = others || p.ranks[r].stream != s;
+    }
+    if (others && rc == HCCL_SUCCESS) {
+        if (w->doneEvent == nullptr) {
+            HIP_OK(hipEventCreateWithFlags(&w->doneEvent, hipEventDisableTiming));
+        }
+        HIP_OK(hipEventRecord(w->doneEvent, s));
+        for (uint32_t r = 0; r < w->n; ++r) {
+            if (p.ranks[r].stream != s) {
+                HIP_OK(hipStreamWaitEvent(p.ranks[r].stream, w->doneEvent, 0));
+            }
+        }
+    }
+    for (hipEvent_t ev : used) {
+        w->eventPool.push_back(ev);
+    }
+    return rc;
+}
+
+uint32_t ExecTimeoutSeconds()
+{
+    // Reference default CUSTOM_TIMEOUT = 1836 s (alg_param.h:91), overridable by HCCL_EXEC_TIMEOUT.
+    static uint32_t t = EnvU32("HCCL_EXEC_TIMEOUT", 1836);
+    return t;
+}
+
+// Deposits one rank's arguments; the call that completes the set launches.
+HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count, const void* send,
+                  void* recv, hipStream_t stream, std::vector<uint64_t>&& var)
+{
+    World* w = c->world;
+    std::unique_lock<std::mutex> lock(w->mu);
+    const uint64_t seq = w->nextSeq[c->rank]++;
+    while (w->baseSeq + w->pending.size() <= seq) {
+        w->pending.push_back(nullptr);
+    }
+    std::shared_ptr<PendingOp>& cell = w->pending[seq - w->baseSeq];
+    if (!cell) {
+        cell = std::make_shared<PendingOp>();
+        cell->type = type;
+        cell->dtype = dtype;
+        cell->op = op;
+        cell->count = count;
+        cell->ranks.resize(w->n);
+    }
+    std::shared_ptr<PendingOp> p = cell;
+    if (p->type != type || p->dtype != dtype || p->op != op || p->count != count) {
+        Log(1, "%s on rank %u does not match the call of the other ranks (%s, count %llu, type %d)", OpName(type),
+            c->rank, OpName(p->type), (unsigned long long)p->count, static_cast<int>(p->dtype));
+        p->result = HCCL_E_PARA;
+    }
+    RankArgs& ra = p->ranks[c->rank];
+    ra.send = send;
+    ra.recv = recv;
+    ra.stream = stream;
+    ra.var = std::move(var);
+    ra.arrived = true;
+    p->arrived++;
+
+    if (p->arrived < w->n) {
+        if (t_groupDepth > 0) {
+            return p->result;   // queued; the group's last call launches
+        }
+        bool ok = w->cv.wait_for(lock, std::chrono::seconds(ExecTimeoutSeconds()), [&] { return p->done; });
+        if (!ok) {
+            Log(1, "%s: rank %u waited %u s for the other ranks", OpName(type), c->rank, ExecTimeoutSeconds());
+            p->result = HCCL_E_TIMEOUT;
+            return HCCL_E_TIMEOUT;
+        }
+        return p->result;
+    }
+
+    // Last arrival: launch.
+    if (p->result == HCCL_SUCCESS) {
+        p->result = Launch(w, *p, c->rank);
+    }
+    p->done = true;
+    while (!w->pending.empty() && w->pending.front() && w->pending.front()->done) {
+        w->pending.pop_front();
+        w->baseSeq++;
+    }
+    w->cv.notify_all();
+    return p->result;
+}
+
+}  // namespace
+}  // namespace hccl_amd
+
+using namespace hccl_amd;
+
+// ---------------------------------------------------------------------------------------------
+// extern "C" surface
+// ---------------------------------------------------------------------------------------------
+#define CHK_PTR(p, what)                               \
+    do {                                               \
+        if ((p) == nullptr) {                          \
+            Log(1, "%s: %s is nullptr", __func__, what); \
+            return HCCL_E_PTR;                         \
+        }                                              \
+    } while (0)
+
+#define CHK_RET(expr)                 \
+    do {                              \
+        HcclResult rc_ = (expr);      \
+        if (rc_ != HCCL_SUCCESS) {    \
+            return rc_;               \
+        }                             \
+    } while (0)
+
+namespace {
+
+// A rank whose stream differs from the launcher's must have its position recorded at call time.
+HcclResult SubmitWithReady(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count,
+                           const void* send, void* recv, aclrtStream stream, std::vector<uint64_t>&& var)
+{
+    return Submit(c, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var));
+}
+
+}  // namespace
+
+extern "C" {
+
+HcclResult HcclAllReduce(void* sendBuf, void* recvBuf, uint64_t count, HcclDataType dataType, HcclReduceOp op,
+                         HcclComm comm, aclrtStream stream)
+{
+    // Order of checks: reference src/ops/all_reduce/all_reduce.cc:41, 111-161.
+    if (count == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(stream, "stream");
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendBuf, "sendBuf");
+    CHK_PTR(recvBuf, "recvBuf");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclAllReduce: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckUserRank(c));
+    CHK_RET(CheckCount(count));
+    CHK_RET(CheckDataType(dataType, true));
+    CHK_RET(CheckReduceOp(dataType, op));
+    return SubmitWithReady(c, OpType::ALL_REDUCE, dataType, op, count, sendBuf, recvBuf, stream, {});
+}
+
+HcclResult HcclReduceScatter(void* sendBuf, void* recvBuf, uint64_t recvCount, HcclDataType dataType,
+                             HcclReduceOp op, HcclComm comm, aclrtStream stream)
+{
+    // Reference src/ops/reduce_scatter/reduce_scatter.cc:48-62.
+    if (recvCount == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(stream, "stream");
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendBuf, "sendBuf");
+    CHK_PTR(recvBuf, "recvBuf");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclReduceScatter: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckUserRank(c));
+    CHK_RET(CheckCount(recvCount));
+    CHK_RET(CheckDataType(dataType, true));
+    CHK_RET(CheckReduceOp(dataType, op));
+    return SubmitWithReady(c, OpType::REDUCE_SCATTER, dataType, op, recvCount, sendBuf, recvBuf, stream, {});
+}
+
+HcclResult HcclAllGather(void* sendBuf, void* recvBuf, uint64_t sendCount, HcclDataType dataType, HcclComm comm,
+                         aclrtStream stream)
+{
+    // Reference src/ops/all_gather/all_gather.cc:37, 118-149.
+    if (sendCount == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(stream, "stream");
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendBuf, "sendBuf");
+    CHK_PTR(recvBuf, "recvBuf");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclAllGather: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckCount(sendCount));
+    CHK_RET(CheckDataType(dataType, false));
+    CHK_RET(CheckUserRank(c));
+    return SubmitWithReady(c, OpType::ALL_GATHER, dataType, HCCL_REDUCE_RESERVED, sendCount, sendBuf, recvBuf, stream,
+                           {});
+}
+
+HcclResult HcclAllGatherV(void* sendBuf, uint64_t sendCount, void* recvBuf, const void* recvCounts,
+                          const void* recvDispls, HcclDataType dataType, HcclComm comm, aclrtStream stream)
+{
+    // Reference src/ops/all_gather_v/all_gather_v.cc:41-55, 137-282.
+    CHK_PTR(comm, "comm");
+    CHK_PTR(recvCounts, "recvCounts");
+    CHK_PTR(recvDispls, "recvDispls");
+    CHK_PTR(stream, "stream");
+    if (sendCount > 0) {
+        CHK_PTR(sendBuf, "sendBuf");
+    }
+    if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
+        Log(1, "HcclAllGatherV: sendBuf and recvBuf cannot be the same");
+        return HCCL_E_PARA;
+    }
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclAllGatherV: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    const uint32_t n = c->world->n;
+    const uint64_t* counts = static_cast<const uint64_t*>(recvCounts);
+    const uint64_t* displs = static_cast<const uint64_t*>(recvDispls);
+    bool allZero = true;
+    for (uint32_t i = 0; i < n; ++i) {
+        allZero = allZero && counts[i] == 0;
+    }
+    if (allZero) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(recvBuf, "recvBuf");
+    CHK_RET(CheckUserRank(c));
+    CHK_RET(CheckCount(sendCount));
+    CHK_RET(CheckDataType(dataType, false));
+    // Non-empty intervals may be unordered and leave holes but must not overlap or overflow.
+    const uint64_t esz = DataTypeSize(dataType);
+    for (uint32_t a = 0; a < n; ++a) {
+        if (counts[a] == 0) {
+            continue;
+        }
+        uint64_t end = displs[a] + counts[a];
+        if (end < displs[a] || end > UINT64_MAX / esz) {
+            Log(1, "HcclAllGatherV: recvDispls[%u] + recvCounts[%u] overflows", a, a);
+            return HCCL_E_PARA;
+        }
+        for (uint32_t b = a + 1; b < n; ++b) {
+            if (counts[b] != 0 && displs[a] < displs[b] + counts[b] && displs[b] < end) {
+                Log(1, "HcclAllGatherV: recvDispls intervals of ranks %u and %u overlap", a, b);
+                return HCCL_E_PARA;
+            }
+        }
+    }
+    std::vector<uint64_t> var(2 * n + 1);
+    memcpy(var.data(), counts, n * sizeof(uint64_t));
+    memcpy(var.data() + n, displs, n * sizeof(uint64_t));
+    var[2 * n] = sendCount;
+    // Every rank passes the same count as "count" of the pending op: use 0 so that ranks with different
+    // sendCount still meet; per-rank counts are validated at launch.
+    return SubmitWithReady(c, OpType::ALL_GATHER_V, dataType, HCCL_REDUCE_RESERVED, 0, sendBuf, recvBuf, stream,
+                           std::move(var));
+}
+
+HcclResult HcclAlltoAllV(const void* sendBuf, const void* sendCounts, const void* sdispls, HcclDataType sendType,
+                         const void* recvBuf, const void* recvCounts, const void* rdispls, HcclDataType recvType,
+                         HcclComm comm, aclrtStream stream)
+{
+    // Reference src/ops/all_to_all_v/all_to_all_v.cc:105-129, 517-598.  Like the reference, only recvType
+    // is consulted for the element size.
+    (void)sendType;
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendCounts, "sendCounts");
+    CHK_PTR(sdispls, "sdispls");
+    CHK_PTR(recvCounts, "recvCounts");
+    CHK_PTR(rdispls, "rdispls");
+    CHK_PTR(stream, "stream");
+    if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
+        Log(1, "HcclAlltoAllV: sendBuf and recvBuf cannot be the same");
+        return HCCL_E_PARA;
+    }
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclAlltoAllV: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    const uint32_t n = c->world->n;
+    const uint64_t* sc = static_cast<const uint64_t*>(sendCounts);
+    const uint64_t* rc = static_cast<const uint64_t*>(recvCounts);
+    bool sendZero = true, recvZero = true;
+    uint64_t maxCount = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        sendZero = sendZero && sc[i] == 0;
+        recvZero = recvZero && rc[i] == 0;
+        maxCount = sc[i] > maxCount ? sc[i] : maxCount;
+        maxCount = rc[i] > maxCount ? rc[i] : maxCount;
+    }
+    if (!sendZero) {
+        CHK_PTR(sendBuf, "sendBuf");
+    }
+    if (!recvZero) {
+        CHK_PTR(recvBuf, "recvBuf");
+    }
+    CHK_RET(CheckUserRank(c));
+    CHK_RET(CheckCount(maxCount));
+    CHK_RET(CheckDataType(recvType, false));
+    std::vector<uint64_t> var(4 * n);
+    memcpy(var.data(), sc, n * sizeof(uint64_t));
+    memcpy(var.data() + n, rc, n * sizeof(uint64_t));
+    memcpy(var.data() + 2 * n, sdispls, n * sizeof(uint64_t));
+    memcpy(var.data() + 3 * n, rdispls, n * sizeof(uint64_t));
+    return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
+                           const_cast<void*>(recvBuf), stream, std::move(var));
+}
+
+// ---- lifecycle -------------------------------------------------------------------------------
+HcclResult HcclCommInitAll(uint32_t ndev, int32_t* devices, HcclComm* comms)
+{
+    CHK_PTR(comms, "comms");
+    if (ndev == 0 || ndev > static_cast<uint32_t>(kMaxRanks)) {
+        Log(1, "HcclCommInitAll: ndev %u outside [1, %d]", ndev, kMaxRanks);
+        return HCCL_E_PARA;
+    }
+    if (devices != nullptr) {
+        for (uint32_t i = 1; i < ndev; ++i) {
+            if (devices[i] != devices[0]) {
+                Log(1, "HcclCommInitAll: a loopback world lives on one GPU; devices[%u]=%d != devices[0]=%d", i,
+                    devices[i], devices[0]);
+                return HCCL_E_NOT_SUPPORT;
+            }
+        }
+    }
+    std::lock_guard<std::mutex> g(g_registryMu);
+    auto w = NewWorld(ndev);
+    w->id = g_nextWorldId++;
+    for (uint32_t r = 0; r < ndev; ++r) {
+        w->comms[r] = std::make_unique<Comm>();
+        w->comms[r]->world = w.get();
+        w->comms[r]->rank = r;
+        comms[r] = w->comms[r].get();
+    }
+    w->joined = ndev;
+    g_worlds[w->id] = std::move(w);
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclGetRootInfo(HcclRootInfo* rootInfo)
+{
+    CHK_PTR(rootInfo, "rootInfo");
+    std::lock_guard<std::mutex> g(g_registryMu);
+    memset(rootInfo, 0, sizeof(*rootInfo));
+    uint64_t id = g_nextWorldId++;
+    memcpy(rootInfo->internal, "HCLAROOT", 8);
+    memcpy(rootInfo->internal + 8, &id, sizeof(id));
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclCommInitRootInfo(uint32_t nRanks, const HcclRootInfo* rootInfo, uint32_t rank, HcclComm* comm)
+{
+    CHK_PTR(rootInfo, "rootInfo");
+    CHK_PTR(comm, "comm");
+    if (memcmp(rootInfo->internal, "HCLAROOT", 8) != 0 || nRanks == 0 || nRanks > static_cast<uint32_t>(kMaxRanks) ||
+        rank >= nRanks) {
+        Log(1, "HcclCommInitRootInfo: invalid rootInfo, nRanks %u or rank %u", nRanks, rank);
+        return HCCL_E_PARA;
+    }
+    uint64_t id;
+    memcpy(&id, rootInfo->internal + 8, sizeof(id));
+    std::lock_guard<std::mutex> g(g_registryMu);
+    auto it = g_worlds.find(id);
+    if (it == g_worlds.end()) {
+        auto w = NewWorld(nRanks);
+        w->id = id;
+        it = g_worlds.emplace(id, std::move(w)).first;
+    }
+    World* w = it->second.get();
+    if (w->n != nRanks || w->comms[rank] != nullptr) {
+        Log(1, "HcclCommInitRootInfo: rank %u joins a world of %u ranks inconsistently", rank, w->n);
+        return HCCL_E_PARA;
+    }
+    w->comms[rank] = std::make_unique<Comm>();
+    w->comms[rank]->world = w;
+    w->comms[rank]->rank = rank;
+    w->joined++;
+    *comm = w->comms[rank].get();
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclCommDestroy(HcclComm comm)
+{
+    CHK_PTR(comm, "comm");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> g(g_registryMu);
+    World* w = c->world;
+    bool last;
+    {
+        std::lock_guard<std::mutex> wl(w->mu);
+        c->destroyed = true;
+        w->destroyed++;
+        last = w->destroyed == w->n;
+    }
+    if (last) {
+        (void)hipDeviceSynchronize();
+        g_worlds.erase(w->id);
+    }
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclGetRankSize(HcclComm comm, uint32_t* rankSize)
+{
+    CHK_PTR(comm, "comm");
+    CHK_PTR(rankSize, "rankSize");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    *rankSize = c->world->n;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclGetRankId(HcclComm comm, uint32_t* rank)
+{
+    CHK_PTR(comm, "comm");
+    CHK_PTR(rank, "rank");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    *rank = c->rank;
+    return HCCL_SUCCESS;
+}
+
+const char* HcclGetErrorString(HcclResult code)
+{
+    switch (code) {
+        case HCCL_SUCCESS: return "no error";
+        case HCCL_E_PARA: return "parameter error";
+        case HCCL_E_PTR: return "empty pointer";
+        case HCCL_E_MEMORY: return "memory error";
+        case HCCL_E_INTERNAL: return "internal error";
+        case HCCL_E_NOT_SUPPORT: return "not support feature";
+        case HCCL_E_NOT_FOUND: return "not found specific resource";
+        case HCCL_E_UNAVAIL: return "resource unavailable";
+        case HCCL_E_TIMEOUT: return "timeout";
+        case HCCL_E_RUNTIME: return "call runtime api fail";
+        default: return "unknown error";
+    }
+}
+
+HcclResult HcclGroupStart(void)
+{
+    t_groupDepth++;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclGroupEnd(void)
+{
+    if (t_groupDepth == 0) {
+        Log(1, "HcclGroupEnd without HcclGroupStart");
+        return HCCL_E_PARA;
+    }
+    t_groupDepth--;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo)
+{
+    CHK_PTR(comm, "comm");
+    Comm* c = AsComm(comm);
+    if (c == nullptr || static_cast<int>(op) < 0 || op >= HCCL_AMD_OP_COUNT || static_cast<int>(algo) < 0 ||
+        algo >= HCCL_AMD_ALGO_COUNT) {
+        return HCCL_E_PARA;
+    }
+    if (op == HCCL_AMD_OP_ALL_REDUCE && algo == HCCL_AMD_ALGO_AIV_MESH) {
+        return HCCL_E_NOT_SUPPORT;
+    }
+    std::lock_guard<std::mutex> wl(c->world->mu);
+    c->world->algo[op] = algo;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdGetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo* algo)
+{
+    CHK_PTR(comm, "comm");
+    CHK_PTR(algo, "algo");
+    Comm* c = AsComm(comm);
+    if (c == nullptr || static_cast<int>(op) < 0 || op >= HCCL_AMD_OP_COUNT) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> wl(c->world->mu);
+    *algo = c->world->algo[op];
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdGetFoldProgram(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t segment,
+                                 uint8_t* out, uint32_t cap, uint32_t* len, uint32_t* segmentCount)
+{
+    CHK_PTR(len, "len");
+    FoldPlan plan;
+    HcclResult rc = BuildFoldPlan(op, algo, rankSize, &plan);
+    if (rc != HCCL_SUCCESS) {
+        return rc;
+    }
+    if (segmentCount != nullptr) {
+        *segmentCount = static_cast<uint32_t>(plan.programs.size());
+    }
+    if (segment >= plan.programs.size()) {
+        return HCCL_E_PARA;
+    }
+    const std::vector<uint8_t>& p = plan.programs[segment];
+    *len = static_cast<uint32_t>(p.size());
+    if (out != nullptr) {
+        if (cap < p.size()) {
+            return HCCL_E_MEMORY;
+        }
+        memcpy(out, p.data(), p.size());
+    }
+    return HCCL_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,348 @@
+// Fold-program construction.  Each builder replays, symbolically, the sequence of pairwise
+// LocalReduce / write-reduce steps the reference's template issues and records, for the slot that ends
+// up holding a segment's result, which rank values were folded into it, in which order and in which role.
+#include "fold_plan.h"
+
+#include <memory>
+
+#include "dataplane.h"
+
+namespace hccl_amd {
+namespace {
+
+// A value under construction: operands folded left to right into the first one.
+struct Expr;
+using ExprPtr = std::shared_ptr<const Expr>;
+struct Operand {
+    int rank;      // >= 0: a rank's input value
+    ExprPtr sub;   // otherwise a nested value
+};
+struct Expr {
+    std::vector<Operand> ops;
+};
+
+ExprPtr Leaf(uint32_t rank)
+{
+    auto e = std::make_shared<Expr>();
+    e->ops.push_back({static_cast<int>(rank), nullptr});
+    return e;
+}
+
+// dst <- src (+) dst : dst stays the accumulator, src becomes one more operand of its level.
+ExprPtr Fold(const ExprPtr& dst, const ExprPtr& src)
+{
+    auto e = std::make_shared<Expr>(*dst);
+    if (src->ops.size() == 1 && src->ops[0].rank >= 0) {
+        e->ops.push_back(src->ops[0]);
+    } else {
+        e->ops.push_back({-1, src});
+    }
+    return e;
+}
+
+uint32_t Depth(const Expr& e)
+{
+    uint32_t d = 1;
+    for (const Operand& o : e.ops) {
+        if (o.rank < 0) {
+            uint32_t sd = 1 + Depth(*o.sub);
+            d = sd > d ? sd : d;
+        }
+    }
+    return d;
+}
+
+void Serialize(const Expr& e, std::vector<uint8_t>* out)
+{
+    size_t i = 0;
+    while (i < e.ops.size()) {
+        if (e.ops[i].rank < 0) {
+            out->push_back(kTokOpen);
+            Serialize(*e.ops[i].sub, out);
+            out->push_back(kTokClose);
+            ++i;
+            continue;
+        }
+        size_t j = i;
+        while (j < e.ops.size() && e.ops[j].rank >= 0 && j - i < static_cast<size_t>(kMaxRun)) {
+            ++j;
+        }
+        out->push_back(static_cast<uint8_t>(kTokRun | (j - i)));
+        for (size_t k = i; k < j; ++k) {
+            out->push_back(static_cast<uint8_t>(e.ops[k].rank));
+        }
+        i = j;
+    }
+}
+
+HcclResult Emit(const ExprPtr& e, FoldPlan* plan)
+{
+    uint32_t d = Depth(*e);
+    if (d > static_cast<uint32_t>(kMaxFoldDepth)) {
+        return HCCL_E_NOT_SUPPORT;
+    }
+    std::vector<uint8_t> prog;
+    Serialize(*e, &prog);
+    prog.push_back(kTokEnd);
+    if (prog.size() > static_cast<size_t>(kProgStride)) {
+        return HCCL_E_INTERNAL;
+    }
+    plan->maxDepth = d > plan->maxDepth ? d : plan->maxDepth;
+    plan->programs.push_back(std::move(prog));
+    return HCCL_SUCCESS;
+}
+
+ExprPtr Chain(const std::vector<uint32_t>& order)
+{
+    ExprPtr e = Leaf(order[0]);
+    for (size_t i = 1; i < order.size(); ++i) {
+        e = Fold(e, Leaf(order[i]));
+    }
+    return e;
+}
+
+uint32_t CeilLog2(uint32_t n)
+{
+    uint32_t s = 0;
+    for (uint32_t t = n - 1; t != 0; t >>= 1) {
+        ++s;
+    }
+    return s;
+}
+
+uint32_t FloorLog2(uint32_t n)
+{
+    uint32_t s = 0;
+    for (uint32_t t = n; t > 1; t >>= 1) {
+        ++s;
+    }
+    return s;
+}
+
+// ---- mesh --------------------------------------------------------------------------------------
+// AllReduce: slot 0 accumulates slots 1..N-1 ascending (reference
+// ins_temp_all_reduce_mesh_1D_one_shot.cc:223-239; two-shot and the host-reduce NHR template fold in
+// the same order, ins_temp_all_reduce_mesh_1D_two_shot.cc:341-357,
+// ins_temp_all_reduce_aicpu_reduce_nhr.cc:272-285).
+HcclResult MeshAllReduce(uint32_t n, FoldPlan* plan)
+{
+    std::vector<uint32_t> order(n);
+    for (uint32_t r = 0; r < n; ++r) {
+        order[r] = r;
+    }
+    plan->segmentsAreSubs = true;
+    return Emit(Chain(order), plan);
+}
+
+// ReduceScatter: rank k copies its own slice, then folds the other ranks ascending (reference
+// ins_temp_reduce_scatter_mesh_1D.cc:203-237).
+HcclResult MeshReduceScatter(uint32_t n, FoldPlan* plan)
+{
+    for (uint32_t k = 0; k < n; ++k) {
+        std::vector<uint32_t> order{k};
+        for (uint32_t t = 0; t < n; ++t) {
+            if (t != k) {
+                order.push_back(t);
+            }
+        }
+        HcclResult rc = Emit(Chain(order), plan);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// Vector-core mesh ReduceScatter: chunk c of an output starts from peer c and folds peers
+// c+1, c+2, ... modulo N (reference aiv_reduce_scatter_mesh_1d.h:34-46, 57-71).
+HcclResult AivMeshReduceScatter(uint32_t n, FoldPlan* plan)
+{
+    plan->segmentsAreSubs = true;
+    for (uint32_t c = 0; c < n; ++c) {
+        std::vector<uint32_t> order(n);
+        for (uint32_t i = 0; i < n; ++i) {
+            order[i] = (c + i) % n;
+        }
+        HcclResult rc = Emit(Chain(order), plan);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// ---- order preserved ---------------------------------------------------------------------------
+// while blocks > 1: M = largest power of two below blocks; block src in [M, blocks) folds into block
+// src % M; blocks = M (reference ins_temp_reduce_scatter_order_preserved_group.cc:353-398).
+HcclResult OrderPreserved(uint32_t n, FoldPlan* plan)
+{
+    std::vector<ExprPtr> slot(n);
+    for (uint32_t v = 0; v < n; ++v) {
+        slot[v] = Leaf(v);
+    }
+    uint32_t remaining = n;
+    while (remaining > 1) {
+        uint32_t m = 1;
+        while (m * 2 < remaining) {
+            m *= 2;
+        }
+        for (uint32_t src = m; src < remaining; ++src) {
+            slot[src % m] = Fold(slot[src % m], slot[src]);
+        }
+        remaining = m;
+    }
+    return Emit(slot[0], plan);
+}
+
+// ---- NHR ---------------------------------------------------------------------------------------
+// Step s: rank m write-reduces slices {m - 2^s - i * 2^(s+1)} into the same slices of rank m - 2^s,
+// i < (N - 1 + 2^s) / 2^(s+1); the receiver's value is the accumulator (reference
+// ins_temp_reduce_scatter_nhr.cc:316-447, 458-506).  Slice k ends at rank k.
+HcclResult Nhr(uint32_t n, FoldPlan* plan)
+{
+    std::vector<std::vector<ExprPtr>> held(n, std::vector<ExprPtr>(n));
+    for (uint32_t m = 0; m < n; ++m) {
+        for (uint32_t k = 0; k < n; ++k) {
+            held[m][k] = Leaf(m);
+        }
+    }
+    uint32_t steps = CeilLog2(n);
+    for (uint32_t s = 0; s < steps; ++s) {
+        const auto before = held;
+        uint32_t delta = 1u << s;
+        uint32_t nSlices = (n - 1 + delta) / (delta * 2);
+        uint32_t stride = (delta * 2) % n;
+        for (uint32_t m = 0; m < n; ++m) {
+            uint32_t to = (m + n - delta) % n;
+            uint32_t slice = to;
+            for (uint32_t i = 0; i < nSlices; ++i) {
+                held[to][slice] = Fold(before[to][slice], before[m][slice]);
+                slice = (slice + n - stride) % n;
+            }
+        }
+    }
+    for (uint32_t k = 0; k < n; ++k) {
+        HcclResult rc = Emit(held[k][k], plan);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// ---- RHD ---------------------------------------------------------------------------------------
+uint32_t VirtualSlotStart(uint32_t r, uint32_t a) { return a < r ? 2 * a : a + r; }
+uint32_t VirtualSlotEnd(uint32_t r, uint32_t b) { return b <= r ? 2 * b : b + r; }
+
+// Mirror: every rank holds p slots, slot sigma(i) = its contribution to share i.
+// PRE:  merged rank t + r write-reduces all p slots into representative t.
+// MAIN: step k, dist = P >> (k + 1): virtual rank v write-reduces the slots of its partner's aligned
+//       half into the partner v ^ dist (the partner's value is the accumulator).
+// Share i ends at the carrier of the virtual rank owning slot sigma(i)
+// (reference template_utils.cc:117-208, ins_temp_reduce_scatter_rhd.cc:365-564).
+HcclResult Rhd(uint32_t p, FoldPlan* plan)
+{
+    uint32_t r = RhdPairCount(p);
+    uint32_t bigP = p - r;
+    std::vector<std::vector<ExprPtr>> held(p, std::vector<ExprPtr>(p));
+    for (uint32_t j = 0; j < p; ++j) {
+        for (uint32_t u = 0; u < p; ++u) {
+            held[j][u] = Leaf(j);
+        }
+    }
+    for (uint32_t t = 0; t < r; ++t) {
+        for (uint32_t u = 0; u < p; ++u) {
+            held[t][u] = Fold(held[t][u], held[t + r][u]);
+        }
+    }
+    uint32_t steps = FloorLog2(bigP);
+    for (uint32_t k = 0; k < steps; ++k) {
+        const auto before = held;
+        uint32_t dist = bigP >> (k + 1);
+        for (uint32_t v = 0; v < bigP; ++v) {
+            uint32_t peer = v ^ dist;
+            uint32_t peerBase = peer & ~(dist - 1);
+            uint32_t from = RhdCarrierOfVirtual(p, v);
+            uint32_t to = RhdCarrierOfVirtual(p, peer);
+            for (uint32_t u = VirtualSlotStart(r, peerBase); u < VirtualSlotEnd(r, peerBase + dist); ++u) {
+                held[to][u] = Fold(before[to][u], before[from][u]);
+            }
+        }
+    }
+    for (uint32_t i = 0; i < p; ++i) {
+        uint32_t slot = RhdSlotOfRank(p, i);
+        uint32_t v = slot < 2 * r ? slot / 2 : slot - r;
+        HcclResult rc = Emit(held[RhdCarrierOfVirtual(p, v)][slot], plan);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+}  // namespace
+
+uint32_t RhdPairCount(uint32_t p)
+{
+    if (p == 0) {
+        return 0;
+    }
+    uint32_t hp = 1;
+    while (hp <= p / 2) {
+        hp *= 2;
+    }
+    return p - hp;
+}
+
+uint32_t RhdSlotOfRank(uint32_t p, uint32_t rank)
+{
+    uint32_t r = RhdPairCount(p);
+    if (rank < r) {
+        return 2 * rank;
+    }
+    if (rank < 2 * r) {
+        return 2 * (rank - r) + 1;
+    }
+    return rank;
+}
+
+uint32_t RhdCarrierOfVirtual(uint32_t p, uint32_t v)
+{
+    uint32_t r = RhdPairCount(p);
+    return v < r ? v : v + r;
+}
+
+HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPlan* plan)
+{
+    *plan = FoldPlan{};
+    if (n == 0 || n > static_cast<uint32_t>(kMaxRanks)) {
+        return HCCL_E_PARA;
+    }
+    bool ar = op == HCCL_AMD_OP_ALL_REDUCE;
+    if (!ar && op != HCCL_AMD_OP_REDUCE_SCATTER) {
+        return HCCL_E_PARA;
+    }
+    switch (algo) {
+        case HCCL_AMD_ALGO_MESH:
+            return ar ? MeshAllReduce(n, plan) : MeshReduceScatter(n, plan);
+        case HCCL_AMD_ALGO_RING:
+            // AllReduce: the host-reduce "ring family" template gathers and folds in rank order.
+            // ReduceScatter: the in-tree ring-family algorithm is the NHR step tree.
+            return ar ? MeshAllReduce(n, plan) : Nhr(n, plan);
+        case HCCL_AMD_ALGO_RHD:
+            plan->segmentsAreSubs = ar;
+            return Rhd(n, plan);
+        case HCCL_AMD_ALGO_NHR:
+            plan->segmentsAreSubs = ar;
+            return Nhr(n, plan);
+        case HCCL_AMD_ALGO_ORDER_PRESERVED:
+            plan->segmentsAreSubs = true;
+            return OrderPreserved(n, plan);
+        case HCCL_AMD_ALGO_AIV_MESH:
+            return ar ? HCCL_E_NOT_SUPPORT : AivMeshReduceScatter(n, plan);
+        default:
+            return HCCL_E_PARA;
+    }
+}
+
+}  // namespace hccl_amd

@@ -1,0 +1,346 @@
+// Fused N-rank reduce for gfx950 (MI355X).
+//
+// One launch performs the local-reduce work of every rank of a loopback world: each lane owns a
+// 16-byte vector position, pulls that position from the N rank buffers with 128-bit loads, combines
+// them in registers in the order a fold program dictates, and writes the result once per
+// destination.  The path is bound by HBM bandwidth (N reads + M writes of the element range, no
+// re-reads, no staging passes), so there is no MFMA and LDS only holds the 320-byte program.
+//
+// Operand roles follow the reference's pairwise step  dst[i] = src[i] (+) dst[i]
+// (alg_data_trans_wrapper.cc:1319-1358):
+//   SUM   src + dst                 integers wrap
+//   PROD  src * dst                 integers wrap (computed unsigned)
+//   MAX   (src < dst) ? dst : src   ties / unordered keep src
+//   MIN   (dst < src) ? dst : src   ties / unordered keep src
+// fp16 / bf16 SUM accumulate in fp32 and round to nearest even once at the end; fp16 PROD rounds
+// after every step like the reference's host path (:1237-1257); fp16 / bf16 MAX and MIN compare the
+// values and carry the original 16-bit pattern.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "dataplane.h"
+
+namespace hccl_amd {
+namespace detail {
+
+constexpr int kSum = 0, kProd = 1, kMax = 2, kMin = 3;
+constexpr int kThreads = 256;
+
+// ---------------------------------------------------------------------------------------------
+// Element semantics.  S = storage type, A = accumulator type.
+// ---------------------------------------------------------------------------------------------
+template <typename T, typename UT, int OP>
+struct IntOps {
+    using S = T;
+    using A = T;
+    static __device__ __forceinline__ A Widen(S x) { return x; }
+    static __device__ __forceinline__ S Narrow(A a) { return a; }
+    static __device__ __forceinline__ A Fold(A src, A dst)
+    {
+        if constexpr (OP == kSum) {
+            return static_cast<T>(static_cast<UT>(static_cast<UT>(src) + static_cast<UT>(dst)));
+        } else if constexpr (OP == kProd) {
+            return static_cast<T>(static_cast<UT>(static_cast<UT>(src) * static_cast<UT>(dst)));
+        } else if constexpr (OP == kMax) {
+            return (src < dst) ? dst : src;
+        } else {
+            return (dst < src) ? dst : src;
+        }
+    }
+};
+
+template <typename T, int OP>
+struct FpOps {
+    using S = T;
+    using A = T;
+    static __device__ __forceinline__ A Widen(S x) { return x; }
+    static __device__ __forceinline__ S Narrow(A a) { return a; }
+    static __device__ __forceinline__ A Fold(A src, A dst)
+    {
+        if constexpr (OP == kSum) {
+            return src + dst;
+        } else if constexpr (OP == kProd) {
+            return src * dst;
+        } else if constexpr (OP == kMax) {
+            return (src < dst) ? dst : src;
+        } else {
+            return (dst < src) ? dst : src;
+        }
+    }
+};
+
+__device__ __forceinline__ float HalfBitsToFloat(uint16_t h) { return static_cast<float>(__builtin_bit_cast(_Float16, h)); }
+__device__ __forceinline__ uint16_t FloatToHalfBits(float f) { return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f)); }
+__device__ __forceinline__ float Bf16BitsToFloat(uint16_t h) { return __builtin_bit_cast(float, static_cast<uint32_t>(h) << 16); }
+__device__ __forceinline__ uint16_t FloatToBf16Bits(float f)
+{
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    uint32_t rounded = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+    uint32_t quiet = (u >> 16) | 0x40u;
+    bool isNan = (u & 0x7FFFFFFFu) > 0x7F800000u;
+    return static_cast<uint16_t>(isNan ? quiet : rounded);
+}
+
+// fp16 / bf16 SUM: fp32 accumulator, one rounding at the end.
+template <bool IS_BF16>
+struct HalfSumOps {
+    using S = uint16_t;
+    using A = float;
+    static __device__ __forceinline__ A Widen(S x) { return IS_BF16 ? Bf16BitsToFloat(x) : HalfBitsToFloat(x); }
+    static __device__ __forceinline__ S Narrow(A a) { return IS_BF16 ? FloatToBf16Bits(a) : FloatToHalfBits(a); }
+    static __device__ __forceinline__ A Fold(A src, A dst) { return src + dst; }
+};
+
+// fp16 PROD: the product of two fp16 values is exact in fp32, so rounding it to fp16 after every step
+// is the IEEE fp16 multiply.
+struct HalfProdOps {
+    using S = uint16_t;
+    using A = _Float16;
+    static __device__ __forceinline__ A Widen(S x) { return __builtin_bit_cast(_Float16, x); }
+    static __device__ __forceinline__ S Narrow(A a) { return __builtin_bit_cast(uint16_t, a); }
+    static __device__ __forceinline__ A Fold(A src, A dst)
+    {
+        return static_cast<_Float16>(static_cast<float>(src) * static_cast<float>(dst));
+    }
+};
+
+// fp16 / bf16 MAX, MIN: pure selection, the bit pattern of the chosen operand survives.
+template <bool IS_BF16, int OP>
+struct HalfSelectOps {
+    using S = uint16_t;
+    using A = uint16_t;
+    static __device__ __forceinline__ A Widen(S x) { return x; }
+    static __device__ __forceinline__ S Narrow(A a) { return a; }
+    static __device__ __forceinline__ A Fold(A src, A dst)
+    {
+        float s = IS_BF16 ? Bf16BitsToFloat(src) : HalfBitsToFloat(src);
+        float d = IS_BF16 ? Bf16BitsToFloat(dst) : HalfBitsToFloat(dst);
+        if constexpr (OP == kMax) {
+            return (s < d) ? dst : src;
+        } else {
+            return (d < s) ? dst : src;
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Packs: W storage elements that travel as one memory transaction.
+// ---------------------------------------------------------------------------------------------
+typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+
+template <typename S, int W>
+struct alignas(sizeof(S) * W >= 16 ? 16 : sizeof(S) * W) Pack {
+    S e[W];
+};
+
+template <typename S, int W>
+__device__ __forceinline__ Pack<S, W> LoadPack(const void* base, uint64_t elemOff)
+{
+    const S* p = static_cast<const S*>(base) + elemOff;
+    if constexpr (sizeof(S) * W == 16) {
+        U32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(p));
+        return __builtin_bit_cast(Pack<S, W>, raw);
+    } else {
+        Pack<S, W> r;
+        r.e[0] = __builtin_nontemporal_load(p);
+        return r;
+    }
+}
+
+template <typename S, int W>
+__device__ __forceinline__ void StorePack(void* base, uint64_t elemOff, const Pack<S, W>& v)
+{
+    S* p = static_cast<S*>(base) + elemOff;
+    if constexpr (sizeof(S) * W == 16) {
+        __builtin_nontemporal_store(__builtin_bit_cast(U32x4, v), reinterpret_cast<U32x4*>(p));
+    } else {
+        __builtin_nontemporal_store(v.e[0], p);
+    }
+}
+
+__device__ __forceinline__ uint32_t Uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// ---------------------------------------------------------------------------------------------
+// Program interpreter.  Control flow depends only on the program, so it is uniform across the
+// wavefront; each nesting level has its own accumulator registers through template recursion.
+// ---------------------------------------------------------------------------------------------
+template <class E, int W>
+struct AccPack {
+    typename E::A a[W];
+};
+
+template <class E, int W>
+__device__ __forceinline__ void FoldRun(const uint8_t* sprog, uint32_t& pc, uint32_t n, const ReduceArgs& args,
+                                        uint64_t off, AccPack<E, W>& acc, bool init)
+{
+    using S = typename E::S;
+    Pack<S, W> v[kMaxRun];
+#pragma unroll
+    for (int i = 0; i < kMaxRun; ++i) {
+        if (static_cast<uint32_t>(i) < n) {
+            uint32_t rank = Uniform(sprog[pc + i]);
+            v[i] = LoadPack<S, W>(args.src[rank], off);
+        }
+    }
+    pc += n;
+    if (init) {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            acc.a[w] = E::Widen(v[0].e[w]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxRun; ++i) {
+        if (static_cast<uint32_t>(i) < n && !(init && i == 0)) {
+#pragma unroll
+            for (int w = 0; w < W; ++w) {
+                acc.a[w] = E::Fold(E::Widen(v[i].e[w]), acc.a[w]);
+            }
+        }
+    }
+}
+
+template <class E, int W, int L>
+__device__ __forceinline__ void EvalLevel(const uint8_t* sprog, uint32_t& pc, const ReduceArgs& args, uint64_t off,
+                                          AccPack<E, W>& acc)
+{
+    // The first operand of every level is a rank value (the builder guarantees a run token here).
+    uint32_t tok = Uniform(sprog[pc]);
+    ++pc;
+    FoldRun<E, W>(sprog, pc, tok & 0x3Fu, args, off, acc, true);
+    for (;;) {
+        tok = Uniform(sprog[pc]);
+        ++pc;
+        if (tok == kTokClose || tok == kTokEnd) {
+            return;
+        }
+        if (tok == kTokOpen) {
+            if constexpr (L + 1 < kMaxFoldDepth) {
+                AccPack<E, W> sub;
+                EvalLevel<E, W, L + 1>(sprog, pc, args, off, sub);
+#pragma unroll
+                for (int w = 0; w < W; ++w) {
+                    acc.a[w] = E::Fold(sub.a[w], acc.a[w]);
+                }
+            } else {
+                return;   // deeper than the host ever emits
+            }
+        } else {
+            FoldRun<E, W>(sprog, pc, tok & 0x3Fu, args, off, acc, false);
+        }
+    }
+}
+
+template <class E, int W>
+__device__ __forceinline__ void ReduceOne(const uint8_t* sprog, const ReduceArgs& args, uint64_t srcOff,
+                                          uint64_t dstOff, uint32_t group)
+{
+    using S = typename E::S;
+    AccPack<E, W> acc;
+    uint32_t pc = 0;
+    EvalLevel<E, W, 0>(sprog, pc, args, srcOff, acc);
+    Pack<S, W> out;
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+        out.e[w] = E::Narrow(acc.a[w]);
+    }
+    if (args.dstOwn) {
+        StorePack<S, W>(args.dst[group], dstOff, out);
+    } else {
+        for (uint32_t d = 0; d < args.nDst; ++d) {
+            StorePack<S, W>(args.dst[d], dstOff, out);
+        }
+    }
+}
+
+template <class E>
+__global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
+{
+    using S = typename E::S;
+    constexpr int W = 16 / sizeof(S);
+    __shared__ __attribute__((aligned(16))) uint8_t sprog[kProgStride];
+
+    const uint32_t sub = blockIdx.x / args.blocksPerSub;
+    const uint32_t blk = blockIdx.x - sub * args.blocksPerSub;
+    const uint32_t g = sub / args.nSub;
+    const uint32_t c = sub - g * args.nSub;
+
+    const uint64_t gBeg = static_cast<uint64_t>(g) * args.groupLen;
+    if (gBeg >= args.total) {
+        return;
+    }
+    const uint64_t gLen = (args.total - gBeg < args.groupLen) ? args.total - gBeg : args.groupLen;
+    const uint64_t sBeg = static_cast<uint64_t>(c) * args.subLen;
+    uint64_t sEnd = (c == args.nSub - 1) ? gLen : sBeg + args.subLen;
+    sEnd = sEnd < gLen ? sEnd : gLen;
+    if (sBeg >= sEnd) {
+        return;
+    }
+    const uint64_t len = sEnd - sBeg;
+
+    const uint8_t* prog = args.prog + static_cast<uint64_t>(g * args.progGroupStride + c * args.progSubStride) * kProgStride;
+    for (uint32_t i = threadIdx.x; i < kProgStride / 4; i += kThreads) {
+        reinterpret_cast<uint32_t*>(sprog)[i] = reinterpret_cast<const uint32_t*>(prog)[i];
+    }
+    __syncthreads();
+
+    const uint64_t srcOff = static_cast<uint64_t>(g) * args.srcGroupStride + sBeg;
+    const uint64_t dstOff = args.dstOwn ? sBeg : static_cast<uint64_t>(g) * args.dstGroupStride + sBeg;
+    const uint64_t stride = static_cast<uint64_t>(args.blocksPerSub) * kThreads;
+    const uint64_t first = static_cast<uint64_t>(blk) * kThreads + threadIdx.x;
+
+    // 128-bit body when every address is 16-byte aligned, then element by element for what is left
+    // (fewer than W elements) or for the whole range when it is not.
+    uint64_t done = 0;
+    if (args.vecOk) {
+        const uint64_t nVec = len / W;
+        for (uint64_t v = first; v < nVec; v += stride) {
+            ReduceOne<E, W>(sprog, args, srcOff + v * W, dstOff + v * W, g);
+        }
+        done = nVec * W;
+    }
+    for (uint64_t e = done + first; e < len; e += stride) {
+        ReduceOne<E, 1>(sprog, args, srcOff + e, dstOff + e, g);
+    }
+}
+
+using ReduceKernelFn = void (*)(const ReduceArgs);
+
+}  // namespace detail
+
+// One translation unit per data type defines its selector (nullptr = combination not offered).
+detail::ReduceKernelFn SelectReduceI8(int op);
+detail::ReduceKernelFn SelectReduceI16(int op);
+detail::ReduceKernelFn SelectReduceI32(int op);
+detail::ReduceKernelFn SelectReduceI64(int op);
+detail::ReduceKernelFn SelectReduceU64(int op);
+detail::ReduceKernelFn SelectReduceF16(int op);
+detail::ReduceKernelFn SelectReduceBf16(int op);
+detail::ReduceKernelFn SelectReduceF32(int op);
+detail::ReduceKernelFn SelectReduceF64(int op);
+
+#define HCCL_AMD_DEFINE_SELECT4(NAME, SUM_T, PROD_T, MAX_T, MIN_T)                 \
+    detail::ReduceKernelFn NAME(int op)                                           \
+    {                                                                             \
+        switch (op) {                                                             \
+            case detail::kSum: return detail::ReduceKernel<SUM_T>;                \
+            case detail::kProd: return detail::ReduceKernel<PROD_T>;              \
+            case detail::kMax: return detail::ReduceKernel<MAX_T>;                \
+            case detail::kMin: return detail::ReduceKernel<MIN_T>;                \
+            default: return nullptr;                                              \
+        }                                                                         \
+    }
+
+#define HCCL_AMD_DEFINE_SELECT3(NAME, SUM_T, MAX_T, MIN_T)                         \
+    detail::ReduceKernelFn NAME(int op)                                           \
+    {                                                                             \
+        switch (op) {                                                             \
+            case detail::kSum: return detail::ReduceKernel<SUM_T>;                \
+            case detail::kMax: return detail::ReduceKernel<MAX_T>;                \
+            case detail::kMin: return detail::ReduceKernel<MIN_T>;                \
+            default: return nullptr;                                              \
+        }                                                                         \
+    }
+
+}  // namespace hccl_amd

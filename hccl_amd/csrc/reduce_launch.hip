@@ -1,0 +1,30 @@
+// Dispatch of the fused reduce kernel by (data type, reduce op).
+#include "reduce_kernel_impl.h"
+
+namespace hccl_amd {
+
+hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t nBlocks,
+                        hipStream_t stream)
+{
+    detail::ReduceKernelFn fn = nullptr;
+    const int o = static_cast<int>(op);
+    switch (dtype) {
+        case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8(o); break;
+        case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16(o); break;
+        case HCCL_DATA_TYPE_INT32: fn = SelectReduceI32(o); break;
+        case HCCL_DATA_TYPE_INT64: fn = SelectReduceI64(o); break;
+        case HCCL_DATA_TYPE_UINT64: fn = SelectReduceU64(o); break;
+        case HCCL_DATA_TYPE_FP16: fn = SelectReduceF16(o); break;
+        case HCCL_DATA_TYPE_BFP16: fn = SelectReduceBf16(o); break;
+        case HCCL_DATA_TYPE_FP32: fn = SelectReduceF32(o); break;
+        case HCCL_DATA_TYPE_FP64: fn = SelectReduceF64(o); break;
+        default: break;
+    }
+    if (fn == nullptr || nBlocks == 0) {
+        return hipErrorInvalidValue;
+    }
+    hipLaunchKernelGGL(fn, dim3(nBlocks), dim3(detail::kThreads), 0, stream, args);
+    return hipGetLastError();
+}
+
+}  // namespace hccl_amd

@@ -1,0 +1,103 @@
+"""Helpers for the GPU parity tests: a loopback world whose per-rank buffers are separate HBM
+allocations, driven through the C ABI exactly as a single-threaded caller would (one call per rank
+inside a group, all on one non-default stream)."""
+import ctypes
+
+import numpy as np
+
+import hccl_amd
+from hccl_amd import Algo, OpKind
+
+ALGO_BY_NAME = {"mesh": Algo.MESH, "ring": Algo.RING, "rhd": Algo.RHD, "nhr": Algo.NHR,
+                "order_preserved": Algo.ORDER_PRESERVED, "aiv_mesh": Algo.AIV_MESH}
+
+
+def require_library_on_gpu():
+    """The GPU tests are meaningless without the native library: fail, never skip."""
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    hccl_amd.lib()
+
+
+def to_dev(arr, pad_front=0):
+    """Uploads a numpy array as raw bytes.  pad_front shifts the payload to break 16-byte alignment."""
+    import torch
+    raw = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+    t = torch.empty(raw.size + pad_front + 64, dtype=torch.uint8, device="cuda")
+    view = t[pad_front:pad_front + raw.size]
+    if raw.size:
+        view.copy_(torch.from_numpy(raw.copy()))
+    return view
+
+
+def dev_zeros(nbytes, pad_front=0, fill=0xAB):
+    import torch
+    t = torch.full((nbytes + pad_front + 64,), fill, dtype=torch.uint8, device="cuda")
+    return t[pad_front:pad_front + nbytes]
+
+
+def to_host(t, np_dtype):
+    return t.cpu().numpy().view(np_dtype).copy()
+
+
+class World:
+    def __init__(self, n):
+        import torch
+        self.n = n
+        self.comms = hccl_amd.comm_init_all(n)
+        self.stream = torch.cuda.Stream()
+
+    def close(self):
+        import torch
+        torch.cuda.synchronize()
+        for c in self.comms:
+            hccl_amd.comm_destroy(c)
+
+    def set_algo(self, kind, name):
+        hccl_amd.set_algo(self.comms[0], kind, ALGO_BY_NAME[name])
+
+    def sync(self):
+        self.stream.synchronize()
+
+    def all_reduce(self, sends, recvs, count, dtype, op, algo="mesh"):
+        self.set_algo(OpKind.ALL_REDUCE, algo)
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.all_reduce(self.comms[r], sends[r], recvs[r], count, dtype, op, self.stream)
+        self.sync()
+
+    def reduce_scatter(self, sends, recvs, recv_count, dtype, op, algo="mesh"):
+        self.set_algo(OpKind.REDUCE_SCATTER, algo)
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.reduce_scatter(self.comms[r], sends[r], recvs[r], recv_count, dtype, op, self.stream)
+        self.sync()
+
+    def all_gather(self, sends, recvs, send_count, dtype):
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.all_gather(self.comms[r], sends[r], recvs[r], send_count, dtype, self.stream)
+        self.sync()
+
+    def all_gather_v(self, sends, recvs, counts, displs, dtype):
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.all_gather_v(self.comms[r], sends[r], int(counts[r]), recvs[r], counts, displs, dtype,
+                                      self.stream)
+        self.sync()
+
+    def all_to_all_v(self, sends, send_counts, sdispls, recvs, recv_counts, rdispls, dtype):
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.all_to_all_v(self.comms[r], sends[r], send_counts[r], sdispls[r], dtype, recvs[r],
+                                      recv_counts[r], rdispls[r], dtype, self.stream)
+        self.sync()
+
+
+def same_bits_nan_class(got, want, float_view=None):
+    """Bit equality; where float_view is given, positions that are NaN on both sides only need to be NaN."""
+    if float_view is None:
+        return np.array_equal(got, want)
+    g, w = float_view(got), float_view(want)
+    both = np.isnan(g) & np.isnan(w)
+    return np.array_equal(got[~both], want[~both]) and np.array_equal(np.isnan(g), np.isnan(w))

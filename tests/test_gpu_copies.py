@@ -1,0 +1,207 @@
+"""GPU parity of the slice-copy (AllGather / AllGatherV) and pack / unpack (AlltoAllV) kernels
+against the CPU oracle: bit-exact, including bytes the collective must not touch."""
+import threading
+
+import numpy as np
+import pytest
+
+import hccl_amd
+import oracle
+from hccl_amd import HcclDataType as DT, HcclReduceOp as OP
+
+from gpu_util import World, dev_zeros, require_library_on_gpu, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+FILL = 0xAB
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _native_library():
+    require_library_on_gpu()
+
+
+def rand_bytes(rng, nbytes):
+    return rng.integers(0, 256, nbytes, dtype=np.uint8)
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 8, 64])
+@pytest.mark.parametrize("dtype,esz", [(DT.UINT8, 1), (DT.BFP16, 2), (DT.FP32, 4), (DT.INT64, 8)])
+def test_all_gather(n, dtype, esz):
+    w = World(n)
+    try:
+        rng = np.random.default_rng(n * 10 + esz)
+        for count in (1, 7, 4096, 70_001):
+            ins = [rand_bytes(rng, count * esz) for _ in range(n)]
+            want = [np.zeros(n * count * esz, dtype=np.uint8) for _ in range(n)]
+            assert oracle.all_gather(ins, want, count, int(dtype)) == 0
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(n * count * esz) for _ in range(n)]
+            w.all_gather(sends, recvs, count, dtype)
+            for r in range(n):
+                assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), (n, count, r)
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("n", [2, 6, 8, 64])
+def test_all_gather_v_unordered_holes_and_odd_offsets(n):
+    w = World(n)
+    try:
+        rng = np.random.default_rng(n)
+        esz = 2
+        for trial in range(3):
+            counts = rng.integers(0, 5000, n).astype(np.uint64)
+            counts[rng.integers(0, n)] = 0                      # an empty contribution
+            if trial == 2:
+                counts = (counts // 8) * 8                      # all 16-byte multiples: vector path
+            order = rng.permutation(n)
+            displs = np.zeros(n, dtype=np.uint64)
+            off = int(rng.integers(0, 4))
+            for j in order:                                     # shuffled layout with gaps
+                displs[j] = off
+                off += int(counts[j]) + (0 if trial == 2 else int(rng.integers(0, 5)))
+            total = off + 3
+            ins = [rand_bytes(rng, max(int(c), 1) * esz) for c in counts]
+            want = [np.full(total * esz, FILL, dtype=np.uint8) for _ in range(n)]
+            assert oracle.all_gather_v(ins, want, counts, displs, int(DT.FP16)) == 0
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(total * esz, fill=FILL) for _ in range(n)]
+            w.all_gather_v(sends, recvs, counts, displs, DT.FP16)
+            for r in range(n):
+                assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), (n, trial, r)
+    finally:
+        w.close()
+
+
+def a2a_case(rng, n, esz, max_count, aligned):
+    send_counts = rng.integers(0, max_count, size=(n, n)).astype(np.uint64)
+    send_counts[rng.random((n, n)) < 0.15] = 0
+    if aligned:
+        send_counts = (send_counts // (16 // esz)) * (16 // esz)
+    recv_counts = send_counts.T.copy()
+    sdispls = np.zeros((n, n), dtype=np.uint64)
+    rdispls = np.zeros((n, n), dtype=np.uint64)
+    for r in range(n):
+        for tab, cnts in ((sdispls, send_counts), (rdispls, recv_counts)):
+            off = 0
+            for j in (range(n) if aligned else rng.permutation(n)):
+                tab[r, j] = off
+                off += int(cnts[r, j]) + (0 if aligned else int(rng.integers(0, 4)))
+    in_sz = int((sdispls + send_counts).max()) + 1
+    out_sz = int((rdispls + recv_counts).max()) + 1
+    return send_counts, sdispls, recv_counts, rdispls, in_sz, out_sz
+
+
+@pytest.mark.parametrize("n", [2, 3, 8, 64])
+@pytest.mark.parametrize("aligned", [True, False])
+def test_all_to_all_v(n, aligned):
+    w = World(n)
+    try:
+        rng = np.random.default_rng(n + 100 * aligned)
+        esz = 2
+        for max_count in (9, 3000, 40_000 if n <= 8 else 6_000):
+            sc, sd, rc, rd, in_sz, out_sz = a2a_case(rng, n, esz, max_count, aligned)
+            ins = [rand_bytes(rng, in_sz * esz) for _ in range(n)]
+            want = [np.full(out_sz * esz, FILL, dtype=np.uint8) for _ in range(n)]
+            assert oracle.all_to_all_v(ins, want, sc, sd, rc, rd, int(DT.BFP16)) == 0
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(out_sz * esz, fill=FILL) for _ in range(n)]
+            w.all_to_all_v(sends, sc, sd, recvs, rc, rd, DT.BFP16)
+            for r in range(n):
+                assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), (n, aligned, max_count, r)
+    finally:
+        w.close()
+
+
+def test_all_to_all_v_moe_shape_zipf_small():
+    """The MoE-dispatch shape of the headline AlltoAllV configuration at 1/64 of its token count:
+    64 ranks, hidden 7168 bf16, per-destination token counts multinomial over Zipf(1.1) weights."""
+    n, hidden, tokens = 64, 7168, 256
+    w = World(n)
+    try:
+        rng = np.random.default_rng(0xC0FFEE + 4000)
+        wts = 1.0 / np.arange(1, n + 1) ** 1.1
+        wts /= wts.sum()
+        tok = np.stack([rng.multinomial(tokens, wts) for _ in range(n)]).astype(np.uint64)
+        sc = tok * hidden
+        rc = sc.T.copy()
+        sd = np.cumsum(sc, axis=1) - sc
+        rd = np.cumsum(rc, axis=1) - rc
+        ins = [rng.integers(0, 65536, tokens * hidden, dtype=np.uint16) for _ in range(n)]
+        outs = [np.zeros(int(rc[i].sum()), dtype=np.uint16) for i in range(n)]
+        assert oracle.all_to_all_v(ins, outs, sc, sd, rc, rd, int(DT.BFP16)) == 0
+        sends = [to_dev(x) for x in ins]
+        recvs = [dev_zeros(max(o.nbytes, 2)) for o in outs]
+        w.all_to_all_v(sends, sc, sd, recvs, rc, rd, DT.BFP16)
+        for i in range(n):
+            assert np.array_equal(to_host(recvs[i], np.uint16)[:outs[i].size], outs[i]), i
+    finally:
+        w.close()
+
+
+def test_rendezvous_mismatch_and_launch_time_checks():
+    w = World(2)
+    try:
+        a = [to_dev(np.arange(16, dtype=np.float32)) for _ in range(2)]
+        b = [dev_zeros(64) for _ in range(2)]
+        with hccl_amd.group():
+            hccl_amd.all_reduce(w.comms[0], a[0], b[0], 16, DT.FP32, OP.SUM, w.stream)
+            with pytest.raises(hccl_amd.HcclError) as e:
+                hccl_amd.all_reduce(w.comms[1], a[1], b[1], 8, DT.FP32, OP.SUM, w.stream)   # different count
+            assert e.value.code == 1
+        # recvCounts of rank 0 disagree with sendCounts of rank 1
+        sc = np.array([[1, 2], [3, 4]], dtype=np.uint64)
+        rc = np.array([[1, 5], [2, 4]], dtype=np.uint64)
+        z = np.zeros((2, 2), dtype=np.uint64)
+        with hccl_amd.group():
+            hccl_amd.all_to_all_v(w.comms[0], a[0], sc[0], z[0], DT.FP32, b[0], rc[0], z[0], DT.FP32, w.stream)
+            with pytest.raises(hccl_amd.HcclError) as e:
+                hccl_amd.all_to_all_v(w.comms[1], a[1], sc[1], z[1], DT.FP32, b[1], rc[1], z[1], DT.FP32, w.stream)
+            assert e.value.code == 1
+        # the world is still usable afterwards
+        with hccl_amd.group():
+            for r in range(2):
+                hccl_amd.all_reduce(w.comms[r], a[r], b[r], 16, DT.FP32, OP.SUM, w.stream)
+        w.sync()
+        assert np.array_equal(to_host(b[1], np.float32), 2 * np.arange(16, dtype=np.float32))
+    finally:
+        w.close()
+
+
+def test_one_host_thread_per_rank_with_own_streams():
+    """The calling pattern of the reference's examples: a thread per rank, each with its own stream,
+    calls block until every rank has arrived (examples/02_collectives/01_allreduce/main.cc:76-85)."""
+    import torch
+    n, count = 4, 300_000
+    info = hccl_amd.get_root_info()
+    rng = np.random.default_rng(9)
+    ins = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]
+    want = ins[0].copy()
+    for r in range(1, n):
+        want = ins[r] + want
+    results, errors = [None] * n, []
+
+    def rank_main(r):
+        try:
+            comm = hccl_amd.comm_init_root_info(n, info, r)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                send = to_dev(ins[r])
+                recv = dev_zeros(4 * count)
+            stream.synchronize()
+            for _ in range(3):
+                hccl_amd.all_reduce(comm, send, recv, count, DT.FP32, OP.SUM, stream)
+            stream.synchronize()
+            results[r] = to_host(recv, np.float32)
+            hccl_amd.comm_destroy(comm)
+        except Exception as exc:   # surfaced below
+            errors.append((r, exc))
+
+    threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(n)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not errors, errors
+    for r in range(n):
+        assert np.array_equal(results[r].view(np.uint32), want.view(np.uint32)), r

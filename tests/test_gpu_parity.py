@@ -1,0 +1,267 @@
+"""GPU parity: the HIP data plane, called through the C ABI, against the CPU oracle on the same seeded
+inputs.  Bar: bit-exact for integers, copies / packs, fp32 / fp64 and every MAX / MIN; fp16 / bf16 SUM
+are compared bit-exactly with the oracle's fp32-accumulate mode and within 1 ulp of a float64
+reference (the tolerance the task states for half precision).  A NaN produced by arithmetic only has
+to be a NaN on both sides (payloads of arithmetic NaNs are machine specific)."""
+import numpy as np
+import pytest
+
+import oracle
+from hccl_amd import HcclDataType as DT, HcclReduceOp as OP, OpKind
+
+from gpu_util import World, dev_zeros, require_library_on_gpu, same_bits_nan_class, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+SUM, PROD, MAX, MIN = range(4)
+NP = {DT.INT8: np.int8, DT.INT16: np.int16, DT.INT32: np.int32, DT.INT64: np.int64, DT.UINT64: np.uint64,
+      DT.FP16: np.uint16, DT.BFP16: np.uint16, DT.FP32: np.float32, DT.FP64: np.float64}
+FLOAT_VIEW = {DT.FP16: lambda a: a.view(np.float16), DT.BFP16: oracle.bf16_bits_to_fp32,
+              DT.FP32: lambda a: a, DT.FP64: lambda a: a}
+REDUCE_TYPES = [DT.INT8, DT.INT16, DT.INT32, DT.INT64, DT.UINT64, DT.FP16, DT.BFP16, DT.FP32, DT.FP64]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _native_library():
+    require_library_on_gpu()
+
+
+def gen(dtype, op, rng, count):
+    """Inputs that make a wrong order, a wrong operand role or a wrong rounding visible."""
+    npdt = NP[dtype]
+    if dtype in (DT.INT8, DT.INT16, DT.INT32, DT.INT64, DT.UINT64):
+        info = np.iinfo(npdt)
+        a = rng.integers(info.min, info.max, count, dtype=npdt, endpoint=True)
+        if op == PROD:   # keep half of the lanes small so that products stay informative
+            small = rng.choice(np.array([-2, -1, 1, 2, 3] if info.min < 0 else [1, 2, 3], dtype=npdt), count)
+            a = np.where(rng.random(count) < 0.5, small, a)
+        return a
+    if op in (MAX, MIN):
+        pools = {DT.FP32: np.array([0, 0x80000000, 0x7FC00001, 0x7FC00002, 0xFFC00003, 0x3F800000, 0xBF800000,
+                                    0x7F800000, 0xFF800000, 0x00000001], dtype=np.uint32),
+                 DT.FP64: np.array([0, 1 << 63, 0x7FF8000000000001, 0xFFF8000000000003, 0x3FF0000000000000,
+                                    0xBFF0000000000000, 0x7FF0000000000000], dtype=np.uint64),
+                 DT.FP16: np.array([0, 0x8000, 0x7E01, 0x7E02, 0xFE03, 0x3C00, 0xBC00, 0x7C00, 0xFC00, 0x0001, 0x7D01],
+                                   dtype=np.uint16),
+                 DT.BFP16: np.array([0, 0x8000, 0x7FC1, 0x7FC2, 0xFFC3, 0x3F80, 0xBF80, 0x7F80, 0xFF80, 0x0001, 0x7FA1],
+                                    dtype=np.uint16)}
+        pool = pools[dtype]
+        a = pool[rng.integers(0, pool.size, count)]
+        rnd = rng.standard_normal(count)
+        mix = rng.random(count) < 0.5
+        if dtype == DT.FP32:
+            return np.where(mix, rnd.astype(np.float32).view(np.uint32), a).view(np.float32)
+        if dtype == DT.FP64:
+            return np.where(mix, rnd.view(np.uint64), a).view(np.float64)
+        if dtype == DT.FP16:
+            return np.where(mix, rnd.astype(np.float16).view(np.uint16), a)
+        return np.where(mix, oracle.np_fp32_to_bf16_bits(rnd.astype(np.float32)), a)
+    scale = 10.0 ** rng.integers(-3, 3, count) if op == SUM else 1.0 + 0.0 * rng.random(count)
+    base = rng.standard_normal(count) * scale
+    if op == PROD:
+        base = 1.0 + 0.5 * rng.standard_normal(count)
+    if dtype == DT.FP32:
+        a = base.astype(np.float32)
+        a[::97] = np.float32(1e-41)      # fp32 subnormals must survive
+        a[5::101] = np.float32(np.inf)
+        return a
+    if dtype == DT.FP64:
+        return base.astype(np.float64)
+    if dtype == DT.FP16:
+        h = base.astype(np.float16)
+        h[::89] = np.float16(6e-8)       # fp16 subnormal
+        h[7::103] = np.float16(60000.0)  # sums overflow to Inf
+        return h.view(np.uint16)
+    return oracle.np_fp32_to_bf16_bits(base.astype(np.float32))
+
+
+def check(dtype, op, got, want, what):
+    fv = FLOAT_VIEW.get(dtype)
+    if fv is not None and op in (SUM, PROD):
+        ok = same_bits_nan_class(got, want, fv)
+    else:
+        ok = np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    if not ok:
+        diff = np.nonzero(got.view(np.uint8).reshape(got.size, -1) != want.view(np.uint8).reshape(want.size, -1))[0]
+        diff = np.unique(diff)
+        raise AssertionError("%s: %d of %d elements differ, first at %s (got %r want %r)" % (
+            what, diff.size, got.size, diff[:4], got[diff[:4]], want[diff[:4]]))
+
+
+def run_all_reduce(world, dtype, op, count, algo, seed, pad=0, in_place=False):
+    rng = np.random.default_rng(seed)
+    n = world.n
+    ins = [gen(dtype, op, rng, count) for _ in range(n)]
+    want = [np.zeros(count, dtype=NP[dtype]) for _ in range(n)]
+    assert oracle.all_reduce(ins, want, count, int(dtype), op, acc=oracle.ACC_FP32, algo=algo) == 0
+    sends = [to_dev(x, pad) for x in ins]
+    recvs = sends if in_place else [dev_zeros(x.nbytes, pad) for x in ins]
+    world.all_reduce(sends, recvs, count, dtype, op, algo)
+    for r in range(n):
+        check(dtype, op, to_host(recvs[r], NP[dtype]), want[r],
+              "all_reduce %s %s n=%d count=%d algo=%s rank=%d" % (dtype.name, OP(op).name, n, count, algo, r))
+
+
+def run_reduce_scatter(world, dtype, op, c, algo, seed, pad=0):
+    rng = np.random.default_rng(seed)
+    n = world.n
+    ins = [gen(dtype, op, rng, n * c) for _ in range(n)]
+    want = [np.zeros(c, dtype=NP[dtype]) for _ in range(n)]
+    assert oracle.reduce_scatter(ins, want, c, int(dtype), op, acc=oracle.ACC_FP32, algo=algo) == 0
+    sends = [to_dev(x, pad) for x in ins]
+    recvs = [dev_zeros(c * ins[0].itemsize, pad) for _ in range(n)]
+    world.reduce_scatter(sends, recvs, c, dtype, op, algo)
+    for r in range(n):
+        check(dtype, op, to_host(recvs[r], NP[dtype]), want[r],
+              "reduce_scatter %s %s n=%d c=%d algo=%s rank=%d" % (dtype.name, OP(op).name, n, c, algo, r))
+
+
+# ---------------------------------------------------------------------------------------------
+# Type / op matrix
+# ---------------------------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def world8():
+    w = World(8)
+    yield w
+    w.close()
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+@pytest.mark.parametrize("op", [SUM, PROD, MAX, MIN])
+def test_all_reduce_type_op_matrix(world8, dtype, op):
+    if op == PROD and dtype in (DT.INT16, DT.BFP16):
+        pytest.skip("PROD is not defined for this type (reference op_common.cc:4392-4413)")
+    run_all_reduce(world8, dtype, op, 40_007, "mesh", seed=int(dtype) * 10 + op)
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+@pytest.mark.parametrize("op", [SUM, MAX])
+def test_reduce_scatter_type_matrix(world8, dtype, op):
+    run_reduce_scatter(world8, dtype, op, 8_192 + 16, "mesh", seed=500 + int(dtype) * 10 + op)
+
+
+# ---------------------------------------------------------------------------------------------
+# Algorithms x rank counts x ragged counts (the sweep of the reference's vector-core unit tests:
+# ranks {1,2,3,4,8,16,32}, counts not divisible by the rank count and smaller than it)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 6, 7, 8, 16, 33, 64])
+def test_all_reduce_algorithms_and_ragged_counts(n):
+    w = World(n)
+    try:
+        for algo in ("mesh", "ring", "rhd", "nhr", "order_preserved"):
+            for count in (1, 3, 17, 129, 1023, 4093, 65_543):
+                run_all_reduce(w, DT.FP32, SUM, count, algo, seed=n * 1000 + count)
+            run_all_reduce(w, DT.FP32, MAX, 2_051, algo, seed=n)
+            run_all_reduce(w, DT.BFP16, SUM, 4_099, algo, seed=n + 1)
+            run_all_reduce(w, DT.INT32, PROD, 1_025, algo, seed=n + 2)
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 6, 8, 16, 64])
+def test_reduce_scatter_algorithms_and_ragged_counts(n):
+    w = World(n)
+    try:
+        for algo in ("mesh", "ring", "nhr", "rhd", "order_preserved", "aiv_mesh"):
+            for c in (1, 3, 17, 129, 1024, 4093):
+                run_reduce_scatter(w, DT.FP32, SUM, c, algo, seed=n * 2000 + c)
+            run_reduce_scatter(w, DT.FP32, MIN, 515, algo, seed=n + 3)
+            run_reduce_scatter(w, DT.FP16, SUM, 2_048, algo, seed=n + 4)
+    finally:
+        w.close()
+
+
+def test_unaligned_buffers_and_in_place(world8):
+    for pad in (2, 4, 8):          # payload starts 2 / 4 / 8 bytes past a 16-byte boundary
+        run_all_reduce(world8, DT.FP16, SUM, 5_001, "mesh", seed=pad, pad=pad)
+        run_reduce_scatter(world8, DT.BFP16, SUM, 999, "mesh", seed=pad + 10, pad=pad)
+    run_all_reduce(world8, DT.FP32, SUM, 70_001, "mesh", seed=77, in_place=True)
+    run_all_reduce(world8, DT.INT64, MAX, 9_999, "rhd", seed=78, in_place=True)
+
+
+# ---------------------------------------------------------------------------------------------
+# BASELINE configurations (C1 at its real size; the others at sizes the oracle finishes in seconds;
+# their full sizes are covered by tests/test_gpu_full_size.py through size-independent properties)
+# ---------------------------------------------------------------------------------------------
+def test_config1_all_reduce_fp32_n8_rank_order(world8):
+    rng = np.random.default_rng(0xC0FFEE + 1000)
+    count = 1_048_576
+    ins = [rng.uniform(-1.0, 1.0, count).astype(np.float32) for _ in range(8)]
+    want = ins[0].copy()
+    for r in range(1, 8):
+        want = ins[r] + want                      # (((x0+x1)+x2)...+x7)
+    o = [np.zeros(count, dtype=np.float32) for _ in range(8)]
+    assert oracle.all_reduce(ins, o, count, 4, SUM, algo="ring") == 0
+    assert np.array_equal(o[0].view(np.uint32), want.view(np.uint32))
+    sends = [to_dev(x) for x in ins]
+    recvs = [dev_zeros(x.nbytes) for x in ins]
+    world8.all_reduce(sends, recvs, count, DT.FP32, SUM, "ring")
+    for r in range(8):
+        assert np.array_equal(to_host(recvs[r], np.uint32), want.view(np.uint32))
+
+
+def test_config2_reduce_scatter_bf16_n8(world8):
+    rng = np.random.default_rng(0xC0FFEE + 2000)
+    c = 1 << 20
+    f = [rng.standard_normal(8 * c).astype(np.float32) for _ in range(8)]
+    ins = [oracle.np_fp32_to_bf16_bits(x) for x in f]
+    sends = [to_dev(x) for x in ins]
+    for algo in ("ring", "mesh"):
+        want = [np.zeros(c, dtype=np.uint16) for _ in range(8)]
+        assert oracle.reduce_scatter(ins, want, c, 11, SUM, acc=oracle.ACC_FP32, algo=algo) == 0
+        recvs = [dev_zeros(2 * c) for _ in range(8)]
+        world8.reduce_scatter(sends, recvs, c, DT.BFP16, SUM, algo)
+        w64 = np.stack([oracle.bf16_bits_to_fp32(x).astype(np.float64) for x in ins])
+        for k in range(8):
+            got = to_host(recvs[k], np.uint16)
+            assert np.array_equal(got, want[k]), (algo, k)
+            # within 1 ulp of the correctly rounded exact sum
+            exact = oracle.np_fp32_to_bf16_bits(w64[:, k * c:(k + 1) * c].sum(axis=0).astype(np.float32))
+            d = np.abs(got.astype(np.int32) - exact.astype(np.int32))
+            assert d[(got >> 15) == (exact >> 15)].max() <= 1
+
+
+def test_config3_all_reduce_int32_n16_max_and_prod():
+    w = World(16)
+    try:
+        rng = np.random.default_rng(0xC0FFEE + 3000)
+        count = 1 << 20
+        mx = [rng.integers(-2 ** 31, 2 ** 31 - 1, count, dtype=np.int32, endpoint=True) for _ in range(16)]
+        pr = [rng.choice(np.array([-2, -1, 1, 2], dtype=np.int32), count) for _ in range(16)]
+        for ins, op in ((mx, MAX), (pr, PROD)):
+            stack = np.stack(ins).astype(np.int64)
+            if op == MAX:
+                want = stack.max(axis=0).astype(np.int32)
+            else:
+                acc = np.ones(count, dtype=np.uint64)
+                for x in ins:
+                    acc = (acc * x.astype(np.int64).astype(np.uint64)) & np.uint64(0xFFFFFFFF)
+                want = acc.astype(np.uint32).view(np.int32)
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(4 * count) for _ in ins]
+            w.all_reduce(sends, recvs, count, DT.INT32, op, "mesh")
+            for r in (0, 7, 15):
+                assert np.array_equal(to_host(recvs[r], np.int32), want)
+    finally:
+        w.close()
+
+
+def test_config5a_all_reduce_fp16_rhd_n6():
+    w = World(6)
+    try:
+        rng = np.random.default_rng(0xC0FFEE + 5000)
+        count = (1 << 20) + 5           # not a multiple of 6: exercises the padded remainder
+        ins = [(rng.standard_normal(count) * 0.5).astype(np.float16).view(np.uint16) for _ in range(6)]
+        x = [h.view(np.float16).astype(np.float32) for h in ins]
+        tree = ((x[0] + x[2]) + x[4]) + ((x[1] + x[3]) + x[5])      # the p = 6 association, fp32 accumulate
+        want = tree.astype(np.float16).view(np.uint16)
+        o = [np.zeros(count, dtype=np.uint16) for _ in range(6)]
+        assert oracle.all_reduce(ins, o, count, 3, SUM, acc=oracle.ACC_FP32, algo="rhd") == 0
+        assert np.array_equal(o[3], want)
+        sends = [to_dev(h) for h in ins]
+        recvs = [dev_zeros(2 * count) for _ in ins]
+        w.all_reduce(sends, recvs, count, DT.FP16, SUM, "rhd")
+        for r in range(6):
+            assert np.array_equal(to_host(recvs[r], np.uint16), want)
+    finally:
+        w.close()

@@ -1,0 +1,257 @@
+"""CPU-only checks of the shipped library's host logic: it loads, exports what include/hccl.h
+declares, rejects bad arguments with the reference's return codes before touching a GPU, and its
+fold programs (the reduction plans the kernels execute) reproduce the oracle's results when
+evaluated with numpy."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import hccl_amd
+from hccl_amd import Algo, HcclDataType as DT, HcclReduceOp as OP, OpKind
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+F32, U64 = 4, 6
+SUM, PROD, MAX, MIN = range(4)
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "hccl.h")).read()
+    names = set(re.findall(r"\b(Hccl[A-Za-z0-9]+)\s*\(", header))
+    assert {"HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV"} <= names
+    L = ctypes.CDLL(hccl_amd.LIB_PATH)
+    for n in sorted(names):
+        assert hasattr(L, n), n
+
+
+# ---- fold programs ----------------------------------------------------------------------------------
+def f32_fold(src, dst, op):
+    with np.errstate(all="ignore"):
+        if op == SUM:
+            return src + dst
+        if op == MAX:
+            return np.where(src < dst, dst, src)
+        return np.where(dst < src, dst, src)
+
+
+def run_program(prog, leaf, op):
+    """Evaluates a fold program; returns the value of the outermost level."""
+    pos = 0
+
+    def level():
+        nonlocal pos
+        acc = None
+        while True:
+            tok = prog[pos]
+            pos += 1
+            if tok in (0x81, 0xFF):
+                return acc
+            if tok == 0x80:
+                sub = level()
+                acc = sub if acc is None else f32_fold(sub, acc, op)
+            else:
+                n = tok & 0x3F if tok >= 0xC0 else 1
+                ranks = prog[pos:pos + n] if tok >= 0xC0 else [tok]
+                pos += n if tok >= 0xC0 else 0
+                for r in ranks:
+                    v = leaf(r)
+                    acc = v if acc is None else f32_fold(v, acc, op)
+
+    out = level()
+    assert pos == len(prog) and prog[-1] == 0xFF
+    return out
+
+
+def program_ranks(prog):
+    ranks, i = [], 0
+    while i < len(prog):
+        t = prog[i]
+        i += 1
+        if t >= 0xC0 and t != 0xFF:
+            ranks += list(prog[i:i + (t & 0x3F)])
+            i += t & 0x3F
+        elif t < 0x40:
+            ranks.append(t)
+    return ranks
+
+
+def wide(rng, n, count):
+    return [(rng.standard_normal(count) * 10.0 ** rng.integers(-6, 6, count)).astype(np.float32) for _ in range(n)]
+
+
+def tricky(rng, n, count):
+    pool = np.array([0, 0x80000000, 0x7FC00001, 0x7FC00002, 0xFFC00003, 0x3F800000, 0xBF800000], dtype=np.uint32)
+    return [pool[rng.integers(0, pool.size, count)].view(np.float32).copy() for _ in range(n)]
+
+
+def same(a, b):
+    nan = np.isnan(a) & np.isnan(b)
+    return np.array_equal(a.view(np.uint32)[~nan], b.view(np.uint32)[~nan]) and np.array_equal(np.isnan(a), np.isnan(b))
+
+
+RANKS = [1, 2, 3, 5, 6, 7, 8, 12, 16, 33, 64]
+ALGO_NAME = {Algo.MESH: "mesh", Algo.RING: "ring", Algo.RHD: "rhd", Algo.NHR: "nhr",
+             Algo.ORDER_PRESERVED: "order_preserved", Algo.AIV_MESH: "aiv_mesh"}
+
+
+@pytest.mark.parametrize("n", RANKS)
+def test_every_program_uses_every_rank_once(n):
+    for kind in (OpKind.ALL_REDUCE, OpKind.REDUCE_SCATTER):
+        for algo in Algo:
+            if kind == OpKind.ALL_REDUCE and algo == Algo.AIV_MESH:
+                continue
+            for prog in hccl_amd.fold_programs(kind, algo, n):
+                assert sorted(program_ranks(prog)) == list(range(n)), (kind, algo, n)
+                assert len(prog) <= 320
+
+
+@pytest.mark.parametrize("n", RANKS)
+@pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED, Algo.AIV_MESH])
+def test_reduce_scatter_programs_match_oracle(orc, n, algo):
+    progs = hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, algo, n)
+    c = 2 * n + 5
+    for op, gen in ((SUM, wide), (MAX, tricky), (MIN, tricky)):
+        rng = np.random.default_rng(1000 * n + 10 * int(algo) + op)
+        ins = gen(rng, n, n * c)
+        outs = [np.zeros(c, dtype=np.float32) for _ in range(n)]
+        assert orc.reduce_scatter(ins, outs, c, F32, op, algo=ALGO_NAME[algo]) == 0
+        for k in range(n):
+            if algo == Algo.AIV_MESH:
+                per = c // n
+                got = np.zeros(c, dtype=np.float32)
+                for ch in range(n):
+                    lo, hi = ch * per, (c if ch == n - 1 else (ch + 1) * per)
+                    if hi > lo:
+                        got[lo:hi] = run_program(progs[ch], lambda r: ins[r][k * c + lo:k * c + hi], op)
+            else:
+                prog = progs[k] if len(progs) > 1 else progs[0]
+                got = run_program(prog, lambda r: ins[r][k * c:(k + 1) * c], op)
+            assert same(got, outs[k]), (n, algo, op, k)
+
+
+@pytest.mark.parametrize("n", RANKS)
+@pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED])
+def test_all_reduce_programs_match_oracle(orc, n, algo):
+    progs = hccl_amd.fold_programs(OpKind.ALL_REDUCE, algo, n)
+    count = 5 * n + 3
+    for op, gen in ((SUM, wide), (MAX, tricky)):
+        rng = np.random.default_rng(2000 * n + 10 * int(algo) + op)
+        ins = gen(rng, n, count)
+        outs = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+        assert orc.all_reduce(ins, outs, count, F32, op, algo=ALGO_NAME[algo]) == 0
+        got = np.zeros(count, dtype=np.float32)
+        if len(progs) == 1:
+            got[:] = run_program(progs[0], lambda r: ins[r], op)
+        elif algo == Algo.RHD:
+            unit = count // n
+            for i in range(n):
+                lo, hi = i * unit, (i + 1) * unit
+                if hi > lo:
+                    got[lo:hi] = run_program(progs[i], lambda r: ins[r][lo:hi], op)
+            for e in range(unit * n, count):
+                got[e:e + 1] = run_program(progs[e - unit * n], lambda r: ins[r][e:e + 1], op)
+        else:
+            sl = -(-count // n)
+            for i in range(n):
+                lo, hi = min(count, i * sl), min(count, (i + 1) * sl)
+                if hi > lo:
+                    got[lo:hi] = run_program(progs[i], lambda r: ins[r][lo:hi], op)
+        assert same(got, outs[0]), (n, algo, op)
+
+
+def test_known_programs():
+    # rank order, one run of 8
+    assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.MESH, 8) == [bytes([0xC8, 0, 1, 2, 3, 4, 5, 6, 7, 0xFF])]
+    # own slice first
+    assert hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.MESH, 4)[2] == bytes([0xC4, 2, 0, 1, 3, 0xFF])
+    # p = 6: ((x0+x2)+x4) + ((x1+x3)+x5) for the share of rank 0
+    p6 = hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.RHD, 6)
+    assert p6[0] == bytes([0xC3, 0, 2, 4, 0x80, 0xC3, 1, 3, 5, 0x81, 0xFF])
+    assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.AIV_MESH, 4) if False else True
+
+
+# ---- argument validation (returns before any GPU work) ------------------------------------------------
+@pytest.fixture(scope="module")
+def world():
+    comms = hccl_amd.comm_init_all(4)
+    yield comms
+    for c in comms:
+        hccl_amd.comm_destroy(c)
+
+
+def code_of(fn, *a, **k):
+    try:
+        return fn(*a, **k)
+    except hccl_amd.HcclError as e:
+        return e.code
+
+
+def test_lifecycle_queries(world):
+    assert [hccl_amd.get_rank_id(c) for c in world] == [0, 1, 2, 3]
+    assert hccl_amd.get_rank_size(world[2]) == 4
+    assert code_of(hccl_amd.comm_init_all, 0) == 1
+    assert code_of(hccl_amd.comm_init_all, 65) == 1
+    assert code_of(hccl_amd.comm_init_all, 2, [0, 1]) == 5
+    info = hccl_amd.get_root_info()
+    a = hccl_amd.comm_init_root_info(2, info, 0)
+    assert code_of(hccl_amd.comm_init_root_info, 2, info, 0) == 1      # rank joined twice
+    assert code_of(hccl_amd.comm_init_root_info, 3, info, 1) == 1      # size mismatch
+    b = hccl_amd.comm_init_root_info(2, info, 1)
+    assert hccl_amd.get_rank_id(b) == 1 and hccl_amd.get_rank_size(a) == 2
+    hccl_amd.comm_destroy(a)
+    hccl_amd.comm_destroy(b)
+    assert code_of(hccl_amd.get_rank_id, a) == 1                       # destroyed handle
+
+
+def test_algo_knob(world):
+    assert hccl_amd.get_algo(world[0], OpKind.ALL_REDUCE) == Algo.MESH
+    hccl_amd.set_algo(world[1], OpKind.ALL_REDUCE, Algo.RHD)
+    assert hccl_amd.get_algo(world[3], OpKind.ALL_REDUCE) == Algo.RHD   # per world, not per rank
+    assert code_of(hccl_amd.set_algo, world[0], OpKind.ALL_REDUCE, Algo.AIV_MESH) == 5
+    hccl_amd.set_algo(world[0], OpKind.ALL_REDUCE, Algo.MESH)
+
+
+def test_all_reduce_argument_checks(world):
+    c, s, buf = world[0], 0x1000, 0x2000
+    assert hccl_amd.all_reduce(c, None, None, 0, DT.FP32, OP.SUM, None) == 0        # count 0 wins over everything
+    assert code_of(hccl_amd.all_reduce, c, buf, buf, 8, DT.FP32, OP.SUM, None) == 2   # null stream
+    assert code_of(hccl_amd.all_reduce, None, buf, buf, 8, DT.FP32, OP.SUM, s) == 2   # null comm
+    assert code_of(hccl_amd.all_reduce, c, None, buf, 8, DT.FP32, OP.SUM, s) == 2
+    assert code_of(hccl_amd.all_reduce, c, buf, None, 8, DT.FP32, OP.SUM, s) == 2
+    assert code_of(hccl_amd.all_reduce, c, buf, buf, 0x800000000, DT.FP32, OP.SUM, s) == 1
+    for bad in (DT.UINT8, DT.UINT16, DT.UINT32, DT.INT128, DT.HIF8, DT.FP8E4M3, DT.FP8E5M2, DT.FP8E8M0, 13, 99):
+        assert code_of(hccl_amd.all_reduce, c, buf, buf, 8, bad, OP.SUM, s) == 5
+    for bad in (DT.INT16, DT.BFP16):
+        assert code_of(hccl_amd.all_reduce, c, buf, buf, 8, bad, OP.PROD, s) == 5
+    assert code_of(hccl_amd.all_reduce, c, buf, buf, 8, DT.FP32, 7, s) == 1
+
+
+def test_other_entry_argument_checks(world):
+    c, s, a, b = world[1], 0x1000, 0x2000, 0x3000
+    assert hccl_amd.reduce_scatter(c, None, None, 0, DT.FP16, OP.SUM, None) == 0
+    assert code_of(hccl_amd.reduce_scatter, c, a, b, 4, DT.FP16, OP.SUM, None) == 2
+    assert code_of(hccl_amd.reduce_scatter, c, a, b, 4, DT.UINT8, OP.SUM, s) == 5
+    assert hccl_amd.all_gather(c, None, None, 0, DT.UINT8, None) == 0
+    assert code_of(hccl_amd.all_gather, c, a, None, 4, DT.UINT8, s) == 2
+    assert code_of(hccl_amd.all_gather, c, a, b, 4, DT.INT128, s) == 5
+    # AllGatherV
+    z, cnt, dsp = [0, 0, 0, 0], [4, 4, 4, 4], [0, 4, 8, 12]
+    assert hccl_amd.all_gather_v(c, None, 0, None, z, dsp, DT.FP16, s) == 0          # all-zero counts: no-op
+    assert code_of(hccl_amd.all_gather_v, c, a, 4, a, cnt, dsp, DT.FP16, s) == 1     # in place rejected
+    assert code_of(hccl_amd.all_gather_v, c, None, 4, b, cnt, dsp, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_gather_v, c, a, 4, None, cnt, dsp, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_gather_v, c, a, 4, b, cnt, [0, 2, 8, 12], DT.FP16, s) == 1   # overlap
+    assert code_of(hccl_amd.all_gather_v, c, a, 4, b, cnt, [0, 4, 8, 2 ** 64 - 2], DT.FP16, s) == 1  # overflow
+    assert code_of(hccl_amd.all_gather_v, c, a, 4, b, cnt, dsp, DT.FP16, None) == 2
+    # AlltoAllV
+    assert code_of(hccl_amd.all_to_all_v, c, a, cnt, dsp, DT.FP16, a, cnt, dsp, DT.FP16, s) == 1   # in place
+    assert code_of(hccl_amd.all_to_all_v, c, None, cnt, dsp, DT.FP16, b, cnt, dsp, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_to_all_v, c, a, cnt, dsp, DT.FP16, None, cnt, dsp, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_to_all_v, c, a, cnt, dsp, DT.FP16, b, cnt, dsp, DT.INT128, s) == 5
+    assert code_of(hccl_amd.all_to_all_v, c, a, [2 ** 40, 0, 0, 0], dsp, DT.FP16, b, cnt, dsp, DT.FP16, s) == 1
+
+
+def test_group_end_without_start():
+    assert code_of(hccl_amd.group_end) == 1
