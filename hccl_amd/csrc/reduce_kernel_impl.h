@@ -77,7 +77,8 @@ __device__ __forceinline__ uint16_t FloatToBf16Bits(float f)
 {
     uint32_t u = __builtin_bit_cast(uint32_t, f);
     uint32_t rounded = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-    uint32_t quiet = (u >> 16) | 0x40u;
+    uint32_t hi = u >> 16;
+    uint32_t quiet = (hi & 0x7Fu) ? hi : (hi | 1u);   // NaN stays NaN, payload bits kept
     bool isNan = (u & 0x7FFFFFFFu) > 0x7F800000u;
     return static_cast<uint16_t>(isNan ? quiet : rounded);
 }

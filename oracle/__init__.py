@@ -124,7 +124,8 @@ def np_fp32_to_bf16_bits(f32):
     u = np.ascontiguousarray(f32, dtype=np.float32).view(np.uint32)
     nan = ((u & 0x7F800000) == 0x7F800000) & ((u & 0x007FFFFF) != 0)
     rounded = ((u.astype(np.uint64) + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
-    return np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), rounded)
+    hi = (u >> 16).astype(np.uint16)
+    return np.where(nan, np.where((hi & 0x7F) != 0, hi, hi | 1), rounded)
 
 
 def bf16_bits_to_fp32(h_bits):

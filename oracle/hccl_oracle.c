@@ -156,7 +156,8 @@ uint16_t orc_fp32_to_bf16(float f)
 {
     uint32_t u = f2u(f);
     if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu) != 0) {
-        return (uint16_t)((u >> 16) | 0x0040u);
+        uint16_t hi = (uint16_t)(u >> 16);
+        return (hi & 0x7Fu) ? hi : (uint16_t)(hi | 1u);
     }
     return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
 }

@@ -53,8 +53,9 @@ size_t orc_dtype_size(int dtype);
 float orc_fp16_to_fp32(uint16_t h);
 uint16_t orc_fp32_to_fp16(float f);
 /* bf16 has no host path in the reference (parity unpinned): widen = bits << 16; narrow =
- * round-to-nearest-even on the upper 16 bits, NaN keeps sign and payload top bits with the
- * quiet bit forced. */
+ * round-to-nearest-even on the upper 16 bits; NaN keeps its upper 16 bits, the mantissa forced
+ * to 1 if they hold none of it (the rule the reference applies to fp16, wrapper.cc:1201-1206), so
+ * that widen followed by narrow is the identity on every bf16 pattern. */
 float orc_bf16_to_fp32(uint16_t h);
 uint16_t orc_fp32_to_bf16(float f);
 /* Array forms of the four conversions (same functions applied element by element). */
