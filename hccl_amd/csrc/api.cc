@@ -177,6 +177,7 @@ struct PendingOp {
 struct DevicePlan {
     uint8_t* dev = nullptr;
     uint32_t nProg = 0;
+    uint32_t maxDepth = 1;
     bool segmentsAreSubs = false;
 };
 
@@ -345,6 +346,7 @@ HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DeviceP
     DevicePlan dp;
     dp.nProg = static_cast<uint32_t>(plan.programs.size());
     dp.segmentsAreSubs = plan.segmentsAreSubs;
+    dp.maxDepth = plan.maxDepth;
     HIP_OK(hipMalloc(reinterpret_cast<void**>(&dp.dev), image.size()));
     HIP_OK(hipMemcpy(dp.dev, image.data(), image.size(), hipMemcpyHostToDevice));
     w->plans[key] = dp;
@@ -407,7 +409,8 @@ uint32_t BlocksPerSub(const World* w, uint64_t subLen, uint32_t esz, uint64_t nS
     return static_cast<uint32_t>(want < maxUseful ? want : maxUseful);
 }
 
-HcclResult LaunchOneReduce(World* w, ReduceArgs& a, HcclDataType dtype, HcclReduceOp op, hipStream_t s)
+HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, HcclDataType dtype, HcclReduceOp op,
+                           hipStream_t s)
 {
     uint32_t esz = DataTypeSize(dtype);
     uint64_t bits = 0;
@@ -419,7 +422,7 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, HcclDataType dtype, HcclRedu
         for (uint32_t d = 0; d < a.nDst; ++d) bits |= reinterpret_cast<uint64_t>(a.dst[d]);
     }
     if (a.nGroup > 1) bits |= a.srcGroupStride * esz | a.dstGroupStride * esz;
-    if (a.nSub > 1) bits |= a.subLen * esz;
+    // Sub-segment starts need no alignment: sources and destinations share them, the kernel peels.
     a.vecOk = (bits & 15u) == 0 ? 1u : 0u;
     uint64_t subs = static_cast<uint64_t>(a.nGroup) * a.nSub;
     uint64_t longest = a.groupLen;   // the last sub-segment takes what the others leave
@@ -433,7 +436,8 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, HcclDataType dtype, HcclRedu
     if (blocks == 0 || blocks > 0x7FFFFFFFull) {
         return HCCL_E_INTERNAL;
     }
-    HIP_OK(LaunchReduce(a, dtype, op, static_cast<uint32_t>(blocks), s));
+    const uint32_t lds = (plan.maxDepth - 1) * ReduceAccBytes(dtype, op) * 256u;
+    HIP_OK(LaunchReduce(a, dtype, op, static_cast<uint32_t>(blocks), lds, s));
     return HCCL_SUCCESS;
 }
 
@@ -459,7 +463,7 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
     if (plan.nProg == 1) {
         a.total = a.groupLen = a.subLen = p.count;
         a.nSub = 1;
-        return LaunchOneReduce(w, a, p.dtype, p.op, s);
+        return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
     }
     a.nSub = n;
     a.progSubStride = 1;
@@ -471,7 +475,7 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
         if (unit > 0) {
             a.total = a.groupLen = prefix;
             a.subLen = unit;
-            rc = LaunchOneReduce(w, a, p.dtype, p.op, s);
+            rc = LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
             if (rc != HCCL_SUCCESS) {
                 return rc;
             }
@@ -483,14 +487,14 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
             }
             a.total = a.groupLen = p.count - prefix;
             a.subLen = 1;
-            return LaunchOneReduce(w, a, p.dtype, p.op, s);
+            return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
         }
         return HCCL_SUCCESS;
     }
     // NHR: slices of ceil(count / n) elements (reference two_shot.cc:184 slicing rule).
     a.total = a.groupLen = p.count;
     a.subLen = (p.count + n - 1) / n;
-    return LaunchOneReduce(w, a, p.dtype, p.op, s);
+    return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
 }
 
 HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
@@ -523,7 +527,7 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
         a.subLen = p.count;
         a.progGroupStride = plan.nProg > 1 ? 1 : 0;
     }
-    return LaunchOneReduce(w, a, p.dtype, p.op, s);
+    return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
 }
 
 HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)

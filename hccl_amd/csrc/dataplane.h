@@ -95,8 +95,14 @@ struct A2aArgs {
 constexpr uint32_t kCopyTileBytes = 16384;
 
 // Launchers (defined in the .hip files).  All are asynchronous on `stream`.
+// ldsBytes = (plan depth - 1) * ReduceAccBytes(dtype, op) * 256: the accumulator stack of nested levels.
 hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t nBlocks,
-                        hipStream_t stream);
+                        uint32_t ldsBytes, hipStream_t stream);
+inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
+{
+    bool half = dtype == HCCL_DATA_TYPE_FP16 || dtype == HCCL_DATA_TYPE_BFP16;
+    return (half && op == HCCL_REDUCE_SUM) ? 32u : 16u;   // eight fp32 accumulators vs one 16-byte pack
+}
 hipError_t LaunchBcastCopy(const BcastCopyArgs& args, hipStream_t stream);
 hipError_t LaunchA2aPlan(const A2aArgs& args, hipStream_t stream);
 hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nBlocks, hipStream_t stream);

@@ -4,7 +4,8 @@
 // 16-byte vector position, pulls that position from the N rank buffers with 128-bit loads, combines
 // them in registers in the order a fold program dictates, and writes the result once per
 // destination.  The path is bound by HBM bandwidth (N reads + M writes of the element range, no
-// re-reads, no staging passes), so there is no MFMA and LDS only holds the 320-byte program.
+// re-reads, no staging passes), so there is no MFMA; LDS only holds the 320-byte program and, for
+// tree-shaped orders, the accumulators of enclosing levels.
 //
 // Operand roles follow the reference's pairwise step  dst[i] = src[i] (+) dst[i]
 // (alg_data_trans_wrapper.cc:1319-1358):
@@ -164,7 +165,9 @@ __device__ __forceinline__ uint32_t Uniform(uint32_t v) { return __builtin_amdgc
 
 // ---------------------------------------------------------------------------------------------
 // Program interpreter.  Control flow depends only on the program, so it is uniform across the
-// wavefront; each nesting level has its own accumulator registers through template recursion.
+// wavefront.  One accumulator lives in registers; when a nested level opens, the enclosing level's
+// accumulator waits in an LDS stack laid out word-major ([level][word][thread], so a wavefront's
+// accesses hit 64 consecutive banks) and is popped when the level closes.
 // ---------------------------------------------------------------------------------------------
 template <class E, int W>
 struct AccPack {
@@ -172,7 +175,36 @@ struct AccPack {
 };
 
 template <class E, int W>
-__device__ __forceinline__ void FoldRun(const uint8_t* sprog, uint32_t& pc, uint32_t n, const ReduceArgs& args,
+struct AccWords {
+    static constexpr int kCount = (sizeof(AccPack<E, W>) + 3) / 4;
+    uint32_t w[kCount];
+};
+
+template <class E, int W>
+__device__ __forceinline__ void PushAcc(uint32_t* stack, uint32_t level, const AccPack<E, W>& acc)
+{
+    AccWords<E, W> words = {};
+    __builtin_memcpy(&words, &acc, sizeof(acc));
+#pragma unroll
+    for (int i = 0; i < AccWords<E, W>::kCount; ++i) {
+        stack[(level * AccWords<E, W>::kCount + i) * kThreads + threadIdx.x] = words.w[i];
+    }
+}
+
+template <class E, int W>
+__device__ __forceinline__ void PopAcc(const uint32_t* stack, uint32_t level, AccPack<E, W>& acc)
+{
+    AccWords<E, W> words;
+#pragma unroll
+    for (int i = 0; i < AccWords<E, W>::kCount; ++i) {
+        words.w[i] = stack[(level * AccWords<E, W>::kCount + i) * kThreads + threadIdx.x];
+    }
+    __builtin_memcpy(&acc, &words, sizeof(acc));
+}
+
+// Folds the n (1..8) ranks listed at sprog[pc..] into acc; all loads are issued before the first fold.
+template <class E, int W>
+__device__ __forceinline__ void FoldRun(const uint8_t* sprog, uint32_t pc, uint32_t n, const ReduceArgs& args,
                                         uint64_t off, AccPack<E, W>& acc, bool init)
 {
     using S = typename E::S;
@@ -184,16 +216,20 @@ __device__ __forceinline__ void FoldRun(const uint8_t* sprog, uint32_t& pc, uint
             v[i] = LoadPack<S, W>(args.src[rank], off);
         }
     }
-    pc += n;
     if (init) {
 #pragma unroll
         for (int w = 0; w < W; ++w) {
             acc.a[w] = E::Widen(v[0].e[w]);
         }
+    } else {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            acc.a[w] = E::Fold(E::Widen(v[0].e[w]), acc.a[w]);
+        }
     }
 #pragma unroll
-    for (int i = 0; i < kMaxRun; ++i) {
-        if (static_cast<uint32_t>(i) < n && !(init && i == 0)) {
+    for (int i = 1; i < kMaxRun; ++i) {
+        if (static_cast<uint32_t>(i) < n) {
 #pragma unroll
             for (int w = 0; w < W; ++w) {
                 acc.a[w] = E::Fold(E::Widen(v[i].e[w]), acc.a[w]);
@@ -202,45 +238,40 @@ __device__ __forceinline__ void FoldRun(const uint8_t* sprog, uint32_t& pc, uint
     }
 }
 
-template <class E, int W, int L>
-__device__ __forceinline__ void EvalLevel(const uint8_t* sprog, uint32_t& pc, const ReduceArgs& args, uint64_t off,
-                                          AccPack<E, W>& acc)
-{
-    // The first operand of every level is a rank value (the builder guarantees a run token here).
-    uint32_t tok = Uniform(sprog[pc]);
-    ++pc;
-    FoldRun<E, W>(sprog, pc, tok & 0x3Fu, args, off, acc, true);
-    for (;;) {
-        tok = Uniform(sprog[pc]);
-        ++pc;
-        if (tok == kTokClose || tok == kTokEnd) {
-            return;
-        }
-        if (tok == kTokOpen) {
-            if constexpr (L + 1 < kMaxFoldDepth) {
-                AccPack<E, W> sub;
-                EvalLevel<E, W, L + 1>(sprog, pc, args, off, sub);
-#pragma unroll
-                for (int w = 0; w < W; ++w) {
-                    acc.a[w] = E::Fold(sub.a[w], acc.a[w]);
-                }
-            } else {
-                return;   // deeper than the host ever emits
-            }
-        } else {
-            FoldRun<E, W>(sprog, pc, tok & 0x3Fu, args, off, acc, false);
-        }
-    }
-}
-
 template <class E, int W>
-__device__ __forceinline__ void ReduceOne(const uint8_t* sprog, const ReduceArgs& args, uint64_t srcOff,
-                                          uint64_t dstOff, uint32_t group)
+__device__ __forceinline__ void ReduceOne(const uint8_t* sprog, uint32_t* stack, const ReduceArgs& args,
+                                          uint64_t srcOff, uint64_t dstOff, uint32_t group)
 {
     using S = typename E::S;
     AccPack<E, W> acc;
     uint32_t pc = 0;
-    EvalLevel<E, W, 0>(sprog, pc, args, srcOff, acc);
+    uint32_t level = 0;
+    bool init = true;   // the next rank value starts a level instead of being folded into it
+    for (;;) {
+        const uint32_t tok = Uniform(sprog[pc]);
+        ++pc;
+        if (tok == kTokEnd) {
+            break;
+        }
+        if (tok == kTokOpen) {
+            PushAcc<E, W>(stack, level, acc);
+            ++level;
+            init = true;
+        } else if (tok == kTokClose) {
+            AccPack<E, W> outer;
+            --level;
+            PopAcc<E, W>(stack, level, outer);
+#pragma unroll
+            for (int w = 0; w < W; ++w) {
+                acc.a[w] = E::Fold(acc.a[w], outer.a[w]);   // nested value is src, enclosing level is dst
+            }
+        } else {
+            const uint32_t n = tok & 0x3Fu;
+            FoldRun<E, W>(sprog, pc, n, args, srcOff, acc, init);
+            pc += n;
+            init = false;
+        }
+    }
     Pack<S, W> out;
 #pragma unroll
     for (int w = 0; w < W; ++w) {
@@ -255,12 +286,14 @@ __device__ __forceinline__ void ReduceOne(const uint8_t* sprog, const ReduceArgs
     }
 }
 
+// Dynamic LDS: the accumulator stack, (maxDepth - 1) * accumulator bytes * kThreads.
 template <class E>
 __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
 {
     using S = typename E::S;
     constexpr int W = 16 / sizeof(S);
     __shared__ __attribute__((aligned(16))) uint8_t sprog[kProgStride];
+    extern __shared__ uint32_t accStack[];
 
     const uint32_t sub = blockIdx.x / args.blocksPerSub;
     const uint32_t blk = blockIdx.x - sub * args.blocksPerSub;
@@ -291,18 +324,25 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     const uint64_t stride = static_cast<uint64_t>(args.blocksPerSub) * kThreads;
     const uint64_t first = static_cast<uint64_t>(blk) * kThreads + threadIdx.x;
 
-    // 128-bit body when every address is 16-byte aligned, then element by element for what is left
-    // (fewer than W elements) or for the whole range when it is not.
-    uint64_t done = 0;
+    // When vecOk, every source and destination address of this sub-segment has the same offset from a
+    // 16-byte boundary: `head` elements bring them all onto it, a 128-bit body follows, and fewer than
+    // W elements remain.  Otherwise everything goes element by element.
+    uint64_t head = len;
+    uint64_t nVec = 0;
     if (args.vecOk) {
-        const uint64_t nVec = len / W;
-        for (uint64_t v = first; v < nVec; v += stride) {
-            ReduceOne<E, W>(sprog, args, srcOff + v * W, dstOff + v * W, g);
-        }
-        done = nVec * W;
+        const uint32_t mis = static_cast<uint32_t>((reinterpret_cast<uint64_t>(args.src[0]) + srcOff * sizeof(S)) & 15u);
+        head = mis ? (16u - mis) / sizeof(S) : 0;
+        head = head < len ? head : len;
+        nVec = (len - head) / W;
     }
-    for (uint64_t e = done + first; e < len; e += stride) {
-        ReduceOne<E, 1>(sprog, args, srcOff + e, dstOff + e, g);
+    for (uint64_t v = first; v < nVec; v += stride) {
+        ReduceOne<E, W>(sprog, accStack, args, srcOff + head + v * W, dstOff + head + v * W, g);
+    }
+    const uint64_t bodyEnd = head + nVec * W;
+    const uint64_t nScalar = head + (len - bodyEnd);
+    for (uint64_t i = first; i < nScalar; i += stride) {
+        const uint64_t e = i < head ? i : i - head + bodyEnd;
+        ReduceOne<E, 1>(sprog, accStack, args, srcOff + e, dstOff + e, g);
     }
 }
 

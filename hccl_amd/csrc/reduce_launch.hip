@@ -4,7 +4,7 @@
 namespace hccl_amd {
 
 hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t nBlocks,
-                        hipStream_t stream)
+                        uint32_t ldsBytes, hipStream_t stream)
 {
     detail::ReduceKernelFn fn = nullptr;
     const int o = static_cast<int>(op);
@@ -23,7 +23,7 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
     if (fn == nullptr || nBlocks == 0) {
         return hipErrorInvalidValue;
     }
-    hipLaunchKernelGGL(fn, dim3(nBlocks), dim3(detail::kThreads), 0, stream, args);
+    hipLaunchKernelGGL(fn, dim3(nBlocks), dim3(detail::kThreads), ldsBytes, stream, args);
     return hipGetLastError();
 }
 
