@@ -214,7 +214,7 @@ struct World {
     hipEvent_t a2aSlotFree[kStagingSlots] = {};
     bool a2aSlotUsed[kStagingSlots] = {};
     uint32_t a2aNext = 0;
-    uint32_t reduceBlocks = 2048;
+    uint32_t reduceBlocks = 32768;
     uint32_t copyBlocks = 2048;
 
     ~World()
@@ -298,7 +298,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (hipGetDevice(&w->device) != hipSuccess) {
         w->device = 0;
     }
-    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 2048);
+    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 32768);
     w->copyBlocks = EnvU32("HCCL_AMD_COPY_BLOCKS", 2048);
     ApplyAlgoEnv(w.get());
     return w;
@@ -339,9 +339,34 @@ HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DeviceP
     if (rc != HCCL_SUCCESS) {
         return rc;
     }
-    std::vector<uint8_t> image(plan.programs.size() * kProgStride, kTokEnd);
+    // Flatten every token program to the kernel's leaf table.
+    std::vector<uint8_t> image(plan.programs.size() * kDevProgBytes, 0);
     for (size_t s = 0; s < plan.programs.size(); ++s) {
-        memcpy(image.data() + s * kProgStride, plan.programs[s].data(), plan.programs[s].size());
+        uint8_t* img = image.data() + s * kDevProgBytes;
+        uint32_t leaves = 0;
+        bool open = false;
+        const std::vector<uint8_t>& prog = plan.programs[s];
+        for (size_t i = 0; i < prog.size() && prog[i] != kTokEnd; ++i) {
+            uint8_t tok = prog[i];
+            if (tok == kTokOpen) {
+                open = true;
+            } else if (tok == kTokClose) {
+                img[kDevProgCtlOff + leaves - 1]++;
+            } else {
+                uint32_t n = tok >= kTokRun ? (tok & 0x3Fu) : 1u;
+                for (uint32_t k = 0; k < n; ++k) {
+                    uint8_t rank = tok >= kTokRun ? prog[++i] : tok;
+                    if (leaves >= static_cast<uint32_t>(kMaxRanks)) {
+                        return HCCL_E_INTERNAL;
+                    }
+                    img[kDevProgRankOff + leaves] = rank;
+                    img[kDevProgCtlOff + leaves] = open ? kCtlOpen : 0;
+                    open = false;
+                    ++leaves;
+                }
+            }
+        }
+        img[0] = static_cast<uint8_t>(leaves);
     }
     DevicePlan dp;
     dp.nProg = static_cast<uint32_t>(plan.programs.size());

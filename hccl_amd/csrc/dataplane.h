@@ -32,9 +32,17 @@ constexpr uint8_t kTokOpen = 0x80;
 constexpr uint8_t kTokClose = 0x81;
 constexpr uint8_t kTokRun = 0xC0;
 constexpr uint8_t kTokEnd = 0xFF;
-constexpr int kProgStride = 320;   // bytes reserved per program in device memory
-constexpr int kMaxFoldDepth = 8;   // nesting levels the kernel instantiates
+constexpr int kProgStride = 320;   // upper bound on the byte length of one program
+constexpr int kMaxFoldDepth = 8;   // deepest nesting a plan may have
 constexpr int kMaxRun = 8;
+
+// Device image of one program (what the kernel reads): the same tree flattened to its leaves in
+// evaluation order.  Leaf i folds rank[i]; ctl[i] bit 7 says a nested level opens right before it
+// (the enclosing accumulator is parked), ctl[i] bits 0..6 count the levels that close right after it.
+constexpr int kDevProgBytes = 160;
+constexpr int kDevProgRankOff = 16;   // byte 0 holds the leaf count
+constexpr int kDevProgCtlOff = 80;
+constexpr uint8_t kCtlOpen = 0x80;
 
 // Geometry of one fused reduce launch.
 //

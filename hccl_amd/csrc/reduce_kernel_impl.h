@@ -202,74 +202,72 @@ __device__ __forceinline__ void PopAcc(const uint32_t* stack, uint32_t level, Ac
     __builtin_memcpy(&acc, &words, sizeof(acc));
 }
 
-// Folds the n (1..8) ranks listed at sprog[pc..] into acc; all loads are issued before the first fold.
-template <class E, int W>
-__device__ __forceinline__ void FoldRun(const uint8_t* sprog, uint32_t pc, uint32_t n, const ReduceArgs& args,
-                                        uint64_t off, AccPack<E, W>& acc, bool init)
+__device__ __forceinline__ uint64_t Uniform64(uint64_t v)
 {
-    using S = typename E::S;
-    Pack<S, W> v[kMaxRun];
-#pragma unroll
-    for (int i = 0; i < kMaxRun; ++i) {
-        if (static_cast<uint32_t>(i) < n) {
-            uint32_t rank = Uniform(sprog[pc + i]);
-            v[i] = LoadPack<S, W>(args.src[rank], off);
-        }
-    }
-    if (init) {
-#pragma unroll
-        for (int w = 0; w < W; ++w) {
-            acc.a[w] = E::Widen(v[0].e[w]);
-        }
-    } else {
-#pragma unroll
-        for (int w = 0; w < W; ++w) {
-            acc.a[w] = E::Fold(E::Widen(v[0].e[w]), acc.a[w]);
-        }
-    }
-#pragma unroll
-    for (int i = 1; i < kMaxRun; ++i) {
-        if (static_cast<uint32_t>(i) < n) {
-#pragma unroll
-            for (int w = 0; w < W; ++w) {
-                acc.a[w] = E::Fold(E::Widen(v[i].e[w]), acc.a[w]);
-            }
-        }
-    }
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
+// Per-block view of the program: leaf i is read at leafPtr[i] (the rank's buffer already advanced to
+// this sub-segment) and carries ctl[i] (see kCtlOpen).
+struct BlockProgram {
+    uint64_t leafPtr[kMaxRanks];
+    uint8_t ctl[kMaxRanks];
+    uint32_t nLeaves;
+};
+
+// Evaluates the whole tree for the W elements at element offset `e` of the sub-segment.  Leaves are
+// taken eight at a time: their loads are all issued before the first fold, whatever the tree shape.
 template <class E, int W>
-__device__ __forceinline__ void ReduceOne(const uint8_t* sprog, uint32_t* stack, const ReduceArgs& args,
-                                          uint64_t srcOff, uint64_t dstOff, uint32_t group)
+__device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stack, const ReduceArgs& args,
+                                          uint64_t e, uint64_t dstOff, uint32_t group)
 {
     using S = typename E::S;
     AccPack<E, W> acc;
-    uint32_t pc = 0;
     uint32_t level = 0;
-    bool init = true;   // the next rank value starts a level instead of being folded into it
-    for (;;) {
-        const uint32_t tok = Uniform(sprog[pc]);
-        ++pc;
-        if (tok == kTokEnd) {
-            break;
-        }
-        if (tok == kTokOpen) {
-            PushAcc<E, W>(stack, level, acc);
-            ++level;
-            init = true;
-        } else if (tok == kTokClose) {
-            AccPack<E, W> outer;
-            --level;
-            PopAcc<E, W>(stack, level, outer);
+    bool init = true;   // the next leaf starts a level instead of being folded into it
+    const uint32_t nLeaves = bp.nLeaves;
+    for (uint32_t b = 0; b < nLeaves; b += kMaxRun) {
+        Pack<S, W> v[kMaxRun];
 #pragma unroll
-            for (int w = 0; w < W; ++w) {
-                acc.a[w] = E::Fold(acc.a[w], outer.a[w]);   // nested value is src, enclosing level is dst
+        for (int i = 0; i < kMaxRun; ++i) {
+            if (b + i < nLeaves) {
+                const void* base = reinterpret_cast<const void*>(Uniform64(bp.leafPtr[b + i]));
+                v[i] = LoadPack<S, W>(base, e);
             }
-        } else {
-            const uint32_t n = tok & 0x3Fu;
-            FoldRun<E, W>(sprog, pc, n, args, srcOff, acc, init);
-            pc += n;
-            init = false;
+        }
+#pragma unroll
+        for (int i = 0; i < kMaxRun; ++i) {
+            if (b + i < nLeaves) {
+                const uint32_t ctl = Uniform(bp.ctl[b + i]);
+                if (ctl & kCtlOpen) {
+                    PushAcc<E, W>(stack, level, acc);
+                    ++level;
+                    init = true;
+                }
+                if (init) {
+#pragma unroll
+                    for (int w = 0; w < W; ++w) {
+                        acc.a[w] = E::Widen(v[i].e[w]);
+                    }
+                    init = false;
+                } else {
+#pragma unroll
+                    for (int w = 0; w < W; ++w) {
+                        acc.a[w] = E::Fold(E::Widen(v[i].e[w]), acc.a[w]);
+                    }
+                }
+                for (uint32_t closes = ctl & 0x7Fu; closes != 0; --closes) {
+                    AccPack<E, W> outer;
+                    --level;
+                    PopAcc<E, W>(stack, level, outer);
+#pragma unroll
+                    for (int w = 0; w < W; ++w) {
+                        acc.a[w] = E::Fold(acc.a[w], outer.a[w]);   // nested value is src, enclosing level is dst
+                    }
+                }
+            }
         }
     }
     Pack<S, W> out;
@@ -278,21 +276,21 @@ __device__ __forceinline__ void ReduceOne(const uint8_t* sprog, uint32_t* stack,
         out.e[w] = E::Narrow(acc.a[w]);
     }
     if (args.dstOwn) {
-        StorePack<S, W>(args.dst[group], dstOff, out);
+        StorePack<S, W>(args.dst[group], dstOff + e, out);
     } else {
         for (uint32_t d = 0; d < args.nDst; ++d) {
-            StorePack<S, W>(args.dst[d], dstOff, out);
+            StorePack<S, W>(args.dst[d], dstOff + e, out);
         }
     }
 }
 
-// Dynamic LDS: the accumulator stack, (maxDepth - 1) * accumulator bytes * kThreads.
+// Dynamic LDS: the accumulator stack, (plan depth - 1) * accumulator bytes * kThreads.
 template <class E>
 __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
 {
     using S = typename E::S;
     constexpr int W = 16 / sizeof(S);
-    __shared__ __attribute__((aligned(16))) uint8_t sprog[kProgStride];
+    __shared__ BlockProgram bp;
     extern __shared__ uint32_t accStack[];
 
     const uint32_t sub = blockIdx.x / args.blocksPerSub;
@@ -312,15 +310,22 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
         return;
     }
     const uint64_t len = sEnd - sBeg;
+    const uint64_t srcOff = static_cast<uint64_t>(g) * args.srcGroupStride + sBeg;
+    const uint64_t dstOff = args.dstOwn ? sBeg : static_cast<uint64_t>(g) * args.dstGroupStride + sBeg;
 
-    const uint8_t* prog = args.prog + static_cast<uint64_t>(g * args.progGroupStride + c * args.progSubStride) * kProgStride;
-    for (uint32_t i = threadIdx.x; i < kProgStride / 4; i += kThreads) {
-        reinterpret_cast<uint32_t*>(sprog)[i] = reinterpret_cast<const uint32_t*>(prog)[i];
+    // Resolve the program once per block: leaf -> address of this sub-segment in that rank's buffer.
+    const uint8_t* prog = args.prog + static_cast<uint64_t>(g * args.progGroupStride + c * args.progSubStride) * kDevProgBytes;
+    const uint32_t nLeaves = prog[0];
+    if (threadIdx.x < nLeaves) {
+        const uint32_t rank = prog[kDevProgRankOff + threadIdx.x];
+        bp.leafPtr[threadIdx.x] = reinterpret_cast<uint64_t>(args.src[rank]) + srcOff * sizeof(S);
+        bp.ctl[threadIdx.x] = prog[kDevProgCtlOff + threadIdx.x];
+    }
+    if (threadIdx.x == 0) {
+        bp.nLeaves = nLeaves;
     }
     __syncthreads();
 
-    const uint64_t srcOff = static_cast<uint64_t>(g) * args.srcGroupStride + sBeg;
-    const uint64_t dstOff = args.dstOwn ? sBeg : static_cast<uint64_t>(g) * args.dstGroupStride + sBeg;
     const uint64_t stride = static_cast<uint64_t>(args.blocksPerSub) * kThreads;
     const uint64_t first = static_cast<uint64_t>(blk) * kThreads + threadIdx.x;
 
@@ -336,13 +341,13 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
         nVec = (len - head) / W;
     }
     for (uint64_t v = first; v < nVec; v += stride) {
-        ReduceOne<E, W>(sprog, accStack, args, srcOff + head + v * W, dstOff + head + v * W, g);
+        ReduceOne<E, W>(bp, accStack, args, head + v * W, dstOff, g);
     }
     const uint64_t bodyEnd = head + nVec * W;
     const uint64_t nScalar = head + (len - bodyEnd);
     for (uint64_t i = first; i < nScalar; i += stride) {
         const uint64_t e = i < head ? i : i - head + bodyEnd;
-        ReduceOne<E, 1>(sprog, accStack, args, srcOff + e, dstOff + e, g);
+        ReduceOne<E, 1>(bp, accStack, args, e, dstOff, g);
     }
 }
 
