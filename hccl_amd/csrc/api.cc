@@ -214,7 +214,7 @@ struct World {
     hipEvent_t a2aSlotFree[kStagingSlots] = {};
     bool a2aSlotUsed[kStagingSlots] = {};
     uint32_t a2aNext = 0;
-    uint32_t reduceBlocks = 32768;
+    uint32_t reduceBlocks = 1u << 20;
     uint32_t copyBlocks = 2048;
 
     ~World()
@@ -298,7 +298,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (hipGetDevice(&w->device) != hipSuccess) {
         w->device = 0;
     }
-    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 32768);
+    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 1u << 20);
     w->copyBlocks = EnvU32("HCCL_AMD_COPY_BLOCKS", 2048);
     ApplyAlgoEnv(w.get());
     return w;
@@ -557,11 +557,10 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
 
 HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
 {
-    (void)w;
     uint64_t bits = 0;
     for (uint32_t d = 0; d < b.nDst; ++d) bits |= reinterpret_cast<uint64_t>(b.dst[d]);
     b.unit = AlignUnitOf(bits);
-    HIP_OK(LaunchBcastCopy(b, s));
+    HIP_OK(LaunchBcastCopy(b, w->copyBlocks, s));
     return HCCL_SUCCESS;
 }
 

@@ -1,9 +1,16 @@
 // Slice-copy (AllGather / AllGatherV) and displacement-driven pack/unpack (AlltoAllV) for gfx950.
 //
 // Both are pure HBM streaming: every payload byte is read once with 128-bit loads and written once
-// per destination.  Work is cut into 16 KiB tiles so that segments of wildly different length (a
-// Zipf-distributed token routing table) load-balance over the whole chip; the tile -> segment map is
-// found with wavefront-level prefix sums (one lane per rank) and ballots, never a per-segment launch.
+// per destination with 128-bit stores.  Work is cut into 16 KiB tiles so that segments of wildly
+// different length (a Zipf-distributed token routing table) load-balance over the whole chip; the
+// tile -> segment map is found with wavefront-level prefix sums (one lane per rank) and ballots, never
+// a per-segment launch.
+//
+// Displacements are in elements, so a segment's source and destination generally sit at different
+// offsets from a 16-byte boundary.  Such irregular segments are staged through LDS: the block loads
+// the aligned 16-byte vectors that cover the tile's source bytes, and every lane rebuilds the vector it
+// has to store from two neighbouring LDS vectors with a byte funnel shift.  Segments whose two sides
+// are congruent modulo 16 skip LDS.  At most 15 bytes at either end of a tile move byte by byte.
 //
 // Data movement follows the reference's templates:
 //   AllGather(V): out_d[displs[r] ...] = in_r   (ins_temp_all_gather_mesh_1D.cc:249-423,
@@ -18,13 +25,18 @@ namespace hccl_amd {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kVecPerThread = kCopyTileBytes / 16 / kThreads;   // 4
-static_assert(kVecPerThread * 16 * kThreads == kCopyTileBytes, "tile must be a whole number of vector rounds");
+constexpr int kVecPerTile = kCopyTileBytes / 16;                // 1024
+constexpr int kVecPerThread = kVecPerTile / kThreads;           // 4
+static_assert(kVecPerThread * kThreads == kVecPerTile, "tile must be a whole number of vector rounds");
 
 typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ uint32_t Uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+// One staging buffer: the tile's vectors plus the one that completes the last shifted vector.
+struct Stage {
+    U32x4 v[kVecPerTile + 1];
+};
 
+__device__ __forceinline__ uint32_t Uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // Inclusive prefix sum over the 64 lanes of a wavefront.
 __device__ __forceinline__ uint32_t WaveInclusiveScan(uint32_t x)
@@ -54,13 +66,100 @@ __device__ __forceinline__ uint32_t AlignUnit(uint64_t bits)
     return low & (0u - low);
 }
 
-// ---- one tile, one source, nDst destinations ---------------------------------------------------
-template <typename U, class DstFn>
-__device__ __forceinline__ void CopyUnits(const uint8_t* src, uint64_t bytes, uint32_t nDst, DstFn dstOf)
+// Copies one tile (bytes <= 16 KiB) from src to dstOf(d), d < nDst.  Every dstOf(d) has the same offset
+// from a 16-byte boundary.  Must be called by all threads of the block (it may synchronise).
+// Four output dwords from five input dwords, dropping `shift` (0..3) leading bytes.
+__device__ __forceinline__ U32x4 Funnel(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3, uint32_t w4, uint32_t shift)
 {
-    const uint64_t n = bytes / sizeof(U);
+    if (shift == 0) {
+        return U32x4{w0, w1, w2, w3};
+    }
+    return U32x4{__builtin_amdgcn_alignbyte(w1, w0, shift), __builtin_amdgcn_alignbyte(w2, w1, shift),
+                 __builtin_amdgcn_alignbyte(w3, w2, shift), __builtin_amdgcn_alignbyte(w4, w3, shift)};
+}
+
+// The two staging buffers alternate between the tiles that use them, so one barrier per tile is enough:
+// a buffer is rewritten only after the barrier of the tile that used the other one.
+template <class DstFn>
+__device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uint32_t nDst, DstFn dstOf, Stage* stages,
+                                         uint32_t& parity)
+{
+    const uint32_t dMis = static_cast<uint32_t>(reinterpret_cast<uint64_t>(dstOf(0)) & 15u);
+    uint32_t head = (16u - dMis) & 15u;     // bytes before the first aligned destination vector
+    head = head < bytes ? head : bytes;
+    const uint32_t nVec = (bytes - head) / 16u;
+    const uint32_t bodyEnd = head + nVec * 16u;
+    const uint8_t* sBody = src + head;
+    const uint32_t sMis = static_cast<uint32_t>(reinterpret_cast<uint64_t>(sBody) & 15u);
+
+    U32x4 out[kVecPerThread];
+    if (sMis == 0) {
+        const U32x4* s = reinterpret_cast<const U32x4*>(sBody);
+#pragma unroll
+        for (int k = 0; k < kVecPerThread; ++k) {
+            const uint32_t idx = threadIdx.x + k * kThreads;
+            if (idx < nVec) {
+                out[k] = __builtin_nontemporal_load(s + idx);
+            }
+        }
+    } else if (nVec != 0) {
+        // Irregular: stage the covering aligned vectors, then funnel-shift pairs of dwords.
+        Stage* st = stages + parity;
+        parity ^= 1u;
+        const U32x4* s = reinterpret_cast<const U32x4*>(sBody - sMis);
+#pragma unroll
+        for (int k = 0; k <= kVecPerThread; ++k) {
+            const uint32_t idx = threadIdx.x + k * kThreads;
+            if (idx <= nVec) {
+                st->v[idx] = __builtin_nontemporal_load(s + idx);
+            }
+        }
+        __syncthreads();
+        const uint32_t q = sMis >> 2;        // whole dwords to skip
+        const uint32_t shift = sMis & 3u;    // bytes to skip inside a dword
+#pragma unroll
+        for (int k = 0; k < kVecPerThread; ++k) {
+            const uint32_t idx = threadIdx.x + k * kThreads;
+            if (idx < nVec) {
+                const U32x4 a = st->v[idx];
+                const U32x4 b = st->v[idx + 1];
+                switch (q) {   // uniform: picks the five dwords that straddle the two staged vectors
+                    case 0: out[k] = Funnel(a.x, a.y, a.z, a.w, b.x, shift); break;
+                    case 1: out[k] = Funnel(a.y, a.z, a.w, b.x, b.y, shift); break;
+                    case 2: out[k] = Funnel(a.z, a.w, b.x, b.y, b.z, shift); break;
+                    default: out[k] = Funnel(a.w, b.x, b.y, b.z, b.w, shift); break;
+                }
+            }
+        }
+    }
+    for (uint32_t d = 0; d < nDst; ++d) {
+        U32x4* o = reinterpret_cast<U32x4*>(dstOf(d) + head);
+#pragma unroll
+        for (int k = 0; k < kVecPerThread; ++k) {
+            const uint32_t idx = threadIdx.x + k * kThreads;
+            if (idx < nVec) {
+                __builtin_nontemporal_store(out[k], o + idx);
+            }
+        }
+    }
+    // Up to 15 bytes in front of the body and up to 15 behind it.
+    const uint32_t edge = head + (bytes - bodyEnd);
+    if (threadIdx.x < edge) {
+        const uint32_t o = threadIdx.x < head ? threadIdx.x : bodyEnd + (threadIdx.x - head);
+        const uint8_t b = src[o];
+        for (uint32_t d = 0; d < nDst; ++d) {
+            dstOf(d)[o] = b;
+        }
+    }
+}
+
+// Fallback when destinations differ in alignment: lane-per-unit copies of the widest common unit.
+template <typename U, class DstFn>
+__device__ __forceinline__ void CopyUnits(const uint8_t* src, uint32_t bytes, uint32_t nDst, DstFn dstOf)
+{
+    const uint32_t n = bytes / sizeof(U);
     const U* s = reinterpret_cast<const U*>(src);
-    for (uint64_t i = threadIdx.x; i < n; i += kThreads) {
+    for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
         U v = __builtin_nontemporal_load(s + i);
         for (uint32_t d = 0; d < nDst; ++d) {
             __builtin_nontemporal_store(v, reinterpret_cast<U*>(dstOf(d)) + i);
@@ -69,30 +168,9 @@ __device__ __forceinline__ void CopyUnits(const uint8_t* src, uint64_t bytes, ui
 }
 
 template <class DstFn>
-__device__ __forceinline__ void CopyTile(const uint8_t* src, uint64_t bytes, uint32_t unit, uint32_t nDst, DstFn dstOf)
+__device__ __forceinline__ void CopyTileByUnit(const uint8_t* src, uint32_t bytes, uint32_t unit, uint32_t nDst, DstFn dstOf)
 {
-    if (unit == 16) {
-        const uint32_t nVec = static_cast<uint32_t>(bytes / 16);
-        const U32x4* s = reinterpret_cast<const U32x4*>(src);
-        U32x4 v[kVecPerThread];
-#pragma unroll
-        for (int k = 0; k < kVecPerThread; ++k) {
-            uint32_t idx = threadIdx.x + k * kThreads;
-            if (idx < nVec) {
-                v[k] = __builtin_nontemporal_load(s + idx);
-            }
-        }
-        for (uint32_t d = 0; d < nDst; ++d) {
-            U32x4* o = reinterpret_cast<U32x4*>(dstOf(d));
-#pragma unroll
-            for (int k = 0; k < kVecPerThread; ++k) {
-                uint32_t idx = threadIdx.x + k * kThreads;
-                if (idx < nVec) {
-                    __builtin_nontemporal_store(v[k], o + idx);
-                }
-            }
-        }
-    } else if (unit == 8) {
+    if (unit >= 8) {
         CopyUnits<uint64_t>(src, bytes, nDst, dstOf);
     } else if (unit == 4) {
         CopyUnits<uint32_t>(src, bytes, nDst, dstOf);
@@ -106,24 +184,29 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint64_t bytes, uin
 // ---- AllGather / AllGatherV --------------------------------------------------------------------
 __global__ __launch_bounds__(kThreads) void BcastCopyKernel(const BcastCopyArgs args)
 {
+    __shared__ Stage stage[2];
     const uint32_t lane = threadIdx.x & 63u;
     const uint64_t myLen = lane < args.nSeg ? args.len[lane] : 0;
     const uint32_t myTiles = static_cast<uint32_t>((myLen + kCopyTileBytes - 1) / kCopyTileBytes);
     const uint32_t incl = WaveInclusiveScan(myTiles);
     const uint32_t total = Uniform(__shfl(incl, 63, 64));
 
+    uint32_t parity = 0;
     for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
         const uint32_t seg = Uniform(SegmentOf(incl, tile));
         const uint32_t segFirst = seg == 0 ? 0u : Uniform(__shfl(incl, seg - 1, 64));
         const uint64_t off = static_cast<uint64_t>(tile - segFirst) * kCopyTileBytes;
         const uint64_t len = args.len[seg];
-        const uint64_t bytes = (len - off < kCopyTileBytes) ? len - off : kCopyTileBytes;
+        const uint32_t bytes = static_cast<uint32_t>((len - off < kCopyTileBytes) ? len - off : kCopyTileBytes);
         const uint8_t* src = static_cast<const uint8_t*>(args.src[seg]) + off;
         const uint64_t dOff = args.dstOff[seg] + off;
-        // args.unit carries the common alignment of the destination bases; the segment adds its own.
-        const uint32_t unit = AlignUnit(reinterpret_cast<uint64_t>(args.src[seg]) | len | args.dstOff[seg] | args.unit);
-        CopyTile(src, bytes, unit, args.nDst,
-                 [&](uint32_t d) { return static_cast<uint8_t*>(args.dst[d]) + dOff; });
+        auto dstOf = [&](uint32_t d) { return static_cast<uint8_t*>(args.dst[d]) + dOff; };
+        if (args.unit == 16) {   // destination bases are all 16-byte aligned, hence congruent
+            CopyTile(src, bytes, args.nDst, dstOf, stage, parity);
+        } else {
+            const uint32_t unit = AlignUnit(reinterpret_cast<uint64_t>(args.src[seg]) | len | args.dstOff[seg] | args.unit);
+            CopyTileByUnit(src, bytes, unit, args.nDst, dstOf);
+        }
     }
 }
 
@@ -165,6 +248,7 @@ __global__ __launch_bounds__(1024) void A2aPlanKernel(const A2aArgs args)
 // ballots when it crosses a segment boundary and then streams the tile.
 __global__ __launch_bounds__(kThreads) void A2aCopyKernel(const A2aArgs args)
 {
+    __shared__ Stage stage[2];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t n = args.n;
     const uint32_t total = args.rowStart[n];
@@ -178,8 +262,8 @@ __global__ __launch_bounds__(kThreads) void A2aCopyKernel(const A2aArgs args)
     const uint8_t* src = nullptr;
     uint8_t* dst = nullptr;
     uint64_t len = 0;
-    uint32_t unit = 1;
     bool haveRow = false;
+    uint32_t parity = 0;
 
     for (uint32_t t = t0; t < t1; ++t) {
         if (!haveRow || t >= rowEnd) {
@@ -201,18 +285,17 @@ __global__ __launch_bounds__(kThreads) void A2aCopyKernel(const A2aArgs args)
             src = static_cast<const uint8_t*>(args.send[seg]) + sd * args.esz;
             dst = static_cast<uint8_t*>(args.recv[row]) + rd * args.esz;
             len = cnt * args.esz;
-            unit = AlignUnit(reinterpret_cast<uint64_t>(src) | reinterpret_cast<uint64_t>(dst) | len);
         }
         const uint64_t off = static_cast<uint64_t>(t - segBegin) * kCopyTileBytes;
-        const uint64_t bytes = (len - off < kCopyTileBytes) ? len - off : kCopyTileBytes;
+        const uint32_t bytes = static_cast<uint32_t>((len - off < kCopyTileBytes) ? len - off : kCopyTileBytes);
         uint8_t* d = dst + off;
-        CopyTile(src + off, bytes, unit, 1u, [&](uint32_t) { return d; });
+        CopyTile(src + off, bytes, 1u, [&](uint32_t) { return d; }, stage, parity);
     }
 }
 
 }  // namespace
 
-hipError_t LaunchBcastCopy(const BcastCopyArgs& args, hipStream_t stream)
+hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t maxBlocks, hipStream_t stream)
 {
     uint64_t tiles = 0;
     for (uint32_t j = 0; j < args.nSeg; ++j) {
@@ -224,7 +307,6 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& args, hipStream_t stream)
     if (tiles > 0xFFFFFFF0ull) {
         return hipErrorInvalidValue;
     }
-    const uint32_t maxBlocks = 256 * 16;
     const uint32_t blocks = tiles < maxBlocks ? static_cast<uint32_t>(tiles) : maxBlocks;
     hipLaunchKernelGGL(BcastCopyKernel, dim3(blocks), dim3(kThreads), 0, stream, args);
     return hipGetLastError();

@@ -111,7 +111,7 @@ inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
     bool half = dtype == HCCL_DATA_TYPE_FP16 || dtype == HCCL_DATA_TYPE_BFP16;
     return (half && op == HCCL_REDUCE_SUM) ? 32u : 16u;   // eight fp32 accumulators vs one 16-byte pack
 }
-hipError_t LaunchBcastCopy(const BcastCopyArgs& args, hipStream_t stream);
+hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t maxBlocks, hipStream_t stream);
 hipError_t LaunchA2aPlan(const A2aArgs& args, hipStream_t stream);
 hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nBlocks, hipStream_t stream);
 
