@@ -215,7 +215,7 @@ struct World {
     bool a2aSlotUsed[kStagingSlots] = {};
     uint32_t a2aNext = 0;
     uint32_t reduceBlocks = 1u << 20;
-    uint32_t copyBlocks = 2048;
+    uint32_t copyTileBytes = 4096;
 
     ~World()
     {
@@ -299,7 +299,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->device = 0;
     }
     w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 1u << 20);
-    w->copyBlocks = EnvU32("HCCL_AMD_COPY_BLOCKS", 2048);
+    w->copyTileBytes = EnvU32("HCCL_AMD_COPY_TILE", 4096) == 16384 ? 16384 : 4096;
     ApplyAlgoEnv(w.get());
     return w;
 }
@@ -560,7 +560,7 @@ HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
     uint64_t bits = 0;
     for (uint32_t d = 0; d < b.nDst; ++d) bits |= reinterpret_cast<uint64_t>(b.dst[d]);
     b.unit = AlignUnitOf(bits);
-    HIP_OK(LaunchBcastCopy(b, w->copyBlocks, s));
+    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s));
     return HCCL_SUCCESS;
 }
 
@@ -624,13 +624,13 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
                     (unsigned long long)expected, j, i, (unsigned long long)sent);
                 return HCCL_E_PARA;
             }
-            tiles += (sent * esz + kCopyTileBytes - 1) / kCopyTileBytes;
+            tiles += (sent * esz + w->copyTileBytes - 1) / w->copyTileBytes;
         }
     }
     if (tiles == 0) {
         return HCCL_SUCCESS;
     }
-    if (tiles > 0xFFFFFFF0ull) {
+    if (tiles > 0x7FFFFFF0ull) {
         return HCCL_E_PARA;
     }
     HcclResult rc = EnsureA2aBuffers(w);
@@ -668,9 +668,9 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
     a.segEnd = a.rowStart + (n + 1);
     a.n = n;
     a.esz = esz;
+    a.tileBytes = w->copyTileBytes;
     HIP_OK(LaunchA2aPlan(a, s));
-    uint32_t blocks = tiles < w->copyBlocks ? static_cast<uint32_t>(tiles) : w->copyBlocks;
-    HIP_OK(LaunchA2aCopy(a, blocks, s));
+    HIP_OK(LaunchA2aCopy(a, static_cast<uint32_t>(tiles), s));
     HIP_OK(hipEventRecord(w->a2aSlotFree[slot], s));
     w->a2aSlotUsed[slot] = true;
     return HCCL_SUCCESS;

@@ -98,9 +98,9 @@ struct A2aArgs {
     uint32_t* segEnd;
     uint32_t n;
     uint32_t esz;
+    uint32_t tileBytes;   // 4096 or 16384: bytes one workgroup copies
 };
 
-constexpr uint32_t kCopyTileBytes = 16384;
 
 // Launchers (defined in the .hip files).  All are asynchronous on `stream`.
 // ldsBytes = (plan depth - 1) * ReduceAccBytes(dtype, op) * 256: the accumulator stack of nested levels.
@@ -111,8 +111,8 @@ inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
     bool half = dtype == HCCL_DATA_TYPE_FP16 || dtype == HCCL_DATA_TYPE_BFP16;
     return (half && op == HCCL_REDUCE_SUM) ? 32u : 16u;   // eight fp32 accumulators vs one 16-byte pack
 }
-hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t maxBlocks, hipStream_t stream);
+hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream);
 hipError_t LaunchA2aPlan(const A2aArgs& args, hipStream_t stream);
-hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nBlocks, hipStream_t stream);
+hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, hipStream_t stream);
 
 }  // namespace hccl_amd
