@@ -29,7 +29,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3max", "c3prod", "c4", "c5a", "c5b"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3max", "c3prod", "c4", "c5a", "c5b", "copycal"])
     ap.add_argument("--algo", default=None, help="override the algorithm of the workload (mesh/ring/rhd/nhr/...)")
     ap.add_argument("--others", action="store_true", help="also time the other BASELINE configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -139,6 +139,20 @@ class Workloads:
         hbm = (1 + n) * total * 2
         return step, hbm, total * 2, (n - 1) / n, (sends, recvs), \
             "AllGatherV fp16 rankSize=6 counts U[1Mi,32Mi]", "u8", n
+
+    def copycal(self, algo):
+        """Plain copy of known size (the rankSize == 1 shortcut): calibrates the HBM byte counters."""
+        t, h = self.torch, self.h
+        comms = self.world(1)
+        nbytes = 1 << 30
+        src = t.randint(0, 255, (nbytes,), generator=self.gen(1), device="cuda", dtype=t.uint8)
+        dst = t.empty(nbytes, dtype=t.uint8, device="cuda")
+        stream = self.stream
+
+        def step():
+            h.all_gather(comms[0], src, dst, nbytes, h.HcclDataType.UINT8, stream)
+
+        return step, 2 * nbytes, nbytes, 1.0, (src, dst), "plain copy 1 GiB (rankSize=1 AllGather)", "u8", 1
 
     def c4(self, algo):
         import numpy as np
