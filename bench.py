@@ -186,6 +186,7 @@ class Workloads:
 
 
 def time_steps(torch, stream, step, steps, warmup):
+    torch.cuda.synchronize()   # inputs were generated on torch's default stream
     for _ in range(warmup):
         step()
     stream.synchronize()

@@ -56,11 +56,17 @@ class World:
     def set_algo(self, kind, name):
         hccl_amd.set_algo(self.comms[0], kind, ALGO_BY_NAME[name])
 
+    def inputs_ready(self):
+        """Inputs are produced on torch's default stream; the collective runs on self.stream."""
+        import torch
+        torch.cuda.current_stream().synchronize()
+
     def sync(self):
         self.stream.synchronize()
 
     def all_reduce(self, sends, recvs, count, dtype, op, algo="mesh"):
         self.set_algo(OpKind.ALL_REDUCE, algo)
+        self.inputs_ready()
         with hccl_amd.group():
             for r in range(self.n):
                 hccl_amd.all_reduce(self.comms[r], sends[r], recvs[r], count, dtype, op, self.stream)
@@ -68,18 +74,21 @@ class World:
 
     def reduce_scatter(self, sends, recvs, recv_count, dtype, op, algo="mesh"):
         self.set_algo(OpKind.REDUCE_SCATTER, algo)
+        self.inputs_ready()
         with hccl_amd.group():
             for r in range(self.n):
                 hccl_amd.reduce_scatter(self.comms[r], sends[r], recvs[r], recv_count, dtype, op, self.stream)
         self.sync()
 
     def all_gather(self, sends, recvs, send_count, dtype):
+        self.inputs_ready()
         with hccl_amd.group():
             for r in range(self.n):
                 hccl_amd.all_gather(self.comms[r], sends[r], recvs[r], send_count, dtype, self.stream)
         self.sync()
 
     def all_gather_v(self, sends, recvs, counts, displs, dtype):
+        self.inputs_ready()
         with hccl_amd.group():
             for r in range(self.n):
                 hccl_amd.all_gather_v(self.comms[r], sends[r], int(counts[r]), recvs[r], counts, displs, dtype,
@@ -87,6 +96,7 @@ class World:
         self.sync()
 
     def all_to_all_v(self, sends, send_counts, sdispls, recvs, recv_counts, rdispls, dtype):
+        self.inputs_ready()
         with hccl_amd.group():
             for r in range(self.n):
                 hccl_amd.all_to_all_v(self.comms[r], sends[r], send_counts[r], sdispls[r], dtype, recvs[r],
