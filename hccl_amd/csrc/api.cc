@@ -215,7 +215,7 @@ struct World {
     bool a2aSlotUsed[kStagingSlots] = {};
     uint32_t a2aNext = 0;
     uint32_t reduceBlocks = 1u << 20;
-    uint32_t copyTileBytes = 4096;
+    uint32_t copyTileBytes = 0;
 
     ~World()
     {
@@ -299,7 +299,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->device = 0;
     }
     w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 1u << 20);
-    w->copyTileBytes = EnvU32("HCCL_AMD_COPY_TILE", 4096) == 16384 ? 16384 : 4096;
+    w->copyTileBytes = EnvU32("HCCL_AMD_COPY_TILE", 0);   // 0: chosen per collective
+    if (w->copyTileBytes != 1024 && w->copyTileBytes != 4096 && w->copyTileBytes != 16384) {
+        w->copyTileBytes = 0;
+    }
     ApplyAlgoEnv(w.get());
     return w;
 }
@@ -390,12 +393,12 @@ HcclResult TakeEvent(World* w, hipEvent_t* ev)
     return HCCL_SUCCESS;
 }
 
-size_t A2aTableBytes(uint32_t n) { return static_cast<size_t>(n) * n * sizeof(uint64_t); }
-
-// Device bytes of one slot: three u64 tables, rowStart (n + 1) and segEnd (n * n) as u32, 256-byte padded.
+// Bytes of one slot (host image == device image): a descriptor and a tile prefix (u32) per segment,
+// then the hint table (u32); 256-byte padded.
 size_t A2aSlotBytes(uint32_t n)
 {
-    size_t bytes = 3 * A2aTableBytes(n) + (static_cast<size_t>(n) * n + n + 1) * sizeof(uint32_t);
+    size_t nn = static_cast<size_t>(n) * n;
+    size_t bytes = nn * (kA2aDescWords * sizeof(uint64_t) + sizeof(uint32_t)) + (kA2aHintMax + 4) * sizeof(uint32_t);
     return (bytes + 255) & ~static_cast<size_t>(255);
 }
 
@@ -406,10 +409,9 @@ HcclResult EnsureA2aBuffers(World* w)
     if (w->a2aDev != nullptr) {
         return HCCL_SUCCESS;
     }
-    size_t tab = A2aTableBytes(w->n);
     HIP_OK(hipMalloc(reinterpret_cast<void**>(&w->a2aDev), kStagingSlots * A2aSlotBytes(w->n)));
     for (int s = 0; s < kStagingSlots; ++s) {
-        HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&w->a2aHost[s]), 3 * tab, hipHostMallocDefault));
+        HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&w->a2aHost[s]), A2aSlotBytes(w->n), hipHostMallocDefault));
         HIP_OK(hipEventCreateWithFlags(&w->a2aSlotFree[s], hipEventDisableTiming));
     }
     return HCCL_SUCCESS;
@@ -560,7 +562,10 @@ HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
     uint64_t bits = 0;
     for (uint32_t d = 0; d < b.nDst; ++d) bits |= reinterpret_cast<uint64_t>(b.dst[d]);
     b.unit = AlignUnitOf(bits);
-    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s));
+    // One wavefront per tile is fastest with a single destination; with several, the stores of a
+    // larger tile keep more of each destination's pages busy at a time.
+    const uint32_t tileBytes = w->copyTileBytes != 0 ? w->copyTileBytes : (b.nDst == 1 ? 1024u : 4096u);
+    HIP_OK(LaunchBcastCopy(b, tileBytes, s));
     return HCCL_SUCCESS;
 }
 
@@ -612,9 +617,10 @@ HcclResult RunAllGatherV(World* w, PendingOp& p, hipStream_t s)
 HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
-    const uint32_t esz = DataTypeSize(p.dtype);
+    const uint64_t esz = DataTypeSize(p.dtype);
+    const uint32_t tileBytes = w->copyTileBytes != 0 ? w->copyTileBytes : 1024u;
     // rank r's var = sendCounts | recvCounts | sdispls | rdispls (reference all_to_all_v.cc:617-643)
-    uint64_t tiles = 0;
+    uint32_t nSeg = 0;
     for (uint32_t i = 0; i < n; ++i) {
         for (uint32_t j = 0; j < n; ++j) {
             uint64_t sent = p.ranks[j].var[i];
@@ -624,14 +630,11 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
                     (unsigned long long)expected, j, i, (unsigned long long)sent);
                 return HCCL_E_PARA;
             }
-            tiles += (sent * esz + w->copyTileBytes - 1) / w->copyTileBytes;
+            nSeg += sent != 0;
         }
     }
-    if (tiles == 0) {
+    if (nSeg == 0) {
         return HCCL_SUCCESS;
-    }
-    if (tiles > 0x7FFFFFF0ull) {
-        return HCCL_E_PARA;
     }
     HcclResult rc = EnsureA2aBuffers(w);
     if (rc != HCCL_SUCCESS) {
@@ -642,35 +645,52 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
     if (w->a2aSlotUsed[slot]) {
         HIP_OK(hipEventSynchronize(w->a2aSlotFree[slot]));   // the call that last used this slot has finished
     }
-    uint8_t* dev = w->a2aDev + slot * A2aSlotBytes(n);
-    const size_t tab = A2aTableBytes(n);
-    uint64_t* host = w->a2aHost[slot];
-    uint64_t* hCnt = host;
-    uint64_t* hSd = host + static_cast<size_t>(n) * n;
-    uint64_t* hRd = host + 2 * static_cast<size_t>(n) * n;
-    for (uint32_t r = 0; r < n; ++r) {
-        const uint64_t* v = p.ranks[r].var.data();
-        memcpy(hCnt + static_cast<size_t>(r) * n, v, n * sizeof(uint64_t));
-        memcpy(hSd + static_cast<size_t>(r) * n, v + 2 * n, n * sizeof(uint64_t));
-        memcpy(hRd + static_cast<size_t>(r) * n, v + 3 * n, n * sizeof(uint64_t));
+    // One descriptor per non-empty segment, destination-major so that neighbouring tiles write
+    // neighbouring addresses: recv_i[rdispls_i[j] ...] = send_j[sdispls_j[i] ...]
+    // (reference ins_temp_all_to_all_v_mesh_1D.cc:229-246).
+    uint64_t* hDesc = w->a2aHost[slot];
+    uint32_t* hEnd = reinterpret_cast<uint32_t*>(hDesc + static_cast<size_t>(kA2aDescWords) * nSeg);
+    uint32_t* hHint = hEnd + ((nSeg + 1u) & ~1u);
+    uint64_t tiles = 0;
+    uint64_t misfit = 0;
+    bool congruent = true;
+    uint32_t k = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint64_t* vi = p.ranks[i].var.data();
+        for (uint32_t j = 0; j < n; ++j) {
+            const uint64_t* vj = p.ranks[j].var.data();
+            const uint64_t len = vj[i] * esz;
+            if (len == 0) {
+                continue;
+            }
+            const uint64_t src = reinterpret_cast<uint64_t>(p.ranks[j].send) + vj[2 * n + i] * esz;
+            const uint64_t dst = reinterpret_cast<uint64_t>(p.ranks[i].recv) + vi[3 * n + j] * esz;
+            uint64_t* d = hDesc + static_cast<size_t>(kA2aDescWords) * k;
+            d[0] = src;
+            d[1] = dst;
+            d[2] = len;
+            d[3] = tiles;
+            tiles += (len + tileBytes - 1) / tileBytes;
+            if (tiles > 0x7FFFFFF0ull) {
+                return HCCL_E_PARA;
+            }
+            hEnd[k] = static_cast<uint32_t>(tiles);
+            misfit |= src | dst | len;
+            congruent = congruent && ((src ^ dst) & 15u) == 0;
+            ++k;
+        }
     }
-    HIP_OK(hipMemcpyAsync(dev, host, 3 * tab, hipMemcpyHostToDevice, s));
-
     A2aArgs a{};
-    for (uint32_t r = 0; r < n; ++r) {
-        a.send[r] = p.ranks[r].send;
-        a.recv[r] = p.ranks[r].recv;
-    }
-    a.cnt = reinterpret_cast<const uint64_t*>(dev);
-    a.sdis = reinterpret_cast<const uint64_t*>(dev + tab);
-    a.rdis = reinterpret_cast<const uint64_t*>(dev + 2 * tab);
-    a.rowStart = reinterpret_cast<uint32_t*>(dev + 3 * tab);
-    a.segEnd = a.rowStart + (n + 1);
-    a.n = n;
-    a.esz = esz;
-    a.tileBytes = w->copyTileBytes;
-    HIP_OK(LaunchA2aPlan(a, s));
-    HIP_OK(LaunchA2aCopy(a, static_cast<uint32_t>(tiles), s));
+    uint32_t nHint = 0;
+    a.hintShift = BuildTileHints(hEnd, nSeg, static_cast<uint32_t>(tiles), kA2aHintMax, hHint, &nHint);
+    a.mode = !congruent ? COPY_GENERAL : ((misfit & 15u) == 0 ? COPY_ALIGNED : COPY_CONGRUENT);
+    const size_t used = reinterpret_cast<uint8_t*>(hHint + nHint + 1) - reinterpret_cast<uint8_t*>(hDesc);
+    uint8_t* dev = w->a2aDev + slot * A2aSlotBytes(n);
+    HIP_OK(hipMemcpyAsync(dev, hDesc, used, hipMemcpyHostToDevice, s));
+    a.desc = reinterpret_cast<const uint64_t*>(dev);
+    a.tileEnd = reinterpret_cast<const uint32_t*>(a.desc + static_cast<size_t>(kA2aDescWords) * nSeg);
+    a.hint = a.tileEnd + ((nSeg + 1u) & ~1u);
+    HIP_OK(LaunchA2aCopy(a, static_cast<uint32_t>(tiles), tileBytes, s));
     HIP_OK(hipEventRecord(w->a2aSlotFree[slot], s));
     w->a2aSlotUsed[slot] = true;
     return HCCL_SUCCESS;

@@ -72,8 +72,50 @@ struct ReduceArgs {
     uint32_t vecOk;   // every address the launch touches is 16-byte aligned
 };
 
+// ---- copies -------------------------------------------------------------------------------------
+// Copy work is a list of segments cut into tiles of `tileBytes`; workgroup t copies tile t.  The host
+// numbers the tiles: tileEnd[s] is the inclusive prefix sum of the segments' tile counts, and a hint
+// table over buckets of 2^hintShift tiles (hint[k] = first segment with tileEnd > k << hintShift, one
+// closing entry) bounds the search of a workgroup to the segments that touch its bucket.  The kernels
+// read these tables with scalar loads only.
+constexpr uint32_t kBcastHintMax = 64;      // buckets of the hint table held in the kernel arguments
+constexpr uint32_t kA2aHintMax = 4096;      // buckets of the hint table held in device memory
+
+enum CopyMode : uint32_t {
+    COPY_GENERAL = 0,     // source and destination of a segment may differ modulo 16: staged through LDS
+    COPY_CONGRUENT = 1,   // every segment has source == destination modulo 16
+    COPY_ALIGNED = 2,     // all addresses and lengths are multiples of 16
+};
+
+// Fills hint[0 .. nHint] and returns the shift; nHint = ((tiles - 1) >> shift) + 1 <= maxHint.
+template <typename HintT>
+inline uint32_t BuildTileHints(const uint32_t* tileEnd, uint32_t nSeg, uint32_t tiles, uint32_t maxHint, HintT* hint,
+                               uint32_t* nHintOut)
+{
+    uint32_t shift = 0;
+    while (((tiles - 1) >> shift) + 1 > maxHint) {
+        ++shift;
+    }
+    const uint32_t nHint = ((tiles - 1) >> shift) + 1;
+    uint32_t s = 0;
+    for (uint32_t k = 0; k < nHint; ++k) {
+        const uint64_t first = static_cast<uint64_t>(k) << shift;
+        while (tileEnd[s] <= first) {
+            ++s;
+        }
+        hint[k] = static_cast<HintT>(s);
+    }
+    while (s + 1 < nSeg && tileEnd[s] < tiles) {
+        ++s;
+    }
+    hint[nHint] = static_cast<HintT>(s);
+    *nHintOut = nHint;
+    return shift;
+}
+
 // One-to-many copy (AllGather / AllGatherV / single-rank shortcut): segment j is `len[j]` bytes read
-// once from src[j] and written to dst[d] + dstOff[j] for every d < nDst.
+// once from src[j] and written to dst[d] + dstOff[j] for every d < nDst.  The caller fills the first
+// six members; LaunchBcastCopy derives the rest.
 struct BcastCopyArgs {
     const void* src[kMaxRanks];
     void* dst[kMaxRanks];
@@ -81,26 +123,23 @@ struct BcastCopyArgs {
     uint64_t dstOff[kMaxRanks];
     uint32_t nSeg;
     uint32_t nDst;
-    uint32_t unit;   // widest power of two (<= 16) dividing every destination base address
+    uint32_t unit;        // widest power of two (<= 16) dividing every destination base address
+    uint32_t hintShift;
+    uint32_t tileEnd[kMaxRanks];
+    uint8_t hint[kBcastHintMax + 8];
 };
 
-// AlltoAllV.  Tables live in device memory, n x n row-major, in elements:
-//   cnt[j*n + i] = sendCounts_j[i], sdis[j*n + i] = sdispls_j[i], rdis[i*n + j] = rdispls_i[j].
-// rowStart[i] (n + 1 entries) and segEnd[i*n + j] are written by the plan kernel: tiles of
-// destination rank i start at rowStart[i]; segEnd is the inclusive tile prefix inside row i.
+// AlltoAllV: one descriptor of four u64 per non-empty segment (i <- j), all tables in device memory:
+//   desc[4s] = send_j + sdispls_j[i] * esz, desc[4s+1] = recv_i + rdispls_i[j] * esz,
+//   desc[4s+2] = length in bytes, desc[4s+3] = index of the segment's first tile.
+constexpr uint32_t kA2aDescWords = 4;
 struct A2aArgs {
-    const void* send[kMaxRanks];
-    void* recv[kMaxRanks];
-    const uint64_t* cnt;
-    const uint64_t* sdis;
-    const uint64_t* rdis;
-    uint32_t* rowStart;
-    uint32_t* segEnd;
-    uint32_t n;
-    uint32_t esz;
-    uint32_t tileBytes;   // 4096 or 16384: bytes one workgroup copies
+    const uint64_t* desc;
+    const uint32_t* tileEnd;
+    const uint32_t* hint;
+    uint32_t hintShift;
+    uint32_t mode;        // CopyMode
 };
-
 
 // Launchers (defined in the .hip files).  All are asynchronous on `stream`.
 // ldsBytes = (plan depth - 1) * ReduceAccBytes(dtype, op) * 256: the accumulator stack of nested levels.
@@ -112,7 +151,6 @@ inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
     return (half && op == HCCL_REDUCE_SUM) ? 32u : 16u;   // eight fp32 accumulators vs one 16-byte pack
 }
 hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream);
-hipError_t LaunchA2aPlan(const A2aArgs& args, hipStream_t stream);
-hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, hipStream_t stream);
+hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, uint32_t tileBytes, hipStream_t stream);
 
 }  // namespace hccl_amd
