@@ -428,7 +428,7 @@ uint32_t AlignUnitOf(uint64_t bits)
 // ---------------------------------------------------------------------------------------------
 uint32_t BlocksPerSub(const World* w, uint64_t subLen, uint32_t esz, uint64_t nSubTotal)
 {
-    uint64_t vecs = (subLen * esz + 15) / 16;
+    uint64_t vecs = (subLen * esz + 15) / 16 + 7;   // the kernel skips up to 7 lanes to start on a 128-byte line
     uint64_t maxUseful = (vecs + 255) / 256;
     if (maxUseful == 0) maxUseful = 1;
     uint64_t want = (w->reduceBlocks + nSubTotal - 1) / nSubTotal;
@@ -670,7 +670,7 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
             d[1] = dst;
             d[2] = len;
             d[3] = tiles;
-            tiles += (len + tileBytes - 1) / tileBytes;
+            tiles += TilesOf(len, dst, tileBytes);
             if (tiles > 0x7FFFFFF0ull) {
                 return HCCL_E_PARA;
             }

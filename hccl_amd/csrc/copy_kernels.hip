@@ -83,6 +83,19 @@ __device__ __forceinline__ U32x4 Funnel(uint32_t w0, uint32_t w1, uint32_t w2, u
                  __builtin_amdgcn_alignbyte(w3, w2, shift), __builtin_amdgcn_alignbyte(w4, w3, shift)};
 }
 
+// Tiles of a segment are cut so that every tile but the first starts on a 128-byte line of the
+// destination: tile k covers bytes [k * kTile - lead, (k + 1) * kTile - lead) of the segment, clipped
+// to [0, len), where lead is the offset of the segment's first destination byte within its line.  A
+// wavefront whose 1 KiB of stores straddles nine lines instead of eight costs write bandwidth.
+template <uint32_t kTile>
+__device__ __forceinline__ void TileRange(uint32_t k, uint32_t lead, uint64_t len, uint64_t* off, uint32_t* bytes)
+{
+    const uint64_t begin = k == 0 ? 0 : static_cast<uint64_t>(k) * kTile - lead;
+    const uint32_t cap = k == 0 ? kTile - lead : kTile;
+    *off = begin;
+    *bytes = static_cast<uint32_t>(len - begin < cap ? len - begin : cap);
+}
+
 // Lane i gets `v` of lane i + 1; lane 63 keeps `last`.  Must run with the whole wavefront active.
 __device__ __forceinline__ U32x4 NextLane(U32x4 v, U32x4 last)
 {
@@ -184,9 +197,11 @@ __global__ __launch_bounds__(T) void BcastCopyKernel(const BcastCopyArgs args)
     const uint32_t tile = blockIdx.x;
     const uint32_t seg = FindSegment(tile, args.hintShift, args.hint, args.tileEnd);
     const uint32_t segFirst = seg == 0 ? 0u : args.tileEnd[seg - 1];
-    const uint64_t off = static_cast<uint64_t>(tile - segFirst) * kTile;
     const uint64_t len = args.len[seg];
-    const uint32_t bytes = static_cast<uint32_t>((len - off < kTile) ? len - off : kTile);
+    const uint32_t lead = TileLead(reinterpret_cast<uint64_t>(args.dst[0]) + args.dstOff[seg]);
+    uint64_t off;
+    uint32_t bytes;
+    TileRange<kTile>(tile - segFirst, lead, len, &off, &bytes);
     const uint8_t* src = static_cast<const uint8_t*>(args.src[seg]) + off;
     const uint64_t dOff = args.dstOff[seg] + off;
     auto dstOf = [&](uint32_t d) { return static_cast<uint8_t*>(args.dst[d]) + dOff; };
@@ -220,8 +235,9 @@ __global__ __launch_bounds__(T) void A2aCopyKernel(const A2aArgs args)
     const uint64_t srcBase = desc[0];
     const uint64_t dstBase = desc[1];
     const uint64_t len = desc[2];
-    const uint64_t off = (tile - desc[3]) * kTile;
-    const uint32_t bytes = static_cast<uint32_t>((len - off < kTile) ? len - off : kTile);
+    uint64_t off;
+    uint32_t bytes;
+    TileRange<kTile>(tile - static_cast<uint32_t>(desc[3]), TileLead(dstBase), len, &off, &bytes);
     const uint8_t* src = reinterpret_cast<const uint8_t*>(srcBase + off);
     uint8_t* dst = reinterpret_cast<uint8_t*>(dstBase + off);
     CopyTile<T, MODE>(src, bytes, 1u, [&](uint32_t) { return dst; });
@@ -258,7 +274,7 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
     uint64_t misfit = 0;      // non-zero low bits: some segment is not 16-byte aligned on both sides
     bool congruent = a.unit == 16;
     for (uint32_t j = 0; j < a.nSeg; ++j) {
-        tiles += (a.len[j] + tileBytes - 1) / tileBytes;
+        tiles += TilesOf(a.len[j], reinterpret_cast<uint64_t>(a.dst[0]) + a.dstOff[j], tileBytes);
         if (tiles > 0x7FFFFFF0ull) {
             return hipErrorInvalidValue;
         }

@@ -87,6 +87,15 @@ enum CopyMode : uint32_t {
     COPY_ALIGNED = 2,     // all addresses and lengths are multiples of 16
 };
 
+// Offset of a destination address within its 128-byte line, and the number of tiles of a segment of
+// `len` bytes whose tiles are cut at the destination's line boundaries (all but the first tile start
+// on a line).
+__host__ __device__ inline uint32_t TileLead(uint64_t dstAddr) { return static_cast<uint32_t>(dstAddr & 127u); }
+inline uint64_t TilesOf(uint64_t len, uint64_t dstAddr, uint32_t tileBytes)
+{
+    return len == 0 ? 0 : (len + TileLead(dstAddr) + tileBytes - 1) / tileBytes;
+}
+
 // Fills hint[0 .. nHint] and returns the shift; nHint = ((tiles - 1) >> shift) + 1 <= maxHint.
 template <typename HintT>
 inline uint32_t BuildTileHints(const uint32_t* tileEnd, uint32_t nSeg, uint32_t tiles, uint32_t maxHint, HintT* hint,

@@ -331,17 +331,24 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
 
     // When vecOk, every source and destination address of this sub-segment has the same offset from a
     // 16-byte boundary: `head` elements bring them all onto it, a 128-bit body follows, and fewer than
-    // W elements remain.  Otherwise everything goes element by element.
+    // W elements remain.  Otherwise everything goes element by element.  The body's vectors are dealt
+    // to the lanes shifted by `lead`, so that lane 0 of every wavefront starts a 128-byte line of the
+    // first source (a wavefront whose 1 KiB straddles nine lines fetches two of them twice).
     uint64_t head = len;
     uint64_t nVec = 0;
+    uint32_t lead = 0;
     if (args.vecOk) {
-        const uint32_t mis = static_cast<uint32_t>((reinterpret_cast<uint64_t>(args.src[0]) + srcOff * sizeof(S)) & 15u);
+        const uint64_t addr = reinterpret_cast<uint64_t>(args.src[0]) + srcOff * sizeof(S);
+        const uint32_t mis = static_cast<uint32_t>(addr & 15u);
         head = mis ? (16u - mis) / sizeof(S) : 0;
         head = head < len ? head : len;
         nVec = (len - head) / W;
+        lead = static_cast<uint32_t>(((addr + head * sizeof(S)) >> 4) & 7u);
     }
-    for (uint64_t v = first; v < nVec; v += stride) {
-        ReduceOne<E, W>(bp, accStack, args, head + v * W, dstOff, g);
+    for (uint64_t u = first; u < nVec + lead; u += stride) {
+        if (u >= lead) {
+            ReduceOne<E, W>(bp, accStack, args, head + (u - lead) * W, dstOff, g);
+        }
     }
     const uint64_t bodyEnd = head + nVec * W;
     const uint64_t nScalar = head + (len - bodyEnd);
