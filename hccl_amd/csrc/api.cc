@@ -215,6 +215,7 @@ struct World {
     bool a2aSlotUsed[kStagingSlots] = {};
     uint32_t a2aNext = 0;
     uint32_t reduceBlocks = 1u << 20;
+    uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
 
     ~World()
@@ -299,6 +300,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->device = 0;
     }
     w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 1u << 20);
+    w->reduceThreads = EnvU32("HCCL_AMD_REDUCE_THREADS", 0);
+    if (w->reduceThreads != 64 && w->reduceThreads != 128 && w->reduceThreads != 256) {
+        w->reduceThreads = 0;
+    }
     w->copyTileBytes = EnvU32("HCCL_AMD_COPY_TILE", 0);   // 0: chosen per collective
     if (w->copyTileBytes != 1024 && w->copyTileBytes != 4096 && w->copyTileBytes != 16384) {
         w->copyTileBytes = 0;
@@ -426,10 +431,10 @@ uint32_t AlignUnitOf(uint64_t bits)
 // ---------------------------------------------------------------------------------------------
 // Launches.  `s` is the stream the fused kernel runs on.
 // ---------------------------------------------------------------------------------------------
-uint32_t BlocksPerSub(const World* w, uint64_t subLen, uint32_t esz, uint64_t nSubTotal)
+uint32_t BlocksPerSub(const World* w, uint64_t subLen, uint32_t esz, uint64_t nSubTotal, uint32_t threads)
 {
     uint64_t vecs = (subLen * esz + 15) / 16 + 7;   // the kernel skips up to 7 lanes to start on a 128-byte line
-    uint64_t maxUseful = (vecs + 255) / 256;
+    uint64_t maxUseful = (vecs + threads - 1) / threads;
     if (maxUseful == 0) maxUseful = 1;
     uint64_t want = (w->reduceBlocks + nSubTotal - 1) / nSubTotal;
     if (want == 0) want = 1;
@@ -458,12 +463,15 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
         uint64_t last = a.groupLen > before ? a.groupLen - before : 0;
         longest = last > a.subLen ? last : a.subLen;
     }
-    a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs);
+    // Small workgroups retire sooner and keep the window of addresses in flight compact; nested fold
+    // programs park accumulators in LDS and want a few more lanes per workgroup to hide that.
+    a.threads = w->reduceThreads != 0 ? w->reduceThreads : (plan.maxDepth > 1 ? 128u : 64u);
+    a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
     uint64_t blocks = subs * a.blocksPerSub;
     if (blocks == 0 || blocks > 0x7FFFFFFFull) {
         return HCCL_E_INTERNAL;
     }
-    const uint32_t lds = (plan.maxDepth - 1) * ReduceAccBytes(dtype, op) * 256u;
+    const uint32_t lds = (plan.maxDepth - 1) * ReduceAccBytes(dtype, op) * a.threads;
     HIP_OK(LaunchReduce(a, dtype, op, static_cast<uint32_t>(blocks), lds, s));
     return HCCL_SUCCESS;
 }

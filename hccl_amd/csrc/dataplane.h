@@ -12,6 +12,7 @@
 namespace hccl_amd {
 
 constexpr int kMaxRanks = HCCL_AMD_MAX_RANKS;
+constexpr uint32_t kMaxReduceThreads = 256;   // lanes of a reduce workgroup (64, 128 or 256), one 16-byte vector each
 
 // ---------------------------------------------------------------------------------------------
 // Fold programs
@@ -70,6 +71,7 @@ struct ReduceArgs {
     uint32_t progSubStride;
     uint32_t blocksPerSub;
     uint32_t vecOk;   // every address the launch touches is 16-byte aligned
+    uint32_t threads; // workgroup size of the launch
 };
 
 // ---- copies -------------------------------------------------------------------------------------
@@ -151,7 +153,7 @@ struct A2aArgs {
 };
 
 // Launchers (defined in the .hip files).  All are asynchronous on `stream`.
-// ldsBytes = (plan depth - 1) * ReduceAccBytes(dtype, op) * 256: the accumulator stack of nested levels.
+// ldsBytes = (plan depth - 1) * ReduceAccBytes(dtype, op) * args.threads: the accumulator stack of nested levels.
 hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t nBlocks,
                         uint32_t ldsBytes, hipStream_t stream);
 inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)

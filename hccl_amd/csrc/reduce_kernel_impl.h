@@ -26,7 +26,7 @@ namespace hccl_amd {
 namespace detail {
 
 constexpr int kSum = 0, kProd = 1, kMax = 2, kMin = 3;
-constexpr int kThreads = 256;
+constexpr int kThreads = kMaxReduceThreads;   // upper bound; the launch picks args.threads
 
 // ---------------------------------------------------------------------------------------------
 // Element semantics.  S = storage type, A = accumulator type.
@@ -181,23 +181,23 @@ struct AccWords {
 };
 
 template <class E, int W>
-__device__ __forceinline__ void PushAcc(uint32_t* stack, uint32_t level, const AccPack<E, W>& acc)
+__device__ __forceinline__ void PushAcc(uint32_t* stack, uint32_t threads, uint32_t level, const AccPack<E, W>& acc)
 {
     AccWords<E, W> words = {};
     __builtin_memcpy(&words, &acc, sizeof(acc));
 #pragma unroll
     for (int i = 0; i < AccWords<E, W>::kCount; ++i) {
-        stack[(level * AccWords<E, W>::kCount + i) * kThreads + threadIdx.x] = words.w[i];
+        stack[(level * AccWords<E, W>::kCount + i) * threads + threadIdx.x] = words.w[i];
     }
 }
 
 template <class E, int W>
-__device__ __forceinline__ void PopAcc(const uint32_t* stack, uint32_t level, AccPack<E, W>& acc)
+__device__ __forceinline__ void PopAcc(const uint32_t* stack, uint32_t threads, uint32_t level, AccPack<E, W>& acc)
 {
     AccWords<E, W> words;
 #pragma unroll
     for (int i = 0; i < AccWords<E, W>::kCount; ++i) {
-        words.w[i] = stack[(level * AccWords<E, W>::kCount + i) * kThreads + threadIdx.x];
+        words.w[i] = stack[(level * AccWords<E, W>::kCount + i) * threads + threadIdx.x];
     }
     __builtin_memcpy(&acc, &words, sizeof(acc));
 }
@@ -242,7 +242,7 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
             if (b + i < nLeaves) {
                 const uint32_t ctl = Uniform(bp.ctl[b + i]);
                 if (ctl & kCtlOpen) {
-                    PushAcc<E, W>(stack, level, acc);
+                    PushAcc<E, W>(stack, args.threads, level, acc);
                     ++level;
                     init = true;
                 }
@@ -261,7 +261,7 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
                 for (uint32_t closes = ctl & 0x7Fu; closes != 0; --closes) {
                     AccPack<E, W> outer;
                     --level;
-                    PopAcc<E, W>(stack, level, outer);
+                    PopAcc<E, W>(stack, args.threads, level, outer);
 #pragma unroll
                     for (int w = 0; w < W; ++w) {
                         acc.a[w] = E::Fold(acc.a[w], outer.a[w]);   // nested value is src, enclosing level is dst
@@ -284,7 +284,7 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
     }
 }
 
-// Dynamic LDS: the accumulator stack, (plan depth - 1) * accumulator bytes * kThreads.
+// Dynamic LDS: the accumulator stack, (plan depth - 1) * accumulator bytes * args.threads.
 template <class E>
 __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
 {
@@ -326,8 +326,8 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     }
     __syncthreads();
 
-    const uint64_t stride = static_cast<uint64_t>(args.blocksPerSub) * kThreads;
-    const uint64_t first = static_cast<uint64_t>(blk) * kThreads + threadIdx.x;
+    const uint64_t stride = static_cast<uint64_t>(args.blocksPerSub) * args.threads;
+    const uint64_t first = static_cast<uint64_t>(blk) * args.threads + threadIdx.x;
 
     // When vecOk, every source and destination address of this sub-segment has the same offset from a
     // 16-byte boundary: `head` elements bring them all onto it, a 128-bit body follows, and fewer than

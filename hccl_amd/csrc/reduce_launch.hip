@@ -20,10 +20,10 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
         case HCCL_DATA_TYPE_FP64: fn = SelectReduceF64(o); break;
         default: break;
     }
-    if (fn == nullptr || nBlocks == 0) {
+    if (fn == nullptr || nBlocks == 0 || (args.threads != 64 && args.threads != 128 && args.threads != 256)) {
         return hipErrorInvalidValue;
     }
-    hipLaunchKernelGGL(fn, dim3(nBlocks), dim3(detail::kThreads), ldsBytes, stream, args);
+    hipLaunchKernelGGL(fn, dim3(nBlocks), dim3(args.threads), ldsBytes, stream, args);
     return hipGetLastError();
 }
 
