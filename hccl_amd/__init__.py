@@ -103,6 +103,12 @@ def lib():
     L.HcclAllGather.argtypes = [vp, vp, u64, i32, vp, vp]
     L.HcclAllGatherV.argtypes = [vp, u64, vp, vp, vp, i32, vp, vp]
     L.HcclAlltoAllV.argtypes = [vp, vp, vp, i32, vp, vp, vp, i32, vp, vp]
+    L.HcclAlltoAll.argtypes = [vp, u64, i32, vp, u64, i32, vp, vp]
+    L.HcclAlltoAllVC.argtypes = [vp, vp, i32, vp, i32, vp, vp]
+    L.HcclReduceScatterV.argtypes = [vp, vp, vp, vp, u64, i32, i32, vp, vp]
+    L.HcclReduce.argtypes = [vp, vp, u64, i32, i32, u32, vp, vp]
+    L.HcclBroadcast.argtypes = [vp, u64, i32, u32, vp, vp]
+    L.HcclScatter.argtypes = [vp, vp, u64, i32, u32, vp, vp]
     L.HcclCommInitAll.argtypes = [u32, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(vp)]
     L.HcclGetRootInfo.argtypes = [vp]
     L.HcclCommInitRootInfo.argtypes = [u32, vp, u32, ctypes.POINTER(vp)]
@@ -117,6 +123,7 @@ def lib():
     L.HcclAmdGetAlgo.argtypes = [vp, i32, ctypes.POINTER(i32)]
     L.HcclAmdGetFoldProgram.argtypes = [i32, i32, u32, u32, vp, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
     for name in ("HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV",
+                 "HcclAlltoAll", "HcclAlltoAllVC", "HcclReduceScatterV", "HcclReduce", "HcclBroadcast", "HcclScatter",
                  "HcclCommInitAll", "HcclGetRootInfo", "HcclCommInitRootInfo", "HcclCommDestroy", "HcclGetRankSize",
                  "HcclGetRankId", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
                  "HcclAmdGetFoldProgram"):
@@ -294,3 +301,48 @@ def all_to_all_v(hccl_comm, send_buf, send_counts, sdispls, send_type, recv_buf,
                                _as_ptr(recv_buf), _u64_array(recv_counts, n), _u64_array(rdispls, n), int(recv_type),
                                hccl_comm, _as_stream(stream))
     return check(code, "HcclAlltoAllV")
+
+
+def all_to_all(hccl_comm, send_buf, send_count, send_type, recv_buf, recv_count, recv_type, stream=None):
+    code = lib().HcclAlltoAll(_as_ptr(send_buf), ctypes.c_uint64(send_count), int(send_type), _as_ptr(recv_buf),
+                              ctypes.c_uint64(recv_count), int(recv_type), hccl_comm, _as_stream(stream))
+    return check(code, "HcclAlltoAll")
+
+
+def all_to_all_vc(hccl_comm, send_buf, send_count_matrix, send_type, recv_buf, recv_type, stream=None):
+    """send_count_matrix: rankSize x rankSize element counts, row = sender, column = receiver (flat or nested)."""
+    n = get_rank_size(hccl_comm)
+    flat = send_count_matrix
+    if not isinstance(flat, ctypes.Array):
+        flat = [int(v) for row in send_count_matrix for v in (row if hasattr(row, "__len__") else [row])]
+    code = lib().HcclAlltoAllVC(_as_ptr(send_buf), _u64_array(flat, n * n), int(send_type), _as_ptr(recv_buf),
+                                int(recv_type), hccl_comm, _as_stream(stream))
+    return check(code, "HcclAlltoAllVC")
+
+
+def reduce_scatter_v(hccl_comm, send_buf, send_counts, send_displs, recv_buf, recv_count,
+                     data_type=HcclDataType.FP32, reduce_op=HcclReduceOp.SUM, stream=None):
+    n = get_rank_size(hccl_comm)
+    code = lib().HcclReduceScatterV(_as_ptr(send_buf), _u64_array(send_counts, n), _u64_array(send_displs, n),
+                                    _as_ptr(recv_buf), ctypes.c_uint64(recv_count), int(data_type), int(reduce_op),
+                                    hccl_comm, _as_stream(stream))
+    return check(code, "HcclReduceScatterV")
+
+
+def reduce(hccl_comm, send_buf, recv_buf, count, data_type=HcclDataType.FP32, reduce_op=HcclReduceOp.SUM, root=0,
+           stream=None):
+    code = lib().HcclReduce(_as_ptr(send_buf), _as_ptr(recv_buf), ctypes.c_uint64(count), int(data_type),
+                            int(reduce_op), ctypes.c_uint32(root), hccl_comm, _as_stream(stream))
+    return check(code, "HcclReduce")
+
+
+def broadcast(hccl_comm, buf, count, data_type=HcclDataType.FP32, root=0, stream=None):
+    code = lib().HcclBroadcast(_as_ptr(buf), ctypes.c_uint64(count), int(data_type), ctypes.c_uint32(root), hccl_comm,
+                               _as_stream(stream))
+    return check(code, "HcclBroadcast")
+
+
+def scatter(hccl_comm, send_buf, recv_buf, recv_count, data_type=HcclDataType.FP32, root=0, stream=None):
+    code = lib().HcclScatter(_as_ptr(send_buf), _as_ptr(recv_buf), ctypes.c_uint64(recv_count), int(data_type),
+                             ctypes.c_uint32(root), hccl_comm, _as_stream(stream))
+    return check(code, "HcclScatter")

@@ -142,7 +142,10 @@ HcclResult CheckReduceOp(HcclDataType t, HcclReduceOp op)
 // ---------------------------------------------------------------------------------------------
 // World, communicators, pending collectives
 // ---------------------------------------------------------------------------------------------
-enum class OpType { ALL_REDUCE, REDUCE_SCATTER, ALL_GATHER, ALL_GATHER_V, ALL_TO_ALL_V };
+enum class OpType {
+    ALL_REDUCE, REDUCE_SCATTER, ALL_GATHER, ALL_GATHER_V, ALL_TO_ALL_V,
+    REDUCE_SCATTER_V, REDUCE, BROADCAST, SCATTER
+};
 
 const char* OpName(OpType t)
 {
@@ -151,6 +154,10 @@ const char* OpName(OpType t)
         case OpType::REDUCE_SCATTER: return "ReduceScatter";
         case OpType::ALL_GATHER: return "AllGather";
         case OpType::ALL_GATHER_V: return "AllGatherV";
+        case OpType::REDUCE_SCATTER_V: return "ReduceScatterV";
+        case OpType::REDUCE: return "Reduce";
+        case OpType::BROADCAST: return "Broadcast";
+        case OpType::SCATTER: return "Scatter";
         default: return "AlltoAllV";
     }
 }
@@ -160,7 +167,9 @@ struct RankArgs {
     void* recv = nullptr;
     hipStream_t stream = nullptr;
     bool arrived = false;
-    std::vector<uint64_t> var;   // AllGatherV: counts | displs ; AlltoAllV: sendCounts | recvCounts | sdispls | rdispls
+    // AllGatherV: counts | displs | sendCount ; AlltoAllV: sendCounts | recvCounts | sdispls | rdispls ;
+    // ReduceScatterV: counts | displs | recvCount
+    std::vector<uint64_t> var;
 };
 
 struct PendingOp {
@@ -168,6 +177,7 @@ struct PendingOp {
     HcclDataType dtype;
     HcclReduceOp op = HCCL_REDUCE_RESERVED;
     uint64_t count = 0;
+    uint32_t root = 0;
     uint32_t arrived = 0;
     bool done = false;
     HcclResult result = HCCL_SUCCESS;
@@ -622,27 +632,24 @@ HcclResult RunAllGatherV(World* w, PendingOp& p, hipStream_t s)
     return RunBcast(w, b, s);
 }
 
-HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
+// One (source, destination, length in bytes) copy; sources and destinations are arbitrary device addresses.
+struct CopySeg {
+    uint64_t src;
+    uint64_t dst;
+    uint64_t len;
+};
+
+// Copies a list of at most n * n non-empty segments with one launch of the descriptor-driven copy kernel.
+HcclResult RunSegmentCopy(World* w, const std::vector<CopySeg>& segs, hipStream_t s)
 {
     const uint32_t n = w->n;
-    const uint64_t esz = DataTypeSize(p.dtype);
     const uint32_t tileBytes = w->copyTileBytes != 0 ? w->copyTileBytes : 1024u;
-    // rank r's var = sendCounts | recvCounts | sdispls | rdispls (reference all_to_all_v.cc:617-643)
-    uint32_t nSeg = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-        for (uint32_t j = 0; j < n; ++j) {
-            uint64_t sent = p.ranks[j].var[i];
-            uint64_t expected = p.ranks[i].var[n + j];
-            if (sent != expected) {
-                Log(1, "AlltoAllV: rank %u recvCounts[%u]=%llu but rank %u sendCounts[%u]=%llu", i, j,
-                    (unsigned long long)expected, j, i, (unsigned long long)sent);
-                return HCCL_E_PARA;
-            }
-            nSeg += sent != 0;
-        }
-    }
+    const uint32_t nSeg = static_cast<uint32_t>(segs.size());
     if (nSeg == 0) {
         return HCCL_SUCCESS;
+    }
+    if (nSeg > n * n) {
+        return HCCL_E_INTERNAL;
     }
     HcclResult rc = EnsureA2aBuffers(w);
     if (rc != HCCL_SUCCESS) {
@@ -653,40 +660,26 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
     if (w->a2aSlotUsed[slot]) {
         HIP_OK(hipEventSynchronize(w->a2aSlotFree[slot]));   // the call that last used this slot has finished
     }
-    // One descriptor per non-empty segment, destination-major so that neighbouring tiles write
-    // neighbouring addresses: recv_i[rdispls_i[j] ...] = send_j[sdispls_j[i] ...]
-    // (reference ins_temp_all_to_all_v_mesh_1D.cc:229-246).
     uint64_t* hDesc = w->a2aHost[slot];
     uint32_t* hEnd = reinterpret_cast<uint32_t*>(hDesc + static_cast<size_t>(kA2aDescWords) * nSeg);
     uint32_t* hHint = hEnd + ((nSeg + 1u) & ~1u);
     uint64_t tiles = 0;
     uint64_t misfit = 0;
     bool congruent = true;
-    uint32_t k = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-        const uint64_t* vi = p.ranks[i].var.data();
-        for (uint32_t j = 0; j < n; ++j) {
-            const uint64_t* vj = p.ranks[j].var.data();
-            const uint64_t len = vj[i] * esz;
-            if (len == 0) {
-                continue;
-            }
-            const uint64_t src = reinterpret_cast<uint64_t>(p.ranks[j].send) + vj[2 * n + i] * esz;
-            const uint64_t dst = reinterpret_cast<uint64_t>(p.ranks[i].recv) + vi[3 * n + j] * esz;
-            uint64_t* d = hDesc + static_cast<size_t>(kA2aDescWords) * k;
-            d[0] = src;
-            d[1] = dst;
-            d[2] = len;
-            d[3] = tiles;
-            tiles += TilesOf(len, dst, tileBytes);
-            if (tiles > 0x7FFFFFF0ull) {
-                return HCCL_E_PARA;
-            }
-            hEnd[k] = static_cast<uint32_t>(tiles);
-            misfit |= src | dst | len;
-            congruent = congruent && ((src ^ dst) & 15u) == 0;
-            ++k;
+    for (uint32_t k = 0; k < nSeg; ++k) {
+        const CopySeg& seg = segs[k];
+        uint64_t* d = hDesc + static_cast<size_t>(kA2aDescWords) * k;
+        d[0] = seg.src;
+        d[1] = seg.dst;
+        d[2] = seg.len;
+        d[3] = tiles;
+        tiles += TilesOf(seg.len, seg.dst, tileBytes);
+        if (tiles > 0x7FFFFFF0ull) {
+            return HCCL_E_PARA;
         }
+        hEnd[k] = static_cast<uint32_t>(tiles);
+        misfit |= seg.src | seg.dst | seg.len;
+        congruent = congruent && ((seg.src ^ seg.dst) & 15u) == 0;
     }
     A2aArgs a{};
     uint32_t nHint = 0;
@@ -704,6 +697,155 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
     return HCCL_SUCCESS;
 }
 
+HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    const uint64_t esz = DataTypeSize(p.dtype);
+    // rank r's var = sendCounts | recvCounts | sdispls | rdispls (reference all_to_all_v.cc:617-643)
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t j = 0; j < n; ++j) {
+            uint64_t sent = p.ranks[j].var[i];
+            uint64_t expected = p.ranks[i].var[n + j];
+            if (sent != expected) {
+                Log(1, "AlltoAllV: rank %u recvCounts[%u]=%llu but rank %u sendCounts[%u]=%llu", i, j,
+                    (unsigned long long)expected, j, i, (unsigned long long)sent);
+                return HCCL_E_PARA;
+            }
+        }
+    }
+    // One descriptor per non-empty segment, destination-major so that neighbouring tiles write
+    // neighbouring addresses: recv_i[rdispls_i[j] ...] = send_j[sdispls_j[i] ...]
+    // (reference ins_temp_all_to_all_v_mesh_1D.cc:229-246).
+    std::vector<CopySeg> segs;
+    segs.reserve(static_cast<size_t>(n) * n);
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint64_t* vi = p.ranks[i].var.data();
+        for (uint32_t j = 0; j < n; ++j) {
+            const uint64_t* vj = p.ranks[j].var.data();
+            const uint64_t len = vj[i] * esz;
+            if (len == 0) {
+                continue;
+            }
+            segs.push_back({reinterpret_cast<uint64_t>(p.ranks[j].send) + vj[2 * n + i] * esz,
+                            reinterpret_cast<uint64_t>(p.ranks[i].recv) + vi[3 * n + j] * esz, len});
+        }
+    }
+    return RunSegmentCopy(w, segs, s);
+}
+
+// ReduceScatterV, mesh order: rank k's output = in_k[displs[k] ..] first, then the other ranks ascending
+// (reference ins_temp_reduce_scatter_v_mesh_1D.cc:109-162).  Every rank must pass the same counts / displs.
+HcclResult RunReduceScatterV(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    const std::vector<uint64_t>& ref = p.ranks[0].var;   // counts | displs | recvCount
+    uint64_t longest = 0;
+    for (uint32_t r = 0; r < n; ++r) {
+        const std::vector<uint64_t>& v = p.ranks[r].var;
+        if (memcmp(v.data(), ref.data(), 2 * n * sizeof(uint64_t)) != 0) {
+            Log(1, "ReduceScatterV: rank %u passed sendCounts / sendDispls that differ from rank 0", r);
+            return HCCL_E_PARA;
+        }
+        if (v[2 * n] != ref[r]) {
+            Log(1, "ReduceScatterV: rank %u recvCount %llu != sendCounts[%u] %llu", r, (unsigned long long)v[2 * n], r,
+                (unsigned long long)ref[r]);
+            return HCCL_E_PARA;
+        }
+        if (ref[r] != 0 && (p.ranks[r].send == nullptr || p.ranks[r].recv == nullptr)) {
+            return HCCL_E_PTR;
+        }
+        longest = ref[r] > longest ? ref[r] : longest;
+    }
+    if (longest == 0) {
+        return HCCL_SUCCESS;
+    }
+    DevicePlan plan;
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, HCCL_AMD_ALGO_MESH, &plan);
+    if (rc != HCCL_SUCCESS) {
+        return rc;
+    }
+    ReduceArgs a{};
+    for (uint32_t r = 0; r < n; ++r) {
+        a.src[r] = p.ranks[r].send;
+        a.dst[r] = p.ranks[r].recv;
+        a.groupLenV[r] = ref[r];
+        a.groupOffV[r] = ref[n + r];
+    }
+    a.prog = plan.dev;
+    a.varGroups = 1;
+    a.nDst = 1;
+    a.dstOwn = 1;
+    a.nGroup = n;
+    a.nSub = 1;
+    a.groupLen = a.subLen = longest;
+    a.total = static_cast<uint64_t>(n) * longest;
+    a.progGroupStride = plan.nProg > 1 ? 1 : 0;
+    return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+}
+
+// Reduce, mesh order: out_root = in_0, then in_1 .. in_{N-1} folded in ascending (reference
+// reduce_mesh_1D.cc:268-300): the AllReduce rank-order program with the root's recvBuf as only destination.
+HcclResult RunReduce(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    if (p.ranks[p.root].recv == nullptr) {
+        return HCCL_E_PTR;
+    }
+    DevicePlan plan;
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_ALL_REDUCE, HCCL_AMD_ALGO_MESH, &plan);
+    if (rc != HCCL_SUCCESS) {
+        return rc;
+    }
+    ReduceArgs a{};
+    for (uint32_t r = 0; r < n; ++r) {
+        a.src[r] = p.ranks[r].send;
+    }
+    a.dst[0] = p.ranks[p.root].recv;
+    a.prog = plan.dev;
+    a.nDst = 1;
+    a.dstOwn = 0;
+    a.nGroup = 1;
+    a.nSub = 1;
+    a.total = a.groupLen = a.subLen = p.count;
+    return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+}
+
+// Broadcast: buf_r = buf_root, one read of the root's buffer and n - 1 writes (reference hccl.h:52-53).
+HcclResult RunBroadcast(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    BcastCopyArgs b{};
+    b.nSeg = 1;
+    b.src[0] = p.ranks[p.root].recv;
+    b.len[0] = p.count * DataTypeSize(p.dtype);
+    b.dstOff[0] = 0;
+    for (uint32_t r = 0; r < n; ++r) {
+        if (r != p.root && p.ranks[r].recv != p.ranks[p.root].recv) {
+            b.dst[b.nDst++] = p.ranks[r].recv;
+        }
+    }
+    if (b.nDst == 0) {
+        return HCCL_SUCCESS;
+    }
+    return RunBcast(w, b, s);
+}
+
+// Scatter: recv_r = send_root[r * recvCount ..] (reference hccl.h:107-109).
+HcclResult RunScatter(World* w, PendingOp& p, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    const uint64_t len = p.count * DataTypeSize(p.dtype);
+    const uint64_t base = reinterpret_cast<uint64_t>(p.ranks[p.root].send);
+    if (base == 0) {
+        return HCCL_E_PTR;
+    }
+    std::vector<CopySeg> segs;
+    for (uint32_t r = 0; r < n; ++r) {
+        segs.push_back({base + r * len, reinterpret_cast<uint64_t>(p.ranks[r].recv), len});
+    }
+    return RunSegmentCopy(w, segs, s);
+}
+
 // rankSize == 1: a plain copy, nothing when in place (reference op_common.cc:4458-4522).
 HcclResult RunSingleRank(World* w, PendingOp& p, hipStream_t s)
 {
@@ -714,11 +856,16 @@ HcclResult RunSingleRank(World* w, PendingOp& p, hipStream_t s)
     const uint64_t esz = DataTypeSize(p.dtype);
     uint64_t len = p.count * esz;
     uint64_t dstOff = 0;
+    if (p.type == OpType::BROADCAST) {
+        return HCCL_SUCCESS;    // the only rank is the root
+    }
     if (p.type == OpType::ALL_GATHER_V) {
         len = r.var[0] * esz;
         dstOff = r.var[1] * esz;
     } else if (p.type == OpType::ALL_TO_ALL_V) {
         len = r.var[0] * esz;   // sendCounts[0], copied from the start of sendBuf to the start of recvBuf
+    } else if (p.type == OpType::REDUCE_SCATTER_V) {
+        len = r.var[0] * esz;   // sendCounts[0], likewise from the start (op_common.cc:4490-4491)
     }
     if (len == 0) {
         return HCCL_SUCCESS;
@@ -768,6 +915,10 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
             case OpType::REDUCE_SCATTER: rc = RunReduceScatter(w, p, s); break;
             case OpType::ALL_GATHER: rc = RunAllGather(w, p, s); break;
             case OpType::ALL_GATHER_V: rc = RunAllGatherV(w, p, s); break;
+            case OpType::REDUCE_SCATTER_V: rc = RunReduceScatterV(w, p, s); break;
+            case OpType::REDUCE: rc = RunReduce(w, p, s); break;
+            case OpType::BROADCAST: rc = RunBroadcast(w, p, s); break;
+            case OpType::SCATTER: rc = RunScatter(w, p, s); break;
             default: rc = RunAlltoAllV(w, p, s); break;
         }
     }
@@ -802,7 +953,7 @@ uint32_t ExecTimeoutSeconds()
 
 // Deposits one rank's arguments; the call that completes the set launches.
 HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count, const void* send,
-                  void* recv, hipStream_t stream, std::vector<uint64_t>&& var)
+                  void* recv, hipStream_t stream, std::vector<uint64_t>&& var, uint32_t root = 0)
 {
     World* w = c->world;
     std::unique_lock<std::mutex> lock(w->mu);
@@ -817,12 +968,13 @@ HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uin
         cell->dtype = dtype;
         cell->op = op;
         cell->count = count;
+        cell->root = root;
         cell->ranks.resize(w->n);
     }
     std::shared_ptr<PendingOp> p = cell;
-    if (p->type != type || p->dtype != dtype || p->op != op || p->count != count) {
-        Log(1, "%s on rank %u does not match the call of the other ranks (%s, count %llu, type %d)", OpName(type),
-            c->rank, OpName(p->type), (unsigned long long)p->count, static_cast<int>(p->dtype));
+    if (p->type != type || p->dtype != dtype || p->op != op || p->count != count || p->root != root) {
+        Log(1, "%s on rank %u does not match the call of the other ranks (%s, count %llu, type %d, root %u)",
+            OpName(type), c->rank, OpName(p->type), (unsigned long long)p->count, static_cast<int>(p->dtype), p->root);
         p->result = HCCL_E_PARA;
     }
     RankArgs& ra = p->ranks[c->rank];
@@ -887,9 +1039,10 @@ namespace {
 
 // A rank whose stream differs from the launcher's must have its position recorded at call time.
 HcclResult SubmitWithReady(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count,
-                           const void* send, void* recv, aclrtStream stream, std::vector<uint64_t>&& var)
+                           const void* send, void* recv, aclrtStream stream, std::vector<uint64_t>&& var,
+                           uint32_t root = 0)
 {
-    return Submit(c, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var));
+    return Submit(c, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var), root);
 }
 
 }  // namespace
@@ -1076,6 +1229,238 @@ HcclResult HcclAlltoAllV(const void* sendBuf, const void* sendCounts, const void
     memcpy(var.data() + 3 * n, rdispls, n * sizeof(uint64_t));
     return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
                            const_cast<void*>(recvBuf), stream, std::move(var));
+}
+
+HcclResult HcclAlltoAll(const void* sendBuf, uint64_t sendCount, HcclDataType sendType, const void* recvBuf,
+                        uint64_t recvCount, HcclDataType recvType, HcclComm comm, aclrtStream stream)
+{
+    // Reference src/ops/all_to_all_v/all_to_all_v.cc:39-82, 475-515.
+    if (sendCount == 0 && recvCount == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendBuf, "sendBuf");
+    CHK_PTR(recvBuf, "recvBuf");
+    if (sendCount != recvCount) {
+        Log(1, "HcclAlltoAll: sendCount %llu and recvCount %llu are not equal", (unsigned long long)sendCount,
+            (unsigned long long)recvCount);
+        return HCCL_E_PARA;
+    }
+    if (sendType != recvType) {
+        Log(1, "HcclAlltoAll: sendType %d and recvType %d are not equal", static_cast<int>(sendType),
+            static_cast<int>(recvType));
+        return HCCL_E_PARA;
+    }
+    CHK_PTR(stream, "stream");
+    if (sendBuf == recvBuf) {
+        Log(1, "HcclAlltoAll: sendBuf and recvBuf cannot be the same");
+        return HCCL_E_PARA;
+    }
+    if (DataTypeSize(sendType) == 0) {
+        Log(1, "HcclAlltoAll: sendType %d is not supported", static_cast<int>(sendType));
+        return HCCL_E_PARA;
+    }
+    if (sendCount > UINT64_MAX / DataTypeSize(sendType)) {
+        Log(1, "HcclAlltoAll: send size overflows");
+        return HCCL_E_PARA;
+    }
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclAlltoAll: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckUserRank(c));
+    CHK_RET(CheckCount(recvCount));
+    CHK_RET(CheckDataType(recvType, false));
+    // Four arrays in AlltoAllV form: counts = recvCount, displacements = i * recvCount (:411-421).
+    const uint32_t n = c->world->n;
+    std::vector<uint64_t> var(4 * n);
+    for (uint32_t i = 0; i < n; ++i) {
+        var[i] = recvCount;
+        var[n + i] = recvCount;
+        var[2 * n + i] = static_cast<uint64_t>(i) * recvCount;
+        var[3 * n + i] = static_cast<uint64_t>(i) * recvCount;
+    }
+    return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
+                           const_cast<void*>(recvBuf), stream, std::move(var));
+}
+
+HcclResult HcclAlltoAllVC(const void* sendBuf, const void* sendCountMatrix, HcclDataType sendType, const void* recvBuf,
+                          HcclDataType recvType, HcclComm comm, aclrtStream stream)
+{
+    // Reference src/ops/all_to_all_v/all_to_all_v.cc:153-209, 423-458, 555-598.  Like the reference, only
+    // recvType is consulted for the element size.
+    (void)sendType;
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendCountMatrix, "sendCountMatrix");
+    CHK_PTR(stream, "stream");
+    if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
+        Log(1, "HcclAlltoAllVC: sendBuf and recvBuf cannot be the same");
+        return HCCL_E_PARA;
+    }
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclAlltoAllVC: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckUserRank(c));
+    const uint32_t n = c->world->n;
+    const uint32_t me = c->rank;
+    const uint64_t* m = static_cast<const uint64_t*>(sendCountMatrix);
+    uint64_t maxCount = 0;
+    for (uint64_t i = 0; i < static_cast<uint64_t>(n) * n; ++i) {
+        maxCount = m[i] > maxCount ? m[i] : maxCount;
+    }
+    CHK_RET(CheckCount(maxCount));
+    // sendCounts = row `me`, recvCounts = column `me`, displacements = exclusive prefix sums (:444-455).
+    std::vector<uint64_t> var(4 * n);
+    uint64_t sOff = 0, rOff = 0;
+    bool sendZero = true, recvZero = true;
+    for (uint32_t i = 0; i < n; ++i) {
+        var[i] = m[static_cast<uint64_t>(me) * n + i];
+        var[n + i] = m[static_cast<uint64_t>(i) * n + me];
+        var[2 * n + i] = sOff;
+        var[3 * n + i] = rOff;
+        sOff += var[i];
+        rOff += var[n + i];
+        sendZero = sendZero && var[i] == 0;
+        recvZero = recvZero && var[n + i] == 0;
+    }
+    if (!sendZero) {
+        CHK_PTR(sendBuf, "sendBuf");
+    }
+    if (!recvZero) {
+        CHK_PTR(recvBuf, "recvBuf");
+    }
+    CHK_RET(CheckDataType(recvType, false));
+    return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
+                           const_cast<void*>(recvBuf), stream, std::move(var));
+}
+
+HcclResult HcclReduceScatterV(void* sendBuf, const void* sendCounts, const void* sendDispls, void* recvBuf,
+                              uint64_t recvCount, HcclDataType dataType, HcclReduceOp op, HcclComm comm,
+                              aclrtStream stream)
+{
+    // Reference src/ops/reduce_scatter_v/reduce_scatter_v.cc:48-79, 180-247.
+    CHK_PTR(stream, "stream");
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendCounts, "sendCounts");
+    CHK_PTR(sendDispls, "sendDispls");
+    if (recvCount > 0) {
+        CHK_PTR(recvBuf, "recvBuf");
+    }
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclReduceScatterV: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    const uint32_t n = c->world->n;
+    const uint64_t* counts = static_cast<const uint64_t*>(sendCounts);
+    const uint64_t* displs = static_cast<const uint64_t*>(sendDispls);
+    bool allZero = true;
+    for (uint32_t i = 0; i < n; ++i) {
+        allZero = allZero && counts[i] == 0;
+    }
+    if (allZero) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(sendBuf, "sendBuf");
+    CHK_RET(CheckUserRank(c));
+    CHK_RET(CheckCount(recvCount));
+    // No uint64 / fp64 here, unlike the other reduce ops (:225-247).
+    if (dataType == HCCL_DATA_TYPE_UINT64 || dataType == HCCL_DATA_TYPE_FP64) {
+        Log(1, "HcclReduceScatterV: data type %d is not supported", static_cast<int>(dataType));
+        return HCCL_E_NOT_SUPPORT;
+    }
+    CHK_RET(CheckDataType(dataType, true));
+    CHK_RET(CheckReduceOp(dataType, op));
+    std::vector<uint64_t> var(2 * n + 1);
+    memcpy(var.data(), counts, n * sizeof(uint64_t));
+    memcpy(var.data() + n, displs, n * sizeof(uint64_t));
+    var[2 * n] = recvCount;
+    // recvCount differs between ranks: 0 is the count the ranks meet on, the per-rank values are checked at launch.
+    return SubmitWithReady(c, OpType::REDUCE_SCATTER_V, dataType, op, 0, sendBuf, recvBuf, stream, std::move(var));
+}
+
+HcclResult HcclReduce(void* sendBuf, void* recvBuf, uint64_t count, HcclDataType dataType, HcclReduceOp op,
+                      uint32_t root, HcclComm comm, aclrtStream stream)
+{
+    // Reference src/ops/reduce/reduce.cc:39, 106-153.
+    if (count == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendBuf, "sendBuf");
+    CHK_PTR(recvBuf, "recvBuf");
+    CHK_PTR(stream, "stream");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclReduce: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckCount(count));
+    CHK_RET(CheckDataType(dataType, true));
+    CHK_RET(CheckReduceOp(dataType, op));
+    if (root >= c->world->n) {
+        Log(1, "HcclReduce: root %u is out of range [0, %u)", root, c->world->n);
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckUserRank(c));
+    return SubmitWithReady(c, OpType::REDUCE, dataType, op, count, sendBuf, recvBuf, stream, {}, root);
+}
+
+HcclResult HcclBroadcast(void* buf, uint64_t count, HcclDataType dataType, uint32_t root, HcclComm comm,
+                         aclrtStream stream)
+{
+    // Reference src/ops/broadcast/broadcast.cc:38, 99-142.
+    if (count == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm, "comm");
+    CHK_PTR(buf, "buf");
+    CHK_PTR(stream, "stream");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclBroadcast: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckUserRank(c));
+    if (root >= c->world->n) {
+        Log(1, "HcclBroadcast: root %u is out of range [0, %u)", root, c->world->n);
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckCount(count));
+    CHK_RET(CheckDataType(dataType, false));
+    return SubmitWithReady(c, OpType::BROADCAST, dataType, HCCL_REDUCE_RESERVED, count, buf, buf, stream, {}, root);
+}
+
+HcclResult HcclScatter(void* sendBuf, void* recvBuf, uint64_t recvCount, HcclDataType dataType, uint32_t root,
+                       HcclComm comm, aclrtStream stream)
+{
+    // Reference src/ops/scatter/scatter.cc:59-73, 115-128.  The reference leaves a null stream to the layers
+    // below the entry point; here it is rejected after the reference's own checks.
+    if (recvCount == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm, "comm");
+    CHK_PTR(recvBuf, "recvBuf");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclScatter: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    if (c->rank == root) {
+        CHK_PTR(sendBuf, "sendBuf");   // only the root's sendBuf is read
+    }
+    if (root >= c->world->n) {
+        Log(1, "HcclScatter: root %u is out of range [0, %u)", root, c->world->n);
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckCount(recvCount));
+    CHK_RET(CheckDataType(dataType, false));
+    CHK_PTR(stream, "stream");
+    return SubmitWithReady(c, OpType::SCATTER, dataType, HCCL_REDUCE_RESERVED, recvCount, sendBuf, recvBuf, stream, {},
+                           root);
 }
 
 // ---- lifecycle -------------------------------------------------------------------------------

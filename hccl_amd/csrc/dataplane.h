@@ -72,6 +72,12 @@ struct ReduceArgs {
     uint32_t blocksPerSub;
     uint32_t vecOk;   // every address the launch touches is 16-byte aligned
     uint32_t threads; // workgroup size of the launch
+    // Groups of unequal length (ReduceScatterV): when varGroups is set, group g spans groupLenV[g]
+    // elements starting groupOffV[g] elements into every source, instead of the uniform
+    // groupLen / srcGroupStride / total geometry; groupLen then only sizes the grid.
+    uint32_t varGroups;
+    uint64_t groupOffV[kMaxRanks];
+    uint64_t groupLenV[kMaxRanks];
 };
 
 // ---- copies -------------------------------------------------------------------------------------

@@ -298,11 +298,19 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     const uint32_t g = sub / args.nSub;
     const uint32_t c = sub - g * args.nSub;
 
-    const uint64_t gBeg = static_cast<uint64_t>(g) * args.groupLen;
-    if (gBeg >= args.total) {
-        return;
+    uint64_t gLen;
+    uint64_t gSrc;
+    if (args.varGroups) {
+        gLen = args.groupLenV[g];
+        gSrc = args.groupOffV[g];
+    } else {
+        const uint64_t gBeg = static_cast<uint64_t>(g) * args.groupLen;
+        if (gBeg >= args.total) {
+            return;
+        }
+        gLen = (args.total - gBeg < args.groupLen) ? args.total - gBeg : args.groupLen;
+        gSrc = static_cast<uint64_t>(g) * args.srcGroupStride;
     }
-    const uint64_t gLen = (args.total - gBeg < args.groupLen) ? args.total - gBeg : args.groupLen;
     const uint64_t sBeg = static_cast<uint64_t>(c) * args.subLen;
     uint64_t sEnd = (c == args.nSub - 1) ? gLen : sBeg + args.subLen;
     sEnd = sEnd < gLen ? sEnd : gLen;
@@ -310,7 +318,7 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
         return;
     }
     const uint64_t len = sEnd - sBeg;
-    const uint64_t srcOff = static_cast<uint64_t>(g) * args.srcGroupStride + sBeg;
+    const uint64_t srcOff = gSrc + sBeg;
     const uint64_t dstOff = args.dstOwn ? sBeg : static_cast<uint64_t>(g) * args.dstGroupStride + sBeg;
 
     // Resolve the program once per block: leaf -> address of this sub-segment in that rank's buffer.
@@ -337,7 +345,8 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     uint64_t head = len;
     uint64_t nVec = 0;
     uint32_t lead = 0;
-    if (args.vecOk) {
+    // A group that starts at an odd offset into the sources is not congruent with its destination.
+    if (args.vecOk && (!args.varGroups || ((gSrc * sizeof(S)) & 15u) == 0)) {
         const uint64_t addr = reinterpret_cast<uint64_t>(args.src[0]) + srcOff * sizeof(S);
         const uint32_t mis = static_cast<uint32_t>(addr & 15u);
         head = mis ? (16u - mis) / sizeof(S) : 0;

@@ -74,8 +74,55 @@ HcclResult HcclAlltoAllV(const void* sendBuf, const void* sendCounts, const void
                          const void* recvBuf, const void* recvCounts, const void* rdispls, HcclDataType recvType,
                          HcclComm comm, aclrtStream stream);
 
+/*
+ * AlltoAllV with sendCounts = recvCounts = recvCount for every peer and displacements i * recvCount:
+ * rank i's recvBuf[j*recvCount + e] = sendBuf_j[i*recvCount + e].  sendCount must equal recvCount and
+ * sendType recvType.  Replaces reference include/hccl.h:234-236 (src/ops/all_to_all_v/all_to_all_v.cc:24).
+ */
+HcclResult HcclAlltoAll(const void* sendBuf, uint64_t sendCount, HcclDataType sendType, const void* recvBuf,
+                        uint64_t recvCount, HcclDataType recvType, HcclComm comm, aclrtStream stream);
+
+/*
+ * AlltoAllV whose arrays every rank derives from one host uint64_t[rankSize * rankSize] matrix, row = sender,
+ * column = receiver: rank r sends row r, receives column r, both packed without gaps.
+ * Replaces reference include/hccl.h:192-194 (src/ops/all_to_all_v/all_to_all_v.cc:153, conversion :423-458).
+ */
+HcclResult HcclAlltoAllVC(const void* sendBuf, const void* sendCountMatrix, HcclDataType sendType, const void* recvBuf,
+                          HcclDataType recvType, HcclComm comm, aclrtStream stream);
+
+/*
+ * Rank k's recvBuf[e] = reduction over ranks t of sendBuf_t[sendDispls[k] + e], e in [0, sendCounts[k]),
+ * folded own rank first, then the others ascending.  sendCounts / sendDispls: host uint64_t[rankSize],
+ * elements, identical on every rank; recvCount must be sendCounts[own rank].  No uint64 / fp64.
+ * Replaces reference include/hccl.h:90-92 (src/ops/reduce_scatter_v/reduce_scatter_v.cc:23).
+ */
+HcclResult HcclReduceScatterV(void* sendBuf, const void* sendCounts, const void* sendDispls, void* recvBuf,
+                              uint64_t recvCount, HcclDataType dataType, HcclReduceOp op, HcclComm comm,
+                              aclrtStream stream);
+
+/*
+ * The root's recvBuf[e] = (((sendBuf_0[e] (+) sendBuf_1[e]) (+) ...) (+) sendBuf_{N-1}[e]); recvBuf of the
+ * other ranks is left alone.  Replaces reference include/hccl.h:253-255 (src/ops/reduce/reduce.cc:23).
+ */
+HcclResult HcclReduce(void* sendBuf, void* recvBuf, uint64_t count, HcclDataType dataType, HcclReduceOp op,
+                      uint32_t root, HcclComm comm, aclrtStream stream);
+
+/*
+ * Every rank's buf = the root's buf.  Replaces reference include/hccl.h:52-53
+ * (src/ops/broadcast/broadcast.cc:23).
+ */
+HcclResult HcclBroadcast(void* buf, uint64_t count, HcclDataType dataType, uint32_t root, HcclComm comm,
+                         aclrtStream stream);
+
+/*
+ * Rank r's recvBuf[e] = the root's sendBuf[r*recvCount + e]; sendBuf of the other ranks is ignored.
+ * Replaces reference include/hccl.h:107-109 (src/ops/scatter/scatter.cc:30).
+ */
+HcclResult HcclScatter(void* sendBuf, void* recvBuf, uint64_t recvCount, HcclDataType dataType, uint32_t root,
+                       HcclComm comm, aclrtStream stream);
+
 /* ------------------------------------------------------------------------------------------
- * Communicator lifecycle.  In the reference these live in the separate HCOMM library and
+ * Communicator lifecycle. In the reference these live in the separate HCOMM library and
  * are only called (examples/02_collectives/01_allreduce/main.cc:76,101,123;
  * docs/en/user_guide/api_comm_impl.md:169-190; src/ops/all_reduce/all_reduce.cc:121-125).
  * ---------------------------------------------------------------------------------------- */

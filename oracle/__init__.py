@@ -260,3 +260,45 @@ def all_to_all_v(ins, outs, send_counts, sdispls, recv_counts, rdispls, dtype):
     rd, rdp = _u64(rdispls)
     return lib().orc_all_to_all_v(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs), scp, sdp, rcp, rdp,
                                   dtype)
+
+
+def all_to_all(ins, outs, count, dtype):
+    return lib().orc_all_to_all(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs), ctypes.c_uint64(count),
+                                dtype)
+
+
+def all_to_all_vc_params(n, rank, matrix):
+    """(sendCounts, recvCounts, sdispls, rdispls) that the reference derives for `rank` from the n x n matrix."""
+    m, mp = _u64(matrix)
+    outs = [np.zeros(max(n, 1), dtype=np.uint64) for _ in range(4)]
+    lib().orc_all_to_all_vc_params(ctypes.c_uint32(n), ctypes.c_uint32(rank), mp,
+                                   *[o.ctypes.data_as(ctypes.POINTER(ctypes.c_uint64)) for o in outs])
+    return tuple(o[:n] for o in outs)
+
+
+def all_to_all_vc(ins, outs, matrix, dtype):
+    m, mp = _u64(matrix)
+    return lib().orc_all_to_all_vc(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs), mp, dtype)
+
+
+def reduce_scatter_v(ins, outs, counts, displs, dtype, op, acc=ACC_FP32):
+    c, cp = _u64(counts)
+    d, dp = _u64(displs)
+    return lib().orc_reduce_scatter_v_mesh(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs), cp, dp,
+                                           dtype, op, acc)
+
+
+def reduce(ins, outs, count, dtype, op, root, acc=ACC_FP32):
+    """Only outs[root] is written."""
+    return lib().orc_reduce_mesh(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs),
+                                 ctypes.c_uint64(count), dtype, op, acc, ctypes.c_uint32(root))
+
+
+def broadcast(bufs, count, dtype, root):
+    return lib().orc_broadcast(ctypes.c_uint32(len(bufs)), _ptr_array(bufs), ctypes.c_uint64(count), dtype,
+                               ctypes.c_uint32(root))
+
+
+def scatter(ins, outs, recv_count, dtype, root):
+    return lib().orc_scatter(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs),
+                             ctypes.c_uint64(recv_count), dtype, ctypes.c_uint32(root))

@@ -1360,6 +1360,161 @@ int orc_all_to_all_v(uint32_t n, const void* const* in, void* const* out, const 
     return ORC_OK;
 }
 
+int orc_all_to_all(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype)
+{
+    uint64_t nn = (uint64_t)n * n;
+    uint64_t* t = (uint64_t*)malloc(sizeof(uint64_t) * nn * 2 + 1);
+    if (!t) {
+        return ORC_E_INTERNAL;
+    }
+    uint64_t* cnt = t;
+    uint64_t* dis = t + nn;
+    for (uint32_t r = 0; r < n; ++r) {
+        uint64_t off = 0;   /* ConvertAlltoAllParam, all_to_all_v.cc:411-421 */
+        for (uint32_t i = 0; i < n; ++i) {
+            cnt[(uint64_t)r * n + i] = count;
+            dis[(uint64_t)r * n + i] = off;
+            off += count;
+        }
+    }
+    int rc = orc_all_to_all_v(n, in, out, cnt, dis, cnt, dis, dtype);
+    free(t);
+    return rc;
+}
+
+void orc_all_to_all_vc_params(uint32_t n, uint32_t rank, const uint64_t* matrix, uint64_t* sendCounts,
+                              uint64_t* recvCounts, uint64_t* sdispls, uint64_t* rdispls)
+{
+    uint64_t off = 0;
+    for (uint32_t i = 0; i < n; ++i) {   /* all_to_all_v.cc:444-448 */
+        sendCounts[i] = matrix[(uint64_t)rank * n + i];
+        sdispls[i] = off;
+        off += sendCounts[i];
+    }
+    off = 0;
+    for (uint32_t i = 0; i < n; ++i) {   /* :450-455 */
+        recvCounts[i] = matrix[(uint64_t)i * n + rank];
+        rdispls[i] = off;
+        off += recvCounts[i];
+    }
+}
+
+int orc_all_to_all_vc(uint32_t n, const void* const* in, void* const* out, const uint64_t* matrix, int dtype)
+{
+    uint64_t nn = (uint64_t)n * n;
+    uint64_t* t = (uint64_t*)malloc(sizeof(uint64_t) * nn * 4 + 1);
+    if (!t) {
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t r = 0; r < n; ++r) {
+        orc_all_to_all_vc_params(n, r, matrix, t + (uint64_t)r * n, t + nn + (uint64_t)r * n,
+                                 t + 2 * nn + (uint64_t)r * n, t + 3 * nn + (uint64_t)r * n);
+    }
+    int rc = orc_all_to_all_v(n, in, out, t, t + 2 * nn, t + nn, t + 3 * nn, dtype);
+    free(t);
+    return rc;
+}
+
+int orc_reduce_scatter_v_mesh(uint32_t n, const void* const* in, void* const* out, const uint64_t* counts,
+                              const uint64_t* displs, int dtype, int op, int accMode)
+{
+    if (dtype == ORC_UINT64 || dtype == ORC_FP64) {
+        return ORC_E_NOT_SUPPORT;   /* reduce_scatter_v.cc:231-236 */
+    }
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    for (uint32_t k = 0; k < n; ++k) {
+        uint64_t count = counts[k];
+        if (count == 0) {
+            continue;
+        }
+        void* acc = malloc(count * r.asz);
+        void* tmp = r.accF32 ? malloc(count * r.asz) : NULL;
+        if (!acc || (r.accF32 && !tmp)) {
+            free(acc);
+            free(tmp);
+            return ORC_E_INTERNAL;
+        }
+        uint64_t base = displs[k] * r.esz;
+        red_widen(&r, cbytes(in[k]) + base, acc, count);          /* own input first (:127-135) */
+        for (uint32_t t = 0; t < n; ++t) {
+            if (t != k) {
+                red_pair_from_storage(&r, acc, cbytes(in[t]) + base, count, tmp);   /* :145-159 */
+            }
+        }
+        red_narrow(&r, acc, out[k], count);
+        free(acc);
+        free(tmp);
+    }
+    return ORC_OK;
+}
+
+int orc_reduce_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                    int accMode, uint32_t root)
+{
+    if (root >= n) {
+        return ORC_E_PARA;
+    }
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (count == 0) {
+        return ORC_OK;
+    }
+    void* acc = malloc(count * r.asz);
+    void* tmp = r.accF32 ? malloc(count * r.asz) : NULL;
+    if (!acc || (r.accF32 && !tmp)) {
+        free(acc);
+        free(tmp);
+        return ORC_E_INTERNAL;
+    }
+    red_widen(&r, in[0], acc, count);                              /* base slot 0 (:268-281) */
+    for (uint32_t idx = 1; idx < n; ++idx) {
+        red_pair_from_storage(&r, acc, in[idx], count, tmp);       /* :295-298 */
+    }
+    red_narrow(&r, acc, out[root], count);
+    free(acc);
+    free(tmp);
+    return ORC_OK;
+}
+
+int orc_broadcast(uint32_t n, void* const* buf, uint64_t count, int dtype, uint32_t root)
+{
+    if (!copy_dtype_ok(dtype)) {
+        return ORC_E_NOT_SUPPORT;
+    }
+    if (root >= n) {
+        return ORC_E_PARA;
+    }
+    size_t esz = orc_dtype_size(dtype);
+    for (uint32_t r = 0; r < n; ++r) {
+        if (r != root) {
+            memcpy(buf[r], buf[root], count * esz);
+        }
+    }
+    return ORC_OK;
+}
+
+int orc_scatter(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype, uint32_t root)
+{
+    if (!copy_dtype_ok(dtype)) {
+        return ORC_E_NOT_SUPPORT;
+    }
+    if (root >= n) {
+        return ORC_E_PARA;
+    }
+    size_t esz = orc_dtype_size(dtype);
+    for (uint32_t r = 0; r < n; ++r) {
+        memcpy(out[r], cbytes(in[root]) + (uint64_t)r * recvCount * esz, recvCount * esz);
+    }
+    return ORC_OK;
+}
+
 /* a5: LocalCopySlices (wrapper.cc:930-997).  Zero-size slices are skipped; a slice whose source and
  * destination both continue the pending run is merged into it; the pending run is issued when the
  * next slice does not continue it or at the last slice. */

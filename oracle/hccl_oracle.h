@@ -144,6 +144,31 @@ int orc_all_gather_v(uint32_t n, const void* const* in, void* const* out, const 
 int orc_all_to_all_v(uint32_t n, const void* const* in, void* const* out, const uint64_t* sendCounts,
                      const uint64_t* sdispls, const uint64_t* recvCounts, const uint64_t* rdispls, int dtype);
 
+/* AlltoAll (all_to_all_v.cc:24-82, 411-421): every rank sends `count` elements to every rank,
+ * sdispls[i] = rdispls[i] = i * count; then orc_all_to_all_v. */
+int orc_all_to_all(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype);
+/* AlltoAllVC parameter conversion for one rank (all_to_all_v.cc:423-458): sendCounts = row `rank` of the
+ * n x n matrix, recvCounts = column `rank`, both displacement arrays = exclusive prefix sums. */
+void orc_all_to_all_vc_params(uint32_t n, uint32_t rank, const uint64_t* matrix, uint64_t* sendCounts,
+                              uint64_t* recvCounts, uint64_t* sdispls, uint64_t* rdispls);
+/* AlltoAllVC (all_to_all_v.cc:153-209): convert per rank, then orc_all_to_all_v. */
+int orc_all_to_all_vc(uint32_t n, const void* const* in, void* const* out, const uint64_t* matrix, int dtype);
+
+/* ReduceScatterV mesh (ins_temp_reduce_scatter_v_mesh_1D.cc:109-162, executor :117-215): counts / displs
+ * are the (identical) per-rank arrays; rank k: out = in_k[displs[k] .. +counts[k]); for t = 0..N-1, t != k:
+ * out = in_t[displs[k] ..] (+) out.  Types as the entry point admits (reduce_scatter_v.cc:225-247: no
+ * uint64 / fp64). */
+int orc_reduce_scatter_v_mesh(uint32_t n, const void* const* in, void* const* out, const uint64_t* counts,
+                              const uint64_t* displs, int dtype, int op, int accMode);
+/* Reduce mesh (reduce_mesh_1D.cc:268-300): slot r = rank r's input; out_root = slot 0, then
+ * out_root = slot_idx (+) out_root for idx = 1..N-1.  Only out[root] is written. */
+int orc_reduce_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                    int accMode, uint32_t root);
+/* Broadcast (hccl.h:52-53): buf_r = buf_root for every r. */
+int orc_broadcast(uint32_t n, void* const* buf, uint64_t count, int dtype, uint32_t root);
+/* Scatter (hccl.h:107-109): out_r = in_root[r * recvCount .. +recvCount). */
+int orc_scatter(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype, uint32_t root);
+
 /* a5: LocalCopySlices merge rule (wrapper.cc:930-997): returns how many copies are issued
  * for slices (offset,size) over one base address; copies[] gets (srcOff,dstOff,size) triples. */
 uint32_t orc_local_copy_slices(uint32_t nSlices, const uint64_t* srcOff, const uint64_t* dstOff,

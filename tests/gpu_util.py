@@ -103,6 +103,50 @@ class World:
                                       recv_counts[r], rdispls[r], dtype, self.stream)
         self.sync()
 
+    def all_to_all(self, sends, recvs, count, dtype):
+        self.inputs_ready()
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.all_to_all(self.comms[r], sends[r], count, dtype, recvs[r], count, dtype, self.stream)
+        self.sync()
+
+    def all_to_all_vc(self, sends, recvs, matrix, dtype):
+        self.inputs_ready()
+        flat = hccl_amd.u64_array(np.asarray(matrix).reshape(-1))
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.all_to_all_vc(self.comms[r], sends[r], flat, dtype, recvs[r], dtype, self.stream)
+        self.sync()
+
+    def reduce_scatter_v(self, sends, recvs, counts, displs, dtype, op):
+        self.inputs_ready()
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.reduce_scatter_v(self.comms[r], sends[r], counts, displs, recvs[r], int(counts[r]), dtype, op,
+                                          self.stream)
+        self.sync()
+
+    def reduce(self, sends, recvs, count, dtype, op, root):
+        self.inputs_ready()
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.reduce(self.comms[r], sends[r], recvs[r], count, dtype, op, root, self.stream)
+        self.sync()
+
+    def broadcast(self, bufs, count, dtype, root):
+        self.inputs_ready()
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.broadcast(self.comms[r], bufs[r], count, dtype, root, self.stream)
+        self.sync()
+
+    def scatter(self, sends, recvs, recv_count, dtype, root):
+        self.inputs_ready()
+        with hccl_amd.group():
+            for r in range(self.n):
+                hccl_amd.scatter(self.comms[r], sends[r], recvs[r], recv_count, dtype, root, self.stream)
+        self.sync()
+
 
 def same_bits_nan_class(got, want, float_view=None):
     """Bit equality; where float_view is given, positions that are NaN on both sides only need to be NaN."""

@@ -20,7 +20,8 @@ SUM, PROD, MAX, MIN = range(4)
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "hccl.h")).read()
     names = set(re.findall(r"\b(Hccl[A-Za-z0-9]+)\s*\(", header))
-    assert {"HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV"} <= names
+    assert {"HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV", "HcclAlltoAll",
+            "HcclAlltoAllVC", "HcclReduceScatterV", "HcclReduce", "HcclBroadcast", "HcclScatter"} <= names
     L = ctypes.CDLL(hccl_amd.LIB_PATH)
     for n in sorted(names):
         assert hasattr(L, n), n
@@ -169,7 +170,6 @@ def test_known_programs():
     # p = 6: ((x0+x2)+x4) + ((x1+x3)+x5) for the share of rank 0
     p6 = hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.RHD, 6)
     assert p6[0] == bytes([0xC3, 0, 2, 4, 0x80, 0xC3, 1, 3, 5, 0x81, 0xFF])
-    assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.AIV_MESH, 4) if False else True
 
 
 # ---- argument validation (returns before any GPU work) ------------------------------------------------
@@ -251,6 +251,69 @@ def test_other_entry_argument_checks(world):
     assert code_of(hccl_amd.all_to_all_v, c, a, cnt, dsp, DT.FP16, None, cnt, dsp, DT.FP16, s) == 2
     assert code_of(hccl_amd.all_to_all_v, c, a, cnt, dsp, DT.FP16, b, cnt, dsp, DT.INT128, s) == 5
     assert code_of(hccl_amd.all_to_all_v, c, a, [2 ** 40, 0, 0, 0], dsp, DT.FP16, b, cnt, dsp, DT.FP16, s) == 1
+
+
+def test_rooted_and_v_entry_argument_checks(world):
+    c, s, a, b = world[1], 0x1000, 0x2000, 0x3000
+    cnt, dsp, z = [4, 4, 4, 4], [0, 4, 8, 12], [0, 0, 0, 0]
+    # AlltoAll (reference all_to_all_v.cc:39-41, 475-515)
+    assert hccl_amd.all_to_all(c, None, 0, DT.FP16, None, 0, DT.FP16, None) == 0          # both counts 0 wins
+    assert code_of(hccl_amd.all_to_all, None, a, 4, DT.FP16, b, 4, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_to_all, c, None, 4, DT.FP16, b, 4, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_to_all, c, a, 4, DT.FP16, None, 4, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_to_all, c, a, 4, DT.FP16, b, 5, DT.FP16, s) == 1          # counts differ
+    assert code_of(hccl_amd.all_to_all, c, a, 4, DT.FP16, b, 4, DT.FP32, s) == 1          # types differ
+    assert code_of(hccl_amd.all_to_all, c, a, 4, DT.FP16, b, 4, DT.FP16, None) == 2
+    assert code_of(hccl_amd.all_to_all, c, a, 4, DT.FP16, a, 4, DT.FP16, s) == 1          # in place
+    assert code_of(hccl_amd.all_to_all, c, a, 4, 99, b, 4, 99, s) == 1                    # unknown type: E_PARA here
+    assert code_of(hccl_amd.all_to_all, c, a, 2 ** 40, DT.FP16, b, 2 ** 40, DT.FP16, s) == 1
+    assert code_of(hccl_amd.all_to_all, c, a, 4, DT.INT128, b, 4, DT.INT128, s) == 5
+    # AlltoAllVC (:153-209, 555-598)
+    m = [1] * 16
+    assert code_of(hccl_amd.all_to_all_vc, None, a, m, DT.FP16, b, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_to_all_vc, c, a, m, DT.FP16, b, DT.FP16, None) == 2
+    assert code_of(hccl_amd.all_to_all_vc, c, a, m, DT.FP16, a, DT.FP16, s) == 1          # in place
+    assert code_of(hccl_amd.all_to_all_vc, c, a, [2 ** 40] + [1] * 15, DT.FP16, b, DT.FP16, s) == 1
+    assert code_of(hccl_amd.all_to_all_vc, c, None, m, DT.FP16, b, DT.FP16, s) == 2       # row 1 is not all zero
+    assert code_of(hccl_amd.all_to_all_vc, c, a, m, DT.FP16, None, DT.FP16, s) == 2
+    assert code_of(hccl_amd.all_to_all_vc, c, a, m, DT.FP16, b, DT.INT128, s) == 5
+    # ReduceScatterV (reduce_scatter_v.cc:48-79, 180-247)
+    assert code_of(hccl_amd.reduce_scatter_v, c, a, cnt, dsp, b, 4, DT.FP16, OP.SUM, None) == 2
+    assert code_of(hccl_amd.reduce_scatter_v, None, a, cnt, dsp, b, 4, DT.FP16, OP.SUM, s) == 2
+    assert code_of(hccl_amd.reduce_scatter_v, c, a, cnt, dsp, None, 4, DT.FP16, OP.SUM, s) == 2
+    assert hccl_amd.reduce_scatter_v(c, None, z, dsp, None, 0, DT.FP16, OP.SUM, s) == 0   # all-zero counts: no-op
+    assert code_of(hccl_amd.reduce_scatter_v, c, None, cnt, dsp, b, 4, DT.FP16, OP.SUM, s) == 2
+    assert code_of(hccl_amd.reduce_scatter_v, c, a, cnt, dsp, b, 2 ** 40, DT.FP16, OP.SUM, s) == 1
+    for bad in (DT.UINT64, DT.FP64, DT.UINT8, DT.INT128, DT.HIF8):
+        assert code_of(hccl_amd.reduce_scatter_v, c, a, cnt, dsp, b, 4, bad, OP.SUM, s) == 5
+    assert code_of(hccl_amd.reduce_scatter_v, c, a, cnt, dsp, b, 4, DT.BFP16, OP.PROD, s) == 5
+    # Reduce (reduce.cc:39, 106-153)
+    assert hccl_amd.reduce(c, None, None, 0, DT.FP32, OP.SUM, 9, None) == 0
+    assert code_of(hccl_amd.reduce, None, a, b, 4, DT.FP32, OP.SUM, 0, s) == 2
+    assert code_of(hccl_amd.reduce, c, None, b, 4, DT.FP32, OP.SUM, 0, s) == 2
+    assert code_of(hccl_amd.reduce, c, a, None, 4, DT.FP32, OP.SUM, 0, s) == 2
+    assert code_of(hccl_amd.reduce, c, a, b, 4, DT.FP32, OP.SUM, 0, None) == 2
+    assert code_of(hccl_amd.reduce, c, a, b, 2 ** 40, DT.FP32, OP.SUM, 0, s) == 1
+    assert code_of(hccl_amd.reduce, c, a, b, 4, DT.UINT32, OP.SUM, 0, s) == 5
+    assert code_of(hccl_amd.reduce, c, a, b, 4, DT.INT16, OP.PROD, 0, s) == 5
+    assert code_of(hccl_amd.reduce, c, a, b, 4, DT.FP32, OP.SUM, 4, s) == 1               # root outside the world
+    # Broadcast (broadcast.cc:38, 99-142)
+    assert hccl_amd.broadcast(c, None, 0, DT.FP32, 9, None) == 0
+    assert code_of(hccl_amd.broadcast, None, a, 4, DT.FP32, 0, s) == 2
+    assert code_of(hccl_amd.broadcast, c, None, 4, DT.FP32, 0, s) == 2
+    assert code_of(hccl_amd.broadcast, c, a, 4, DT.FP32, 0, None) == 2
+    assert code_of(hccl_amd.broadcast, c, a, 4, DT.FP32, 4, s) == 1
+    assert code_of(hccl_amd.broadcast, c, a, 2 ** 40, DT.FP32, 0, s) == 1
+    assert code_of(hccl_amd.broadcast, c, a, 4, DT.INT128, 0, s) == 5
+    # Scatter (scatter.cc:59-73)
+    assert hccl_amd.scatter(c, None, None, 0, DT.FP32, 9, None) == 0
+    assert code_of(hccl_amd.scatter, None, a, b, 4, DT.FP32, 0, s) == 2
+    assert code_of(hccl_amd.scatter, c, a, None, 4, DT.FP32, 0, s) == 2
+    assert code_of(hccl_amd.scatter, c, None, b, 4, DT.FP32, 1, s) == 2                   # this rank is the root
+    assert code_of(hccl_amd.scatter, c, a, b, 4, DT.FP32, 4, s) == 1
+    assert code_of(hccl_amd.scatter, c, a, b, 2 ** 40, DT.FP32, 0, s) == 1
+    assert code_of(hccl_amd.scatter, c, a, b, 4, DT.INT128, 0, s) == 5
+    assert code_of(hccl_amd.scatter, c, a, b, 4, DT.FP32, 0, None) == 2
 
 
 def test_group_end_without_start():
