@@ -29,7 +29,8 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3max", "c3prod", "c4", "c5a", "c5b", "copycal"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3max", "c3prod", "c4", "c5a", "c5b", "copycal", "rsv", "reduce", "bcast", "scatter",
+                             "a2a"])
     ap.add_argument("--algo", default=None, help="override the algorithm of the workload (mesh/ring/rhd/nhr/...)")
     ap.add_argument("--others", action="store_true", help="also time the other BASELINE configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -153,6 +154,99 @@ class Workloads:
             h.all_gather(comms[0], src, dst, nbytes, h.HcclDataType.UINT8, stream)
 
         return step, 2 * nbytes, nbytes, 1.0, (src, dst), "plain copy 1 GiB (rankSize=1 AllGather)", "u8", 1
+
+    # ---- the entry points that marshal onto the same kernels (not BASELINE configurations) ----------
+    def rsv(self, algo):
+        """ReduceScatterV bf16, 8 ranks, uneven slices between 8 Mi and 24 Mi elements (16-byte aligned starts)."""
+        import numpy as np
+        t, h = self.torch, self.h
+        n = 8
+        comms = self.world(n)
+        rng = np.random.default_rng(0xC0FFEE + 6000)
+        counts = (rng.integers(1 << 20, 3 << 20, n) * 8).astype(np.uint64)
+        displs = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.uint64)
+        total = int(counts.sum())
+        sends = [t.randn(total, generator=self.gen(0xC0FFEE + 6100 + r), device="cuda", dtype=t.bfloat16)
+                 for r in range(n)]
+        recvs = [t.empty(int(c), dtype=t.bfloat16, device="cuda") for c in counts]
+        stream = self.stream
+        cu, du = h.u64_array(counts), h.u64_array(displs)
+
+        def step():
+            with h.group():
+                for r in range(n):
+                    h.reduce_scatter_v(comms[r], sends[r], cu, du, recvs[r], int(counts[r]), h.HcclDataType.BFP16,
+                                       h.HcclReduceOp.SUM, stream)
+
+        return step, (n + 1) * total * 2, total * 2, (n - 1) / n, (sends, recvs), \
+            "ReduceScatterV SUM bf16 rankSize=8 slices U[8Mi,24Mi]", "bf16", n
+
+    def reduce(self, algo):
+        t, h = self.torch, self.h
+        n, count, root = 8, 1 << 26, 3
+        comms = self.world(n)
+        sends = [t.randn(count, generator=self.gen(0xC0FFEE + 6200 + r), device="cuda", dtype=t.float32)
+                 for r in range(n)]
+        recv = t.empty(count, dtype=t.float32, device="cuda")
+        stream = self.stream
+
+        def step():
+            with h.group():
+                for r in range(n):
+                    h.reduce(comms[r], sends[r], recv, count, h.HcclDataType.FP32, h.HcclReduceOp.SUM, root, stream)
+
+        return step, (n + 1) * count * 4, count * 4, 1.0, (sends, recv), \
+            "Reduce SUM fp32 rankSize=8 64Mi el/rank", "f32", n
+
+    def bcast(self, algo):
+        t, h = self.torch, self.h
+        n, count, root = 8, 1 << 27, 5
+        comms = self.world(n)
+        bufs = [t.randint(0, 255, (count,), generator=self.gen(0xC0FFEE + 6300 + r), device="cuda", dtype=t.uint8)
+                for r in range(n)]
+        stream = self.stream
+
+        def step():
+            with h.group():
+                for r in range(n):
+                    h.broadcast(comms[r], bufs[r], count, h.HcclDataType.UINT8, root, stream)
+
+        return step, n * count, count, 1.0, bufs, "Broadcast rankSize=8 128 MiB", "u8", n
+
+    def scatter(self, algo):
+        t, h = self.torch, self.h
+        n, count, root = 8, 1 << 27, 2
+        comms = self.world(n)
+        send = t.randint(0, 255, (n * count,), generator=self.gen(0xC0FFEE + 6400), device="cuda", dtype=t.uint8)
+        recvs = [t.empty(count, dtype=t.uint8, device="cuda") for _ in range(n)]
+        stream = self.stream
+
+        def step():
+            with h.group():
+                for r in range(n):
+                    h.scatter(comms[r], send if r == root else None, recvs[r], count, h.HcclDataType.UINT8, root,
+                              stream)
+
+        return step, 2 * n * count, n * count, (n - 1) / n, (send, recvs), "Scatter rankSize=8 128 MiB per rank", "u8", n
+
+    def a2a(self, algo):
+        t, h = self.torch, self.h
+        n, count = 16, 1 << 22
+        comms = self.world(n)
+        sends = [t.randint(-32768, 32767, (n * count,), generator=self.gen(0xC0FFEE + 6500 + r), device="cuda",
+                           dtype=t.int16) for r in range(n)]
+        recvs = [t.empty(n * count, dtype=t.int16, device="cuda") for _ in range(n)]
+        stream = self.stream
+
+        def step():
+            with h.group():
+                for r in range(n):
+                    h.all_to_all(comms[r], sends[r], count, h.HcclDataType.BFP16, recvs[r], count,
+                                 h.HcclDataType.BFP16, stream)
+
+        total = n * n * count * 2
+        return step, 2 * total, total // n, (n - 1) / n, (sends, recvs), \
+            "AlltoAll bf16 rankSize=16 4Mi el per pair", "u8", n
 
     def c4(self, algo):
         import numpy as np
@@ -285,6 +379,9 @@ def main():
                 others[name] = measure(torch, wl, name, None, max(3, args.steps // 2), 2)
         if args.workload == "c2":
             others["c2_mesh_order"] = measure(torch, wl, "c2", "mesh", args.steps, 2)
+        for name in ("rsv", "reduce", "bcast", "scatter", "a2a"):
+            if name != args.workload:
+                others[name] = measure(torch, wl, name, None, max(3, args.steps // 2), 2)
 
     cpu = None
     if not args.no_cpu:
@@ -301,7 +398,8 @@ def main():
                    "rank_size": main_res["n_ranks"], "algbw_GBs": main_res["algbw_GBs"],
                    "hbm_percent_of_peak": round(100 * main_res["hbm_frac"], 2)},
         "roofline": {"bound": "hbm", "achieved": round(hbm / t / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(hbm / t / 1e9 / HBM_PEAK_GBS, 4), "traffic": traffic_from_profiles(),
+                     "frac": round(hbm / t / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": traffic_from_profiles() if args.workload == "c2" else None,
                      "algorithmic_bytes_per_launch": hbm, "kernel_ms": main_res["ms_per_step"]},
         "cpu_baseline": cpu,
     }
