@@ -136,16 +136,21 @@ struct alignas(sizeof(S) * W >= 16 ? 16 : sizeof(S) * W) Pack {
     S e[W];
 };
 
+// Every buffer the kernel touches is global memory.  Saying so keeps the accesses off the flat path:
+// a flat load also counts as an LDS operation, and waiting for the next LDS read (a leaf pointer)
+// would then wait for every load issued before it.
+#define HCCL_AMD_GLOBAL __attribute__((address_space(1)))
+
 template <typename S, int W>
 __device__ __forceinline__ Pack<S, W> LoadPack(const void* base, uint64_t elemOff)
 {
     const S* p = static_cast<const S*>(base) + elemOff;
     if constexpr (sizeof(S) * W == 16) {
-        U32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(p));
+        U32x4 raw = __builtin_nontemporal_load((const HCCL_AMD_GLOBAL U32x4*)p);
         return __builtin_bit_cast(Pack<S, W>, raw);
     } else {
         Pack<S, W> r;
-        r.e[0] = __builtin_nontemporal_load(p);
+        r.e[0] = __builtin_nontemporal_load((const HCCL_AMD_GLOBAL S*)p);
         return r;
     }
 }
@@ -155,9 +160,9 @@ __device__ __forceinline__ void StorePack(void* base, uint64_t elemOff, const Pa
 {
     S* p = static_cast<S*>(base) + elemOff;
     if constexpr (sizeof(S) * W == 16) {
-        __builtin_nontemporal_store(__builtin_bit_cast(U32x4, v), reinterpret_cast<U32x4*>(p));
+        __builtin_nontemporal_store(__builtin_bit_cast(U32x4, v), (HCCL_AMD_GLOBAL U32x4*)p);
     } else {
-        __builtin_nontemporal_store(v.e[0], p);
+        __builtin_nontemporal_store(v.e[0], (HCCL_AMD_GLOBAL S*)p);
     }
 }
 
@@ -236,6 +241,24 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
                 const void* base = reinterpret_cast<const void*>(Uniform64(bp.leafPtr[b + i]));
                 v[i] = LoadPack<S, W>(base, e);
             }
+        }
+        if constexpr (sizeof(S) * W == 16) {
+            // Nothing may consume a loaded vector before the whole batch has been issued: without this the
+            // compiler sinks the first unpacking instruction of each operand next to its load and waits there.
+            static_assert(kMaxRun == 8, "the fence lists eight operands");
+            U32x4 r0 = __builtin_bit_cast(U32x4, v[0]), r1 = __builtin_bit_cast(U32x4, v[1]);
+            U32x4 r2 = __builtin_bit_cast(U32x4, v[2]), r3 = __builtin_bit_cast(U32x4, v[3]);
+            U32x4 r4 = __builtin_bit_cast(U32x4, v[4]), r5 = __builtin_bit_cast(U32x4, v[5]);
+            U32x4 r6 = __builtin_bit_cast(U32x4, v[6]), r7 = __builtin_bit_cast(U32x4, v[7]);
+            asm volatile("" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3), "+v"(r4), "+v"(r5), "+v"(r6), "+v"(r7));
+            v[0] = __builtin_bit_cast(Pack<S, W>, r0);
+            v[1] = __builtin_bit_cast(Pack<S, W>, r1);
+            v[2] = __builtin_bit_cast(Pack<S, W>, r2);
+            v[3] = __builtin_bit_cast(Pack<S, W>, r3);
+            v[4] = __builtin_bit_cast(Pack<S, W>, r4);
+            v[5] = __builtin_bit_cast(Pack<S, W>, r5);
+            v[6] = __builtin_bit_cast(Pack<S, W>, r6);
+            v[7] = __builtin_bit_cast(Pack<S, W>, r7);
         }
 #pragma unroll
         for (int i = 0; i < kMaxRun; ++i) {
