@@ -222,8 +222,35 @@ struct BlockProgram {
     uint32_t nLeaves;
 };
 
+// Leaves whose loads are issued together: sixteen for 4- and 8-byte elements, eight for the narrower ones
+// (their unpacked accumulators need the registers).
+template <typename S, int W>
+__device__ constexpr int LoadBatch()
+{
+    return (sizeof(S) >= 4 && W > 1) ? 16 : 8;
+}
+
+// Makes eight loaded vectors opaque to the optimiser at this point of the instruction stream.
+template <typename S, int W>
+__device__ __forceinline__ void IssueFence8(Pack<S, W>* v)
+{
+    U32x4 r0 = __builtin_bit_cast(U32x4, v[0]), r1 = __builtin_bit_cast(U32x4, v[1]);
+    U32x4 r2 = __builtin_bit_cast(U32x4, v[2]), r3 = __builtin_bit_cast(U32x4, v[3]);
+    U32x4 r4 = __builtin_bit_cast(U32x4, v[4]), r5 = __builtin_bit_cast(U32x4, v[5]);
+    U32x4 r6 = __builtin_bit_cast(U32x4, v[6]), r7 = __builtin_bit_cast(U32x4, v[7]);
+    asm volatile("" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3), "+v"(r4), "+v"(r5), "+v"(r6), "+v"(r7));
+    v[0] = __builtin_bit_cast(Pack<S, W>, r0);
+    v[1] = __builtin_bit_cast(Pack<S, W>, r1);
+    v[2] = __builtin_bit_cast(Pack<S, W>, r2);
+    v[3] = __builtin_bit_cast(Pack<S, W>, r3);
+    v[4] = __builtin_bit_cast(Pack<S, W>, r4);
+    v[5] = __builtin_bit_cast(Pack<S, W>, r5);
+    v[6] = __builtin_bit_cast(Pack<S, W>, r6);
+    v[7] = __builtin_bit_cast(Pack<S, W>, r7);
+}
+
 // Evaluates the whole tree for the W elements at element offset `e` of the sub-segment.  Leaves are
-// taken eight at a time: their loads are all issued before the first fold, whatever the tree shape.
+// taken a batch at a time: their loads are all issued before the first fold, whatever the tree shape.
 template <class E, int W>
 __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stack, const ReduceArgs& args,
                                           uint64_t e, uint64_t dstOff, uint32_t group)
@@ -233,10 +260,11 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
     uint32_t level = 0;
     bool init = true;   // the next leaf starts a level instead of being folded into it
     const uint32_t nLeaves = bp.nLeaves;
-    for (uint32_t b = 0; b < nLeaves; b += kMaxRun) {
-        Pack<S, W> v[kMaxRun];
+    constexpr int kBatch = LoadBatch<S, W>();
+    for (uint32_t b = 0; b < nLeaves; b += kBatch) {
+        Pack<S, W> v[kBatch];
 #pragma unroll
-        for (int i = 0; i < kMaxRun; ++i) {
+        for (int i = 0; i < kBatch; ++i) {
             if (b + i < nLeaves) {
                 const void* base = reinterpret_cast<const void*>(Uniform64(bp.leafPtr[b + i]));
                 v[i] = LoadPack<S, W>(base, e);
@@ -245,23 +273,13 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
         if constexpr (sizeof(S) * W == 16) {
             // Nothing may consume a loaded vector before the whole batch has been issued: without this the
             // compiler sinks the first unpacking instruction of each operand next to its load and waits there.
-            static_assert(kMaxRun == 8, "the fence lists eight operands");
-            U32x4 r0 = __builtin_bit_cast(U32x4, v[0]), r1 = __builtin_bit_cast(U32x4, v[1]);
-            U32x4 r2 = __builtin_bit_cast(U32x4, v[2]), r3 = __builtin_bit_cast(U32x4, v[3]);
-            U32x4 r4 = __builtin_bit_cast(U32x4, v[4]), r5 = __builtin_bit_cast(U32x4, v[5]);
-            U32x4 r6 = __builtin_bit_cast(U32x4, v[6]), r7 = __builtin_bit_cast(U32x4, v[7]);
-            asm volatile("" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3), "+v"(r4), "+v"(r5), "+v"(r6), "+v"(r7));
-            v[0] = __builtin_bit_cast(Pack<S, W>, r0);
-            v[1] = __builtin_bit_cast(Pack<S, W>, r1);
-            v[2] = __builtin_bit_cast(Pack<S, W>, r2);
-            v[3] = __builtin_bit_cast(Pack<S, W>, r3);
-            v[4] = __builtin_bit_cast(Pack<S, W>, r4);
-            v[5] = __builtin_bit_cast(Pack<S, W>, r5);
-            v[6] = __builtin_bit_cast(Pack<S, W>, r6);
-            v[7] = __builtin_bit_cast(Pack<S, W>, r7);
+#pragma unroll
+            for (int i = 0; i < kBatch; i += 8) {
+                IssueFence8<S, W>(v + i);
+            }
         }
 #pragma unroll
-        for (int i = 0; i < kMaxRun; ++i) {
+        for (int i = 0; i < kBatch; ++i) {
             if (b + i < nLeaves) {
                 const uint32_t ctl = Uniform(bp.ctl[b + i]);
                 if (ctl & kCtlOpen) {
