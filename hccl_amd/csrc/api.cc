@@ -6,6 +6,7 @@
 // a rendezvous of the N per-rank calls, and one fused kernel launch per collective.
 #include <hip/hip_runtime.h>
 
+#include <cctype>
 #include <chrono>
 #include <condition_variable>
 #include <cstdarg>
@@ -227,6 +228,8 @@ struct World {
     uint32_t reduceBlocks = 1u << 20;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
+    // HCCL_DETERMINISTIC (reference alg_env_config.cc:1113-1153): 0 false, 1 true, 2 strict, 0xFF unparsable
+    uint8_t deterministic = 0;
 
     ~World()
     {
@@ -319,6 +322,14 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->copyTileBytes = 0;
     }
     ApplyAlgoEnv(w.get());
+    if (const char* det = getenv("HCCL_DETERMINISTIC")) {
+        std::string v(det);
+        for (char& ch : v) ch = static_cast<char>(toupper(static_cast<unsigned char>(ch)));
+        w->deterministic = v == "STRICT" ? 2 : v == "TRUE" ? 1 : v == "FALSE" ? 0 : 0xFF;
+        if (w->deterministic == 0xFF) {
+            Log(1, "HCCL_DETERMINISTIC is set to [%s], which is incorrect (true, false or strict)", det);
+        }
+    }
     return w;
 }
 
@@ -486,10 +497,22 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     return HCCL_SUCCESS;
 }
 
+// HCCL_DETERMINISTIC=strict moves float SUM / PROD over more than two ranks to the order-preserved fold
+// (reference src/common/order_preserved_common.h:104-114); everything else keeps the configured algorithm.
+HcclAmdAlgo EffectiveAlgo(const World* w, HcclAmdOpKind kind, HcclDataType dtype, HcclReduceOp op)
+{
+    const bool isFloat = dtype == HCCL_DATA_TYPE_FP16 || dtype == HCCL_DATA_TYPE_FP32 ||
+                         dtype == HCCL_DATA_TYPE_BFP16 || dtype == HCCL_DATA_TYPE_FP64;
+    if (w->deterministic == 2 && isFloat && (op == HCCL_REDUCE_SUM || op == HCCL_REDUCE_PROD) && w->n > 2) {
+        return HCCL_AMD_ALGO_ORDER_PRESERVED;
+    }
+    return w->algo[kind];
+}
+
 HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
-    HcclAmdAlgo algo = w->algo[HCCL_AMD_OP_ALL_REDUCE];
+    HcclAmdAlgo algo = EffectiveAlgo(w, HCCL_AMD_OP_ALL_REDUCE, p.dtype, p.op);
     DevicePlan plan;
     HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_ALL_REDUCE, algo, &plan);
     if (rc != HCCL_SUCCESS) {
@@ -545,7 +568,7 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
 HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
-    HcclAmdAlgo algo = w->algo[HCCL_AMD_OP_REDUCE_SCATTER];
+    HcclAmdAlgo algo = EffectiveAlgo(w, HCCL_AMD_OP_REDUCE_SCATTER, p.dtype, p.op);
     DevicePlan plan;
     HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, algo, &plan);
     if (rc != HCCL_SUCCESS) {
@@ -1042,6 +1065,9 @@ HcclResult SubmitWithReady(Comm* c, OpType type, HcclDataType dtype, HcclReduceO
                            const void* send, void* recv, aclrtStream stream, std::vector<uint64_t>&& var,
                            uint32_t root = 0)
 {
+    if (c->world->deterministic == 0xFF) {
+        return HCCL_E_PARA;   // the reference's environment parsing fails every entry point the same way
+    }
     return Submit(c, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var), root);
 }
 

@@ -265,3 +265,43 @@ def test_config5a_all_reduce_fp16_rhd_n6():
             assert np.array_equal(to_host(recvs[r], np.uint16), want)
     finally:
         w.close()
+
+
+def test_hccl_deterministic_strict_selects_the_order_preserved_fold(monkeypatch):
+    """reference order_preserved_common.h:104-114: strict + float + SUM/PROD + more than two ranks."""
+    import hccl_amd
+    monkeypatch.setenv("HCCL_DETERMINISTIC", "Strict")
+    n, count = 6, 4099
+    w = World(n)                                     # the variable is read when the world is created
+    monkeypatch.delenv("HCCL_DETERMINISTIC")
+    try:
+        rng = np.random.default_rng(77)
+        ins = [gen(DT.FP32, SUM, rng, count) for _ in range(n)]
+        strict = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+        plain = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+        assert oracle.all_reduce(ins, strict, count, int(DT.FP32), SUM, algo="order_preserved") == 0
+        assert oracle.all_reduce(ins, plain, count, int(DT.FP32), SUM, algo="mesh") == 0
+        assert not np.array_equal(strict[0].view(np.uint32), plain[0].view(np.uint32))   # the orders are told apart
+        sends = [to_dev(x) for x in ins]
+        recvs = [dev_zeros(x.nbytes) for x in ins]
+        w.all_reduce(sends, recvs, count, DT.FP32, SUM, "mesh")                  # configured: mesh; strict wins
+        check(DT.FP32, SUM, to_host(recvs[2], np.float32), strict[2], "strict all_reduce")
+        # MAX is not covered by the rule: the configured order applies
+        ins = [gen(DT.FP32, MAX, rng, count) for _ in range(n)]
+        want = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+        assert oracle.all_reduce(ins, want, count, int(DT.FP32), MAX, algo="mesh") == 0
+        sends = [to_dev(x) for x in ins]
+        w.all_reduce(sends, recvs, count, DT.FP32, MAX, "mesh")
+        check(DT.FP32, MAX, to_host(recvs[4], np.float32), want[4], "strict all_reduce MAX")
+        # ReduceScatter follows the same rule
+        c = 1031
+        ins = [gen(DT.FP32, SUM, rng, n * c) for _ in range(n)]
+        want = [np.zeros(c, dtype=np.float32) for _ in range(n)]
+        assert oracle.reduce_scatter(ins, want, c, int(DT.FP32), SUM, algo="order_preserved") == 0
+        sends = [to_dev(x) for x in ins]
+        recvs = [dev_zeros(4 * c) for _ in range(n)]
+        w.reduce_scatter(sends, recvs, c, DT.FP32, SUM, "mesh")
+        for r in range(n):
+            check(DT.FP32, SUM, to_host(recvs[r], np.float32), want[r], "strict reduce_scatter rank %d" % r)
+    finally:
+        w.close()

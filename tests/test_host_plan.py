@@ -316,5 +316,17 @@ def test_rooted_and_v_entry_argument_checks(world):
     assert code_of(hccl_amd.scatter, c, a, b, 4, DT.FP32, 0, None) == 2
 
 
+def test_unparsable_hccl_deterministic_fails_every_collective(monkeypatch):
+    # reference alg_env_config.cc:1113-1125: anything but true / false / strict is HCCL_E_PARA at the entry point
+    monkeypatch.setenv("HCCL_DETERMINISTIC", "maybe")
+    comms = hccl_amd.comm_init_all(2)
+    try:
+        assert code_of(hccl_amd.all_reduce, comms[0], 0x2000, 0x3000, 8, DT.FP32, OP.SUM, 0x1000) == 1
+        assert code_of(hccl_amd.all_gather, comms[1], 0x2000, 0x3000, 8, DT.FP32, 0x1000) == 1
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)
+
+
 def test_group_end_without_start():
     assert code_of(hccl_amd.group_end) == 1

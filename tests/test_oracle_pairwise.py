@@ -130,6 +130,13 @@ def test_bf16_narrow_is_rne_on_upper_half(orc):
     assert np.array_equal(orc.np_fp32_to_bf16_bits(f), orc.fp32_to_bf16_bits(bits))
 
 
+def test_bf16_round_trip_is_identity(orc):
+    h = np.arange(65536, dtype=np.uint16)
+    wide = (h.astype(np.uint32) << 16).view(np.float32)
+    assert np.array_equal(orc.bf16_bits_to_fp32(h).view(np.uint32), wide.view(np.uint32))
+    assert np.array_equal(orc.fp32_to_bf16_bits(wide.view(np.uint32)), h)  # includes every NaN payload
+
+
 # ---------------------------------------------------------------------------------------------
 # a1: integers = two's-complement modular arithmetic
 # ---------------------------------------------------------------------------------------------
