@@ -63,6 +63,7 @@ class Algo(enum.IntEnum):
     NHR = 3
     ORDER_PRESERVED = 4
     AIV_MESH = 5
+    MESH_SYMMETRIC = 6
 
 
 class OpKind(enum.IntEnum):

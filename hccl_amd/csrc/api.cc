@@ -266,7 +266,7 @@ bool ParseAlgoName(const std::string& s, HcclAmdAlgo* algo)
     static const struct { const char* name; HcclAmdAlgo algo; } table[] = {
         {"mesh", HCCL_AMD_ALGO_MESH}, {"ring", HCCL_AMD_ALGO_RING}, {"rhd", HCCL_AMD_ALGO_RHD},
         {"nhr", HCCL_AMD_ALGO_NHR}, {"order_preserved", HCCL_AMD_ALGO_ORDER_PRESERVED},
-        {"aiv_mesh", HCCL_AMD_ALGO_AIV_MESH}};
+        {"aiv_mesh", HCCL_AMD_ALGO_AIV_MESH}, {"mesh_symmetric", HCCL_AMD_ALGO_MESH_SYMMETRIC}};
     for (const auto& e : table) {
         if (s == e.name) {
             *algo = e.algo;
@@ -559,7 +559,7 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
         }
         return HCCL_SUCCESS;
     }
-    // NHR: slices of ceil(count / n) elements (reference two_shot.cc:184 slicing rule).
+    // NHR, order-preserved, symmetric two-shot: slices of ceil(count / n) elements (reference two_shot.cc:184).
     a.total = a.groupLen = p.count;
     a.subLen = (p.count + n - 1) / n;
     return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);

@@ -340,6 +340,10 @@ HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPla
             return OrderPreserved(n, plan);
         case HCCL_AMD_ALGO_AIV_MESH:
             return ar ? HCCL_E_NOT_SUPPORT : AivMeshReduceScatter(n, plan);
+        case HCCL_AMD_ALGO_MESH_SYMMETRIC:
+            // Slice k of the AllReduce result is folded like rank k's ReduceScatter output.
+            plan->segmentsAreSubs = ar;
+            return MeshReduceScatter(n, plan);
         default:
             return HCCL_E_PARA;
     }

@@ -1,7 +1,7 @@
 /*
  * C ABI of the MI355X loopback data plane.
  *
- * The five collective entry points have the signatures of the reference's public
+ * The collective entry points have the signatures of the reference's public
  * header (reference include/hccl.h) so that a caller built against that header links
  * against this library unchanged.  `aclrtStream` carries a hipStream_t; every buffer
  * is a device pointer in the HBM of the one GPU; count / displacement arrays are host
@@ -178,6 +178,10 @@ typedef enum {
     /* Vector-core mesh order: chunk c of a rank's output starts at peer c and wraps upward
      * (reference aiv_reduce_scatter_mesh_1d.h:23-71). ReduceScatter only. */
     HCCL_AMD_ALGO_AIV_MESH = 5,
+    /* AllReduce in the order of the mesh two-shot template over symmetric memory: the result is cut into
+     * N slices of ceil(count / N) elements and slice k starts from rank k's input, then adds the other
+     * ranks ascending (reference ins_temp_all_reduce_mesh_1D_two_shot.cc:341-357).  ReduceScatter: MESH. */
+    HCCL_AMD_ALGO_MESH_SYMMETRIC = 6,
     HCCL_AMD_ALGO_COUNT
 } HcclAmdAlgo;
 

@@ -215,6 +215,8 @@ def all_reduce(ins, outs, count, dtype, op, acc=ACC_FP32, algo="mesh", max_count
         return _reduce_call("orc_all_reduce_mesh", ins, outs, count, dtype, op, acc)
     if algo == "two_shot":
         return _reduce_call("orc_all_reduce_two_shot", ins, outs, count, dtype, op, acc)
+    if algo == "mesh_symmetric":
+        return _reduce_call("orc_all_reduce_two_shot_symmetric", ins, outs, count, dtype, op, acc)
     if algo == "rhd":
         return _reduce_call("orc_all_reduce_rhd", ins, outs, count, dtype, op, acc,
                             ctypes.c_uint64(max_count_per_loop))
@@ -226,7 +228,7 @@ def all_reduce(ins, outs, count, dtype, op, acc=ACC_FP32, algo="mesh", max_count
 
 
 def reduce_scatter(ins, outs, recv_count, dtype, op, acc=ACC_FP32, algo="mesh"):
-    name = {"mesh": "orc_reduce_scatter_mesh", "nhr": "orc_reduce_scatter_nhr", "ring": "orc_reduce_scatter_nhr",
+    name = {"mesh": "orc_reduce_scatter_mesh", "mesh_symmetric": "orc_reduce_scatter_mesh", "nhr": "orc_reduce_scatter_nhr", "ring": "orc_reduce_scatter_nhr",
             "rhd": "orc_reduce_scatter_rhd", "order_preserved": "orc_reduce_scatter_order_preserved",
             "aiv_mesh": "orc_reduce_scatter_aiv_mesh"}[algo]
     return _reduce_call(name, ins, outs, recv_count, dtype, op, acc)

@@ -755,6 +755,49 @@ int orc_all_reduce_two_shot(uint32_t n, const void* const* in, void* const* out,
     return ORC_OK;
 }
 
+/* Two-shot, symmetric-memory variant (two_shot.cc:341-357 with supportSymmetricMemAccess_): slice k starts
+ * from rank k's own input slice, then the other ranks ascending; every rank gets every slice. */
+int orc_all_reduce_two_shot_symmetric(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype,
+                                      int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    uint64_t sliceCount = orc_round_up(count, n);   /* two_shot.cc:184 */
+    void* acc = malloc((sliceCount ? sliceCount : 1) * r.asz);
+    void* tmp = malloc((sliceCount ? sliceCount : 1) * r.asz);
+    uint8_t* res = (uint8_t*)malloc((count ? count : 1) * r.esz);
+    if (!acc || !tmp || !res) {
+        free(acc);
+        free(tmp);
+        free(res);
+        return ORC_E_INTERNAL;
+    }
+    uint64_t off = 0;
+    for (uint32_t k = 0; k < n; ++k) {
+        uint64_t cur = (count - off > sliceCount) ? sliceCount : count - off;
+        if (cur != 0) {
+            red_widen(&r, cbytes(in[k]) + off * r.esz, acc, cur);
+            for (uint32_t t = 0; t < n; ++t) {
+                if (t != k) {
+                    red_pair_from_storage(&r, acc, cbytes(in[t]) + off * r.esz, cur, tmp);
+                }
+            }
+            red_narrow(&r, acc, res + off * r.esz, cur);
+        }
+        off += cur;
+    }
+    for (uint32_t d = 0; d < n; ++d) {
+        memcpy(out[d], res, count * r.esz);
+    }
+    free(acc);
+    free(tmp);
+    free(res);
+    return ORC_OK;
+}
+
 /* a9: rank k: out = in_k[k]; for t = 0..N-1, t != k: out = in_t[k] (+) out. */
 static int reduce_scatter_mesh_range(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount,
                                      uint64_t first, uint64_t count, const red_t* r)

@@ -109,6 +109,9 @@ int orc_all_reduce_mesh(uint32_t n, const void* const* in, void* const* out, uin
 /* a8: two-shot slicing (two_shot.cc:178-210, 326-360) then gather; same values as one-shot. */
 int orc_all_reduce_two_shot(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
                             int accMode);
+/* two-shot over symmetric memory (two_shot.cc:341-357): slice k = x_k first, then ranks ascending skipping k. */
+int orc_all_reduce_two_shot_symmetric(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype,
+                                      int op, int accMode);
 /* a11: RS-RHD (skip POST) + bridge + AG-RHD (skip PRE), looped per rhd_tail.h; maxCountPerLoop 0 = unbounded. */
 int orc_all_reduce_rhd(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
                        int accMode, uint64_t maxCountPerLoop);

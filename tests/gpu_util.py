@@ -9,7 +9,7 @@ import hccl_amd
 from hccl_amd import Algo, OpKind
 
 ALGO_BY_NAME = {"mesh": Algo.MESH, "ring": Algo.RING, "rhd": Algo.RHD, "nhr": Algo.NHR,
-                "order_preserved": Algo.ORDER_PRESERVED, "aiv_mesh": Algo.AIV_MESH}
+                "order_preserved": Algo.ORDER_PRESERVED, "aiv_mesh": Algo.AIV_MESH, "mesh_symmetric": Algo.MESH_SYMMETRIC}
 
 
 def require_library_on_gpu():

@@ -148,7 +148,7 @@ def test_reduce_scatter_type_matrix(world8, dtype, op):
 def test_all_reduce_algorithms_and_ragged_counts(n):
     w = World(n)
     try:
-        for algo in ("mesh", "ring", "rhd", "nhr", "order_preserved"):
+        for algo in ("mesh", "ring", "rhd", "nhr", "order_preserved", "mesh_symmetric"):
             for count in (1, 3, 17, 129, 1023, 4093, 65_543):
                 run_all_reduce(w, DT.FP32, SUM, count, algo, seed=n * 1000 + count)
             run_all_reduce(w, DT.FP32, MAX, 2_051, algo, seed=n)
@@ -162,7 +162,7 @@ def test_all_reduce_algorithms_and_ragged_counts(n):
 def test_reduce_scatter_algorithms_and_ragged_counts(n):
     w = World(n)
     try:
-        for algo in ("mesh", "ring", "nhr", "rhd", "order_preserved", "aiv_mesh"):
+        for algo in ("mesh", "ring", "nhr", "rhd", "order_preserved", "aiv_mesh", "mesh_symmetric"):
             for c in (1, 3, 17, 129, 1024, 4093):
                 run_reduce_scatter(w, DT.FP32, SUM, c, algo, seed=n * 2000 + c)
             run_reduce_scatter(w, DT.FP32, MIN, 515, algo, seed=n + 3)

@@ -94,7 +94,8 @@ def same(a, b):
 
 RANKS = [1, 2, 3, 5, 6, 7, 8, 12, 16, 33, 64]
 ALGO_NAME = {Algo.MESH: "mesh", Algo.RING: "ring", Algo.RHD: "rhd", Algo.NHR: "nhr",
-             Algo.ORDER_PRESERVED: "order_preserved", Algo.AIV_MESH: "aiv_mesh"}
+             Algo.ORDER_PRESERVED: "order_preserved", Algo.AIV_MESH: "aiv_mesh",
+             Algo.MESH_SYMMETRIC: "mesh_symmetric"}
 
 
 @pytest.mark.parametrize("n", RANKS)
@@ -109,7 +110,8 @@ def test_every_program_uses_every_rank_once(n):
 
 
 @pytest.mark.parametrize("n", RANKS)
-@pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED, Algo.AIV_MESH])
+@pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED, Algo.AIV_MESH,
+                                  Algo.MESH_SYMMETRIC])
 def test_reduce_scatter_programs_match_oracle(orc, n, algo):
     progs = hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, algo, n)
     c = 2 * n + 5
@@ -133,7 +135,7 @@ def test_reduce_scatter_programs_match_oracle(orc, n, algo):
 
 
 @pytest.mark.parametrize("n", RANKS)
-@pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED])
+@pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED, Algo.MESH_SYMMETRIC])
 def test_all_reduce_programs_match_oracle(orc, n, algo):
     progs = hccl_amd.fold_programs(OpKind.ALL_REDUCE, algo, n)
     count = 5 * n + 3

@@ -437,3 +437,29 @@ def test_all_to_all_v_index_map(orc, n):
     bad = recv_counts.copy()
     bad[0, 1] += 1
     assert orc.all_to_all_v(ins, outs, send_counts, sdispls, bad, rdispls, I64) == 1
+
+
+# ---------------------------------------------------------------------------------------------
+# AllReduce two-shot over symmetric memory: slice k starts from rank k's input (two_shot.cc:341-357)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n,count", [(2, 7), (3, 100), (5, 3), (8, 1031), (16, 40)])
+def test_all_reduce_symmetric_two_shot_slice_k_starts_from_rank_k(orc, n, count):
+    rng = np.random.default_rng(n * 10 + count)
+    ins = wide_f32(rng, n, count)
+    outs = outs_like(ins)
+    assert orc.all_reduce(ins, outs, count, F32, SUM, algo="mesh_symmetric") == 0
+    sl = -(-count // n)                               # ceil(count / n), two_shot.cc:184
+    want = np.zeros(count, dtype=np.float32)
+    for k in range(n):
+        lo, hi = min(count, k * sl), min(count, (k + 1) * sl)
+        acc = ins[k][lo:hi].copy()
+        for t in range(n):
+            if t != k:
+                acc = ins[t][lo:hi] + acc
+        want[lo:hi] = acc
+    for r in range(n):
+        assert np.array_equal(outs[r].view(np.uint32), want.view(np.uint32)), r
+    if n > 2 and count > n:                             # and it is a different order from the plain two-shot
+        plain = outs_like(ins)
+        assert orc.all_reduce(ins, plain, count, F32, SUM, algo="two_shot") == 0
+        assert not np.array_equal(plain[0].view(np.uint32), want.view(np.uint32))
