@@ -230,6 +230,9 @@ struct World {
     uint32_t copyTileBytes = 0;
     // HCCL_DETERMINISTIC (reference alg_env_config.cc:1113-1153): 0 false, 1 true, 2 strict, 0xFF unparsable
     uint8_t deterministic = 0;
+    // Longest a rank waits on the host for its peers: the reference's CUSTOM_TIMEOUT = 1836 s (alg_param.h:91),
+    // overridable by HCCL_EXEC_TIMEOUT (seconds), read when the world is created.
+    uint32_t execTimeout = 1836;
 
     ~World()
     {
@@ -321,6 +324,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->copyTileBytes != 1024 && w->copyTileBytes != 4096 && w->copyTileBytes != 16384) {
         w->copyTileBytes = 0;
     }
+    w->execTimeout = EnvU32("HCCL_EXEC_TIMEOUT", 1836);
     ApplyAlgoEnv(w.get());
     if (const char* det = getenv("HCCL_DETERMINISTIC")) {
         std::string v(det);
@@ -967,13 +971,6 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
     return rc;
 }
 
-uint32_t ExecTimeoutSeconds()
-{
-    // Reference default CUSTOM_TIMEOUT = 1836 s (alg_param.h:91), overridable by HCCL_EXEC_TIMEOUT.
-    static uint32_t t = EnvU32("HCCL_EXEC_TIMEOUT", 1836);
-    return t;
-}
-
 // Deposits one rank's arguments; the call that completes the set launches.
 HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count, const void* send,
                   void* recv, hipStream_t stream, std::vector<uint64_t>&& var, uint32_t root = 0)
@@ -1012,9 +1009,9 @@ HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uin
         if (t_groupDepth > 0) {
             return p->result;   // queued; the group's last call launches
         }
-        bool ok = w->cv.wait_for(lock, std::chrono::seconds(ExecTimeoutSeconds()), [&] { return p->done; });
+        bool ok = w->cv.wait_for(lock, std::chrono::seconds(w->execTimeout), [&] { return p->done; });
         if (!ok) {
-            Log(1, "%s: rank %u waited %u s for the other ranks", OpName(type), c->rank, ExecTimeoutSeconds());
+            Log(1, "%s: rank %u waited %u s for the other ranks", OpName(type), c->rank, w->execTimeout);
             p->result = HCCL_E_TIMEOUT;
             return HCCL_E_TIMEOUT;
         }

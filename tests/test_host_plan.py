@@ -330,5 +330,40 @@ def test_unparsable_hccl_deterministic_fails_every_collective(monkeypatch):
             hccl_amd.comm_destroy(c)
 
 
+def test_a_rank_whose_peers_never_call_times_out(monkeypatch):
+    import time
+    monkeypatch.setenv("HCCL_EXEC_TIMEOUT", "1")
+    comms = hccl_amd.comm_init_all(2)
+    try:
+        t0 = time.perf_counter()
+        assert code_of(hccl_amd.all_reduce, comms[0], 0x2000, 0x3000, 8, DT.FP32, OP.SUM, 0x1000) == 9   # HCCL_E_TIMEOUT
+        assert 0.9 < time.perf_counter() - t0 < 5.0
+        # the late peer completes the set: the collective is not launched, both sides learn about the time-out
+        assert code_of(hccl_amd.all_reduce, comms[1], 0x2000, 0x3000, 8, DT.FP32, OP.SUM, 0x1000) == 9
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)
+
+
+def test_calls_that_disagree_are_rejected_without_a_launch():
+    comms = hccl_amd.comm_init_all(3)
+    try:
+        cases = [
+            lambda r: hccl_amd.all_reduce(comms[r], 0x2000, 0x3000, 8 if r < 2 else 9, DT.FP32, OP.SUM, 0x1000),
+            lambda r: hccl_amd.all_reduce(comms[r], 0x2000, 0x3000, 8, DT.FP32 if r < 2 else DT.FP16, OP.SUM, 0x1000),
+            lambda r: hccl_amd.all_reduce(comms[r], 0x2000, 0x3000, 8, DT.FP32, OP.SUM if r < 2 else OP.MAX, 0x1000),
+            lambda r: hccl_amd.reduce(comms[r], 0x2000, 0x3000, 8, DT.FP32, OP.SUM, 0 if r < 2 else 1, 0x1000),
+            lambda r: (hccl_amd.all_reduce if r < 2 else hccl_amd.reduce_scatter)(comms[r], 0x2000, 0x3000, 8, DT.FP32,
+                                                                                 OP.SUM, 0x1000),
+        ]
+        for case in cases:
+            with hccl_amd.group():
+                codes = [code_of(case, r) for r in range(3)]
+            assert codes == [0, 0, 1], codes          # the call that completes the set reports HCCL_E_PARA
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)
+
+
 def test_group_end_without_start():
     assert code_of(hccl_amd.group_end) == 1
