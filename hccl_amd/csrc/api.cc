@@ -228,6 +228,7 @@ struct World {
     uint32_t reduceBlocks = 1u << 20;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
+    uint32_t storePolicy = 0;     // HCCL_AMD_STORE_POLICY for the reduce kernel: 0 non-temporal, 1 write-through
     // HCCL_DETERMINISTIC (reference alg_env_config.cc:1113-1153): 0 false, 1 true, 2 strict, 0xFF unparsable
     uint8_t deterministic = 0;
     // Longest a rank waits on the host for its peers: the reference's CUSTOM_TIMEOUT = 1836 s (alg_param.h:91),
@@ -325,6 +326,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->copyTileBytes = 0;
     }
     w->execTimeout = EnvU32("HCCL_EXEC_TIMEOUT", 1836);
+    w->storePolicy = EnvU32("HCCL_AMD_STORE_POLICY", 0) == 1 ? 1 : 0;
     ApplyAlgoEnv(w.get());
     if (const char* det = getenv("HCCL_DETERMINISTIC")) {
         std::string v(det);
@@ -490,6 +492,9 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     }
     // Small workgroups retire sooner and keep the window of addresses in flight compact; nested fold
     // programs park accumulators in LDS and want a few more lanes per workgroup to hide that.
+    // Results of a reduce leave through non-temporal stores: measured equal to write-through stores with one
+    // result stream and 2-3 % better with sixteen.  (The copy kernels always write through.)
+    a.writeThrough = w->storePolicy == 1 ? 1u : 0u;
     a.threads = w->reduceThreads != 0 ? w->reduceThreads : (plan.maxDepth > 1 ? 128u : 64u);
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
     uint64_t blocks = subs * a.blocksPerSub;

@@ -40,7 +40,11 @@ __device__ __forceinline__ V LoadNt(const void* p)
 template <typename V>
 __device__ __forceinline__ void StoreNt(V v, void* p)
 {
-    __builtin_nontemporal_store(v, (__attribute__((address_space(1))) V*)p);
+    if constexpr (sizeof(V) == 16) {
+        StoreStream16(p, __builtin_bit_cast(StreamVec, v));
+    } else {
+        __builtin_nontemporal_store(v, (__attribute__((address_space(1))) V*)p);
+    }
 }
 
 // Tables are read through the constant address space so that the loads are scalar.

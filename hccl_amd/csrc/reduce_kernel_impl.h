@@ -156,11 +156,15 @@ __device__ __forceinline__ Pack<S, W> LoadPack(const void* base, uint64_t elemOf
 }
 
 template <typename S, int W>
-__device__ __forceinline__ void StorePack(void* base, uint64_t elemOff, const Pack<S, W>& v)
+__device__ __forceinline__ void StorePack(void* base, uint64_t elemOff, const Pack<S, W>& v, bool writeThrough)
 {
     S* p = static_cast<S*>(base) + elemOff;
     if constexpr (sizeof(S) * W == 16) {
-        __builtin_nontemporal_store(__builtin_bit_cast(U32x4, v), (HCCL_AMD_GLOBAL U32x4*)p);
+        if (writeThrough) {
+            StoreStream16(p, __builtin_bit_cast(StreamVec, v));
+        } else {
+            __builtin_nontemporal_store(__builtin_bit_cast(U32x4, v), (HCCL_AMD_GLOBAL U32x4*)p);
+        }
     } else {
         __builtin_nontemporal_store(v.e[0], (HCCL_AMD_GLOBAL S*)p);
     }
@@ -317,10 +321,10 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
         out.e[w] = E::Narrow(acc.a[w]);
     }
     if (args.dstOwn) {
-        StorePack<S, W>(args.dst[group], dstOff + e, out);
+        StorePack<S, W>(args.dst[group], dstOff + e, out, args.writeThrough != 0);
     } else {
         for (uint32_t d = 0; d < args.nDst; ++d) {
-            StorePack<S, W>(args.dst[d], dstOff + e, out);
+            StorePack<S, W>(args.dst[d], dstOff + e, out, args.writeThrough != 0);
         }
     }
 }
