@@ -3,10 +3,10 @@
 
 namespace hccl_amd {
 namespace {
-using Ops0 = detail::IntOps<int8_t, uint8_t, detail::kSum>;
-using Ops1 = detail::IntOps<int8_t, uint8_t, detail::kProd>;
-using Ops2 = detail::IntOps<int8_t, uint8_t, detail::kMax>;
-using Ops3 = detail::IntOps<int8_t, uint8_t, detail::kMin>;
+using Ops0 = detail::Int8Ops<detail::kSum>;
+using Ops1 = detail::Int8Ops<detail::kProd>;
+using Ops2 = detail::Int8Ops<detail::kMax>;
+using Ops3 = detail::Int8Ops<detail::kMin>;
 }  // namespace
 
 HCCL_AMD_DEFINE_SELECT4(SelectReduceI8, Ops0, Ops1, Ops2, Ops3)

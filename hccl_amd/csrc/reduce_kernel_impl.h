@@ -51,6 +51,31 @@ struct IntOps {
     }
 };
 
+// int8 with a 16-bit accumulator per element: the low byte of a 16-bit sum or product is the 8-bit result
+// (alg_data_trans_wrapper.cc:1332-1343), MAX / MIN see the sign-extended value.  `Swar` switches the 16-byte
+// vector path to the packed form of PackOps.
+template <int OP>
+struct Int8Ops {
+    using S = int8_t;
+    using A = int16_t;
+    using Swar = void;
+    static constexpr int kOp = OP;
+    static __device__ __forceinline__ A Widen(S x) { return x; }
+    static __device__ __forceinline__ S Narrow(A a) { return static_cast<S>(static_cast<uint8_t>(a)); }
+    static __device__ __forceinline__ A Fold(A src, A dst)
+    {
+        if constexpr (OP == kSum) {
+            return static_cast<A>(static_cast<uint16_t>(static_cast<uint16_t>(src) + static_cast<uint16_t>(dst)));
+        } else if constexpr (OP == kProd) {
+            return static_cast<A>(static_cast<uint16_t>(static_cast<uint16_t>(src) * static_cast<uint16_t>(dst)));
+        } else if constexpr (OP == kMax) {
+            return (src < dst) ? dst : src;
+        } else {
+            return (dst < src) ? dst : src;
+        }
+    }
+};
+
 template <typename T, int OP>
 struct FpOps {
     using S = T;
@@ -84,14 +109,41 @@ __device__ __forceinline__ uint16_t FloatToBf16Bits(float f)
     return static_cast<uint16_t>(isNan ? quiet : rounded);
 }
 
+// 1.0f the optimiser cannot see through: multiplying by it keeps a fused multiply-add a fused multiply-add.
+__device__ __forceinline__ float OpaqueOne()
+{
+    float one;
+    asm volatile("v_mov_b32 %0, 1.0" : "=v"(one));
+    return one;
+}
+
 // fp16 / bf16 SUM: fp32 accumulator, one rounding at the end.
+//  * fp16 operands are folded with fma(x, 1, acc): x * 1 is exact, so the result is the IEEE sum, and the
+//    hardware's mixed-precision fma converts and adds in one instruction.
+//  * bf16 results are narrowed by the hardware's round-to-nearest-even conversion.  A NaN result is some
+//    NaN (NaNs produced or carried by a sum have no defined payload); MAX / MIN never come here.
 template <bool IS_BF16>
 struct HalfSumOps {
     using S = uint16_t;
     using A = float;
     static __device__ __forceinline__ A Widen(S x) { return IS_BF16 ? Bf16BitsToFloat(x) : HalfBitsToFloat(x); }
-    static __device__ __forceinline__ S Narrow(A a) { return IS_BF16 ? FloatToBf16Bits(a) : FloatToHalfBits(a); }
+    static __device__ __forceinline__ S Narrow(A a)
+    {
+        if constexpr (IS_BF16) {
+            return __builtin_bit_cast(uint16_t, static_cast<__bf16>(a));
+        } else {
+            return FloatToHalfBits(a);
+        }
+    }
     static __device__ __forceinline__ A Fold(A src, A dst) { return src + dst; }
+    static __device__ __forceinline__ A Accumulate(S x, A acc, float one)
+    {
+        if constexpr (IS_BF16) {
+            return Bf16BitsToFloat(x) + acc;
+        } else {
+            return __builtin_fmaf(static_cast<float>(__builtin_bit_cast(_Float16, x)), one, acc);
+        }
+    }
 };
 
 // fp16 PROD: the product of two fp16 values is exact in fp32, so rounding it to fp16 after every step
@@ -226,32 +278,166 @@ struct BlockProgram {
     uint32_t nLeaves;
 };
 
-// Leaves whose loads are issued together: sixteen for 4- and 8-byte elements, eight for the narrower ones
-// (their unpacked accumulators need the registers).
+// Leaves whose loads are issued together: sixteen vectors, or eight single elements.
 template <typename S, int W>
 __device__ constexpr int LoadBatch()
 {
-    return (sizeof(S) >= 4 && W > 1) ? 16 : 8;
+    return W > 1 ? 16 : 8;
 }
 
 // Makes eight loaded vectors opaque to the optimiser at this point of the instruction stream.
-template <typename S, int W>
-__device__ __forceinline__ void IssueFence8(Pack<S, W>* v)
+__device__ __forceinline__ void IssueFence8(U32x4* r)
 {
-    U32x4 r0 = __builtin_bit_cast(U32x4, v[0]), r1 = __builtin_bit_cast(U32x4, v[1]);
-    U32x4 r2 = __builtin_bit_cast(U32x4, v[2]), r3 = __builtin_bit_cast(U32x4, v[3]);
-    U32x4 r4 = __builtin_bit_cast(U32x4, v[4]), r5 = __builtin_bit_cast(U32x4, v[5]);
-    U32x4 r6 = __builtin_bit_cast(U32x4, v[6]), r7 = __builtin_bit_cast(U32x4, v[7]);
-    asm volatile("" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3), "+v"(r4), "+v"(r5), "+v"(r6), "+v"(r7));
-    v[0] = __builtin_bit_cast(Pack<S, W>, r0);
-    v[1] = __builtin_bit_cast(Pack<S, W>, r1);
-    v[2] = __builtin_bit_cast(Pack<S, W>, r2);
-    v[3] = __builtin_bit_cast(Pack<S, W>, r3);
-    v[4] = __builtin_bit_cast(Pack<S, W>, r4);
-    v[5] = __builtin_bit_cast(Pack<S, W>, r5);
-    v[6] = __builtin_bit_cast(Pack<S, W>, r6);
-    v[7] = __builtin_bit_cast(Pack<S, W>, r7);
+    asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
 }
+
+// acc <- x (+) acc for a stored element x: the traits' fused form where they have one.
+template <class E, class = void>
+struct HasAccumulate {
+    static constexpr bool value = false;
+};
+template <class E>
+struct HasAccumulate<E, decltype(void(E::Accumulate(typename E::S{}, typename E::A{}, 1.0f)))> {
+    static constexpr bool value = true;
+};
+
+template <class E>
+__device__ __forceinline__ typename E::A Accumulate(typename E::S x, typename E::A acc, float one)
+{
+    if constexpr (HasAccumulate<E>::value) {
+        return E::Accumulate(x, acc, one);
+    } else {
+        return E::Fold(E::Widen(x), acc);
+    }
+}
+
+// The four things the interpreter does with a loaded vector of W elements.  The default goes element by
+// element; a traits class may bring a packed form for its 16-byte vectors (E::Swar).
+template <class E, int W, class = void>
+struct PackOps {
+    using S = typename E::S;
+    static __device__ __forceinline__ void Init(AccPack<E, W>& acc, const Pack<S, W>& v)
+    {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            acc.a[w] = E::Widen(v.e[w]);
+        }
+    }
+    static __device__ __forceinline__ void Accumulate(AccPack<E, W>& acc, const Pack<S, W>& v, float one)
+    {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            acc.a[w] = detail::Accumulate<E>(v.e[w], acc.a[w], one);
+        }
+    }
+    static __device__ __forceinline__ void Merge(AccPack<E, W>& acc, const AccPack<E, W>& outer)
+    {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            acc.a[w] = E::Fold(acc.a[w], outer.a[w]);
+        }
+    }
+    static __device__ __forceinline__ Pack<S, W> Narrow(const AccPack<E, W>& acc)
+    {
+        Pack<S, W> out;
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            out.e[w] = E::Narrow(acc.a[w]);
+        }
+        return out;
+    }
+};
+
+// int8 vectors, four elements per dword: the accumulator of a dword is two dwords of two 16-bit lanes each,
+// `even` for bytes 0 and 2, `odd` for bytes 1 and 3.  SUM and PROD only need the low byte of a lane to be right
+// (it never depends on what sits above it), so operands go in unmasked: `x` for the even lanes, `x >> 8` for the
+// odd ones.  MAX / MIN compare sign-extended lanes.  The 32 bytes of AccPack<E, 16> hold the eight dwords.
+template <class E>
+struct PackOps<E, 16, typename E::Swar> {
+    using S = typename E::S;
+    typedef int16_t S16x2 __attribute__((ext_vector_type(2)));
+    typedef uint16_t U16x2 __attribute__((ext_vector_type(2)));
+    struct Lanes {
+        uint32_t even[4];
+        uint32_t odd[4];
+    };
+    static_assert(sizeof(Lanes) == sizeof(AccPack<E, 16>), "accumulator layout");
+
+    static __device__ __forceinline__ uint32_t EvenOperand(uint32_t x)
+    {
+        if constexpr (E::kOp == kMax || E::kOp == kMin) {
+            return __builtin_bit_cast(uint32_t, (__builtin_bit_cast(S16x2, x) << 8) >> 8);
+        } else {
+            return x;
+        }
+    }
+    static __device__ __forceinline__ uint32_t OddOperand(uint32_t x)
+    {
+        if constexpr (E::kOp == kMax || E::kOp == kMin) {
+            return __builtin_bit_cast(uint32_t, __builtin_bit_cast(S16x2, x) >> 8);
+        } else {
+            return x >> 8;
+        }
+    }
+    // dst <- src (+) dst on both lanes of a dword
+    static __device__ __forceinline__ uint32_t FoldLanes(uint32_t src, uint32_t dst)
+    {
+        if constexpr (E::kOp == kSum) {
+            return __builtin_bit_cast(uint32_t, __builtin_bit_cast(U16x2, src) + __builtin_bit_cast(U16x2, dst));
+        } else if constexpr (E::kOp == kProd) {
+            return __builtin_bit_cast(uint32_t, __builtin_bit_cast(U16x2, src) * __builtin_bit_cast(U16x2, dst));
+        } else if constexpr (E::kOp == kMax) {
+            return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(S16x2, src),
+                                                                          __builtin_bit_cast(S16x2, dst)));
+        } else {
+            return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(S16x2, src),
+                                                                          __builtin_bit_cast(S16x2, dst)));
+        }
+    }
+    static __device__ __forceinline__ void Init(AccPack<E, 16>& acc, const Pack<S, 16>& v)
+    {
+        const U32x4 x = __builtin_bit_cast(U32x4, v);
+        Lanes l;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            l.even[k] = EvenOperand(x[k]);
+            l.odd[k] = OddOperand(x[k]);
+        }
+        acc = __builtin_bit_cast(AccPack<E, 16>, l);
+    }
+    static __device__ __forceinline__ void Accumulate(AccPack<E, 16>& acc, const Pack<S, 16>& v, float)
+    {
+        const U32x4 x = __builtin_bit_cast(U32x4, v);
+        Lanes l = __builtin_bit_cast(Lanes, acc);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            l.even[k] = FoldLanes(EvenOperand(x[k]), l.even[k]);
+            l.odd[k] = FoldLanes(OddOperand(x[k]), l.odd[k]);
+        }
+        acc = __builtin_bit_cast(AccPack<E, 16>, l);
+    }
+    static __device__ __forceinline__ void Merge(AccPack<E, 16>& acc, const AccPack<E, 16>& outer)
+    {
+        Lanes l = __builtin_bit_cast(Lanes, acc);
+        const Lanes o = __builtin_bit_cast(Lanes, outer);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            l.even[k] = FoldLanes(l.even[k], o.even[k]);
+            l.odd[k] = FoldLanes(l.odd[k], o.odd[k]);
+        }
+        acc = __builtin_bit_cast(AccPack<E, 16>, l);
+    }
+    static __device__ __forceinline__ Pack<S, 16> Narrow(const AccPack<E, 16>& acc)
+    {
+        const Lanes l = __builtin_bit_cast(Lanes, acc);
+        U32x4 x;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            x[k] = (l.even[k] & 0x00FF00FFu) | ((l.odd[k] & 0x00FF00FFu) << 8);
+        }
+        return __builtin_bit_cast(Pack<S, 16>, x);
+    }
+};
 
 // Evaluates the whole tree for the W elements at element offset `e` of the sub-segment.  Leaves are
 // taken a batch at a time: their loads are all issued before the first fold, whatever the tree shape.
@@ -261,25 +447,44 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
 {
     using S = typename E::S;
     AccPack<E, W> acc;
+    float one = 1.0f;
+    if constexpr (HasAccumulate<E>::value) {
+        one = OpaqueOne();
+    }
     uint32_t level = 0;
     bool init = true;   // the next leaf starts a level instead of being folded into it
     const uint32_t nLeaves = bp.nLeaves;
     constexpr int kBatch = LoadBatch<S, W>();
     for (uint32_t b = 0; b < nLeaves; b += kBatch) {
         Pack<S, W> v[kBatch];
-#pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-            if (b + i < nLeaves) {
-                const void* base = reinterpret_cast<const void*>(Uniform64(bp.leafPtr[b + i]));
-                v[i] = LoadPack<S, W>(base, e);
-            }
-        }
         if constexpr (sizeof(S) * W == 16) {
-            // Nothing may consume a loaded vector before the whole batch has been issued: without this the
-            // compiler sinks the first unpacking instruction of each operand next to its load and waits there.
+            // The vectors stay untyped 128-bit values until the whole batch has been issued: nothing may
+            // consume one earlier (the compiler would sink the first unpacking instruction of each operand
+            // next to its load and wait there), and a load retyped to the element type loses its
+            // non-temporal hint.
+            U32x4 raw[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                if (b + i < nLeaves) {
+                    const S* p = reinterpret_cast<const S*>(Uniform64(bp.leafPtr[b + i])) + e;
+                    raw[i] = __builtin_nontemporal_load((const HCCL_AMD_GLOBAL U32x4*)p);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < kBatch; i += 8) {
-                IssueFence8<S, W>(v + i);
+                IssueFence8(raw + i);
+            }
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                v[i] = __builtin_bit_cast(Pack<S, W>, raw[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                if (b + i < nLeaves) {
+                    const void* base = reinterpret_cast<const void*>(Uniform64(bp.leafPtr[b + i]));
+                    v[i] = LoadPack<S, W>(base, e);
+                }
             }
         }
 #pragma unroll
@@ -292,34 +497,21 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
                     init = true;
                 }
                 if (init) {
-#pragma unroll
-                    for (int w = 0; w < W; ++w) {
-                        acc.a[w] = E::Widen(v[i].e[w]);
-                    }
+                    PackOps<E, W>::Init(acc, v[i]);
                     init = false;
                 } else {
-#pragma unroll
-                    for (int w = 0; w < W; ++w) {
-                        acc.a[w] = E::Fold(E::Widen(v[i].e[w]), acc.a[w]);
-                    }
+                    PackOps<E, W>::Accumulate(acc, v[i], one);
                 }
                 for (uint32_t closes = ctl & 0x7Fu; closes != 0; --closes) {
                     AccPack<E, W> outer;
                     --level;
                     PopAcc<E, W>(stack, args.threads, level, outer);
-#pragma unroll
-                    for (int w = 0; w < W; ++w) {
-                        acc.a[w] = E::Fold(acc.a[w], outer.a[w]);   // nested value is src, enclosing level is dst
-                    }
+                    PackOps<E, W>::Merge(acc, outer);   // nested value is src, enclosing level is dst
                 }
             }
         }
     }
-    Pack<S, W> out;
-#pragma unroll
-    for (int w = 0; w < W; ++w) {
-        out.e[w] = E::Narrow(acc.a[w]);
-    }
+    const Pack<S, W> out = PackOps<E, W>::Narrow(acc);
     if (args.dstOwn) {
         StorePack<S, W>(args.dst[group], dstOff + e, out, args.writeThrough != 0);
     } else {
