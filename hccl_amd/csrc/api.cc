@@ -472,16 +472,15 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
                            hipStream_t s)
 {
     uint32_t esz = DataTypeSize(dtype);
+    // The 128-bit path needs the destinations of one output position to share their offset from a 16-byte
+    // boundary (one head for all the stores); sources are loaded unaligned and need nothing.
     uint64_t bits = 0;
-    uint32_t nSrc = w->n;
-    for (uint32_t r = 0; r < nSrc; ++r) bits |= reinterpret_cast<uint64_t>(a.src[r]);
-    if (a.dstOwn) {
-        for (uint32_t g = 0; g < a.nGroup; ++g) bits |= reinterpret_cast<uint64_t>(a.dst[g]);
-    } else {
-        for (uint32_t d = 0; d < a.nDst; ++d) bits |= reinterpret_cast<uint64_t>(a.dst[d]);
+    if (!a.dstOwn) {
+        for (uint32_t d = 1; d < a.nDst; ++d) {
+            bits |= reinterpret_cast<uint64_t>(a.dst[d]) ^ reinterpret_cast<uint64_t>(a.dst[0]);
+        }
+        if (a.nGroup > 1) bits |= a.dstGroupStride * esz;
     }
-    if (a.nGroup > 1) bits |= a.srcGroupStride * esz | a.dstGroupStride * esz;
-    // Sub-segment starts need no alignment: sources and destinations share them, the kernel peels.
     a.vecOk = (bits & 15u) == 0 ? 1u : 0u;
     uint64_t subs = static_cast<uint64_t>(a.nGroup) * a.nSub;
     uint64_t longest = a.groupLen;   // the last sub-segment takes what the others leave

@@ -192,6 +192,7 @@ struct alignas(sizeof(S) * W >= 16 ? 16 : sizeof(S) * W) Pack {
 // a flat load also counts as an LDS operation, and waiting for the next LDS read (a leaf pointer)
 // would then wait for every load issued before it.
 #define HCCL_AMD_GLOBAL __attribute__((address_space(1)))
+typedef U32x4 U32x4Unaligned __attribute__((aligned(1)));   // a 128-bit load that may start on any element
 
 template <typename S, int W>
 __device__ __forceinline__ Pack<S, W> LoadPack(const void* base, uint64_t elemOff)
@@ -467,7 +468,7 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
             for (int i = 0; i < kBatch; ++i) {
                 if (b + i < nLeaves) {
                     const S* p = reinterpret_cast<const S*>(Uniform64(bp.leafPtr[b + i])) + e;
-                    raw[i] = __builtin_nontemporal_load((const HCCL_AMD_GLOBAL U32x4*)p);
+                    raw[i] = __builtin_nontemporal_load((const HCCL_AMD_GLOBAL U32x4Unaligned*)p);
                 }
             }
 #pragma unroll
@@ -574,17 +575,18 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     const uint64_t stride = static_cast<uint64_t>(args.blocksPerSub) * args.threads;
     const uint64_t first = static_cast<uint64_t>(blk) * args.threads + threadIdx.x;
 
-    // When vecOk, every source and destination address of this sub-segment has the same offset from a
-    // 16-byte boundary: `head` elements bring them all onto it, a 128-bit body follows, and fewer than
-    // W elements remain.  Otherwise everything goes element by element.  The body's vectors are dealt
-    // to the lanes shifted by `lead`, so that lane 0 of every wavefront starts a 128-byte line of the
-    // first source (a wavefront whose 1 KiB straddles nine lines fetches two of them twice).
+    // When vecOk, every destination address of this sub-segment has the same offset from a 16-byte
+    // boundary: `head` elements bring the stores onto it, a 128-bit body follows, and fewer than W elements
+    // remain.  Sources only need element alignment: their 128-bit loads may be unaligned (full speed when
+    // they are congruent with the destination, a few percent less otherwise).  Without vecOk everything
+    // goes element by element.  The body's vectors are dealt to the lanes shifted by `lead`, so that lane 0
+    // of every wavefront starts a 128-byte line of the destination (a wavefront whose 1 KiB straddles nine
+    // lines moves two of them twice).
     uint64_t head = len;
     uint64_t nVec = 0;
     uint32_t lead = 0;
-    // A group that starts at an odd offset into the sources is not congruent with its destination.
-    if (args.vecOk && (!args.varGroups || ((gSrc * sizeof(S)) & 15u) == 0)) {
-        const uint64_t addr = reinterpret_cast<uint64_t>(args.src[0]) + srcOff * sizeof(S);
+    if (args.vecOk) {
+        const uint64_t addr = reinterpret_cast<uint64_t>(args.dstOwn ? args.dst[g] : args.dst[0]) + dstOff * sizeof(S);
         const uint32_t mis = static_cast<uint32_t>(addr & 15u);
         head = mis ? (16u - mis) / sizeof(S) : 0;
         head = head < len ? head : len;
