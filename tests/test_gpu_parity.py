@@ -88,14 +88,19 @@ def check(dtype, op, got, want, what):
             what, diff.size, got.size, diff[:4], got[diff[:4]], want[diff[:4]]))
 
 
+def pad_of(pad, r, which):
+    """pad may be a number (every buffer alike) or a function (rank, 'send' | 'recv') -> bytes."""
+    return pad(r, which) if callable(pad) else pad
+
+
 def run_all_reduce(world, dtype, op, count, algo, seed, pad=0, in_place=False):
     rng = np.random.default_rng(seed)
     n = world.n
     ins = [gen(dtype, op, rng, count) for _ in range(n)]
     want = [np.zeros(count, dtype=NP[dtype]) for _ in range(n)]
     assert oracle.all_reduce(ins, want, count, int(dtype), op, acc=oracle.ACC_FP32, algo=algo) == 0
-    sends = [to_dev(x, pad) for x in ins]
-    recvs = sends if in_place else [dev_zeros(x.nbytes, pad) for x in ins]
+    sends = [to_dev(x, pad_of(pad, r, "send")) for r, x in enumerate(ins)]
+    recvs = sends if in_place else [dev_zeros(x.nbytes, pad_of(pad, r, "recv")) for r, x in enumerate(ins)]
     world.all_reduce(sends, recvs, count, dtype, op, algo)
     for r in range(n):
         check(dtype, op, to_host(recvs[r], NP[dtype]), want[r],
@@ -108,8 +113,8 @@ def run_reduce_scatter(world, dtype, op, c, algo, seed, pad=0):
     ins = [gen(dtype, op, rng, n * c) for _ in range(n)]
     want = [np.zeros(c, dtype=NP[dtype]) for _ in range(n)]
     assert oracle.reduce_scatter(ins, want, c, int(dtype), op, acc=oracle.ACC_FP32, algo=algo) == 0
-    sends = [to_dev(x, pad) for x in ins]
-    recvs = [dev_zeros(c * ins[0].itemsize, pad) for _ in range(n)]
+    sends = [to_dev(x, pad_of(pad, r, "send")) for r, x in enumerate(ins)]
+    recvs = [dev_zeros(c * ins[0].itemsize, pad_of(pad, r, "recv")) for r in range(n)]
     world.reduce_scatter(sends, recvs, c, dtype, op, algo)
     for r in range(n):
         check(dtype, op, to_host(recvs[r], NP[dtype]), want[r],
@@ -175,6 +180,15 @@ def test_unaligned_buffers_and_in_place(world8):
     for pad in (2, 4, 8):          # payload starts 2 / 4 / 8 bytes past a 16-byte boundary
         run_all_reduce(world8, DT.FP16, SUM, 5_001, "mesh", seed=pad, pad=pad)
         run_reduce_scatter(world8, DT.BFP16, SUM, 999, "mesh", seed=pad + 10, pad=pad)
+    # every buffer at its own offset from a 16-byte boundary: sources are read unaligned; AllReduce into
+    # differently aligned recvBufs is the one case left to the element path
+    mixed = lambda r, which: (2 * r + (4 if which == "recv" else 0)) % 16
+    run_all_reduce(world8, DT.FP16, SUM, 20_011, "mesh", seed=31, pad=mixed)
+    run_all_reduce(world8, DT.BFP16, MAX, 4_097, "rhd", seed=32, pad=mixed)
+    run_all_reduce(world8, DT.FP16, SUM, 20_011, "nhr", seed=33, pad=lambda r, which: 2 * r % 16 if which == "send" else 6)
+    run_reduce_scatter(world8, DT.BFP16, SUM, 5_003, "ring", seed=34, pad=mixed)
+    run_reduce_scatter(world8, DT.INT8, SUM, 5_003, "mesh", seed=35, pad=lambda r, which: (r * 5 + 1) % 16)
+    run_reduce_scatter(world8, DT.INT32, MAX, 1_001, "rhd", seed=36, pad=lambda r, which: 4 * (r % 4))
     run_all_reduce(world8, DT.FP32, SUM, 70_001, "mesh", seed=77, in_place=True)
     run_all_reduce(world8, DT.INT64, MAX, 9_999, "rhd", seed=78, in_place=True)
 
