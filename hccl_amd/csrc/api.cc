@@ -228,6 +228,7 @@ struct World {
     uint32_t reduceBlocks = 1u << 20;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
+    bool reduceVector = true;
     uint32_t storePolicy = 0;     // HCCL_AMD_STORE_POLICY for the reduce kernel: 0 non-temporal, 1 write-through
     // HCCL_DETERMINISTIC (reference alg_env_config.cc:1113-1153): 0 false, 1 true, 2 strict, 0xFF unparsable
     uint8_t deterministic = 0;
@@ -327,6 +328,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     }
     w->execTimeout = EnvU32("HCCL_EXEC_TIMEOUT", 1836);
     w->storePolicy = EnvU32("HCCL_AMD_STORE_POLICY", 0) == 1 ? 1 : 0;
+    w->reduceVector = EnvU32("HCCL_AMD_REDUCE_VECTOR", 1) != 0;
     ApplyAlgoEnv(w.get());
     if (const char* det = getenv("HCCL_DETERMINISTIC")) {
         std::string v(det);
@@ -472,16 +474,10 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
                            hipStream_t s)
 {
     uint32_t esz = DataTypeSize(dtype);
-    // The 128-bit path needs the destinations of one output position to share their offset from a 16-byte
-    // boundary (one head for all the stores); sources are loaded unaligned and need nothing.
-    uint64_t bits = 0;
-    if (!a.dstOwn) {
-        for (uint32_t d = 1; d < a.nDst; ++d) {
-            bits |= reinterpret_cast<uint64_t>(a.dst[d]) ^ reinterpret_cast<uint64_t>(a.dst[0]);
-        }
-        if (a.nGroup > 1) bits |= a.dstGroupStride * esz;
-    }
-    a.vecOk = (bits & 15u) == 0 ? 1u : 0u;
+    // 128-bit loads and stores may start on any element (the head is peeled for the first destination, which
+    // makes every store aligned in the usual case of equally aligned recvBufs).  HCCL_AMD_REDUCE_VECTOR=0
+    // forces the element-by-element path.
+    a.vecOk = w->reduceVector ? 1u : 0u;
     uint64_t subs = static_cast<uint64_t>(a.nGroup) * a.nSub;
     uint64_t longest = a.groupLen;   // the last sub-segment takes what the others leave
     if (a.nSub > 1) {

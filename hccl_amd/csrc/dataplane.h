@@ -70,7 +70,7 @@ struct ReduceArgs {
     uint32_t progGroupStride;
     uint32_t progSubStride;
     uint32_t blocksPerSub;
-    uint32_t vecOk;   // the destinations of one output position share their offset from a 16-byte boundary
+    uint32_t vecOk;   // take the 128-bit path (0: element by element, for testing)
     uint32_t threads; // workgroup size of the launch
     uint32_t writeThrough;   // 16-byte results leave through StoreStream16 instead of a non-temporal store
     // Groups of unequal length (ReduceScatterV): when varGroups is set, group g spans groupLenV[g]

@@ -216,7 +216,7 @@ __device__ __forceinline__ void StorePack(void* base, uint64_t elemOff, const Pa
         if (writeThrough) {
             StoreStream16(p, __builtin_bit_cast(StreamVec, v));
         } else {
-            __builtin_nontemporal_store(__builtin_bit_cast(U32x4, v), (HCCL_AMD_GLOBAL U32x4*)p);
+            __builtin_nontemporal_store(__builtin_bit_cast(U32x4, v), (HCCL_AMD_GLOBAL U32x4Unaligned*)p);
         }
     } else {
         __builtin_nontemporal_store(v.e[0], (HCCL_AMD_GLOBAL S*)p);
@@ -575,11 +575,10 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     const uint64_t stride = static_cast<uint64_t>(args.blocksPerSub) * args.threads;
     const uint64_t first = static_cast<uint64_t>(blk) * args.threads + threadIdx.x;
 
-    // When vecOk, every destination address of this sub-segment has the same offset from a 16-byte
-    // boundary: `head` elements bring the stores onto it, a 128-bit body follows, and fewer than W elements
-    // remain.  Sources only need element alignment: their 128-bit loads may be unaligned (full speed when
-    // they are congruent with the destination, a few percent less otherwise).  Without vecOk everything
-    // goes element by element.  The body's vectors are dealt to the lanes shifted by `lead`, so that lane 0
+    // When vecOk, `head` elements bring the stores to the first destination onto a 16-byte boundary, a 128-bit
+    // body follows, and fewer than W elements remain.  Sources and further destinations only need element
+    // alignment: their 128-bit accesses may be unaligned (full speed when they are congruent with the first
+    // destination, up to 15 % less otherwise).  Without vecOk everything goes element by element.  The body's vectors are dealt to the lanes shifted by `lead`, so that lane 0
     // of every wavefront starts a 128-byte line of the destination (a wavefront whose 1 KiB straddles nine
     // lines moves two of them twice).
     uint64_t head = len;

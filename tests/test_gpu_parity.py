@@ -319,3 +319,20 @@ def test_hccl_deterministic_strict_selects_the_order_preserved_fold(monkeypatch)
             check(DT.FP32, SUM, to_host(recvs[r], np.float32), want[r], "strict reduce_scatter rank %d" % r)
     finally:
         w.close()
+
+
+def test_element_by_element_path_for_every_type(monkeypatch):
+    """The path heads, tails and single elements take, forced for whole buffers (HCCL_AMD_REDUCE_VECTOR=0)."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_VECTOR", "0")
+    w = World(5)                                     # the variable is read when the world is created
+    monkeypatch.delenv("HCCL_AMD_REDUCE_VECTOR")
+    try:
+        for dtype in REDUCE_TYPES:
+            for op in (SUM, PROD, MAX, MIN):
+                if op == PROD and dtype in (DT.INT16, DT.BFP16):
+                    continue
+                run_all_reduce(w, dtype, op, 1_237, "mesh", seed=900 + int(dtype) * 4 + op)
+            run_reduce_scatter(w, dtype, SUM, 333, "nhr", seed=950 + int(dtype))
+            run_all_reduce(w, dtype, MAX, 515, "rhd", seed=960 + int(dtype))
+    finally:
+        w.close()
