@@ -451,11 +451,6 @@ HcclResult EnsureA2aBuffers(World* w)
     return HCCL_SUCCESS;
 }
 
-uint32_t AlignUnitOf(uint64_t bits)
-{
-    uint32_t low = static_cast<uint32_t>(bits) | 16u;
-    return low & (0u - low);
-}
 
 // ---------------------------------------------------------------------------------------------
 // Launches.  `s` is the stream the fused kernel runs on.
@@ -604,9 +599,6 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
 
 HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
 {
-    uint64_t bits = 0;
-    for (uint32_t d = 0; d < b.nDst; ++d) bits |= reinterpret_cast<uint64_t>(b.dst[d]);
-    b.unit = AlignUnitOf(bits);
     // One wavefront per tile is fastest with a single destination; with several, the stores of a
     // larger tile keep more of each destination's pages busy at a time.
     const uint32_t tileBytes = w->copyTileBytes != 0 ? w->copyTileBytes : (b.nDst == 1 ? 1024u : 4096u);

@@ -70,13 +70,6 @@ __device__ __forceinline__ uint32_t FindSegment(uint32_t tile, uint32_t shift, H
     return lo;
 }
 
-__device__ __forceinline__ uint32_t AlignUnit(uint64_t bits)
-{
-    // largest power of two <= 16 dividing `bits`
-    uint32_t low = static_cast<uint32_t>(bits) | 16u;
-    return low & (0u - low);
-}
-
 // Four output dwords from five input dwords, dropping `shift` (0..3) leading bytes.
 __device__ __forceinline__ U32x4 Funnel(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3, uint32_t w4, uint32_t shift)
 {
@@ -112,8 +105,10 @@ __device__ __forceinline__ U32x4 NextLane(U32x4 v, U32x4 last)
     return r;
 }
 
-// Copies one tile (bytes <= T * 16) from src to dstOf(d), d < nDst, one 16-byte vector per lane.  Every
-// dstOf(d) has the same offset from a 16-byte boundary.  Must be called by all T threads of the workgroup.
+// Copies one tile (bytes <= T * 16) from src to dstOf(d), d < nDst, one 16-byte vector per lane.  The stores
+// to dstOf(0) are 16-byte aligned; those to the other destinations are too when they share its offset from a
+// 16-byte boundary (the usual case) and are unaligned 128-bit stores otherwise.  Must be called by all T
+// threads of the workgroup.
 template <int T, int MODE, class DstFn>
 __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uint32_t nDst, DstFn dstOf)
 {
@@ -178,20 +173,6 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
     }
 }
 
-// Fallback when destinations differ in alignment: lane-per-unit copies of the widest common unit.
-template <int T, typename U, class DstFn>
-__device__ __forceinline__ void CopyUnits(const uint8_t* src, uint32_t bytes, uint32_t nDst, DstFn dstOf)
-{
-    const uint32_t n = bytes / sizeof(U);
-    const U* s = reinterpret_cast<const U*>(src);
-    for (uint32_t i = threadIdx.x; i < n; i += T) {
-        U v = LoadNt<U>(s + i);
-        for (uint32_t d = 0; d < nDst; ++d) {
-            StoreNt(v, reinterpret_cast<U*>(dstOf(d)) + i);
-        }
-    }
-}
-
 // ---- AllGather / AllGatherV --------------------------------------------------------------------
 // Workgroup b copies tile b of the segment list held in the kernel arguments.
 template <int T, int MODE>
@@ -209,20 +190,7 @@ __global__ __launch_bounds__(T) void BcastCopyKernel(const BcastCopyArgs args)
     const uint8_t* src = static_cast<const uint8_t*>(args.src[seg]) + off;
     const uint64_t dOff = args.dstOff[seg] + off;
     auto dstOf = [&](uint32_t d) { return static_cast<uint8_t*>(args.dst[d]) + dOff; };
-    if (MODE != COPY_GENERAL || args.unit == 16) {   // destination bases are all 16-byte aligned, hence congruent
-        CopyTile<T, MODE>(src, bytes, args.nDst, dstOf);
-    } else {
-        const uint32_t unit = AlignUnit(reinterpret_cast<uint64_t>(args.src[seg]) | len | args.dstOff[seg] | args.unit);
-        if (unit >= 8) {
-            CopyUnits<T, uint64_t>(src, bytes, args.nDst, dstOf);
-        } else if (unit == 4) {
-            CopyUnits<T, uint32_t>(src, bytes, args.nDst, dstOf);
-        } else if (unit == 2) {
-            CopyUnits<T, uint16_t>(src, bytes, args.nDst, dstOf);
-        } else {
-            CopyUnits<T, uint8_t>(src, bytes, args.nDst, dstOf);
-        }
-    }
+    CopyTile<T, MODE>(src, bytes, args.nDst, dstOf);
 }
 
 // ---- AlltoAllV -------------------------------------------------------------------------------------
@@ -275,10 +243,14 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
 {
     BcastCopyArgs a = in;
     uint64_t tiles = 0;
-    uint64_t misfit = 0;      // non-zero low bits: some segment is not 16-byte aligned on both sides
-    bool congruent = a.unit == 16;
+    uint64_t misfit = 0;      // non-zero low bits: something is not 16-byte aligned
+    bool congruent = true;    // every segment's source shares the offset of its first destination
+    for (uint32_t d = 0; d < a.nDst; ++d) {
+        misfit |= reinterpret_cast<uint64_t>(a.dst[d]);
+    }
+    const uint64_t dst0 = reinterpret_cast<uint64_t>(a.dst[0]);
     for (uint32_t j = 0; j < a.nSeg; ++j) {
-        tiles += TilesOf(a.len[j], reinterpret_cast<uint64_t>(a.dst[0]) + a.dstOff[j], tileBytes);
+        tiles += TilesOf(a.len[j], dst0 + a.dstOff[j], tileBytes);
         if (tiles > 0x7FFFFFF0ull) {
             return hipErrorInvalidValue;
         }
@@ -286,7 +258,7 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
         if (a.len[j] != 0) {
             const uint64_t s = reinterpret_cast<uint64_t>(a.src[j]);
             misfit |= s | a.dstOff[j] | a.len[j];
-            congruent = congruent && ((s ^ a.dstOff[j]) & 15u) == 0;
+            congruent = congruent && ((s ^ (dst0 + a.dstOff[j])) & 15u) == 0;
         }
     }
     if (tiles == 0) {

@@ -153,7 +153,6 @@ struct BcastCopyArgs {
     uint64_t dstOff[kMaxRanks];
     uint32_t nSeg;
     uint32_t nDst;
-    uint32_t unit;        // widest power of two (<= 16) dividing every destination base address
     uint32_t hintShift;
     uint32_t tileEnd[kMaxRanks];
     uint8_t hint[kBcastHintMax + 8];

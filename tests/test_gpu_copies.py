@@ -205,3 +205,39 @@ def test_one_host_thread_per_rank_with_own_streams():
     assert not errors, errors
     for r in range(n):
         assert np.array_equal(results[r].view(np.uint32), want.view(np.uint32)), r
+
+
+def test_all_gather_and_broadcast_into_differently_aligned_buffers():
+    """Every rank's buffers sit at their own offset from a 16-byte boundary: the stores to all but the first
+    destination are unaligned 128-bit stores."""
+    import hccl_amd
+    n, count = 6, 33_333
+    w = World(n)
+    try:
+        rng = np.random.default_rng(404)
+        ins = [rand_bytes(rng, count * 2) for _ in range(n)]
+        want = [np.zeros(n * count * 2, dtype=np.uint8) for _ in range(n)]
+        assert oracle.all_gather(ins, want, count, int(DT.FP16)) == 0
+        sends = [to_dev(x, (2 * r) % 16) for r, x in enumerate(ins)]
+        recvs = [dev_zeros(n * count * 2, (6 * r + 2) % 16) for r in range(n)]
+        w.all_gather(sends, recvs, count, DT.FP16)
+        for r in range(n):
+            assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), r
+        counts = np.array([100, 0, 7_777, 1, 40_001, 16], dtype=np.uint64)
+        displs = np.array([3, 0, 200, 150, 9_000, 120], dtype=np.uint64)
+        total = 50_000
+        vins = [rand_bytes(rng, max(int(c), 1)) for c in counts]
+        vwant = [np.full(total, FILL, dtype=np.uint8) for _ in range(n)]
+        assert oracle.all_gather_v([x[:int(c)] for x, c in zip(vins, counts)], vwant, counts, displs, int(DT.UINT8)) == 0
+        sends = [to_dev(x, (3 * r) % 16) for r, x in enumerate(vins)]
+        recvs = [dev_zeros(total, (5 * r + 1) % 16, fill=FILL) for r in range(n)]
+        w.all_gather_v(sends, recvs, counts, displs, DT.UINT8)
+        for r in range(n):
+            assert np.array_equal(to_host(recvs[r], np.uint8), vwant[r]), r
+        bufs = [to_dev(rand_bytes(rng, 70_001), (7 * r) % 16) for r in range(n)]
+        src = to_host(bufs[4], np.uint8)
+        w.broadcast(bufs, 70_001, DT.UINT8, 4)
+        for r in range(n):
+            assert np.array_equal(to_host(bufs[r], np.uint8), src), r
+    finally:
+        w.close()
