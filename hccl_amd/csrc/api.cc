@@ -488,6 +488,16 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     a.threads = w->reduceThreads != 0 ? w->reduceThreads : (plan.maxDepth > 1 ? 128u : 64u);
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
     uint64_t blocks = subs * a.blocksPerSub;
+    if (a.varGroups) {
+        // every group gets the workgroups its own length needs (an empty group gets none)
+        blocks = 0;
+        for (uint32_t g = 0; g < a.nGroup; ++g) {
+            if (a.groupLenV[g] != 0) {
+                blocks += BlocksPerSub(w, a.groupLenV[g], a.vecOk ? esz : 16, subs, a.threads);
+            }
+            a.groupBlockEnd[g] = static_cast<uint32_t>(blocks < 0x7FFFFFFFull ? blocks : 0x7FFFFFFFull);
+        }
+    }
     if (blocks == 0 || blocks > 0x7FFFFFFFull) {
         return HCCL_E_INTERNAL;
     }

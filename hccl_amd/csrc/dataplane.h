@@ -75,8 +75,10 @@ struct ReduceArgs {
     uint32_t writeThrough;   // 16-byte results leave through StoreStream16 instead of a non-temporal store
     // Groups of unequal length (ReduceScatterV): when varGroups is set, group g spans groupLenV[g]
     // elements starting groupOffV[g] elements into every source, instead of the uniform
-    // groupLen / srcGroupStride / total geometry; groupLen then only sizes the grid.
+    // groupLen / srcGroupStride / total geometry, and owns the workgroups
+    // [groupBlockEnd[g-1], groupBlockEnd[g]) of the grid (filled by the launcher's caller).
     uint32_t varGroups;
+    uint32_t groupBlockEnd[kMaxRanks];
     uint64_t groupOffV[kMaxRanks];
     uint64_t groupLenV[kMaxRanks];
 };

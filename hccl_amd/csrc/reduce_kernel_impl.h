@@ -531,17 +531,34 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     __shared__ BlockProgram bp;
     extern __shared__ uint32_t accStack[];
 
-    const uint32_t sub = blockIdx.x / args.blocksPerSub;
-    const uint32_t blk = blockIdx.x - sub * args.blocksPerSub;
-    const uint32_t g = sub / args.nSub;
-    const uint32_t c = sub - g * args.nSub;
-
+    uint32_t g, c, blk, blocksHere;   // group, sub-segment, this workgroup's index among the blocksHere of it
     uint64_t gLen;
     uint64_t gSrc;
     if (args.varGroups) {
+        // Groups of unequal length own unequal shares of the grid: first group whose last block is not before us.
+        uint32_t lo = 0;
+        uint32_t hi = args.nGroup - 1;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (blockIdx.x >= args.groupBlockEnd[mid]) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        g = lo;
+        c = 0;
+        const uint32_t firstBlock = g == 0 ? 0u : args.groupBlockEnd[g - 1];
+        blk = blockIdx.x - firstBlock;
+        blocksHere = args.groupBlockEnd[g] - firstBlock;
         gLen = args.groupLenV[g];
         gSrc = args.groupOffV[g];
     } else {
+        const uint32_t sub = blockIdx.x / args.blocksPerSub;
+        blk = blockIdx.x - sub * args.blocksPerSub;
+        blocksHere = args.blocksPerSub;
+        g = sub / args.nSub;
+        c = sub - g * args.nSub;
         const uint64_t gBeg = static_cast<uint64_t>(g) * args.groupLen;
         if (gBeg >= args.total) {
             return;
@@ -572,7 +589,7 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     }
     __syncthreads();
 
-    const uint64_t stride = static_cast<uint64_t>(args.blocksPerSub) * args.threads;
+    const uint64_t stride = static_cast<uint64_t>(blocksHere) * args.threads;
     const uint64_t first = static_cast<uint64_t>(blk) * args.threads + threadIdx.x;
 
     // When vecOk, `head` elements bring the stores to the first destination onto a 16-byte boundary, a 128-bit
