@@ -609,10 +609,7 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
 
 HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
 {
-    // One wavefront per tile is fastest with a single destination; with several, the stores of a
-    // larger tile keep more of each destination's pages busy at a time.
-    const uint32_t tileBytes = w->copyTileBytes != 0 ? w->copyTileBytes : (b.nDst == 1 ? 1024u : 4096u);
-    HIP_OK(LaunchBcastCopy(b, tileBytes, s));
+    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s));   // 0: the launcher picks the tile
     return HCCL_SUCCESS;
 }
 

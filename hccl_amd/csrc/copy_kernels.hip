@@ -242,7 +242,6 @@ hipError_t LaunchA2aT(const A2aArgs& a, uint32_t tiles, hipStream_t stream)
 hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStream_t stream)
 {
     BcastCopyArgs a = in;
-    uint64_t tiles = 0;
     uint64_t misfit = 0;      // non-zero low bits: something is not 16-byte aligned
     bool congruent = true;    // every segment's source shares the offset of its first destination
     for (uint32_t d = 0; d < a.nDst; ++d) {
@@ -250,23 +249,31 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
     }
     const uint64_t dst0 = reinterpret_cast<uint64_t>(a.dst[0]);
     for (uint32_t j = 0; j < a.nSeg; ++j) {
-        tiles += TilesOf(a.len[j], dst0 + a.dstOff[j], tileBytes);
-        if (tiles > 0x7FFFFFF0ull) {
-            return hipErrorInvalidValue;
-        }
-        a.tileEnd[j] = static_cast<uint32_t>(tiles);
         if (a.len[j] != 0) {
             const uint64_t s = reinterpret_cast<uint64_t>(a.src[j]);
             misfit |= s | a.dstOff[j] | a.len[j];
             congruent = congruent && ((s ^ (dst0 + a.dstOff[j])) & 15u) == 0;
         }
     }
+    const uint32_t mode = !congruent ? COPY_GENERAL : ((misfit & 15u) == 0 ? COPY_ALIGNED : COPY_CONGRUENT);
+    if (tileBytes == 0) {
+        // One wavefront per tile, except where lanes realign their source for several destinations: there the
+        // larger workgroup measured 1-2 % faster.
+        tileBytes = (mode == COPY_GENERAL && a.nDst > 1) ? 4096u : 1024u;
+    }
+    uint64_t tiles = 0;
+    for (uint32_t j = 0; j < a.nSeg; ++j) {
+        tiles += TilesOf(a.len[j], dst0 + a.dstOff[j], tileBytes);
+        if (tiles > 0x7FFFFFF0ull) {
+            return hipErrorInvalidValue;
+        }
+        a.tileEnd[j] = static_cast<uint32_t>(tiles);
+    }
     if (tiles == 0) {
         return hipSuccess;
     }
     uint32_t nHint = 0;
     a.hintShift = BuildTileHints(a.tileEnd, a.nSeg, static_cast<uint32_t>(tiles), kBcastHintMax, a.hint, &nHint);
-    const uint32_t mode = !congruent ? COPY_GENERAL : ((misfit & 15u) == 0 ? COPY_ALIGNED : COPY_CONGRUENT);
     const uint32_t nTiles = static_cast<uint32_t>(tiles);
     switch (tileBytes) {
         case 1024: return LaunchBcastT<64>(a, mode, nTiles, stream);

@@ -182,6 +182,7 @@ inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
     // eight fp32 accumulators (half SUM) or sixteen 16-bit ones (int8) vs one 16-byte pack
     return ((half && op == HCCL_REDUCE_SUM) || dtype == HCCL_DATA_TYPE_INT8) ? 32u : 16u;
 }
+// tileBytes: 1024, 4096 or 16384; 0 lets the launcher choose.
 hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream);
 hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, uint32_t tileBytes, hipStream_t stream);
 
