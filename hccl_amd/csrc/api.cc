@@ -480,12 +480,13 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
         uint64_t last = a.groupLen > before ? a.groupLen - before : 0;
         longest = last > a.subLen ? last : a.subLen;
     }
-    // Small workgroups retire sooner and keep the window of addresses in flight compact; nested fold
-    // programs park accumulators in LDS and want a few more lanes per workgroup to hide that.
+    // One wavefront per workgroup: a wavefront needs nothing from its neighbours (the fold program is read
+    // with scalar loads, no barrier), small workgroups retire sooner and keep the window of addresses in
+    // flight compact.  Measured best for flat and nested programs alike.
     // Results of a reduce leave through non-temporal stores: measured equal to write-through stores with one
     // result stream and 2-3 % better with sixteen.  (The copy kernels always write through.)
     a.writeThrough = w->storePolicy == 1 ? 1u : 0u;
-    a.threads = w->reduceThreads != 0 ? w->reduceThreads : (plan.maxDepth > 1 ? 128u : 64u);
+    a.threads = w->reduceThreads != 0 ? w->reduceThreads : 64u;
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
     uint64_t blocks = subs * a.blocksPerSub;
     if (a.varGroups) {

@@ -271,12 +271,28 @@ __device__ __forceinline__ uint64_t Uniform64(uint64_t v)
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
-// Per-block view of the program: leaf i is read at leafPtr[i] (the rank's buffer already advanced to
-// this sub-segment) and carries ctl[i] (see kCtlOpen).
-struct BlockProgram {
-    uint64_t leafPtr[kMaxRanks];
-    uint8_t ctl[kMaxRanks];
+// The fold program of this workgroup's sub-segment, read with scalar loads only (the image sits in device
+// memory, 16-byte aligned; see kDevProgRankOff / kDevProgCtlOff): leaf i folds rank RankOf(i) and carries
+// CtlOf(i) (see kCtlOpen).  srcByteOff advances every rank's buffer to the sub-segment.
+typedef const uint32_t __attribute__((address_space(4))) * ProgWords;
+struct ProgramView {
+    ProgWords words;       // the program image as dwords
+    uint64_t srcByteOff;
     uint32_t nLeaves;
+};
+
+// Byte `i` (static) of the 16 table bytes that start at byte offset `off` (a multiple of 16) of the image.
+template <int kBytes>
+struct TableBytes {
+    uint32_t w[kBytes / 4];
+    __device__ __forceinline__ void Load(ProgWords words, uint32_t off)
+    {
+#pragma unroll
+        for (int k = 0; k < kBytes / 4; ++k) {
+            w[k] = words[off / 4 + k];
+        }
+    }
+    __device__ __forceinline__ uint32_t operator[](int i) const { return (w[i / 4] >> (8 * (i % 4))) & 0xFFu; }
 };
 
 // Leaves whose loads are issued together: sixteen vectors, or eight single elements.
@@ -284,6 +300,12 @@ template <typename S, int W>
 __device__ constexpr int LoadBatch()
 {
     return W > 1 ? 16 : 8;
+}
+
+// The same for eight uniform 64-bit values (leaf addresses): all of them exist before the first is used.
+__device__ __forceinline__ void ScalarFence8(uint64_t* r)
+{
+    asm volatile("" : "+s"(r[0]), "+s"(r[1]), "+s"(r[2]), "+s"(r[3]), "+s"(r[4]), "+s"(r[5]), "+s"(r[6]), "+s"(r[7]));
 }
 
 // Makes eight loaded vectors opaque to the optimiser at this point of the instruction stream.
@@ -443,7 +465,7 @@ struct PackOps<E, 16, typename E::Swar> {
 // Evaluates the whole tree for the W elements at element offset `e` of the sub-segment.  Leaves are
 // taken a batch at a time: their loads are all issued before the first fold, whatever the tree shape.
 template <class E, int W>
-__device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stack, const ReduceArgs& args,
+__device__ __forceinline__ void ReduceOne(const ProgramView& pv, uint32_t* stack, const ReduceArgs& args,
                                           uint64_t e, uint64_t dstOff, uint32_t group)
 {
     using S = typename E::S;
@@ -454,9 +476,27 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
     }
     uint32_t level = 0;
     bool init = true;   // the next leaf starts a level instead of being folded into it
-    const uint32_t nLeaves = bp.nLeaves;
+    const uint32_t nLeaves = pv.nLeaves;
     constexpr int kBatch = LoadBatch<S, W>();
     for (uint32_t b = 0; b < nLeaves; b += kBatch) {
+        TableBytes<kBatch> ranks, ctls;
+        ranks.Load(pv.words, kDevProgRankOff + b);
+        ctls.Load(pv.words, kDevProgCtlOff + b);
+        // Leaf addresses first and unconditionally (table bytes past the last leaf name rank 0), so that their
+        // scalar loads go out together instead of one wait per leaf.
+        uint64_t leaf[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            leaf[i] = reinterpret_cast<uint64_t>(args.src[ranks[i]]);
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; i += 8) {
+            ScalarFence8(leaf + i);
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            leaf[i] += pv.srcByteOff;
+        }
         Pack<S, W> v[kBatch];
         if constexpr (sizeof(S) * W == 16) {
             // The vectors stay untyped 128-bit values until the whole batch has been issued: nothing may
@@ -467,7 +507,7 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
 #pragma unroll
             for (int i = 0; i < kBatch; ++i) {
                 if (b + i < nLeaves) {
-                    const S* p = reinterpret_cast<const S*>(Uniform64(bp.leafPtr[b + i])) + e;
+                    const S* p = reinterpret_cast<const S*>(leaf[i]) + e;
                     raw[i] = __builtin_nontemporal_load((const HCCL_AMD_GLOBAL U32x4Unaligned*)p);
                 }
             }
@@ -483,15 +523,14 @@ __device__ __forceinline__ void ReduceOne(const BlockProgram& bp, uint32_t* stac
 #pragma unroll
             for (int i = 0; i < kBatch; ++i) {
                 if (b + i < nLeaves) {
-                    const void* base = reinterpret_cast<const void*>(Uniform64(bp.leafPtr[b + i]));
-                    v[i] = LoadPack<S, W>(base, e);
+                    v[i] = LoadPack<S, W>(reinterpret_cast<const void*>(leaf[i]), e);
                 }
             }
         }
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
             if (b + i < nLeaves) {
-                const uint32_t ctl = Uniform(bp.ctl[b + i]);
+                const uint32_t ctl = ctls[i];
                 if (ctl & kCtlOpen) {
                     PushAcc<E, W>(stack, args.threads, level, acc);
                     ++level;
@@ -528,7 +567,6 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
 {
     using S = typename E::S;
     constexpr int W = 16 / sizeof(S);
-    __shared__ BlockProgram bp;
     extern __shared__ uint32_t accStack[];
 
     uint32_t g, c, blk, blocksHere;   // group, sub-segment, this workgroup's index among the blocksHere of it
@@ -576,18 +614,11 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     const uint64_t srcOff = gSrc + sBeg;
     const uint64_t dstOff = args.dstOwn ? sBeg : static_cast<uint64_t>(g) * args.dstGroupStride + sBeg;
 
-    // Resolve the program once per block: leaf -> address of this sub-segment in that rank's buffer.
-    const uint8_t* prog = args.prog + static_cast<uint64_t>(g * args.progGroupStride + c * args.progSubStride) * kDevProgBytes;
-    const uint32_t nLeaves = prog[0];
-    if (threadIdx.x < nLeaves) {
-        const uint32_t rank = prog[kDevProgRankOff + threadIdx.x];
-        bp.leafPtr[threadIdx.x] = reinterpret_cast<uint64_t>(args.src[rank]) + srcOff * sizeof(S);
-        bp.ctl[threadIdx.x] = prog[kDevProgCtlOff + threadIdx.x];
-    }
-    if (threadIdx.x == 0) {
-        bp.nLeaves = nLeaves;
-    }
-    __syncthreads();
+    ProgramView pv;
+    pv.words = (ProgWords)(uintptr_t)(args.prog + static_cast<uint64_t>(g * args.progGroupStride + c * args.progSubStride) *
+                                                      kDevProgBytes);
+    pv.srcByteOff = srcOff * sizeof(S);
+    pv.nLeaves = pv.words[0] & 0xFFu;
 
     const uint64_t stride = static_cast<uint64_t>(blocksHere) * args.threads;
     const uint64_t first = static_cast<uint64_t>(blk) * args.threads + threadIdx.x;
@@ -611,14 +642,14 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     }
     for (uint64_t u = first; u < nVec + lead; u += stride) {
         if (u >= lead) {
-            ReduceOne<E, W>(bp, accStack, args, head + (u - lead) * W, dstOff, g);
+            ReduceOne<E, W>(pv, accStack, args, head + (u - lead) * W, dstOff, g);
         }
     }
     const uint64_t bodyEnd = head + nVec * W;
     const uint64_t nScalar = head + (len - bodyEnd);
     for (uint64_t i = first; i < nScalar; i += stride) {
         const uint64_t e = i < head ? i : i - head + bodyEnd;
-        ReduceOne<E, 1>(bp, accStack, args, e, dstOff, g);
+        ReduceOne<E, 1>(pv, accStack, args, e, dstOff, g);
     }
 }
 
