@@ -32,7 +32,7 @@ def parse_args():
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3max", "c3prod", "c4", "c5a", "c5b", "copycal", "rsv", "reduce", "bcast", "scatter",
                              "a2a"])
     ap.add_argument("--algo", default=None, help="override the algorithm of the workload (mesh/ring/rhd/nhr/...)")
-    ap.add_argument("--others", action="store_true", help="also time the other BASELINE configurations")
+    ap.add_argument("--others", action="store_true", help="also time the other benchmark configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
@@ -155,7 +155,7 @@ class Workloads:
 
         return step, 2 * nbytes, nbytes, 1.0, (src, dst), "plain copy 1 GiB (rankSize=1 AllGather)", "u8", 1
 
-    # ---- the entry points that marshal onto the same kernels (not BASELINE configurations) ----------
+    # ---- the entry points that marshal onto the same kernels (not among the five benchmark configurations) ----------
     def rsv(self, algo):
         """ReduceScatterV bf16, 8 ranks, uneven slices between 8 Mi and 24 Mi elements (16-byte aligned starts)."""
         import numpy as np

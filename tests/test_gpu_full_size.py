@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes.  The CPU oracle would take minutes there, so the
+"""The five benchmark configurations at their full sizes.  The CPU oracle would take minutes there, so the
 results are checked on the GPU through properties that do not depend on size: the reduction is recomputed
 slice by slice with torch in the association order the algorithm fixes (fp32 accumulate, one rounding),
 integer reductions against torch's exact integer ops, AlltoAllV by a round trip through its inverse plus

@@ -194,7 +194,7 @@ def test_unaligned_buffers_and_in_place(world8):
 
 
 # ---------------------------------------------------------------------------------------------
-# BASELINE configurations (C1 at its real size; the others at sizes the oracle finishes in seconds;
+# The benchmark configurations (C1 at its real size; the others at sizes the oracle finishes in seconds;
 # their full sizes are covered by tests/test_gpu_full_size.py through size-independent properties)
 # ---------------------------------------------------------------------------------------------
 def test_config1_all_reduce_fp32_n8_rank_order(world8):
