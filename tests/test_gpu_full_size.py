@@ -164,3 +164,79 @@ def test_config4_all_to_all_v_moe_full_size_round_trip():
             assert torch.equal(back[r], sends[r]), r
     finally:
         w.close()
+
+
+def test_reduce_scatter_v_uneven_slices_full_size():
+    import torch
+    n = 8
+    w = World(n)
+    try:
+        rng = np.random.default_rng(0xC0FFEE + 6000)
+        counts = (rng.integers(1 << 20, 3 << 20, n) * 8).astype(np.uint64)
+        counts[3] += 5                                     # one slice that ends off a 16-byte boundary
+        displs = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.uint64)
+        total = int(counts.sum())
+        sends = [torch.randn(total, generator=gen(6100 + r), device="cuda", dtype=torch.bfloat16) for r in range(n)]
+        recvs = [torch.empty(int(c), dtype=torch.bfloat16, device="cuda") for c in counts]
+        w.reduce_scatter_v(sends, recvs, counts, displs, DT.BFP16, OP.SUM)
+        for k in range(n):
+            lo, c = int(displs[k]), int(counts[k])
+            want = sends[k][lo:lo + c].float()               # own slice first, then ranks ascending, fp32
+            for t in range(n):
+                if t != k:
+                    want = sends[t][lo:lo + c].float() + want
+            assert torch.equal(recvs[k].view(torch.int16), want.bfloat16().view(torch.int16)), k
+            del want
+    finally:
+        w.close()
+
+
+def test_reduce_then_broadcast_equals_all_reduce_full_size():
+    import torch
+    n, count, root = 8, 1 << 26, 3
+    w = World(n)
+    try:
+        sends = [torch.randn(count, generator=gen(6200 + r), device="cuda", dtype=torch.float32) for r in range(n)]
+        recvs = [torch.full((count,), -1.0, dtype=torch.float32, device="cuda") for _ in range(n)]
+        w.reduce(sends, recvs, count, DT.FP32, OP.SUM, root)
+        want = sends[0].clone()
+        for r in range(1, n):
+            want = sends[r] + want                           # rank order, bit exact in fp32
+        assert torch.equal(recvs[root].view(torch.int32), want.view(torch.int32))
+        assert all(bool((recvs[r] == -1.0).all()) for r in range(n) if r != root)
+        w.broadcast(recvs, count, DT.FP32, root)
+        for r in range(n):
+            assert torch.equal(recvs[r].view(torch.int32), want.view(torch.int32)), r
+        allr = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(n)]
+        w.all_reduce(sends, allr, count, DT.FP32, OP.SUM, "mesh")
+        assert torch.equal(allr[5].view(torch.int32), want.view(torch.int32))
+    finally:
+        w.close()
+
+
+def test_scatter_and_all_to_all_full_size():
+    import torch
+    n = 16
+    w = World(n)
+    try:
+        count = 1 << 22
+        sends = [torch.randint(-32768, 32767, (n * count,), generator=gen(6500 + r), device="cuda", dtype=torch.int16)
+                 for r in range(n)]
+        recvs = [torch.empty(n * count, dtype=torch.int16, device="cuda") for _ in range(n)]
+        w.all_to_all(sends, recvs, count, DT.BFP16)
+        for i in (0, 7, 15):
+            got = recvs[i].view(n, count)
+            for j in range(n):
+                assert torch.equal(got[j], sends[j].view(n, count)[i]), (i, j)
+        # applying the exchange twice is the identity (a block transpose)
+        back = [torch.empty(n * count, dtype=torch.int16, device="cuda") for _ in range(n)]
+        w.all_to_all(recvs, back, count, DT.BFP16)
+        for r in range(n):
+            assert torch.equal(back[r], sends[r]), r
+        root = 9
+        outs = [torch.empty(count, dtype=torch.int16, device="cuda") for _ in range(n)]
+        w.scatter([sends[r] if r == root else None for r in range(n)], outs, count, DT.INT16, root)
+        for r in range(n):
+            assert torch.equal(outs[r], sends[root].view(n, count)[r]), r
+    finally:
+        w.close()
