@@ -229,7 +229,7 @@ struct World {
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
     bool reduceVector = true;
-    uint32_t storePolicy = 0;     // HCCL_AMD_STORE_POLICY for the reduce kernel: 0 non-temporal, 1 write-through
+    uint32_t storePolicy = 2;     // HCCL_AMD_STORE_POLICY for the reduce kernel: 0 non-temporal, 1 write-through, 2 per launch
     // HCCL_DETERMINISTIC (reference alg_env_config.cc:1113-1153): 0 false, 1 true, 2 strict, 0xFF unparsable
     uint8_t deterministic = 0;
     // Longest a rank waits on the host for its peers: the reference's CUSTOM_TIMEOUT = 1836 s (alg_param.h:91),
@@ -327,7 +327,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->copyTileBytes = 0;
     }
     w->execTimeout = EnvU32("HCCL_EXEC_TIMEOUT", 1836);
-    w->storePolicy = EnvU32("HCCL_AMD_STORE_POLICY", 0) == 1 ? 1 : 0;
+    w->storePolicy = EnvU32("HCCL_AMD_STORE_POLICY", 2);
+    if (w->storePolicy > 2) {
+        w->storePolicy = 2;
+    }
     w->reduceVector = EnvU32("HCCL_AMD_REDUCE_VECTOR", 1) != 0;
     ApplyAlgoEnv(w.get());
     if (const char* det = getenv("HCCL_DETERMINISTIC")) {
@@ -483,9 +486,10 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     // One wavefront per workgroup: a wavefront needs nothing from its neighbours (the fold program is read
     // with scalar loads, no barrier), small workgroups retire sooner and keep the window of addresses in
     // flight compact.  Measured best for flat and nested programs alike.
-    // Results of a reduce leave through non-temporal stores: measured equal to write-through stores with one
-    // result stream and 2-3 % better with sixteen.  (The copy kernels always write through.)
-    a.writeThrough = w->storePolicy == 1 ? 1u : 0u;
+    // A result that is written once (ReduceScatter(V), Reduce) leaves through write-through stores, 3-4 % faster
+    // than non-temporal ones next to eight read streams; results written to many destinations (AllReduce)
+    // keep non-temporal stores, 2-3 % faster there.  HCCL_AMD_STORE_POLICY = 0 / 1 forces one of them.
+    a.writeThrough = w->storePolicy != 2 ? w->storePolicy : ((a.dstOwn || a.nDst == 1) ? 1u : 0u);
     a.threads = w->reduceThreads != 0 ? w->reduceThreads : 64u;
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
     uint64_t blocks = subs * a.blocksPerSub;
