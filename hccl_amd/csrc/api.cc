@@ -225,7 +225,7 @@ struct World {
     hipEvent_t a2aSlotFree[kStagingSlots] = {};
     bool a2aSlotUsed[kStagingSlots] = {};
     uint32_t a2aNext = 0;
-    uint32_t reduceBlocks = 1u << 20;
+    uint32_t reduceBlocks = 1u << 26;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
     bool reduceVector = true;
@@ -317,7 +317,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (hipGetDevice(&w->device) != hipSuccess) {
         w->device = 0;
     }
-    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 1u << 20);
+    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 1u << 26);
     w->reduceThreads = EnvU32("HCCL_AMD_REDUCE_THREADS", 0);
     if (w->reduceThreads != 64 && w->reduceThreads != 128 && w->reduceThreads != 256) {
         w->reduceThreads = 0;

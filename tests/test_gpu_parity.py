@@ -336,3 +336,39 @@ def test_element_by_element_path_for_every_type(monkeypatch):
             run_all_reduce(w, dtype, MAX, 515, "rhd", seed=960 + int(dtype))
     finally:
         w.close()
+
+
+def test_workgroups_that_loop_over_several_positions(monkeypatch):
+    """With the grid capped (HCCL_AMD_REDUCE_BLOCKS) every workgroup strides over many vector positions."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_BLOCKS", "7")
+    w = World(6)
+    monkeypatch.delenv("HCCL_AMD_REDUCE_BLOCKS")
+    try:
+        run_all_reduce(w, DT.FP32, SUM, 70_001, "mesh", seed=1)
+        run_all_reduce(w, DT.BFP16, SUM, 50_003, "rhd", seed=2)
+        run_all_reduce(w, DT.FP16, MAX, 33_333, "nhr", seed=3, pad=2)
+        run_reduce_scatter(w, DT.INT8, SUM, 20_011, "ring", seed=4)
+        run_reduce_scatter(w, DT.INT32, PROD, 9_999, "aiv_mesh", seed=5)
+    finally:
+        w.close()
+
+
+def test_all_reduce_larger_than_a_million_workgroups():
+    """2 x 1 GiB of fp16 per rank: 2^26 vector positions, one per lane, 2^20 workgroups per destination."""
+    import torch
+    n, count = 2, 1 << 29
+    w = World(n)
+    try:
+        g = torch.Generator(device="cuda")
+        g.manual_seed(99)
+        sends = [torch.randn(count, generator=g, device="cuda", dtype=torch.float16) for _ in range(n)]
+        recvs = [torch.empty(count, dtype=torch.float16, device="cuda") for _ in range(n)]
+        w.all_reduce(sends, recvs, count, DT.FP16, OP.SUM, "mesh")
+        step = 1 << 27
+        for lo in range(0, count, step):
+            want = (sends[1][lo:lo + step].float() + sends[0][lo:lo + step].float()).half()
+            for r in range(n):
+                assert torch.equal(recvs[r][lo:lo + step].view(torch.int16), want.view(torch.int16)), (lo, r)
+            del want
+    finally:
+        w.close()
