@@ -229,6 +229,7 @@ struct World {
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
     bool reduceVector = true;
+    uint32_t reduceBatch = 0;     // HCCL_AMD_REDUCE_BATCH: 8 or 16, 0 = per launch
     uint32_t storePolicy = 2;     // HCCL_AMD_STORE_POLICY for the reduce kernel: 0 non-temporal, 1 write-through, 2 per launch
     // HCCL_DETERMINISTIC (reference alg_env_config.cc:1113-1153): 0 false, 1 true, 2 strict, 0xFF unparsable
     uint8_t deterministic = 0;
@@ -332,6 +333,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->storePolicy = 2;
     }
     w->reduceVector = EnvU32("HCCL_AMD_REDUCE_VECTOR", 1) != 0;
+    w->reduceBatch = EnvU32("HCCL_AMD_REDUCE_BATCH", 0);
+    if (w->reduceBatch != 8 && w->reduceBatch != 16) {
+        w->reduceBatch = 0;
+    }
     ApplyAlgoEnv(w.get());
     if (const char* det = getenv("HCCL_DETERMINISTIC")) {
         std::string v(det);
@@ -490,6 +495,9 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     // than non-temporal ones next to eight read streams; results written to many destinations (AllReduce)
     // keep non-temporal stores, 2-3 % faster there.  HCCL_AMD_STORE_POLICY = 0 / 1 forces one of them.
     a.writeThrough = w->storePolicy != 2 ? w->storePolicy : ((a.dstOwn || a.nDst == 1) ? 1u : 0u);
+    // Up to eight ranks folded into one result stream run best with eight-load batches (fewer registers, more
+    // wavefronts in flight: +1-2 %); AllReduce's many result streams and larger worlds with sixteen (+5 %).
+    a.vecBatch = w->reduceBatch != 0 ? w->reduceBatch : ((w->n <= 8 && (a.dstOwn || a.nDst == 1)) ? 8u : 16u);
     a.threads = w->reduceThreads != 0 ? w->reduceThreads : 64u;
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
     uint64_t blocks = subs * a.blocksPerSub;

@@ -72,6 +72,7 @@ struct ReduceArgs {
     uint32_t blocksPerSub;
     uint32_t vecOk;   // take the 128-bit path (0: element by element, for testing)
     uint32_t threads; // workgroup size of the launch
+    uint32_t vecBatch;       // leaves per load batch of the 128-bit path: 8 or 16 (picks the kernel instantiation)
     uint32_t writeThrough;   // 16-byte results leave through StoreStream16 instead of a non-temporal store
     // Groups of unequal length (ReduceScatterV): when varGroups is set, group g spans groupLenV[g]
     // elements starting groupOffV[g] elements into every source, instead of the uniform

@@ -295,13 +295,6 @@ struct TableBytes {
     __device__ __forceinline__ uint32_t operator[](int i) const { return (w[i / 4] >> (8 * (i % 4))) & 0xFFu; }
 };
 
-// Leaves whose loads are issued together: sixteen vectors, or eight single elements.
-template <typename S, int W>
-__device__ constexpr int LoadBatch()
-{
-    return W > 1 ? 16 : 8;
-}
-
 // The same for eight uniform 64-bit values (leaf addresses): all of them exist before the first is used.
 __device__ __forceinline__ void ScalarFence8(uint64_t* r)
 {
@@ -464,7 +457,8 @@ struct PackOps<E, 16, typename E::Swar> {
 
 // Evaluates the whole tree for the W elements at element offset `e` of the sub-segment.  Leaves are
 // taken a batch at a time: their loads are all issued before the first fold, whatever the tree shape.
-template <class E, int W>
+// kBatch leaves are taken at a time (a multiple of 8).
+template <class E, int W, int kBatch>
 __device__ __forceinline__ void ReduceOne(const ProgramView& pv, uint32_t* stack, const ReduceArgs& args,
                                           uint64_t e, uint64_t dstOff, uint32_t group)
 {
@@ -477,7 +471,6 @@ __device__ __forceinline__ void ReduceOne(const ProgramView& pv, uint32_t* stack
     uint32_t level = 0;
     bool init = true;   // the next leaf starts a level instead of being folded into it
     const uint32_t nLeaves = pv.nLeaves;
-    constexpr int kBatch = LoadBatch<S, W>();
     for (uint32_t b = 0; b < nLeaves; b += kBatch) {
         TableBytes<kBatch> ranks, ctls;
         ranks.Load(pv.words, kDevProgRankOff + b);
@@ -562,7 +555,9 @@ __device__ __forceinline__ void ReduceOne(const ProgramView& pv, uint32_t* stack
 }
 
 // Dynamic LDS: the accumulator stack, (plan depth - 1) * accumulator bytes * args.threads.
-template <class E>
+// VB = leaves per batch of the 128-bit path: 8 keeps the register count low (more wavefronts in flight), 16 has
+// every load of up to sixteen ranks in flight at once; the launcher picks per launch.
+template <class E, int VB>
 __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
 {
     using S = typename E::S;
@@ -642,14 +637,14 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     }
     for (uint64_t u = first; u < nVec + lead; u += stride) {
         if (u >= lead) {
-            ReduceOne<E, W>(pv, accStack, args, head + (u - lead) * W, dstOff, g);
+            ReduceOne<E, W, VB>(pv, accStack, args, head + (u - lead) * W, dstOff, g);
         }
     }
     const uint64_t bodyEnd = head + nVec * W;
     const uint64_t nScalar = head + (len - bodyEnd);
     for (uint64_t i = first; i < nScalar; i += stride) {
         const uint64_t e = i < head ? i : i - head + bodyEnd;
-        ReduceOne<E, 1>(pv, accStack, args, e, dstOff, g);
+        ReduceOne<E, 1, 8>(pv, accStack, args, e, dstOff, g);
     }
 }
 
@@ -658,35 +653,37 @@ using ReduceKernelFn = void (*)(const ReduceArgs);
 }  // namespace detail
 
 // One translation unit per data type defines its selector (nullptr = combination not offered).
-detail::ReduceKernelFn SelectReduceI8(int op);
-detail::ReduceKernelFn SelectReduceI16(int op);
-detail::ReduceKernelFn SelectReduceI32(int op);
-detail::ReduceKernelFn SelectReduceI64(int op);
-detail::ReduceKernelFn SelectReduceU64(int op);
-detail::ReduceKernelFn SelectReduceF16(int op);
-detail::ReduceKernelFn SelectReduceBf16(int op);
-detail::ReduceKernelFn SelectReduceF32(int op);
-detail::ReduceKernelFn SelectReduceF64(int op);
+detail::ReduceKernelFn SelectReduceI8(int op, int batch);
+detail::ReduceKernelFn SelectReduceI16(int op, int batch);
+detail::ReduceKernelFn SelectReduceI32(int op, int batch);
+detail::ReduceKernelFn SelectReduceI64(int op, int batch);
+detail::ReduceKernelFn SelectReduceU64(int op, int batch);
+detail::ReduceKernelFn SelectReduceF16(int op, int batch);
+detail::ReduceKernelFn SelectReduceBf16(int op, int batch);
+detail::ReduceKernelFn SelectReduceF32(int op, int batch);
+detail::ReduceKernelFn SelectReduceF64(int op, int batch);
+
+#define HCCL_AMD_PICK(T, batch) ((batch) == 8 ? detail::ReduceKernel<T, 8> : detail::ReduceKernel<T, 16>)
 
 #define HCCL_AMD_DEFINE_SELECT4(NAME, SUM_T, PROD_T, MAX_T, MIN_T)                 \
-    detail::ReduceKernelFn NAME(int op)                                           \
+    detail::ReduceKernelFn NAME(int op, int batch)                                \
     {                                                                             \
         switch (op) {                                                             \
-            case detail::kSum: return detail::ReduceKernel<SUM_T>;                \
-            case detail::kProd: return detail::ReduceKernel<PROD_T>;              \
-            case detail::kMax: return detail::ReduceKernel<MAX_T>;                \
-            case detail::kMin: return detail::ReduceKernel<MIN_T>;                \
+            case detail::kSum: return HCCL_AMD_PICK(SUM_T, batch);                \
+            case detail::kProd: return HCCL_AMD_PICK(PROD_T, batch);              \
+            case detail::kMax: return HCCL_AMD_PICK(MAX_T, batch);                \
+            case detail::kMin: return HCCL_AMD_PICK(MIN_T, batch);                \
             default: return nullptr;                                              \
         }                                                                         \
     }
 
 #define HCCL_AMD_DEFINE_SELECT3(NAME, SUM_T, MAX_T, MIN_T)                         \
-    detail::ReduceKernelFn NAME(int op)                                           \
+    detail::ReduceKernelFn NAME(int op, int batch)                                \
     {                                                                             \
         switch (op) {                                                             \
-            case detail::kSum: return detail::ReduceKernel<SUM_T>;                \
-            case detail::kMax: return detail::ReduceKernel<MAX_T>;                \
-            case detail::kMin: return detail::ReduceKernel<MIN_T>;                \
+            case detail::kSum: return HCCL_AMD_PICK(SUM_T, batch);                \
+            case detail::kMax: return HCCL_AMD_PICK(MAX_T, batch);                \
+            case detail::kMin: return HCCL_AMD_PICK(MIN_T, batch);                \
             default: return nullptr;                                              \
         }                                                                         \
     }

@@ -8,16 +8,17 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
 {
     detail::ReduceKernelFn fn = nullptr;
     const int o = static_cast<int>(op);
+    const int batch = args.vecBatch == 8 ? 8 : 16;
     switch (dtype) {
-        case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8(o); break;
-        case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16(o); break;
-        case HCCL_DATA_TYPE_INT32: fn = SelectReduceI32(o); break;
-        case HCCL_DATA_TYPE_INT64: fn = SelectReduceI64(o); break;
-        case HCCL_DATA_TYPE_UINT64: fn = SelectReduceU64(o); break;
-        case HCCL_DATA_TYPE_FP16: fn = SelectReduceF16(o); break;
-        case HCCL_DATA_TYPE_BFP16: fn = SelectReduceBf16(o); break;
-        case HCCL_DATA_TYPE_FP32: fn = SelectReduceF32(o); break;
-        case HCCL_DATA_TYPE_FP64: fn = SelectReduceF64(o); break;
+        case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8(o, batch); break;
+        case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16(o, batch); break;
+        case HCCL_DATA_TYPE_INT32: fn = SelectReduceI32(o, batch); break;
+        case HCCL_DATA_TYPE_INT64: fn = SelectReduceI64(o, batch); break;
+        case HCCL_DATA_TYPE_UINT64: fn = SelectReduceU64(o, batch); break;
+        case HCCL_DATA_TYPE_FP16: fn = SelectReduceF16(o, batch); break;
+        case HCCL_DATA_TYPE_BFP16: fn = SelectReduceBf16(o, batch); break;
+        case HCCL_DATA_TYPE_FP32: fn = SelectReduceF32(o, batch); break;
+        case HCCL_DATA_TYPE_FP64: fn = SelectReduceF64(o, batch); break;
         default: break;
     }
     if (fn == nullptr || nBlocks == 0 || (args.threads != 64 && args.threads != 128 && args.threads != 256)) {
