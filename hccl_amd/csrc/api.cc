@@ -497,7 +497,7 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     a.writeThrough = w->storePolicy != 2 ? w->storePolicy : ((a.dstOwn || a.nDst == 1) ? 1u : 0u);
     // Up to eight ranks folded into one result stream run best with eight-load batches (fewer registers, more
     // wavefronts in flight: +1-2 %); AllReduce's many result streams and larger worlds with sixteen (+5 %).
-    a.vecBatch = w->reduceBatch != 0 ? w->reduceBatch : ((w->n <= 8 && (a.dstOwn || a.nDst == 1)) ? 8u : 16u);
+    a.vecBatch = w->reduceBatch != 0 ? w->reduceBatch : ((w->n <= 8 && !a.varGroups && (a.dstOwn || a.nDst == 1)) ? 8u : 16u);
     a.threads = w->reduceThreads != 0 ? w->reduceThreads : 64u;
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
     uint64_t blocks = subs * a.blocksPerSub;
