@@ -123,11 +123,13 @@ def lib():
     L.HcclAmdSetAlgo.argtypes = [vp, i32, i32]
     L.HcclAmdGetAlgo.argtypes = [vp, i32, ctypes.POINTER(i32)]
     L.HcclAmdGetFoldProgram.argtypes = [i32, i32, u32, u32, vp, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
+    L.HcclAmdSetCclBufferSize.argtypes = [vp, u64]
+    L.HcclAmdGetCclBufferSize.argtypes = [vp, ctypes.POINTER(u64)]
     for name in ("HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV",
                  "HcclAlltoAll", "HcclAlltoAllVC", "HcclReduceScatterV", "HcclReduce", "HcclBroadcast", "HcclScatter",
                  "HcclCommInitAll", "HcclGetRootInfo", "HcclCommInitRootInfo", "HcclCommDestroy", "HcclGetRankSize",
                  "HcclGetRankId", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
-                 "HcclAmdGetFoldProgram"):
+                 "HcclAmdGetFoldProgram", "HcclAmdSetCclBufferSize", "HcclAmdGetCclBufferSize"):
         getattr(L, name).restype = ctypes.c_int
     _lib = L
     return L
@@ -246,6 +248,17 @@ def get_algo(hccl_comm, op_kind):
     v = ctypes.c_int()
     check(lib().HcclAmdGetAlgo(hccl_comm, int(op_kind), ctypes.byref(v)), "HcclAmdGetAlgo")
     return Algo(v.value)
+
+
+def set_ccl_buffer_size(hccl_comm, nbytes):
+    """Size of the staging buffer whose loops NHR / RHD AllReduce reproduce; 0 = one loop."""
+    return check(lib().HcclAmdSetCclBufferSize(hccl_comm, ctypes.c_uint64(nbytes)), "HcclAmdSetCclBufferSize")
+
+
+def get_ccl_buffer_size(hccl_comm):
+    v = ctypes.c_uint64()
+    check(lib().HcclAmdGetCclBufferSize(hccl_comm, ctypes.byref(v)), "HcclAmdGetCclBufferSize")
+    return v.value
 
 
 def fold_programs(op_kind, algo, rank_size):

@@ -236,6 +236,10 @@ struct World {
     // Longest a rank waits on the host for its peers: the reference's CUSTOM_TIMEOUT = 1836 s (alg_param.h:91),
     // overridable by HCCL_EXEC_TIMEOUT (seconds), read when the world is created.
     uint32_t execTimeout = 1836;
+    // Size of the staging buffer whose loops the slice-dependent AllReduce orders (NHR, RHD) reproduce; 0 = one
+    // loop.  HCCL_BUFFSIZE when set, or HcclAmdSetCclBufferSize.
+    uint64_t cclBytes = 0;
+    bool envInvalid = false;      // an environment variable of the reference failed its parser
 
     ~World()
     {
@@ -344,6 +348,13 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->deterministic = v == "STRICT" ? 2 : v == "TRUE" ? 1 : v == "FALSE" ? 0 : 0xFF;
         if (w->deterministic == 0xFF) {
             Log(1, "HCCL_DETERMINISTIC is set to [%s], which is incorrect (true, false or strict)", det);
+            w->envInvalid = true;
+        }
+    }
+    if (const char* buf = getenv("HCCL_BUFFSIZE")) {
+        if (CclBufferAvailableSize(buf, &w->cclBytes) != HCCL_SUCCESS) {
+            Log(1, "HCCL_BUFFSIZE is set to [%s], which is not a number of MB between 2 and 4294967295", buf);
+            w->envInvalid = true;
         }
     }
     return w;
@@ -557,34 +568,67 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
     }
     a.nSub = n;
     a.progSubStride = 1;
+    // One launch per loop of the reference's executor: elements [done, done + len) cut into n sub-segments of
+    // `unit` elements, the last one taking what the others leave.
+    auto launchLoop = [&](uint64_t done, uint64_t len, uint64_t unit) {
+        for (uint32_t r = 0; r < n; ++r) {
+            a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + done * esz;
+            a.dst[r] = static_cast<uint8_t*>(p.ranks[r].recv) + done * esz;
+        }
+        a.total = a.groupLen = len;
+        a.subLen = unit;
+        return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+    };
     if (algo == HCCL_AMD_ALGO_RHD) {
-        // Aligned prefix in n uniform units, then a remainder shorter than n with one element per unit
-        // (reference ins_v2_all_reduce_sequence_rhd_tail.h:98-113, staging buffer taken as unbounded).
-        uint64_t unit = p.count / n;
-        uint64_t prefix = unit * n;
-        if (unit > 0) {
-            a.total = a.groupLen = prefix;
-            a.subLen = unit;
-            rc = LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+        // Whole frames of n uniform units while they last, then a remainder shorter than n with one element per
+        // unit (reference ins_v2_all_reduce_sequence_rhd_tail.h:94-113); a bounded staging buffer limits the
+        // frames one loop holds.
+        uint64_t maxPerLoop = ~0ull / 2 / n * n;
+        if (w->cclBytes != 0) {
+            rc = RhdMaxCountPerLoop(w->cclBytes, p.count, n, esz, &maxPerLoop);
             if (rc != HCCL_SUCCESS) {
+                Log(1, "AllReduce: the staging buffer of %llu bytes holds no loop of the RHD order",
+                    static_cast<unsigned long long>(w->cclBytes));
                 return rc;
             }
         }
-        if (p.count > prefix) {
-            for (uint32_t r = 0; r < n; ++r) {
-                a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + prefix * esz;
-                a.dst[r] = static_cast<uint8_t*>(p.ranks[r].recv) + prefix * esz;
+        for (uint64_t done = 0; done < p.count;) {
+            const uint64_t valid = RhdSelectLoopCount(p.count - done, maxPerLoop, n);
+            rc = launchLoop(done, valid, valid >= n ? valid / n : 1);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
             }
-            a.total = a.groupLen = p.count - prefix;
-            a.subLen = 1;
-            return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+            done += valid;
         }
         return HCCL_SUCCESS;
     }
-    // NHR, order-preserved, symmetric two-shot: slices of ceil(count / n) elements (reference two_shot.cc:184).
-    a.total = a.groupLen = p.count;
-    a.subLen = (p.count + n - 1) / n;
-    return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+    if (algo == HCCL_AMD_ALGO_NHR) {
+        // Slices of floor(len / n) elements, the last slice takes the rest (reference
+        // ins_temp_all_reduce_nhr.cc:214-216); the executor loops over the staging buffer, which this template
+        // uses once (scratch multiple 1, reference ins_temp_all_reduce_nhr.cc:65-71,
+        // ins_v2_all_reduce_sole_executor.cc:241-300).
+        uint64_t maxPerLoop = p.count;
+        if (w->cclBytes != 0) {
+            maxPerLoop = SoleMaxCountPerLoop(w->cclBytes, 1, esz);
+            if (maxPerLoop == 0) {
+                Log(1, "AllReduce: the staging buffer of %llu bytes holds no element",
+                    static_cast<unsigned long long>(w->cclBytes));
+                return HCCL_E_INTERNAL;
+            }
+        }
+        for (uint64_t done = 0; done < p.count;) {
+            const uint64_t len = std::min(p.count - done, maxPerLoop);
+            rc = launchLoop(done, len, len / n);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+            done += len;
+        }
+        return HCCL_SUCCESS;
+    }
+    // Symmetric two-shot: slices of ceil(count / n) elements (reference two_shot.cc:184), always in one loop
+    // (reference ins_v2_all_reduce_sole_executor.cc:273-282).
+    return launchLoop(0, p.count, (p.count + n - 1) / n);
 }
 
 HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
@@ -1074,7 +1118,7 @@ HcclResult SubmitWithReady(Comm* c, OpType type, HcclDataType dtype, HcclReduceO
                            const void* send, void* recv, aclrtStream stream, std::vector<uint64_t>&& var,
                            uint32_t root = 0)
 {
-    if (c->world->deterministic == 0xFF) {
+    if (c->world->envInvalid) {
         return HCCL_E_PARA;   // the reference's environment parsing fails every entry point the same way
     }
     return Submit(c, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var), root);
@@ -1664,6 +1708,31 @@ HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo)
     }
     std::lock_guard<std::mutex> wl(c->world->mu);
     c->world->algo[op] = algo;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdSetCclBufferSize(HcclComm comm, uint64_t bytes)
+{
+    CHK_PTR(comm, "comm");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> wl(c->world->mu);
+    c->world->cclBytes = bytes;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdGetCclBufferSize(HcclComm comm, uint64_t* bytes)
+{
+    CHK_PTR(comm, "comm");
+    CHK_PTR(bytes, "bytes");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> wl(c->world->mu);
+    *bytes = c->world->cclBytes;
     return HCCL_SUCCESS;
 }
 

@@ -3,6 +3,8 @@
 // up holding a segment's result, which rank values were folded into it, in which order and in which role.
 #include "fold_plan.h"
 
+#include <algorithm>
+#include <cstdlib>
 #include <memory>
 
 #include "dataplane.h"
@@ -347,6 +349,57 @@ HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPla
         default:
             return HCCL_E_PARA;
     }
+}
+
+HcclResult CclBufferAvailableSize(const char* envValue, uint64_t* bytes)
+{
+    constexpr uint64_t kMiB = 1024ull * 1024ull;
+    uint64_t mb = 200;
+    if (envValue != nullptr) {
+        char* end = nullptr;
+        mb = std::strtoull(envValue, &end, 10);
+        if (end == envValue || *end != '\0' || mb < 2 || mb > 0xFFFFFFFFull) {
+            return HCCL_E_PARA;
+        }
+    }
+    *bytes = mb * kMiB - kMiB;
+    return HCCL_SUCCESS;
+}
+
+uint64_t SoleMaxCountPerLoop(uint64_t cclBytes, uint64_t scratchMultiple, uint64_t elemSize)
+{
+    uint64_t perLoop = cclBytes;
+    if (scratchMultiple != 0) {
+        perLoop = std::min(cclBytes, cclBytes / scratchMultiple / 128 * 128);
+    }
+    return elemSize == 0 ? 0 : perLoop / elemSize;
+}
+
+HcclResult RhdMaxCountPerLoop(uint64_t cclBytes, uint64_t count, uint32_t p, uint64_t elemSize, uint64_t* maxCount)
+{
+    if (p == 0 || elemSize == 0) {
+        return HCCL_E_PARA;
+    }
+    uint64_t workspace = cclBytes;
+    if (count % p != 0) {
+        if (p > workspace / elemSize / 2) {
+            return HCCL_E_INTERNAL;
+        }
+        const uint64_t tile = p * elemSize;
+        const uint64_t slot = (tile + 127) / 128 * 128;
+        if (slot >= workspace / 2) {
+            return HCCL_E_INTERNAL;
+        }
+        workspace -= 2 * slot;
+    }
+    *maxCount = workspace / 2 / 128 * 128 / elemSize / p * p;
+    return *maxCount == 0 ? HCCL_E_INTERNAL : HCCL_SUCCESS;
+}
+
+uint64_t RhdSelectLoopCount(uint64_t remaining, uint64_t maxCountPerLoop, uint64_t p)
+{
+    const uint64_t count = std::min(remaining, maxCountPerLoop);
+    return count >= p ? count / p * p : count;
 }
 
 }  // namespace hccl_amd

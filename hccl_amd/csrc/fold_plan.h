@@ -27,4 +27,20 @@ uint32_t RhdPairCount(uint32_t p);                    // r = p - 2^floor(log2 p)
 uint32_t RhdSlotOfRank(uint32_t p, uint32_t rank);    // sigma: t -> 2t, t+r -> 2t+1, others identity
 uint32_t RhdCarrierOfVirtual(uint32_t p, uint32_t v); // physical rank that plays virtual rank v
 
+// Loop limits of the reference's executors, which stage every AllReduce through a bounded buffer and cut the
+// count into loops that are each sliced afresh.  cclBytes is that buffer's size.
+// HCCL_BUFFSIZE (MB, digits only, 2 .. UINT32_MAX) less the 1 MiB kept back; nullptr = unset = 200 MB
+// (reference src/common/op_graph/hccl_op_utils.cc:204-225).  HCCL_E_PARA for anything else.
+HcclResult CclBufferAvailableSize(const char* envValue, uint64_t* bytes);
+// Elements per loop of a single-template executor (reference ins_v2_all_reduce_sole_executor.cc:241-262).
+uint64_t SoleMaxCountPerLoop(uint64_t cclBytes, uint64_t scratchMultiple, uint64_t elemSize);
+// Elements per loop of the RHD sequence executor with one rank per level-0 group: two 128-byte-rounded tiles of
+// p elements leave the buffer when count is not a multiple of p, half of the rest receives, floored to 128
+// bytes, whole elements and a multiple of p (reference ins_v2_all_reduce_sequence_rhd_tail.h:64-92,
+// ins_v2_all_reduce_sequence_executor_aicpu.cc:592-600, 645-675).  HCCL_E_INTERNAL when nothing fits.
+HcclResult RhdMaxCountPerLoop(uint64_t cclBytes, uint64_t count, uint32_t p, uint64_t elemSize, uint64_t* maxCount);
+// Elements the next RHD loop takes: whole frames of p while they last, then the remainder below p alone
+// (reference ins_v2_all_reduce_sequence_rhd_tail.h:94-99).
+uint64_t RhdSelectLoopCount(uint64_t remaining, uint64_t maxCountPerLoop, uint64_t p);
+
 }  // namespace hccl_amd

@@ -170,7 +170,9 @@ typedef enum {
     /* Recursive halving-doubling with pre-fold of non-power-of-two ranks
      * (reference template_utils.cc:117-307, ins_temp_reduce_scatter_rhd.cc). */
     HCCL_AMD_ALGO_RHD = 2,
-    /* Non-uniform hierarchical ring step tree (reference ins_temp_reduce_scatter_nhr.cc:458-506). */
+    /* Non-uniform hierarchical ring step tree (reference ins_temp_reduce_scatter_nhr.cc:458-506).  AllReduce
+     * cuts the count into N slices of floor(count / N) elements, the last slice taking the rest, and folds
+     * slice k by rank k's tree (reference ins_temp_all_reduce_nhr.cc:214-216, 646-687). */
     HCCL_AMD_ALGO_NHR = 3,
     /* Power-of-two block fold used when results must not depend on arrival order
      * (reference ins_temp_reduce_scatter_order_preserved_group.cc:306-409). */
@@ -189,6 +191,22 @@ typedef enum {
  * world creation through HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr". */
 HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo);
 HcclResult HcclAmdGetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo* algo);
+
+/*
+ * Staging-buffer loops.  The reference's executors move every AllReduce through a bounded buffer: the count is
+ * cut into loops and each loop is sliced afresh (ins_v2_all_reduce_sole_executor.cc:241-300,
+ * ins_v2_all_reduce_sequence_executor_aicpu.cc:645-760), so under the orders whose fold depends on the slice
+ * (NHR, RHD) the association order of an element depends on the loop it falls in.  No staging exists here;
+ * `bytes` only tells the library which loop boundaries to reproduce: 0 (default) = one loop.  The environment
+ * variable HCCL_BUFFSIZE (MB), when set at world creation, gives MB * 2^20 - 2^20 bytes
+ * (src/common/op_graph/hccl_op_utils.cc:204-225); a value its parser rejects makes every collective return
+ * HCCL_E_PARA.  Orders that fold every position alike (MESH, RING, ORDER_PRESERVED) and ReduceScatter, whose
+ * fold depends on the receiving rank only, are not affected; MESH_SYMMETRIC always runs as one loop
+ * (ins_v2_all_reduce_sole_executor.cc:273-282).  A buffer too small for one loop returns HCCL_E_INTERNAL from the
+ * collective, like the reference.
+ */
+HcclResult HcclAmdSetCclBufferSize(HcclComm comm, uint64_t bytes);
+HcclResult HcclAmdGetCclBufferSize(HcclComm comm, uint64_t* bytes);
 
 /*
  * Host-only view of the reduction plan: writes the fold program the kernel would run for

@@ -78,6 +78,12 @@ def lib():
         L.orc_rhd_alg_rank_of_virtual.restype = ctypes.c_uint32
         L.orc_rhd_alg_rank_of_virtual.argtypes = [ctypes.c_uint32] * 3
         L.orc_local_copy_slices.restype = ctypes.c_uint32
+        L.orc_ccl_buffer_available_size.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_uint64)]
+        L.orc_sole_max_count_per_loop.restype = ctypes.c_uint64
+        L.orc_sole_max_count_per_loop.argtypes = [ctypes.c_uint64] * 3
+        L.orc_rhd_prepare_tail_workspace.argtypes = [ctypes.c_uint64] * 3 + [ctypes.POINTER(ctypes.c_uint64)] * 3
+        L.orc_rhd_max_count_per_loop.argtypes = [ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint64,
+                                                 ctypes.POINTER(ctypes.c_uint64)]
         _lib = L
     return _lib
 
@@ -192,6 +198,31 @@ def nhr_step_info(n, rank, step):
     return rc, to.value, frm.value, list(tx[:cnt.value]), list(rx[:cnt.value])
 
 
+def ccl_buffer_available_size(env_value):
+    """(rc, bytes) for a HCCL_BUFFSIZE string, None = unset."""
+    out = ctypes.c_uint64(0)
+    rc = lib().orc_ccl_buffer_available_size(None if env_value is None else env_value.encode(), ctypes.byref(out))
+    return rc, out.value
+
+
+def sole_max_count_per_loop(ccl_bytes, scratch_multiple, elem_size):
+    return lib().orc_sole_max_count_per_loop(ccl_bytes, scratch_multiple, elem_size)
+
+
+def rhd_prepare_tail_workspace(count, rank_align, elem_size, workspace_bytes):
+    """(rc, workspace bytes left, input tile offset, output tile offset)."""
+    ws, i, o = ctypes.c_uint64(workspace_bytes), ctypes.c_uint64(0), ctypes.c_uint64(0)
+    rc = lib().orc_rhd_prepare_tail_workspace(count, rank_align, elem_size, ctypes.byref(ws), ctypes.byref(i),
+                                              ctypes.byref(o))
+    return rc, ws.value, i.value, o.value
+
+
+def rhd_max_count_per_loop(ccl_bytes, count, p, elem_size):
+    out = ctypes.c_uint64(0)
+    rc = lib().orc_rhd_max_count_per_loop(ccl_bytes, count, p, elem_size, ctypes.byref(out))
+    return rc, out.value
+
+
 def local_copy_slices(src_off, dst_off, sizes):
     n = len(sizes)
     s, sp = _u64(src_off)
@@ -221,7 +252,8 @@ def all_reduce(ins, outs, count, dtype, op, acc=ACC_FP32, algo="mesh", max_count
         return _reduce_call("orc_all_reduce_rhd", ins, outs, count, dtype, op, acc,
                             ctypes.c_uint64(max_count_per_loop))
     if algo == "nhr":
-        return _reduce_call("orc_all_reduce_nhr", ins, outs, count, dtype, op, acc)
+        return _reduce_call("orc_all_reduce_nhr_looped", ins, outs, count, dtype, op, acc,
+                            ctypes.c_uint64(max_count_per_loop))
     if algo == "order_preserved":
         return _reduce_call("orc_all_reduce_order_preserved", ins, outs, count, dtype, op, acc)
     raise ValueError(algo)

@@ -934,40 +934,133 @@ int orc_reduce_scatter_nhr(uint32_t n, const void* const* in, void* const* out, 
     return rc;
 }
 
-int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
-                       int accMode)
+/* One KernelRun of InsTempAllReduceNHR (ins_temp_all_reduce_nhr.cc:214-216): the first n - 1 slices hold
+ * floor(count / n) elements, the last one takes the rest; slice k is folded by the NHR step tree. */
+static int nhr_all_reduce_once(red_t* r, uint32_t n, const void* const* in, void* const* out, uint64_t first,
+                               uint64_t count)
+{
+    uint64_t slice = count / n;
+    uint64_t tail = count - slice * (n - 1);
+    scratch_t sc;
+    if (scratch_alloc(&sc, n, tail, r->asz) != ORC_OK) {
+        return ORC_E_INTERNAL;
+    }
+    memset(sc.mem, 0, (uint64_t)n * n * tail * r->asz);
+    for (uint32_t m = 0; m < n; ++m) {
+        for (uint32_t i = 0; i < n; ++i) {
+            uint64_t cur = i == n - 1 ? tail : slice;
+            red_widen(r, cbytes(in[m]) + (first + (uint64_t)i * slice) * r->esz, scratch_at(&sc, m, i), cur);
+        }
+    }
+    int rc = nhr_reduce_scatter_scratch(r, &sc);
+    if (rc == ORC_OK) {
+        for (uint32_t i = 0; i < n; ++i) {
+            uint64_t cur = i == n - 1 ? tail : slice;
+            for (uint32_t m = 0; m < n; ++m) {
+                red_narrow(r, scratch_at(&sc, i, i), bytes(out[m]) + (first + (uint64_t)i * slice) * r->esz, cur);
+            }
+        }
+    }
+    free(sc.mem);
+    return rc;
+}
+
+int orc_all_reduce_nhr_looped(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                              int accMode, uint64_t maxCountPerLoop)
 {
     red_t r;
     int rc = red_init(&r, dtype, op, accMode);
     if (rc != ORC_OK) {
         return rc;
     }
-    if (count == 0) {
+    if (maxCountPerLoop == 0) {
+        maxCountPerLoop = count;
+    }
+    /* ins_v2_all_reduce_sole_executor.cc:266-300: full loops, the last one takes what is left */
+    for (uint64_t done = 0; done < count && rc == ORC_OK;) {
+        uint64_t cur = count - done < maxCountPerLoop ? count - done : maxCountPerLoop;
+        rc = nhr_all_reduce_once(&r, n, in, out, done, cur);
+        done += cur;
+    }
+    return rc;
+}
+
+int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                       int accMode)
+{
+    return orc_all_reduce_nhr_looped(n, in, out, count, dtype, op, accMode, 0);
+}
+
+/* ---- staging-buffer loop limits ----------------------------------------------------------------
+ * hccl_op_utils.cc:204-225: HCCL_BUFFSIZE in MB (default 200, at least 2, at most UINT32_MAX, digits only),
+ * less 1 MiB that is kept back. */
+int orc_ccl_buffer_available_size(const char* envValue, uint64_t* bytes)
+{
+    uint64_t mb = 200;
+    if (envValue != NULL) {
+        char* end = NULL;
+        unsigned long long v = strtoull(envValue, &end, 10);
+        if (end == envValue || *end != '\0' || v < 2 || v > 0xFFFFFFFFull) {
+            return ORC_E_PARA;
+        }
+        mb = v;
+    }
+    *bytes = mb * 1024 * 1024 - 1024 * 1024;
+    return ORC_OK;
+}
+
+/* ins_v2_all_reduce_sole_executor.cc:241-262: elements one loop of a single-template executor may take. */
+uint64_t orc_sole_max_count_per_loop(uint64_t cclBytes, uint64_t scratchMultiple, uint64_t elemSize)
+{
+    uint64_t bytes = cclBytes;
+    if (scratchMultiple != 0) {
+        uint64_t bound = cclBytes / scratchMultiple / 128 * 128;
+        bytes = bound < cclBytes ? bound : cclBytes;
+    }
+    return elemSize ? bytes / elemSize : 0;
+}
+
+/* ins_v2_all_reduce_sequence_rhd_tail.h:64-92: two 128-byte-rounded tiles of rankAlign elements are taken
+ * from the end of the workspace when count is not a multiple of rankAlign. */
+int orc_rhd_prepare_tail_workspace(uint64_t count, uint64_t rankAlign, uint64_t elemSize, uint64_t* workspaceBytes,
+                                   uint64_t* inputOffset, uint64_t* outputOffset)
+{
+    if (rankAlign == 0 || elemSize == 0) {
+        return ORC_E_PARA;
+    }
+    if (count % rankAlign == 0) {
         return ORC_OK;
     }
-    uint64_t slice = orc_round_up(count, n);
-    scratch_t sc;
-    if (scratch_alloc(&sc, n, slice, r.asz) != ORC_OK) {
+    uint64_t size = *workspaceBytes;
+    if (rankAlign > size / elemSize / 2) {
         return ORC_E_INTERNAL;
     }
-    memset(sc.mem, 0, (uint64_t)n * n * slice * r.asz);
-    for (uint32_t m = 0; m < n; ++m) {
-        for (uint32_t i = 0; i < n; ++i) {
-            uint64_t off = (uint64_t)i * slice;
-            uint64_t cur = off >= count ? 0 : (count - off > slice ? slice : count - off);
-            red_widen(&r, cbytes(in[m]) + off * r.esz, scratch_at(&sc, m, i), cur);
-        }
+    uint64_t tile = rankAlign * elemSize;
+    uint64_t slot = (tile / 128 + (tile % 128 != 0)) * 128;
+    if (slot >= size / 2) {
+        return ORC_E_INTERNAL;
     }
-    rc = nhr_reduce_scatter_scratch(&r, &sc);
-    if (rc == ORC_OK) {
-        for (uint32_t i = 0; i < n; ++i) {
-            uint64_t off = (uint64_t)i * slice;
-            uint64_t cur = off >= count ? 0 : (count - off > slice ? slice : count - off);
-            for (uint32_t m = 0; m < n; ++m) red_narrow(&r, scratch_at(&sc, i, i), bytes(out[m]) + off * r.esz, cur);
-        }
+    *inputOffset = size - 2 * slot;
+    *outputOffset = size - slot;
+    *workspaceBytes = *inputOffset;
+    return ORC_OK;
+}
+
+/* ins_v2_all_reduce_sequence_executor_aicpu.cc:592-600, 645-662, 668-675 with one rank per level-0 group:
+ * the tail tiles come off first, half of what remains is the receive area, floored to 128 bytes, to whole
+ * elements and to a multiple of p. */
+int orc_rhd_max_count_per_loop(uint64_t cclBytes, uint64_t count, uint32_t p, uint64_t elemSize, uint64_t* maxCount)
+{
+    uint64_t size = cclBytes;
+    uint64_t inOff = 0;
+    uint64_t outOff = 0;
+    int rc = orc_rhd_prepare_tail_workspace(count, p, elemSize, &size, &inOff, &outOff);
+    if (rc != ORC_OK) {
+        return rc;
     }
-    free(sc.mem);
-    return rc;
+    uint64_t outHalf = size / 2;
+    *maxCount = outHalf / 128 * 128 / elemSize / p * p;
+    return *maxCount == 0 ? ORC_E_INTERNAL : ORC_OK;
 }
 
 /* ---------------------------------------------------------------------------------------------

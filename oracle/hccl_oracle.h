@@ -96,6 +96,13 @@ void orc_rhd_seg_bytes_uniform(uint32_t unitStart, uint32_t unitEnd, uint64_t sl
                                uint32_t tailUnit, uint64_t* offset, uint64_t* len);          /* :310 */
 /* ins_v2_all_reduce_sequence_rhd_tail.h:98-113 */
 uint64_t orc_rhd_select_loop_count(uint64_t remaining, uint64_t maxCountPerLoop, uint64_t rankAlign);
+/* Staging-buffer ("CCL buffer") loop limits.  hccl_op_utils.cc:204-225; sole_executor.cc:241-262;
+ * rhd_tail.h:64-92; sequence_executor_aicpu.cc:592-600, 645-675 (one rank per level-0 group). */
+int orc_ccl_buffer_available_size(const char* envValue /* NULL = unset */, uint64_t* bytes);
+uint64_t orc_sole_max_count_per_loop(uint64_t cclBytes, uint64_t scratchMultiple, uint64_t elemSize);
+int orc_rhd_prepare_tail_workspace(uint64_t count, uint64_t rankAlign, uint64_t elemSize, uint64_t* workspaceBytes,
+                                   uint64_t* inputOffset, uint64_t* outputOffset);
+int orc_rhd_max_count_per_loop(uint64_t cclBytes, uint64_t count, uint32_t p, uint64_t elemSize, uint64_t* maxCount);
 /* ins_temp_reduce_scatter_nhr.cc:458-506; tx/rx arrays need rankSize entries. */
 int orc_nhr_step_info(uint32_t rankSize, uint32_t algRank, uint32_t step, uint32_t* toRank, uint32_t* fromRank,
                       uint32_t* nSlices, uint32_t* txSliceIdxs, uint32_t* rxSliceIdxs);
@@ -132,10 +139,14 @@ int orc_all_reduce_order_preserved(uint32_t n, const void* const* in, void* cons
 /* vector-core mesh order (aiv_reduce_scatter_mesh_1d.h:23-71). */
 int orc_reduce_scatter_aiv_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
                                 int op, int accMode);
-/* AllReduce whose every element follows the NHR reduce-scatter tree of its slice
- * (slices of ceil(count/n) elements), then gather. */
+/* One-level NHR AllReduce (ins_temp_all_reduce_nhr.cc:214-216, 646-687): slices of floor(count/n) elements, the
+ * last slice takes the rest; every element follows the NHR reduce-scatter tree of its slice, then gather. */
 int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
                        int accMode);
+/* The same inside the executor's loop over the staging buffer (ins_v2_all_reduce_sole_executor.cc:266-300):
+ * every loop of maxCountPerLoop elements (the last one shorter) is sliced afresh; 0 = one loop. */
+int orc_all_reduce_nhr_looped(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                              int accMode, uint64_t maxCountPerLoop);
 
 /* a13: all_gather_mesh_1D.cc:249-423. */
 int orc_all_gather(uint32_t n, const void* const* in, void* const* out, uint64_t sendCount, int dtype);

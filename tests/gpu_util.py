@@ -56,6 +56,9 @@ class World:
     def set_algo(self, kind, name):
         hccl_amd.set_algo(self.comms[0], kind, ALGO_BY_NAME[name])
 
+    def set_ccl_buffer_size(self, nbytes):
+        hccl_amd.set_ccl_buffer_size(self.comms[0], nbytes)
+
     def inputs_ready(self):
         """Inputs are produced on torch's default stream; the collective runs on self.stream."""
         import torch

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 import oracle
+import hccl_amd
 from hccl_amd import HcclDataType as DT, HcclReduceOp as OP, OpKind
 
 from gpu_util import World, dev_zeros, require_library_on_gpu, same_bits_nan_class, to_dev, to_host
@@ -93,12 +94,13 @@ def pad_of(pad, r, which):
     return pad(r, which) if callable(pad) else pad
 
 
-def run_all_reduce(world, dtype, op, count, algo, seed, pad=0, in_place=False):
+def run_all_reduce(world, dtype, op, count, algo, seed, pad=0, in_place=False, max_count_per_loop=0):
     rng = np.random.default_rng(seed)
     n = world.n
     ins = [gen(dtype, op, rng, count) for _ in range(n)]
     want = [np.zeros(count, dtype=NP[dtype]) for _ in range(n)]
-    assert oracle.all_reduce(ins, want, count, int(dtype), op, acc=oracle.ACC_FP32, algo=algo) == 0
+    assert oracle.all_reduce(ins, want, count, int(dtype), op, acc=oracle.ACC_FP32, algo=algo,
+                             max_count_per_loop=max_count_per_loop) == 0
     sends = [to_dev(x, pad_of(pad, r, "send")) for r, x in enumerate(ins)]
     recvs = sends if in_place else [dev_zeros(x.nbytes, pad_of(pad, r, "recv")) for r, x in enumerate(ins)]
     world.all_reduce(sends, recvs, count, dtype, op, algo)
@@ -371,4 +373,41 @@ def test_all_reduce_larger_than_a_million_workgroups():
                 assert torch.equal(recvs[r][lo:lo + step].view(torch.int16), want.view(torch.int16)), (lo, r)
             del want
     finally:
+        w.close()
+
+
+# ---------------------------------------------------------------------------------------------
+# Loops over a bounded staging buffer: every loop is sliced afresh (NHR, RHD)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [6, 8])
+@pytest.mark.parametrize("algo", ["nhr", "rhd"])
+def test_all_reduce_follows_staging_buffer_loops(n, algo):
+    w = World(n)
+    try:
+        for dtype, count, ccl in ((DT.FP32, 100_003, 65536), (DT.FP32, 6 * 8 * 1000, 4096), (DT.FP16, 33_333, 8192),
+                                  (DT.INT32, 5, 65536)):
+            esz = np.dtype(NP[dtype]).itemsize
+            if algo == "nhr":
+                per_loop = oracle.sole_max_count_per_loop(ccl, 1, esz)
+            else:
+                rc, per_loop = oracle.rhd_max_count_per_loop(ccl, count, n, esz)
+                assert rc == 0
+            w.set_ccl_buffer_size(ccl)
+            run_all_reduce(w, dtype, SUM, count, algo, seed=n * 100 + count % 97, max_count_per_loop=per_loop)
+        # one loop again: differs from the looped result for wide-range fp32 inputs, equals the oracle's one loop
+        w.set_ccl_buffer_size(0)
+        run_all_reduce(w, DT.FP32, SUM, 100_003, algo, seed=77)
+        # a buffer that holds no loop is refused like in the reference
+        w.set_ccl_buffer_size(16 if algo == "rhd" else 2)
+        x = [to_dev(np.ones(64, dtype=np.float32)) for _ in range(n)]
+        y = [dev_zeros(256) for _ in range(n)]
+        with pytest.raises(hccl_amd.HcclError) as e:
+            w.all_reduce(x, y, 64, DT.FP32, SUM, algo)
+        assert e.value.code == 4
+        # orders that fold every position alike ignore the buffer
+        w.set_ccl_buffer_size(4096)
+        run_all_reduce(w, DT.FP32, SUM, 10_001, "mesh", seed=78)
+        run_all_reduce(w, DT.FP32, SUM, 10_001, "mesh_symmetric", seed=79)
+    finally:
+        w.set_ccl_buffer_size(0)
         w.close()

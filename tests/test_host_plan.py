@@ -155,7 +155,13 @@ def test_all_reduce_programs_match_oracle(orc, n, algo):
                     got[lo:hi] = run_program(progs[i], lambda r: ins[r][lo:hi], op)
             for e in range(unit * n, count):
                 got[e:e + 1] = run_program(progs[e - unit * n], lambda r: ins[r][e:e + 1], op)
-        else:
+        elif algo == Algo.NHR:       # floor slices, the last one takes the rest
+            sl = count // n
+            for i in range(n):
+                lo, hi = i * sl, (count if i == n - 1 else (i + 1) * sl)
+                if hi > lo:
+                    got[lo:hi] = run_program(progs[i], lambda r: ins[r][lo:hi], op)
+        else:                        # ceil slices, the last ones may be short or empty
             sl = -(-count // n)
             for i in range(n):
                 lo, hi = min(count, i * sl), min(count, (i + 1) * sl)
@@ -328,6 +334,35 @@ def test_unparsable_hccl_deterministic_fails_every_collective(monkeypatch):
     finally:
         for c in comms:
             hccl_amd.comm_destroy(c)
+
+
+def test_staging_buffer_size_knob_and_environment(monkeypatch):
+    monkeypatch.delenv("HCCL_BUFFSIZE", raising=False)
+    comms = hccl_amd.comm_init_all(2)
+    try:
+        assert hccl_amd.get_ccl_buffer_size(comms[0]) == 0                 # unset: one loop
+        hccl_amd.set_ccl_buffer_size(comms[1], 65536)
+        assert hccl_amd.get_ccl_buffer_size(comms[0]) == 65536             # a property of the world
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)
+    # the reference's own known answers (test/ut/op_graph_utils/hccl_op_utils_test.cc:287-296)
+    for env, want in (("100", 99 << 20), ("2048", 2047 << 20)):
+        monkeypatch.setenv("HCCL_BUFFSIZE", env)
+        comms = hccl_amd.comm_init_all(2)
+        try:
+            assert hccl_amd.get_ccl_buffer_size(comms[0]) == want
+        finally:
+            for c in comms:
+                hccl_amd.comm_destroy(c)
+    for env in ("abc", "-5", "0", "1", "12x", "4294967296"):              # :299-307
+        monkeypatch.setenv("HCCL_BUFFSIZE", env)
+        comms = hccl_amd.comm_init_all(2)
+        try:
+            assert code_of(hccl_amd.all_reduce, comms[0], 0x2000, 0x3000, 8, DT.FP32, OP.SUM, 0x1000) == 1, env
+        finally:
+            for c in comms:
+                hccl_amd.comm_destroy(c)
 
 
 def test_a_rank_whose_peers_never_call_times_out(monkeypatch):

@@ -162,6 +162,50 @@ def test_reduce_scatter_nhr_roles_n4(orc):
             assert np.array_equal(outs[k].view(np.uint32), want.view(np.uint32))
 
 
+def nhr_tree_n8(x):
+    """The N=8 tree of one slice, x[i] = rank (k + i) mod 8's values of slice k."""
+    return ((x[7] + x[6]) + (x[5] + x[4])) + ((x[3] + x[2]) + (x[1] + x[0]))
+
+
+def nhr_all_reduce_expected_n8(ins, lo, hi):
+    """Elements [lo, hi) handled by one run of the one-level NHR AllReduce template: seven slices of
+    floor((hi - lo) / 8) elements and the last slice with the rest."""
+    want = np.zeros(hi - lo, dtype=np.float32)
+    cnt = hi - lo
+    sl = cnt // 8
+    for k in range(8):
+        a, b = k * sl, (cnt if k == 7 else (k + 1) * sl)
+        want[a:b] = nhr_tree_n8([ins[(k + i) % 8][lo + a:lo + b] for i in range(8)])
+    return want
+
+
+@pytest.mark.parametrize("count", [8 * 300, 8 * 300 + 5, 5, 8, 15])
+def test_all_reduce_nhr_floor_slices_last_takes_rest(orc, count):
+    rng = np.random.default_rng(23 + count)
+    ins = wide_f32(rng, 8, count)
+    outs = outs_like(ins)
+    assert orc.all_reduce(ins, outs, count, F32, SUM, algo="nhr") == 0
+    want = nhr_all_reduce_expected_n8(ins, 0, count)
+    for o in outs:
+        assert np.array_equal(o.view(np.uint32), want.view(np.uint32))
+
+
+def test_all_reduce_nhr_loop_re_cuts_slices(orc):
+    """Each loop over the staging buffer slices its own share afresh."""
+    rng = np.random.default_rng(24)
+    count, per_loop = 2000, 640
+    ins = wide_f32(rng, 8, count)
+    outs = outs_like(ins)
+    assert orc.all_reduce(ins, outs, count, F32, SUM, algo="nhr", max_count_per_loop=per_loop) == 0
+    want = np.concatenate([nhr_all_reduce_expected_n8(ins, lo, min(count, lo + per_loop))
+                           for lo in range(0, count, per_loop)])
+    for o in outs:
+        assert np.array_equal(o.view(np.uint32), want.view(np.uint32))
+    one_loop = outs_like(ins)
+    assert orc.all_reduce(ins, one_loop, count, F32, SUM, algo="nhr") == 0
+    assert np.count_nonzero(one_loop[0] != outs[0]) > 0           # wide-range inputs: the order shows
+
+
 def test_order_preserved_six_block_example(orc):
     """The worked example in the reference's own comment: E->A, F->B, C->(AE), D->(BF), (BFD)->(AEC)."""
     rng = np.random.default_rng(30)

@@ -242,3 +242,40 @@ def test_local_copy_slices_merges_contiguous_runs(orc):
     got = orc.local_copy_slices([0, 16], [0, 32], [16, 16])
     assert got == [(0, 0, 16), (16, 32, 16)]
     assert orc.local_copy_slices([5], [9], [7]) == [(5, 9, 7)]
+
+
+def test_ccl_buffer_available_size_known_answers(orc):
+    g = GOLD["ccl_buffer_available_size"]
+    for env, want in g["valid"]:
+        assert orc.ccl_buffer_available_size(env) == (0, want)
+    for env in g["invalid"]:
+        assert orc.ccl_buffer_available_size(env)[0] != 0, env
+
+
+def test_rhd_tail_workspace_known_answers(orc):
+    for count, align, esz, ws, rc, left, in_off, out_off in GOLD["rhd_tail_workspace"]["rows"]:
+        got = orc.rhd_prepare_tail_workspace(count, align, esz, ws)
+        assert got[0] == rc and got[1] == left, (count, align, esz, ws, got)
+        if in_off is not None:
+            assert got[2:] == (in_off, out_off)
+            assert in_off % 128 == 0 and out_off % 128 == 0            # the reference's own assertions
+            assert in_off + align * esz <= out_off and out_off + align * esz <= ws
+
+
+def test_loop_limits_closed_forms(orc):
+    """Sole executor: floor(ccl / multiple / 128) * 128 bytes, never above ccl, in whole elements.
+    RHD sequence: the tail tiles come off first, then half, 128-byte floor, whole elements, multiple of p."""
+    for ccl in (1 << 20, 199 << 20, 1000, 4096 + 17):
+        for mult in (0, 1, 2, 6, 8):
+            for esz in (1, 2, 4, 8):
+                want = (ccl if mult == 0 else min(ccl, ccl // mult // 128 * 128)) // esz
+                assert orc.sole_max_count_per_loop(ccl, mult, esz) == want
+    for ccl, count, p, esz in ((4096, 144, 6, 4), (4096, 145, 6, 4), (1 << 20, 1000, 6, 2), (1 << 20, 1001, 7, 2)):
+        left = ccl
+        if count % p:
+            slot = -(-p * esz // 128) * 128
+            left = ccl - 2 * slot
+        want = left // 2 // 128 * 128 // esz // p * p
+        assert orc.rhd_max_count_per_loop(ccl, count, p, esz) == (0, want)
+    assert orc.rhd_max_count_per_loop(512, 73, 72, 4)[0] == 4       # too small for the tail tiles
+    assert orc.rhd_max_count_per_loop(200, 12, 6, 8)[0] == 4        # half of it, floored to 128 B, holds no whole frame
