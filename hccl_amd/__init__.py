@@ -64,6 +64,7 @@ class Algo(enum.IntEnum):
     ORDER_PRESERVED = 4
     AIV_MESH = 5
     MESH_SYMMETRIC = 6
+    MESH_CHUNK = 7
 
 
 class OpKind(enum.IntEnum):

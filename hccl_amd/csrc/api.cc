@@ -276,7 +276,8 @@ bool ParseAlgoName(const std::string& s, HcclAmdAlgo* algo)
     static const struct { const char* name; HcclAmdAlgo algo; } table[] = {
         {"mesh", HCCL_AMD_ALGO_MESH}, {"ring", HCCL_AMD_ALGO_RING}, {"rhd", HCCL_AMD_ALGO_RHD},
         {"nhr", HCCL_AMD_ALGO_NHR}, {"order_preserved", HCCL_AMD_ALGO_ORDER_PRESERVED},
-        {"aiv_mesh", HCCL_AMD_ALGO_AIV_MESH}, {"mesh_symmetric", HCCL_AMD_ALGO_MESH_SYMMETRIC}};
+        {"aiv_mesh", HCCL_AMD_ALGO_AIV_MESH}, {"mesh_symmetric", HCCL_AMD_ALGO_MESH_SYMMETRIC},
+        {"mesh_chunk", HCCL_AMD_ALGO_MESH_CHUNK}};
     for (const auto& e : table) {
         if (s == e.name) {
             *algo = e.algo;
@@ -542,6 +543,41 @@ HcclAmdAlgo EffectiveAlgo(const World* w, HcclAmdOpKind kind, HcclDataType dtype
     return w->algo[kind];
 }
 
+// Mesh-chunk order: one launch per run of equally long segments.  `nGroup` slices of `len` elements start
+// `sliceStride` elements apart from element `base` of every send buffer; slice g is slice firstSlice + g of the
+// plan.  The results go to dst[...] + dstBase (+ g * sliceStride when every destination receives every slice).
+HcclResult LaunchMeshChunk(World* w, const DevicePlan& plan, const PendingOp& p, ReduceArgs a, uint32_t firstSlice,
+                           uint32_t nGroup, uint64_t len, uint64_t sliceStride, bool alignTo4K, hipStream_t s)
+{
+    const uint32_t n = w->n;
+    const uint32_t esz = DataTypeSize(p.dtype);
+    const uint32_t segs = n - 1;
+    for (const SegmentRun& run : MeshChunkSegments(len, n, esz, alignTo4K)) {
+        ReduceArgs r = a;
+        for (uint32_t k = 0; k < n; ++k) {
+            r.src[k] = static_cast<const uint8_t*>(a.src[k]) + run.first * esz;
+            if (a.dst[k] != nullptr) {
+                r.dst[k] = static_cast<uint8_t*>(a.dst[k]) + run.first * esz;
+            }
+        }
+        r.prog = plan.dev + (static_cast<uint64_t>(firstSlice) * segs + run.firstSeg) * kDevProgBytes;
+        r.progGroupStride = segs;
+        r.progSubStride = 1;
+        r.nGroup = nGroup;
+        r.nSub = run.nSeg;
+        r.subLen = run.segLen;
+        r.groupLen = run.segLen * (run.nSeg - 1) + run.lastLen;
+        r.total = r.groupLen * nGroup;
+        r.srcGroupStride = sliceStride;
+        r.dstGroupStride = sliceStride;
+        HcclResult rc = LaunchOneReduce(w, r, plan, p.dtype, p.op, s);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
 HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
@@ -565,6 +601,46 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
         a.total = a.groupLen = a.subLen = p.count;
         a.nSub = 1;
         return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+    }
+    if (algo == HCCL_AMD_ALGO_MESH_CHUNK) {
+        // Slices of ceil(len / n) elements, short or empty towards the end (reference
+        // ins_temp_all_reduce_mesh_1D_two_shot_mesh_chunk.cc:86-112); the executor loops over half of the
+        // staging buffer (:55-62, ins_v2_all_reduce_sole_executor.cc:241-300).
+        uint64_t maxPerLoop = p.count;
+        if (w->cclBytes != 0) {
+            maxPerLoop = SoleMaxCountPerLoop(w->cclBytes, 2, esz);
+            if (maxPerLoop == 0) {
+                return HCCL_E_INTERNAL;
+            }
+        }
+        for (uint64_t done = 0; done < p.count;) {
+            const uint64_t len = std::min(p.count - done, maxPerLoop);
+            const uint64_t slice = (len + n - 1) / n;
+            const uint32_t nFull = static_cast<uint32_t>(len / slice);
+            for (uint32_t r = 0; r < n; ++r) {
+                a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + done * esz;
+                a.dst[r] = static_cast<uint8_t*>(p.ranks[r].recv) + done * esz;
+            }
+            if (nFull != 0) {
+                rc = LaunchMeshChunk(w, plan, p, a, 0, nFull, slice, slice, false, s);
+                if (rc != HCCL_SUCCESS) {
+                    return rc;
+                }
+            }
+            const uint64_t rest = len - static_cast<uint64_t>(nFull) * slice;
+            if (rest != 0) {
+                for (uint32_t r = 0; r < n; ++r) {
+                    a.src[r] = static_cast<const uint8_t*>(a.src[r]) + static_cast<uint64_t>(nFull) * slice * esz;
+                    a.dst[r] = static_cast<uint8_t*>(a.dst[r]) + static_cast<uint64_t>(nFull) * slice * esz;
+                }
+                rc = LaunchMeshChunk(w, plan, p, a, nFull, 1, rest, 0, false, s);
+                if (rc != HCCL_SUCCESS) {
+                    return rc;
+                }
+            }
+            done += len;
+        }
+        return HCCL_SUCCESS;
     }
     a.nSub = n;
     a.progSubStride = 1;
@@ -648,6 +724,32 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
     a.prog = plan.dev;
     a.nDst = 1;
     a.dstOwn = 1;
+    if (algo == HCCL_AMD_ALGO_MESH_CHUNK) {
+        // The executor loops over the staging buffer, of which this template keeps n - 1 slots (reference
+        // ins_temp_reduce_scatter_mesh_1D_meshchunk.cc:119-125, ins_v2_reduce_scatter_sole_executor.cc:212-277);
+        // every loop cuts its share of each rank's output into segments of its own.
+        const uint32_t esz = DataTypeSize(p.dtype);
+        uint64_t maxPerLoop = p.count;
+        if (w->cclBytes != 0) {
+            maxPerLoop = SoleMaxCountPerLoop(w->cclBytes, n - 1, esz);
+            if (maxPerLoop == 0) {
+                return HCCL_E_INTERNAL;
+            }
+        }
+        for (uint64_t done = 0; done < p.count;) {
+            const uint64_t len = std::min(p.count - done, maxPerLoop);
+            for (uint32_t r = 0; r < n; ++r) {
+                a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + done * esz;
+                a.dst[r] = static_cast<uint8_t*>(p.ranks[r].recv) + done * esz;
+            }
+            rc = LaunchMeshChunk(w, plan, p, a, 0, n, len, p.count, true, s);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+            done += len;
+        }
+        return HCCL_SUCCESS;
+    }
     a.nGroup = n;
     a.groupLen = p.count;                  // input slice stride = recvCount (reference
     a.srcGroupStride = p.count;            // ins_v2_reduce_scatter_sole_executor.cc:260)
@@ -842,10 +944,39 @@ HcclResult RunReduceScatterV(World* w, PendingOp& p, hipStream_t s)
     if (longest == 0) {
         return HCCL_SUCCESS;
     }
+    const bool meshChunk = w->algo[HCCL_AMD_OP_REDUCE_SCATTER] == HCCL_AMD_ALGO_MESH_CHUNK;
     DevicePlan plan;
-    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, HCCL_AMD_ALGO_MESH, &plan);
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, meshChunk ? HCCL_AMD_ALGO_MESH_CHUNK : HCCL_AMD_ALGO_MESH,
+                                  &plan);
     if (rc != HCCL_SUCCESS) {
         return rc;
+    }
+    if (meshChunk) {
+        // Always one loop; the reference refuses a count its single accumulation slot cannot hold (reference
+        // ins_v2_reduce_scatter_v_sole_executor.cc:158-171, ins_temp_reduce_scatter_v_mesh_1D_meshchunk.cc:49-55).
+        const uint32_t esz = DataTypeSize(p.dtype);
+        if (w->cclBytes != 0 && longest > SoleMaxCountPerLoop(w->cclBytes, 1, esz)) {
+            Log(1, "ReduceScatterV: %llu elements exceed the staging buffer of %llu bytes in the mesh-chunk order",
+                static_cast<unsigned long long>(longest), static_cast<unsigned long long>(w->cclBytes));
+            return HCCL_E_NOT_SUPPORT;
+        }
+        for (uint32_t k = 0; k < n; ++k) {
+            if (ref[k] == 0) {
+                continue;
+            }
+            ReduceArgs a{};
+            for (uint32_t r = 0; r < n; ++r) {
+                a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + ref[n + k] * esz;
+            }
+            a.dst[0] = p.ranks[k].recv;
+            a.nDst = 1;
+            a.dstOwn = 1;
+            rc = LaunchMeshChunk(w, plan, p, a, k, 1, ref[k], 0, true, s);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+        }
+        return HCCL_SUCCESS;
     }
     ReduceArgs a{};
     for (uint32_t r = 0; r < n; ++r) {
@@ -963,12 +1094,43 @@ HcclResult RunSingleRank(World* w, PendingOp& p, hipStream_t s)
     return RunBcast(w, b, s);
 }
 
+// Makes the world's device current for the calling thread while the launch is prepared (the last rank to
+// arrive may run on a thread that never selected a device) and puts the previous one back afterwards.
+struct DeviceScope {
+    int previous = -1;
+    explicit DeviceScope(int device)
+    {
+        int current = -1;
+        if (hipGetDevice(&current) == hipSuccess && current != device && hipSetDevice(device) == hipSuccess) {
+            previous = current;
+        }
+    }
+    ~DeviceScope()
+    {
+        if (previous >= 0) {
+            (void)hipSetDevice(previous);
+        }
+    }
+};
+
 HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
 {
+    DeviceScope onWorldDevice(w->device);
     hipStream_t s = p.ranks[launcher].stream;
     // Order the fused kernel after everything queued so far on the other ranks' streams (a superset of
     // what each rank had queued when it called).  Ranks that share the launch stream need nothing.
     std::vector<hipEvent_t> used;
+    // Events go back to the pool on every path out of here.
+    struct Returner {
+        World* w;
+        std::vector<hipEvent_t>& used;
+        ~Returner()
+        {
+            for (hipEvent_t ev : used) {
+                w->eventPool.push_back(ev);
+            }
+        }
+    } returner{w, used};
     for (uint32_t r = 0; r < w->n; ++r) {
         if (p.ranks[r].stream == s) {
             continue;
@@ -1020,9 +1182,6 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
                 HIP_OK(hipStreamWaitEvent(p.ranks[r].stream, w->doneEvent, 0));
             }
         }
-    }
-    for (hipEvent_t ev : used) {
-        w->eventPool.push_back(ev);
     }
     return rc;
 }
@@ -1113,7 +1272,7 @@ using namespace hccl_amd;
 
 namespace {
 
-// A rank whose stream differs from the launcher's must have its position recorded at call time.
+// Common tail of every entry point: the environment verdict, then the rendezvous.
 HcclResult SubmitWithReady(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count,
                            const void* send, void* recv, aclrtStream stream, std::vector<uint64_t>&& var,
                            uint32_t root = 0)
@@ -1753,10 +1912,21 @@ HcclResult HcclAmdGetFoldProgram(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t ra
                                  uint8_t* out, uint32_t cap, uint32_t* len, uint32_t* segmentCount)
 {
     CHK_PTR(len, "len");
-    FoldPlan plan;
-    HcclResult rc = BuildFoldPlan(op, algo, rankSize, &plan);
-    if (rc != HCCL_SUCCESS) {
-        return rc;
+    // Callers walk all segments of one plan: keep the last plan built.
+    static std::mutex cacheMu;
+    static FoldPlan plan;
+    static int cachedOp = -1, cachedAlgo = -1;
+    static uint32_t cachedSize = 0;
+    std::lock_guard<std::mutex> cacheLock(cacheMu);
+    if (cachedOp != static_cast<int>(op) || cachedAlgo != static_cast<int>(algo) || cachedSize != rankSize) {
+        cachedOp = -1;
+        HcclResult rc = BuildFoldPlan(op, algo, rankSize, &plan);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+        cachedOp = static_cast<int>(op);
+        cachedAlgo = static_cast<int>(algo);
+        cachedSize = rankSize;
     }
     if (segmentCount != nullptr) {
         *segmentCount = static_cast<uint32_t>(plan.programs.size());

@@ -173,6 +173,48 @@ HcclResult AivMeshReduceScatter(uint32_t n, FoldPlan* plan)
     return HCCL_SUCCESS;
 }
 
+// ---- mesh chunk --------------------------------------------------------------------------------
+// Every slice is cut into N - 1 segments.  In step s a rank sends, for i = 0 .. N-2, segment i of the slice of
+// the rank `num` places below it, num = s + i + 1, one more once that reaches N (which skips the sender itself),
+// and the owner write-reduces it into its copy, which began as its own input (reference
+// ins_temp_reduce_scatter_mesh_1D_meshchunk.cc:277-375, ins_temp_reduce_scatter_v_mesh_1D_meshchunk.cc:202-265,
+// ins_temp_all_reduce_mesh_1D_two_shot_mesh_chunk.cc:220-295).  Program k * (N - 1) + i is segment i of slice k.
+HcclResult MeshChunk(uint32_t n, FoldPlan* plan)
+{
+    if (n == 1) {
+        return Emit(Leaf(0), plan);
+    }
+    const uint32_t segs = n - 1;
+    std::vector<std::vector<ExprPtr>> held(n, std::vector<ExprPtr>(segs));
+    for (uint32_t k = 0; k < n; ++k) {
+        for (uint32_t i = 0; i < segs; ++i) {
+            held[k][i] = Leaf(k);
+        }
+    }
+    for (uint32_t step = 0; step < segs; ++step) {
+        for (uint32_t i = 0; i < segs; ++i) {
+            uint32_t num = step + i + 1;
+            if (num >= n) {
+                num += 1;
+            }
+            for (uint32_t sender = 0; sender < n; ++sender) {
+                const uint32_t next = (sender + num) % n;
+                const uint32_t owner = (2 * sender + n - next) % n;
+                held[owner][i] = Fold(held[owner][i], Leaf(sender));
+            }
+        }
+    }
+    for (uint32_t k = 0; k < n; ++k) {
+        for (uint32_t i = 0; i < segs; ++i) {
+            HcclResult rc = Emit(held[k][i], plan);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
 // ---- order preserved ---------------------------------------------------------------------------
 // while blocks > 1: M = largest power of two below blocks; block src in [M, blocks) folds into block
 // src % M; blocks = M (reference ins_temp_reduce_scatter_order_preserved_group.cc:353-398).
@@ -346,6 +388,9 @@ HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPla
             // Slice k of the AllReduce result is folded like rank k's ReduceScatter output.
             plan->segmentsAreSubs = ar;
             return MeshReduceScatter(n, plan);
+        case HCCL_AMD_ALGO_MESH_CHUNK:
+            plan->segmentsAreSubs = true;
+            return MeshChunk(n, plan);
         default:
             return HCCL_E_PARA;
     }
@@ -394,6 +439,33 @@ HcclResult RhdMaxCountPerLoop(uint64_t cclBytes, uint64_t count, uint32_t p, uin
     }
     *maxCount = workspace / 2 / 128 * 128 / elemSize / p * p;
     return *maxCount == 0 ? HCCL_E_INTERNAL : HCCL_SUCCESS;
+}
+
+std::vector<SegmentRun> MeshChunkSegments(uint64_t len, uint32_t n, uint32_t elemSize, bool alignTo4K)
+{
+    std::vector<SegmentRun> runs;
+    if (len == 0 || n < 2 || elemSize == 0) {
+        return runs;
+    }
+    const uint64_t segs = n - 1;
+    if (alignTo4K) {
+        const uint64_t alignedBytes = (len * elemSize / segs) / 4096 * 4096;
+        if (segs >= 2 && alignedBytes > 0) {
+            const uint64_t segLen = alignedBytes / elemSize;
+            runs.push_back({0, 0, static_cast<uint32_t>(segs), segLen, len - segLen * (segs - 1)});
+            return runs;
+        }
+    }
+    const uint64_t small = len / segs;
+    const uint32_t nBig = static_cast<uint32_t>(len % segs);
+    if (nBig != 0) {
+        runs.push_back({0, 0, nBig, small + 1, small + 1});
+    }
+    if (small != 0) {
+        runs.push_back({static_cast<uint64_t>(nBig) * (small + 1), nBig, static_cast<uint32_t>(segs) - nBig, small,
+                        small});
+    }
+    return runs;
 }
 
 uint64_t RhdSelectLoopCount(uint64_t remaining, uint64_t maxCountPerLoop, uint64_t p)

@@ -27,6 +27,22 @@ uint32_t RhdPairCount(uint32_t p);                    // r = p - 2^floor(log2 p)
 uint32_t RhdSlotOfRank(uint32_t p, uint32_t rank);    // sigma: t -> 2t, t+r -> 2t+1, others identity
 uint32_t RhdCarrierOfVirtual(uint32_t p, uint32_t v); // physical rank that plays virtual rank v
 
+// Segments of one slice under the mesh-chunk order, as runs of equally long neighbours: segments
+// [firstSeg, firstSeg + nSeg) start `first` elements into the slice, hold segLen elements each and lastLen in the
+// last one.  With alignTo4K (ReduceScatter, ReduceScatterV) the first N - 2 segments are floor(bytes / (N - 1))
+// rounded down to 4 KiB and the last takes the rest; slices too small for that, and AllReduce always, are dealt
+// element-wise, the first len mod (N - 1) segments one element longer, possibly leaving empty segments
+// (reference ins_temp_reduce_scatter_mesh_1D_meshchunk.cc:233-258,
+// ins_temp_reduce_scatter_v_mesh_1D_meshchunk.cc:147-191, ins_temp_all_reduce_mesh_1D_two_shot_mesh_chunk.cc:181-199).
+struct SegmentRun {
+    uint64_t first;
+    uint32_t firstSeg;
+    uint32_t nSeg;
+    uint64_t segLen;
+    uint64_t lastLen;
+};
+std::vector<SegmentRun> MeshChunkSegments(uint64_t len, uint32_t rankSize, uint32_t elemSize, bool alignTo4K);
+
 // Loop limits of the reference's executors, which stage every AllReduce through a bounded buffer and cut the
 // count into loops that are each sliced afresh.  cclBytes is that buffer's size.
 // HCCL_BUFFSIZE (MB, digits only, 2 .. UINT32_MAX) less the 1 MiB kept back; nullptr = unset = 200 MB

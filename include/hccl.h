@@ -184,6 +184,16 @@ typedef enum {
      * N slices of ceil(count / N) elements and slice k starts from rank k's input, then adds the other
      * ranks ascending (reference ins_temp_all_reduce_mesh_1D_two_shot.cc:341-357).  ReduceScatter: MESH. */
     HCCL_AMD_ALGO_MESH_SYMMETRIC = 6,
+    /* The mesh order the reference's selector picks for large messages: every slice (a rank's ReduceScatter(V)
+     * output; for AllReduce one of N slices of ceil(count / N) elements) is cut into N - 1 segments, and segment
+     * i of slice k starts from rank k's input, then adds ranks k+i+1, k+i+2, ... wrapping past k
+     * (reference ins_temp_reduce_scatter_mesh_1D_meshchunk.cc:233-375,
+     * ins_temp_reduce_scatter_v_mesh_1D_meshchunk.cc:147-265,
+     * ins_temp_all_reduce_mesh_1D_two_shot_mesh_chunk.cc:177-295).  ReduceScatter(V) segments are
+     * floor(bytes / (N - 1)) rounded down to 4 KiB with the last one taking the rest, or dealt element-wise when
+     * that is zero; AllReduce segments are always dealt element-wise.  Set for ReduceScatter it also governs
+     * ReduceScatterV, which otherwise always uses MESH. */
+    HCCL_AMD_ALGO_MESH_CHUNK = 7,
     HCCL_AMD_ALGO_COUNT
 } HcclAmdAlgo;
 
@@ -196,12 +206,14 @@ HcclResult HcclAmdGetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo* algo);
  * Staging-buffer loops.  The reference's executors move every AllReduce through a bounded buffer: the count is
  * cut into loops and each loop is sliced afresh (ins_v2_all_reduce_sole_executor.cc:241-300,
  * ins_v2_all_reduce_sequence_executor_aicpu.cc:645-760), so under the orders whose fold depends on the slice
- * (NHR, RHD) the association order of an element depends on the loop it falls in.  No staging exists here;
+ * (NHR, RHD, MESH_CHUNK) the association order of an element depends on the loop it falls in.  No staging exists here;
  * `bytes` only tells the library which loop boundaries to reproduce: 0 (default) = one loop.  The environment
  * variable HCCL_BUFFSIZE (MB), when set at world creation, gives MB * 2^20 - 2^20 bytes
  * (src/common/op_graph/hccl_op_utils.cc:204-225); a value its parser rejects makes every collective return
- * HCCL_E_PARA.  Orders that fold every position alike (MESH, RING, ORDER_PRESERVED) and ReduceScatter, whose
- * fold depends on the receiving rank only, are not affected; MESH_SYMMETRIC always runs as one loop
+ * HCCL_E_PARA.  Orders that fold every position alike (MESH, RING, ORDER_PRESERVED) and ReduceScatter under the
+ * orders whose fold depends on the receiving rank only are not affected; MESH_CHUNK ReduceScatter loops over the
+ * buffer's N - 1 slots, MESH_CHUNK ReduceScatterV runs one loop and returns HCCL_E_NOT_SUPPORT for a slice the
+ * buffer cannot hold (ins_v2_reduce_scatter_v_sole_executor.cc:158-171); MESH_SYMMETRIC always runs as one loop
  * (ins_v2_all_reduce_sole_executor.cc:273-282).  A buffer too small for one loop returns HCCL_E_INTERNAL from the
  * collective, like the reference.
  */

@@ -198,6 +198,14 @@ def nhr_step_info(n, rank, step):
     return rc, to.value, frm.value, list(tx[:cnt.value]), list(rx[:cnt.value])
 
 
+def mesh_chunk_segments(length, n, elem_size, align4k):
+    """Element counts of the n - 1 segments of a slice."""
+    out = (ctypes.c_uint64 * max(n - 1, 1))()
+    lib().orc_mesh_chunk_segments(ctypes.c_uint64(length), ctypes.c_uint32(n), ctypes.c_uint32(elem_size),
+                                  int(align4k), out)
+    return list(out[:max(n - 1, 0)])
+
+
 def ccl_buffer_available_size(env_value):
     """(rc, bytes) for a HCCL_BUFFSIZE string, None = unset."""
     out = ctypes.c_uint64(0)
@@ -256,10 +264,16 @@ def all_reduce(ins, outs, count, dtype, op, acc=ACC_FP32, algo="mesh", max_count
                             ctypes.c_uint64(max_count_per_loop))
     if algo == "order_preserved":
         return _reduce_call("orc_all_reduce_order_preserved", ins, outs, count, dtype, op, acc)
+    if algo == "mesh_chunk":
+        return _reduce_call("orc_all_reduce_mesh_chunk", ins, outs, count, dtype, op, acc,
+                            ctypes.c_uint64(max_count_per_loop))
     raise ValueError(algo)
 
 
-def reduce_scatter(ins, outs, recv_count, dtype, op, acc=ACC_FP32, algo="mesh"):
+def reduce_scatter(ins, outs, recv_count, dtype, op, acc=ACC_FP32, algo="mesh", max_count_per_loop=0):
+    if algo == "mesh_chunk":
+        return _reduce_call("orc_reduce_scatter_mesh_chunk", ins, outs, recv_count, dtype, op, acc,
+                            ctypes.c_uint64(max_count_per_loop))
     name = {"mesh": "orc_reduce_scatter_mesh", "mesh_symmetric": "orc_reduce_scatter_mesh", "nhr": "orc_reduce_scatter_nhr", "ring": "orc_reduce_scatter_nhr",
             "rhd": "orc_reduce_scatter_rhd", "order_preserved": "orc_reduce_scatter_order_preserved",
             "aiv_mesh": "orc_reduce_scatter_aiv_mesh"}[algo]
@@ -315,11 +329,11 @@ def all_to_all_vc(ins, outs, matrix, dtype):
     return lib().orc_all_to_all_vc(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs), mp, dtype)
 
 
-def reduce_scatter_v(ins, outs, counts, displs, dtype, op, acc=ACC_FP32):
+def reduce_scatter_v(ins, outs, counts, displs, dtype, op, acc=ACC_FP32, algo="mesh"):
     c, cp = _u64(counts)
     d, dp = _u64(displs)
-    return lib().orc_reduce_scatter_v_mesh(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs), cp, dp,
-                                           dtype, op, acc)
+    fn = {"mesh": "orc_reduce_scatter_v_mesh", "mesh_chunk": "orc_reduce_scatter_v_mesh_chunk"}[algo]
+    return getattr(lib(), fn)(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs), cp, dp, dtype, op, acc)
 
 
 def reduce(ins, outs, count, dtype, op, root, acc=ACC_FP32):

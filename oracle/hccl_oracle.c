@@ -1423,6 +1423,211 @@ int orc_reduce_scatter_aiv_mesh(uint32_t n, const void* const* in, void* const* 
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * Mesh-chunk order (reduce_scatter_mesh_1D_meshchunk.cc, reduce_scatter_v_mesh_1D_meshchunk.cc,
+ * all_reduce_mesh_1D_two_shot_mesh_chunk.cc)
+ * ------------------------------------------------------------------------------------------- */
+/* Sizes in elements of the n - 1 segments of a slice of len elements.  align4k: the ReduceScatter(V) rule
+ * (meshchunk.cc:233-258, v_meshchunk.cc:147-191): floor(bytes / (n-1)) rounded down to 4096 bytes for all but
+ * the last segment, which takes the rest; when that is zero or n - 1 < 2, and always for AllReduce
+ * (two_shot_mesh_chunk.cc:181-199), element-wise with the first len mod (n-1) segments one longer. */
+#define ORC_MAX_RANKS 1024u   /* bound of the stack tables below */
+
+void orc_mesh_chunk_segments(uint64_t len, uint32_t n, uint32_t elemSize, int align4k, uint64_t* segLen)
+{
+    if (n < 2) {
+        return;
+    }
+    uint64_t segs = n - 1;
+    uint64_t aligned = align4k ? (len * elemSize / segs) / 4096 * 4096 : 0;
+    if (align4k && segs >= 2 && aligned > 0) {
+        for (uint64_t i = 0; i + 1 < segs; ++i) segLen[i] = aligned / elemSize;
+        segLen[segs - 1] = len - (aligned / elemSize) * (segs - 1);
+        return;
+    }
+    uint64_t big = len % segs;
+    for (uint64_t i = 0; i < segs; ++i) segLen[i] = len / segs + (i < big ? 1 : 0);
+}
+
+/* The exchange itself: slice k (sliceLen[k] elements, sliceOff[k] elements into every input) starts as rank
+ * k's own input (PreCopy / LocalDataCopy); in step s every sender pushes, for i = 0 .. n-2, segment i of the
+ * slice of the rank num = s + i + 1 (+1 from n on) places below it, and the owner write-reduces it
+ * (DoMeshChunk, meshchunk.cc:277-375; v_meshchunk.cc:202-265; two_shot_mesh_chunk.cc:220-295).
+ * acc[k] receives the widened result of slice k. */
+static int mesh_chunk_exchange(const red_t* r, uint32_t n, const void* const* in, const uint64_t* sliceOff,
+                               const uint64_t* sliceLen, int align4k, void** acc)
+{
+    uint64_t longest = 0;
+    for (uint32_t k = 0; k < n; ++k) longest = sliceLen[k] > longest ? sliceLen[k] : longest;
+    void* tmp = malloc((longest ? longest : 1) * r->asz);
+    uint64_t* seg = (uint64_t*)malloc(sizeof(uint64_t) * n * n);
+    uint64_t* off = (uint64_t*)malloc(sizeof(uint64_t) * n * n);
+    if (!tmp || !seg || !off) {
+        free(tmp);
+        free(seg);
+        free(off);
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t k = 0; k < n; ++k) {
+        red_widen(r, cbytes(in[k]) + sliceOff[k] * r->esz, acc[k], sliceLen[k]);
+        orc_mesh_chunk_segments(sliceLen[k], n, (uint32_t)r->esz, align4k, seg + (size_t)k * n);
+        uint64_t o = 0;
+        for (uint32_t i = 0; i + 1 < n; ++i) {
+            off[(size_t)k * n + i] = o;
+            o += seg[(size_t)k * n + i];
+        }
+    }
+    for (uint32_t step = 0; step + 1 < n; ++step) {
+        for (uint32_t i = 0; i + 1 < n; ++i) {
+            uint32_t num = step + i + 1;
+            if (num >= n) {
+                num += 1;
+            }
+            for (uint32_t sender = 0; sender < n; ++sender) {
+                uint32_t next = (sender + num) % n;
+                uint32_t owner = (2 * sender + n - next) % n;
+                uint64_t cnt = seg[(size_t)owner * n + i];
+                uint64_t at = off[(size_t)owner * n + i];
+                if (cnt != 0) {
+                    red_pair_from_storage(r, bytes(acc[owner]) + at * r->asz,
+                                          cbytes(in[sender]) + (sliceOff[owner] + at) * r->esz, cnt, tmp);
+                }
+            }
+        }
+    }
+    free(tmp);
+    free(seg);
+    free(off);
+    return ORC_OK;
+}
+
+static int mesh_chunk_run(const red_t* r, uint32_t n, const void* const* in, const uint64_t* sliceOff,
+                          const uint64_t* sliceLen, int align4k, void** acc)
+{
+    for (uint32_t k = 0; k < n; ++k) {
+        acc[k] = malloc((sliceLen[k] ? sliceLen[k] : 1) * r->asz);
+        if (!acc[k]) {
+            for (uint32_t j = 0; j < k; ++j) free(acc[j]);
+            return ORC_E_INTERNAL;
+        }
+    }
+    int rc = mesh_chunk_exchange(r, n, in, sliceOff, sliceLen, align4k, acc);
+    if (rc != ORC_OK) {
+        for (uint32_t k = 0; k < n; ++k) free(acc[k]);
+    }
+    return rc;
+}
+
+int orc_reduce_scatter_mesh_chunk(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                                  int op, int accMode, uint64_t maxCountPerLoop)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK || recvCount == 0) {
+        return rc;
+    }
+    if (n == 0 || n > ORC_MAX_RANKS) {
+        return ORC_E_PARA;
+    }
+    if (n == 1) {
+        memmove(out[0], in[0], recvCount * r.esz);
+        return ORC_OK;
+    }
+    if (maxCountPerLoop == 0) {
+        maxCountPerLoop = recvCount;
+    }
+    uint64_t sliceOff[ORC_MAX_RANKS], sliceLen[ORC_MAX_RANKS];
+    void* acc[ORC_MAX_RANKS];
+    /* reduce_scatter_sole_executor.cc:250-277: full loops, the last one takes what is left */
+    for (uint64_t done = 0; done < recvCount && rc == ORC_OK;) {
+        uint64_t cur = recvCount - done < maxCountPerLoop ? recvCount - done : maxCountPerLoop;
+        for (uint32_t k = 0; k < n; ++k) {
+            sliceOff[k] = (uint64_t)k * recvCount + done;
+            sliceLen[k] = cur;
+        }
+        rc = mesh_chunk_run(&r, n, in, sliceOff, sliceLen, 1, acc);
+        if (rc == ORC_OK) {
+            for (uint32_t k = 0; k < n; ++k) {
+                red_narrow(&r, acc[k], bytes(out[k]) + done * r.esz, cur);
+                free(acc[k]);
+            }
+        }
+        done += cur;
+    }
+    return rc;
+}
+
+int orc_reduce_scatter_v_mesh_chunk(uint32_t n, const void* const* in, void* const* out, const uint64_t* counts,
+                                    const uint64_t* displs, int dtype, int op, int accMode)
+{
+    if (dtype == ORC_UINT64 || dtype == ORC_FP64) {
+        return ORC_E_NOT_SUPPORT;   /* reduce_scatter_v.cc:231-236 */
+    }
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (n == 0 || n > ORC_MAX_RANKS) {
+        return ORC_E_PARA;
+    }
+    if (n == 1) {
+        memmove(out[0], in[0], counts[0] * r.esz);     /* op_common.cc:4490-4491: from the start of sendBuf */
+        return ORC_OK;
+    }
+    void* acc[ORC_MAX_RANKS];
+    rc = mesh_chunk_run(&r, n, in, displs, counts, 1, acc);     /* always one loop (v_sole_executor.cc:158-171) */
+    if (rc == ORC_OK) {
+        for (uint32_t k = 0; k < n; ++k) {
+            red_narrow(&r, acc[k], out[k], counts[k]);
+            free(acc[k]);
+        }
+    }
+    return rc;
+}
+
+int orc_all_reduce_mesh_chunk(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                              int accMode, uint64_t maxCountPerLoop)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK || count == 0) {
+        return rc;
+    }
+    if (n == 0 || n > ORC_MAX_RANKS) {
+        return ORC_E_PARA;
+    }
+    if (n == 1) {
+        memmove(out[0], in[0], count * r.esz);
+        return ORC_OK;
+    }
+    if (maxCountPerLoop == 0) {
+        maxCountPerLoop = count;
+    }
+    uint64_t sliceOff[ORC_MAX_RANKS], sliceLen[ORC_MAX_RANKS];
+    void* acc[ORC_MAX_RANKS];
+    for (uint64_t done = 0; done < count && rc == ORC_OK;) {
+        uint64_t cur = count - done < maxCountPerLoop ? count - done : maxCountPerLoop;
+        uint64_t chunk = orc_round_up(cur, n);          /* two_shot_mesh_chunk.cc:86-112 */
+        for (uint32_t k = 0; k < n; ++k) {
+            uint64_t at = (uint64_t)k * chunk;
+            sliceOff[k] = done + (at < cur ? at : cur);
+            sliceLen[k] = at >= cur ? 0 : (cur - at > chunk ? chunk : cur - at);
+        }
+        rc = mesh_chunk_run(&r, n, in, sliceOff, sliceLen, 0, acc);
+        if (rc == ORC_OK) {
+            for (uint32_t k = 0; k < n; ++k) {
+                for (uint32_t m = 0; m < n; ++m) {
+                    red_narrow(&r, acc[k], bytes(out[m]) + sliceOff[k] * r.esz, sliceLen[k]);
+                }
+                free(acc[k]);
+            }
+        }
+        done += cur;
+    }
+    return rc;
+}
+
+/* ---------------------------------------------------------------------------------------------
  * a13 / a14 / a15: copies
  * ------------------------------------------------------------------------------------------- */
 static int copy_dtype_ok(int dtype)

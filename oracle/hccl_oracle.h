@@ -139,6 +139,18 @@ int orc_all_reduce_order_preserved(uint32_t n, const void* const* in, void* cons
 /* vector-core mesh order (aiv_reduce_scatter_mesh_1d.h:23-71). */
 int orc_reduce_scatter_aiv_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
                                 int op, int accMode);
+/* Mesh-chunk order, the mesh variant the reference's selectors pick for large messages: every slice is cut
+ * into n - 1 segments, segment i of slice k = x_k, then x_{k+i+1}, x_{k+i+2}, ... wrapping past k.
+ * reduce_scatter_mesh_1D_meshchunk.cc:233-375, reduce_scatter_v_mesh_1D_meshchunk.cc:147-265,
+ * all_reduce_mesh_1D_two_shot_mesh_chunk.cc:86-112, 177-295.  maxCountPerLoop: elements per executor loop, 0 = one
+ * loop; ReduceScatterV always runs one loop (reduce_scatter_v_sole_executor.cc:158-171). */
+void orc_mesh_chunk_segments(uint64_t len, uint32_t n, uint32_t elemSize, int align4k, uint64_t* segLen /* n-1 */);
+int orc_reduce_scatter_mesh_chunk(uint32_t n, const void* const* in, void* const* out, uint64_t recvCount, int dtype,
+                                  int op, int accMode, uint64_t maxCountPerLoop);
+int orc_reduce_scatter_v_mesh_chunk(uint32_t n, const void* const* in, void* const* out, const uint64_t* counts,
+                                    const uint64_t* displs, int dtype, int op, int accMode);
+int orc_all_reduce_mesh_chunk(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                              int accMode, uint64_t maxCountPerLoop);
 /* One-level NHR AllReduce (ins_temp_all_reduce_nhr.cc:214-216, 646-687): slices of floor(count/n) elements, the
  * last slice takes the rest; every element follows the NHR reduce-scatter tree of its slice, then gather. */
 int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,

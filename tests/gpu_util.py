@@ -9,7 +9,8 @@ import hccl_amd
 from hccl_amd import Algo, OpKind
 
 ALGO_BY_NAME = {"mesh": Algo.MESH, "ring": Algo.RING, "rhd": Algo.RHD, "nhr": Algo.NHR,
-                "order_preserved": Algo.ORDER_PRESERVED, "aiv_mesh": Algo.AIV_MESH, "mesh_symmetric": Algo.MESH_SYMMETRIC}
+                "order_preserved": Algo.ORDER_PRESERVED, "aiv_mesh": Algo.AIV_MESH, "mesh_symmetric": Algo.MESH_SYMMETRIC,
+                "mesh_chunk": Algo.MESH_CHUNK}
 
 
 def require_library_on_gpu():
@@ -121,7 +122,8 @@ class World:
                 hccl_amd.all_to_all_vc(self.comms[r], sends[r], flat, dtype, recvs[r], dtype, self.stream)
         self.sync()
 
-    def reduce_scatter_v(self, sends, recvs, counts, displs, dtype, op):
+    def reduce_scatter_v(self, sends, recvs, counts, displs, dtype, op, algo="mesh"):
+        self.set_algo(OpKind.REDUCE_SCATTER, algo)
         self.inputs_ready()
         with hccl_amd.group():
             for r in range(self.n):

@@ -109,12 +109,13 @@ def run_all_reduce(world, dtype, op, count, algo, seed, pad=0, in_place=False, m
               "all_reduce %s %s n=%d count=%d algo=%s rank=%d" % (dtype.name, OP(op).name, n, count, algo, r))
 
 
-def run_reduce_scatter(world, dtype, op, c, algo, seed, pad=0):
+def run_reduce_scatter(world, dtype, op, c, algo, seed, pad=0, max_count_per_loop=0):
     rng = np.random.default_rng(seed)
     n = world.n
     ins = [gen(dtype, op, rng, n * c) for _ in range(n)]
     want = [np.zeros(c, dtype=NP[dtype]) for _ in range(n)]
-    assert oracle.reduce_scatter(ins, want, c, int(dtype), op, acc=oracle.ACC_FP32, algo=algo) == 0
+    kw = {"max_count_per_loop": max_count_per_loop} if max_count_per_loop else {}
+    assert oracle.reduce_scatter(ins, want, c, int(dtype), op, acc=oracle.ACC_FP32, algo=algo, **kw) == 0
     sends = [to_dev(x, pad_of(pad, r, "send")) for r, x in enumerate(ins)]
     recvs = [dev_zeros(c * ins[0].itemsize, pad_of(pad, r, "recv")) for r in range(n)]
     world.reduce_scatter(sends, recvs, c, dtype, op, algo)
@@ -155,7 +156,7 @@ def test_reduce_scatter_type_matrix(world8, dtype, op):
 def test_all_reduce_algorithms_and_ragged_counts(n):
     w = World(n)
     try:
-        for algo in ("mesh", "ring", "rhd", "nhr", "order_preserved", "mesh_symmetric"):
+        for algo in ("mesh", "ring", "rhd", "nhr", "order_preserved", "mesh_symmetric", "mesh_chunk"):
             for count in (1, 3, 17, 129, 1023, 4093, 65_543):
                 run_all_reduce(w, DT.FP32, SUM, count, algo, seed=n * 1000 + count)
             run_all_reduce(w, DT.FP32, MAX, 2_051, algo, seed=n)
@@ -169,7 +170,7 @@ def test_all_reduce_algorithms_and_ragged_counts(n):
 def test_reduce_scatter_algorithms_and_ragged_counts(n):
     w = World(n)
     try:
-        for algo in ("mesh", "ring", "nhr", "rhd", "order_preserved", "aiv_mesh", "mesh_symmetric"):
+        for algo in ("mesh", "ring", "nhr", "rhd", "order_preserved", "aiv_mesh", "mesh_symmetric", "mesh_chunk"):
             for c in (1, 3, 17, 129, 1024, 4093):
                 run_reduce_scatter(w, DT.FP32, SUM, c, algo, seed=n * 2000 + c)
             run_reduce_scatter(w, DT.FP32, MIN, 515, algo, seed=n + 3)
@@ -408,6 +409,29 @@ def test_all_reduce_follows_staging_buffer_loops(n, algo):
         w.set_ccl_buffer_size(4096)
         run_all_reduce(w, DT.FP32, SUM, 10_001, "mesh", seed=78)
         run_all_reduce(w, DT.FP32, SUM, 10_001, "mesh_symmetric", seed=79)
+    finally:
+        w.set_ccl_buffer_size(0)
+        w.close()
+
+
+@pytest.mark.parametrize("n", [2, 3, 8, 16])
+def test_mesh_chunk_order_with_aligned_segments_and_staging_loops(n):
+    """Slices long enough for the 4 KiB rule, odd sizes, several types; then the executor's loops, which cut
+    every loop's share into segments of its own."""
+    w = World(n)
+    try:
+        for dtype, c in ((DT.FP32, 100_000), (DT.FP32, 7 * 1024 * (n - 1) - 1), (DT.BFP16, 300_001), (DT.INT8, 77_777),
+                         (DT.FP16, 65_536)):
+            run_reduce_scatter(w, dtype, SUM, c, "mesh_chunk", seed=n * 7 + c % 91)
+            run_all_reduce(w, dtype, SUM, c + 13, "mesh_chunk", seed=n * 9 + c % 89)
+        run_reduce_scatter(w, DT.FP32, MAX, 50_001, "mesh_chunk", seed=5, pad=lambda r, which: 4 * (r % 4))
+        run_all_reduce(w, DT.FP32, MIN, 50_001, "mesh_chunk", seed=6, in_place=True)
+        ccl = 1 << 20
+        w.set_ccl_buffer_size(ccl)
+        run_reduce_scatter(w, DT.FP32, SUM, 300_000, "mesh_chunk", seed=7,
+                           max_count_per_loop=oracle.sole_max_count_per_loop(ccl, n - 1, 4))
+        run_all_reduce(w, DT.FP32, SUM, 700_001, "mesh_chunk", seed=8,
+                       max_count_per_loop=oracle.sole_max_count_per_loop(ccl, 2, 4))
     finally:
         w.set_ccl_buffer_size(0)
         w.close()

@@ -101,17 +101,17 @@ def rsv_layout(rng, n, lo, hi, layout, esz):
     return counts, displs, off + 5
 
 
-def run_rsv(w, dtype, op, lo, hi, layout, seed, pad=0):
+def run_rsv(w, dtype, op, lo, hi, layout, seed, pad=0, algo="mesh"):
     n = w.n
     rng = np.random.default_rng(seed)
     esz = np.dtype(NP[dtype]).itemsize
     counts, displs, total = rsv_layout(rng, n, lo, hi, layout, esz)
     ins = [gen(dtype, op, rng, total) for _ in range(n)]
     want = [np.zeros(max(int(c), 1), dtype=NP[dtype]) for c in counts]
-    assert oracle.reduce_scatter_v(ins, want, counts, displs, int(dtype), op, acc=oracle.ACC_FP32) == 0
+    assert oracle.reduce_scatter_v(ins, want, counts, displs, int(dtype), op, acc=oracle.ACC_FP32, algo=algo) == 0
     sends = [to_dev(x, pad) for x in ins]
     recvs = [dev_zeros(x.nbytes, pad) for x in want]
-    w.reduce_scatter_v(sends, recvs, counts, displs, dtype, op)
+    w.reduce_scatter_v(sends, recvs, counts, displs, dtype, op, algo)
     for r in range(n):
         c = int(counts[r])
         got = to_host(recvs[r], NP[dtype])
@@ -138,6 +138,30 @@ def test_reduce_scatter_v_other_ops(worlds, dtype, op):
 def test_reduce_scatter_v_large_uneven_slices(worlds):
     run_rsv(worlds(6), DT.BFP16, SUM, 1 << 18, 1 << 21, "aligned", 5)
     run_rsv(worlds(6), DT.FP32, SUM, 1 << 16, 1 << 19, "prefix", 6, pad=4)
+
+
+@pytest.mark.parametrize("n", [2, 3, 8, 16])
+def test_reduce_scatter_v_mesh_chunk_order(worlds, n):
+    """Slices long enough for 4 KiB-aligned segments, slices dealt element-wise, and slices shorter than n - 1."""
+    w = worlds(n)
+    run_rsv(w, DT.FP32, SUM, 1, 40_000, "gaps", 900 + n, algo="mesh_chunk")
+    run_rsv(w, DT.FP32, SUM, 1, 12, "prefix", 910 + n, algo="mesh_chunk")
+    run_rsv(w, DT.BFP16, SUM, 1 << 14, 1 << 17, "aligned", 920 + n, algo="mesh_chunk")
+    run_rsv(w, DT.FP32, MAX, 1, 9_000, "gaps", 930 + n, pad=4, algo="mesh_chunk")
+    run_rsv(w, DT.FP32, SUM, 1, 5_000, "gaps", 940 + n)          # back to the plain mesh order
+
+
+def test_reduce_scatter_v_mesh_chunk_refuses_more_than_the_staging_buffer_holds(worlds):
+    w = worlds(3)
+    hccl_amd.set_ccl_buffer_size(w.comms[0], 4096)
+    try:
+        run_rsv(w, DT.FP32, SUM, 900, 1024, "prefix", 950, algo="mesh_chunk")       # at most 4096 bytes per slice
+        with pytest.raises(hccl_amd.HcclError) as e:
+            run_rsv(w, DT.FP32, SUM, 1025, 1100, "prefix", 951, algo="mesh_chunk")
+        assert e.value.code == 5
+    finally:
+        hccl_amd.set_ccl_buffer_size(w.comms[0], 0)
+        w.set_algo(hccl_amd.OpKind.REDUCE_SCATTER, "mesh")
 
 
 def test_reduce_scatter_v_counts_that_differ_between_ranks_are_rejected(worlds):

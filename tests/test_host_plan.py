@@ -93,7 +93,7 @@ def same(a, b):
 
 
 RANKS = [1, 2, 3, 5, 6, 7, 8, 12, 16, 33, 64]
-ALGO_NAME = {Algo.MESH: "mesh", Algo.RING: "ring", Algo.RHD: "rhd", Algo.NHR: "nhr",
+ALGO_NAME = {Algo.MESH_CHUNK: "mesh_chunk", Algo.MESH: "mesh", Algo.RING: "ring", Algo.RHD: "rhd", Algo.NHR: "nhr",
              Algo.ORDER_PRESERVED: "order_preserved", Algo.AIV_MESH: "aiv_mesh",
              Algo.MESH_SYMMETRIC: "mesh_symmetric"}
 
@@ -111,7 +111,7 @@ def test_every_program_uses_every_rank_once(n):
 
 @pytest.mark.parametrize("n", RANKS)
 @pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED, Algo.AIV_MESH,
-                                  Algo.MESH_SYMMETRIC])
+                                  Algo.MESH_SYMMETRIC, Algo.MESH_CHUNK])
 def test_reduce_scatter_programs_match_oracle(orc, n, algo):
     progs = hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, algo, n)
     c = 2 * n + 5
@@ -121,7 +121,15 @@ def test_reduce_scatter_programs_match_oracle(orc, n, algo):
         outs = [np.zeros(c, dtype=np.float32) for _ in range(n)]
         assert orc.reduce_scatter(ins, outs, c, F32, op, algo=ALGO_NAME[algo]) == 0
         for k in range(n):
-            if algo == Algo.AIV_MESH:
+            if algo == Algo.MESH_CHUNK and n > 1:
+                got = np.zeros(c, dtype=np.float32)
+                lo = 0
+                for i, ln in enumerate(orc.mesh_chunk_segments(c, n, 4, True)):
+                    if ln:
+                        got[lo:lo + ln] = run_program(progs[k * (n - 1) + i],
+                                                      lambda r: ins[r][k * c + lo:k * c + lo + ln], op)
+                    lo += ln
+            elif algo == Algo.AIV_MESH:
                 per = c // n
                 got = np.zeros(c, dtype=np.float32)
                 for ch in range(n):
@@ -135,7 +143,8 @@ def test_reduce_scatter_programs_match_oracle(orc, n, algo):
 
 
 @pytest.mark.parametrize("n", RANKS)
-@pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED, Algo.MESH_SYMMETRIC])
+@pytest.mark.parametrize("algo", [Algo.MESH, Algo.RING, Algo.RHD, Algo.NHR, Algo.ORDER_PRESERVED, Algo.MESH_SYMMETRIC,
+                                  Algo.MESH_CHUNK])
 def test_all_reduce_programs_match_oracle(orc, n, algo):
     progs = hccl_amd.fold_programs(OpKind.ALL_REDUCE, algo, n)
     count = 5 * n + 3
@@ -155,6 +164,14 @@ def test_all_reduce_programs_match_oracle(orc, n, algo):
                     got[lo:hi] = run_program(progs[i], lambda r: ins[r][lo:hi], op)
             for e in range(unit * n, count):
                 got[e:e + 1] = run_program(progs[e - unit * n], lambda r: ins[r][e:e + 1], op)
+        elif algo == Algo.MESH_CHUNK:
+            sl = -(-count // n)
+            for k in range(n):
+                lo = min(count, k * sl)
+                for i, ln in enumerate(orc.mesh_chunk_segments(max(0, min(sl, count - k * sl)), n, 4, False)):
+                    if ln:
+                        got[lo:lo + ln] = run_program(progs[k * (n - 1) + i], lambda r: ins[r][lo:lo + ln], op)
+                    lo += ln
         elif algo == Algo.NHR:       # floor slices, the last one takes the rest
             sl = count // n
             for i in range(n):
@@ -175,6 +192,11 @@ def test_known_programs():
     assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.MESH, 8) == [bytes([0xC8, 0, 1, 2, 3, 4, 5, 6, 7, 0xFF])]
     # own slice first
     assert hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.MESH, 4)[2] == bytes([0xC4, 2, 0, 1, 3, 0xFF])
+    # mesh chunk, 4 ranks, slice 1: segments fold 1,2,3,0 / 1,3,0,2 / 1,0,2,3
+    mc = hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.MESH_CHUNK, 4)
+    assert len(mc) == 12
+    assert mc[3:6] == [bytes([0xC4, 1, 2, 3, 0, 0xFF]), bytes([0xC4, 1, 3, 0, 2, 0xFF]), bytes([0xC4, 1, 0, 2, 3, 0xFF])]
+    assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.MESH_CHUNK, 4) == mc
     # p = 6: ((x0+x2)+x4) + ((x1+x3)+x5) for the share of rank 0
     p6 = hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.RHD, 6)
     assert p6[0] == bytes([0xC3, 0, 2, 4, 0x80, 0xC3, 1, 3, 5, 0x81, 0xFF])

@@ -206,6 +206,125 @@ def test_all_reduce_nhr_loop_re_cuts_slices(orc):
     assert np.count_nonzero(one_loop[0] != outs[0]) > 0           # wide-range inputs: the order shows
 
 
+# ---- mesh chunk ----------------------------------------------------------------------------------
+def test_mesh_chunk_segment_sizes(orc):
+    """ReduceScatter(V): floor(bytes / (n-1)) down to 4 KiB, the last takes the rest; too small: element-wise,
+    the first len mod (n-1) one longer.  AllReduce: always element-wise."""
+    # 8 ranks, fp32: 100000 el = 400000 B / 7 = 57142 -> 53248 B = 13312 el; last = 100000 - 6 * 13312
+    assert orc.mesh_chunk_segments(100000, 8, 4, True) == [13312] * 6 + [100000 - 6 * 13312]
+    # below 4 KiB per segment: 7000 B / 7 = 1000 B -> element-wise: 1750 el = 7 * 250
+    assert orc.mesh_chunk_segments(1750, 8, 4, True) == [250] * 7
+    assert orc.mesh_chunk_segments(1753, 8, 4, True) == [251] * 3 + [250] * 4
+    assert orc.mesh_chunk_segments(3, 8, 4, True) == [1, 1, 1, 0, 0, 0, 0]
+    # two ranks: a single segment, never the aligned rule
+    assert orc.mesh_chunk_segments(1 << 20, 2, 4, True) == [1 << 20]
+    # exactly 4 KiB per segment
+    assert orc.mesh_chunk_segments(7 * 1024, 8, 4, True) == [1024] * 7
+    assert orc.mesh_chunk_segments(7 * 1024 - 1, 8, 4, True) == [1024] * 6 + [1023]     # 28668 B / 7 = 4095 -> 0 -> element-wise
+    assert orc.mesh_chunk_segments(100000, 8, 4, False) == [14286] * 5 + [14285] * 2
+    # bf16: 3 ranks, 10000 el = 20000 B / 2 = 10000 -> 8192 B = 4096 el
+    assert orc.mesh_chunk_segments(10000, 3, 2, True) == [4096, 5904]
+    for n in (2, 3, 5, 8, 64):
+        for ln in (0, 1, n - 2, n - 1, 4097, 1 << 16):
+            for align in (True, False):
+                assert sum(orc.mesh_chunk_segments(ln, n, 2, align)) == ln
+
+
+def mesh_chunk_order(n, k, i):
+    """Ranks folded into segment i of slice k, worked out by hand from the step loop: step s delivers the
+    segment from the rank s + i + 1 places above k, places n .. n+i-1 standing for 1 .. i after the sender
+    skips itself: k, k+i+1, ..., k+n-1, k+1, ..., k+i."""
+    return [k] + [(k + d) % n for d in list(range(i + 1, n)) + list(range(1, i + 1))]
+
+
+def test_mesh_chunk_order_n4_by_hand():
+    # n = 4, slice 1: segment 0 <- 2, 3, 0 ; segment 1 <- 3, 0, 2 ; segment 2 <- 0, 2, 3
+    assert [mesh_chunk_order(4, 1, i) for i in range(3)] == [[1, 2, 3, 0], [1, 3, 0, 2], [1, 0, 2, 3]]
+
+
+@pytest.mark.parametrize("n,c", [(4, 3 * 5000), (8, 100000), (8, 1753), (3, 10000), (2, 777), (5, 3)])
+def test_reduce_scatter_mesh_chunk_rotation(orc, n, c):
+    rng = np.random.default_rng(300 + n + c)
+    ins = wide_f32(rng, n, n * c)
+    outs = outs_like(ins, c)
+    assert orc.reduce_scatter(ins, outs, c, F32, SUM, algo="mesh_chunk") == 0
+    segs = orc.mesh_chunk_segments(c, n, 4, True)
+    for k in range(n):
+        lo = 0
+        for i, ln in enumerate(segs):
+            order = mesh_chunk_order(n, k, i)
+            acc = ins[order[0]][k * c + lo:k * c + lo + ln].copy()
+            for t in order[1:]:
+                acc = ins[t][k * c + lo:k * c + lo + ln] + acc
+            assert np.array_equal(outs[k][lo:lo + ln].view(np.uint32), acc.view(np.uint32)), (k, i)
+            lo += ln
+    if n == 8 and c == 100000:
+        plain = rs_expected(ins, n, c, 3, [3] + [t for t in range(n) if t != 3])
+        assert np.count_nonzero(plain != outs[3]) > c // 10       # not the plain mesh order
+
+
+def test_reduce_scatter_mesh_chunk_loops_re_cut_segments(orc):
+    rng = np.random.default_rng(310)
+    n, c, per_loop = 4, 40000, 16384
+    ins = wide_f32(rng, n, n * c)
+    outs = outs_like(ins, c)
+    assert orc.reduce_scatter(ins, outs, c, F32, SUM, algo="mesh_chunk", max_count_per_loop=per_loop) == 0
+    for k in range(n):
+        for done in range(0, c, per_loop):
+            cur = min(per_loop, c - done)
+            lo = done
+            for i, ln in enumerate(orc.mesh_chunk_segments(cur, n, 4, True)):
+                order = mesh_chunk_order(n, k, i)
+                acc = ins[order[0]][k * c + lo:k * c + lo + ln].copy()
+                for t in order[1:]:
+                    acc = ins[t][k * c + lo:k * c + lo + ln] + acc
+                assert np.array_equal(outs[k][lo:lo + ln].view(np.uint32), acc.view(np.uint32)), (k, done, i)
+                lo += ln
+
+
+@pytest.mark.parametrize("n,count", [(4, 40003), (8, 100000), (8, 5), (3, 7), (2, 1001), (6, 6 * 7 * 100 + 11)])
+def test_all_reduce_mesh_chunk_rotation(orc, n, count):
+    rng = np.random.default_rng(320 + n + count)
+    ins = wide_f32(rng, n, count)
+    outs = outs_like(ins)
+    assert orc.all_reduce(ins, outs, count, F32, SUM, algo="mesh_chunk") == 0
+    chunk = -(-count // n)
+    want = np.zeros(count, dtype=np.float32)
+    for k in range(n):
+        base, ln_k = min(count, k * chunk), max(0, min(chunk, count - k * chunk))
+        lo = base
+        for i, ln in enumerate(orc.mesh_chunk_segments(ln_k, n, 4, False)):
+            order = mesh_chunk_order(n, k, i)
+            acc = ins[order[0]][lo:lo + ln].copy()
+            for t in order[1:]:
+                acc = ins[t][lo:lo + ln] + acc
+            want[lo:lo + ln] = acc
+            lo += ln
+    for o in outs:
+        assert np.array_equal(o.view(np.uint32), want.view(np.uint32))
+
+
+def test_reduce_scatter_v_mesh_chunk_rotation(orc):
+    rng = np.random.default_rng(330)
+    n = 5
+    counts = [30000, 0, 7, 4100, 12345]
+    displs = [100, 40000, 31000, 50000, 60000]
+    total = 80000
+    ins = wide_f32(rng, n, total)
+    outs = [np.zeros(max(c, 1), dtype=np.float32) for c in counts]
+    assert orc.reduce_scatter_v(ins, outs, counts, displs, F32, SUM, algo="mesh_chunk") == 0
+    for k in range(n):
+        lo = 0
+        for i, ln in enumerate(orc.mesh_chunk_segments(counts[k], n, 4, True)):
+            order = mesh_chunk_order(n, k, i)
+            a, b = displs[k] + lo, displs[k] + lo + ln
+            acc = ins[order[0]][a:b].copy()
+            for t in order[1:]:
+                acc = ins[t][a:b] + acc
+            assert np.array_equal(outs[k][lo:lo + ln].view(np.uint32), acc.view(np.uint32)), (k, i)
+            lo += ln
+
+
 def test_order_preserved_six_block_example(orc):
     """The worked example in the reference's own comment: E->A, F->B, C->(AE), D->(BF), (BFD)->(AEC)."""
     rng = np.random.default_rng(30)
@@ -331,8 +450,8 @@ def test_rhd_all_reduce_loop_bound_changes_only_roles(orc):
 # ---------------------------------------------------------------------------------------------
 # Every algorithm uses every rank exactly once; integer results are order independent
 # ---------------------------------------------------------------------------------------------
-AR_ALGOS = ["mesh", "two_shot", "rhd", "nhr", "order_preserved"]
-RS_ALGOS = ["mesh", "nhr", "rhd", "order_preserved", "aiv_mesh"]
+AR_ALGOS = ["mesh", "two_shot", "rhd", "nhr", "order_preserved", "mesh_chunk"]
+RS_ALGOS = ["mesh", "nhr", "rhd", "order_preserved", "aiv_mesh", "mesh_chunk"]
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 5, 6, 7, 8, 16, 33, 64])
