@@ -532,7 +532,11 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
 }
 
 // HCCL_DETERMINISTIC=strict moves float SUM / PROD over more than two ranks to the order-preserved fold
-// (reference src/common/order_preserved_common.h:104-114); everything else keeps the configured algorithm.
+// (reference src/common/order_preserved_common.h:104-114).  The reference offers its write-reduce templates
+// (NHR, RHD, mesh chunk) and the vector-core mesh neither PROD nor 64-bit types (REGISTER_ALG_ATTRS in
+// ins_v2_all_reduce_sole_executor.cc:401-431, ins_v2_reduce_scatter_sole_executor.cc:377-476, filtered by
+// op_common/selector/cost_table.cc:104-131) and its selector then lands on the host-reduce mesh templates, so
+// those combinations fold in the MESH order here too.  Everything else keeps the configured algorithm.
 HcclAmdAlgo EffectiveAlgo(const World* w, HcclAmdOpKind kind, HcclDataType dtype, HcclReduceOp op)
 {
     const bool isFloat = dtype == HCCL_DATA_TYPE_FP16 || dtype == HCCL_DATA_TYPE_FP32 ||
@@ -540,7 +544,15 @@ HcclAmdAlgo EffectiveAlgo(const World* w, HcclAmdOpKind kind, HcclDataType dtype
     if (w->deterministic == 2 && isFloat && (op == HCCL_REDUCE_SUM || op == HCCL_REDUCE_PROD) && w->n > 2) {
         return HCCL_AMD_ALGO_ORDER_PRESERVED;
     }
-    return w->algo[kind];
+    const HcclAmdAlgo algo = w->algo[kind];
+    const bool hostOnly = op == HCCL_REDUCE_PROD || dtype == HCCL_DATA_TYPE_INT64 || dtype == HCCL_DATA_TYPE_UINT64 ||
+                          dtype == HCCL_DATA_TYPE_FP64;
+    if (hostOnly && (algo == HCCL_AMD_ALGO_NHR || algo == HCCL_AMD_ALGO_RHD || algo == HCCL_AMD_ALGO_MESH_CHUNK ||
+                     algo == HCCL_AMD_ALGO_AIV_MESH ||
+                     (algo == HCCL_AMD_ALGO_RING && kind == HCCL_AMD_OP_REDUCE_SCATTER))) {
+        return HCCL_AMD_ALGO_MESH;
+    }
+    return algo;
 }
 
 // Mesh-chunk order: one launch per run of equally long segments.  `nGroup` slices of `len` elements start
@@ -944,7 +956,7 @@ HcclResult RunReduceScatterV(World* w, PendingOp& p, hipStream_t s)
     if (longest == 0) {
         return HCCL_SUCCESS;
     }
-    const bool meshChunk = w->algo[HCCL_AMD_OP_REDUCE_SCATTER] == HCCL_AMD_ALGO_MESH_CHUNK;
+    const bool meshChunk = EffectiveAlgo(w, HCCL_AMD_OP_REDUCE_SCATTER, p.dtype, p.op) == HCCL_AMD_ALGO_MESH_CHUNK;
     DevicePlan plan;
     HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, meshChunk ? HCCL_AMD_ALGO_MESH_CHUNK : HCCL_AMD_ALGO_MESH,
                                   &plan);

@@ -198,7 +198,10 @@ typedef enum {
 } HcclAmdAlgo;
 
 /* Sets the algorithm every later call of `op` on comm's world uses.  Also settable before
- * world creation through HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr". */
+ * world creation through HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr".  Calls with PROD or a 64-bit type
+ * fold in the MESH order under NHR, RHD, MESH_CHUNK, AIV_MESH and (ReduceScatter) RING: the reference does not
+ * offer those templates for them and falls back to its host-reduce mesh templates
+ * (op_common/selector/cost_table.cc:104-131). */
 HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo);
 HcclResult HcclAmdGetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo* algo);
 

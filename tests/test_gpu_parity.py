@@ -94,13 +94,21 @@ def pad_of(pad, r, which):
     return pad(r, which) if callable(pad) else pad
 
 
+def order_of(algo, dtype, op, reduce_scatter):
+    """PROD and the 64-bit types are not offered by the reference's write-reduce templates: mesh order."""
+    host_only = op == PROD or dtype in (DT.INT64, DT.UINT64, DT.FP64)
+    if host_only and (algo in ("nhr", "rhd", "mesh_chunk", "aiv_mesh") or (algo == "ring" and reduce_scatter)):
+        return "mesh"
+    return algo
+
+
 def run_all_reduce(world, dtype, op, count, algo, seed, pad=0, in_place=False, max_count_per_loop=0):
     rng = np.random.default_rng(seed)
     n = world.n
     ins = [gen(dtype, op, rng, count) for _ in range(n)]
     want = [np.zeros(count, dtype=NP[dtype]) for _ in range(n)]
-    assert oracle.all_reduce(ins, want, count, int(dtype), op, acc=oracle.ACC_FP32, algo=algo,
-                             max_count_per_loop=max_count_per_loop) == 0
+    assert oracle.all_reduce(ins, want, count, int(dtype), op, acc=oracle.ACC_FP32,
+                             algo=order_of(algo, dtype, op, False), max_count_per_loop=max_count_per_loop) == 0
     sends = [to_dev(x, pad_of(pad, r, "send")) for r, x in enumerate(ins)]
     recvs = sends if in_place else [dev_zeros(x.nbytes, pad_of(pad, r, "recv")) for r, x in enumerate(ins)]
     world.all_reduce(sends, recvs, count, dtype, op, algo)
@@ -115,7 +123,8 @@ def run_reduce_scatter(world, dtype, op, c, algo, seed, pad=0, max_count_per_loo
     ins = [gen(dtype, op, rng, n * c) for _ in range(n)]
     want = [np.zeros(c, dtype=NP[dtype]) for _ in range(n)]
     kw = {"max_count_per_loop": max_count_per_loop} if max_count_per_loop else {}
-    assert oracle.reduce_scatter(ins, want, c, int(dtype), op, acc=oracle.ACC_FP32, algo=algo, **kw) == 0
+    assert oracle.reduce_scatter(ins, want, c, int(dtype), op, acc=oracle.ACC_FP32,
+                                 algo=order_of(algo, dtype, op, True), **kw) == 0
     sends = [to_dev(x, pad_of(pad, r, "send")) for r, x in enumerate(ins)]
     recvs = [dev_zeros(c * ins[0].itemsize, pad_of(pad, r, "recv")) for r in range(n)]
     world.reduce_scatter(sends, recvs, c, dtype, op, algo)
@@ -435,3 +444,38 @@ def test_mesh_chunk_order_with_aligned_segments_and_staging_loops(n):
     finally:
         w.set_ccl_buffer_size(0)
         w.close()
+
+
+def test_prod_and_64_bit_types_fold_in_mesh_order_under_write_reduce_algorithms(world8):
+    """The reference offers NHR / RHD / mesh chunk / vector-core mesh neither PROD nor 64-bit types and falls back
+    to its host-reduce mesh templates: those calls must equal the oracle's MESH order bit for bit."""
+    def all_reduce_as_mesh(dtype, op, count, algo, seed):
+        rng = np.random.default_rng(seed)
+        ins = [gen(dtype, op, rng, count) for _ in range(8)]
+        want = [np.zeros(count, dtype=NP[dtype]) for _ in range(8)]
+        assert oracle.all_reduce(ins, want, count, int(dtype), op, acc=oracle.ACC_FP32, algo="mesh") == 0
+        sends = [to_dev(x) for x in ins]
+        recvs = [dev_zeros(x.nbytes) for x in ins]
+        world8.all_reduce(sends, recvs, count, dtype, op, algo)
+        for r in range(8):
+            check(dtype, op, to_host(recvs[r], NP[dtype]), want[r], "all_reduce %s as mesh, rank %d" % (algo, r))
+
+    def reduce_scatter_as_mesh(dtype, op, c, algo, seed):
+        rng = np.random.default_rng(seed)
+        ins = [gen(dtype, op, rng, 8 * c) for _ in range(8)]
+        want = [np.zeros(c, dtype=NP[dtype]) for _ in range(8)]
+        assert oracle.reduce_scatter(ins, want, c, int(dtype), op, acc=oracle.ACC_FP32, algo="mesh") == 0
+        sends = [to_dev(x) for x in ins]
+        recvs = [dev_zeros(c * ins[0].itemsize) for _ in range(8)]
+        world8.reduce_scatter(sends, recvs, c, dtype, op, algo)
+        for r in range(8):
+            check(dtype, op, to_host(recvs[r], NP[dtype]), want[r], "reduce_scatter %s as mesh, rank %d" % (algo, r))
+
+    for algo in ("nhr", "rhd", "mesh_chunk"):
+        all_reduce_as_mesh(DT.FP64, SUM, 30_001, algo, 1)
+        all_reduce_as_mesh(DT.FP32, PROD, 30_001, algo, 2)
+        all_reduce_as_mesh(DT.FP64, MAX, 5_001, algo, 3)
+    for algo in ("nhr", "ring", "rhd", "mesh_chunk", "aiv_mesh"):
+        reduce_scatter_as_mesh(DT.FP64, SUM, 9_001, algo, 4)
+        reduce_scatter_as_mesh(DT.FP32, PROD, 9_001, algo, 5)
+        reduce_scatter_as_mesh(DT.FP16, PROD, 9_001, algo, 6)
