@@ -65,11 +65,13 @@ class Algo(enum.IntEnum):
     AIV_MESH = 5
     MESH_SYMMETRIC = 6
     MESH_CHUNK = 7
+    MESH_TWO_SHOT = 8
 
 
 class OpKind(enum.IntEnum):
     ALL_REDUCE = 0
     REDUCE_SCATTER = 1
+    REDUCE = 2
 
 
 DTYPE_SIZE = {0: 1, 1: 2, 2: 4, 3: 2, 4: 4, 5: 8, 6: 8, 7: 1, 8: 2, 9: 4, 10: 8, 11: 2, 12: 16, 14: 1, 15: 1,

@@ -277,7 +277,7 @@ bool ParseAlgoName(const std::string& s, HcclAmdAlgo* algo)
         {"mesh", HCCL_AMD_ALGO_MESH}, {"ring", HCCL_AMD_ALGO_RING}, {"rhd", HCCL_AMD_ALGO_RHD},
         {"nhr", HCCL_AMD_ALGO_NHR}, {"order_preserved", HCCL_AMD_ALGO_ORDER_PRESERVED},
         {"aiv_mesh", HCCL_AMD_ALGO_AIV_MESH}, {"mesh_symmetric", HCCL_AMD_ALGO_MESH_SYMMETRIC},
-        {"mesh_chunk", HCCL_AMD_ALGO_MESH_CHUNK}};
+        {"mesh_chunk", HCCL_AMD_ALGO_MESH_CHUNK}, {"mesh_two_shot", HCCL_AMD_ALGO_MESH_TWO_SHOT}};
     for (const auto& e : table) {
         if (s == e.name) {
             *algo = e.algo;
@@ -287,7 +287,22 @@ bool ParseAlgoName(const std::string& s, HcclAmdAlgo* algo)
     return false;
 }
 
-// HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr"
+// Which orders exist for which operator.
+bool AlgoFitsOp(HcclAmdOpKind kind, HcclAmdAlgo algo)
+{
+    switch (kind) {
+        case HCCL_AMD_OP_ALL_REDUCE:
+            return algo != HCCL_AMD_ALGO_AIV_MESH && algo != HCCL_AMD_ALGO_MESH_TWO_SHOT;
+        case HCCL_AMD_OP_REDUCE_SCATTER:
+            return algo != HCCL_AMD_ALGO_MESH_TWO_SHOT;
+        case HCCL_AMD_OP_REDUCE:
+            return algo == HCCL_AMD_ALGO_MESH || algo == HCCL_AMD_ALGO_RING || algo == HCCL_AMD_ALGO_MESH_TWO_SHOT;
+        default:
+            return false;
+    }
+}
+
+// HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr;reduce=mesh_two_shot"
 void ApplyAlgoEnv(World* w)
 {
     const char* env = getenv("HCCL_AMD_ALGO");
@@ -305,8 +320,14 @@ void ApplyAlgoEnv(World* w)
             std::string key = item.substr(0, eq), val = item.substr(eq + 1);
             HcclAmdAlgo a;
             if (ParseAlgoName(val, &a)) {
-                if (key == "allreduce" && a != HCCL_AMD_ALGO_AIV_MESH) w->algo[HCCL_AMD_OP_ALL_REDUCE] = a;
-                if (key == "reducescatter") w->algo[HCCL_AMD_OP_REDUCE_SCATTER] = a;
+                HcclAmdOpKind kind = key == "allreduce" ? HCCL_AMD_OP_ALL_REDUCE :
+                                     key == "reducescatter" ? HCCL_AMD_OP_REDUCE_SCATTER :
+                                     key == "reduce" ? HCCL_AMD_OP_REDUCE : HCCL_AMD_OP_COUNT;
+                if (kind != HCCL_AMD_OP_COUNT && AlgoFitsOp(kind, a)) {
+                    w->algo[kind] = a;
+                } else {
+                    Log(1, "HCCL_AMD_ALGO: '%s' does not apply to '%s'", val.c_str(), key.c_str());
+                }
             } else {
                 Log(1, "HCCL_AMD_ALGO: unknown algorithm '%s'", val.c_str());
             }
@@ -1009,16 +1030,21 @@ HcclResult RunReduceScatterV(World* w, PendingOp& p, hipStream_t s)
     return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
 }
 
-// Reduce, mesh order: out_root = in_0, then in_1 .. in_{N-1} folded in ascending (reference
-// reduce_mesh_1D.cc:268-300): the AllReduce rank-order program with the root's recvBuf as only destination.
+// Reduce.  MESH: out_root = in_0, then in_1 .. in_{N-1} folded ascending (reference reduce_mesh_1D.cc:268-300):
+// the AllReduce rank-order program with the root's recvBuf as only destination.  MESH_TWO_SHOT: every loop of the
+// executor deals its elements into N slices, the first len mod N one element longer, and slice k folds rank k's
+// input first (reference reduce_mesh_1D_two_shot.cc:138-162, 228-265; N staging slots, :79-84,
+// reduce_sole_executor.cc:178-232).
 HcclResult RunReduce(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
     if (p.ranks[p.root].recv == nullptr) {
         return HCCL_E_PTR;
     }
+    const bool twoShot = w->algo[HCCL_AMD_OP_REDUCE] == HCCL_AMD_ALGO_MESH_TWO_SHOT;
     DevicePlan plan;
-    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_ALL_REDUCE, HCCL_AMD_ALGO_MESH, &plan);
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE, twoShot ? HCCL_AMD_ALGO_MESH_TWO_SHOT : HCCL_AMD_ALGO_MESH,
+                                  &plan);
     if (rc != HCCL_SUCCESS) {
         return rc;
     }
@@ -1031,9 +1057,49 @@ HcclResult RunReduce(World* w, PendingOp& p, hipStream_t s)
     a.nDst = 1;
     a.dstOwn = 0;
     a.nGroup = 1;
-    a.nSub = 1;
-    a.total = a.groupLen = a.subLen = p.count;
-    return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+    if (!twoShot) {
+        a.nSub = 1;
+        a.total = a.groupLen = a.subLen = p.count;
+        return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+    }
+    const uint32_t esz = DataTypeSize(p.dtype);
+    uint64_t maxPerLoop = p.count;
+    if (w->cclBytes != 0) {
+        maxPerLoop = SoleMaxCountPerLoop(w->cclBytes, n, esz);
+        if (maxPerLoop == 0) {
+            return HCCL_E_INTERNAL;
+        }
+    }
+    a.progSubStride = 1;
+    for (uint64_t done = 0; done < p.count;) {
+        const uint64_t len = std::min(p.count - done, maxPerLoop);
+        const uint64_t base = len / n;
+        const uint32_t nBig = static_cast<uint32_t>(len % n);
+        // two runs of equally long slices: nBig of base + 1 elements, then n - nBig of base
+        const uint64_t runFirst[2] = {0, static_cast<uint64_t>(nBig) * (base + 1)};
+        const uint32_t runSlices[2] = {nBig, n - nBig};
+        const uint64_t runLen[2] = {base + 1, base};
+        for (int run = 0; run < 2; ++run) {
+            if (runSlices[run] == 0 || runLen[run] == 0) {
+                continue;
+            }
+            const uint64_t at = (done + runFirst[run]) * esz;
+            for (uint32_t r = 0; r < n; ++r) {
+                a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + at;
+            }
+            a.dst[0] = static_cast<uint8_t*>(p.ranks[p.root].recv) + at;
+            a.prog = plan.dev + static_cast<uint64_t>(run == 0 ? 0 : nBig) * kDevProgBytes;
+            a.nSub = runSlices[run];
+            a.subLen = runLen[run];
+            a.total = a.groupLen = runLen[run] * runSlices[run];
+            rc = LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+        }
+        done += len;
+    }
+    return HCCL_SUCCESS;
 }
 
 // Broadcast: buf_r = buf_root, one read of the root's buffer and n - 1 writes (reference hccl.h:52-53).
@@ -1874,7 +1940,7 @@ HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo)
         algo >= HCCL_AMD_ALGO_COUNT) {
         return HCCL_E_PARA;
     }
-    if (op == HCCL_AMD_OP_ALL_REDUCE && algo == HCCL_AMD_ALGO_AIV_MESH) {
+    if (!AlgoFitsOp(op, algo)) {
         return HCCL_E_NOT_SUPPORT;
     }
     std::lock_guard<std::mutex> wl(c->world->mu);

@@ -362,6 +362,18 @@ HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPla
     if (n == 0 || n > static_cast<uint32_t>(kMaxRanks)) {
         return HCCL_E_PARA;
     }
+    if (op == HCCL_AMD_OP_REDUCE) {
+        // One-shot: rank 0's slot is the base, the others fold ascending (reference reduce_mesh_1D.cc:268-300).
+        // Two-shot: slice k is folded at rank k, own input first (reference reduce_mesh_1D_two_shot.cc:228-265).
+        if (algo == HCCL_AMD_ALGO_MESH || algo == HCCL_AMD_ALGO_RING) {
+            return MeshAllReduce(n, plan);
+        }
+        if (algo == HCCL_AMD_ALGO_MESH_TWO_SHOT) {
+            plan->segmentsAreSubs = true;
+            return MeshReduceScatter(n, plan);
+        }
+        return HCCL_E_NOT_SUPPORT;
+    }
     bool ar = op == HCCL_AMD_OP_ALL_REDUCE;
     if (!ar && op != HCCL_AMD_OP_REDUCE_SCATTER) {
         return HCCL_E_PARA;
@@ -391,6 +403,8 @@ HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPla
         case HCCL_AMD_ALGO_MESH_CHUNK:
             plan->segmentsAreSubs = true;
             return MeshChunk(n, plan);
+        case HCCL_AMD_ALGO_MESH_TWO_SHOT:
+            return HCCL_E_NOT_SUPPORT;   // Reduce only; AllReduce's two-shot folds in the MESH order
         default:
             return HCCL_E_PARA;
     }

@@ -153,7 +153,8 @@ HcclResult HcclGroupEnd(void);
  * ---------------------------------------------------------------------------------------- */
 typedef enum {
     HCCL_AMD_OP_ALL_REDUCE = 0,
-    HCCL_AMD_OP_REDUCE_SCATTER = 1,
+    HCCL_AMD_OP_REDUCE_SCATTER = 1,   /* also ReduceScatterV */
+    HCCL_AMD_OP_REDUCE = 2,           /* MESH (alias RING) or MESH_TWO_SHOT */
     HCCL_AMD_OP_COUNT
 } HcclAmdOpKind;
 
@@ -194,11 +195,17 @@ typedef enum {
      * that is zero; AllReduce segments are always dealt element-wise.  Set for ReduceScatter it also governs
      * ReduceScatterV, which otherwise always uses MESH. */
     HCCL_AMD_ALGO_MESH_CHUNK = 7,
+    /* Reduce only, the template the reference's selector picks from 8 MiB on: the count is dealt into N slices,
+     * the first count mod N of them one element longer; slice k starts from rank k's input and adds the other
+     * ranks ascending; the root gathers the slices (reference reduce_mesh_1D_two_shot.cc:138-162, 228-265,
+     * reduce_auto_selector.cc:346-351).  Reduce under MESH folds rank 0's input first and the others ascending
+     * (reduce_mesh_1D.cc:268-300). */
+    HCCL_AMD_ALGO_MESH_TWO_SHOT = 8,
     HCCL_AMD_ALGO_COUNT
 } HcclAmdAlgo;
 
 /* Sets the algorithm every later call of `op` on comm's world uses.  Also settable before
- * world creation through HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr".  Calls with PROD or a 64-bit type
+ * world creation through HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr;reduce=mesh_two_shot".  Calls with PROD or a 64-bit type
  * fold in the MESH order under NHR, RHD, MESH_CHUNK, AIV_MESH and (ReduceScatter) RING: the reference does not
  * offer those templates for them and falls back to its host-reduce mesh templates
  * (op_common/selector/cost_table.cc:104-131). */

@@ -336,8 +336,12 @@ def reduce_scatter_v(ins, outs, counts, displs, dtype, op, acc=ACC_FP32, algo="m
     return getattr(lib(), fn)(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs), cp, dp, dtype, op, acc)
 
 
-def reduce(ins, outs, count, dtype, op, root, acc=ACC_FP32):
+def reduce(ins, outs, count, dtype, op, root, acc=ACC_FP32, algo="mesh", max_count_per_loop=0):
     """Only outs[root] is written."""
+    if algo == "mesh_two_shot":
+        return lib().orc_reduce_two_shot(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs),
+                                         ctypes.c_uint64(count), dtype, op, acc, ctypes.c_uint32(root),
+                                         ctypes.c_uint64(max_count_per_loop))
     return lib().orc_reduce_mesh(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs),
                                  ctypes.c_uint64(count), dtype, op, acc, ctypes.c_uint32(root))
 

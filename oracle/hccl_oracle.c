@@ -1824,6 +1824,53 @@ int orc_reduce_mesh(uint32_t n, const void* const* in, void* const* out, uint64_
     return ORC_OK;
 }
 
+int orc_reduce_two_shot(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                        int accMode, uint32_t root, uint64_t maxCountPerLoop)
+{
+    if (root >= n) {
+        return ORC_E_PARA;
+    }
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK || count == 0) {
+        return rc;
+    }
+    if (maxCountPerLoop == 0) {
+        maxCountPerLoop = count;
+    }
+    void* acc = malloc(count * r.asz);
+    void* tmp = malloc(count * r.asz);
+    if (!acc || !tmp) {
+        free(acc);
+        free(tmp);
+        return ORC_E_INTERNAL;
+    }
+    /* reduce_sole_executor.cc:203-232: full loops, the last one takes what is left */
+    for (uint64_t done = 0; done < count;) {
+        uint64_t cur = count - done < maxCountPerLoop ? count - done : maxCountPerLoop;
+        uint64_t base = cur / n, rem = cur % n;                       /* CalcSlice :138-162 */
+        uint64_t off = done;
+        for (uint32_t k = 0; k < n; ++k) {
+            uint64_t len = base + (k < rem ? 1 : 0);
+            if (len != 0) {
+                /* slot k holds rank k's own slice (:191-198); the others fold into it ascending (:254-263) */
+                red_widen(&r, cbytes(in[k]) + off * r.esz, acc, len);
+                for (uint32_t t = 0; t < n; ++t) {
+                    if (t != k) {
+                        red_pair_from_storage(&r, acc, cbytes(in[t]) + off * r.esz, len, tmp);
+                    }
+                }
+                red_narrow(&r, acc, bytes(out[root]) + off * r.esz, len);    /* gathered by the root */
+            }
+            off += len;
+        }
+        done += cur;
+    }
+    free(acc);
+    free(tmp);
+    return ORC_OK;
+}
+
 int orc_broadcast(uint32_t n, void* const* buf, uint64_t count, int dtype, uint32_t root)
 {
     if (!copy_dtype_ok(dtype)) {

@@ -190,6 +190,10 @@ int orc_reduce_scatter_v_mesh(uint32_t n, const void* const* in, void* const* ou
  * out_root = slot_idx (+) out_root for idx = 1..N-1.  Only out[root] is written. */
 int orc_reduce_mesh(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
                     int accMode, uint32_t root);
+/* Reduce two-shot (reduce_mesh_1D_two_shot.cc:138-162, 228-265): every executor loop deals its elements into n
+ * slices, the first len mod n one longer; slice k = x_k first, then the other ranks ascending; out[root] only. */
+int orc_reduce_two_shot(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                        int accMode, uint32_t root, uint64_t maxCountPerLoop);
 /* Broadcast (hccl.h:52-53): buf_r = buf_root for every r. */
 int orc_broadcast(uint32_t n, void* const* buf, uint64_t count, int dtype, uint32_t root);
 /* Scatter (hccl.h:107-109): out_r = in_root[r * recvCount .. +recvCount). */

@@ -10,7 +10,7 @@ from hccl_amd import Algo, OpKind
 
 ALGO_BY_NAME = {"mesh": Algo.MESH, "ring": Algo.RING, "rhd": Algo.RHD, "nhr": Algo.NHR,
                 "order_preserved": Algo.ORDER_PRESERVED, "aiv_mesh": Algo.AIV_MESH, "mesh_symmetric": Algo.MESH_SYMMETRIC,
-                "mesh_chunk": Algo.MESH_CHUNK}
+                "mesh_chunk": Algo.MESH_CHUNK, "mesh_two_shot": Algo.MESH_TWO_SHOT}
 
 
 def require_library_on_gpu():
@@ -131,7 +131,8 @@ class World:
                                           self.stream)
         self.sync()
 
-    def reduce(self, sends, recvs, count, dtype, op, root):
+    def reduce(self, sends, recvs, count, dtype, op, root, algo="mesh"):
+        self.set_algo(OpKind.REDUCE, algo)
         self.inputs_ready()
         with hccl_amd.group():
             for r in range(self.n):

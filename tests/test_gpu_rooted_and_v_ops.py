@@ -182,6 +182,33 @@ def test_reduce_scatter_v_counts_that_differ_between_ranks_are_rejected(worlds):
 
 
 # ---- Reduce ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n,root", [(2, 0), (5, 3), (8, 7), (16, 9)])
+def test_reduce_two_shot_order(worlds, n, root):
+    w = worlds(n)
+    try:
+        for dtype, op, count, ccl in ((DT.FP32, SUM, 100_003, 0), (DT.FP32, SUM, 5, 0), (DT.BFP16, SUM, 65_536, 0),
+                                      (DT.FP16, MAX, 33_333, 0), (DT.FP64, SUM, 10_001, 0), (DT.INT32, PROD, 999, 0),
+                                      (DT.FP32, SUM, 200_001, 1 << 18)):
+            rng = np.random.default_rng(n * 37 + root + count)
+            ins = [gen(dtype, op, rng, count) for _ in range(n)]
+            want = [np.zeros(count, dtype=NP[dtype]) for _ in range(n)]
+            hccl_amd.set_ccl_buffer_size(w.comms[0], ccl)
+            per_loop = oracle.sole_max_count_per_loop(ccl, n, np.dtype(NP[dtype]).itemsize) if ccl else 0
+            assert oracle.reduce(ins, want, count, int(dtype), op, root, acc=oracle.ACC_FP32, algo="mesh_two_shot",
+                                 max_count_per_loop=per_loop) == 0
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(x.nbytes) for x in ins]
+            w.reduce(sends, recvs, count, dtype, op, root, "mesh_two_shot")
+            check(dtype, op, to_host(recvs[root], NP[dtype]), want[root], "reduce two-shot %s n=%d" % (dtype.name, n))
+            for r in range(n):
+                if r != root:
+                    assert np.all(to_host(recvs[r], np.uint8) == 0xAB)
+    finally:
+        hccl_amd.set_ccl_buffer_size(w.comms[0], 0)
+        w.set_algo(hccl_amd.OpKind.REDUCE, "mesh")
+
+
+
 @pytest.mark.parametrize("n,root", [(2, 1), (5, 3), (8, 0), (16, 9)])
 @pytest.mark.parametrize("dtype,op", [(DT.FP32, SUM), (DT.BFP16, SUM), (DT.INT32, PROD), (DT.FP16, MAX),
                                       (DT.INT64, MIN), (DT.FP64, SUM)])

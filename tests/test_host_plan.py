@@ -100,9 +100,12 @@ ALGO_NAME = {Algo.MESH_CHUNK: "mesh_chunk", Algo.MESH: "mesh", Algo.RING: "ring"
 
 @pytest.mark.parametrize("n", RANKS)
 def test_every_program_uses_every_rank_once(n):
-    for kind in (OpKind.ALL_REDUCE, OpKind.REDUCE_SCATTER):
+    for kind in (OpKind.ALL_REDUCE, OpKind.REDUCE_SCATTER, OpKind.REDUCE):
         for algo in Algo:
             if kind == OpKind.ALL_REDUCE and algo == Algo.AIV_MESH:
+                continue
+            if (kind == OpKind.REDUCE) != (algo == Algo.MESH_TWO_SHOT) and not (
+                    kind == OpKind.REDUCE and algo in (Algo.MESH, Algo.RING)):
                 continue
             for prog in hccl_amd.fold_programs(kind, algo, n):
                 assert sorted(program_ranks(prog)) == list(range(n)), (kind, algo, n)
@@ -241,6 +244,35 @@ def test_algo_knob(world):
     assert hccl_amd.get_algo(world[3], OpKind.ALL_REDUCE) == Algo.RHD   # per world, not per rank
     assert code_of(hccl_amd.set_algo, world[0], OpKind.ALL_REDUCE, Algo.AIV_MESH) == 5
     hccl_amd.set_algo(world[0], OpKind.ALL_REDUCE, Algo.MESH)
+    # Reduce knows its one-shot and two-shot orders only; the two-shot order exists for Reduce only
+    assert hccl_amd.get_algo(world[0], OpKind.REDUCE) == Algo.MESH
+    hccl_amd.set_algo(world[0], OpKind.REDUCE, Algo.MESH_TWO_SHOT)
+    assert hccl_amd.get_algo(world[2], OpKind.REDUCE) == Algo.MESH_TWO_SHOT
+    hccl_amd.set_algo(world[0], OpKind.REDUCE, Algo.MESH)
+    for kind, algo in ((OpKind.REDUCE, Algo.NHR), (OpKind.REDUCE, Algo.MESH_CHUNK), (OpKind.ALL_REDUCE, Algo.MESH_TWO_SHOT),
+                       (OpKind.REDUCE_SCATTER, Algo.MESH_TWO_SHOT)):
+        assert code_of(hccl_amd.set_algo, world[0], kind, algo) == 5
+
+
+@pytest.mark.parametrize("n", [1, 2, 5, 8, 33])
+def test_reduce_programs_match_oracle(orc, n):
+    count = 4 * n + 3
+    rng = np.random.default_rng(3000 + n)
+    ins = wide(rng, n, count)
+    one = hccl_amd.fold_programs(OpKind.REDUCE, Algo.MESH, n)
+    two = hccl_amd.fold_programs(OpKind.REDUCE, Algo.MESH_TWO_SHOT, n)
+    assert len(one) == 1 and len(two) == n
+    outs = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+    assert orc.reduce(ins, outs, count, F32, SUM, n - 1) == 0
+    assert same(run_program(one[0], lambda r: ins[r], SUM), outs[n - 1])
+    assert orc.reduce(ins, outs, count, F32, SUM, 0, algo="mesh_two_shot") == 0
+    got = np.zeros(count, dtype=np.float32)
+    lo = 0
+    for k in range(n):
+        ln = count // n + (1 if k < count % n else 0)
+        got[lo:lo + ln] = run_program(two[k], lambda r: ins[r][lo:lo + ln], SUM)
+        lo += ln
+    assert same(got, outs[0])
 
 
 def test_all_reduce_argument_checks(world):

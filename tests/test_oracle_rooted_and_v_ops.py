@@ -198,6 +198,57 @@ def test_reduce_equals_all_reduce_mesh_at_the_root_for_bf16_and_int_prod(orc):
             assert np.array_equal(a[root], b[root])
 
 
+@pytest.mark.parametrize("n,root,count", [(2, 1, 257), (5, 3, 1003), (8, 0, 8 * 100), (8, 7, 5), (3, 2, 2)])
+def test_reduce_two_shot_deals_slices_and_folds_the_own_slice_first(orc, n, root, count):
+    """Slices: count // n elements, the first count % n one longer; slice k = x_k, then the others ascending."""
+    rng = np.random.default_rng(n * 80 + root + count)
+    ins = wide_f32(rng, n, count)
+    outs = [np.full(count, 123.0, dtype=np.float32) for _ in range(n)]
+    assert orc.reduce(ins, outs, count, F32, SUM, root, algo="mesh_two_shot") == 0
+    want = np.zeros(count, dtype=np.float32)
+    lo = 0
+    for k in range(n):
+        ln = count // n + (1 if k < count % n else 0)
+        acc = ins[k][lo:lo + ln].copy()
+        for t in range(n):
+            if t != k:
+                acc = ins[t][lo:lo + ln] + acc
+        want[lo:lo + ln] = acc
+        lo += ln
+    assert lo == count
+    assert np.array_equal(outs[root].view(np.uint32), want.view(np.uint32))
+    for r in range(n):
+        if r != root:
+            assert np.all(outs[r] == 123.0)
+
+
+def test_reduce_two_shot_loops_deal_afresh_and_integers_do_not_care(orc):
+    rng = np.random.default_rng(81)
+    n, count, per_loop = 4, 1000, 300
+    ins = wide_f32(rng, n, count)
+    outs = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+    assert orc.reduce(ins, outs, count, F32, SUM, 2, algo="mesh_two_shot", max_count_per_loop=per_loop) == 0
+    want = np.zeros(count, dtype=np.float32)
+    for done in range(0, count, per_loop):
+        cur = min(per_loop, count - done)
+        lo = done
+        for k in range(n):
+            ln = cur // n + (1 if k < cur % n else 0)
+            acc = ins[k][lo:lo + ln].copy()
+            for t in range(n):
+                if t != k:
+                    acc = ins[t][lo:lo + ln] + acc
+            want[lo:lo + ln] = acc
+            lo += ln
+    assert np.array_equal(outs[2].view(np.uint32), want.view(np.uint32))
+    ints = [rng.integers(-2 ** 31, 2 ** 31 - 1, count, dtype=np.int32) for _ in range(n)]
+    a = [np.zeros(count, dtype=np.int32) for _ in range(n)]
+    b = [np.zeros(count, dtype=np.int32) for _ in range(n)]
+    assert orc.reduce(ints, a, count, I32, SUM, 1) == 0
+    assert orc.reduce(ints, b, count, I32, SUM, 1, algo="mesh_two_shot", max_count_per_loop=77) == 0
+    assert np.array_equal(a[1], b[1])
+
+
 def test_reduce_rejects_a_root_outside_the_world(orc):
     ins = [np.zeros(4, dtype=np.float32) for _ in range(2)]
     assert orc.reduce(ins, [x.copy() for x in ins], 4, F32, SUM, 2) == 1   # HCCL_E_PARA
