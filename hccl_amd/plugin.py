@@ -44,6 +44,35 @@ class HcclAlgoPluginTable(ctypes.Structure):
     ]
 
 
+ALG_DIR = os.path.join(_HERE, "plugin_algs")     # what a maintainer points HCCL_PLUGIN_ALG_DIR at
+ENTRY_MAGIC = 0x48415045
+
+
+class HcclAlgoPluginAlgEntry(ctypes.Structure):
+    """reference src/algo_plugin/inc/hccl_algo_plugin_common.h:104-115."""
+    _fields_ = [("version", ctypes.c_uint32), ("magic", ctypes.c_uint32), ("structSize", ctypes.c_uint32),
+                ("algName", ctypes.c_char * 128), ("soPath", ctypes.c_char * 512), ("fnSymbol", ctypes.c_char * 128)]
+
+
+def selector_path(op_name):
+    """<ALG_DIR>/<Op>/libhccl_plugin_<op>_selector.so, the name the reference's broker derives
+    (reference experimental/eco_system/algo_plugin/hccl_algo_plugin/plugin_broker/src/plugin_broker.cc:192)."""
+    return os.path.join(ALG_DIR, op_name, "libhccl_plugin_%s_selector.so" % op_name.lower())
+
+
+def load_selector(op_name):
+    """dlopen-s a selector library the way the reference's broker does and types its two exports."""
+    path = selector_path(op_name)
+    if not os.path.exists(path):
+        raise ImportError("%s is missing: run `make -C hccl_amd/csrc` first" % path)
+    lib = ctypes.CDLL(path)
+    lib.HcclAlgoPluginQueryEntries.restype = ctypes.POINTER(HcclAlgoPluginAlgEntry)
+    lib.HcclAlgoPluginQueryEntries.argtypes = [ctypes.POINTER(ctypes.c_int)]
+    lib.Select.restype = ctypes.c_bool
+    lib.Select.argtypes = [_PARAM_P, ctypes.c_char_p, ctypes.c_size_t]
+    return lib
+
+
 _table = None
 
 

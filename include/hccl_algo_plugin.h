@@ -78,6 +78,34 @@ typedef struct HcclAlgoPlugin_t {
 #define HCCL_ALGO_PLUGIN_GET_TABLE_SYMBOL "GetHcclAlgoPlugin"
 HcclAlgoPlugin_t* GetHcclAlgoPlugin(void);
 
+/*
+ * Selector libraries.  The reference's own PluginBroker does not implement algorithms: for every operator
+ * directory <HCCL_PLUGIN_ALG_DIR>/<OpName>/ it loads libhccl_plugin_<opname>_selector.so, copies the entries
+ * HcclAlgoPluginQueryEntries() returns, asks Select() per invocation and then calls the symbol `fnSymbol` of
+ * the library `soPath`, which must have the operator's hccl.h signature (reference
+ * experimental/eco_system/algo_plugin/hccl_algo_plugin/plugin_broker/src/plugin_broker.cc:140-207, 280-330;
+ * entry layout src/algo_plugin/inc/hccl_algo_plugin_common.h:104-115; exported symbols
+ * experimental/eco_system/algo_plugin/hccl_algo_plugin/sdk/hccl_algo_plugin_sdk.h:168-181).
+ * hccl_amd/plugin_algs/<OpName>/libhccl_plugin_<opname>_selector.so are such libraries: one entry each,
+ * naming libhccl_amd.so and its hccl.h entry point.
+ */
+#define HCCL_ALGO_PLUGIN_ENTRY_MAGIC 0x48415045U   /* "HAPE" */
+#define HCCL_ALGO_PLUGIN_SO_PATH_LEN 512U
+#define HCCL_ALGO_PLUGIN_FN_SYMBOL_LEN 128U
+
+typedef struct {
+    uint32_t version;          /* HCCL_ALGO_PLUGIN_STRUCT_VERSION */
+    uint32_t magic;            /* HCCL_ALGO_PLUGIN_ENTRY_MAGIC */
+    uint32_t structSize;       /* sizeof(HcclAlgoPluginAlgEntry) */
+    char algName[HCCL_ALGO_PLUGIN_ALG_NAME_LEN];
+    char soPath[HCCL_ALGO_PLUGIN_SO_PATH_LEN];       /* library that implements the algorithm */
+    char fnSymbol[HCCL_ALGO_PLUGIN_FN_SYMBOL_LEN];   /* its entry point, with the operator's hccl.h signature */
+} HcclAlgoPluginAlgEntry;
+
+/* Exported by every selector library. */
+const HcclAlgoPluginAlgEntry* HcclAlgoPluginQueryEntries(int* count);
+bool Select(const HcclAlgoPluginParam* param, char* algName, size_t algNameLen);
+
 #ifdef __cplusplus
 }
 #endif
