@@ -68,6 +68,17 @@ class Algo(enum.IntEnum):
     MESH_TWO_SHOT = 8
 
 
+class HcclSendRecvType(enum.IntEnum):
+    SEND = 0
+    RECV = 1
+
+
+class HcclSendRecvItem(ctypes.Structure):
+    """One transfer of batch_send_recv (include/hccl_types.h)."""
+    _fields_ = [("sendRecvType", ctypes.c_int), ("buf", ctypes.c_void_p), ("count", ctypes.c_uint64),
+                ("dataType", ctypes.c_int), ("remoteRank", ctypes.c_uint32)]
+
+
 class OpKind(enum.IntEnum):
     ALL_REDUCE = 0
     REDUCE_SCATTER = 1
@@ -113,6 +124,9 @@ def lib():
     L.HcclReduce.argtypes = [vp, vp, u64, i32, i32, u32, vp, vp]
     L.HcclBroadcast.argtypes = [vp, u64, i32, u32, vp, vp]
     L.HcclScatter.argtypes = [vp, vp, u64, i32, u32, vp, vp]
+    L.HcclSend.argtypes = [vp, u64, i32, u32, vp, vp]
+    L.HcclRecv.argtypes = [vp, u64, i32, u32, vp, vp]
+    L.HcclBatchSendRecv.argtypes = [ctypes.POINTER(HcclSendRecvItem), u32, vp, vp]
     L.HcclCommInitAll.argtypes = [u32, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(vp)]
     L.HcclGetRootInfo.argtypes = [vp]
     L.HcclCommInitRootInfo.argtypes = [u32, vp, u32, ctypes.POINTER(vp)]
@@ -130,6 +144,7 @@ def lib():
     L.HcclAmdGetCclBufferSize.argtypes = [vp, ctypes.POINTER(u64)]
     for name in ("HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV",
                  "HcclAlltoAll", "HcclAlltoAllVC", "HcclReduceScatterV", "HcclReduce", "HcclBroadcast", "HcclScatter",
+                 "HcclSend", "HcclRecv", "HcclBatchSendRecv",
                  "HcclCommInitAll", "HcclGetRootInfo", "HcclCommInitRootInfo", "HcclCommDestroy", "HcclGetRankSize",
                  "HcclGetRankId", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
                  "HcclAmdGetFoldProgram", "HcclAmdSetCclBufferSize", "HcclAmdGetCclBufferSize"):
@@ -357,6 +372,46 @@ def broadcast(hccl_comm, buf, count, data_type=HcclDataType.FP32, root=0, stream
     code = lib().HcclBroadcast(_as_ptr(buf), ctypes.c_uint64(count), int(data_type), ctypes.c_uint32(root), hccl_comm,
                                _as_stream(stream))
     return check(code, "HcclBroadcast")
+
+
+def send(hccl_comm, send_buf, count, data_type=HcclDataType.FP32, dest_rank=0, stream=None):
+    code = lib().HcclSend(_as_ptr(send_buf), ctypes.c_uint64(count), int(data_type), ctypes.c_uint32(dest_rank),
+                          hccl_comm, _as_stream(stream))
+    return check(code, "HcclSend")
+
+
+def recv(hccl_comm, recv_buf, count, data_type=HcclDataType.FP32, src_rank=0, stream=None):
+    code = lib().HcclRecv(_as_ptr(recv_buf), ctypes.c_uint64(count), int(data_type), ctypes.c_uint32(src_rank),
+                          hccl_comm, _as_stream(stream))
+    return check(code, "HcclRecv")
+
+
+def make_send_recv_item(send_recv_type, buf, count, data_type, remote_rank):
+    """One HcclSendRecvItem for batch_send_recv (reference hccl4py/ops.py:485-498)."""
+    item = HcclSendRecvItem()
+    item.sendRecvType = int(send_recv_type)
+    ptr = _as_ptr(buf)
+    item.buf = ptr.value if ptr is not None else None
+    item.count = int(count)
+    item.dataType = int(data_type)
+    item.remoteRank = int(remote_rank)
+    return item
+
+
+def batch_send_recv(hccl_comm, items, stream=None):
+    """items: a sequence of HcclSendRecvItem or a prebuilt (HcclSendRecvItem * n) array
+    (reference hccl4py/ops.py:450-482)."""
+    if items is None:
+        raise TypeError("items must be a sequence of HcclSendRecvItem")
+    if isinstance(items, ctypes.Array) and getattr(items, "_type_", None) is HcclSendRecvItem:
+        arr = items
+    else:
+        for i, item in enumerate(items):
+            if not isinstance(item, HcclSendRecvItem):
+                raise TypeError("items[%d] must be HcclSendRecvItem, got %s" % (i, type(item).__name__))
+        arr = (HcclSendRecvItem * len(items))(*items)
+    code = lib().HcclBatchSendRecv(arr, ctypes.c_uint32(len(arr)), hccl_comm, _as_stream(stream))
+    return check(code, "HcclBatchSendRecv")
 
 
 def scatter(hccl_comm, send_buf, recv_buf, recv_count, data_type=HcclDataType.FP32, root=0, stream=None):

@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
 #include <deque>
 #include <map>
 #include <memory>
@@ -185,6 +186,20 @@ struct PendingOp {
     std::vector<RankArgs> ranks;
 };
 
+// One Send / Recv pair.  The side that arrives second launches the copy.
+struct P2pOp {
+    uint64_t count = 0;
+    HcclDataType dtype = HCCL_DATA_TYPE_RESERVED;
+    const void* src = nullptr;
+    void* dst = nullptr;
+    hipStream_t sendStream = nullptr;
+    hipStream_t recvStream = nullptr;
+    bool haveSend = false;
+    bool haveRecv = false;
+    bool done = false;
+    HcclResult result = HCCL_SUCCESS;
+};
+
 struct DevicePlan {
     uint8_t* dev = nullptr;
     uint32_t nProg = 0;
@@ -214,6 +229,8 @@ struct World {
     std::vector<std::unique_ptr<Comm>> comms;
     HcclAmdAlgo algo[HCCL_AMD_OP_COUNT] = {HCCL_AMD_ALGO_MESH, HCCL_AMD_ALGO_MESH};
     std::deque<std::shared_ptr<PendingOp>> pending;
+    // Sends and receives that wait for their counterpart, first in first out per (source, destination) pair.
+    std::map<std::pair<uint32_t, uint32_t>, std::deque<std::shared_ptr<P2pOp>>> p2p;
     uint64_t baseSeq = 0;
     uint64_t nextSeq[kMaxRanks] = {};
     std::map<uint32_t, DevicePlan> plans;
@@ -1324,6 +1341,120 @@ HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uin
     return p->result;
 }
 
+// Runs `run` on stream `s` after everything queued on `other`, and makes `other` wait for it.
+template <class F>
+HcclResult RunBetweenStreams(World* w, hipStream_t s, hipStream_t other, F run)
+{
+    DeviceScope onWorldDevice(w->device);
+    hipEvent_t ev = nullptr;
+    if (other != s) {
+        HcclResult rc = TakeEvent(w, &ev);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+        w->eventPool.push_back(ev);   // reusable as soon as the wait below has been queued
+        HIP_OK(hipEventRecord(ev, other));
+        HIP_OK(hipStreamWaitEvent(s, ev, 0));
+    }
+    HcclResult rc = run();
+    if (rc == HCCL_SUCCESS && other != s) {
+        if (w->doneEvent == nullptr) {
+            HIP_OK(hipEventCreateWithFlags(&w->doneEvent, hipEventDisableTiming));
+        }
+        HIP_OK(hipEventRecord(w->doneEvent, s));
+        HIP_OK(hipStreamWaitEvent(other, w->doneEvent, 0));
+    }
+    return rc;
+}
+
+// Deposits one side of a Send / Recv pair (src -> dst); completes the pair when the other side is waiting.
+// Caller holds w->mu.  Returns the op so that the caller can wait for it.
+std::shared_ptr<P2pOp> DepositP2p(World* w, bool isSend, uint32_t src, uint32_t dst, void* buf, uint64_t count,
+                                  HcclDataType dtype, hipStream_t stream)
+{
+    std::deque<std::shared_ptr<P2pOp>>& q = w->p2p[{src, dst}];
+    std::shared_ptr<P2pOp> op;
+    for (const std::shared_ptr<P2pOp>& cand : q) {
+        if (isSend ? !cand->haveSend : !cand->haveRecv) {
+            op = cand;
+            break;
+        }
+    }
+    if (!op) {
+        op = std::make_shared<P2pOp>();
+        op->count = count;
+        op->dtype = dtype;
+        q.push_back(op);
+    } else if (op->result == HCCL_SUCCESS && (op->count != count || op->dtype != dtype)) {
+        Log(1, "%s %u -> %u: count %llu / type %d do not match the other side's %llu / %d", isSend ? "Send" : "Recv", src,
+            dst, (unsigned long long)count, static_cast<int>(dtype), (unsigned long long)op->count,
+            static_cast<int>(op->dtype));
+        op->result = HCCL_E_PARA;
+    }
+    if (isSend) {
+        op->haveSend = true;
+        op->src = buf;
+        op->sendStream = stream;
+    } else {
+        op->haveRecv = true;
+        op->dst = buf;
+        op->recvStream = stream;
+    }
+    if (op->haveSend && op->haveRecv) {
+        if (op->result == HCCL_SUCCESS && op->src != op->dst) {
+            BcastCopyArgs b{};
+            b.nSeg = 1;
+            b.nDst = 1;
+            b.src[0] = op->src;
+            b.dst[0] = op->dst;
+            b.len[0] = op->count * DataTypeSize(op->dtype);
+            op->result = RunBetweenStreams(w, stream, isSend ? op->recvStream : op->sendStream,
+                                           [&] { return RunBcast(w, b, stream); });
+        }
+        op->done = true;
+        for (auto it = q.begin(); it != q.end(); ++it) {
+            if (*it == op) {
+                q.erase(it);
+                break;
+            }
+        }
+        w->cv.notify_all();
+    }
+    return op;
+}
+
+// Blocks until every op of `ops` is complete (outside a group); the worst result wins.
+HcclResult AwaitP2p(World* w, std::unique_lock<std::mutex>& lock, const std::vector<std::shared_ptr<P2pOp>>& ops,
+                    const char* what, uint32_t rank)
+{
+    HcclResult rc = HCCL_SUCCESS;
+    if (t_groupDepth == 0) {
+        bool ok = w->cv.wait_for(lock, std::chrono::seconds(w->execTimeout), [&] {
+            for (const auto& op : ops) {
+                if (!op->done) {
+                    return false;
+                }
+            }
+            return true;
+        });
+        if (!ok) {
+            Log(1, "%s: rank %u waited %u s for its peer", what, rank, w->execTimeout);
+            for (const auto& op : ops) {
+                if (!op->done) {
+                    op->result = HCCL_E_TIMEOUT;   // the late peer finds the verdict and copies nothing
+                }
+            }
+            return HCCL_E_TIMEOUT;
+        }
+    }
+    for (const auto& op : ops) {
+        if (op->result != HCCL_SUCCESS) {
+            rc = op->result;
+        }
+    }
+    return rc;
+}
+
 }  // namespace
 }  // namespace hccl_amd
 
@@ -1914,6 +2045,156 @@ const char* HcclGetErrorString(HcclResult code)
         case HCCL_E_RUNTIME: return "call runtime api fail";
         default: return "unknown error";
     }
+}
+
+// Reference src/ops/send/send.cc:25-49, 136-163.
+HcclResult HcclSend(void* sendBuf, uint64_t count, HcclDataType dataType, uint32_t destRank, HcclComm comm,
+                    aclrtStream stream)
+{
+    if (count == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(stream, "stream");
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendBuf, "sendBuf");
+    CHK_RET(CheckCount(count));
+    CHK_RET(CheckDataType(dataType, false));
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclSend: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    if (c->rank == destRank) {
+        Log(1, "HcclSend: destRank cannot be equal to self");
+        return HCCL_E_NOT_SUPPORT;
+    }
+    CHK_RET(CheckUserRank(c));
+    if (destRank >= c->world->n) {
+        Log(1, "HcclSend: destRank %u is out of range [0, %u)", destRank, c->world->n);
+        return HCCL_E_PARA;
+    }
+    if (c->world->envInvalid) {
+        return HCCL_E_PARA;
+    }
+    World* w = c->world;
+    std::unique_lock<std::mutex> lock(w->mu);
+    std::vector<std::shared_ptr<P2pOp>> ops{
+        DepositP2p(w, true, c->rank, destRank, sendBuf, count, dataType, static_cast<hipStream_t>(stream))};
+    return AwaitP2p(w, lock, ops, "HcclSend", c->rank);
+}
+
+// Reference src/ops/recv/recv.cc:25-49, 134-161.
+HcclResult HcclRecv(void* recvBuf, uint64_t count, HcclDataType dataType, uint32_t srcRank, HcclComm comm,
+                    aclrtStream stream)
+{
+    if (count == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(stream, "stream");
+    CHK_PTR(comm, "comm");
+    CHK_PTR(recvBuf, "recvBuf");
+    CHK_RET(CheckCount(count));
+    CHK_RET(CheckDataType(dataType, false));
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclRecv: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    if (c->rank == srcRank) {
+        Log(1, "HcclRecv: srcRank cannot be equal to self");
+        return HCCL_E_NOT_SUPPORT;
+    }
+    CHK_RET(CheckUserRank(c));
+    if (srcRank >= c->world->n) {
+        Log(1, "HcclRecv: srcRank %u is out of range [0, %u)", srcRank, c->world->n);
+        return HCCL_E_PARA;
+    }
+    if (c->world->envInvalid) {
+        return HCCL_E_PARA;
+    }
+    World* w = c->world;
+    std::unique_lock<std::mutex> lock(w->mu);
+    std::vector<std::shared_ptr<P2pOp>> ops{
+        DepositP2p(w, false, srcRank, c->rank, recvBuf, count, dataType, static_cast<hipStream_t>(stream))};
+    return AwaitP2p(w, lock, ops, "HcclRecv", c->rank);
+}
+
+// Reference src/ops/batch_send_recv/batch_send_recv.cc:22-60, 72-90 and, for which send meets which receive,
+// algorithm/executor/ins_v2_batch_send_recv_executor.cc:96-200: items without elements are skipped, several
+// transfers between the same two ranks pair up by descending count, then descending data type (stable), and a
+// rank may send to itself when the batch holds the matching receive.
+HcclResult HcclBatchSendRecv(HcclSendRecvItem* sendRecvInfo, uint32_t itemNum, HcclComm comm, aclrtStream stream)
+{
+    if (itemNum == 0) {
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(stream, "stream");
+    CHK_PTR(comm, "comm");
+    CHK_PTR(sendRecvInfo, "sendRecvInfo");
+    for (uint32_t i = 0; i < itemNum; ++i) {
+        CHK_RET(CheckCount(sendRecvInfo[i].count));
+        CHK_RET(CheckDataType(sendRecvInfo[i].dataType, false));
+    }
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclBatchSendRecv: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckUserRank(c));
+    World* w = c->world;
+    std::vector<const HcclSendRecvItem*> sends, recvs;
+    for (uint32_t i = 0; i < itemNum; ++i) {
+        const HcclSendRecvItem& it = sendRecvInfo[i];
+        if (it.remoteRank >= w->n) {
+            Log(1, "HcclBatchSendRecv: item %u names rank %u outside [0, %u)", i, it.remoteRank, w->n);
+            return HCCL_E_PARA;
+        }
+        if (it.count == 0) {
+            continue;
+        }
+        CHK_PTR(it.buf, "item buf");
+        if (it.sendRecvType == HCCL_SEND) {
+            sends.push_back(&it);
+        } else if (it.sendRecvType == HCCL_RECV) {
+            recvs.push_back(&it);
+        } else {
+            Log(1, "HcclBatchSendRecv: item %u has send / recv type %d", i, static_cast<int>(it.sendRecvType));
+            return HCCL_E_PARA;
+        }
+    }
+    // Transfers to the own rank must come in pairs (reference ins_v2_batch_send_recv_executor.cc:183-200).
+    size_t selfSends = 0, selfRecvs = 0;
+    for (const HcclSendRecvItem* it : sends) selfSends += it->remoteRank == c->rank;
+    for (const HcclSendRecvItem* it : recvs) selfRecvs += it->remoteRank == c->rank;
+    if (selfSends != selfRecvs) {
+        Log(1, "HcclBatchSendRecv: %zu sends to the own rank but %zu receives from it", selfSends, selfRecvs);
+        return HCCL_E_PARA;
+    }
+    if (w->envInvalid) {
+        return HCCL_E_PARA;
+    }
+    auto bigFirst = [](const HcclSendRecvItem* a, const HcclSendRecvItem* b) {
+        if (a->remoteRank != b->remoteRank) {
+            return a->remoteRank < b->remoteRank;   // any fixed order of the peers: pairs are matched per peer
+        }
+        if (a->count != b->count) {
+            return a->count > b->count;
+        }
+        return static_cast<int>(a->dataType) > static_cast<int>(b->dataType);
+    };
+    std::stable_sort(sends.begin(), sends.end(), bigFirst);
+    std::stable_sort(recvs.begin(), recvs.end(), bigFirst);
+    std::unique_lock<std::mutex> lock(w->mu);
+    std::vector<std::shared_ptr<P2pOp>> ops;
+    for (const HcclSendRecvItem* it : sends) {
+        ops.push_back(DepositP2p(w, true, c->rank, it->remoteRank, it->buf, it->count, it->dataType,
+                                 static_cast<hipStream_t>(stream)));
+    }
+    for (const HcclSendRecvItem* it : recvs) {
+        ops.push_back(DepositP2p(w, false, it->remoteRank, c->rank, it->buf, it->count, it->dataType,
+                                 static_cast<hipStream_t>(stream)));
+    }
+    return AwaitP2p(w, lock, ops, "HcclBatchSendRecv", c->rank);
 }
 
 HcclResult HcclGroupStart(void)

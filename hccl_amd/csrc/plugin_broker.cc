@@ -1,5 +1,5 @@
 // PluginBroker on top of the loopback data plane: the function table of include/hccl_algo_plugin.h,
-// dispatching the fixed-count operators the reference's plugin manager can describe with one scalar
+// dispatching the fixed-count operators and Send / Recv the reference's plugin manager can describe with one scalar
 // count (reference src/algo_plugin/hccl_algo_plugin_mgr.cc: ExtractCountAndDataType, OpTypeToName) to
 // the entry points of include/hccl.h.  The V operators have no plugin signature in the reference and
 // are answered with "not selected" / HCCL_E_NOT_SUPPORT, like its manager does.
@@ -25,7 +25,8 @@ const OpEntry kOps[] = {
     {"AllReduce", "HcclAmdLoopbackAllReduce"},       {"ReduceScatter", "HcclAmdLoopbackReduceScatter"},
     {"AllGather", "HcclAmdLoopbackAllGather"},       {"Reduce", "HcclAmdLoopbackReduce"},
     {"Broadcast", "HcclAmdLoopbackBroadcast"},       {"Scatter", "HcclAmdLoopbackScatter"},
-    {"AllToAll", "HcclAmdLoopbackAllToAll"},
+    {"AllToAll", "HcclAmdLoopbackAllToAll"},         {"Send", "HcclAmdLoopbackSend"},
+    {"Recv", "HcclAmdLoopbackRecv"},
 };
 
 const OpEntry* FindOp(const char* opName)
@@ -98,6 +99,13 @@ int ExecuteAlg(void* ctx, const char* algName, const char* opName, const HcclAlg
     }
     if (strcmp(opName, "Scatter") == 0) {
         return HcclScatter(p.sendBuf, p.recvBuf, p.count, p.dataType, p.root, comm, p.stream);
+    }
+    // the peer of a point-to-point transfer travels as remoteRank (reference hccl_algo_plugin_mgr.cc:251)
+    if (strcmp(opName, "Send") == 0) {
+        return HcclSend(p.sendBuf, p.count, p.dataType, p.remoteRank, comm, p.stream);
+    }
+    if (strcmp(opName, "Recv") == 0) {
+        return HcclRecv(p.recvBuf, p.count, p.dataType, p.remoteRank, comm, p.stream);
     }
     return HcclAlltoAll(p.sendBuf, p.count, p.dataType, p.recvBuf, p.count, p.dataType, comm, p.stream);
 }

@@ -89,11 +89,12 @@ def table():
 
 
 def make_param(op_name, count=0, data_type=4, reduce_op=0, root=0, send_buf=None, recv_buf=None, stream=None,
-               rank_num=0):
+               rank_num=0, remote_rank=0):
     p = HcclAlgoPluginParam()
     p.version, p.magic, p.structSize = STRUCT_VERSION, PARAM_MAGIC, ctypes.sizeof(HcclAlgoPluginParam)
     p.opName = op_name.encode()
     p.count, p.dataType, p.reduceOp, p.root, p.rankNum = count, int(data_type), int(reduce_op), root, rank_num
+    p.remoteRank = remote_rank
     p.sendBuf = send_buf
     p.recvBuf = recv_buf
     p.stream = stream

@@ -121,6 +121,27 @@ HcclResult HcclBroadcast(void* buf, uint64_t count, HcclDataType dataType, uint3
 HcclResult HcclScatter(void* sendBuf, void* recvBuf, uint64_t recvCount, HcclDataType dataType, uint32_t root,
                        HcclComm comm, aclrtStream stream);
 
+/*
+ * Point to point.  destRank's HcclRecv(…, srcRank = this rank) receives what this rank sends; sends and receives
+ * between the same two ranks pair up in call order.  A rank cannot send to itself (HCCL_E_NOT_SUPPORT).  The side
+ * that arrives second launches the copy; the first one blocks until then unless it is inside
+ * HcclGroupStart / HcclGroupEnd.  Replace reference include/hccl.h:158-159, 175-176 (src/ops/send/send.cc:25-49,
+ * 136-163; src/ops/recv/recv.cc:25-49, 134-161).
+ */
+HcclResult HcclSend(void* sendBuf, uint64_t count, HcclDataType dataType, uint32_t destRank, HcclComm comm,
+                    aclrtStream stream);
+HcclResult HcclRecv(void* recvBuf, uint64_t count, HcclDataType dataType, uint32_t srcRank, HcclComm comm,
+                    aclrtStream stream);
+
+/*
+ * A batch of sends and receives issued together.  Items without elements are skipped; several transfers between
+ * the same two ranks pair up by descending count, then descending data type, whatever their order in the array;
+ * a send to the own rank is legal when the batch also holds the receive.  Replaces reference
+ * include/hccl.h:265-266 (src/ops/batch_send_recv/batch_send_recv.cc:22-90,
+ * algorithm/executor/ins_v2_batch_send_recv_executor.cc:96-200).
+ */
+HcclResult HcclBatchSendRecv(HcclSendRecvItem* sendRecvInfo, uint32_t itemNum, HcclComm comm, aclrtStream stream);
+
 /* ------------------------------------------------------------------------------------------
  * Communicator lifecycle. In the reference these live in the separate HCOMM library and
  * are only called (examples/02_collectives/01_allreduce/main.cc:76,101,123;

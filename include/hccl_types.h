@@ -80,6 +80,25 @@ typedef enum {
     HCCL_DATA_TYPE_RESERVED = 255
 } HcclDataType;
 
+/* One transfer of HcclBatchSendRecv.  The type comes from the CANN headers, which are not part of the
+ * reference tree; the tree fixes the field names (src/ops/batch_send_recv/algorithm/executor/
+ * ins_v2_batch_send_recv_executor.cc:143-160), their order as the Python constructor fills them
+ * (experimental/eco_system/python/hccl4py/ops.py:485-498) and "0: send, 1: recv"
+ * (src/ops/op_common/algorithm/template/aiv/hccl_aiv_utils.h:111). */
+typedef enum {
+    HCCL_SEND = 0,
+    HCCL_RECV = 1,
+    HCCL_SEND_RECV_RESERVED
+} HcclSendRecvType;
+
+typedef struct HcclSendRecvItemDef {
+    HcclSendRecvType sendRecvType;
+    void* buf;
+    uint64_t count;        /* elements */
+    HcclDataType dataType;
+    uint32_t remoteRank;   /* destination of a send, source of a receive */
+} HcclSendRecvItem;
+
 /* Opaque communicator handle: one per rank of a loopback world. */
 typedef void* HcclComm;
 

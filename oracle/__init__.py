@@ -354,3 +354,25 @@ def broadcast(bufs, count, dtype, root):
 def scatter(ins, outs, recv_count, dtype, root):
     return lib().orc_scatter(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs),
                              ctypes.c_uint64(recv_count), dtype, ctypes.c_uint32(root))
+
+
+# ---- point to point --------------------------------------------------------------------------
+class SendRecvItem(ctypes.Structure):
+    _fields_ = [("sendRecvType", ctypes.c_int), ("buf", ctypes.c_void_p), ("count", ctypes.c_uint64),
+                ("dataType", ctypes.c_int), ("remoteRank", ctypes.c_uint32)]
+
+
+def batch_send_recv(items_per_rank):
+    """items_per_rank[r] = [(0 send / 1 recv, numpy array, count, dtype, remote rank), ...]; receive arrays are
+    written in place."""
+    n = len(items_per_rank)
+    arrays = []
+    for items in items_per_rank:
+        arr = (SendRecvItem * max(len(items), 1))()
+        for i, (kind, buf, count, dtype, remote) in enumerate(items):
+            arr[i].sendRecvType, arr[i].count, arr[i].dataType, arr[i].remoteRank = kind, count, dtype, remote
+            arr[i].buf = None if buf is None else buf.ctypes.data
+        arrays.append(arr)
+    ptrs = (ctypes.POINTER(SendRecvItem) * n)(*[ctypes.cast(a, ctypes.POINTER(SendRecvItem)) for a in arrays])
+    nums = (ctypes.c_uint32 * n)(*[len(items) for items in items_per_rank])
+    return lib().orc_batch_send_recv(ctypes.c_uint32(n), ptrs, nums)

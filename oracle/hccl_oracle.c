@@ -2009,3 +2009,102 @@ int orc_all_reduce_mesh_mt(uint32_t n, const void* const* in, void* const* out, 
 {
     return run_mt(0, n, in, out, count, dtype, op, accMode, nThreads);
 }
+
+/* ---------------------------------------------------------------------------------------------
+ * Point to point: BatchSendRecv (batch_send_recv_executor.cc:96-200, 202-275)
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+    const orc_send_recv_item_t* item;
+    uint32_t flag;     /* peer order of the pair-wise schedule */
+    uint32_t index;    /* position in the caller's array: keeps the sort stable */
+} bsr_entry_t;
+
+static int bsr_cmp_send(const void* pa, const void* pb)
+{
+    const bsr_entry_t* a = (const bsr_entry_t*)pa;
+    const bsr_entry_t* b = (const bsr_entry_t*)pb;
+    if (a->flag != b->flag) return a->flag > b->flag ? -1 : 1;                        /* :109-110 descending */
+    if (a->item->count != b->item->count) return a->item->count > b->item->count ? -1 : 1;
+    if (a->item->dataType != b->item->dataType) return a->item->dataType > b->item->dataType ? -1 : 1;
+    return a->index < b->index ? -1 : 1;
+}
+
+static int bsr_cmp_recv(const void* pa, const void* pb)
+{
+    const bsr_entry_t* a = (const bsr_entry_t*)pa;
+    const bsr_entry_t* b = (const bsr_entry_t*)pb;
+    if (a->flag != b->flag) return a->flag < b->flag ? -1 : 1;                        /* :121-122 ascending */
+    if (a->item->count != b->item->count) return a->item->count > b->item->count ? -1 : 1;
+    if (a->item->dataType != b->item->dataType) return a->item->dataType > b->item->dataType ? -1 : 1;
+    return a->index < b->index ? -1 : 1;
+}
+
+/* Sorted send (isSend) or receive list of one rank; items without elements are dropped (:150). */
+static uint32_t bsr_sorted(uint32_t n, uint32_t me, const orc_send_recv_item_t* items, uint32_t itemNum, int isSend,
+                           bsr_entry_t* out)
+{
+    uint32_t k = 0;
+    for (uint32_t i = 0; i < itemNum; ++i) {
+        if (items[i].count == 0 || (items[i].sendRecvType == 0) != (isSend != 0)) {
+            continue;
+        }
+        uint32_t peer = items[i].remoteRank;
+        out[k].item = &items[i];
+        out[k].index = i;
+        out[k].flag = isSend ? (peer <= me ? peer + n : peer) : (peer < me ? peer + n : peer);   /* :107-108, :119-120 */
+        ++k;
+    }
+    qsort(out, k, sizeof(bsr_entry_t), isSend ? bsr_cmp_send : bsr_cmp_recv);
+    return k;
+}
+
+int orc_batch_send_recv(uint32_t n, const orc_send_recv_item_t* const* items, const uint32_t* itemNum)
+{
+    uint32_t most = 0;
+    for (uint32_t r = 0; r < n; ++r) {
+        most = itemNum[r] > most ? itemNum[r] : most;
+        for (uint32_t i = 0; i < itemNum[r]; ++i) {
+            const orc_send_recv_item_t* it = &items[r][i];
+            if (!copy_dtype_ok(it->dataType)) return ORC_E_NOT_SUPPORT;
+            if (it->remoteRank >= n) return ORC_E_PARA;
+            if (it->count != 0 && it->buf == NULL) return ORC_E_PTR;
+            if (it->count != 0 && it->sendRecvType != 0 && it->sendRecvType != 1) return ORC_E_PARA;
+        }
+    }
+    bsr_entry_t* tx = (bsr_entry_t*)malloc(sizeof(bsr_entry_t) * (most ? most : 1));
+    bsr_entry_t* rx = (bsr_entry_t*)malloc(sizeof(bsr_entry_t) * (most ? most : 1));
+    if (!tx || !rx) {
+        free(tx);
+        free(rx);
+        return ORC_E_INTERNAL;
+    }
+    int rc = ORC_OK;
+    /* The k-th send of a to b in a's sorted list meets the k-th receive from a in b's sorted list. */
+    for (uint32_t a = 0; a < n && rc == ORC_OK; ++a) {
+        uint32_t nTx = bsr_sorted(n, a, items[a], itemNum[a], 1, tx);
+        for (uint32_t b = 0; b < n && rc == ORC_OK; ++b) {
+            uint32_t nRx = bsr_sorted(n, b, items[b], itemNum[b], 0, rx);
+            uint32_t i = 0, j = 0;
+            for (;;) {
+                while (i < nTx && tx[i].item->remoteRank != b) ++i;
+                while (j < nRx && rx[j].item->remoteRank != a) ++j;
+                if (i >= nTx || j >= nRx) {
+                    if (i < nTx || j < nRx) rc = ORC_E_PARA;           /* a transfer without its counterpart */
+                    break;
+                }
+                const orc_send_recv_item_t* s = tx[i].item;
+                const orc_send_recv_item_t* d = rx[j].item;
+                if (s->count != d->count || s->dataType != d->dataType) {
+                    rc = ORC_E_PARA;                                    /* :88-101 for the own rank */
+                    break;
+                }
+                memmove(d->buf, s->buf, s->count * orc_dtype_size(s->dataType));
+                ++i;
+                ++j;
+            }
+        }
+    }
+    free(tx);
+    free(rx);
+    return rc;
+}

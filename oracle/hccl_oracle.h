@@ -211,6 +211,21 @@ int orc_reduce_scatter_mesh_mt(uint32_t n, const void* const* in, void* const* o
 int orc_all_reduce_mesh_mt(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
                            int accMode, uint32_t nThreads);
 
+/* --- point to point ----------------------------------------------------------------------
+ * BatchSendRecv over n loopback ranks: items[r] / itemNum[r] are rank r's array.  Every rank sorts its sends and
+ * its receives pair-wise (peer order, then count descending, then data type descending, stable;
+ * ins_v2_batch_send_recv_executor.cc:105-128, 137-200) and the k-th send of a to b meets the k-th receive from a
+ * at b.  A transfer without counterpart or with unequal count / type is E_PARA.  Plain Send / Recv are batches of
+ * one item. */
+typedef struct {
+    int sendRecvType;      /* 0 send, 1 receive */
+    void* buf;
+    uint64_t count;
+    int dataType;
+    uint32_t remoteRank;
+} orc_send_recv_item_t;
+int orc_batch_send_recv(uint32_t n, const orc_send_recv_item_t* const* items, const uint32_t* itemNum);
+
 #ifdef __cplusplus
 }
 #endif

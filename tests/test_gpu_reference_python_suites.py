@@ -173,10 +173,30 @@ def test_dtype_suite(dtype_name, nranks):
                     s, r = to_dev(pack(dtype_name, [mine] * nranks)), zeros(nranks * esize)
                     h.all_to_all_v(comm, s, ones, ramp, dt, r, ones, ramp, dt, stream=stream)
                     ok = close(unpack(dtype_name, to_host(r), nranks), gathered)
-                else:
+                elif op == "all_to_all_vc":
                     s, r = to_dev(pack(dtype_name, [mine] * nranks)), zeros(nranks * esize)
                     h.all_to_all_vc(comm, s, [1] * (nranks * nranks), dt, r, dt, stream=stream)
                     ok = close(unpack(dtype_name, to_host(r), nranks), gathered)
+                elif op == "send_recv":
+                    if nranks != 2:
+                        res[op] = True           # the reference runs this case on two ranks only
+                        continue
+                    peer = 1 - rank
+                    s, r = to_dev(pack(dtype_name, [mine] * 4)), zeros(4 * esize)
+                    if rank == 0:
+                        h.send(comm, s, 4, dt, dest_rank=peer, stream=stream)
+                        h.recv(comm, r, 4, dt, src_rank=peer, stream=stream)
+                    else:
+                        h.recv(comm, r, 4, dt, src_rank=peer, stream=stream)
+                        h.send(comm, s, 4, dt, dest_rank=peer, stream=stream)
+                    ok = close(unpack(dtype_name, to_host(r), 4), float(peer + 1))
+                else:
+                    nxt, prv = (rank + 1) % nranks, (rank - 1 + nranks) % nranks
+                    s, r = to_dev(pack(dtype_name, [mine] * 4)), zeros(4 * esize)
+                    items = [h.make_send_recv_item(h.HcclSendRecvType.SEND, s, 4, dt, nxt),
+                             h.make_send_recv_item(h.HcclSendRecvType.RECV, r, 4, dt, prv)]
+                    h.batch_send_recv(comm, items, stream=stream)
+                    ok = close(unpack(dtype_name, to_host(r), 4), float(prv + 1))
                 res[op] = ok and not (reducing and refused)
             except h.HcclError as e:
                 res[op] = reducing and refused and e.code == 5      # HCCL_E_NOT_SUPPORT, like the reference

@@ -378,6 +378,50 @@ def test_rooted_and_v_entry_argument_checks(world):
     assert code_of(hccl_amd.scatter, c, a, b, 4, DT.FP32, 0, None) == 2
 
 
+def test_point_to_point_argument_checks(world):
+    c, s, a = world[0], 0x1000, 0x2000
+    # reference send.cc:33-38, 136-163 / recv.cc likewise: nothing to move is a success before any other check
+    assert code_of(hccl_amd.send, c, None, 0, DT.FP32, 1, None) == 0
+    assert code_of(hccl_amd.recv, c, None, 0, DT.FP32, 1, None) == 0
+    assert code_of(hccl_amd.send, c, a, 4, DT.FP32, 1, None) == 2
+    assert code_of(hccl_amd.send, None, a, 4, DT.FP32, 1, s) == 2
+    assert code_of(hccl_amd.send, c, None, 4, DT.FP32, 1, s) == 2
+    assert code_of(hccl_amd.recv, c, None, 4, DT.FP32, 1, s) == 2
+    assert code_of(hccl_amd.send, c, a, 0x800000000, DT.FP32, 1, s) == 1
+    assert code_of(hccl_amd.send, c, a, 4, DT.INT128, 1, s) == 5
+    assert code_of(hccl_amd.send, c, a, 4, DT.FP32, 0, s) == 5              # to itself
+    assert code_of(hccl_amd.recv, c, a, 4, DT.FP32, 0, s) == 5
+    assert code_of(hccl_amd.send, c, a, 4, DT.FP32, 4, s) == 1              # no such rank
+    assert code_of(hccl_amd.recv, c, a, 4, DT.FP32, 99, s) == 1
+    # batch_send_recv.cc:34-60 and ins_v2_batch_send_recv_executor.cc:143-200
+    item = hccl_amd.make_send_recv_item
+    T = hccl_amd.HcclSendRecvType
+    assert code_of(hccl_amd.batch_send_recv, c, [], None) == 0
+    assert code_of(hccl_amd.batch_send_recv, c, [item(T.SEND, a, 4, DT.FP32, 1)], None) == 2
+    assert code_of(hccl_amd.batch_send_recv, None, [item(T.SEND, a, 4, DT.FP32, 1)], s) == 2
+    assert code_of(hccl_amd.batch_send_recv, c, [item(T.SEND, a, 0x800000000, DT.FP32, 1)], s) == 1
+    assert code_of(hccl_amd.batch_send_recv, c, [item(T.SEND, a, 4, DT.INT128, 1)], s) == 5
+    assert code_of(hccl_amd.batch_send_recv, c, [item(T.SEND, a, 4, DT.FP32, 4)], s) == 1
+    assert code_of(hccl_amd.batch_send_recv, c, [item(T.SEND, None, 4, DT.FP32, 1)], s) == 2
+    assert code_of(hccl_amd.batch_send_recv, c, [item(2, a, 4, DT.FP32, 1)], s) == 1
+    assert code_of(hccl_amd.batch_send_recv, c, [item(T.SEND, a, 4, DT.FP32, 0)], s) == 1    # own rank, no receive
+    assert code_of(hccl_amd.batch_send_recv, c, [item(T.SEND, None, 0, DT.FP32, 1)], s) == 0  # nothing to move
+    with pytest.raises(TypeError):
+        hccl_amd.batch_send_recv(c, [object()], s)
+
+
+def test_a_send_whose_peer_never_receives_times_out(monkeypatch):
+    monkeypatch.setenv("HCCL_EXEC_TIMEOUT", "1")
+    comms = hccl_amd.comm_init_all(2)
+    try:
+        assert code_of(hccl_amd.send, comms[0], 0x2000, 8, DT.FP32, 1, 0x1000) == 9
+        # the late receive finds the verdict: nothing is copied
+        assert code_of(hccl_amd.recv, comms[1], 0x3000, 8, DT.FP32, 0, 0x1000) == 9
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)
+
+
 def test_unparsable_hccl_deterministic_fails_every_collective(monkeypatch):
     # reference alg_env_config.cc:1113-1125: anything but true / false / strict is HCCL_E_PARA at the entry point
     monkeypatch.setenv("HCCL_DETERMINISTIC", "maybe")

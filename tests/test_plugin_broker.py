@@ -11,7 +11,8 @@ import pytest
 import hccl_amd
 from hccl_amd import HcclDataType as DT, HcclReduceOp as OP, plugin
 
-FIXED_COUNT_OPS = ["AllReduce", "ReduceScatter", "AllGather", "Reduce", "Broadcast", "Scatter", "AllToAll"]
+FIXED_COUNT_OPS = ["AllReduce", "ReduceScatter", "AllGather", "Reduce", "Broadcast", "Scatter", "AllToAll", "Send",
+                   "Recv"]
 
 
 def test_param_struct_has_the_reference_layout():
@@ -47,7 +48,7 @@ def test_operators_without_a_plugin_signature_are_not_taken():
     t = plugin.table()
     ctx = t.FetchContext()
     name = ctypes.create_string_buffer(128)
-    for op in ("AllToAllV", "AllGatherV", "ReduceScatterV", "Send", "Recv", ""):
+    for op in ("AllToAllV", "AllToAllVC", "AllGatherV", "ReduceScatterV", "BatchSendRecv", ""):
         assert t.SelectAlg(ctx, ctypes.byref(plugin.make_param(op, 8)), name, 128) is False
         listed = ctypes.create_string_buffer(16)
         assert t.QueryAlgs(ctx, op.encode(), listed, 16) == 0 and listed.raw[0:1] == b"\0"
@@ -77,7 +78,8 @@ def test_malformed_requests_are_rejected():
 
 # ---- selector libraries for the reference's own broker --------------------------------------------------
 ENTRY_POINT = {"AllReduce": "HcclAllReduce", "ReduceScatter": "HcclReduceScatter", "AllGather": "HcclAllGather",
-               "Reduce": "HcclReduce", "Broadcast": "HcclBroadcast", "Scatter": "HcclScatter", "AllToAll": "HcclAlltoAll"}
+               "Reduce": "HcclReduce", "Broadcast": "HcclBroadcast", "Scatter": "HcclScatter", "AllToAll": "HcclAlltoAll",
+               "Send": "HcclSend", "Recv": "HcclRecv"}
 
 
 def test_entry_struct_has_the_reference_layout():
@@ -206,6 +208,21 @@ def test_all_reduce_and_broadcast_through_the_table_match_the_oracle():
         w.sync()
         for r in range(n):
             assert np.array_equal(to_host(recvs[r], np.float32).view(np.uint32), want[r].view(np.uint32)), r
+        # Send / Recv: the peer travels as remoteRank
+        outs = [dev_zeros(ins[0].nbytes) for _ in range(n)]
+        w.inputs_ready()
+        hccl_amd.group_start()
+        for r in range(n):
+            ps = plugin.make_param("Send", count, DT.FP32, 0, 0, sends[r].data_ptr(), None, w.stream.cuda_stream, n,
+                                   remote_rank=(r + 1) % n)
+            pr = plugin.make_param("Recv", count, DT.FP32, 0, 0, None, outs[r].data_ptr(), w.stream.cuda_stream, n,
+                                   remote_rank=(r - 1) % n)
+            assert t.ExecuteAlg(ctx, b"HcclAmdLoopbackSend", b"Send", ctypes.byref(ps), w.comms[r]) == 0
+            assert t.ExecuteAlg(ctx, b"HcclAmdLoopbackRecv", b"Recv", ctypes.byref(pr), w.comms[r]) == 0
+        hccl_amd.group_end()
+        w.sync()
+        for r in range(n):
+            assert np.array_equal(to_host(outs[r], np.float32).view(np.uint32), ins[(r - 1) % n].view(np.uint32)), r
         # Broadcast: the one buffer travels as sendBuf
         bufs = [to_dev(x) for x in ins]
         w.inputs_ready()
