@@ -124,6 +124,7 @@ def lib():
     L.HcclReduce.argtypes = [vp, vp, u64, i32, i32, u32, vp, vp]
     L.HcclBroadcast.argtypes = [vp, u64, i32, u32, vp, vp]
     L.HcclScatter.argtypes = [vp, vp, u64, i32, u32, vp, vp]
+    L.HcclBarrier.argtypes = [vp, vp]
     L.HcclSend.argtypes = [vp, u64, i32, u32, vp, vp]
     L.HcclRecv.argtypes = [vp, u64, i32, u32, vp, vp]
     L.HcclBatchSendRecv.argtypes = [ctypes.POINTER(HcclSendRecvItem), u32, vp, vp]
@@ -144,7 +145,7 @@ def lib():
     L.HcclAmdGetCclBufferSize.argtypes = [vp, ctypes.POINTER(u64)]
     for name in ("HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV",
                  "HcclAlltoAll", "HcclAlltoAllVC", "HcclReduceScatterV", "HcclReduce", "HcclBroadcast", "HcclScatter",
-                 "HcclSend", "HcclRecv", "HcclBatchSendRecv",
+                 "HcclSend", "HcclRecv", "HcclBatchSendRecv", "HcclBarrier",
                  "HcclCommInitAll", "HcclGetRootInfo", "HcclCommInitRootInfo", "HcclCommDestroy", "HcclGetRankSize",
                  "HcclGetRankId", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
                  "HcclAmdGetFoldProgram", "HcclAmdSetCclBufferSize", "HcclAmdGetCclBufferSize"):
@@ -372,6 +373,10 @@ def broadcast(hccl_comm, buf, count, data_type=HcclDataType.FP32, root=0, stream
     code = lib().HcclBroadcast(_as_ptr(buf), ctypes.c_uint64(count), int(data_type), ctypes.c_uint32(root), hccl_comm,
                                _as_stream(stream))
     return check(code, "HcclBroadcast")
+
+
+def barrier(hccl_comm, stream=None):
+    return check(lib().HcclBarrier(hccl_comm, _as_stream(stream)), "HcclBarrier")
 
 
 def send(hccl_comm, send_buf, count, data_type=HcclDataType.FP32, dest_rank=0, stream=None):

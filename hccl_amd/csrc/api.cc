@@ -146,7 +146,7 @@ HcclResult CheckReduceOp(HcclDataType t, HcclReduceOp op)
 // ---------------------------------------------------------------------------------------------
 enum class OpType {
     ALL_REDUCE, REDUCE_SCATTER, ALL_GATHER, ALL_GATHER_V, ALL_TO_ALL_V,
-    REDUCE_SCATTER_V, REDUCE, BROADCAST, SCATTER
+    REDUCE_SCATTER_V, REDUCE, BROADCAST, SCATTER, BARRIER
 };
 
 const char* OpName(OpType t)
@@ -160,6 +160,7 @@ const char* OpName(OpType t)
         case OpType::REDUCE: return "Reduce";
         case OpType::BROADCAST: return "Broadcast";
         case OpType::SCATTER: return "Scatter";
+        case OpType::BARRIER: return "Barrier";
         default: return "AlltoAllV";
     }
 }
@@ -1247,7 +1248,9 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
         HIP_OK(hipStreamWaitEvent(s, ev, 0));
     }
     HcclResult rc;
-    if (w->n == 1) {
+    if (p.type == OpType::BARRIER) {
+        rc = HCCL_SUCCESS;   // the ordering of the streams around this point is the whole operation
+    } else if (w->n == 1) {
         rc = RunSingleRank(w, p, s);
     } else {
         switch (p.type) {
@@ -2045,6 +2048,22 @@ const char* HcclGetErrorString(HcclResult code)
         case HCCL_E_RUNTIME: return "call runtime api fail";
         default: return "unknown error";
     }
+}
+
+// Every rank's stream waits until all ranks' streams have reached their HcclBarrier.  Reference
+// src/ops/barrier/barrier.cc:47-101 (null stream, then null comm, then the rank check).
+HcclResult HcclBarrier(HcclComm comm, aclrtStream stream)
+{
+    CHK_PTR(stream, "stream");
+    CHK_PTR(comm, "comm");
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "HcclBarrier: comm is not a live communicator");
+        return HCCL_E_PARA;
+    }
+    CHK_RET(CheckUserRank(c));
+    return SubmitWithReady(c, OpType::BARRIER, HCCL_DATA_TYPE_RESERVED, HCCL_REDUCE_RESERVED, 0, nullptr, nullptr, stream,
+                           {});
 }
 
 // Reference src/ops/send/send.cc:25-49, 136-163.

@@ -122,6 +122,13 @@ HcclResult HcclScatter(void* sendBuf, void* recvBuf, uint64_t recvCount, HcclDat
                        HcclComm comm, aclrtStream stream);
 
 /*
+ * Orders the ranks' streams: work queued after the call on any rank's stream starts only when the work queued
+ * before the call on every rank's stream has finished.  Replaces the HcclBarrier the reference exports from
+ * src/ops/barrier/barrier.cc:47-72 (declared by the CANN header hccl/hccl_comm.h, which is outside its tree).
+ */
+HcclResult HcclBarrier(HcclComm comm, aclrtStream stream);
+
+/*
  * Point to point.  destRank's HcclRecv(…, srcRank = this rank) receives what this rank sends; sends and receives
  * between the same two ranks pair up in call order.  A rank cannot send to itself (HCCL_E_NOT_SUPPORT).  The side
  * that arrives second launches the copy; the first one blocks until then unless it is inside

@@ -156,3 +156,35 @@ def test_unequal_counts_on_the_two_sides_are_reported_to_both():
         assert np.all(to_host(b, np.uint8) == 0xAB)                  # nothing was copied
     finally:
         w.close()
+
+
+def test_barrier_orders_the_streams_of_all_ranks():
+    """Every rank fills its buffer on its own stream, all meet at the barrier, then every rank reads its
+    neighbour's buffer on its own stream: without the barrier's ordering the read could overtake the fill."""
+    import torch
+    n, count = 4, 1 << 22
+    comms = hccl_amd.comm_init_all(n)
+    try:
+        streams = [torch.cuda.Stream() for _ in range(n)]
+        bufs = [torch.zeros(count, dtype=torch.float32, device="cuda") for _ in range(n)]
+        sums = [None] * n
+        torch.cuda.synchronize()
+        for r in range(n):
+            with torch.cuda.stream(streams[r]):
+                for _ in range(10):
+                    bufs[r].add_(0.1 * (r + 1))
+        with hccl_amd.group():
+            for r in range(n):
+                hccl_amd.barrier(comms[r], streams[r])
+        for r in range(n):
+            with torch.cuda.stream(streams[r]):
+                sums[r] = bufs[(r + 1) % n].sum(dtype=torch.float64)
+        torch.cuda.synchronize()
+        for r in range(n):
+            acc = torch.zeros(1, dtype=torch.float32)
+            for _ in range(10):
+                acc.add_(0.1 * (((r + 1) % n) + 1))
+            assert abs(float(sums[r].item()) - float(acc.item()) * count) < 1e-3 * count, r
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)

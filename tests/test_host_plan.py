@@ -378,6 +378,11 @@ def test_rooted_and_v_entry_argument_checks(world):
     assert code_of(hccl_amd.scatter, c, a, b, 4, DT.FP32, 0, None) == 2
 
 
+def test_barrier_argument_checks(world):
+    assert code_of(hccl_amd.barrier, world[0], None) == 2
+    assert code_of(hccl_amd.barrier, None, 0x1000) == 2
+
+
 def test_point_to_point_argument_checks(world):
     c, s, a = world[0], 0x1000, 0x2000
     # reference send.cc:33-38, 136-163 / recv.cc likewise: nothing to move is a success before any other check
