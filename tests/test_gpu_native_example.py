@@ -17,3 +17,13 @@ def test_native_thread_per_rank_program(ranks, count):
     done = subprocess.run([BINARY, str(ranks), str(count)], capture_output=True, text=True, timeout=110)
     assert done.returncode == 0, done.stdout + done.stderr
     assert done.stdout.startswith("PASS"), done.stdout
+
+
+def test_native_latency_program_runs_and_reports_every_size():
+    binary = os.path.join(ROOT, "examples", "bin", "allreduce_latency")
+    assert os.path.exists(binary), "run `make -C examples` (or __graft_entry__.build()) first"
+    done = subprocess.run([binary, "8"], capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0, done.stdout + done.stderr
+    rows = [line.split() for line in done.stdout.splitlines()[2:]]
+    assert [int(r[0]) for r in rows] == [1, 1024, 65536, 1 << 18, 1 << 20, 1 << 22]
+    assert all(float(r[1]) > 0 for r in rows)
