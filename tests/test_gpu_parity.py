@@ -479,3 +479,66 @@ def test_prod_and_64_bit_types_fold_in_mesh_order_under_write_reduce_algorithms(
         reduce_scatter_as_mesh(DT.FP64, SUM, 9_001, algo, 4)
         reduce_scatter_as_mesh(DT.FP32, PROD, 9_001, algo, 5)
         reduce_scatter_as_mesh(DT.FP16, PROD, 9_001, algo, 6)
+
+
+def test_warmed_up_collectives_can_be_captured_into_a_graph_and_replayed():
+    """After one eager call (which uploads the fold programs) AllReduce, ReduceScatter and AllGather are plain kernel
+    launches on the caller's stream: a captured graph of them must reproduce the eager results on every replay,
+    with eager work and synchronisations between the replays."""
+    import torch
+    n, count = 8, 50_000
+    w = World(n)
+    try:
+        rng = np.random.default_rng(4242)
+        ins = [torch.from_numpy(rng.standard_normal(n * count).astype(np.float32)).cuda() for _ in range(n)]
+        ar = [torch.zeros(n * count, device="cuda") for _ in range(n)]
+        rs = [torch.zeros(count, device="cuda") for _ in range(n)]
+        ag = [torch.zeros(n * count, device="cuda") for _ in range(n)]
+        w.set_algo(OpKind.ALL_REDUCE, "rhd")
+        w.set_algo(OpKind.REDUCE_SCATTER, "nhr")
+
+        def step():
+            with hccl_amd.group():
+                for r in range(n):
+                    hccl_amd.all_reduce(w.comms[r], ins[r], ar[r], n * count, DT.FP32, OP.SUM, w.stream)
+            with hccl_amd.group():
+                for r in range(n):
+                    hccl_amd.reduce_scatter(w.comms[r], ins[r], rs[r], count, DT.FP32, OP.SUM, w.stream)
+            with hccl_amd.group():
+                for r in range(n):
+                    hccl_amd.all_gather(w.comms[r], rs[r], ag[r], count, DT.FP32, w.stream)
+
+        torch.cuda.synchronize()
+        step()
+        w.sync()
+        eager = [[t.clone() for t in group] for group in (ar, rs, ag)]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=w.stream):
+            step()
+        for replay in range(4):
+            for group in (ar, rs, ag):
+                for t in group:
+                    t.fill_(float(replay))                  # eager work between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for got, want in zip((ar, rs, ag), eager):
+                for r in range(n):
+                    assert torch.equal(got[r], want[r]), (replay, r)
+        # new inputs through the same graph: the kernels read the buffers, not a snapshot
+        for t in ins:
+            t.mul_(-0.5)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        step()
+        w.sync()
+        for r in range(n):
+            assert torch.equal(ar[r], ar[0]) and torch.equal(ag[r], ag[0])
+        want = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+        host = [t.cpu().numpy() for t in ins]
+        assert oracle.reduce_scatter(host, want, count, int(DT.FP32), SUM, acc=oracle.ACC_FP32, algo="nhr") == 0
+        for r in range(n):
+            assert np.array_equal(rs[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32))
+    finally:
+        w.close()
