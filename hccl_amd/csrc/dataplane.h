@@ -106,7 +106,7 @@ constexpr uint32_t kBcastHintMax = 64;      // buckets of the hint table held in
 constexpr uint32_t kA2aHintMax = 4096;      // buckets of the hint table held in device memory
 
 enum CopyMode : uint32_t {
-    COPY_GENERAL = 0,     // source and destination of a segment may differ modulo 16: staged through LDS
+    COPY_GENERAL = 0,     // source and destination of a segment may differ modulo 16: lanes realign the bytes
     COPY_CONGRUENT = 1,   // every segment has source == destination modulo 16
     COPY_ALIGNED = 2,     // all addresses and lengths are multiples of 16
 };

@@ -4,8 +4,8 @@
 // 16-byte vector position, pulls that position from the N rank buffers with 128-bit loads, combines
 // them in registers in the order a fold program dictates, and writes the result once per
 // destination.  The path is bound by HBM bandwidth (N reads + M writes of the element range, no
-// re-reads, no staging passes), so there is no MFMA; LDS only holds the 320-byte program and, for
-// tree-shaped orders, the accumulators of enclosing levels.
+// re-reads, no staging passes), so there is no MFMA; the fold program is read with scalar loads, and LDS only
+// holds, for tree-shaped orders, the accumulators of enclosing levels.
 //
 // Operand roles follow the reference's pairwise step  dst[i] = src[i] (+) dst[i]
 // (alg_data_trans_wrapper.cc:1319-1358):
