@@ -2108,3 +2108,50 @@ int orc_batch_send_recv(uint32_t n, const orc_send_recv_item_t* const* items, co
     free(rx);
     return rc;
 }
+
+/* ---------------------------------------------------------------------------------------------
+ * a16: the variable-length argument area of AlltoAllV (all_to_all_v.cc:600-643, template_utils.h:110-159)
+ * ------------------------------------------------------------------------------------------- */
+/* ConstructVarData: [sendCounts | recvCounts | sdispls | rdispls], n values each. */
+void orc_a2a_construct_var_data(uint32_t n, const uint64_t* sendCounts, const uint64_t* recvCounts,
+                                const uint64_t* sdispls, const uint64_t* rdispls, uint64_t* varData)
+{
+    for (uint64_t i = 0; i < 4ull * n; ++i) {
+        const uint64_t* from = i / n == 0 ? sendCounts : i / n == 1 ? recvCounts : i / n == 2 ? sdispls : rdispls;
+        varData[i] = from[i % n];
+    }
+}
+
+/* ParseAlltoAllVarData: element counts / displacements and their byte lengths / offsets; the area must hold
+ * exactly four vectors (up to five for AlltoAllVC) of n values.  out = 8 arrays of n values:
+ * sendCounts, sendLength, recvCounts, recvLength, sendDispls, sendOffset, recvDispls, recvOffset. */
+int orc_a2a_parse_var_data(const uint64_t* varData, uint64_t varBytes, uint64_t n, uint64_t elemSize, int isVC,
+                           uint64_t* out)
+{
+    uint64_t minBytes = 4 * n * sizeof(uint64_t);
+    uint64_t maxBytes = isVC ? 5 * n * sizeof(uint64_t) : minBytes;
+    if (n == 0 || varData == NULL || varBytes < minBytes || varBytes > maxBytes ||
+        varBytes % (n * sizeof(uint64_t)) != 0) {
+        return ORC_E_PARA;
+    }
+    for (uint64_t index = 0; index < 4 * n; ++index) {
+        uint64_t vec = index / n, rank = index % n;
+        out[(2 * vec) * n + rank] = varData[index];
+        out[(2 * vec + 1) * n + rank] = varData[index] * elemSize;
+    }
+    return ORC_OK;
+}
+
+/* CalcInputOutputSize: the furthest byte either buffer is touched at. */
+void orc_a2a_io_size(uint32_t n, const uint64_t* sendCounts, const uint64_t* recvCounts, const uint64_t* sdispls,
+                     const uint64_t* rdispls, uint64_t elemSize, uint64_t* inputBytes, uint64_t* outputBytes)
+{
+    *inputBytes = 0;
+    *outputBytes = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        uint64_t in = (sdispls[i] + sendCounts[i]) * elemSize;
+        uint64_t out = (rdispls[i] + recvCounts[i]) * elemSize;
+        *inputBytes = in > *inputBytes ? in : *inputBytes;
+        *outputBytes = out > *outputBytes ? out : *outputBytes;
+    }
+}

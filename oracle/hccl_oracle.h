@@ -226,6 +226,17 @@ typedef struct {
 } orc_send_recv_item_t;
 int orc_batch_send_recv(uint32_t n, const orc_send_recv_item_t* const* items, const uint32_t* itemNum);
 
+/* --- a16: AlltoAllV's variable-length argument area --------------------------------------
+ * all_to_all_v.cc:600-643 (CalcInputOutputSize, ConstructVarData), template_utils.h:110-159
+ * (ParseAlltoAllVarData: out = sendCounts, sendLength, recvCounts, recvLength, sendDispls, sendOffset,
+ * recvDispls, recvOffset, n values each). */
+void orc_a2a_construct_var_data(uint32_t n, const uint64_t* sendCounts, const uint64_t* recvCounts,
+                                const uint64_t* sdispls, const uint64_t* rdispls, uint64_t* varData);
+int orc_a2a_parse_var_data(const uint64_t* varData, uint64_t varBytes, uint64_t n, uint64_t elemSize, int isVC,
+                           uint64_t* out);
+void orc_a2a_io_size(uint32_t n, const uint64_t* sendCounts, const uint64_t* recvCounts, const uint64_t* sdispls,
+                     const uint64_t* rdispls, uint64_t elemSize, uint64_t* inputBytes, uint64_t* outputBytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -279,3 +279,31 @@ def test_loop_limits_closed_forms(orc):
         assert orc.rhd_max_count_per_loop(ccl, count, p, esz) == (0, want)
     assert orc.rhd_max_count_per_loop(512, 73, 72, 4)[0] == 4       # too small for the tail tiles
     assert orc.rhd_max_count_per_loop(200, 12, 6, 8)[0] == 4        # half of it, floored to 128 B, holds no whole frame
+
+
+def test_all_to_all_v_var_area_layout_and_parse(orc):
+    """[sendCounts | recvCounts | sdispls | rdispls]; parsing yields counts and byte lengths, displacements and
+    byte offsets; the furthest touched byte of either buffer; the size rules of the parser."""
+    import ctypes
+    L = orc.lib()
+    n = 3
+    u64 = lambda v: (ctypes.c_uint64 * len(v))(*v)
+    sc, rc_, sd, rd = [5, 0, 7], [1, 2, 3], [0, 5, 9], [4, 0, 10]
+    var = (ctypes.c_uint64 * (4 * n))()
+    L.orc_a2a_construct_var_data(ctypes.c_uint32(n), u64(sc), u64(rc_), u64(sd), u64(rd), var)
+    assert list(var) == sc + rc_ + sd + rd
+    out = (ctypes.c_uint64 * (8 * n))()
+    assert L.orc_a2a_parse_var_data(var, ctypes.c_uint64(4 * n * 8), ctypes.c_uint64(n), ctypes.c_uint64(2), 0, out) == 0
+    assert list(out) == sc + [2 * v for v in sc] + rc_ + [2 * v for v in rc_] + sd + [2 * v for v in sd] + rd + \
+        [2 * v for v in rd]
+    # exactly four vectors; AlltoAllVC may carry a fifth; a ragged size is refused
+    for nbytes, vc, want in ((4 * n * 8, 0, 0), (4 * n * 8 - 8, 0, 1), (5 * n * 8, 0, 1), (5 * n * 8, 1, 0),
+                             (4 * n * 8 + 8, 1, 1), (6 * n * 8, 1, 1)):
+        big = (ctypes.c_uint64 * (6 * n))()
+        assert L.orc_a2a_parse_var_data(big, ctypes.c_uint64(nbytes), ctypes.c_uint64(n), ctypes.c_uint64(2), vc,
+                                        out) == want, (nbytes, vc)
+    assert L.orc_a2a_parse_var_data(var, ctypes.c_uint64(0), ctypes.c_uint64(0), ctypes.c_uint64(2), 0, out) == 1
+    i, o = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    L.orc_a2a_io_size(ctypes.c_uint32(n), u64(sc), u64(rc_), u64(sd), u64(rd), ctypes.c_uint64(2), ctypes.byref(i),
+                      ctypes.byref(o))
+    assert (i.value, o.value) == ((9 + 7) * 2, (10 + 3) * 2)
