@@ -237,6 +237,9 @@ int orc_a2a_parse_var_data(const uint64_t* varData, uint64_t varBytes, uint64_t 
 void orc_a2a_io_size(uint32_t n, const uint64_t* sendCounts, const uint64_t* recvCounts, const uint64_t* sdispls,
                      const uint64_t* rdispls, uint64_t elemSize, uint64_t* inputBytes, uint64_t* outputBytes);
 
+/* a4: LocalReduce's routing (wrapper.cc:901-928): 1 = host arithmetic (64-bit types, PROD), 0 = device. */
+int orc_local_reduce_runs_on_host(int dtype, int op);
+
 #ifdef __cplusplus
 }
 #endif
