@@ -323,10 +323,10 @@ def test_chain_operand_roles(orc):
     assert not np.signbit(acc[0])
 
 
-def test_local_reduce_routing():
+def test_local_reduce_routing(orc):
     """64-bit types and PROD are reduced on the host, everything else on the device: the same rule decides where
     the library falls back to the host-reduce mesh order."""
-    L = oracle.lib()
+    L = orc.lib()
     host = {(t, op) for t in range(18) for op in range(4) if L.orc_local_reduce_runs_on_host(t, op)}
     want = {(t, op) for t in range(18) for op in range(4) if t in (5, 6, 10) or op == 1}
     assert host == want
