@@ -241,3 +241,24 @@ def test_all_gather_and_broadcast_into_differently_aligned_buffers():
             assert np.array_equal(to_host(bufs[r], np.uint8), src), r
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("n,count", [(4, 10_001), (8, 65_536)])
+def test_all_gather_with_the_send_buffer_inside_the_receive_buffer(n, count):
+    """Every rank sends the slice of its own recvBuf where its contribution belongs (the entry point puts no
+    restriction on overlapping buffers, reference all_gather.cc:118-149): the own slot is copied onto itself."""
+    import torch
+    w = World(n)
+    try:
+        rng = np.random.default_rng(n + count)
+        parts = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]
+        recvs = [torch.zeros(n * count, dtype=torch.float32, device="cuda") for _ in range(n)]
+        for r in range(n):
+            recvs[r][r * count:(r + 1) * count] = torch.from_numpy(parts[r]).cuda()
+        sends = [recvs[r][r * count:(r + 1) * count] for r in range(n)]
+        w.all_gather(sends, recvs, count, DT.FP32)
+        want = np.concatenate(parts)
+        for r in range(n):
+            assert np.array_equal(recvs[r].cpu().numpy().view(np.uint32), want.view(np.uint32)), r
+    finally:
+        w.close()
