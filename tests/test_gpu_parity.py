@@ -542,3 +542,26 @@ def test_warmed_up_collectives_can_be_captured_into_a_graph_and_replayed():
             assert np.array_equal(rs[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32))
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("algo", ["mesh", "nhr", "rhd", "mesh_chunk"])
+def test_reduce_scatter_into_the_own_slice_of_the_send_buffer(algo):
+    """recvBuf = sendBuf + rank * recvCount: every position of a rank's own slice is read and then overwritten by
+    the one lane that folds it, so the overlap is harmless."""
+    import torch
+    n, c = 8, 30_011
+    w = World(n)
+    try:
+        rng = np.random.default_rng(7070)
+        ins = [rng.standard_normal(n * c).astype(np.float32) for _ in range(n)]
+        want = [np.zeros(c, dtype=np.float32) for _ in range(n)]
+        assert oracle.reduce_scatter(ins, want, c, int(DT.FP32), SUM, acc=oracle.ACC_FP32, algo=algo) == 0
+        sends = [torch.from_numpy(x).cuda() for x in ins]
+        recvs = [sends[r][r * c:(r + 1) * c] for r in range(n)]
+        w.reduce_scatter(sends, recvs, c, DT.FP32, OP.SUM, algo)
+        for r in range(n):
+            assert np.array_equal(recvs[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)), (algo, r)
+            other = (r + 1) % n          # the slices a rank does not own are untouched
+            assert np.array_equal(sends[r][other * c:(other + 1) * c].cpu().numpy(), ins[r][other * c:(other + 1) * c])
+    finally:
+        w.close()
