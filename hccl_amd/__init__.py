@@ -118,6 +118,7 @@ def lib():
     L.HcclAllGather.argtypes = [vp, vp, u64, i32, vp, vp]
     L.HcclAllGatherV.argtypes = [vp, u64, vp, vp, vp, i32, vp, vp]
     L.HcclAlltoAllV.argtypes = [vp, vp, vp, i32, vp, vp, vp, i32, vp, vp]
+    L.HcclAmdAlltoAllVNoAlloc.argtypes = [vp, vp, vp, i32, vp, vp, vp, i32, vp, vp]
     L.HcclAlltoAll.argtypes = [vp, u64, i32, vp, u64, i32, vp, vp]
     L.HcclAlltoAllVC.argtypes = [vp, vp, i32, vp, i32, vp, vp]
     L.HcclReduceScatterV.argtypes = [vp, vp, vp, vp, u64, i32, i32, vp, vp]
@@ -148,7 +149,8 @@ def lib():
                  "HcclSend", "HcclRecv", "HcclBatchSendRecv", "HcclBarrier",
                  "HcclCommInitAll", "HcclGetRootInfo", "HcclCommInitRootInfo", "HcclCommDestroy", "HcclGetRankSize",
                  "HcclGetRankId", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
-                 "HcclAmdGetFoldProgram", "HcclAmdSetCclBufferSize", "HcclAmdGetCclBufferSize"):
+                 "HcclAmdGetFoldProgram", "HcclAmdSetCclBufferSize", "HcclAmdGetCclBufferSize",
+                 "HcclAmdAlltoAllVNoAlloc"):
         getattr(L, name).restype = ctypes.c_int
     _lib = L
     return L
@@ -334,6 +336,16 @@ def all_to_all_v(hccl_comm, send_buf, send_counts, sdispls, send_type, recv_buf,
                                _as_ptr(recv_buf), _u64_array(recv_counts, n), _u64_array(rdispls, n), int(recv_type),
                                hccl_comm, _as_stream(stream))
     return check(code, "HcclAlltoAllV")
+
+
+def all_to_all_v_no_alloc(hccl_comm, send_buf, send_counts, sdispls, send_type, recv_buf, recv_counts, rdispls,
+                          recv_type, stream=None):
+    """all_to_all_v for callers that cannot allocate device memory (HcclAmdAlltoAllVNoAlloc)."""
+    n = get_rank_size(hccl_comm)
+    code = lib().HcclAmdAlltoAllVNoAlloc(_as_ptr(send_buf), _u64_array(send_counts, n), _u64_array(sdispls, n),
+                                         int(send_type), _as_ptr(recv_buf), _u64_array(recv_counts, n),
+                                         _u64_array(rdispls, n), int(recv_type), hccl_comm, _as_stream(stream))
+    return check(code, "HcclAmdAlltoAllVNoAlloc")
 
 
 def all_to_all(hccl_comm, send_buf, send_count, send_type, recv_buf, recv_count, recv_type, stream=None):

@@ -184,6 +184,7 @@ struct PendingOp {
     uint32_t arrived = 0;
     bool done = false;
     HcclResult result = HCCL_SUCCESS;
+    bool noAlloc = false;   // the allocation-free variant of the entry point was called
     std::vector<RankArgs> ranks;
 };
 
@@ -243,6 +244,9 @@ struct World {
     hipEvent_t a2aSlotFree[kStagingSlots] = {};
     bool a2aSlotUsed[kStagingSlots] = {};
     uint32_t a2aNext = 0;
+    // Allocation-free AlltoAllV: host image of the tables and the device array that receives them.
+    std::vector<uint64_t> a2aImage;
+    uint8_t* a2aScratch = nullptr;
     uint32_t reduceBlocks = 1u << 26;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
@@ -486,13 +490,10 @@ HcclResult TakeEvent(World* w, hipEvent_t* ev)
     return HCCL_SUCCESS;
 }
 
-// Bytes of one slot (host image == device image): a descriptor and a tile prefix (u32) per segment,
-// then the hint table (u32); 256-byte padded.
+// Bytes of one slot: the tables of a world whose n * n segments are all non-empty.
 size_t A2aSlotBytes(uint32_t n)
 {
-    size_t nn = static_cast<size_t>(n) * n;
-    size_t bytes = nn * (kA2aDescWords * sizeof(uint64_t) + sizeof(uint32_t)) + (kA2aHintMax + 4) * sizeof(uint32_t);
-    return (bytes + 255) & ~static_cast<size_t>(255);
+    return A2aTableBytes(static_cast<size_t>(n) * n);
 }
 
 // Calls may be in flight on different streams, so each of the kStagingSlots calls owns its own host
@@ -507,6 +508,29 @@ HcclResult EnsureA2aBuffers(World* w)
         HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&w->a2aHost[s]), A2aSlotBytes(w->n), hipHostMallocDefault));
         HIP_OK(hipEventCreateWithFlags(&w->a2aSlotFree[s], hipEventDisableTiming));
     }
+    return HCCL_SUCCESS;
+}
+
+// Set-up of the allocation-free entry point, on its first call in a world (the world's device is current):
+// the address of the device-resident table array, and the events a launch over several streams takes from
+// the pool, so that later calls create nothing.
+HcclResult PrepareNoAlloc(World* w)
+{
+    if (w->a2aScratch != nullptr) {
+        return HCCL_SUCCESS;
+    }
+    uint8_t* ptr = nullptr;
+    HIP_OK(A2aScratchOfCurrentDevice(&ptr));
+    while (w->eventPool.size() < w->n) {
+        hipEvent_t ev;
+        HIP_OK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        w->eventPool.push_back(ev);
+    }
+    if (w->doneEvent == nullptr) {
+        HIP_OK(hipEventCreateWithFlags(&w->doneEvent, hipEventDisableTiming));
+    }
+    w->a2aImage.assign(kA2aScratchBytes / sizeof(uint64_t), 0);
+    w->a2aScratch = ptr;
     return HCCL_SUCCESS;
 }
 
@@ -876,7 +900,9 @@ struct CopySeg {
 };
 
 // Copies a list of at most n * n non-empty segments with one launch of the descriptor-driven copy kernel.
-HcclResult RunSegmentCopy(World* w, const std::vector<CopySeg>& segs, hipStream_t s)
+// With `noAlloc` the tables travel in kernel arguments to the library's device-resident array instead of
+// through a pinned staging slot into allocated device memory.
+HcclResult RunSegmentCopy(World* w, const std::vector<CopySeg>& segs, hipStream_t s, bool noAlloc = false)
 {
     const uint32_t n = w->n;
     const uint32_t tileBytes = w->copyTileBytes != 0 ? w->copyTileBytes : 1024u;
@@ -887,16 +913,30 @@ HcclResult RunSegmentCopy(World* w, const std::vector<CopySeg>& segs, hipStream_
     if (nSeg > n * n) {
         return HCCL_E_INTERNAL;
     }
-    HcclResult rc = EnsureA2aBuffers(w);
-    if (rc != HCCL_SUCCESS) {
-        return rc;
+    uint64_t* hDesc;
+    uint8_t* dev;
+    uint32_t slot = 0;
+    if (noAlloc) {
+        if (A2aTableBytes(nSeg) > kA2aScratchBytes) {
+            Log(1, "the tables of %u segments (%zu bytes) exceed the %zu bytes of the allocation-free entry point", nSeg,
+                A2aTableBytes(nSeg), kA2aScratchBytes);
+            return HCCL_E_MEMORY;
+        }
+        hDesc = w->a2aImage.data();
+        dev = w->a2aScratch;
+    } else {
+        HcclResult rc = EnsureA2aBuffers(w);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+        slot = w->a2aNext;
+        w->a2aNext = (w->a2aNext + 1) % kStagingSlots;
+        if (w->a2aSlotUsed[slot]) {
+            HIP_OK(hipEventSynchronize(w->a2aSlotFree[slot]));   // the call that last used this slot has finished
+        }
+        hDesc = w->a2aHost[slot];
+        dev = w->a2aDev + slot * A2aSlotBytes(n);
     }
-    const uint32_t slot = w->a2aNext;
-    w->a2aNext = (w->a2aNext + 1) % kStagingSlots;
-    if (w->a2aSlotUsed[slot]) {
-        HIP_OK(hipEventSynchronize(w->a2aSlotFree[slot]));   // the call that last used this slot has finished
-    }
-    uint64_t* hDesc = w->a2aHost[slot];
     uint32_t* hEnd = reinterpret_cast<uint32_t*>(hDesc + static_cast<size_t>(kA2aDescWords) * nSeg);
     uint32_t* hHint = hEnd + ((nSeg + 1u) & ~1u);
     uint64_t tiles = 0;
@@ -922,14 +962,19 @@ HcclResult RunSegmentCopy(World* w, const std::vector<CopySeg>& segs, hipStream_
     a.hintShift = BuildTileHints(hEnd, nSeg, static_cast<uint32_t>(tiles), kA2aHintMax, hHint, &nHint);
     a.mode = !congruent ? COPY_GENERAL : ((misfit & 15u) == 0 ? COPY_ALIGNED : COPY_CONGRUENT);
     const size_t used = reinterpret_cast<uint8_t*>(hHint + nHint + 1) - reinterpret_cast<uint8_t*>(hDesc);
-    uint8_t* dev = w->a2aDev + slot * A2aSlotBytes(n);
-    HIP_OK(hipMemcpyAsync(dev, hDesc, used, hipMemcpyHostToDevice, s));
+    if (noAlloc) {
+        HIP_OK(LaunchTableWrite(dev, hDesc, static_cast<uint32_t>((used + 7) / 8), s));
+    } else {
+        HIP_OK(hipMemcpyAsync(dev, hDesc, used, hipMemcpyHostToDevice, s));
+    }
     a.desc = reinterpret_cast<const uint64_t*>(dev);
     a.tileEnd = reinterpret_cast<const uint32_t*>(a.desc + static_cast<size_t>(kA2aDescWords) * nSeg);
     a.hint = a.tileEnd + ((nSeg + 1u) & ~1u);
     HIP_OK(LaunchA2aCopy(a, static_cast<uint32_t>(tiles), tileBytes, s));
-    HIP_OK(hipEventRecord(w->a2aSlotFree[slot], s));
-    w->a2aSlotUsed[slot] = true;
+    if (!noAlloc) {
+        HIP_OK(hipEventRecord(w->a2aSlotFree[slot], s));
+        w->a2aSlotUsed[slot] = true;
+    }
     return HCCL_SUCCESS;
 }
 
@@ -966,7 +1011,7 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
                             reinterpret_cast<uint64_t>(p.ranks[i].recv) + vi[3 * n + j] * esz, len});
         }
     }
-    return RunSegmentCopy(w, segs, s);
+    return RunSegmentCopy(w, segs, s, p.noAlloc);
 }
 
 // ReduceScatterV, mesh order: rank k's output = in_k[displs[k] ..] first, then the other ranks ascending
@@ -1213,6 +1258,12 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
 {
     DeviceScope onWorldDevice(w->device);
     hipStream_t s = p.ranks[launcher].stream;
+    if (p.noAlloc) {
+        HcclResult prc = PrepareNoAlloc(w);
+        if (prc != HCCL_SUCCESS) {
+            return prc;
+        }
+    }
     // Order the fused kernel after everything queued so far on the other ranks' streams (a superset of
     // what each rank had queued when it called).  Ranks that share the launch stream need nothing.
     std::vector<hipEvent_t> used;
@@ -1286,7 +1337,7 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
 
 // Deposits one rank's arguments; the call that completes the set launches.
 HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count, const void* send,
-                  void* recv, hipStream_t stream, std::vector<uint64_t>&& var, uint32_t root = 0)
+                  void* recv, hipStream_t stream, std::vector<uint64_t>&& var, uint32_t root = 0, bool noAlloc = false)
 {
     World* w = c->world;
     std::unique_lock<std::mutex> lock(w->mu);
@@ -1302,10 +1353,12 @@ HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uin
         cell->op = op;
         cell->count = count;
         cell->root = root;
+        cell->noAlloc = noAlloc;
         cell->ranks.resize(w->n);
     }
     std::shared_ptr<PendingOp> p = cell;
-    if (p->type != type || p->dtype != dtype || p->op != op || p->count != count || p->root != root) {
+    if (p->type != type || p->dtype != dtype || p->op != op || p->count != count || p->root != root ||
+        p->noAlloc != noAlloc) {
         Log(1, "%s on rank %u does not match the call of the other ranks (%s, count %llu, type %d, root %u)",
             OpName(type), c->rank, OpName(p->type), (unsigned long long)p->count, static_cast<int>(p->dtype), p->root);
         p->result = HCCL_E_PARA;
@@ -1487,12 +1540,71 @@ namespace {
 // Common tail of every entry point: the environment verdict, then the rendezvous.
 HcclResult SubmitWithReady(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count,
                            const void* send, void* recv, aclrtStream stream, std::vector<uint64_t>&& var,
-                           uint32_t root = 0)
+                           uint32_t root = 0, bool noAlloc = false)
 {
     if (c->world->envInvalid) {
         return HCCL_E_PARA;   // the reference's environment parsing fails every entry point the same way
     }
-    return Submit(c, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var), root);
+    return Submit(c, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var), root,
+                  noAlloc);
+}
+
+// HcclAlltoAllV and its allocation-free variant: reference src/ops/all_to_all_v/all_to_all_v.cc:105-129, 517-598.
+// Like the reference, only recvType is consulted for the element size.
+HcclResult AlltoAllVEntry(const char* name, const void* sendBuf, const void* sendCounts, const void* sdispls,
+                          const void* recvBuf, const void* recvCounts, const void* rdispls, HcclDataType recvType,
+                          HcclComm comm, aclrtStream stream, bool noAlloc)
+{
+#define CHK_ENTRY_PTR(p, what)                                \
+    do {                                                      \
+        if ((p) == nullptr) {                                 \
+            Log(1, "%s: %s is nullptr", name, what);  \
+            return HCCL_E_PTR;                                \
+        }                                                     \
+    } while (0)
+    CHK_ENTRY_PTR(comm, "comm");
+    CHK_ENTRY_PTR(sendCounts, "sendCounts");
+    CHK_ENTRY_PTR(sdispls, "sdispls");
+    CHK_ENTRY_PTR(recvCounts, "recvCounts");
+    CHK_ENTRY_PTR(rdispls, "rdispls");
+    CHK_ENTRY_PTR(stream, "stream");
+    if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
+        Log(1, "%s: sendBuf and recvBuf cannot be the same", name);
+        return HCCL_E_PARA;
+    }
+    Comm* c = AsComm(comm);
+    if (c == nullptr) {
+        Log(1, "%s: comm is not a live communicator", name);
+        return HCCL_E_PARA;
+    }
+    const uint32_t n = c->world->n;
+    const uint64_t* sc = static_cast<const uint64_t*>(sendCounts);
+    const uint64_t* rc = static_cast<const uint64_t*>(recvCounts);
+    bool sendZero = true, recvZero = true;
+    uint64_t maxCount = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        sendZero = sendZero && sc[i] == 0;
+        recvZero = recvZero && rc[i] == 0;
+        maxCount = sc[i] > maxCount ? sc[i] : maxCount;
+        maxCount = rc[i] > maxCount ? rc[i] : maxCount;
+    }
+    if (!sendZero) {
+        CHK_ENTRY_PTR(sendBuf, "sendBuf");
+    }
+    if (!recvZero) {
+        CHK_ENTRY_PTR(recvBuf, "recvBuf");
+    }
+#undef CHK_ENTRY_PTR
+    CHK_RET(CheckUserRank(c));
+    CHK_RET(CheckCount(maxCount));
+    CHK_RET(CheckDataType(recvType, false));
+    std::vector<uint64_t> var(4 * n);
+    memcpy(var.data(), sc, n * sizeof(uint64_t));
+    memcpy(var.data() + n, rc, n * sizeof(uint64_t));
+    memcpy(var.data() + 2 * n, sdispls, n * sizeof(uint64_t));
+    memcpy(var.data() + 3 * n, rdispls, n * sizeof(uint64_t));
+    return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
+                           const_cast<void*>(recvBuf), stream, std::move(var), 0, noAlloc);
 }
 
 }  // namespace
@@ -1634,51 +1746,18 @@ HcclResult HcclAlltoAllV(const void* sendBuf, const void* sendCounts, const void
                          const void* recvBuf, const void* recvCounts, const void* rdispls, HcclDataType recvType,
                          HcclComm comm, aclrtStream stream)
 {
-    // Reference src/ops/all_to_all_v/all_to_all_v.cc:105-129, 517-598.  Like the reference, only recvType
-    // is consulted for the element size.
     (void)sendType;
-    CHK_PTR(comm, "comm");
-    CHK_PTR(sendCounts, "sendCounts");
-    CHK_PTR(sdispls, "sdispls");
-    CHK_PTR(recvCounts, "recvCounts");
-    CHK_PTR(rdispls, "rdispls");
-    CHK_PTR(stream, "stream");
-    if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
-        Log(1, "HcclAlltoAllV: sendBuf and recvBuf cannot be the same");
-        return HCCL_E_PARA;
-    }
-    Comm* c = AsComm(comm);
-    if (c == nullptr) {
-        Log(1, "HcclAlltoAllV: comm is not a live communicator");
-        return HCCL_E_PARA;
-    }
-    const uint32_t n = c->world->n;
-    const uint64_t* sc = static_cast<const uint64_t*>(sendCounts);
-    const uint64_t* rc = static_cast<const uint64_t*>(recvCounts);
-    bool sendZero = true, recvZero = true;
-    uint64_t maxCount = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-        sendZero = sendZero && sc[i] == 0;
-        recvZero = recvZero && rc[i] == 0;
-        maxCount = sc[i] > maxCount ? sc[i] : maxCount;
-        maxCount = rc[i] > maxCount ? rc[i] : maxCount;
-    }
-    if (!sendZero) {
-        CHK_PTR(sendBuf, "sendBuf");
-    }
-    if (!recvZero) {
-        CHK_PTR(recvBuf, "recvBuf");
-    }
-    CHK_RET(CheckUserRank(c));
-    CHK_RET(CheckCount(maxCount));
-    CHK_RET(CheckDataType(recvType, false));
-    std::vector<uint64_t> var(4 * n);
-    memcpy(var.data(), sc, n * sizeof(uint64_t));
-    memcpy(var.data() + n, rc, n * sizeof(uint64_t));
-    memcpy(var.data() + 2 * n, sdispls, n * sizeof(uint64_t));
-    memcpy(var.data() + 3 * n, rdispls, n * sizeof(uint64_t));
-    return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
-                           const_cast<void*>(recvBuf), stream, std::move(var));
+    return AlltoAllVEntry("HcclAlltoAllV", sendBuf, sendCounts, sdispls, recvBuf, recvCounts, rdispls, recvType, comm,
+                          stream, false);
+}
+
+HcclResult HcclAmdAlltoAllVNoAlloc(const void* sendBuf, const void* sendCounts, const void* sdispls,
+                                   HcclDataType sendType, const void* recvBuf, const void* recvCounts,
+                                   const void* rdispls, HcclDataType recvType, HcclComm comm, aclrtStream stream)
+{
+    (void)sendType;
+    return AlltoAllVEntry("HcclAmdAlltoAllVNoAlloc", sendBuf, sendCounts, sdispls, recvBuf, recvCounts, rdispls,
+                          recvType, comm, stream, true);
 }
 
 HcclResult HcclAlltoAll(const void* sendBuf, uint64_t sendCount, HcclDataType sendType, const void* recvBuf,

@@ -23,7 +23,14 @@
 //                 (ins_temp_all_to_all_v_mesh_1D.cc:229-246, 459-611)
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "dataplane.h"
+
+// Tables (descriptors, tile prefixes, hints) of the allocation-free AlltoAllV.  Every GPU the library runs on
+// holds its own copy of this array at its own address; host code never uses the array's name as an address but
+// the pointer hipGetSymbolAddress returns for the current device (A2aScratchOfCurrentDevice).
+static __device__ __align__(256) uint8_t scratch[hccl_amd::kA2aScratchBytes];
 
 namespace hccl_amd {
 namespace {
@@ -237,7 +244,69 @@ hipError_t LaunchA2aT(const A2aArgs& a, uint32_t tiles, hipStream_t stream)
     return hipGetLastError();
 }
 
+// One argument-borne piece of a table image: words[0 .. nWords) go to table[firstWord ...].
+constexpr uint32_t kChunkWords = 448;
+struct TableChunk {
+    uint32_t firstWord;
+    uint32_t nWords;
+    uint64_t words[kChunkWords];
+};
+
+__global__ __launch_bounds__(64) void TableWriteKernel(uint64_t* table, const TableChunk chunk)
+{
+    const uint32_t i = blockIdx.x * 64u + threadIdx.x;
+    if (i < chunk.nWords) {
+        table[chunk.firstWord + i] = chunk.words[i];
+    }
+}
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratchMu;
+uint8_t* g_scratchPtr[kMaxDevices] = {};
+
 }  // namespace
+
+hipError_t A2aScratchOfCurrentDevice(uint8_t** ptr)
+{
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) {
+        return e;
+    }
+    if (device < 0 || device >= kMaxDevices) {
+        return hipErrorInvalidDevice;
+    }
+    std::lock_guard<std::mutex> lock(g_scratchMu);
+    if (g_scratchPtr[device] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) {
+            return e;
+        }
+        g_scratchPtr[device] = static_cast<uint8_t*>(p);
+    }
+    *ptr = g_scratchPtr[device];
+    return hipSuccess;
+}
+
+hipError_t LaunchTableWrite(uint8_t* table, const uint64_t* image, uint32_t nWords, hipStream_t stream)
+{
+    TableChunk chunk = {};
+    for (uint32_t first = 0; first < nWords; first += kChunkWords) {
+        chunk.firstWord = first;
+        chunk.nWords = nWords - first < kChunkWords ? nWords - first : kChunkWords;
+        for (uint32_t i = 0; i < chunk.nWords; ++i) {
+            chunk.words[i] = image[first + i];
+        }
+        hipLaunchKernelGGL(TableWriteKernel, dim3((chunk.nWords + 63u) / 64u), dim3(64), 0, stream,
+                           reinterpret_cast<uint64_t*>(table), chunk);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            return e;
+        }
+    }
+    return hipSuccess;
+}
 
 hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStream_t stream)
 {

@@ -173,6 +173,26 @@ struct A2aArgs {
     uint32_t mode;        // CopyMode
 };
 
+// Tables of one AlltoAllV launch (host image == device image): a descriptor and a tile prefix (u32) per
+// segment, then the hint table (u32); 256-byte padded.
+inline size_t A2aTableBytes(size_t nSeg)
+{
+    size_t bytes = nSeg * (kA2aDescWords * sizeof(uint64_t) + sizeof(uint32_t)) + (kA2aHintMax + 4) * sizeof(uint32_t);
+    return (bytes + 255) & ~static_cast<size_t>(255);
+}
+
+// The allocation-free AlltoAllV keeps its tables in a device array that is part of the library's code object
+// (one copy per GPU, held until the process ends) instead of allocated memory: room for the tables of the
+// largest world, kMaxRanks * kMaxRanks non-empty segments.
+constexpr size_t kA2aScratchBytes =
+    ((static_cast<size_t>(kMaxRanks) * kMaxRanks * (kA2aDescWords * sizeof(uint64_t) + sizeof(uint32_t)) +
+      (kA2aHintMax + 4) * sizeof(uint32_t)) + 255) & ~static_cast<size_t>(255);
+// Address of that array on the current device (looked up once per device).
+hipError_t A2aScratchOfCurrentDevice(uint8_t** ptr);
+// Writes `nWords` 64-bit words of a host image to `table` (device memory) with small kernels that carry the words
+// in their arguments: no copy engine, no staging memory, and the launches can be captured in a graph.
+hipError_t LaunchTableWrite(uint8_t* table, const uint64_t* image, uint32_t nWords, hipStream_t stream);
+
 // Launchers (defined in the .hip files).  All are asynchronous on `stream`.
 // ldsBytes = (plan depth - 1) * ReduceAccBytes(dtype, op) * args.threads: the accumulator stack of nested levels.
 hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t nBlocks,

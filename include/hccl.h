@@ -75,6 +75,21 @@ HcclResult HcclAlltoAllV(const void* sendBuf, const void* sendCounts, const void
                          HcclComm comm, aclrtStream stream);
 
 /*
+ * HcclAlltoAllV for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same arguments, checks and result as
+ * HcclAlltoAllV; every rank of a collective must call the same variant (HCCL_E_PARA otherwise).  The
+ * segment tables live in a device array that is part of the library (164,096 bytes per GPU, held until the
+ * process ends) and reach it inside kernel arguments, so the call performs no hipMalloc / hipFree /
+ * hipHostMalloc and no copy from host memory.  The first call in a world looks up the array's address and
+ * creates the events a launch over several streams uses.  HCCL_E_MEMORY if the tables of the call's non-empty
+ * segments exceed the array (cannot happen up to HCCL_AMD_MAX_RANKS ranks).  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (different streams without ordering, different worlds) race.
+ */
+HcclResult HcclAmdAlltoAllVNoAlloc(const void* sendBuf, const void* sendCounts, const void* sdispls,
+                                   HcclDataType sendType, const void* recvBuf, const void* recvCounts,
+                                   const void* rdispls, HcclDataType recvType, HcclComm comm, aclrtStream stream);
+
+/*
  * AlltoAllV with sendCounts = recvCounts = recvCount for every peer and displacements i * recvCount:
  * rank i's recvBuf[j*recvCount + e] = sendBuf_j[i*recvCount + e].  sendCount must equal recvCount and
  * sendType recvType.  Replaces reference include/hccl.h:234-236 (src/ops/all_to_all_v/all_to_all_v.cc:24).

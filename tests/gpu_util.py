@@ -161,3 +161,28 @@ def same_bits_nan_class(got, want, float_view=None):
     g, w = float_view(got), float_view(want)
     both = np.isnan(g) & np.isnan(w)
     return np.array_equal(got[~both], want[~both]) and np.array_equal(np.isnan(g), np.isnan(w))
+
+
+def rand_bytes(rng, nbytes):
+    return rng.integers(0, 256, nbytes, dtype=np.uint8)
+
+
+# A random AlltoAllV case: counts up to max_count with some empty segments; unless `aligned`, displacements are
+# shuffled and leave gaps, so sources and destinations sit at arbitrary element offsets.
+def a2a_case(rng, n, esz, max_count, aligned):
+    send_counts = rng.integers(0, max_count, size=(n, n)).astype(np.uint64)
+    send_counts[rng.random((n, n)) < 0.15] = 0
+    if aligned:
+        send_counts = (send_counts // (16 // esz)) * (16 // esz)
+    recv_counts = send_counts.T.copy()
+    sdispls = np.zeros((n, n), dtype=np.uint64)
+    rdispls = np.zeros((n, n), dtype=np.uint64)
+    for r in range(n):
+        for tab, cnts in ((sdispls, send_counts), (rdispls, recv_counts)):
+            off = 0
+            for j in (range(n) if aligned else rng.permutation(n)):
+                tab[r, j] = off
+                off += int(cnts[r, j]) + (0 if aligned else int(rng.integers(0, 4)))
+    in_sz = int((sdispls + send_counts).max()) + 1
+    out_sz = int((rdispls + recv_counts).max()) + 1
+    return send_counts, sdispls, recv_counts, rdispls, in_sz, out_sz

@@ -9,7 +9,7 @@ import hccl_amd
 import oracle
 from hccl_amd import HcclDataType as DT, HcclReduceOp as OP
 
-from gpu_util import World, dev_zeros, require_library_on_gpu, to_dev, to_host
+from gpu_util import World, a2a_case, dev_zeros, rand_bytes, require_library_on_gpu, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
 FILL = 0xAB
@@ -18,10 +18,6 @@ FILL = 0xAB
 @pytest.fixture(scope="module", autouse=True)
 def _native_library():
     require_library_on_gpu()
-
-
-def rand_bytes(rng, nbytes):
-    return rng.integers(0, 256, nbytes, dtype=np.uint8)
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 8, 64])
@@ -71,25 +67,6 @@ def test_all_gather_v_unordered_holes_and_odd_offsets(n):
                 assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), (n, trial, r)
     finally:
         w.close()
-
-
-def a2a_case(rng, n, esz, max_count, aligned):
-    send_counts = rng.integers(0, max_count, size=(n, n)).astype(np.uint64)
-    send_counts[rng.random((n, n)) < 0.15] = 0
-    if aligned:
-        send_counts = (send_counts // (16 // esz)) * (16 // esz)
-    recv_counts = send_counts.T.copy()
-    sdispls = np.zeros((n, n), dtype=np.uint64)
-    rdispls = np.zeros((n, n), dtype=np.uint64)
-    for r in range(n):
-        for tab, cnts in ((sdispls, send_counts), (rdispls, recv_counts)):
-            off = 0
-            for j in (range(n) if aligned else rng.permutation(n)):
-                tab[r, j] = off
-                off += int(cnts[r, j]) + (0 if aligned else int(rng.integers(0, 4)))
-    in_sz = int((sdispls + send_counts).max()) + 1
-    out_sz = int((rdispls + recv_counts).max()) + 1
-    return send_counts, sdispls, recv_counts, rdispls, in_sz, out_sz
 
 
 @pytest.mark.parametrize("n", [2, 3, 8, 64])
