@@ -250,8 +250,10 @@ struct World {
     uint32_t reduceBlocks = 1u << 26;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t copyTileBytes = 0;
+    uint32_t copyDstPerGroup = 0;   // HCCL_AMD_COPY_DST_PER_WAVE: destinations one wavefront stores to, 0 = per launch
     bool reduceVector = true;
     uint32_t reduceBatch = 0;     // HCCL_AMD_REDUCE_BATCH: 8 or 16, 0 = per launch
+    bool leadFromSrc = true;      // HCCL_AMD_LEAD_FROM_SRC=0: wavefronts always start on the destination's lines
     uint32_t storePolicy = 2;     // HCCL_AMD_STORE_POLICY for the reduce kernel: 0 non-temporal, 1 write-through, 2 per launch
     // HCCL_DETERMINISTIC (reference alg_env_config.cc:1113-1153): 0 false, 1 true, 2 strict, 0xFF unparsable
     uint8_t deterministic = 0;
@@ -375,12 +377,14 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->copyTileBytes != 1024 && w->copyTileBytes != 4096 && w->copyTileBytes != 16384) {
         w->copyTileBytes = 0;
     }
+    w->copyDstPerGroup = EnvU32("HCCL_AMD_COPY_DST_PER_WAVE", 0);
     w->execTimeout = EnvU32("HCCL_EXEC_TIMEOUT", 1836);
     w->storePolicy = EnvU32("HCCL_AMD_STORE_POLICY", 2);
     if (w->storePolicy > 2) {
         w->storePolicy = 2;
     }
     w->reduceVector = EnvU32("HCCL_AMD_REDUCE_VECTOR", 1) != 0;
+    w->leadFromSrc = getenv("HCCL_AMD_LEAD_FROM_SRC") == nullptr || atoi(getenv("HCCL_AMD_LEAD_FROM_SRC")) != 0;
     w->reduceBatch = EnvU32("HCCL_AMD_REDUCE_BATCH", 0);
     if (w->reduceBatch != 8 && w->reduceBatch != 16) {
         w->reduceBatch = 0;
@@ -569,7 +573,12 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     // A result that is written once (ReduceScatter(V), Reduce) leaves through write-through stores, 3-4 % faster
     // than non-temporal ones next to eight read streams; results written to many destinations (AllReduce)
     // keep non-temporal stores, 2-3 % faster there.  HCCL_AMD_STORE_POLICY = 0 / 1 forces one of them.
-    a.writeThrough = w->storePolicy != 2 ? w->storePolicy : ((a.dstOwn || a.nDst == 1) ? 1u : 0u);
+    const bool oneStream = a.dstOwn || a.nDst == 1;
+    a.writeThrough = w->storePolicy != 2 ? w->storePolicy : (oneStream ? 1u : 0u);
+    // Many sources folded into one result stream: the wavefronts start on the sources' 128-byte lines (a
+    // ReduceScatterV slice begins wherever its displacement puts it; measured 0.74 -> 0.80 of peak on uneven
+    // slices) and the single store stream straddles.  HCCL_AMD_LEAD_FROM_SRC=0 keeps the destination's lines.
+    a.leadFromSrc = (oneStream && w->leadFromSrc) ? 1u : 0u;
     // Up to eight ranks folded into one result stream run best with eight-load batches (fewer registers, more
     // wavefronts in flight: +1-2 %); AllReduce's many result streams and larger worlds with sixteen (+5 %).
     a.vecBatch = w->reduceBatch != 0 ? w->reduceBatch : ((w->n <= 8 && !a.varGroups && (a.dstOwn || a.nDst == 1)) ? 8u : 16u);
@@ -843,7 +852,7 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
 
 HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
 {
-    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s));   // 0: the launcher picks the tile
+    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s, w->copyDstPerGroup));   // 0: the launcher picks
     return HCCL_SUCCESS;
 }
 

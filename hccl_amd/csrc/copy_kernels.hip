@@ -23,6 +23,7 @@
 //                 (ins_temp_all_to_all_v_mesh_1D.cc:229-246, 459-611)
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
 #include <mutex>
 
 #include "dataplane.h"
@@ -39,16 +40,30 @@ typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
 
 // Payload pointers are rebuilt from integers; telling the compiler they are global memory keeps the
 // accesses off the flat path.
-template <typename V>
-__device__ __forceinline__ V LoadNt(const void* p)
+//
+// Cache policies.  A tile that one wavefront moves on its own (SHARED == false) is loaded non-temporally and its
+// 16-byte vectors are written through at system scope, the fastest pair for one read and one write stream.  A
+// tile whose destinations are split over several wavefronts of the same XCD (SHARED == true) is loaded with a
+// plain load, so that the XCD's L2 serves the wavefronts that come after the first, and stored non-temporally:
+// with two or three store streams per wavefront that measured 0.84-0.91 of the HBM peak for 1 read + 6..8
+// writes, against 0.71-0.74 for one wavefront storing to every destination under either store policy.
+template <typename V, bool SHARED>
+__device__ __forceinline__ V LoadVec(const void* p)
 {
-    return __builtin_nontemporal_load((const __attribute__((address_space(1))) V*)p);
+    if constexpr (SHARED) {
+        return *((const __attribute__((address_space(1))) V*)p);
+    } else {
+        return __builtin_nontemporal_load((const __attribute__((address_space(1))) V*)p);
+    }
 }
-template <typename V>
-__device__ __forceinline__ void StoreNt(V v, void* p)
+template <typename V, bool SHARED>
+__device__ __forceinline__ void StoreVec(V v, void* p)
 {
-    if constexpr (sizeof(V) == 16) {
+    if constexpr (sizeof(V) == 16 && !SHARED) {
         StoreStream16(p, __builtin_bit_cast(StreamVec, v));
+    } else if constexpr (sizeof(V) == 16) {
+        typedef V Unaligned __attribute__((aligned(1)));   // destinations may differ modulo 16 from the first
+        __builtin_nontemporal_store(v, (__attribute__((address_space(1))) Unaligned*)p);
     } else {
         __builtin_nontemporal_store(v, (__attribute__((address_space(1))) V*)p);
     }
@@ -75,6 +90,14 @@ __device__ __forceinline__ uint32_t FindSegment(uint32_t tile, uint32_t shift, H
         }
     }
     return lo;
+}
+
+// 1 when tileEnd <= tile, else 0, for tile < 2^31: in scalar arithmetic (a comparison result that is added up
+// as a number would travel through a vector register and back for every term).
+__device__ __forceinline__ uint32_t EndsAtOrBefore(uint32_t tileEnd, uint32_t tile)
+{
+    const uint32_t above = tile + 1u;
+    return (tileEnd > above ? tileEnd : above) - (tileEnd > tile ? tileEnd : tile);
 }
 
 // Four output dwords from five input dwords, dropping `shift` (0..3) leading bytes.
@@ -112,24 +135,82 @@ __device__ __forceinline__ U32x4 NextLane(U32x4 v, U32x4 last)
     return r;
 }
 
-// Copies one tile (bytes <= T * 16) from src to dstOf(d), d < nDst, one 16-byte vector per lane.  The stores
-// to dstOf(0) are 16-byte aligned; those to the other destinations are too when they share its offset from a
-// 16-byte boundary (the usual case) and are unaligned 128-bit stores otherwise.  Must be called by all T
-// threads of the workgroup.
-template <int T, int MODE, class DstFn>
-__device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uint32_t nDst, DstFn dstOf)
+// Calls store(address) for the destinations d < nDst, address = pointer of destination d + dOff.  The pointers
+// come in batches: kBatch scalar loads go out together (ptrOf(d) for a run of d, clamped to the last one) and
+// the stores follow back to back.  A loop that fetched one pointer per store would put a scalar-load round
+// trip between any two stores of a wavefront.  With kStatic the batch is ptrOf(0 .. kBatch - 1) exactly, so
+// that ptrOf may index registers.
+// Waits until at most `pace` of the wavefront's memory operations are outstanding (3 and above: no wait).
+__device__ __forceinline__ void PaceStores(uint32_t pace)
+{
+    if (pace == 0) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+    } else if (pace == 1) {
+        __builtin_amdgcn_s_waitcnt(0x0F71);
+    } else if (pace == 2) {
+        __builtin_amdgcn_s_waitcnt(0x0F72);
+    }
+}
+
+template <int kBatch, bool kStatic, class PtrFn, class StoreFn>
+__device__ __forceinline__ void ForEachDst(uint32_t nDst, uint64_t dOff, uint32_t pace, PtrFn ptrOf, StoreFn store)
+{
+    static_assert(kBatch == 1 || kBatch == 4 || kBatch == 8, "the fences below name every pointer of a batch");
+    for (uint32_t base = 0; base < nDst; base += kBatch) {
+        uint64_t ptr[kBatch];
+#pragma unroll
+        for (uint32_t k = 0; k < static_cast<uint32_t>(kBatch); ++k) {
+            if constexpr (kStatic) {
+                ptr[k] = ptrOf(k);
+            } else {
+                ptr[k] = ptrOf(base + k < nDst ? base + k : nDst - 1);
+            }
+        }
+        if constexpr (kBatch == 4) {
+            asm volatile("" : "+s"(ptr[0]), "+s"(ptr[1]), "+s"(ptr[2]), "+s"(ptr[3]));
+        } else if constexpr (kBatch == 8) {
+            asm volatile("" : "+s"(ptr[0]), "+s"(ptr[1]), "+s"(ptr[2]), "+s"(ptr[3]), "+s"(ptr[4]), "+s"(ptr[5]),
+                              "+s"(ptr[6]), "+s"(ptr[7]));
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < static_cast<uint32_t>(kBatch); ++k) {
+            if (base + k < nDst) {
+                store(reinterpret_cast<uint8_t*>(ptr[k] + dOff));
+                PaceStores(pace);
+            }
+        }
+        if constexpr (kStatic) {
+            break;
+        }
+    }
+}
+
+// A loaded value is made ready here, once, before the stores that take it: where each store sits in a block of
+// its own the compiler would otherwise wait in front of every one of them for all outstanding memory
+// operations, the previous store included, and a wavefront's stores would go out one round trip at a time.
+__device__ __forceinline__ void Ready(U32x4& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void Ready(uint32_t& v) { asm volatile("" : "+v"(v)); }
+
+// Copies one tile (bytes <= T * 16) from src to ptrOf(d) + dOff, d < nDst, one 16-byte vector per lane.  The
+// stores to destination 0 are 16-byte aligned; those to the other destinations are too when they share its
+// offset from a 16-byte boundary (the usual case) and are unaligned 128-bit stores otherwise.  Must be called
+// by all T threads of the workgroup.
+template <int T, int MODE, bool SHARED, int kBatch, bool kStatic, class PtrFn>
+__device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uint32_t nDst, uint64_t dOff, uint32_t pace,
+                                         PtrFn ptrOf)
 {
     const uint32_t idx = threadIdx.x;
     if (MODE == COPY_ALIGNED) {
         if (idx < bytes / 16u) {
-            const U32x4 v = LoadNt<U32x4>(reinterpret_cast<const U32x4*>(src) + idx);
-            for (uint32_t d = 0; d < nDst; ++d) {
-                StoreNt(v, reinterpret_cast<U32x4*>(dstOf(d)) + idx);
-            }
+            U32x4 v = LoadVec<U32x4, SHARED>(reinterpret_cast<const U32x4*>(src) + idx);
+            Ready(v);
+            ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
+                StoreVec<U32x4, SHARED>(v, reinterpret_cast<U32x4*>(dst) + idx);
+            });
         }
         return;
     }
-    const uint32_t dMis = static_cast<uint32_t>(reinterpret_cast<uint64_t>(dstOf(0)) & 15u);
+    const uint32_t dMis = static_cast<uint32_t>((ptrOf(0) + dOff) & 15u);
     uint32_t head = (16u - dMis) & 15u;     // bytes before the first aligned destination vector
     head = head < bytes ? head : bytes;
     const uint32_t nVec = (bytes - head) / 16u;   // <= T
@@ -140,7 +221,7 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
     U32x4 out = {0, 0, 0, 0};
     if (sMis == 0) {
         if (idx < nVec) {
-            out = LoadNt<U32x4>(reinterpret_cast<const U32x4*>(sBody) + idx);
+            out = LoadVec<U32x4, SHARED>(reinterpret_cast<const U32x4*>(sBody) + idx);
         }
     } else if (nVec != 0) {
         // Irregular: lane i loads the aligned vector i that covers the start of its output and takes
@@ -150,10 +231,10 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
         U32x4 a = {0, 0, 0, 0};
         U32x4 b = {0, 0, 0, 0};
         if (idx <= nVec) {
-            a = LoadNt<U32x4>(s + idx);
+            a = LoadVec<U32x4, SHARED>(s + idx);
         }
         if ((idx & 63u) == 63u && idx < nVec) {
-            b = LoadNt<U32x4>(s + idx + 1);
+            b = LoadVec<U32x4, SHARED>(s + idx + 1);
         }
         b = NextLane(a, b);
         const uint32_t shift = sMis & 3u;    // bytes to skip inside a dword
@@ -164,40 +245,106 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
             default: out = Funnel(a.w, b.x, b.y, b.z, b.w, shift); break;
         }
     }
-    if (idx < nVec) {
-        for (uint32_t d = 0; d < nDst; ++d) {
-            StoreNt(out, reinterpret_cast<U32x4*>(dstOf(d) + head) + idx);
-        }
-    }
-    // Up to 15 bytes in front of the body and up to 15 behind it.
+    // The edge byte (up to 15 in front of the body and up to 15 behind it) is requested before the body is stored.
     const uint32_t edge = head + (bytes - bodyEnd);
+    const uint32_t edgeAt = idx < head ? idx : bodyEnd + (idx - head);
+    uint32_t edgeByte = 0;
     if (idx < edge) {
-        const uint32_t o = idx < head ? idx : bodyEnd + (idx - head);
-        const uint8_t b = LoadNt<uint8_t>(src + o);
-        for (uint32_t d = 0; d < nDst; ++d) {
-            StoreNt(b, dstOf(d) + o);
-        }
+        edgeByte = LoadVec<uint8_t, SHARED>(src + edgeAt);
+    }
+    Ready(out);
+    Ready(edgeByte);
+    if (idx < nVec) {
+        ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
+            StoreVec<U32x4, SHARED>(out, reinterpret_cast<U32x4*>(dst + head) + idx);
+        });
+    }
+    if (idx < edge) {
+        ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
+            StoreVec<uint8_t, SHARED>(static_cast<uint8_t>(edgeByte), dst + edgeAt);
+        });
     }
 }
 
 // ---- AllGather / AllGatherV --------------------------------------------------------------------
-// Workgroup b copies tile b of the segment list held in the kernel arguments.
-template <int T, int MODE>
+// Workgroup b copies tile b of the segment list held in the kernel arguments to every destination (SPLIT ==
+// false), or to one group of at most kMaxSplitDst destinations (SPLIT == true).  In the split form the grid is
+// (8 * groups, blocks of eight tiles): workgroup x of a row copies tile x % 8 of the row's eight tiles to group
+// x / 8.  Workgroups are dealt to the eight XCDs in turn, so the groups of one tile land on the same XCD within
+// a short time of each other and all but the first find the tile in its L2.
+//
+// A wavefront has one 16-byte vector per lane in flight, so whatever it waits for before that load is issued is
+// lost bandwidth, the more so the fewer destinations it stores to.  Everything a wavefront needs therefore
+// comes in with two rounds of scalar loads of the kernel arguments: the first brings the tile prefixes (the tile
+// -> segment map is a branch-free count over them) and, in the split form, the group's destination pointers,
+// which the host has laid out by group; the second what the segment index selects.
+template <int T, int MODE, bool SPLIT>
 __global__ __launch_bounds__(T) void BcastCopyKernel(const BcastCopyArgs args)
 {
     constexpr uint32_t kTile = T * 16u;
-    const uint32_t tile = blockIdx.x;
-    const uint32_t seg = FindSegment(tile, args.hintShift, args.hint, args.tileEnd);
+    // First round: everything that does not depend on the segment.
+    uint32_t nTiles = args.nTiles;
+    uint32_t nDst = args.nDst;
+    uint32_t dstPerGroup = args.dstPerGroup;
+    uint32_t superY = args.superY;
+    uint32_t nSegPadded = args.nSegPadded;
+    uint32_t ends[16];
+#pragma unroll
+    for (uint32_t k = 0; k < 16; ++k) {
+        ends[k] = args.tileEnd[k];
+    }
+    uint64_t group[kMaxSplitDst] = {};
+    if constexpr (SPLIT) {
+#pragma unroll
+        for (uint32_t d = 0; d < kMaxSplitDst; ++d) {
+            group[d] = reinterpret_cast<uint64_t>(args.dst[(blockIdx.x >> 3) * kMaxSplitDst + d]);
+        }
+        static_assert(kMaxSplitDst == 4, "the fence below names every pointer of a group");
+        asm volatile("" : "+s"(group[0]), "+s"(group[1]), "+s"(group[2]), "+s"(group[3]));
+    }
+    asm volatile("" : "+s"(nTiles), "+s"(nDst), "+s"(dstPerGroup), "+s"(superY), "+s"(nSegPadded));
+    asm volatile("" : "+s"(ends[0]), "+s"(ends[1]), "+s"(ends[2]), "+s"(ends[3]), "+s"(ends[4]), "+s"(ends[5]),
+                      "+s"(ends[6]), "+s"(ends[7]), "+s"(ends[8]), "+s"(ends[9]), "+s"(ends[10]), "+s"(ends[11]),
+                      "+s"(ends[12]), "+s"(ends[13]), "+s"(ends[14]), "+s"(ends[15]));
+    uint32_t tile = blockIdx.x;
+    if constexpr (SPLIT) {
+        tile = ((blockIdx.z * superY + blockIdx.y) << 3) + (blockIdx.x & 7u);
+        const uint32_t firstDst = (blockIdx.x >> 3) * dstPerGroup;
+        nDst = nDst - firstDst < dstPerGroup ? nDst - firstDst : dstPerGroup;
+    }
+    // Number of segments that end at or before this tile = index of the tile's segment (prefixes past the last
+    // segment hold 0xFFFFFFFF; empty segments repeat their predecessor's prefix and are skipped by the count).
+    uint32_t seg = 0;
+#pragma unroll
+    for (uint32_t k = 0; k < 16; ++k) {
+        seg += EndsAtOrBefore(ends[k], tile);
+    }
+    for (uint32_t i = 16; i < nSegPadded; i += 16) {
+#pragma unroll
+        for (uint32_t k = 0; k < 16; ++k) {
+            seg += EndsAtOrBefore(args.tileEnd[i + k], tile);
+        }
+    }
+    if (SPLIT && tile >= nTiles) {
+        return;   // the last row of eight tiles may be short
+    }
     const uint32_t segFirst = seg == 0 ? 0u : args.tileEnd[seg - 1];
-    const uint64_t len = args.len[seg];
-    const uint32_t lead = TileLead(reinterpret_cast<uint64_t>(args.dst[0]) + args.dstOff[seg]);
+    uint64_t len = args.len[seg];
+    uint64_t srcBase = reinterpret_cast<uint64_t>(args.src[seg]);
+    uint64_t segDstOff = args.dstOff[seg];
+    asm volatile("" : "+s"(srcBase), "+s"(len), "+s"(segDstOff));   // second round: all requested together
+    const uint32_t lead = TileLead(args.leadBase + segDstOff);
     uint64_t off;
     uint32_t bytes;
     TileRange<kTile>(tile - segFirst, lead, len, &off, &bytes);
-    const uint8_t* src = static_cast<const uint8_t*>(args.src[seg]) + off;
-    const uint64_t dOff = args.dstOff[seg] + off;
-    auto dstOf = [&](uint32_t d) { return static_cast<uint8_t*>(args.dst[d]) + dOff; };
-    CopyTile<T, MODE>(src, bytes, args.nDst, dstOf);
+    const uint8_t* src = reinterpret_cast<const uint8_t*>(srcBase + off);
+    const uint64_t dOff = segDstOff + off;
+    if constexpr (SPLIT) {
+        CopyTile<T, MODE, true, kMaxSplitDst, true>(src, bytes, nDst, dOff, args.pace, [&](uint32_t d) { return group[d]; });
+    } else {
+        CopyTile<T, MODE, false, 8, false>(src, bytes, nDst, dOff, args.pace,
+                                           [&](uint32_t d) { return reinterpret_cast<uint64_t>(args.dst[d]); });
+    }
 }
 
 // ---- AlltoAllV -------------------------------------------------------------------------------------
@@ -218,17 +365,16 @@ __global__ __launch_bounds__(T) void A2aCopyKernel(const A2aArgs args)
     uint32_t bytes;
     TileRange<kTile>(tile - static_cast<uint32_t>(desc[3]), TileLead(dstBase), len, &off, &bytes);
     const uint8_t* src = reinterpret_cast<const uint8_t*>(srcBase + off);
-    uint8_t* dst = reinterpret_cast<uint8_t*>(dstBase + off);
-    CopyTile<T, MODE>(src, bytes, 1u, [&](uint32_t) { return dst; });
+    CopyTile<T, MODE, false, 1, true>(src, bytes, 1u, off, 3u, [&](uint32_t) { return dstBase; });
 }
 
-template <int T>
-hipError_t LaunchBcastT(const BcastCopyArgs& a, uint32_t mode, uint32_t tiles, hipStream_t stream)
+template <int T, bool SPLIT>
+hipError_t LaunchBcastT(const BcastCopyArgs& a, uint32_t mode, dim3 grid, hipStream_t stream)
 {
     switch (mode) {
-        case COPY_ALIGNED: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_ALIGNED>), dim3(tiles), dim3(T), 0, stream, a); break;
-        case COPY_CONGRUENT: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_CONGRUENT>), dim3(tiles), dim3(T), 0, stream, a); break;
-        default: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_GENERAL>), dim3(tiles), dim3(T), 0, stream, a); break;
+        case COPY_ALIGNED: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_ALIGNED, SPLIT>), grid, dim3(T), 0, stream, a); break;
+        case COPY_CONGRUENT: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_CONGRUENT, SPLIT>), grid, dim3(T), 0, stream, a); break;
+        default: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_GENERAL, SPLIT>), grid, dim3(T), 0, stream, a); break;
     }
     return hipGetLastError();
 }
@@ -308,15 +454,46 @@ hipError_t LaunchTableWrite(uint8_t* table, const uint64_t* image, uint32_t nWor
     return hipSuccess;
 }
 
-hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStream_t stream)
+hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStream_t stream, uint32_t dstPerGroup)
 {
     BcastCopyArgs a = in;
+    // Destinations split over wavefronts, two per wavefront up to sixteen destinations, four beyond (the tile is
+    // read once per group through L2): 0.85-0.92 of the HBM peak against 0.68-0.75 for one wavefront per tile,
+    // as long as the range written in each destination stays within 256 MiB; beyond that the split form
+    // measured slower (0.52-0.73) than the plain one and is not used.  Up to three destinations stay with one
+    // wavefront.
+    if (dstPerGroup == 0) {
+        uint64_t lo = ~0ull, hi = 0;
+        for (uint32_t j = 0; j < a.nSeg; ++j) {
+            if (a.len[j] != 0) {
+                lo = a.dstOff[j] < lo ? a.dstOff[j] : lo;
+                hi = a.dstOff[j] + a.len[j] > hi ? a.dstOff[j] + a.len[j] : hi;
+            }
+        }
+        const bool compact = hi > lo && hi - lo <= kSplitMaxExtent;
+        dstPerGroup = (a.nDst <= 3 || !compact) ? a.nDst : (a.nDst <= 16 ? 2u : 4u);
+    }
+    if (dstPerGroup > kMaxSplitDst && dstPerGroup < a.nDst) {
+        dstPerGroup = kMaxSplitDst;
+    }
+    if (dstPerGroup > a.nDst) {
+        dstPerGroup = a.nDst;
+    }
+    if (dstPerGroup == 0) {
+        return hipErrorInvalidValue;
+    }
+    a.dstPerGroup = dstPerGroup;
+    a.nGroup = (a.nDst + dstPerGroup - 1) / dstPerGroup;
+    const bool split = a.nGroup > 1;
     uint64_t misfit = 0;      // non-zero low bits: something is not 16-byte aligned
-    bool congruent = true;    // every segment's source shares the offset of its first destination
+    bool congruent = true;    // every segment's source shares the offset of the first destination of every group
+    const uint64_t dst0 = reinterpret_cast<uint64_t>(a.dst[0]);
     for (uint32_t d = 0; d < a.nDst; ++d) {
         misfit |= reinterpret_cast<uint64_t>(a.dst[d]);
+        if (d % dstPerGroup == 0) {
+            congruent = congruent && ((reinterpret_cast<uint64_t>(a.dst[d]) ^ dst0) & 15u) == 0;
+        }
     }
-    const uint64_t dst0 = reinterpret_cast<uint64_t>(a.dst[0]);
     for (uint32_t j = 0; j < a.nSeg; ++j) {
         if (a.len[j] != 0) {
             const uint64_t s = reinterpret_cast<uint64_t>(a.src[j]);
@@ -328,7 +505,7 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
     if (tileBytes == 0) {
         // One wavefront per tile, except where lanes realign their source for several destinations: there the
         // larger workgroup measured 1-2 % faster.
-        tileBytes = (mode == COPY_GENERAL && a.nDst > 1) ? 4096u : 1024u;
+        tileBytes = (mode == COPY_GENERAL && a.nDst > 1 && !split) ? 4096u : 1024u;
     }
     uint64_t tiles = 0;
     for (uint32_t j = 0; j < a.nSeg; ++j) {
@@ -341,13 +518,43 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
     if (tiles == 0) {
         return hipSuccess;
     }
-    uint32_t nHint = 0;
-    a.hintShift = BuildTileHints(a.tileEnd, a.nSeg, static_cast<uint32_t>(tiles), kBcastHintMax, a.hint, &nHint);
-    const uint32_t nTiles = static_cast<uint32_t>(tiles);
+    a.nSegPadded = (a.nSeg + 15u) & ~15u;
+    for (uint32_t j = a.nSeg; j < a.nSegPadded; ++j) {
+        a.tileEnd[j] = 0xFFFFFFFFu;
+    }
+    a.nTiles = static_cast<uint32_t>(tiles);
+    a.leadBase = dst0;
+    // A wavefront of the split form waits for each store before it issues the next; one that stores to every
+    // destination keeps two in flight (each measured best for its form; HCCL_AMD_COPY_PACE = 0..3 overrides).
+    static const int paceEnv = getenv("HCCL_AMD_COPY_PACE") ? atoi(getenv("HCCL_AMD_COPY_PACE")) : -1;
+    a.pace = paceEnv >= 0 ? static_cast<uint32_t>(paceEnv) : (split ? 0u : 1u);
+    if (!split) {
+        const dim3 grid(a.nTiles);
+        switch (tileBytes) {
+            case 1024: return LaunchBcastT<64, false>(a, mode, grid, stream);
+            case 4096: return LaunchBcastT<256, false>(a, mode, grid, stream);
+            case 16384: return LaunchBcastT<1024, false>(a, mode, grid, stream);
+            default: return hipErrorInvalidValue;
+        }
+    }
+    // Destination pointers by group, kMaxSplitDst slots each; rows of eight tiles (one per XCD), every row
+    // repeated once per group along x.
+    if (a.nGroup * kMaxSplitDst > static_cast<uint32_t>(kMaxRanks)) {
+        return hipErrorInvalidValue;
+    }
+    for (uint32_t k = 0; k < static_cast<uint32_t>(kMaxRanks); ++k) {
+        a.dst[k] = nullptr;
+    }
+    for (uint32_t d = 0; d < a.nDst; ++d) {
+        a.dst[(d / dstPerGroup) * kMaxSplitDst + d % dstPerGroup] = in.dst[d];
+    }
+    const uint32_t supers = static_cast<uint32_t>((tiles + 7) / 8);
+    a.superY = supers < 32768u ? supers : 32768u;
+    const dim3 grid(8u * a.nGroup, a.superY, (supers + a.superY - 1) / a.superY);
     switch (tileBytes) {
-        case 1024: return LaunchBcastT<64>(a, mode, nTiles, stream);
-        case 4096: return LaunchBcastT<256>(a, mode, nTiles, stream);
-        case 16384: return LaunchBcastT<1024>(a, mode, nTiles, stream);
+        case 1024: return LaunchBcastT<64, true>(a, mode, grid, stream);
+        case 4096: return LaunchBcastT<256, true>(a, mode, grid, stream);
+        case 16384: return LaunchBcastT<1024, true>(a, mode, grid, stream);
         default: return hipErrorInvalidValue;
     }
 }

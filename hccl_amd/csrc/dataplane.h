@@ -74,6 +74,7 @@ struct ReduceArgs {
     uint32_t threads; // workgroup size of the launch
     uint32_t vecBatch;       // leaves per load batch of the 128-bit path: 8 or 16 (picks the kernel instantiation)
     uint32_t writeThrough;   // 16-byte results leave through StoreStream16 instead of a non-temporal store
+    uint32_t leadFromSrc;    // wavefronts start on a 128-byte line of the sources instead of the destination
     // Groups of unequal length (ReduceScatterV): when varGroups is set, group g spans groupLenV[g]
     // elements starting groupOffV[g] elements into every source, instead of the uniform
     // groupLen / srcGroupStride / total geometry, and owns the workgroups
@@ -102,7 +103,6 @@ __device__ __forceinline__ void StoreStream16(void* p, StreamVec v)
 // table over buckets of 2^hintShift tiles (hint[k] = first segment with tileEnd > k << hintShift, one
 // closing entry) bounds the search of a workgroup to the segments that touch its bucket.  The kernels
 // read these tables with scalar loads only.
-constexpr uint32_t kBcastHintMax = 64;      // buckets of the hint table held in the kernel arguments
 constexpr uint32_t kA2aHintMax = 4096;      // buckets of the hint table held in device memory
 
 enum CopyMode : uint32_t {
@@ -146,9 +146,12 @@ inline uint32_t BuildTileHints(const uint32_t* tileEnd, uint32_t nSeg, uint32_t 
     return shift;
 }
 
-// One-to-many copy (AllGather / AllGatherV / single-rank shortcut): segment j is `len[j]` bytes read
-// once from src[j] and written to dst[d] + dstOff[j] for every d < nDst.  The caller fills the first
-// six members; LaunchBcastCopy derives the rest.
+// One-to-many copy (AllGather / AllGatherV / Broadcast / single-rank shortcut): segment j is `len[j]` bytes read
+// once from src[j] and written to dst[d] + dstOff[j] for every d < nDst.  The caller fills the first six
+// members; LaunchBcastCopy derives the rest: tileEnd[j] = inclusive prefix sum of the segments' tile counts,
+// padded with 0xFFFFFFFF up to nSegPadded (a multiple of 16) entries.
+constexpr uint32_t kMaxSplitDst = 4;   // most destinations one wavefront stores to when a tile's destinations are split
+constexpr uint64_t kSplitMaxExtent = 256ull << 20;   // largest written range per destination the split form is used for
 struct BcastCopyArgs {
     const void* src[kMaxRanks];
     void* dst[kMaxRanks];
@@ -156,10 +159,16 @@ struct BcastCopyArgs {
     uint64_t dstOff[kMaxRanks];
     uint32_t nSeg;
     uint32_t nDst;
-    uint32_t hintShift;
+    uint32_t nSegPadded;
+    uint32_t nTiles;
+    uint32_t dstPerGroup;   // destinations one wavefront stores to; nGroup = ceil(nDst / dstPerGroup) wavefronts per tile
+    uint32_t nGroup;        // when > 1, dst[] is laid out by group: group g's destinations at dst[g * kMaxSplitDst ...]
+    uint32_t superY;        // split form: rows of eight tiles along y before the grid continues along z
+    uint64_t leadBase;      // address of the first destination: tiles are cut on its 128-byte lines
+    uint32_t pace;          // stores of a wavefront that may be outstanding when it issues the next (3: no limit)
     uint32_t tileEnd[kMaxRanks];
-    uint8_t hint[kBcastHintMax + 8];
 };
+static_assert(kMaxRanks % 16 == 0, "the tile prefixes are searched sixteen at a time");
 
 // AlltoAllV: one descriptor of four u64 per non-empty segment (i <- j), all tables in device memory:
 //   desc[4s] = send_j + sdispls_j[i] * esz, desc[4s+1] = recv_i + rdispls_i[j] * esz,
@@ -203,8 +212,9 @@ inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
     // eight fp32 accumulators (half SUM) or sixteen 16-bit ones (int8) vs one 16-byte pack
     return ((half && op == HCCL_REDUCE_SUM) || dtype == HCCL_DATA_TYPE_INT8) ? 32u : 16u;
 }
-// tileBytes: 1024, 4096 or 16384; 0 lets the launcher choose.
-hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream);
+// tileBytes: 1024, 4096 or 16384; 0 lets the launcher choose.  dstPerGroup: destinations per wavefront, 0 lets
+// the launcher choose.
+hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream, uint32_t dstPerGroup = 0);
 hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, uint32_t tileBytes, hipStream_t stream);
 
 }  // namespace hccl_amd

@@ -622,8 +622,8 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     // body follows, and fewer than W elements remain.  Sources and further destinations only need element
     // alignment: their 128-bit accesses may be unaligned (full speed when they are congruent with the first
     // destination, up to 15 % less otherwise).  Without vecOk everything goes element by element.  The body's vectors are dealt to the lanes shifted by `lead`, so that lane 0
-    // of every wavefront starts a 128-byte line of the destination (a wavefront whose 1 KiB straddles nine
-    // lines moves two of them twice).
+    // of every wavefront starts a 128-byte line (a wavefront whose 1 KiB straddles nine lines moves two of them
+    // twice): of the destination, or with leadFromSrc of the sources.
     uint64_t head = len;
     uint64_t nVec = 0;
     uint32_t lead = 0;
@@ -633,7 +633,12 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
         head = mis ? (16u - mis) / sizeof(S) : 0;
         head = head < len ? head : len;
         nVec = (len - head) / W;
-        lead = static_cast<uint32_t>(((addr + head * sizeof(S)) >> 4) & 7u);
+        // One result stream fed by many sources: the sources' lines count (those of the first rank stand for all;
+        // peers' buffers are usually congruent), otherwise the destination's.
+        const uint64_t lineOf = args.leadFromSrc
+                                    ? reinterpret_cast<uint64_t>(args.src[0]) + (srcOff + head) * sizeof(S)
+                                    : addr + head * sizeof(S);
+        lead = static_cast<uint32_t>((lineOf >> 4) & 7u);
     }
     for (uint64_t u = first; u < nVec + lead; u += stride) {
         if (u >= lead) {
