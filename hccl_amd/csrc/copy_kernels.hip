@@ -482,6 +482,10 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
     if (dstPerGroup == 0) {
         return hipErrorInvalidValue;
     }
+    // the destination pointers of all groups, kMaxSplitDst slots each, must fit the argument array
+    while ((a.nDst + dstPerGroup - 1) / dstPerGroup * kMaxSplitDst > static_cast<uint32_t>(kMaxRanks)) {
+        ++dstPerGroup;
+    }
     a.dstPerGroup = dstPerGroup;
     a.nGroup = (a.nDst + dstPerGroup - 1) / dstPerGroup;
     const bool split = a.nGroup > 1;

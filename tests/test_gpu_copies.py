@@ -90,6 +90,69 @@ def test_all_to_all_v(n, aligned):
         w.close()
 
 
+@pytest.mark.parametrize("per_wave", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("n", [4, 7, 17, 64])
+def test_all_gather_v_with_destinations_split_over_wavefronts(monkeypatch, n, per_wave):
+    """The copy kernel's split form (every tile copied by several wavefronts, each storing to a few
+    destinations): group sizes 1 to 4 and the launcher's own choice, destination counts that leave a short last
+    group, segments that end inside a row of eight tiles, odd element displacements, differently aligned
+    buffers, empty segments."""
+    if per_wave:
+        monkeypatch.setenv("HCCL_AMD_COPY_DST_PER_WAVE", str(per_wave))
+    w = World(n)
+    monkeypatch.delenv("HCCL_AMD_COPY_DST_PER_WAVE", raising=False)
+    try:
+        rng = np.random.default_rng(5000 + 10 * n + per_wave)
+        esz = 2
+        for trial in range(3):
+            counts = rng.integers(0, 9_000 if n <= 17 else 1_500, n).astype(np.uint64)
+            counts[rng.integers(0, n)] = 0
+            if trial == 2:
+                counts = (counts // 8) * 8                      # everything 16-byte aligned
+            displs = np.zeros(n, dtype=np.uint64)
+            off = 0
+            for j in rng.permutation(n):
+                displs[j] = off
+                off += int(counts[j]) + (0 if trial == 2 else int(rng.integers(0, 3)))
+            total = off + 5
+            ins = [rand_bytes(rng, max(int(c), 1) * esz) for c in counts]
+            want = [np.full(total * esz, FILL, dtype=np.uint8) for _ in range(n)]
+            assert oracle.all_gather_v(ins, want, counts, displs, int(DT.FP16)) == 0
+            sends = [to_dev(x, pad_front=0 if trial == 2 else int(rng.integers(0, 8)) * 2) for x in ins]
+            recvs = [dev_zeros(total * esz, pad_front=0 if trial != 1 else 2 * (r % 5), fill=FILL) for r in range(n)]
+            w.all_gather_v(sends, recvs, counts, displs, DT.FP16)
+            for r in range(n):
+                assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), (n, per_wave, trial, r)
+    finally:
+        w.close()
+
+
+def test_broadcast_and_all_gather_beyond_the_split_form_s_extent():
+    """Destinations written over more than 256 MiB take the plain form of the copy kernel; checked by equality
+    with the source on the device (512 MiB broadcast to 4 ranks, AllGather of 5 x 80 MiB)."""
+    import torch
+    n, nbytes = 5, 512 << 20
+    w = World(n)
+    try:
+        g = torch.Generator(device="cuda")
+        g.manual_seed(77)
+        bufs = [torch.randint(0, 256, (nbytes,), generator=g, device="cuda", dtype=torch.uint8) for _ in range(n)]
+        want = bufs[3].clone()
+        w.broadcast(bufs, nbytes, DT.UINT8, 3)
+        for r in range(n):
+            assert torch.equal(bufs[r], want), r
+        del bufs, want
+        per = 80 << 20
+        sends = [torch.randint(0, 256, (per,), generator=g, device="cuda", dtype=torch.uint8) for _ in range(n)]
+        recvs = [torch.zeros(n * per, device="cuda", dtype=torch.uint8) for _ in range(n)]
+        w.all_gather(sends, recvs, per, DT.UINT8)
+        whole = torch.cat(sends)
+        for r in range(n):
+            assert torch.equal(recvs[r], whole), r
+    finally:
+        w.close()
+
+
 def test_all_to_all_v_moe_shape_zipf_small():
     """The MoE-dispatch shape of the headline AlltoAllV configuration at 1/64 of its token count:
     64 ranks, hidden 7168 bf16, per-destination token counts multinomial over Zipf(1.1) weights."""

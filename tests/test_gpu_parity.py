@@ -365,6 +365,31 @@ def test_workgroups_that_loop_over_several_positions(monkeypatch):
         w.close()
 
 
+@pytest.mark.parametrize("n", [2, 5, 16])
+def test_all_reduce_through_the_staging_slab(monkeypatch, n):
+    """The two-kernel form of the rank-order AllReduce (fold into a slab, slab to every recvBuf), forced for
+    small messages with a slab of 4 KiB so that counts span several pieces and end in a ragged one."""
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB", "1")
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB_BYTES", "4096")
+    w = World(n)
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB_BYTES")
+    try:
+        seed = 2000 + n
+        for dtype in REDUCE_TYPES:
+            for op in (SUM, MAX):
+                run_all_reduce(w, dtype, op, 4_093, "mesh", seed=seed)
+                seed += 1
+        run_all_reduce(w, DT.INT32, PROD, 17, "mesh", seed=seed)            # less than one piece
+        run_all_reduce(w, DT.FP32, SUM, 1_024, "ring", seed=seed + 1)       # exactly one piece
+        run_all_reduce(w, DT.FP32, SUM, 65_543, "ring", seed=seed + 2, pad=4)
+        run_all_reduce(w, DT.BFP16, SUM, 10_007, "mesh", seed=seed + 3, pad=lambda r, which: 2 * r + (6 if which == "recv" else 0))
+        run_all_reduce(w, DT.FP16, MIN, 9_001, "mesh", seed=seed + 4, in_place=True)
+        run_all_reduce(w, DT.FP32, SUM, 5_000, "rhd", seed=seed + 5)        # tree orders keep the fused kernel
+    finally:
+        w.close()
+
+
 def test_all_reduce_larger_than_a_million_workgroups():
     """2 x 1 GiB of fp16 per rank: 2^26 vector positions, one per lane, 2^20 workgroups per destination."""
     import torch
