@@ -19,6 +19,7 @@
 #include <memory>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "dataplane.h"
@@ -238,6 +239,10 @@ struct World {
     std::map<uint32_t, DevicePlan> plans;
     std::vector<hipEvent_t> eventPool;
     hipEvent_t doneEvent = nullptr;
+    // One launch at a time per world; while it runs, launchLock is the lock its caller holds on `mu`, so that
+    // a step that has to wait for the GPU can release it for the duration of the wait.
+    bool launchBusy = false;
+    std::unique_lock<std::mutex>* launchLock = nullptr;
     // AlltoAllV tables
     uint8_t* a2aDev = nullptr;
     uint64_t* a2aHost[kStagingSlots] = {};
@@ -285,10 +290,28 @@ struct World {
     }
 };
 
+// Worlds by id, and the live communicator handles with the world each belongs to.  A handle that is not in
+// g_liveComms (never issued, destroyed, or of a world that is gone) is rejected without being dereferenced; a
+// call holds its world through the shared pointer until it returns, whatever other threads destroy meanwhile.
 std::mutex g_registryMu;
-std::map<uint64_t, std::unique_ptr<World>> g_worlds;
+std::map<uint64_t, std::shared_ptr<World>> g_worlds;
+std::unordered_map<const void*, std::shared_ptr<World>> g_liveComms;
 uint64_t g_nextWorldId = 1;
 thread_local int t_groupDepth = 0;
+
+// What a thread queued since its outermost HcclGroupStart: HcclGroupEnd waits for these and reports their results.
+struct GroupItem {
+    std::shared_ptr<World> world;
+    std::shared_ptr<PendingOp> op;
+    std::shared_ptr<P2pOp> p2p;
+};
+thread_local std::vector<GroupItem> t_groupItems;
+
+// A validated handle; keeps the world alive for the duration of the call.
+struct CommRef {
+    Comm* c = nullptr;
+    std::shared_ptr<World> hold;
+};
 
 uint32_t EnvU32(const char* name, uint32_t dflt)
 {
@@ -418,13 +441,19 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     return w;
 }
 
-Comm* AsComm(HcclComm h)
+CommRef AsComm(HcclComm h)
 {
-    Comm* c = static_cast<Comm*>(h);
-    if (c == nullptr || c->magic != kMagic || c->destroyed || c->world == nullptr) {
-        return nullptr;
+    CommRef ref;
+    if (h == nullptr) {
+        return ref;
     }
-    return c;
+    std::lock_guard<std::mutex> g(g_registryMu);
+    auto it = g_liveComms.find(h);
+    if (it != g_liveComms.end()) {
+        ref.hold = it->second;
+        ref.c = static_cast<Comm*>(h);
+    }
+    return ref;
 }
 
 // Reference src/common/param_check.cc:153-162.
@@ -1010,8 +1039,18 @@ HcclResult RunSegmentCopy(World* w, const std::vector<CopySeg>& segs, hipStream_
         }
         slot = w->a2aNext;
         w->a2aNext = (w->a2aNext + 1) % kStagingSlots;
-        if (w->a2aSlotUsed[slot]) {
-            HIP_OK(hipEventSynchronize(w->a2aSlotFree[slot]));   // the call that last used this slot has finished
+        if (w->a2aSlotUsed[slot] && hipEventQuery(w->a2aSlotFree[slot]) != hipSuccess) {
+            // The call that last used this slot is still running: wait for it without the world's lock, so that
+            // other ranks can keep depositing their calls (launches stay one at a time: launchBusy is set).
+            hipEvent_t busy = w->a2aSlotFree[slot];
+            if (w->launchLock != nullptr) {
+                w->launchLock->unlock();
+            }
+            const hipError_t waited = hipEventSynchronize(busy);
+            if (w->launchLock != nullptr) {
+                w->launchLock->lock();
+            }
+            HIP_OK(waited);
         }
         hDesc = w->a2aHost[slot];
         dev = w->a2aDev + slot * A2aSlotBytes(n);
@@ -1414,17 +1453,27 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
     return rc;
 }
 
-// Deposits one rank's arguments; the call that completes the set launches.
-HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count, const void* send,
-                  void* recv, hipStream_t stream, std::vector<uint64_t>&& var, uint32_t root = 0, bool noAlloc = false)
+// Drops the collectives at the head of the queue that every rank has been through.
+void PopFinished(World* w)
 {
-    World* w = c->world;
-    std::unique_lock<std::mutex> lock(w->mu);
-    const uint64_t seq = w->nextSeq[c->rank]++;
+    while (!w->pending.empty() && w->pending.front() && w->pending.front()->done &&
+           w->pending.front()->arrived == w->n) {
+        w->pending.pop_front();
+        w->baseSeq++;
+    }
+}
+
+// The cell of rank `rank`'s next call in the world's sequence of collectives (created by the first rank to get
+// there).  Caller holds w->mu.
+std::shared_ptr<PendingOp> NextCell(World* w, uint32_t rank, OpType type, HcclDataType dtype, HcclReduceOp op,
+                                    uint64_t count, uint32_t root, bool noAlloc, bool* created)
+{
+    const uint64_t seq = w->nextSeq[rank]++;
     while (w->baseSeq + w->pending.size() <= seq) {
         w->pending.push_back(nullptr);
     }
     std::shared_ptr<PendingOp>& cell = w->pending[seq - w->baseSeq];
+    *created = !cell;
     if (!cell) {
         cell = std::make_shared<PendingOp>();
         cell->type = type;
@@ -1435,7 +1484,29 @@ HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uin
         cell->noAlloc = noAlloc;
         cell->ranks.resize(w->n);
     }
-    std::shared_ptr<PendingOp> p = cell;
+    return cell;
+}
+
+// Deposits one rank's arguments; the call that completes the set launches.
+HcclResult Submit(const CommRef& ref, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count, const void* send,
+                  void* recv, hipStream_t stream, std::vector<uint64_t>&& var, uint32_t root = 0, bool noAlloc = false)
+{
+    Comm* c = ref.c;
+    World* w = c->world;
+    std::unique_lock<std::mutex> lock(w->mu);
+    if (w->destroyed != 0) {
+        Log(1, "%s on rank %u: a communicator of this world has been destroyed", OpName(type), c->rank);
+        return HCCL_E_UNAVAIL;
+    }
+    bool created = false;
+    std::shared_ptr<PendingOp> p = NextCell(w, c->rank, type, dtype, op, count, root, noAlloc, &created);
+    p->arrived++;
+    if (p->done) {
+        // Settled before this rank arrived: a peer's call failed its checks, or timed out.
+        const HcclResult rc = p->result;
+        PopFinished(w);
+        return rc;
+    }
     if (p->type != type || p->dtype != dtype || p->op != op || p->count != count || p->root != root ||
         p->noAlloc != noAlloc) {
         Log(1, "%s on rank %u does not match the call of the other ranks (%s, count %llu, type %d, root %u)",
@@ -1448,11 +1519,11 @@ HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uin
     ra.stream = stream;
     ra.var = std::move(var);
     ra.arrived = true;
-    p->arrived++;
 
     if (p->arrived < w->n) {
         if (t_groupDepth > 0) {
-            return p->result;   // queued; the group's last call launches
+            t_groupItems.push_back({ref.hold, p, nullptr});
+            return p->result;   // queued; the call that completes the set launches, HcclGroupEnd waits for it
         }
         bool ok = w->cv.wait_for(lock, std::chrono::seconds(w->execTimeout), [&] { return p->done; });
         if (!ok) {
@@ -1463,18 +1534,54 @@ HcclResult Submit(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uin
         return p->result;
     }
 
-    // Last arrival: launch.
-    if (p->result == HCCL_SUCCESS) {
+    // Last arrival: launch, one launch at a time per world.
+    w->cv.wait(lock, [&] { return !w->launchBusy; });
+    if (p->result == HCCL_SUCCESS && w->destroyed == 0) {
+        w->launchBusy = true;
+        w->launchLock = &lock;
         p->result = Launch(w, *p, c->rank);
+        w->launchLock = nullptr;
+        w->launchBusy = false;
+    } else if (p->result == HCCL_SUCCESS) {
+        p->result = HCCL_E_UNAVAIL;
     }
     p->done = true;
-    while (!w->pending.empty() && w->pending.front() && w->pending.front()->done) {
-        w->pending.pop_front();
-        w->baseSeq++;
-    }
+    PopFinished(w);
     w->cv.notify_all();
     return p->result;
 }
+
+// A call that fails its argument checks after its communicator has been identified still takes its place in
+// the rank's sequence of collectives: the peers of that collective wake at once with the same verdict (nothing
+// is launched), and the calls that follow pair up as they would have.
+HcclResult Reject(const CommRef& ref, OpType type, HcclResult rc)
+{
+    if (ref.c == nullptr) {
+        return rc;
+    }
+    World* w = ref.c->world;
+    std::unique_lock<std::mutex> lock(w->mu);
+    if (w->destroyed != 0) {
+        return rc;
+    }
+    bool created = false;
+    std::shared_ptr<PendingOp> p = NextCell(w, ref.c->rank, type, HCCL_DATA_TYPE_RESERVED, HCCL_REDUCE_RESERVED, 0, 0,
+                                            false, &created);
+    p->arrived++;
+    if (!p->done) {
+        if (p->result == HCCL_SUCCESS) {
+            p->result = rc;
+        }
+        p->done = true;
+        Log(1, "%s: the call of rank %u was rejected (%d); the collective is abandoned on every rank", OpName(type),
+            ref.c->rank, static_cast<int>(rc));
+    }
+    PopFinished(w);
+    w->cv.notify_all();
+    return rc;
+}
+
+inline HcclResult RejectIfKnown(const CommRef& ref, OpType type, HcclResult rc) { return Reject(ref, type, rc); }
 
 // Runs `run` on stream `s` after everything queued on `other`, and makes `other` wait for it.
 template <class F>
@@ -1559,10 +1666,18 @@ std::shared_ptr<P2pOp> DepositP2p(World* w, bool isSend, uint32_t src, uint32_t 
 }
 
 // Blocks until every op of `ops` is complete (outside a group); the worst result wins.
-HcclResult AwaitP2p(World* w, std::unique_lock<std::mutex>& lock, const std::vector<std::shared_ptr<P2pOp>>& ops,
-                    const char* what, uint32_t rank)
+HcclResult AwaitP2p(const CommRef& ref, std::unique_lock<std::mutex>& lock,
+                    const std::vector<std::shared_ptr<P2pOp>>& ops, const char* what, uint32_t rank)
 {
+    World* w = ref.c->world;
     HcclResult rc = HCCL_SUCCESS;
+    if (t_groupDepth > 0) {
+        for (const auto& op : ops) {
+            if (!op->done) {
+                t_groupItems.push_back({ref.hold, nullptr, op});   // HcclGroupEnd waits for the peer
+            }
+        }
+    }
     if (t_groupDepth == 0) {
         bool ok = w->cv.wait_for(lock, std::chrono::seconds(w->execTimeout), [&] {
             for (const auto& op : ops) {
@@ -1614,17 +1729,36 @@ using namespace hccl_amd;
         }                             \
     } while (0)
 
+// The same two checks inside a collective's entry point, where `ref` is the looked-up communicator: a call that
+// fails them keeps its place in the rank's sequence of collectives when the communicator is a live one (see
+// Reject); the code returned is the same either way.
+#define CHK_RET_Q(type, expr)                       \
+    do {                                            \
+        HcclResult rc_ = (expr);                    \
+        if (rc_ != HCCL_SUCCESS) {                  \
+            return RejectIfKnown(ref, type, rc_);   \
+        }                                           \
+    } while (0)
+
+#define CHK_PTR_Q(type, p, what)                          \
+    do {                                                  \
+        if ((p) == nullptr) {                             \
+            Log(1, "%s: %s is nullptr", __func__, what);  \
+            return RejectIfKnown(ref, type, HCCL_E_PTR);  \
+        }                                                 \
+    } while (0)
+
 namespace {
 
 // Common tail of every entry point: the environment verdict, then the rendezvous.
-HcclResult SubmitWithReady(Comm* c, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count,
+HcclResult SubmitWithReady(const CommRef& ref, OpType type, HcclDataType dtype, HcclReduceOp op, uint64_t count,
                            const void* send, void* recv, aclrtStream stream, std::vector<uint64_t>&& var,
                            uint32_t root = 0, bool noAlloc = false)
 {
-    if (c->world->envInvalid) {
+    if (ref.c->world->envInvalid) {
         return HCCL_E_PARA;   // the reference's environment parsing fails every entry point the same way
     }
-    return Submit(c, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var), root,
+    return Submit(ref, type, dtype, op, count, send, recv, static_cast<hipStream_t>(stream), std::move(var), root,
                   noAlloc);
 }
 
@@ -1634,11 +1768,12 @@ HcclResult AlltoAllVEntry(const char* name, const void* sendBuf, const void* sen
                           const void* recvBuf, const void* recvCounts, const void* rdispls, HcclDataType recvType,
                           HcclComm comm, aclrtStream stream, bool noAlloc)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
 #define CHK_ENTRY_PTR(p, what)                                \
     do {                                                      \
         if ((p) == nullptr) {                                 \
             Log(1, "%s: %s is nullptr", name, what);  \
-            return HCCL_E_PTR;                                \
+            return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PTR); \
         }                                                     \
     } while (0)
     CHK_ENTRY_PTR(comm, "comm");
@@ -1649,12 +1784,12 @@ HcclResult AlltoAllVEntry(const char* name, const void* sendBuf, const void* sen
     CHK_ENTRY_PTR(stream, "stream");
     if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
         Log(1, "%s: sendBuf and recvBuf cannot be the same", name);
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
-    Comm* c = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "%s: comm is not a live communicator", name);
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
     const uint32_t n = c->world->n;
     const uint64_t* sc = static_cast<const uint64_t*>(sendCounts);
@@ -1667,22 +1802,20 @@ HcclResult AlltoAllVEntry(const char* name, const void* sendBuf, const void* sen
         maxCount = sc[i] > maxCount ? sc[i] : maxCount;
         maxCount = rc[i] > maxCount ? rc[i] : maxCount;
     }
-    if (!sendZero) {
-        CHK_ENTRY_PTR(sendBuf, "sendBuf");
-    }
-    if (!recvZero) {
-        CHK_ENTRY_PTR(recvBuf, "recvBuf");
+    if ((!sendZero && sendBuf == nullptr) || (!recvZero && recvBuf == nullptr)) {
+        Log(1, "%s: %s is nullptr", name, (!sendZero && sendBuf == nullptr) ? "sendBuf" : "recvBuf");
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PTR);
     }
 #undef CHK_ENTRY_PTR
-    CHK_RET(CheckUserRank(c));
-    CHK_RET(CheckCount(maxCount));
-    CHK_RET(CheckDataType(recvType, false));
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckUserRank(c));
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckCount(maxCount));
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckDataType(recvType, false));
     std::vector<uint64_t> var(4 * n);
     memcpy(var.data(), sc, n * sizeof(uint64_t));
     memcpy(var.data() + n, rc, n * sizeof(uint64_t));
     memcpy(var.data() + 2 * n, sdispls, n * sizeof(uint64_t));
     memcpy(var.data() + 3 * n, rdispls, n * sizeof(uint64_t));
-    return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
+    return SubmitWithReady(ref, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
                            const_cast<void*>(recvBuf), stream, std::move(var), 0, noAlloc);
 }
 
@@ -1693,91 +1826,95 @@ extern "C" {
 HcclResult HcclAllReduce(void* sendBuf, void* recvBuf, uint64_t count, HcclDataType dataType, HcclReduceOp op,
                          HcclComm comm, aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Order of checks: reference src/ops/all_reduce/all_reduce.cc:41, 111-161.
     if (count == 0) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(stream, "stream");
-    CHK_PTR(comm, "comm");
-    CHK_PTR(sendBuf, "sendBuf");
-    CHK_PTR(recvBuf, "recvBuf");
-    Comm* c = AsComm(comm);
+    CHK_PTR_Q(OpType::ALL_REDUCE, stream, "stream");
+    CHK_PTR_Q(OpType::ALL_REDUCE, comm, "comm");
+    CHK_PTR_Q(OpType::ALL_REDUCE, sendBuf, "sendBuf");
+    CHK_PTR_Q(OpType::ALL_REDUCE, recvBuf, "recvBuf");
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclAllReduce: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_REDUCE, HCCL_E_PARA);
     }
-    CHK_RET(CheckUserRank(c));
-    CHK_RET(CheckCount(count));
-    CHK_RET(CheckDataType(dataType, true));
-    CHK_RET(CheckReduceOp(dataType, op));
-    return SubmitWithReady(c, OpType::ALL_REDUCE, dataType, op, count, sendBuf, recvBuf, stream, {});
+    CHK_RET_Q(OpType::ALL_REDUCE, CheckUserRank(c));
+    CHK_RET_Q(OpType::ALL_REDUCE, CheckCount(count));
+    CHK_RET_Q(OpType::ALL_REDUCE, CheckDataType(dataType, true));
+    CHK_RET_Q(OpType::ALL_REDUCE, CheckReduceOp(dataType, op));
+    return SubmitWithReady(ref, OpType::ALL_REDUCE, dataType, op, count, sendBuf, recvBuf, stream, {});
 }
 
 HcclResult HcclReduceScatter(void* sendBuf, void* recvBuf, uint64_t recvCount, HcclDataType dataType,
                              HcclReduceOp op, HcclComm comm, aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/reduce_scatter/reduce_scatter.cc:48-62.
     if (recvCount == 0) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(stream, "stream");
-    CHK_PTR(comm, "comm");
-    CHK_PTR(sendBuf, "sendBuf");
-    CHK_PTR(recvBuf, "recvBuf");
-    Comm* c = AsComm(comm);
+    CHK_PTR_Q(OpType::REDUCE_SCATTER, stream, "stream");
+    CHK_PTR_Q(OpType::REDUCE_SCATTER, comm, "comm");
+    CHK_PTR_Q(OpType::REDUCE_SCATTER, sendBuf, "sendBuf");
+    CHK_PTR_Q(OpType::REDUCE_SCATTER, recvBuf, "recvBuf");
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclReduceScatter: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::REDUCE_SCATTER, HCCL_E_PARA);
     }
-    CHK_RET(CheckUserRank(c));
-    CHK_RET(CheckCount(recvCount));
-    CHK_RET(CheckDataType(dataType, true));
-    CHK_RET(CheckReduceOp(dataType, op));
-    return SubmitWithReady(c, OpType::REDUCE_SCATTER, dataType, op, recvCount, sendBuf, recvBuf, stream, {});
+    CHK_RET_Q(OpType::REDUCE_SCATTER, CheckUserRank(c));
+    CHK_RET_Q(OpType::REDUCE_SCATTER, CheckCount(recvCount));
+    CHK_RET_Q(OpType::REDUCE_SCATTER, CheckDataType(dataType, true));
+    CHK_RET_Q(OpType::REDUCE_SCATTER, CheckReduceOp(dataType, op));
+    return SubmitWithReady(ref, OpType::REDUCE_SCATTER, dataType, op, recvCount, sendBuf, recvBuf, stream, {});
 }
 
 HcclResult HcclAllGather(void* sendBuf, void* recvBuf, uint64_t sendCount, HcclDataType dataType, HcclComm comm,
                          aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/all_gather/all_gather.cc:37, 118-149.
     if (sendCount == 0) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(stream, "stream");
-    CHK_PTR(comm, "comm");
-    CHK_PTR(sendBuf, "sendBuf");
-    CHK_PTR(recvBuf, "recvBuf");
-    Comm* c = AsComm(comm);
+    CHK_PTR_Q(OpType::ALL_GATHER, stream, "stream");
+    CHK_PTR_Q(OpType::ALL_GATHER, comm, "comm");
+    CHK_PTR_Q(OpType::ALL_GATHER, sendBuf, "sendBuf");
+    CHK_PTR_Q(OpType::ALL_GATHER, recvBuf, "recvBuf");
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclAllGather: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_GATHER, HCCL_E_PARA);
     }
-    CHK_RET(CheckCount(sendCount));
-    CHK_RET(CheckDataType(dataType, false));
-    CHK_RET(CheckUserRank(c));
-    return SubmitWithReady(c, OpType::ALL_GATHER, dataType, HCCL_REDUCE_RESERVED, sendCount, sendBuf, recvBuf, stream,
+    CHK_RET_Q(OpType::ALL_GATHER, CheckCount(sendCount));
+    CHK_RET_Q(OpType::ALL_GATHER, CheckDataType(dataType, false));
+    CHK_RET_Q(OpType::ALL_GATHER, CheckUserRank(c));
+    return SubmitWithReady(ref, OpType::ALL_GATHER, dataType, HCCL_REDUCE_RESERVED, sendCount, sendBuf, recvBuf, stream,
                            {});
 }
 
 HcclResult HcclAllGatherV(void* sendBuf, uint64_t sendCount, void* recvBuf, const void* recvCounts,
                           const void* recvDispls, HcclDataType dataType, HcclComm comm, aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/all_gather_v/all_gather_v.cc:41-55, 137-282.
-    CHK_PTR(comm, "comm");
-    CHK_PTR(recvCounts, "recvCounts");
-    CHK_PTR(recvDispls, "recvDispls");
-    CHK_PTR(stream, "stream");
+    CHK_PTR_Q(OpType::ALL_GATHER_V, comm, "comm");
+    CHK_PTR_Q(OpType::ALL_GATHER_V, recvCounts, "recvCounts");
+    CHK_PTR_Q(OpType::ALL_GATHER_V, recvDispls, "recvDispls");
+    CHK_PTR_Q(OpType::ALL_GATHER_V, stream, "stream");
     if (sendCount > 0) {
-        CHK_PTR(sendBuf, "sendBuf");
+        CHK_PTR_Q(OpType::ALL_GATHER_V, sendBuf, "sendBuf");
     }
     if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
         Log(1, "HcclAllGatherV: sendBuf and recvBuf cannot be the same");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_GATHER_V, HCCL_E_PARA);
     }
-    Comm* c = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclAllGatherV: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_GATHER_V, HCCL_E_PARA);
     }
     const uint32_t n = c->world->n;
     const uint64_t* counts = static_cast<const uint64_t*>(recvCounts);
@@ -1789,10 +1926,10 @@ HcclResult HcclAllGatherV(void* sendBuf, uint64_t sendCount, void* recvBuf, cons
     if (allZero) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(recvBuf, "recvBuf");
-    CHK_RET(CheckUserRank(c));
-    CHK_RET(CheckCount(sendCount));
-    CHK_RET(CheckDataType(dataType, false));
+    CHK_PTR_Q(OpType::ALL_GATHER_V, recvBuf, "recvBuf");
+    CHK_RET_Q(OpType::ALL_GATHER_V, CheckUserRank(c));
+    CHK_RET_Q(OpType::ALL_GATHER_V, CheckCount(sendCount));
+    CHK_RET_Q(OpType::ALL_GATHER_V, CheckDataType(dataType, false));
     // Non-empty intervals may be unordered and leave holes but must not overlap or overflow.
     const uint64_t esz = DataTypeSize(dataType);
     for (uint32_t a = 0; a < n; ++a) {
@@ -1802,12 +1939,12 @@ HcclResult HcclAllGatherV(void* sendBuf, uint64_t sendCount, void* recvBuf, cons
         uint64_t end = displs[a] + counts[a];
         if (end < displs[a] || end > UINT64_MAX / esz) {
             Log(1, "HcclAllGatherV: recvDispls[%u] + recvCounts[%u] overflows", a, a);
-            return HCCL_E_PARA;
+            return RejectIfKnown(ref, OpType::ALL_GATHER_V, HCCL_E_PARA);
         }
         for (uint32_t b = a + 1; b < n; ++b) {
             if (counts[b] != 0 && displs[a] < displs[b] + counts[b] && displs[b] < end) {
                 Log(1, "HcclAllGatherV: recvDispls intervals of ranks %u and %u overlap", a, b);
-                return HCCL_E_PARA;
+                return RejectIfKnown(ref, OpType::ALL_GATHER_V, HCCL_E_PARA);
             }
         }
     }
@@ -1817,7 +1954,7 @@ HcclResult HcclAllGatherV(void* sendBuf, uint64_t sendCount, void* recvBuf, cons
     var[2 * n] = sendCount;
     // Every rank passes the same count as "count" of the pending op: use 0 so that ranks with different
     // sendCount still meet; per-rank counts are validated at launch.
-    return SubmitWithReady(c, OpType::ALL_GATHER_V, dataType, HCCL_REDUCE_RESERVED, 0, sendBuf, recvBuf, stream,
+    return SubmitWithReady(ref, OpType::ALL_GATHER_V, dataType, HCCL_REDUCE_RESERVED, 0, sendBuf, recvBuf, stream,
                            std::move(var));
 }
 
@@ -1842,44 +1979,45 @@ HcclResult HcclAmdAlltoAllVNoAlloc(const void* sendBuf, const void* sendCounts, 
 HcclResult HcclAlltoAll(const void* sendBuf, uint64_t sendCount, HcclDataType sendType, const void* recvBuf,
                         uint64_t recvCount, HcclDataType recvType, HcclComm comm, aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/all_to_all_v/all_to_all_v.cc:39-82, 475-515.
     if (sendCount == 0 && recvCount == 0) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(comm, "comm");
-    CHK_PTR(sendBuf, "sendBuf");
-    CHK_PTR(recvBuf, "recvBuf");
+    CHK_PTR_Q(OpType::ALL_TO_ALL_V, comm, "comm");
+    CHK_PTR_Q(OpType::ALL_TO_ALL_V, sendBuf, "sendBuf");
+    CHK_PTR_Q(OpType::ALL_TO_ALL_V, recvBuf, "recvBuf");
     if (sendCount != recvCount) {
         Log(1, "HcclAlltoAll: sendCount %llu and recvCount %llu are not equal", (unsigned long long)sendCount,
             (unsigned long long)recvCount);
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
     if (sendType != recvType) {
         Log(1, "HcclAlltoAll: sendType %d and recvType %d are not equal", static_cast<int>(sendType),
             static_cast<int>(recvType));
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
-    CHK_PTR(stream, "stream");
+    CHK_PTR_Q(OpType::ALL_TO_ALL_V, stream, "stream");
     if (sendBuf == recvBuf) {
         Log(1, "HcclAlltoAll: sendBuf and recvBuf cannot be the same");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
     if (DataTypeSize(sendType) == 0) {
         Log(1, "HcclAlltoAll: sendType %d is not supported", static_cast<int>(sendType));
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
     if (sendCount > UINT64_MAX / DataTypeSize(sendType)) {
         Log(1, "HcclAlltoAll: send size overflows");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
-    Comm* c = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclAlltoAll: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
-    CHK_RET(CheckUserRank(c));
-    CHK_RET(CheckCount(recvCount));
-    CHK_RET(CheckDataType(recvType, false));
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckUserRank(c));
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckCount(recvCount));
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckDataType(recvType, false));
     // Four arrays in AlltoAllV form: counts = recvCount, displacements = i * recvCount (:411-421).
     const uint32_t n = c->world->n;
     std::vector<uint64_t> var(4 * n);
@@ -1889,29 +2027,30 @@ HcclResult HcclAlltoAll(const void* sendBuf, uint64_t sendCount, HcclDataType se
         var[2 * n + i] = static_cast<uint64_t>(i) * recvCount;
         var[3 * n + i] = static_cast<uint64_t>(i) * recvCount;
     }
-    return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
+    return SubmitWithReady(ref, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
                            const_cast<void*>(recvBuf), stream, std::move(var));
 }
 
 HcclResult HcclAlltoAllVC(const void* sendBuf, const void* sendCountMatrix, HcclDataType sendType, const void* recvBuf,
                           HcclDataType recvType, HcclComm comm, aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/all_to_all_v/all_to_all_v.cc:153-209, 423-458, 555-598.  Like the reference, only
     // recvType is consulted for the element size.
     (void)sendType;
-    CHK_PTR(comm, "comm");
-    CHK_PTR(sendCountMatrix, "sendCountMatrix");
-    CHK_PTR(stream, "stream");
+    CHK_PTR_Q(OpType::ALL_TO_ALL_V, comm, "comm");
+    CHK_PTR_Q(OpType::ALL_TO_ALL_V, sendCountMatrix, "sendCountMatrix");
+    CHK_PTR_Q(OpType::ALL_TO_ALL_V, stream, "stream");
     if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
         Log(1, "HcclAlltoAllVC: sendBuf and recvBuf cannot be the same");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
-    Comm* c = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclAlltoAllVC: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::ALL_TO_ALL_V, HCCL_E_PARA);
     }
-    CHK_RET(CheckUserRank(c));
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckUserRank(c));
     const uint32_t n = c->world->n;
     const uint32_t me = c->rank;
     const uint64_t* m = static_cast<const uint64_t*>(sendCountMatrix);
@@ -1919,7 +2058,7 @@ HcclResult HcclAlltoAllVC(const void* sendBuf, const void* sendCountMatrix, Hccl
     for (uint64_t i = 0; i < static_cast<uint64_t>(n) * n; ++i) {
         maxCount = m[i] > maxCount ? m[i] : maxCount;
     }
-    CHK_RET(CheckCount(maxCount));
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckCount(maxCount));
     // sendCounts = row `me`, recvCounts = column `me`, displacements = exclusive prefix sums (:444-455).
     std::vector<uint64_t> var(4 * n);
     uint64_t sOff = 0, rOff = 0;
@@ -1935,13 +2074,13 @@ HcclResult HcclAlltoAllVC(const void* sendBuf, const void* sendCountMatrix, Hccl
         recvZero = recvZero && var[n + i] == 0;
     }
     if (!sendZero) {
-        CHK_PTR(sendBuf, "sendBuf");
+        CHK_PTR_Q(OpType::ALL_TO_ALL_V, sendBuf, "sendBuf");
     }
     if (!recvZero) {
-        CHK_PTR(recvBuf, "recvBuf");
+        CHK_PTR_Q(OpType::ALL_TO_ALL_V, recvBuf, "recvBuf");
     }
-    CHK_RET(CheckDataType(recvType, false));
-    return SubmitWithReady(c, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
+    CHK_RET_Q(OpType::ALL_TO_ALL_V, CheckDataType(recvType, false));
+    return SubmitWithReady(ref, OpType::ALL_TO_ALL_V, recvType, HCCL_REDUCE_RESERVED, 0, sendBuf,
                            const_cast<void*>(recvBuf), stream, std::move(var));
 }
 
@@ -1949,18 +2088,19 @@ HcclResult HcclReduceScatterV(void* sendBuf, const void* sendCounts, const void*
                               uint64_t recvCount, HcclDataType dataType, HcclReduceOp op, HcclComm comm,
                               aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/reduce_scatter_v/reduce_scatter_v.cc:48-79, 180-247.
-    CHK_PTR(stream, "stream");
-    CHK_PTR(comm, "comm");
-    CHK_PTR(sendCounts, "sendCounts");
-    CHK_PTR(sendDispls, "sendDispls");
+    CHK_PTR_Q(OpType::REDUCE_SCATTER_V, stream, "stream");
+    CHK_PTR_Q(OpType::REDUCE_SCATTER_V, comm, "comm");
+    CHK_PTR_Q(OpType::REDUCE_SCATTER_V, sendCounts, "sendCounts");
+    CHK_PTR_Q(OpType::REDUCE_SCATTER_V, sendDispls, "sendDispls");
     if (recvCount > 0) {
-        CHK_PTR(recvBuf, "recvBuf");
+        CHK_PTR_Q(OpType::REDUCE_SCATTER_V, recvBuf, "recvBuf");
     }
-    Comm* c = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclReduceScatterV: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::REDUCE_SCATTER_V, HCCL_E_PARA);
     }
     const uint32_t n = c->world->n;
     const uint64_t* counts = static_cast<const uint64_t*>(sendCounts);
@@ -1972,102 +2112,105 @@ HcclResult HcclReduceScatterV(void* sendBuf, const void* sendCounts, const void*
     if (allZero) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(sendBuf, "sendBuf");
-    CHK_RET(CheckUserRank(c));
-    CHK_RET(CheckCount(recvCount));
+    CHK_PTR_Q(OpType::REDUCE_SCATTER_V, sendBuf, "sendBuf");
+    CHK_RET_Q(OpType::REDUCE_SCATTER_V, CheckUserRank(c));
+    CHK_RET_Q(OpType::REDUCE_SCATTER_V, CheckCount(recvCount));
     // No uint64 / fp64 here, unlike the other reduce ops (:225-247).
     if (dataType == HCCL_DATA_TYPE_UINT64 || dataType == HCCL_DATA_TYPE_FP64) {
         Log(1, "HcclReduceScatterV: data type %d is not supported", static_cast<int>(dataType));
-        return HCCL_E_NOT_SUPPORT;
+        return RejectIfKnown(ref, OpType::REDUCE_SCATTER_V, HCCL_E_NOT_SUPPORT);
     }
-    CHK_RET(CheckDataType(dataType, true));
-    CHK_RET(CheckReduceOp(dataType, op));
+    CHK_RET_Q(OpType::REDUCE_SCATTER_V, CheckDataType(dataType, true));
+    CHK_RET_Q(OpType::REDUCE_SCATTER_V, CheckReduceOp(dataType, op));
     std::vector<uint64_t> var(2 * n + 1);
     memcpy(var.data(), counts, n * sizeof(uint64_t));
     memcpy(var.data() + n, displs, n * sizeof(uint64_t));
     var[2 * n] = recvCount;
     // recvCount differs between ranks: 0 is the count the ranks meet on, the per-rank values are checked at launch.
-    return SubmitWithReady(c, OpType::REDUCE_SCATTER_V, dataType, op, 0, sendBuf, recvBuf, stream, std::move(var));
+    return SubmitWithReady(ref, OpType::REDUCE_SCATTER_V, dataType, op, 0, sendBuf, recvBuf, stream, std::move(var));
 }
 
 HcclResult HcclReduce(void* sendBuf, void* recvBuf, uint64_t count, HcclDataType dataType, HcclReduceOp op,
                       uint32_t root, HcclComm comm, aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/reduce/reduce.cc:39, 106-153.
     if (count == 0) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(comm, "comm");
-    CHK_PTR(sendBuf, "sendBuf");
-    CHK_PTR(recvBuf, "recvBuf");
-    CHK_PTR(stream, "stream");
-    Comm* c = AsComm(comm);
+    CHK_PTR_Q(OpType::REDUCE, comm, "comm");
+    CHK_PTR_Q(OpType::REDUCE, sendBuf, "sendBuf");
+    CHK_PTR_Q(OpType::REDUCE, recvBuf, "recvBuf");
+    CHK_PTR_Q(OpType::REDUCE, stream, "stream");
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclReduce: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::REDUCE, HCCL_E_PARA);
     }
-    CHK_RET(CheckCount(count));
-    CHK_RET(CheckDataType(dataType, true));
-    CHK_RET(CheckReduceOp(dataType, op));
+    CHK_RET_Q(OpType::REDUCE, CheckCount(count));
+    CHK_RET_Q(OpType::REDUCE, CheckDataType(dataType, true));
+    CHK_RET_Q(OpType::REDUCE, CheckReduceOp(dataType, op));
     if (root >= c->world->n) {
         Log(1, "HcclReduce: root %u is out of range [0, %u)", root, c->world->n);
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::REDUCE, HCCL_E_PARA);
     }
-    CHK_RET(CheckUserRank(c));
-    return SubmitWithReady(c, OpType::REDUCE, dataType, op, count, sendBuf, recvBuf, stream, {}, root);
+    CHK_RET_Q(OpType::REDUCE, CheckUserRank(c));
+    return SubmitWithReady(ref, OpType::REDUCE, dataType, op, count, sendBuf, recvBuf, stream, {}, root);
 }
 
 HcclResult HcclBroadcast(void* buf, uint64_t count, HcclDataType dataType, uint32_t root, HcclComm comm,
                          aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/broadcast/broadcast.cc:38, 99-142.
     if (count == 0) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(comm, "comm");
-    CHK_PTR(buf, "buf");
-    CHK_PTR(stream, "stream");
-    Comm* c = AsComm(comm);
+    CHK_PTR_Q(OpType::BROADCAST, comm, "comm");
+    CHK_PTR_Q(OpType::BROADCAST, buf, "buf");
+    CHK_PTR_Q(OpType::BROADCAST, stream, "stream");
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclBroadcast: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::BROADCAST, HCCL_E_PARA);
     }
-    CHK_RET(CheckUserRank(c));
+    CHK_RET_Q(OpType::BROADCAST, CheckUserRank(c));
     if (root >= c->world->n) {
         Log(1, "HcclBroadcast: root %u is out of range [0, %u)", root, c->world->n);
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::BROADCAST, HCCL_E_PARA);
     }
-    CHK_RET(CheckCount(count));
-    CHK_RET(CheckDataType(dataType, false));
-    return SubmitWithReady(c, OpType::BROADCAST, dataType, HCCL_REDUCE_RESERVED, count, buf, buf, stream, {}, root);
+    CHK_RET_Q(OpType::BROADCAST, CheckCount(count));
+    CHK_RET_Q(OpType::BROADCAST, CheckDataType(dataType, false));
+    return SubmitWithReady(ref, OpType::BROADCAST, dataType, HCCL_REDUCE_RESERVED, count, buf, buf, stream, {}, root);
 }
 
 HcclResult HcclScatter(void* sendBuf, void* recvBuf, uint64_t recvCount, HcclDataType dataType, uint32_t root,
                        HcclComm comm, aclrtStream stream)
 {
+    CommRef ref = AsComm(comm);   // looked up first, so that a call that fails any check below keeps its place
     // Reference src/ops/scatter/scatter.cc:59-73, 115-128.  The reference leaves a null stream to the layers
     // below the entry point; here it is rejected after the reference's own checks.
     if (recvCount == 0) {
         return HCCL_SUCCESS;
     }
-    CHK_PTR(comm, "comm");
-    CHK_PTR(recvBuf, "recvBuf");
-    Comm* c = AsComm(comm);
+    CHK_PTR_Q(OpType::SCATTER, comm, "comm");
+    CHK_PTR_Q(OpType::SCATTER, recvBuf, "recvBuf");
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclScatter: comm is not a live communicator");
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::SCATTER, HCCL_E_PARA);
     }
     if (c->rank == root) {
-        CHK_PTR(sendBuf, "sendBuf");   // only the root's sendBuf is read
+        CHK_PTR_Q(OpType::SCATTER, sendBuf, "sendBuf");   // only the root's sendBuf is read
     }
     if (root >= c->world->n) {
         Log(1, "HcclScatter: root %u is out of range [0, %u)", root, c->world->n);
-        return HCCL_E_PARA;
+        return RejectIfKnown(ref, OpType::SCATTER, HCCL_E_PARA);
     }
-    CHK_RET(CheckCount(recvCount));
-    CHK_RET(CheckDataType(dataType, false));
-    CHK_PTR(stream, "stream");
-    return SubmitWithReady(c, OpType::SCATTER, dataType, HCCL_REDUCE_RESERVED, recvCount, sendBuf, recvBuf, stream, {},
+    CHK_RET_Q(OpType::SCATTER, CheckCount(recvCount));
+    CHK_RET_Q(OpType::SCATTER, CheckDataType(dataType, false));
+    CHK_PTR_Q(OpType::SCATTER, stream, "stream");
+    return SubmitWithReady(ref, OpType::SCATTER, dataType, HCCL_REDUCE_RESERVED, recvCount, sendBuf, recvBuf, stream, {},
                            root);
 }
 
@@ -2098,7 +2241,11 @@ HcclResult HcclCommInitAll(uint32_t ndev, int32_t* devices, HcclComm* comms)
         comms[r] = w->comms[r].get();
     }
     w->joined = ndev;
-    g_worlds[w->id] = std::move(w);
+    std::shared_ptr<World> shared(std::move(w));
+    for (uint32_t r = 0; r < ndev; ++r) {
+        g_liveComms[comms[r]] = shared;
+    }
+    g_worlds[shared->id] = shared;
     return HCCL_SUCCESS;
 }
 
@@ -2129,7 +2276,7 @@ HcclResult HcclCommInitRootInfo(uint32_t nRanks, const HcclRootInfo* rootInfo, u
     if (it == g_worlds.end()) {
         auto w = NewWorld(nRanks);
         w->id = id;
-        it = g_worlds.emplace(id, std::move(w)).first;
+        it = g_worlds.emplace(id, std::shared_ptr<World>(std::move(w))).first;
     }
     World* w = it->second.get();
     if (w->n != nRanks || w->comms[rank] != nullptr) {
@@ -2141,28 +2288,54 @@ HcclResult HcclCommInitRootInfo(uint32_t nRanks, const HcclRootInfo* rootInfo, u
     w->comms[rank]->rank = rank;
     w->joined++;
     *comm = w->comms[rank].get();
+    g_liveComms[*comm] = it->second;
     return HCCL_SUCCESS;
 }
 
 HcclResult HcclCommDestroy(HcclComm comm)
 {
     CHK_PTR(comm, "comm");
-    Comm* c = AsComm(comm);
-    if (c == nullptr) {
-        return HCCL_E_PARA;
+    std::shared_ptr<World> w;
+    {
+        std::lock_guard<std::mutex> g(g_registryMu);
+        auto it = g_liveComms.find(comm);
+        if (it == g_liveComms.end()) {
+            Log(1, "HcclCommDestroy: comm is not a live communicator");
+            return HCCL_E_PARA;   // never issued, or destroyed before: the handle is not dereferenced
+        }
+        w = it->second;
+        g_liveComms.erase(it);
     }
-    std::lock_guard<std::mutex> g(g_registryMu);
-    World* w = c->world;
+    Comm* c = static_cast<Comm*>(comm);
     bool last;
     {
         std::lock_guard<std::mutex> wl(w->mu);
         c->destroyed = true;
         w->destroyed++;
         last = w->destroyed == w->n;
+        // A rank that leaves will not join what its peers are still waiting for: those calls end now, with an
+        // error, and nothing more is launched in this world.
+        for (std::shared_ptr<PendingOp>& op : w->pending) {
+            if (op && !op->done) {
+                op->result = HCCL_E_UNAVAIL;
+                op->done = true;
+            }
+        }
+        for (auto& kv : w->p2p) {
+            for (std::shared_ptr<P2pOp>& op : kv.second) {
+                if (!op->done) {
+                    op->result = HCCL_E_UNAVAIL;
+                    op->done = true;
+                }
+            }
+            kv.second.clear();
+        }
+        w->cv.notify_all();
     }
     if (last) {
         (void)hipDeviceSynchronize();
-        g_worlds.erase(w->id);
+        std::lock_guard<std::mutex> g(g_registryMu);
+        g_worlds.erase(w->id);   // the world itself goes when the last call that holds it returns
     }
     return HCCL_SUCCESS;
 }
@@ -2171,7 +2344,8 @@ HcclResult HcclGetRankSize(HcclComm comm, uint32_t* rankSize)
 {
     CHK_PTR(comm, "comm");
     CHK_PTR(rankSize, "rankSize");
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         return HCCL_E_PARA;
     }
@@ -2183,7 +2357,8 @@ HcclResult HcclGetRankId(HcclComm comm, uint32_t* rank)
 {
     CHK_PTR(comm, "comm");
     CHK_PTR(rank, "rank");
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         return HCCL_E_PARA;
     }
@@ -2214,13 +2389,14 @@ HcclResult HcclBarrier(HcclComm comm, aclrtStream stream)
 {
     CHK_PTR(stream, "stream");
     CHK_PTR(comm, "comm");
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclBarrier: comm is not a live communicator");
         return HCCL_E_PARA;
     }
     CHK_RET(CheckUserRank(c));
-    return SubmitWithReady(c, OpType::BARRIER, HCCL_DATA_TYPE_RESERVED, HCCL_REDUCE_RESERVED, 0, nullptr, nullptr, stream,
+    return SubmitWithReady(ref, OpType::BARRIER, HCCL_DATA_TYPE_RESERVED, HCCL_REDUCE_RESERVED, 0, nullptr, nullptr, stream,
                            {});
 }
 
@@ -2236,7 +2412,8 @@ HcclResult HcclSend(void* sendBuf, uint64_t count, HcclDataType dataType, uint32
     CHK_PTR(sendBuf, "sendBuf");
     CHK_RET(CheckCount(count));
     CHK_RET(CheckDataType(dataType, false));
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclSend: comm is not a live communicator");
         return HCCL_E_PARA;
@@ -2257,7 +2434,7 @@ HcclResult HcclSend(void* sendBuf, uint64_t count, HcclDataType dataType, uint32
     std::unique_lock<std::mutex> lock(w->mu);
     std::vector<std::shared_ptr<P2pOp>> ops{
         DepositP2p(w, true, c->rank, destRank, sendBuf, count, dataType, static_cast<hipStream_t>(stream))};
-    return AwaitP2p(w, lock, ops, "HcclSend", c->rank);
+    return AwaitP2p(ref, lock, ops, "HcclSend", c->rank);
 }
 
 // Reference src/ops/recv/recv.cc:25-49, 134-161.
@@ -2272,7 +2449,8 @@ HcclResult HcclRecv(void* recvBuf, uint64_t count, HcclDataType dataType, uint32
     CHK_PTR(recvBuf, "recvBuf");
     CHK_RET(CheckCount(count));
     CHK_RET(CheckDataType(dataType, false));
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclRecv: comm is not a live communicator");
         return HCCL_E_PARA;
@@ -2293,7 +2471,7 @@ HcclResult HcclRecv(void* recvBuf, uint64_t count, HcclDataType dataType, uint32
     std::unique_lock<std::mutex> lock(w->mu);
     std::vector<std::shared_ptr<P2pOp>> ops{
         DepositP2p(w, false, srcRank, c->rank, recvBuf, count, dataType, static_cast<hipStream_t>(stream))};
-    return AwaitP2p(w, lock, ops, "HcclRecv", c->rank);
+    return AwaitP2p(ref, lock, ops, "HcclRecv", c->rank);
 }
 
 // Reference src/ops/batch_send_recv/batch_send_recv.cc:22-60, 72-90 and, for which send meets which receive,
@@ -2312,7 +2490,8 @@ HcclResult HcclBatchSendRecv(HcclSendRecvItem* sendRecvInfo, uint32_t itemNum, H
         CHK_RET(CheckCount(sendRecvInfo[i].count));
         CHK_RET(CheckDataType(sendRecvInfo[i].dataType, false));
     }
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         Log(1, "HcclBatchSendRecv: comm is not a live communicator");
         return HCCL_E_PARA;
@@ -2371,7 +2550,7 @@ HcclResult HcclBatchSendRecv(HcclSendRecvItem* sendRecvInfo, uint32_t itemNum, H
         ops.push_back(DepositP2p(w, false, it->remoteRank, c->rank, it->buf, it->count, it->dataType,
                                  static_cast<hipStream_t>(stream)));
     }
-    return AwaitP2p(w, lock, ops, "HcclBatchSendRecv", c->rank);
+    return AwaitP2p(ref, lock, ops, "HcclBatchSendRecv", c->rank);
 }
 
 HcclResult HcclGroupStart(void)
@@ -2386,14 +2565,46 @@ HcclResult HcclGroupEnd(void)
         Log(1, "HcclGroupEnd without HcclGroupStart");
         return HCCL_E_PARA;
     }
-    t_groupDepth--;
-    return HCCL_SUCCESS;
+    if (--t_groupDepth != 0) {
+        return HCCL_SUCCESS;
+    }
+    // The outermost end: every call this thread queued since the group began has been launched (by this thread
+    // or by the thread that completed its set) or has failed when this returns; the worst result is reported.
+    // A set that is never completed ends here after the world's time-out instead of staying pending for ever.
+    HcclResult worst = HCCL_SUCCESS;
+    std::vector<GroupItem> items;
+    items.swap(t_groupItems);
+    for (GroupItem& item : items) {
+        World* w = item.world.get();
+        std::unique_lock<std::mutex> lock(w->mu);
+        HcclResult rc;
+        if (item.op) {
+            const bool ok = w->cv.wait_for(lock, std::chrono::seconds(w->execTimeout), [&] { return item.op->done; });
+            if (!ok) {
+                Log(1, "HcclGroupEnd: %s waited %u s for the other ranks", OpName(item.op->type), w->execTimeout);
+                item.op->result = HCCL_E_TIMEOUT;   // the late ranks find the verdict and launch nothing
+            }
+            rc = ok ? item.op->result : HCCL_E_TIMEOUT;
+        } else {
+            const bool ok = w->cv.wait_for(lock, std::chrono::seconds(w->execTimeout), [&] { return item.p2p->done; });
+            if (!ok) {
+                Log(1, "HcclGroupEnd: a send or receive waited %u s for its peer", w->execTimeout);
+                item.p2p->result = HCCL_E_TIMEOUT;
+            }
+            rc = ok ? item.p2p->result : HCCL_E_TIMEOUT;
+        }
+        if (rc != HCCL_SUCCESS) {
+            worst = rc;
+        }
+    }
+    return worst;
 }
 
 HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo)
 {
     CHK_PTR(comm, "comm");
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr || static_cast<int>(op) < 0 || op >= HCCL_AMD_OP_COUNT || static_cast<int>(algo) < 0 ||
         algo >= HCCL_AMD_ALGO_COUNT) {
         return HCCL_E_PARA;
@@ -2409,7 +2620,8 @@ HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo)
 HcclResult HcclAmdSetCclBufferSize(HcclComm comm, uint64_t bytes)
 {
     CHK_PTR(comm, "comm");
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         return HCCL_E_PARA;
     }
@@ -2422,7 +2634,8 @@ HcclResult HcclAmdGetCclBufferSize(HcclComm comm, uint64_t* bytes)
 {
     CHK_PTR(comm, "comm");
     CHK_PTR(bytes, "bytes");
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr) {
         return HCCL_E_PARA;
     }
@@ -2435,7 +2648,8 @@ HcclResult HcclAmdGetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo* algo)
 {
     CHK_PTR(comm, "comm");
     CHK_PTR(algo, "algo");
-    Comm* c = AsComm(comm);
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
     if (c == nullptr || static_cast<int>(op) < 0 || op >= HCCL_AMD_OP_COUNT) {
         return HCCL_E_PARA;
     }

@@ -184,20 +184,26 @@ def test_rendezvous_mismatch_and_launch_time_checks():
     try:
         a = [to_dev(np.arange(16, dtype=np.float32)) for _ in range(2)]
         b = [dev_zeros(64) for _ in range(2)]
-        with hccl_amd.group():
-            hccl_amd.all_reduce(w.comms[0], a[0], b[0], 16, DT.FP32, OP.SUM, w.stream)
-            with pytest.raises(hccl_amd.HcclError) as e:
-                hccl_amd.all_reduce(w.comms[1], a[1], b[1], 8, DT.FP32, OP.SUM, w.stream)   # different count
-            assert e.value.code == 1
+        hccl_amd.group_start()
+        hccl_amd.all_reduce(w.comms[0], a[0], b[0], 16, DT.FP32, OP.SUM, w.stream)
+        with pytest.raises(hccl_amd.HcclError) as e:
+            hccl_amd.all_reduce(w.comms[1], a[1], b[1], 8, DT.FP32, OP.SUM, w.stream)   # different count
+        assert e.value.code == 1
+        with pytest.raises(hccl_amd.HcclError) as e:
+            hccl_amd.group_end()                      # reports the verdict for the call that was queued
+        assert e.value.code == 1
         # recvCounts of rank 0 disagree with sendCounts of rank 1
         sc = np.array([[1, 2], [3, 4]], dtype=np.uint64)
         rc = np.array([[1, 5], [2, 4]], dtype=np.uint64)
         z = np.zeros((2, 2), dtype=np.uint64)
-        with hccl_amd.group():
-            hccl_amd.all_to_all_v(w.comms[0], a[0], sc[0], z[0], DT.FP32, b[0], rc[0], z[0], DT.FP32, w.stream)
-            with pytest.raises(hccl_amd.HcclError) as e:
-                hccl_amd.all_to_all_v(w.comms[1], a[1], sc[1], z[1], DT.FP32, b[1], rc[1], z[1], DT.FP32, w.stream)
-            assert e.value.code == 1
+        hccl_amd.group_start()
+        hccl_amd.all_to_all_v(w.comms[0], a[0], sc[0], z[0], DT.FP32, b[0], rc[0], z[0], DT.FP32, w.stream)
+        with pytest.raises(hccl_amd.HcclError) as e:
+            hccl_amd.all_to_all_v(w.comms[1], a[1], sc[1], z[1], DT.FP32, b[1], rc[1], z[1], DT.FP32, w.stream)
+        assert e.value.code == 1
+        with pytest.raises(hccl_amd.HcclError) as e:
+            hccl_amd.group_end()
+        assert e.value.code == 1
         # the world is still usable afterwards
         with hccl_amd.group():
             for r in range(2):

@@ -150,7 +150,9 @@ def test_unequal_counts_on_the_two_sides_are_reported_to_both():
                 codes.append(fn(*args))
             except hccl_amd.HcclError as e:
                 codes.append(e.code)
-        hccl_amd.group_end()
+        with pytest.raises(hccl_amd.HcclError) as ended:
+            hccl_amd.group_end()
+        assert ended.value.code == 1                                 # the group's end reports it for the queued side
         assert codes[-1] == 1                                        # HCCL_E_PARA at the call that completes the pair
         w.sync()
         assert np.all(to_host(b, np.uint8) == 0xAB)                  # nothing was copied

@@ -177,7 +177,9 @@ def test_reduce_scatter_v_counts_that_differ_between_ranks_are_rejected(worlds):
                                                    DT.FP32, OP.SUM, w.stream))
         except hccl_amd.HcclError as e:
             codes.append(e.code)
-    hccl_amd.group_end()
+    with pytest.raises(hccl_amd.HcclError) as ended:
+        hccl_amd.group_end()
+    assert ended.value.code == 1                            # the group's end reports it for the queued calls
     assert codes[-1] == 1                                   # HCCL_E_PARA, reported by the call that completes the set
 
 

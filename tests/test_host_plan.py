@@ -495,9 +495,10 @@ def test_calls_that_disagree_are_rejected_without_a_launch():
                                                                                  OP.SUM, 0x1000),
         ]
         for case in cases:
-            with hccl_amd.group():
-                codes = [code_of(case, r) for r in range(3)]
+            hccl_amd.group_start()
+            codes = [code_of(case, r) for r in range(3)]
             assert codes == [0, 0, 1], codes          # the call that completes the set reports HCCL_E_PARA
+            assert code_of(hccl_amd.group_end) == 1   # and the group's end reports it for the queued calls
     finally:
         for c in comms:
             hccl_amd.comm_destroy(c)
@@ -505,3 +506,138 @@ def test_calls_that_disagree_are_rejected_without_a_launch():
 
 def test_group_end_without_start():
     assert code_of(hccl_amd.group_end) == 1
+
+
+# ---- lifetime of handles, groups over several threads, rejected calls --------------------------------------------
+FAKE_STREAM = 0x1000
+
+
+def test_calls_on_a_destroyed_communicator_are_rejected():
+    """A handle that was destroyed (its world possibly freed) is refused, not dereferenced."""
+    comms = hccl_amd.comm_init_all(2)
+    for c in comms:
+        hccl_amd.comm_destroy(c)
+    for c in comms:
+        assert code_of(hccl_amd.comm_destroy, c) == 1                      # double destroy
+        assert code_of(hccl_amd.get_rank_size, c) == 1
+        assert code_of(hccl_amd.get_rank_id, c) == 1
+        assert code_of(hccl_amd.all_reduce, c, 0x2000, 0x3000, 8, DT.FP32, OP.SUM, FAKE_STREAM) == 1
+        assert code_of(hccl_amd.reduce_scatter, c, 0x2000, 0x3000, 8, DT.FP32, OP.SUM, FAKE_STREAM) == 1
+        assert code_of(hccl_amd.all_gather, c, 0x2000, 0x3000, 8, DT.FP32, FAKE_STREAM) == 1
+        assert code_of(hccl_amd.all_to_all_v, c, 0x2000, [1, 1], [0, 1], DT.FP32, 0x3000, [1, 1], [0, 1], DT.FP32,
+                       FAKE_STREAM) == 1
+        assert code_of(hccl_amd.barrier, c, FAKE_STREAM) == 1
+        assert code_of(hccl_amd.send, c, 0x2000, 8, DT.FP32, 1, FAKE_STREAM) == 1
+        assert code_of(hccl_amd.set_algo, c, OpKind.ALL_REDUCE, Algo.MESH) == 1
+    assert code_of(hccl_amd.get_rank_size, ctypes.c_void_p(0x1234560)) == 1    # never issued
+
+
+def test_a_live_rank_learns_that_a_peer_left():
+    """Rank 0 waits in a collective; rank 1 destroys its communicator instead of joining: rank 0 wakes at once
+    with an error, and nothing else runs in that world."""
+    import threading
+    import time
+    comms = hccl_amd.comm_init_all(2)
+    got = {}
+
+    def waiter():
+        t0 = time.perf_counter()
+        got["code"] = code_of(hccl_amd.barrier, comms[0], FAKE_STREAM)
+        got["seconds"] = time.perf_counter() - t0
+
+    th = threading.Thread(target=waiter, daemon=True)
+    th.start()
+    time.sleep(0.3)
+    assert th.is_alive()                                         # parked, waiting for rank 1
+    hccl_amd.comm_destroy(comms[1])
+    th.join(10)
+    assert not th.is_alive()
+    assert got["code"] == 7 and got["seconds"] < 5               # HCCL_E_UNAVAIL, long before the time-out
+    assert code_of(hccl_amd.barrier, comms[0], FAKE_STREAM) == 7
+    hccl_amd.comm_destroy(comms[0])
+    assert code_of(hccl_amd.barrier, comms[0], FAKE_STREAM) == 1
+
+
+def test_two_threads_each_grouping_half_of_the_ranks():
+    """Every HcclGroupEnd returns only when the calls its thread queued are complete, whichever thread completed
+    the set (a barrier over one stream launches nothing, so this runs without a GPU)."""
+    import threading
+    comms = hccl_amd.comm_init_all(4)
+    codes = [None, None]
+    try:
+        def half(k):
+            try:
+                for _ in range(50):
+                    with hccl_amd.group():
+                        for r in (2 * k, 2 * k + 1):
+                            hccl_amd.barrier(comms[r], FAKE_STREAM)
+                codes[k] = 0
+            except hccl_amd.HcclError as e:
+                codes[k] = e.code
+
+        ths = [threading.Thread(target=half, args=(k,), daemon=True) for k in range(2)]
+        for th in ths:
+            th.start()
+        for th in ths:
+            th.join(30)
+            assert not th.is_alive()
+        assert codes == [0, 0]
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)
+
+
+def test_a_group_that_is_never_completed_ends_with_a_time_out(monkeypatch):
+    import time
+    monkeypatch.setenv("HCCL_EXEC_TIMEOUT", "1")
+    comms = hccl_amd.comm_init_all(3)
+    monkeypatch.delenv("HCCL_EXEC_TIMEOUT")
+    try:
+        hccl_amd.group_start()
+        assert code_of(hccl_amd.barrier, comms[0], FAKE_STREAM) == 0      # queued
+        assert code_of(hccl_amd.barrier, comms[1], FAKE_STREAM) == 0      # queued; rank 2 never calls
+        t0 = time.perf_counter()
+        assert code_of(hccl_amd.group_end) == 9                           # HCCL_E_TIMEOUT
+        assert 0.9 < time.perf_counter() - t0 < 8.0
+        # the late rank completes the set and finds the verdict
+        assert code_of(hccl_amd.barrier, comms[2], FAKE_STREAM) == 9
+        # nested groups: only the outermost end waits and reports
+        hccl_amd.group_start()
+        hccl_amd.group_start()
+        for r in range(3):
+            assert code_of(hccl_amd.barrier, comms[r], FAKE_STREAM) == 0
+        assert code_of(hccl_amd.group_end) == 0
+        assert code_of(hccl_amd.group_end) == 0
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)
+
+
+def test_a_rejected_call_keeps_its_place_in_the_sequence():
+    """Rank 1's AllReduce fails its argument checks: rank 0, already waiting in that collective, wakes with the
+    same code instead of waiting for the time-out, and the next collective pairs up as usual."""
+    import threading
+    import time
+    comms = hccl_amd.comm_init_all(2)
+    got = {}
+    try:
+        def waiter():
+            t0 = time.perf_counter()
+            got["code"] = code_of(hccl_amd.all_reduce, comms[0], 0x2000, 0x3000, 8, DT.FP32, OP.SUM, FAKE_STREAM)
+            got["seconds"] = time.perf_counter() - t0
+
+        th = threading.Thread(target=waiter, daemon=True)
+        th.start()
+        time.sleep(0.3)
+        assert code_of(hccl_amd.all_reduce, comms[1], None, 0x3000, 8, DT.FP32, OP.SUM, FAKE_STREAM) == 2   # HCCL_E_PTR
+        th.join(10)
+        assert not th.is_alive() and got["code"] == 2 and got["seconds"] < 5
+        # the other way round: the rejected call comes first, the valid one finds the verdict
+        assert code_of(hccl_amd.all_reduce, comms[0], 0x2000, 0x3000, 8, DT.UINT8, OP.SUM, FAKE_STREAM) == 5   # NOT_SUPPORT
+        assert code_of(hccl_amd.all_reduce, comms[1], 0x2000, 0x3000, 8, DT.FP32, OP.SUM, FAKE_STREAM) == 5
+        with hccl_amd.group():                                   # the numbering is intact
+            for c in comms:
+                hccl_amd.barrier(c, FAKE_STREAM)
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)

@@ -104,7 +104,9 @@ def test_mixing_the_two_entry_points_in_one_collective_is_rejected():
                 codes.append(0)
             except hccl_amd.HcclError as e:
                 codes.append(e.code)
-        hccl_amd.group_end()
+        with pytest.raises(hccl_amd.HcclError) as ended:
+            hccl_amd.group_end()
+        assert ended.value.code == hccl_amd.HcclResult.E_PARA
         assert codes[-1] == hccl_amd.HcclResult.E_PARA
         for r in range(n):
             assert np.all(to_host(recvs[r], np.uint8) == FILL)
