@@ -251,7 +251,8 @@ struct World {
     uint32_t a2aNext = 0;
     // Large rank-order AllReduce over many ranks: the staging slab between its reduce and broadcast kernels.
     uint8_t* slab = nullptr;
-    uint64_t slabBytes = 128ull << 20;   // HCCL_AMD_ALLREDUCE_SLAB_BYTES
+    uint64_t slabHeld = 0;               // bytes allocated
+    uint64_t slabBytes = 256ull << 20;   // HCCL_AMD_ALLREDUCE_SLAB_BYTES
     int slabMode = 2;                    // HCCL_AMD_ALLREDUCE_SLAB: 0 never, 1 always, 2 by rank count and size
     // Allocation-free AlltoAllV: host image of the tables and the device array that receives them.
     std::vector<uint64_t> a2aImage;
@@ -416,7 +417,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->slabMode < 0 || w->slabMode > 2) {
         w->slabMode = 2;
     }
-    w->slabBytes = (static_cast<uint64_t>(EnvU32("HCCL_AMD_ALLREDUCE_SLAB_BYTES", 128u << 20)) + 255) & ~255ull;
+    w->slabBytes = (static_cast<uint64_t>(EnvU32("HCCL_AMD_ALLREDUCE_SLAB_BYTES", 256u << 20)) + 255) & ~255ull;
     w->leadFromSrc = getenv("HCCL_AMD_LEAD_FROM_SRC") == nullptr || atoi(getenv("HCCL_AMD_LEAD_FROM_SRC")) != 0;
     w->reduceBatch = EnvU32("HCCL_AMD_REDUCE_BATCH", 0);
     if (w->reduceBatch != 8 && w->reduceBatch != 16) {
@@ -705,25 +706,42 @@ HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s);
 
 // Rank-order AllReduce in two kernels per slab-sized piece: the fold of all ranks into a slab the library owns
 // (N reads, one write that stays in the last-level cache), then the slab to every recvBuf with the split copy
-// kernel.  Same fold program, same bits as the fused kernel.  Measured on sixteen ranks of 256 MiB: 0.69 / 0.73 /
-// 0.74 / 0.75 of the HBM peak with slabs of 16 / 32 / 64 / 128 MiB against 0.70 fused; on eight ranks 0.74
-// against 0.73, on six 0.73 against 0.75, hence only for twelve ranks and more and messages of at least a slab.
+// kernel.  Same fold program, same bits as the fused kernel.  Measured fractions of the HBM peak, slab form
+// against fused kernel, int32 SUM, pieces of up to 256 MiB (the largest range per destination the split copy
+// form takes; smaller slabs lose to launch gaps: 16 / 32 / 64 / 128 MiB gave 0.70 / 0.73 / 0.74 / 0.74 on sixteen
+// ranks of 256 MiB):
+//   ranks    32 MiB        128 MiB       256 MiB       512 MiB per rank
+//     6    0.67 / 0.70   0.74 / 0.74   0.75 / 0.70   0.73 / 0.73
+//     8    0.66 / 0.67   0.77 / 0.73   0.76 / 0.68   0.76 / 0.70
+//    10    0.67 / 0.63   0.77 / 0.71   0.76 / 0.71   0.75 / 0.69
+//    16    0.70 / 0.65   0.77 / 0.71   0.76 / 0.70
+//    32    0.74 / 0.62   0.75 / 0.67   0.74 / 0.67
+// hence the slab from ten ranks on for messages of 16 MiB and more, and for eight and nine ranks from 64 MiB.
 bool UseSlab(const World* w, uint64_t bytes)
 {
     if (w->slabMode != 2) {
         return w->slabMode == 1;
     }
-    return w->n >= 12 && bytes >= w->slabBytes;
+    return (w->n >= 10 && bytes >= (16ull << 20)) || (w->n >= 8 && bytes >= (64ull << 20));
 }
 
 HcclResult RunAllReduceViaSlab(World* w, PendingOp& p, const DevicePlan& plan, const ReduceArgs& flat, hipStream_t s)
 {
     const uint32_t n = w->n;
     const uint32_t esz = DataTypeSize(p.dtype);
-    if (w->slab == nullptr) {
-        HIP_OK(hipMalloc(reinterpret_cast<void**>(&w->slab), w->slabBytes));
+    // The slab is allocated on first use, as large as this message needs (up to slabBytes), and grows with later
+    // messages: a world that only moves 16 MiB does not hold 256 MiB.
+    const uint64_t want = std::min<uint64_t>(w->slabBytes, (p.count * esz + 255) & ~255ull);
+    if (w->slab == nullptr || w->slabHeld < want) {
+        if (w->slab != nullptr) {
+            HIP_OK(hipDeviceSynchronize());   // an earlier collective may still be using the smaller slab
+            HIP_OK(hipFree(w->slab));
+            w->slab = nullptr;
+        }
+        HIP_OK(hipMalloc(reinterpret_cast<void**>(&w->slab), want));
+        w->slabHeld = want;
     }
-    const uint64_t pieceEl = w->slabBytes / esz;
+    const uint64_t pieceEl = w->slabHeld / esz;
     if (pieceEl == 0) {
         return HCCL_E_INTERNAL;
     }
