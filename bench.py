@@ -153,25 +153,28 @@ class Workloads:
     def c5b(self, algo):
         import numpy as np
         t, h = self.torch, self.h
-        n = 6
+        n, sets = 6, 4   # 4 buffer sets of 0.9 GB in rotation: no step finds its source in the last-level cache
         comms = self.world(n)
         counts = gather_v_counts(np, n, 1 << 20, 32 << 20, SEED + 5000 + 500)
         displs = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.uint64)
         total = int(counts.sum())
-        sends = [t.randn(int(c), generator=self.gen(SEED + 5000 + 600 + r), device="cuda", dtype=t.float16)
-                 for r, c in enumerate(counts)]
-        recvs = [t.empty(total, dtype=t.float16, device="cuda") for _ in range(n)]
+        sends = [[t.randn(int(c), generator=self.gen(SEED + 5000 + 600 + 10 * k + r), device="cuda", dtype=t.float16)
+                  for r, c in enumerate(counts)] for k in range(sets)]
+        recvs = [[t.empty(total, dtype=t.float16, device="cuda") for _ in range(n)] for _ in range(sets)]
         stream = self.stream
+        turn = [0]
 
         def step():
+            k = turn[0]
+            turn[0] = (k + 1) % sets
             with h.group():
                 for r in range(n):
-                    h.all_gather_v(comms[r], sends[r], int(counts[r]), recvs[r], counts, displs,
+                    h.all_gather_v(comms[r], sends[k][r], int(counts[r]), recvs[k][r], counts, displs,
                                    h.HcclDataType.FP16, stream)
 
         hbm = (1 + n) * total * 2
         return step, hbm, total * 2, (n - 1) / n, (sends, recvs), \
-            "AllGatherV fp16 rankSize=6 counts U[1Mi,32Mi]", "u8", n, "mesh"
+            "AllGatherV fp16 rankSize=6 counts U[1Mi,32Mi], 4 buffer sets in rotation", "u8", n, "mesh"
 
     def copycal(self, algo):
         """Plain copy of known size (the rankSize == 1 shortcut): calibrates the HBM byte counters."""
@@ -234,18 +237,21 @@ class Workloads:
 
     def bcast(self, algo):
         t, h = self.torch, self.h
-        n, count, root = 8, 1 << 27, 5
+        n, count, root, sets = 8, 1 << 27, 5, 4   # 4 buffer sets of 1 GiB in rotation
         comms = self.world(n)
-        bufs = [t.randint(0, 255, (count,), generator=self.gen(SEED + 6300 + r), device="cuda", dtype=t.uint8)
-                for r in range(n)]
+        bufs = [[t.randint(0, 255, (count,), generator=self.gen(SEED + 6300 + 10 * k + r), device="cuda", dtype=t.uint8)
+                 for r in range(n)] for k in range(sets)]
         stream = self.stream
+        turn = [0]
 
         def step():
+            k = turn[0]
+            turn[0] = (k + 1) % sets
             with h.group():
                 for r in range(n):
-                    h.broadcast(comms[r], bufs[r], count, h.HcclDataType.UINT8, root, stream)
+                    h.broadcast(comms[r], bufs[k][r], count, h.HcclDataType.UINT8, root, stream)
 
-        return step, n * count, count, 1.0, bufs, "Broadcast rankSize=8 128 MiB", "u8", n, "mesh"
+        return step, n * count, count, 1.0, bufs, "Broadcast rankSize=8 128 MiB, 4 buffer sets in rotation", "u8", n, "mesh"
 
     def scatter(self, algo):
         t, h = self.torch, self.h

@@ -702,7 +702,7 @@ HcclResult LaunchMeshChunk(World* w, const DevicePlan& plan, const PendingOp& p,
     return HCCL_SUCCESS;
 }
 
-HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s);
+HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s, bool sourceIsHot = false);
 
 // Rank-order AllReduce in two kernels per slab-sized piece: the fold of all ranks into a slab the library owns
 // (N reads, one write that stays in the last-level cache), then the slab to every recvBuf with the split copy
@@ -768,7 +768,7 @@ HcclResult RunAllReduceViaSlab(World* w, PendingOp& p, const DevicePlan& plan, c
         for (uint32_t k = 0; k < n; ++k) {
             b.dst[k] = static_cast<uint8_t*>(p.ranks[k].recv) + done * esz;
         }
-        rc = RunBcast(w, b, s);
+        rc = RunBcast(w, b, s, true);   // the slab has just been written
         if (rc != HCCL_SUCCESS) {
             return rc;
         }
@@ -967,9 +967,9 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
     return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
 }
 
-HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
+HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s, bool sourceIsHot)
 {
-    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s, w->copyDstPerGroup));   // 0: the launcher picks
+    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s, w->copyDstPerGroup, sourceIsHot));   // 0: the launcher picks
     return HCCL_SUCCESS;
 }
 

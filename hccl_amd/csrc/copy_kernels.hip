@@ -44,9 +44,8 @@ typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
 // Cache policies.  A tile that one wavefront moves on its own (SHARED == false) is loaded non-temporally and its
 // 16-byte vectors are written through at system scope, the fastest pair for one read and one write stream.  A
 // tile whose destinations are split over several wavefronts of the same XCD (SHARED == true) is loaded with a
-// plain load, so that the XCD's L2 serves the wavefronts that come after the first, and stored non-temporally:
-// with two or three store streams per wavefront that measured 0.84-0.91 of the HBM peak for 1 read + 6..8
-// writes, against 0.71-0.74 for one wavefront storing to every destination under either store policy.
+// plain load, so that the XCD's L2 serves the wavefronts that come after the first, and stored non-temporally
+// (the pair that measured best for that form).
 template <typename V, bool SHARED>
 __device__ __forceinline__ V LoadVec(const void* p)
 {
@@ -454,14 +453,18 @@ hipError_t LaunchTableWrite(uint8_t* table, const uint64_t* image, uint32_t nWor
     return hipSuccess;
 }
 
-hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStream_t stream, uint32_t dstPerGroup)
+hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStream_t stream, uint32_t dstPerGroup,
+                           bool sourceIsHot)
 {
     BcastCopyArgs a = in;
-    // Destinations split over wavefronts, two per wavefront up to sixteen destinations, four beyond (the tile is
-    // read once per group through L2): 0.85-0.92 of the HBM peak against 0.68-0.75 for one wavefront per tile,
-    // as long as the range written in each destination stays within 256 MiB; beyond that the split form
-    // measured slower (0.52-0.73) than the plain one and is not used.  Up to three destinations stay with one
-    // wavefront.
+    // Destinations split over wavefronts (two per wavefront up to sixteen destinations, four beyond; the tile is
+    // read once per group through L2) when the caller knows that the source is still in the last-level cache
+    // because it has just been written, and the range written in each destination stays within 256 MiB: the
+    // copy of a freshly folded slab to sixteen cold 256 MiB destinations runs at 0.80 of the HBM peak this way,
+    // against 0.66-0.72 with one wavefront per tile.  With a source that has to come from HBM the split form is
+    // the slower one (Broadcast of 128 MiB to 7 ranks over rotating buffer sets: 0.65 against 0.73; on buffers
+    // that are reused every step it reaches 0.9 and more, but that is the cache, not the memory), so sources of
+    // unknown state take the plain form.
     if (dstPerGroup == 0) {
         uint64_t lo = ~0ull, hi = 0;
         for (uint32_t j = 0; j < a.nSeg; ++j) {
@@ -471,7 +474,7 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
             }
         }
         const bool compact = hi > lo && hi - lo <= kSplitMaxExtent;
-        dstPerGroup = (a.nDst <= 3 || !compact) ? a.nDst : (a.nDst <= 16 ? 2u : 4u);
+        dstPerGroup = (a.nDst <= 3 || !compact || !sourceIsHot) ? a.nDst : (a.nDst <= 16 ? 2u : 4u);
     }
     if (dstPerGroup > kMaxSplitDst && dstPerGroup < a.nDst) {
         dstPerGroup = kMaxSplitDst;

@@ -213,8 +213,9 @@ inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
     return ((half && op == HCCL_REDUCE_SUM) || dtype == HCCL_DATA_TYPE_INT8) ? 32u : 16u;
 }
 // tileBytes: 1024, 4096 or 16384; 0 lets the launcher choose.  dstPerGroup: destinations per wavefront, 0 lets
-// the launcher choose.
-hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream, uint32_t dstPerGroup = 0);
+// the launcher choose.  sourceIsHot: the source has just been written by the previous kernel on the stream.
+hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream, uint32_t dstPerGroup = 0,
+                           bool sourceIsHot = false);
 hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, uint32_t tileBytes, hipStream_t stream);
 
 }  // namespace hccl_amd
