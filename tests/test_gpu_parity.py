@@ -390,6 +390,46 @@ def test_all_reduce_through_the_staging_slab(monkeypatch, n):
         w.close()
 
 
+def test_slab_all_reduce_can_be_captured_into_a_graph(monkeypatch):
+    """Once the slab exists (one eager call of that size) the two-kernel AllReduce is launches only."""
+    import torch
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB", "1")
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB_BYTES", "65536")
+    n, count = 8, 40_003
+    w = World(n)
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB_BYTES")
+    try:
+        rng = np.random.default_rng(4343)
+        host = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]
+        want = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+        assert oracle.all_reduce(host, want, count, int(DT.FP32), SUM, algo="mesh") == 0
+        ins = [torch.from_numpy(x).cuda() for x in host]
+        outs = [torch.zeros(count, device="cuda") for _ in range(n)]
+
+        def step():
+            with hccl_amd.group():
+                for r in range(n):
+                    hccl_amd.all_reduce(w.comms[r], ins[r], outs[r], count, DT.FP32, OP.SUM, w.stream)
+
+        torch.cuda.synchronize()
+        step()
+        w.sync()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=w.stream):
+            step()
+        for replay in range(3):
+            for t in outs:
+                t.fill_(float(replay))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for r in range(n):
+                assert np.array_equal(outs[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)), (replay, r)
+    finally:
+        w.close()
+
+
 def test_all_reduce_larger_than_a_million_workgroups():
     """2 x 1 GiB of fp16 per rank: 2^26 vector positions, one per lane, 2^20 workgroups per destination."""
     import torch
