@@ -142,6 +142,7 @@ def lib():
     L.HcclAmdSetAlgo.argtypes = [vp, i32, i32]
     L.HcclAmdGetAlgo.argtypes = [vp, i32, ctypes.POINTER(i32)]
     L.HcclAmdGetFoldProgram.argtypes = [i32, i32, u32, u32, vp, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
+    L.HcclAmdGetStuckCounters.argtypes = [vp, ctypes.POINTER(u64), ctypes.POINTER(u64)]
     L.HcclAmdSetCclBufferSize.argtypes = [vp, u64]
     L.HcclAmdGetCclBufferSize.argtypes = [vp, ctypes.POINTER(u64)]
     for name in ("HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAllGatherV", "HcclAlltoAllV",
@@ -150,7 +151,7 @@ def lib():
                  "HcclCommInitAll", "HcclGetRootInfo", "HcclCommInitRootInfo", "HcclCommDestroy", "HcclGetRankSize",
                  "HcclGetRankId", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
                  "HcclAmdGetFoldProgram", "HcclAmdSetCclBufferSize", "HcclAmdGetCclBufferSize",
-                 "HcclAmdAlltoAllVNoAlloc"):
+                 "HcclAmdAlltoAllVNoAlloc", "HcclAmdGetStuckCounters"):
         getattr(L, name).restype = ctypes.c_int
     _lib = L
     return L
@@ -280,6 +281,14 @@ def get_ccl_buffer_size(hccl_comm):
     v = ctypes.c_uint64()
     check(lib().HcclAmdGetCclBufferSize(hccl_comm, ctypes.byref(v)), "HcclAmdGetCclBufferSize")
     return v.value
+
+
+def get_stuck_counters(hccl_comm):
+    """(head, tail): numbers of the last collective of the world whose kernels have started / finished; needs
+    HCCL_AMD_STUCK_COUNTERS=1 when the communicators are created."""
+    head, tail = ctypes.c_uint64(), ctypes.c_uint64()
+    check(lib().HcclAmdGetStuckCounters(hccl_comm, ctypes.byref(head), ctypes.byref(tail)), "HcclAmdGetStuckCounters")
+    return head.value, tail.value
 
 
 def fold_programs(op_kind, algo, rank_size):

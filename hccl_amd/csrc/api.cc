@@ -249,6 +249,14 @@ struct World {
     hipEvent_t a2aSlotFree[kStagingSlots] = {};
     bool a2aSlotUsed[kStagingSlots] = {};
     uint32_t a2aNext = 0;
+    // Hang triage (HCCL_AMD_STUCK_COUNTERS=1): two words in pinned host memory, written from the launch stream in
+    // front of (head) and behind (tail) the kernels of every collective with the collective's number in this
+    // world, like the reference's head / tail counters (aiv_communication_base_v2.h:365-378,
+    // stuck_detect_counter_helper.h).  head != tail while the host can still read them = a kernel of collective
+    // `head` started and has not finished.
+    bool stuckEnabled = false;
+    uint64_t* stuck = nullptr;
+    uint64_t launchSeq = 0;
     // Large rank-order AllReduce over many ranks: the staging slab between its reduce and broadcast kernels.
     uint8_t* slab = nullptr;
     uint64_t slabHeld = 0;               // bytes allocated
@@ -284,6 +292,7 @@ struct World {
         if (doneEvent) (void)hipEventDestroy(doneEvent);
         if (a2aDev) (void)hipFree(a2aDev);
         if (slab) (void)hipFree(slab);
+        if (stuck) (void)hipHostFree(stuck);
         for (int s = 0; s < kStagingSlots; ++s) {
             if (a2aHost[s]) (void)hipHostFree(a2aHost[s]);
             if (a2aSlotFree[s]) (void)hipEventDestroy(a2aSlotFree[s]);
@@ -413,6 +422,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->storePolicy = 2;
     }
     w->reduceVector = EnvU32("HCCL_AMD_REDUCE_VECTOR", 1) != 0;
+    w->stuckEnabled = EnvU32("HCCL_AMD_STUCK_COUNTERS", 0) != 0;
     w->slabMode = getenv("HCCL_AMD_ALLREDUCE_SLAB") != nullptr ? atoi(getenv("HCCL_AMD_ALLREDUCE_SLAB")) : 2;
     if (w->slabMode < 0 || w->slabMode > 2) {
         w->slabMode = 2;
@@ -1434,6 +1444,13 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
         HIP_OK(hipEventRecord(ev, p.ranks[r].stream));
         HIP_OK(hipStreamWaitEvent(s, ev, 0));
     }
+    if (w->stuckEnabled) {
+        if (w->stuck == nullptr) {
+            HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&w->stuck), 2 * sizeof(uint64_t), hipHostMallocDefault));
+            w->stuck[0] = w->stuck[1] = 0;
+        }
+        HIP_OK(LaunchMark(w->stuck, ++w->launchSeq, s));
+    }
     HcclResult rc;
     if (p.type == OpType::BARRIER) {
         rc = HCCL_SUCCESS;   // the ordering of the streams around this point is the whole operation
@@ -1451,6 +1468,9 @@ HcclResult Launch(World* w, PendingOp& p, uint32_t launcher)
             case OpType::SCATTER: rc = RunScatter(w, p, s); break;
             default: rc = RunAlltoAllV(w, p, s); break;
         }
+    }
+    if (w->stuckEnabled && w->stuck != nullptr) {
+        HIP_OK(LaunchMark(w->stuck + 1, w->launchSeq, s));
     }
     // Order every other rank's stream after the fused kernel.
     bool others = false;
@@ -2673,6 +2693,27 @@ HcclResult HcclAmdGetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo* algo)
     }
     std::lock_guard<std::mutex> wl(c->world->mu);
     *algo = c->world->algo[op];
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdGetStuckCounters(HcclComm comm, uint64_t* head, uint64_t* tail)
+{
+    CHK_PTR(comm, "comm");
+    CHK_PTR(head, "head");
+    CHK_PTR(tail, "tail");
+    CommRef ref = AsComm(comm);
+    if (ref.c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    World* w = ref.c->world;
+    std::lock_guard<std::mutex> wl(w->mu);
+    if (!w->stuckEnabled) {
+        return HCCL_E_UNAVAIL;
+    }
+    // The GPU writes these words; read them as they are now.
+    volatile uint64_t* words = w->stuck;
+    *head = words != nullptr ? words[0] : 0;
+    *tail = words != nullptr ? words[1] : 0;
     return HCCL_SUCCESS;
 }
 

@@ -405,6 +405,14 @@ __global__ __launch_bounds__(64) void TableWriteKernel(uint64_t* table, const Ta
     }
 }
 
+// Writes one word: the marks in front of and behind a collective's kernels on its launch stream.
+__global__ __launch_bounds__(64) void MarkKernel(uint64_t* word, uint64_t value)
+{
+    if (threadIdx.x == 0) {
+        *word = value;
+    }
+}
+
 constexpr int kMaxDevices = 64;
 std::mutex g_scratchMu;
 uint8_t* g_scratchPtr[kMaxDevices] = {};
@@ -432,6 +440,12 @@ hipError_t A2aScratchOfCurrentDevice(uint8_t** ptr)
     }
     *ptr = g_scratchPtr[device];
     return hipSuccess;
+}
+
+hipError_t LaunchMark(uint64_t* word, uint64_t value, hipStream_t stream)
+{
+    hipLaunchKernelGGL(MarkKernel, dim3(1), dim3(64), 0, stream, word, value);
+    return hipGetLastError();
 }
 
 hipError_t LaunchTableWrite(uint8_t* table, const uint64_t* image, uint32_t nWords, hipStream_t stream)

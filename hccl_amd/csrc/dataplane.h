@@ -202,6 +202,9 @@ hipError_t A2aScratchOfCurrentDevice(uint8_t** ptr);
 // in their arguments: no copy engine, no staging memory, and the launches can be captured in a graph.
 hipError_t LaunchTableWrite(uint8_t* table, const uint64_t* image, uint32_t nWords, hipStream_t stream);
 
+// Stores `value` to `*word` (device-visible memory) from a one-wavefront kernel on `stream`.
+hipError_t LaunchMark(uint64_t* word, uint64_t value, hipStream_t stream);
+
 // Launchers (defined in the .hip files).  All are asynchronous on `stream`.
 // ldsBytes = (plan depth - 1) * ReduceAccBytes(dtype, op) * args.threads: the accumulator stack of nested levels.
 hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t nBlocks,

@@ -274,6 +274,17 @@ HcclResult HcclAmdSetCclBufferSize(HcclComm comm, uint64_t bytes);
 HcclResult HcclAmdGetCclBufferSize(HcclComm comm, uint64_t* bytes);
 
 /*
+ * Hang triage.  With HCCL_AMD_STUCK_COUNTERS=1 in the environment when the communicators are created, every
+ * collective of the world is numbered (1, 2, ...) and its launch stream writes that number to a head word in front
+ * of the collective's kernels and to a tail word behind them (pinned host memory, readable while the GPU is
+ * busy or hung).  head == tail: nothing is running; head == tail + 1: a kernel of collective `head` has started
+ * and not finished.  Follows the reference's head / tail counters
+ * (src/ops/op_common/algorithm/template/aiv/aiv_communication_base_v2.h:365-378,
+ * src/ops/op_common/stuck_detect_counter_helper.h).  HCCL_E_UNAVAIL when the counters are not enabled.
+ */
+HcclResult HcclAmdGetStuckCounters(HcclComm comm, uint64_t* head, uint64_t* tail);
+
+/*
  * Host-only view of the reduction plan: writes the fold program the kernel would run for
  * segment `segment` of (op, algo, rankSize) into `out` (at most `cap` bytes) and its length
  * into *len.  Program bytes: 0x00-0x3F = fold rank r into the accumulator of the current

@@ -430,6 +430,23 @@ def test_slab_all_reduce_can_be_captured_into_a_graph(monkeypatch):
         w.close()
 
 
+def test_head_and_tail_counters_follow_the_collectives(monkeypatch):
+    """HCCL_AMD_STUCK_COUNTERS=1: the launch stream writes the number of every collective in front of and behind its
+    kernels; after a synchronisation both words hold the number of the last collective, and results are unchanged."""
+    monkeypatch.setenv("HCCL_AMD_STUCK_COUNTERS", "1")
+    w = World(4)
+    monkeypatch.delenv("HCCL_AMD_STUCK_COUNTERS")
+    try:
+        assert hccl_amd.get_stuck_counters(w.comms[0]) == (0, 0)
+        run_all_reduce(w, DT.FP32, SUM, 10_007, "mesh", seed=31)
+        assert hccl_amd.get_stuck_counters(w.comms[1]) == (1, 1)
+        run_reduce_scatter(w, DT.BFP16, SUM, 4_099, "nhr", seed=32)
+        run_all_reduce(w, DT.INT32, MAX, 77, "rhd", seed=33)
+        assert hccl_amd.get_stuck_counters(w.comms[3]) == (3, 3)
+    finally:
+        w.close()
+
+
 def test_all_reduce_larger_than_a_million_workgroups():
     """2 x 1 GiB of fp16 per rank: 2^26 vector positions, one per lane, 2^20 workgroups per destination."""
     import torch

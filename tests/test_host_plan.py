@@ -641,3 +641,14 @@ def test_a_rejected_call_keeps_its_place_in_the_sequence():
     finally:
         for c in comms:
             hccl_amd.comm_destroy(c)
+
+
+def test_stuck_counters_are_unavailable_unless_enabled(monkeypatch):
+    monkeypatch.delenv("HCCL_AMD_STUCK_COUNTERS", raising=False)
+    comms = hccl_amd.comm_init_all(2)
+    try:
+        assert code_of(hccl_amd.get_stuck_counters, comms[0]) == 7          # HCCL_E_UNAVAIL
+    finally:
+        for c in comms:
+            hccl_amd.comm_destroy(c)
+    assert code_of(hccl_amd.get_stuck_counters, comms[0]) == 1              # stale handle
