@@ -267,6 +267,7 @@ struct World {
     uint8_t* a2aScratch = nullptr;
     uint32_t reduceBlocks = 1u << 26;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
+    uint32_t storeWaves = 0;      // wavefronts sharing the stores of a many-destination reduce tile; 0: chosen per launch
     uint32_t copyTileBytes = 0;
     uint32_t copyDstPerGroup = 0;   // HCCL_AMD_COPY_DST_PER_WAVE: destinations one wavefront stores to, 0 = per launch
     bool reduceVector = true;
@@ -407,6 +408,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         w->device = 0;
     }
     w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 1u << 26);
+    w->storeWaves = EnvU32("HCCL_AMD_REDUCE_STORE_WAVES", 0);
+    if (w->storeWaves > kMaxReduceThreads / 64) {
+        w->storeWaves = 0;
+    }
     w->reduceThreads = EnvU32("HCCL_AMD_REDUCE_THREADS", 0);
     if (w->reduceThreads != 64 && w->reduceThreads != 128 && w->reduceThreads != 256) {
         w->reduceThreads = 0;
@@ -633,6 +638,34 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     // wavefronts in flight: +1-2 %); AllReduce's many result streams and larger worlds with sixteen (+5 %).
     a.vecBatch = w->reduceBatch != 0 ? w->reduceBatch : ((w->n <= 8 && !a.varGroups && (a.dstOwn || a.nDst == 1)) ? 8u : 16u);
     a.threads = w->reduceThreads != 0 ? w->reduceThreads : 64u;
+    // A result that goes to many destinations: a wavefront that stores to six or more streams one after the other
+    // is what bounds the launch, so wavefront 0 of a workgroup folds the tile and two or three wavefronts share its
+    // stores.  The extra wavefronts hold slots while they wait, which costs more than it gains on short messages
+    // and where folding a tile takes long (8- and 16-bit types with their wide accumulators): measured, fp32 SUM
+    // in rank order, 6 ranks 0.72 -> 0.75 / 0.74 -> 0.79 / 0.73 -> 0.78 of the HBM peak at 64 / 128 / 512 MiB per
+    // rank with two wavefronts (32 MiB: 0.69 -> 0.67), 8 ranks 0.65 -> 0.72 / 0.70 -> 0.77 / 0.72 -> 0.78 at 32 / 64 /
+    // 128 MiB with three (16 MiB: 0.62 -> 0.61); four ranks lose at every size.  HCCL_AMD_REDUCE_STORE_WAVES forces
+    // a count (1 = one wavefront per tile).
+    a.storeWaves = 1;
+    if (!oneStream && a.threads == 64 && a.vecOk) {
+        const uint64_t bytes = a.total * esz;
+        const bool longFold = esz < 4;
+        uint32_t waves = 1;
+        if (a.nDst >= 8) {
+            waves = longFold ? (bytes >= (64ull << 20) ? 2u : 1u) : (bytes >= (24ull << 20) ? 3u : 1u);
+        } else if (a.nDst >= 6) {
+            waves = bytes >= (48ull << 20) ? 2u : 1u;
+        }
+        if (w->storeWaves != 0) {
+            waves = w->storeWaves < a.nDst ? w->storeWaves : a.nDst;
+        }
+        a.storeWaves = waves;
+        // With the stores elsewhere the folding wavefront is better off with the smaller load batch where that
+        // holds every leaf (fp16 RHD over 6 ranks: 0.71 -> 0.75, fp16 NHR over 8: 0.71 -> 0.77).
+        if (waves > 1 && w->reduceBatch == 0 && w->n <= 8) {
+            a.vecBatch = 8;
+        }
+    }
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
     uint64_t blocks = subs * a.blocksPerSub;
     if (a.varGroups) {

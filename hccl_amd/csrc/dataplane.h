@@ -75,6 +75,9 @@ struct ReduceArgs {
     uint32_t vecBatch;       // leaves per load batch of the 128-bit path: 8 or 16 (picks the kernel instantiation)
     uint32_t writeThrough;   // 16-byte results leave through StoreStream16 instead of a non-temporal store
     uint32_t leadFromSrc;    // wavefronts start on a 128-byte line of the sources instead of the destination
+    uint32_t storeWaves;     // > 1: workgroups of 64 * storeWaves threads, wavefront 0 folds and wavefront k stores to
+                             // destinations k, k + storeWaves, ... (threads must be 64, dstOwn 0); 0 or 1: every wavefront
+                             // folds and stores its own tile
     // Groups of unequal length (ReduceScatterV): when varGroups is set, group g spans groupLenV[g]
     // elements starting groupOffV[g] elements into every source, instead of the uniform
     // groupLen / srcGroupStride / total geometry, and owns the workgroups

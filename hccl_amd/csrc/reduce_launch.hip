@@ -24,7 +24,14 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
     if (fn == nullptr || nBlocks == 0 || (args.threads != 64 && args.threads != 128 && args.threads != 256)) {
         return hipErrorInvalidValue;
     }
-    hipLaunchKernelGGL(fn, dim3(nBlocks), dim3(args.threads), ldsBytes, stream, args);
+    uint32_t threads = args.threads;
+    if (args.storeWaves > 1) {
+        if (args.threads != 64 || args.dstOwn != 0 || args.storeWaves * 64 > kMaxReduceThreads) {
+            return hipErrorInvalidValue;
+        }
+        threads = 64 * args.storeWaves;
+    }
+    hipLaunchKernelGGL(fn, dim3(nBlocks), dim3(threads), ldsBytes, stream, args);
     return hipGetLastError();
 }
 

@@ -390,6 +390,33 @@ def test_all_reduce_through_the_staging_slab(monkeypatch, n):
         w.close()
 
 
+@pytest.mark.parametrize("n,waves", [(2, 2), (5, 2), (6, 3), (8, 4), (16, 4), (3, 4)])
+def test_all_reduce_with_the_stores_of_a_tile_shared_by_wavefronts(monkeypatch, n, waves):
+    """The many-destination form of the fused kernel (wavefront 0 folds a tile, `waves` wavefronts store it),
+    forced for small messages; a slab never steps in, and a small grid makes every workgroup loop over tiles."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_STORE_WAVES", str(waves))
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB", "0")
+    monkeypatch.setenv("HCCL_AMD_REDUCE_BLOCKS", "24")
+    w = World(n)
+    monkeypatch.delenv("HCCL_AMD_REDUCE_STORE_WAVES")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB")
+    monkeypatch.delenv("HCCL_AMD_REDUCE_BLOCKS")
+    try:
+        seed = 5200 + 10 * n + waves
+        for dtype in REDUCE_TYPES:
+            run_all_reduce(w, dtype, SUM, 20_011, "mesh", seed=seed)
+            seed += 1
+        run_all_reduce(w, DT.FP32, SUM, 70_001, "nhr", seed=seed)                # nested order, LDS stack in wavefront 0
+        run_all_reduce(w, DT.BFP16, SUM, 50_003, "rhd", seed=seed + 1)
+        run_all_reduce(w, DT.FP16, MAX, 33_333, "order_preserved", seed=seed + 2, pad=2)   # unaligned: head and tail elements
+        run_all_reduce(w, DT.INT8, MIN, 9, "mesh", seed=seed + 3)                # less than one vector
+        run_all_reduce(w, DT.INT32, PROD, 4_099, "mesh", seed=seed + 4, in_place=True)
+        run_all_reduce(w, DT.FP64, SUM, 12_345, "mesh", seed=seed + 5, pad=lambda r, which: r + (3 if which == "recv" else 0))
+        run_reduce_scatter(w, DT.FP32, SUM, 5_001, "mesh", seed=seed + 6)        # one result stream: form not taken
+    finally:
+        w.close()
+
+
 def test_slab_all_reduce_can_be_captured_into_a_graph(monkeypatch):
     """Once the slab exists (one eager call of that size) the two-kernel AllReduce is launches only."""
     import torch
