@@ -2,14 +2,16 @@
 // that do nothing but the loads, one add per operand and the stores: the yardstick the library's kernels are
 // held against, and the experiments behind the shapes they have.
 //
-//   reads / writes alone          N read streams, or N write streams, one 16-byte vector per lane
-//   fused N reads + N writes      the AllReduce pattern in one kernel
-//   slab                          the same work as two kernels per piece: N reads folded into a slab of P MiB,
-//                                 then the slab written to the N destinations (by one wavefront per tile, or by
-//                                 wavefronts that take D destinations each)
-//   one source, N destinations    the AllGather / Broadcast pattern: one wavefront per tile storing to every
-//                                 destination, against D destinations per wavefront with the wavefronts of one
-//                                 tile on the same XCD (workgroup indices 8 apart)
+//   reads alone                   N read streams, one 16-byte vector per lane, one wavefront per 1 KiB tile
+//   writes alone                  N write streams from one wavefront per tile, or dealt to the W wavefronts of a
+//                                 workgroup (W = N: one stream per wavefront)
+//   fused N reads + N writes      the AllReduce pattern in one kernel; with the stores of a tile shared by W
+//                                 wavefronts (wavefront 0 folds and hands the result over through LDS)
+//   fold + fan-out                the same work as two kernels per piece of P MiB: N reads folded into the first
+//                                 destination, then that range (still cached) to the other N - 1 destinations with
+//                                 one wavefront per destination; also with the two kernels of neighbouring pieces
+//                                 overlapped on two streams
+//   one source, N destinations    the AllGather / Broadcast pattern, source read from memory
 //
 // Build: make -C examples      Run: examples/bin/hbm_patterns [ranks=16] [MiB per rank=256]
 // Prints one line per pattern: time per pass, bytes moved per second, fraction of the 8 TB/s HBM peak.
@@ -34,21 +36,18 @@ constexpr double kPeakGBs = 8000.0;
 struct Bufs {
     const U4* src[kMaxStreams];
     U4* dst[kMaxStreams];
-    U4* slab;
 };
 
 __device__ __forceinline__ U4 LoadNt(const U4* p) { return __builtin_nontemporal_load((const __attribute__((address_space(1))) U4*)p); }
 __device__ __forceinline__ U4 LoadPlain(const U4* p) { return *((const __attribute__((address_space(1))) U4*)p); }
-// STORE: 0 non-temporal, 1 written through at system scope, 2 plain
+// STORE: 0 non-temporal, 1 written through at system scope
 template <int STORE>
 __device__ __forceinline__ void Store(U4 v, U4* p)
 {
     if (STORE == 0) {
         __builtin_nontemporal_store(v, (__attribute__((address_space(1))) U4*)p);
-    } else if (STORE == 1) {
-        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
     } else {
-        *((__attribute__((address_space(1))) U4*)p) = v;
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
     }
 }
 template <int N>
@@ -59,51 +58,13 @@ __device__ __forceinline__ void AllIssued(U4* v)
         asm volatile("" : "+v"(v[i]));
     }
 }
-
-template <int N, bool READ, bool WRITE, int STORE>
-__global__ __launch_bounds__(64) void Streams(Bufs b, size_t first, size_t nVec)
-{
-    const size_t o = static_cast<size_t>(blockIdx.x) * 64 + threadIdx.x;
-    if (o >= nVec) {
-        return;
-    }
-    const size_t idx = first + o;
-    U4 acc = {1u, 2u, 3u, static_cast<uint32_t>(idx)};
-    if (READ) {
-        U4 v[N];
-#pragma unroll
-        for (int i = 0; i < N; ++i) {
-            v[i] = LoadNt(b.src[i] + idx);
-        }
-        AllIssued<N>(v);
-        acc = v[0];
-#pragma unroll
-        for (int i = 1; i < N; ++i) {
-            acc += v[i];
-        }
-    }
-    if (WRITE) {
-#pragma unroll
-        for (int i = 0; i < N; ++i) {
-            Store<STORE>(acc, b.dst[i] + idx);
-        }
-    } else if (acc.x == 0x12345678u && acc.y == 0x9ABCDEF0u) {
-        Store<STORE>(acc, b.dst[0] + idx);   // keeps the loads alive
-    }
-}
-
-// N reads folded into slab[o]
 template <int N>
-__global__ __launch_bounds__(64) void ToSlab(Bufs b, size_t first, size_t nVec)
+__device__ __forceinline__ U4 Fold(const Bufs& b, size_t idx)
 {
-    const size_t o = static_cast<size_t>(blockIdx.x) * 64 + threadIdx.x;
-    if (o >= nVec) {
-        return;
-    }
     U4 v[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-        v[i] = LoadNt(b.src[i] + first + o);
+        v[i] = LoadNt(b.src[i] + idx);
     }
     AllIssued<N>(v);
     U4 acc = v[0];
@@ -111,37 +72,70 @@ __global__ __launch_bounds__(64) void ToSlab(Bufs b, size_t first, size_t nVec)
     for (int i = 1; i < N; ++i) {
         acc += v[i];
     }
-    Store<1>(acc, b.slab + o);
+    return acc;
 }
 
-// source[o] (the slab, or src[0] + first) to D destinations per wavefront.  XCD: the G = N / D wavefronts of one
-// tile have workgroup indices 8 apart (same XCD), and the source is loaded with a plain load so that its L2
-// serves all but the first; otherwise group g covers all tiles before group g + 1 starts.
-template <int N, int D, int STORE, bool XCD>
-__global__ __launch_bounds__(64) void Fan(Bufs b, const U4* source, size_t first, size_t nVec)
+// Every size here is a multiple of 1 KiB, so a workgroup never has lanes without a vector.
+//
+// W wavefronts per tile.  READ: wavefront 0 folds the tile (and hands the result to the others through LDS when
+// W > 1).  WRITE: wavefront w stores to destinations w, w + W, ...
+template <int N, int W, bool READ, bool WRITE, int STORE>
+__global__ __launch_bounds__(64 * W) void Streams(Bufs b, size_t nVec)
 {
-    constexpr int G = N / D;
-    const size_t blk = blockIdx.x;
-    size_t tile;
-    int g;
-    if (XCD) {
-        const size_t row = blk / (8 * G);
-        const size_t j = blk % (8 * G);
-        tile = row * 8 + (j & 7);
-        g = static_cast<int>(j >> 3);
-    } else {
-        const size_t tiles = (nVec + 63) / 64;
-        g = static_cast<int>(blk / tiles);
-        tile = blk - static_cast<size_t>(g) * tiles;
+    __shared__ U4 parked[64];
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned wave = threadIdx.x >> 6;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 64 + lane;
+    U4 acc = {1u, 2u, 3u, static_cast<uint32_t>(idx)};
+    if (READ) {
+        if (wave == 0) {
+            acc = Fold<N>(b, idx);
+            if (W > 1) {
+                parked[lane] = acc;
+            }
+        }
+        if (W > 1) {
+            __syncthreads();
+            if (wave != 0) {
+                acc = parked[lane];
+            }
+        }
     }
-    const size_t o = tile * 64 + threadIdx.x;
-    if (o >= nVec) {
-        return;
-    }
-    const U4 v = XCD ? LoadPlain(source + o) : LoadNt(source + o);
+    if (WRITE) {
 #pragma unroll
-    for (int i = 0; i < D; ++i) {
-        Store<STORE>(v, b.dst[g * D + i] + first + o);
+        for (int i = 0; i < (N + W - 1) / W; ++i) {
+            if (wave + W * i < N) {
+                Store<STORE>(acc, b.dst[wave + W * i] + idx);
+            }
+        }
+    } else if (acc.x == 0x12345678u && acc.y == 0x9ABCDEF0u) {
+        Store<STORE>(acc, b.dst[0] + idx);   // keeps the loads alive
+    }
+}
+
+// N reads folded into dst[0], from element `first` on
+template <int N>
+__global__ __launch_bounds__(64) void FoldToFirst(Bufs b, size_t first)
+{
+    const size_t idx = first + static_cast<size_t>(blockIdx.x) * 64 + threadIdx.x;
+    Store<1>(Fold<N>(b, idx), b.dst[0] + idx);
+}
+
+// `source` to the destinations firstDst, firstDst + 1, ...: wavefront w of the workgroup takes destinations
+// firstDst + w, firstDst + w + W, ... below N.  HOT: the source has just been written (plain load, non-temporal
+// stores); otherwise it comes from memory (non-temporal load, stores written through).
+template <int N, int W, bool HOT>
+__global__ __launch_bounds__(64 * W) void FanOut(Bufs b, const U4* source, int firstDst, size_t first)
+{
+    const unsigned wave = threadIdx.x >> 6;
+    const size_t idx = first + static_cast<size_t>(blockIdx.x) * 64 + (threadIdx.x & 63u);
+    const U4 v = HOT ? LoadPlain(source + idx) : LoadNt(source + idx);
+#pragma unroll
+    for (int i = 0; i < (N + W - 1) / W; ++i) {
+        const int d = firstDst + static_cast<int>(wave) + W * i;
+        if (d < N) {
+            Store<HOT ? 0 : 1>(v, b.dst[d] + idx);
+        }
     }
 }
 
@@ -165,26 +159,46 @@ float MsPerPass(F pass)
 
 void Report(int n, const char* what, float ms, double bytes)
 {
-    printf("N=%-2d %-66s %8.3f ms %6.0f GB/s  %.3f\n", n, what, ms, bytes / ms / 1e6, bytes / ms / 1e6 / kPeakGBs);
+    printf("N=%-2d %-72s %8.3f ms %6.0f GB/s  %.3f\n", n, what, ms, bytes / ms / 1e6, bytes / ms / 1e6 / kPeakGBs);
     fflush(stdout);
 }
 
-template <int N, int D>
-void SlabRow(const Bufs& b, size_t nVec, size_t pieceMiB, double total)
+template <int N, int W>
+void SplitRows(const Bufs& b, size_t nVec, double half)
+{
+    const unsigned blocks = static_cast<unsigned>(nVec / 64);
+    char what[128];
+    snprintf(what, sizeof what, "writes alone over %d wavefronts per tile, written through", W);
+    Report(N, what, MsPerPass([&] { hipLaunchKernelGGL((Streams<N, W, false, true, 1>), dim3(blocks), dim3(64 * W), 0, 0, b, nVec); }), half);
+    snprintf(what, sizeof what, "fused, wavefront 0 folds, %d wavefronts store, non-temporal", W);
+    Report(N, what, MsPerPass([&] { hipLaunchKernelGGL((Streams<N, W, true, true, 0>), dim3(blocks), dim3(64 * W), 0, 0, b, nVec); }), 2 * half);
+}
+
+template <int N>
+void FoldFanRow(const Bufs& b, size_t nVec, size_t pieceMiB, bool twoStreams, hipStream_t other, hipEvent_t* folded, hipEvent_t joined)
 {
     size_t piece = (pieceMiB << 20) / 16;
     piece = piece < nVec ? piece : nVec;
-    const unsigned blocks = static_cast<unsigned>((piece + 63) / 64);
-    const unsigned fanBlocks = D == N ? blocks : (blocks + 7) / 8 * 8 * (N / D);
+    constexpr int W = N - 1;
     const float ms = MsPerPass([&] {
-        for (size_t first = 0; first < nVec; first += piece) {
-            hipLaunchKernelGGL((ToSlab<N>), dim3(blocks), dim3(64), 0, 0, b, first, piece);
-            hipLaunchKernelGGL((Fan<N, D, D == N ? 1 : 0, D != N>), dim3(fanBlocks), dim3(64), 0, 0, b, b.slab, first, piece);
+        int k = 0;
+        for (size_t first = 0; first < nVec; first += piece, ++k) {
+            const unsigned blocks = static_cast<unsigned>((first + piece <= nVec ? piece : nVec - first) / 64);
+            hipLaunchKernelGGL((FoldToFirst<N>), dim3(blocks), dim3(64), 0, 0, b, first);
+            if (twoStreams) {
+                CK(hipEventRecord(folded[k % 64], 0));
+                CK(hipStreamWaitEvent(other, folded[k % 64], 0));
+            }
+            hipLaunchKernelGGL((FanOut<N, W, true>), dim3(blocks), dim3(64 * W), 0, twoStreams ? other : 0, b, b.dst[0], 1, first);
+        }
+        if (twoStreams) {
+            CK(hipEventRecord(joined, other));
+            CK(hipStreamWaitEvent(0, joined, 0));
         }
     });
     char what[128];
-    snprintf(what, sizeof what, "slab of %3zu MiB: fold kernel, then %d destination(s) per wavefront", pieceMiB, D);
-    Report(N, what, ms, total);
+    snprintf(what, sizeof what, "fold + fan-out, pieces of %3zu MiB%s", pieceMiB, twoStreams ? ", neighbouring pieces overlapped on two streams" : "");
+    Report(N, what, ms, 2.0 * N * nVec * 16);
 }
 
 template <int N>
@@ -197,36 +211,42 @@ void Run(size_t bytesPerRank)
         CK(hipMemset((void*)b.src[i], 1 + i, bytesPerRank));
         CK(hipMalloc((void**)&b.dst[i], bytesPerRank));
     }
-    CK(hipMalloc((void**)&b.slab, 128u << 20));
-    const unsigned blocks = static_cast<unsigned>((nVec + 63) / 64);
+    hipStream_t other;
+    CK(hipStreamCreateWithFlags(&other, hipStreamNonBlocking));
+    hipEvent_t folded[64], joined;
+    for (hipEvent_t& ev : folded) {
+        CK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    }
+    CK(hipEventCreateWithFlags(&joined, hipEventDisableTiming));
+    const unsigned blocks = static_cast<unsigned>(nVec / 64);
     const double half = static_cast<double>(N) * bytesPerRank;
-    Report(N, "reads alone", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, true, false, 0>), dim3(blocks), dim3(64), 0, 0, b, size_t(0), nVec); }), half);
-    Report(N, "writes alone, non-temporal", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, false, true, 0>), dim3(blocks), dim3(64), 0, 0, b, size_t(0), nVec); }), half);
-    Report(N, "writes alone, written through", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, false, true, 1>), dim3(blocks), dim3(64), 0, 0, b, size_t(0), nVec); }), half);
-    Report(N, "fused N reads + N writes, non-temporal stores", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, true, true, 0>), dim3(blocks), dim3(64), 0, 0, b, size_t(0), nVec); }), 2 * half);
-    Report(N, "fused N reads + N writes, stores written through", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, true, true, 1>), dim3(blocks), dim3(64), 0, 0, b, size_t(0), nVec); }), 2 * half);
-    for (size_t pieceMiB : {16, 32, 64, 128}) {
-        SlabRow<N, N>(b, nVec, pieceMiB, 2 * half);
-        SlabRow<N, 2>(b, nVec, pieceMiB, 2 * half);
+    Report(N, "reads alone", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, true, false, 0>), dim3(blocks), dim3(64), 0, 0, b, nVec); }), half);
+    Report(N, "writes alone, one wavefront per tile, non-temporal", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, false, true, 0>), dim3(blocks), dim3(64), 0, 0, b, nVec); }), half);
+    Report(N, "writes alone, one wavefront per tile, written through", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, false, true, 1>), dim3(blocks), dim3(64), 0, 0, b, nVec); }), half);
+    Report(N, "fused N reads + N writes, non-temporal stores", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, true, true, 0>), dim3(blocks), dim3(64), 0, 0, b, nVec); }), 2 * half);
+    Report(N, "fused N reads + N writes, stores written through", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, true, true, 1>), dim3(blocks), dim3(64), 0, 0, b, nVec); }), 2 * half);
+    SplitRows<N, 2>(b, nVec, half);
+    SplitRows<N, 3>(b, nVec, half);
+    SplitRows<N, 4>(b, nVec, half);
+    SplitRows<N, N>(b, nVec, half);
+    for (size_t pieceMiB : {16, 64, 256}) {
+        FoldFanRow<N>(b, nVec, pieceMiB, false, other, folded, joined);
     }
-    // one source (src[0]), N destinations, whole buffers and the first 64 MiB of them
-    for (size_t span : {bytesPerRank, static_cast<size_t>(64) << 20}) {
-        const size_t vecs = (span < bytesPerRank ? span : bytesPerRank) / 16;
-        const unsigned bl = static_cast<unsigned>((vecs + 63) / 64);
-        const double moved = (1.0 + N) * vecs * 16;
-        char what[128];
-        snprintf(what, sizeof what, "1 source of %zu MiB to N destinations, one wavefront per tile", vecs >> 16);
-        Report(N, what, MsPerPass([&] { hipLaunchKernelGGL((Fan<N, N, 1, false>), dim3(bl), dim3(64), 0, 0, b, b.src[0], size_t(0), vecs); }), moved);
-        snprintf(what, sizeof what, "1 source of %zu MiB to N destinations, 2 per wavefront, tile's wavefronts on one XCD", vecs >> 16);
-        Report(N, what, MsPerPass([&] { hipLaunchKernelGGL((Fan<N, 2, 0, true>), dim3((bl + 7) / 8 * 8 * (N / 2)), dim3(64), 0, 0, b, b.src[0], size_t(0), vecs); }), moved);
-        snprintf(what, sizeof what, "1 source of %zu MiB to N destinations, 2 per wavefront, group after group", vecs >> 16);
-        Report(N, what, MsPerPass([&] { hipLaunchKernelGGL((Fan<N, 2, 0, false>), dim3(bl * (N / 2)), dim3(64), 0, 0, b, b.src[0], size_t(0), vecs); }), moved);
-    }
+    FoldFanRow<N>(b, nVec, 64, true, other, folded, joined);
+    // one source (src[k], another one every pass) to N destinations
+    int pass = 0;
+    const double moved = (1.0 + N) * bytesPerRank;
+    Report(N, "1 source to N destinations, one wavefront per tile", MsPerPass([&] {
+               hipLaunchKernelGGL((FanOut<N, 1, false>), dim3(blocks), dim3(64), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
+           }), moved);
+    Report(N, "1 source to N destinations, two wavefronts per tile", MsPerPass([&] {
+               hipLaunchKernelGGL((FanOut<N, 2, false>), dim3(blocks), dim3(128), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
+           }), moved);
     for (int i = 0; i < N; ++i) {
         CK(hipFree((void*)b.src[i]));
         CK(hipFree(b.dst[i]));
     }
-    CK(hipFree(b.slab));
+    CK(hipStreamDestroy(other));
 }
 
 int main(int argc, char** argv)
@@ -239,7 +259,7 @@ int main(int argc, char** argv)
     }
     CK(hipEventCreate(&g_start));
     CK(hipEventCreate(&g_stop));
-    printf("pattern%62s time per pass   moved   of 8 TB/s\n", "");
+    printf("pattern%68s time per pass   moved   of 8 TB/s\n", "");
     if (n == 16) {
         Run<16>(mib << 20);
     } else if (n == 8) {

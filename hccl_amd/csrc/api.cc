@@ -257,11 +257,9 @@ struct World {
     bool stuckEnabled = false;
     uint64_t* stuck = nullptr;
     uint64_t launchSeq = 0;
-    // Large rank-order AllReduce over many ranks: the staging slab between its reduce and broadcast kernels.
-    uint8_t* slab = nullptr;
-    uint64_t slabHeld = 0;               // bytes allocated
-    uint64_t slabBytes = 256ull << 20;   // HCCL_AMD_ALLREDUCE_SLAB_BYTES
-    int slabMode = 2;                    // HCCL_AMD_ALLREDUCE_SLAB: 0 never, 1 always, 2 by rank count and size
+    // AllReduce as fold + fan-out (two kernels per piece of at most pieceBytes of results).
+    uint64_t pieceBytes = 256ull << 20;   // HCCL_AMD_ALLREDUCE_PIECE_BYTES
+    int twoKernelMode = 2;                // HCCL_AMD_ALLREDUCE_TWO_KERNELS: 0 never, 1 always, unset: by rank count and size
     // Allocation-free AlltoAllV: host image of the tables and the device array that receives them.
     std::vector<uint64_t> a2aImage;
     uint8_t* a2aScratch = nullptr;
@@ -269,7 +267,6 @@ struct World {
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t storeWaves = 0;      // wavefronts sharing the stores of a many-destination reduce tile; 0: chosen per launch
     uint32_t copyTileBytes = 0;
-    uint32_t copyDstPerGroup = 0;   // HCCL_AMD_COPY_DST_PER_WAVE: destinations one wavefront stores to, 0 = per launch
     bool reduceVector = true;
     uint32_t reduceBatch = 0;     // HCCL_AMD_REDUCE_BATCH: 8 or 16, 0 = per launch
     bool leadFromSrc = true;      // HCCL_AMD_LEAD_FROM_SRC=0: wavefronts always start on the destination's lines
@@ -292,7 +289,6 @@ struct World {
         for (hipEvent_t e : eventPool) (void)hipEventDestroy(e);
         if (doneEvent) (void)hipEventDestroy(doneEvent);
         if (a2aDev) (void)hipFree(a2aDev);
-        if (slab) (void)hipFree(slab);
         if (stuck) (void)hipHostFree(stuck);
         for (int s = 0; s < kStagingSlots; ++s) {
             if (a2aHost[s]) (void)hipHostFree(a2aHost[s]);
@@ -420,7 +416,6 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->copyTileBytes != 1024 && w->copyTileBytes != 4096 && w->copyTileBytes != 16384) {
         w->copyTileBytes = 0;
     }
-    w->copyDstPerGroup = EnvU32("HCCL_AMD_COPY_DST_PER_WAVE", 0);
     w->execTimeout = EnvU32("HCCL_EXEC_TIMEOUT", 1836);
     w->storePolicy = EnvU32("HCCL_AMD_STORE_POLICY", 2);
     if (w->storePolicy > 2) {
@@ -428,11 +423,14 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     }
     w->reduceVector = EnvU32("HCCL_AMD_REDUCE_VECTOR", 1) != 0;
     w->stuckEnabled = EnvU32("HCCL_AMD_STUCK_COUNTERS", 0) != 0;
-    w->slabMode = getenv("HCCL_AMD_ALLREDUCE_SLAB") != nullptr ? atoi(getenv("HCCL_AMD_ALLREDUCE_SLAB")) : 2;
-    if (w->slabMode < 0 || w->slabMode > 2) {
-        w->slabMode = 2;
+    w->twoKernelMode = getenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS") != nullptr ? atoi(getenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS")) : 2;
+    if (w->twoKernelMode < 0 || w->twoKernelMode > 1) {
+        w->twoKernelMode = 2;
     }
-    w->slabBytes = (static_cast<uint64_t>(EnvU32("HCCL_AMD_ALLREDUCE_SLAB_BYTES", 256u << 20)) + 255) & ~255ull;
+    w->pieceBytes = (static_cast<uint64_t>(EnvU32("HCCL_AMD_ALLREDUCE_PIECE_BYTES", 256u << 20)) + 255) & ~255ull;
+    if (w->pieceBytes == 0) {
+        w->pieceBytes = 256;
+    }
     w->leadFromSrc = getenv("HCCL_AMD_LEAD_FROM_SRC") == nullptr || atoi(getenv("HCCL_AMD_LEAD_FROM_SRC")) != 0;
     w->reduceBatch = EnvU32("HCCL_AMD_REDUCE_BATCH", 0);
     if (w->reduceBatch != 8 && w->reduceBatch != 16) {
@@ -745,76 +743,123 @@ HcclResult LaunchMeshChunk(World* w, const DevicePlan& plan, const PendingOp& p,
     return HCCL_SUCCESS;
 }
 
-HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s, bool sourceIsHot = false);
+HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s);
 
-// Rank-order AllReduce in two kernels per slab-sized piece: the fold of all ranks into a slab the library owns
-// (N reads, one write that stays in the last-level cache), then the slab to every recvBuf with the split copy
-// kernel.  Same fold program, same bits as the fused kernel.  Measured fractions of the HBM peak, slab form
-// against fused kernel, int32 SUM, pieces of up to 256 MiB (the largest range per destination the split copy
-// form takes; smaller slabs lose to launch gaps: 16 / 32 / 64 / 128 MiB gave 0.70 / 0.73 / 0.74 / 0.74 on sixteen
-// ranks of 256 MiB):
-//   ranks    32 MiB        128 MiB       256 MiB       512 MiB per rank
-//     6    0.67 / 0.70   0.74 / 0.74   0.75 / 0.70   0.73 / 0.73
-//     8    0.66 / 0.67   0.77 / 0.73   0.76 / 0.68   0.76 / 0.70
-//    10    0.67 / 0.63   0.77 / 0.71   0.76 / 0.71   0.75 / 0.69
-//    16    0.70 / 0.65   0.77 / 0.71   0.76 / 0.70
-//    32    0.74 / 0.62   0.75 / 0.67   0.74 / 0.67
-// hence the slab from ten ranks on for messages of 16 MiB and more, and for eight and nine ranks from 64 MiB.
-bool UseSlab(const World* w, uint64_t bytes)
+// A result that every rank receives, as two kernels per piece: the fold of all ranks into the first rank's recvBuf
+// (N reads and one write, the shape of a ReduceScatter launch), then that range, just written and therefore still in
+// the last-level cache, to the other recvBufs with one wavefront per destination stream.  Exactly the algorithmic
+// traffic, no memory of the library's own, same fold program and same bits as the fused kernel.  Reads and writes
+// each run near what the part gives them alone (reads 0.80-0.85 of the HBM peak, writes from one wavefront per
+// stream 0.89-0.91), where the fused kernel, whose wavefronts store to every destination after loading from every
+// source, reaches 0.70-0.78.  Measured, fp32 SUM in rank order, two kernels / fused:
+//   ranks    8 MiB         16 MiB        32 MiB        64 MiB        256 MiB per rank
+//     4                  0.62 / 0.62   0.69 / 0.69                 0.78 / 0.78
+//     6    0.57 / 0.58   0.66 / 0.63   0.73 / 0.69   0.78 / 0.74   0.82 / 0.79
+//     8    0.60 / 0.60   0.68 / 0.62   0.75 / 0.71   0.80 / 0.77   0.82 / 0.76
+//    16    0.65 / 0.57   0.74 / 0.58   0.79 / 0.73   0.82 / 0.76   0.83 / 0.74
+// (2 and 3 ranks lose: 0.64 / 0.78, 0.76 / 0.77.)  A piece must still be cached when it is read back: 256 MiB pieces
+// are the best (1 GiB per rank over 6 ranks: 0.76 / 0.78 / 0.78 with 64 / 128 / 256 MiB, 0.64 with 512 MiB).
+bool FoldThenFanOut(const World* w, uint32_t nDst, uint64_t bytes)
 {
-    if (w->slabMode != 2) {
-        return w->slabMode == 1;
+    if (nDst < 2) {
+        return false;
     }
-    return (w->n >= 10 && bytes >= (16ull << 20)) || (w->n >= 8 && bytes >= (64ull << 20));
+    if (w->twoKernelMode != 2) {
+        return w->twoKernelMode == 1;
+    }
+    return nDst >= 12 ? bytes >= (8ull << 20) : (nDst >= 5 && bytes >= (16ull << 20));
 }
 
-HcclResult RunAllReduceViaSlab(World* w, PendingOp& p, const DevicePlan& plan, const ReduceArgs& flat, hipStream_t s)
+// Launch of a fold whose result [0, a.total) goes to all a.nDst destinations (a.nGroup == 1, a.dstOwn == 0): the
+// fused kernel, or fold + fan-out per piece.  Pieces are whole sub-segments while those fit (each has its own fold
+// program), and parts of a sub-segment that is longer than a piece.
+HcclResult LaunchToAll(World* w, const ReduceArgs& a, const DevicePlan& plan, HcclDataType dtype, HcclReduceOp op,
+                       hipStream_t s)
 {
-    const uint32_t n = w->n;
-    const uint32_t esz = DataTypeSize(p.dtype);
-    // The slab is allocated on first use, as large as this message needs (up to slabBytes), and grows with later
-    // messages: a world that only moves 16 MiB does not hold 256 MiB.
-    const uint64_t want = std::min<uint64_t>(w->slabBytes, (p.count * esz + 255) & ~255ull);
-    if (w->slab == nullptr || w->slabHeld < want) {
-        if (w->slab != nullptr) {
-            HIP_OK(hipDeviceSynchronize());   // an earlier collective may still be using the smaller slab
-            HIP_OK(hipFree(w->slab));
-            w->slab = nullptr;
+    const uint32_t esz = DataTypeSize(dtype);
+    if (a.nGroup != 1 || a.dstOwn != 0 || a.varGroups != 0 || !FoldThenFanOut(w, a.nDst, a.total * esz)) {
+        ReduceArgs fused = a;
+        return LaunchOneReduce(w, fused, plan, dtype, op, s);
+    }
+    const uint64_t pieceEl = std::max<uint64_t>(1, w->pieceBytes / esz);
+    auto piece = [&](uint32_t firstSub, uint32_t nSub, uint64_t begin, uint64_t len) -> HcclResult {
+        if (len == 0) {
+            return HCCL_SUCCESS;
         }
-        HIP_OK(hipMalloc(reinterpret_cast<void**>(&w->slab), want));
-        w->slabHeld = want;
-    }
-    const uint64_t pieceEl = w->slabHeld / esz;
-    if (pieceEl == 0) {
-        return HCCL_E_INTERNAL;
-    }
-    for (uint64_t done = 0; done < p.count; done += pieceEl) {
-        const uint64_t len = std::min(pieceEl, p.count - done);
-        ReduceArgs r = flat;
-        for (uint32_t k = 0; k < n; ++k) {
-            r.src[k] = static_cast<const uint8_t*>(p.ranks[k].send) + done * esz;
+        ReduceArgs r = a;
+        for (uint32_t k = 0; k < w->n; ++k) {
+            r.src[k] = static_cast<const uint8_t*>(a.src[k]) + begin * esz;
+        }
+        for (uint32_t k = 0; k < static_cast<uint32_t>(kMaxRanks); ++k) {
             r.dst[k] = nullptr;
         }
-        r.dst[0] = w->slab;
+        uint8_t* first = static_cast<uint8_t*>(a.dst[0]) + begin * esz;
+        r.dst[0] = first;
         r.nDst = 1;
-        r.total = r.groupLen = r.subLen = len;
-        HcclResult rc = LaunchOneReduce(w, r, plan, p.dtype, p.op, s);
+        r.prog = a.prog + static_cast<uint64_t>(firstSub) * a.progSubStride * kDevProgBytes;
+        r.nSub = nSub;
+        r.total = r.groupLen = len;
+        if (nSub == 1) {
+            r.subLen = len;
+        }
+        HcclResult rc = LaunchOneReduce(w, r, plan, dtype, op, s);
         if (rc != HCCL_SUCCESS) {
             return rc;
         }
-        BcastCopyArgs b{};
+        FanOutArgs f{};
+        f.src = first;
+        f.bytes = len * esz;
+        f.nDst = a.nDst - 1;
+        for (uint32_t k = 1; k < a.nDst; ++k) {
+            f.dst[k - 1] = static_cast<uint8_t*>(a.dst[k]) + begin * esz;
+        }
+        if (FanOutTakes(f)) {
+            HIP_OK(LaunchFanOut(f, s));
+            return HCCL_SUCCESS;
+        }
+        BcastCopyArgs b{};   // recvBufs that differ modulo 16: the general copy
         b.nSeg = 1;
-        b.src[0] = w->slab;
-        b.len[0] = len * esz;
+        b.src[0] = first;
+        b.len[0] = f.bytes;
         b.dstOff[0] = 0;
-        b.nDst = n;
-        for (uint32_t k = 0; k < n; ++k) {
-            b.dst[k] = static_cast<uint8_t*>(p.ranks[k].recv) + done * esz;
+        b.nDst = f.nDst;
+        for (uint32_t k = 0; k < f.nDst; ++k) {
+            b.dst[k] = f.dst[k];
         }
-        rc = RunBcast(w, b, s, true);   // the slab has just been written
-        if (rc != HCCL_SUCCESS) {
-            return rc;
+        return RunBcast(w, b, s);
+    };
+    uint32_t heldFirst = 0;     // sub-segments [heldFirst, c) wait for their launch
+    uint64_t heldBegin = 0;
+    uint64_t heldLen = 0;
+    for (uint32_t c = 0; c < a.nSub; ++c) {
+        const uint64_t sBeg = static_cast<uint64_t>(c) * a.subLen;
+        uint64_t sEnd = (c == a.nSub - 1) ? a.total : sBeg + a.subLen;
+        sEnd = sEnd < a.total ? sEnd : a.total;
+        const uint64_t len = sEnd > sBeg ? sEnd - sBeg : 0;
+        if (heldLen + len > pieceEl && heldLen != 0) {
+            HcclResult rc = piece(heldFirst, c - heldFirst, heldBegin, heldLen);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+            heldLen = 0;
         }
+        if (len > pieceEl) {
+            for (uint64_t at = 0; at < len; at += pieceEl) {
+                HcclResult rc = piece(c, 1, sBeg + at, std::min(pieceEl, len - at));
+                if (rc != HCCL_SUCCESS) {
+                    return rc;
+                }
+            }
+            continue;
+        }
+        if (heldLen == 0) {
+            heldFirst = c;
+            heldBegin = sBeg;
+        }
+        heldLen += len;
+    }
+    if (heldLen != 0) {
+        return piece(heldFirst, a.nSub - heldFirst, heldBegin, heldLen);
     }
     return HCCL_SUCCESS;
 }
@@ -841,10 +886,7 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
     if (plan.nProg == 1) {
         a.total = a.groupLen = a.subLen = p.count;
         a.nSub = 1;
-        if (UseSlab(w, p.count * esz)) {
-            return RunAllReduceViaSlab(w, p, plan, a, s);
-        }
-        return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+        return LaunchToAll(w, a, plan, p.dtype, p.op, s);
     }
     if (algo == HCCL_AMD_ALGO_MESH_CHUNK) {
         // Slices of ceil(len / n) elements, short or empty towards the end (reference
@@ -897,7 +939,7 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
         }
         a.total = a.groupLen = len;
         a.subLen = unit;
-        return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+        return LaunchToAll(w, a, plan, p.dtype, p.op, s);
     };
     if (algo == HCCL_AMD_ALGO_RHD) {
         // Whole frames of n uniform units while they last, then a remainder shorter than n with one element per
@@ -1010,9 +1052,9 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
     return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
 }
 
-HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s, bool sourceIsHot)
+HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
 {
-    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s, w->copyDstPerGroup, sourceIsHot));   // 0: the launcher picks
+    HIP_OK(LaunchBcastCopy(b, w->copyTileBytes, s));   // 0: the launcher picks
     return HCCL_SUCCESS;
 }
 

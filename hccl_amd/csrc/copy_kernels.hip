@@ -41,28 +41,18 @@ typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
 // Payload pointers are rebuilt from integers; telling the compiler they are global memory keeps the
 // accesses off the flat path.
 //
-// Cache policies.  A tile that one wavefront moves on its own (SHARED == false) is loaded non-temporally and its
-// 16-byte vectors are written through at system scope, the fastest pair for one read and one write stream.  A
-// tile whose destinations are split over several wavefronts of the same XCD (SHARED == true) is loaded with a
-// plain load, so that the XCD's L2 serves the wavefronts that come after the first, and stored non-temporally
-// (the pair that measured best for that form).
-template <typename V, bool SHARED>
+// Cache policy: a tile is loaded non-temporally and its 16-byte vectors are written through at system scope, the
+// fastest pair for one read stream next to one or several write streams.
+template <typename V>
 __device__ __forceinline__ V LoadVec(const void* p)
 {
-    if constexpr (SHARED) {
-        return *((const __attribute__((address_space(1))) V*)p);
-    } else {
-        return __builtin_nontemporal_load((const __attribute__((address_space(1))) V*)p);
-    }
+    return __builtin_nontemporal_load((const __attribute__((address_space(1))) V*)p);
 }
-template <typename V, bool SHARED>
+template <typename V>
 __device__ __forceinline__ void StoreVec(V v, void* p)
 {
-    if constexpr (sizeof(V) == 16 && !SHARED) {
+    if constexpr (sizeof(V) == 16) {
         StoreStream16(p, __builtin_bit_cast(StreamVec, v));
-    } else if constexpr (sizeof(V) == 16) {
-        typedef V Unaligned __attribute__((aligned(1)));   // destinations may differ modulo 16 from the first
-        __builtin_nontemporal_store(v, (__attribute__((address_space(1))) Unaligned*)p);
     } else {
         __builtin_nontemporal_store(v, (__attribute__((address_space(1))) V*)p);
     }
@@ -194,17 +184,17 @@ __device__ __forceinline__ void Ready(uint32_t& v) { asm volatile("" : "+v"(v));
 // stores to destination 0 are 16-byte aligned; those to the other destinations are too when they share its
 // offset from a 16-byte boundary (the usual case) and are unaligned 128-bit stores otherwise.  Must be called
 // by all T threads of the workgroup.
-template <int T, int MODE, bool SHARED, int kBatch, bool kStatic, class PtrFn>
+template <int T, int MODE, int kBatch, bool kStatic, class PtrFn>
 __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uint32_t nDst, uint64_t dOff, uint32_t pace,
                                          PtrFn ptrOf)
 {
     const uint32_t idx = threadIdx.x;
     if (MODE == COPY_ALIGNED) {
         if (idx < bytes / 16u) {
-            U32x4 v = LoadVec<U32x4, SHARED>(reinterpret_cast<const U32x4*>(src) + idx);
+            U32x4 v = LoadVec<U32x4>(reinterpret_cast<const U32x4*>(src) + idx);
             Ready(v);
             ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
-                StoreVec<U32x4, SHARED>(v, reinterpret_cast<U32x4*>(dst) + idx);
+                StoreVec<U32x4>(v, reinterpret_cast<U32x4*>(dst) + idx);
             });
         }
         return;
@@ -220,7 +210,7 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
     U32x4 out = {0, 0, 0, 0};
     if (sMis == 0) {
         if (idx < nVec) {
-            out = LoadVec<U32x4, SHARED>(reinterpret_cast<const U32x4*>(sBody) + idx);
+            out = LoadVec<U32x4>(reinterpret_cast<const U32x4*>(sBody) + idx);
         }
     } else if (nVec != 0) {
         // Irregular: lane i loads the aligned vector i that covers the start of its output and takes
@@ -230,10 +220,10 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
         U32x4 a = {0, 0, 0, 0};
         U32x4 b = {0, 0, 0, 0};
         if (idx <= nVec) {
-            a = LoadVec<U32x4, SHARED>(s + idx);
+            a = LoadVec<U32x4>(s + idx);
         }
         if ((idx & 63u) == 63u && idx < nVec) {
-            b = LoadVec<U32x4, SHARED>(s + idx + 1);
+            b = LoadVec<U32x4>(s + idx + 1);
         }
         b = NextLane(a, b);
         const uint32_t shift = sMis & 3u;    // bytes to skip inside a dword
@@ -249,68 +239,46 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
     const uint32_t edgeAt = idx < head ? idx : bodyEnd + (idx - head);
     uint32_t edgeByte = 0;
     if (idx < edge) {
-        edgeByte = LoadVec<uint8_t, SHARED>(src + edgeAt);
+        edgeByte = LoadVec<uint8_t>(src + edgeAt);
     }
     Ready(out);
     Ready(edgeByte);
     if (idx < nVec) {
         ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
-            StoreVec<U32x4, SHARED>(out, reinterpret_cast<U32x4*>(dst + head) + idx);
+            StoreVec<U32x4>(out, reinterpret_cast<U32x4*>(dst + head) + idx);
         });
     }
     if (idx < edge) {
         ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
-            StoreVec<uint8_t, SHARED>(static_cast<uint8_t>(edgeByte), dst + edgeAt);
+            StoreVec<uint8_t>(static_cast<uint8_t>(edgeByte), dst + edgeAt);
         });
     }
 }
 
 // ---- AllGather / AllGatherV --------------------------------------------------------------------
-// Workgroup b copies tile b of the segment list held in the kernel arguments to every destination (SPLIT ==
-// false), or to one group of at most kMaxSplitDst destinations (SPLIT == true).  In the split form the grid is
-// (8 * groups, blocks of eight tiles): workgroup x of a row copies tile x % 8 of the row's eight tiles to group
-// x / 8.  Workgroups are dealt to the eight XCDs in turn, so the groups of one tile land on the same XCD within
-// a short time of each other and all but the first find the tile in its L2.
+// Workgroup b copies tile b of the segment list held in the kernel arguments to every destination.
 //
 // A wavefront has one 16-byte vector per lane in flight, so whatever it waits for before that load is issued is
-// lost bandwidth, the more so the fewer destinations it stores to.  Everything a wavefront needs therefore
-// comes in with two rounds of scalar loads of the kernel arguments: the first brings the tile prefixes (the tile
-// -> segment map is a branch-free count over them) and, in the split form, the group's destination pointers,
-// which the host has laid out by group; the second what the segment index selects.
-template <int T, int MODE, bool SPLIT>
+// lost bandwidth.  Everything a wavefront needs therefore comes in with two rounds of scalar loads of the kernel
+// arguments: the first brings the tile prefixes (the tile -> segment map is a branch-free count over them), the
+// second what the segment index selects.
+template <int T, int MODE>
 __global__ __launch_bounds__(T) void BcastCopyKernel(const BcastCopyArgs args)
 {
     constexpr uint32_t kTile = T * 16u;
     // First round: everything that does not depend on the segment.
-    uint32_t nTiles = args.nTiles;
     uint32_t nDst = args.nDst;
-    uint32_t dstPerGroup = args.dstPerGroup;
-    uint32_t superY = args.superY;
     uint32_t nSegPadded = args.nSegPadded;
     uint32_t ends[16];
 #pragma unroll
     for (uint32_t k = 0; k < 16; ++k) {
         ends[k] = args.tileEnd[k];
     }
-    uint64_t group[kMaxSplitDst] = {};
-    if constexpr (SPLIT) {
-#pragma unroll
-        for (uint32_t d = 0; d < kMaxSplitDst; ++d) {
-            group[d] = reinterpret_cast<uint64_t>(args.dst[(blockIdx.x >> 3) * kMaxSplitDst + d]);
-        }
-        static_assert(kMaxSplitDst == 4, "the fence below names every pointer of a group");
-        asm volatile("" : "+s"(group[0]), "+s"(group[1]), "+s"(group[2]), "+s"(group[3]));
-    }
-    asm volatile("" : "+s"(nTiles), "+s"(nDst), "+s"(dstPerGroup), "+s"(superY), "+s"(nSegPadded));
+    asm volatile("" : "+s"(nDst), "+s"(nSegPadded));
     asm volatile("" : "+s"(ends[0]), "+s"(ends[1]), "+s"(ends[2]), "+s"(ends[3]), "+s"(ends[4]), "+s"(ends[5]),
                       "+s"(ends[6]), "+s"(ends[7]), "+s"(ends[8]), "+s"(ends[9]), "+s"(ends[10]), "+s"(ends[11]),
                       "+s"(ends[12]), "+s"(ends[13]), "+s"(ends[14]), "+s"(ends[15]));
-    uint32_t tile = blockIdx.x;
-    if constexpr (SPLIT) {
-        tile = ((blockIdx.z * superY + blockIdx.y) << 3) + (blockIdx.x & 7u);
-        const uint32_t firstDst = (blockIdx.x >> 3) * dstPerGroup;
-        nDst = nDst - firstDst < dstPerGroup ? nDst - firstDst : dstPerGroup;
-    }
+    const uint32_t tile = blockIdx.x;
     // Number of segments that end at or before this tile = index of the tile's segment (prefixes past the last
     // segment hold 0xFFFFFFFF; empty segments repeat their predecessor's prefix and are skipped by the count).
     uint32_t seg = 0;
@@ -324,9 +292,6 @@ __global__ __launch_bounds__(T) void BcastCopyKernel(const BcastCopyArgs args)
             seg += EndsAtOrBefore(args.tileEnd[i + k], tile);
         }
     }
-    if (SPLIT && tile >= nTiles) {
-        return;   // the last row of eight tiles may be short
-    }
     const uint32_t segFirst = seg == 0 ? 0u : args.tileEnd[seg - 1];
     uint64_t len = args.len[seg];
     uint64_t srcBase = reinterpret_cast<uint64_t>(args.src[seg]);
@@ -338,12 +303,8 @@ __global__ __launch_bounds__(T) void BcastCopyKernel(const BcastCopyArgs args)
     TileRange<kTile>(tile - segFirst, lead, len, &off, &bytes);
     const uint8_t* src = reinterpret_cast<const uint8_t*>(srcBase + off);
     const uint64_t dOff = segDstOff + off;
-    if constexpr (SPLIT) {
-        CopyTile<T, MODE, true, kMaxSplitDst, true>(src, bytes, nDst, dOff, args.pace, [&](uint32_t d) { return group[d]; });
-    } else {
-        CopyTile<T, MODE, false, 8, false>(src, bytes, nDst, dOff, args.pace,
-                                           [&](uint32_t d) { return reinterpret_cast<uint64_t>(args.dst[d]); });
-    }
+    CopyTile<T, MODE, 8, false>(src, bytes, nDst, dOff, args.pace,
+                                [&](uint32_t d) { return reinterpret_cast<uint64_t>(args.dst[d]); });
 }
 
 // ---- AlltoAllV -------------------------------------------------------------------------------------
@@ -364,16 +325,16 @@ __global__ __launch_bounds__(T) void A2aCopyKernel(const A2aArgs args)
     uint32_t bytes;
     TileRange<kTile>(tile - static_cast<uint32_t>(desc[3]), TileLead(dstBase), len, &off, &bytes);
     const uint8_t* src = reinterpret_cast<const uint8_t*>(srcBase + off);
-    CopyTile<T, MODE, false, 1, true>(src, bytes, 1u, off, 3u, [&](uint32_t) { return dstBase; });
+    CopyTile<T, MODE, 1, true>(src, bytes, 1u, off, 3u, [&](uint32_t) { return dstBase; });
 }
 
-template <int T, bool SPLIT>
-hipError_t LaunchBcastT(const BcastCopyArgs& a, uint32_t mode, dim3 grid, hipStream_t stream)
+template <int T>
+hipError_t LaunchBcastT(const BcastCopyArgs& a, uint32_t mode, uint32_t tiles, hipStream_t stream)
 {
     switch (mode) {
-        case COPY_ALIGNED: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_ALIGNED, SPLIT>), grid, dim3(T), 0, stream, a); break;
-        case COPY_CONGRUENT: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_CONGRUENT, SPLIT>), grid, dim3(T), 0, stream, a); break;
-        default: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_GENERAL, SPLIT>), grid, dim3(T), 0, stream, a); break;
+        case COPY_ALIGNED: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_ALIGNED>), dim3(tiles), dim3(T), 0, stream, a); break;
+        case COPY_CONGRUENT: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_CONGRUENT>), dim3(tiles), dim3(T), 0, stream, a); break;
+        default: hipLaunchKernelGGL((BcastCopyKernel<T, COPY_GENERAL>), dim3(tiles), dim3(T), 0, stream, a); break;
     }
     return hipGetLastError();
 }
@@ -387,6 +348,49 @@ hipError_t LaunchA2aT(const A2aArgs& a, uint32_t tiles, hipStream_t stream)
         default: hipLaunchKernelGGL((A2aCopyKernel<T, COPY_GENERAL>), dim3(tiles), dim3(T), 0, stream, a); break;
     }
     return hipGetLastError();
+}
+
+// ---- fan-out of a cached range ------------------------------------------------------------------
+// Wavefront y of workgroup b copies tile b (64 vectors) of the source to destinations y * dstPerWave ... : one
+// plain load (the first wavefront of a tile brings it into the caches, the others find it there) and one
+// non-temporal store per destination.  A wavefront with a single store stream is the fastest way to write on this
+// part (sixteen streams from sixteen wavefronts: 0.89 of the HBM peak, all sixteen from one wavefront: 0.72), and
+// with next to no preamble the extra wavefronts cost little.  Source and destinations share their offset from a
+// 16-byte boundary: up to 15 bytes in front of the aligned body and up to 15 behind it move byte by byte, and
+// the body's vectors are dealt to the lanes shifted by `lead`, so that every wavefront covers whole 128-byte lines.
+constexpr uint32_t kFanOutWaves = 16;
+__global__ __launch_bounds__(64 * kFanOutWaves) void FanOutKernel(const FanOutArgs args)
+{
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const uint32_t first = wave * args.dstPerWave;
+    if (first >= args.nDst) {
+        return;
+    }
+    const uint32_t mine = args.nDst - first < args.dstPerWave ? args.nDst - first : args.dstPerWave;
+    const uint64_t srcAddr = reinterpret_cast<uint64_t>(args.src);
+    const uint32_t mis = static_cast<uint32_t>(srcAddr & 15u);
+    uint64_t head = mis ? 16u - mis : 0u;
+    head = head < args.bytes ? head : args.bytes;
+    const uint64_t nVec = (args.bytes - head) >> 4;
+    const uint32_t lead = static_cast<uint32_t>(((srcAddr + head) >> 4) & 7u);
+    const uint64_t u = static_cast<uint64_t>(blockIdx.x) * 64u + threadIdx.x;
+    if (u >= lead && u < nVec + lead) {
+        const uint64_t at = head + ((u - lead) << 4);
+        const U32x4 v = *((const __attribute__((address_space(1))) U32x4*)(srcAddr + at));
+        for (uint32_t d = 0; d < mine; ++d) {
+            __builtin_nontemporal_store(
+                v, (__attribute__((address_space(1))) U32x4*)(reinterpret_cast<uint64_t>(args.dst[first + d]) + at));
+        }
+    }
+    const uint64_t bodyEnd = head + (nVec << 4);
+    const uint32_t edge = static_cast<uint32_t>(head + (args.bytes - bodyEnd));   // < 32
+    if (blockIdx.x == 0 && threadIdx.x < edge) {
+        const uint64_t at = threadIdx.x < head ? threadIdx.x : bodyEnd + (threadIdx.x - head);
+        const uint8_t byte = *((const __attribute__((address_space(1))) uint8_t*)(srcAddr + at));
+        for (uint32_t d = 0; d < mine; ++d) {
+            *((__attribute__((address_space(1))) uint8_t*)(reinterpret_cast<uint64_t>(args.dst[first + d]) + at)) = byte;
+        }
+    }
 }
 
 // One argument-borne piece of a table image: words[0 .. nWords) go to table[firstWord ...].
@@ -467,53 +471,17 @@ hipError_t LaunchTableWrite(uint8_t* table, const uint64_t* image, uint32_t nWor
     return hipSuccess;
 }
 
-hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStream_t stream, uint32_t dstPerGroup,
-                           bool sourceIsHot)
+hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStream_t stream)
 {
     BcastCopyArgs a = in;
-    // Destinations split over wavefronts (two per wavefront up to sixteen destinations, four beyond; the tile is
-    // read once per group through L2) when the caller knows that the source is still in the last-level cache
-    // because it has just been written, and the range written in each destination stays within 256 MiB: the
-    // copy of a freshly folded slab to sixteen cold 256 MiB destinations runs at 0.80 of the HBM peak this way,
-    // against 0.66-0.72 with one wavefront per tile.  With a source that has to come from HBM the split form is
-    // the slower one (Broadcast of 128 MiB to 7 ranks over rotating buffer sets: 0.65 against 0.73; on buffers
-    // that are reused every step it reaches 0.9 and more, but that is the cache, not the memory), so sources of
-    // unknown state take the plain form.
-    if (dstPerGroup == 0) {
-        uint64_t lo = ~0ull, hi = 0;
-        for (uint32_t j = 0; j < a.nSeg; ++j) {
-            if (a.len[j] != 0) {
-                lo = a.dstOff[j] < lo ? a.dstOff[j] : lo;
-                hi = a.dstOff[j] + a.len[j] > hi ? a.dstOff[j] + a.len[j] : hi;
-            }
-        }
-        const bool compact = hi > lo && hi - lo <= kSplitMaxExtent;
-        dstPerGroup = (a.nDst <= 3 || !compact || !sourceIsHot) ? a.nDst : (a.nDst <= 16 ? 2u : 4u);
-    }
-    if (dstPerGroup > kMaxSplitDst && dstPerGroup < a.nDst) {
-        dstPerGroup = kMaxSplitDst;
-    }
-    if (dstPerGroup > a.nDst) {
-        dstPerGroup = a.nDst;
-    }
-    if (dstPerGroup == 0) {
+    if (a.nDst == 0 || a.nDst > static_cast<uint32_t>(kMaxRanks)) {
         return hipErrorInvalidValue;
     }
-    // the destination pointers of all groups, kMaxSplitDst slots each, must fit the argument array
-    while ((a.nDst + dstPerGroup - 1) / dstPerGroup * kMaxSplitDst > static_cast<uint32_t>(kMaxRanks)) {
-        ++dstPerGroup;
-    }
-    a.dstPerGroup = dstPerGroup;
-    a.nGroup = (a.nDst + dstPerGroup - 1) / dstPerGroup;
-    const bool split = a.nGroup > 1;
     uint64_t misfit = 0;      // non-zero low bits: something is not 16-byte aligned
-    bool congruent = true;    // every segment's source shares the offset of the first destination of every group
+    bool congruent = true;    // every segment's source shares the offset of the first destination
     const uint64_t dst0 = reinterpret_cast<uint64_t>(a.dst[0]);
     for (uint32_t d = 0; d < a.nDst; ++d) {
         misfit |= reinterpret_cast<uint64_t>(a.dst[d]);
-        if (d % dstPerGroup == 0) {
-            congruent = congruent && ((reinterpret_cast<uint64_t>(a.dst[d]) ^ dst0) & 15u) == 0;
-        }
     }
     for (uint32_t j = 0; j < a.nSeg; ++j) {
         if (a.len[j] != 0) {
@@ -526,7 +494,7 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
     if (tileBytes == 0) {
         // One wavefront per tile, except where lanes realign their source for several destinations: there the
         // larger workgroup measured 1-2 % faster.
-        tileBytes = (mode == COPY_GENERAL && a.nDst > 1 && !split) ? 4096u : 1024u;
+        tileBytes = (mode == COPY_GENERAL && a.nDst > 1) ? 4096u : 1024u;
     }
     uint64_t tiles = 0;
     for (uint32_t j = 0; j < a.nSeg; ++j) {
@@ -545,39 +513,45 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
     }
     a.nTiles = static_cast<uint32_t>(tiles);
     a.leadBase = dst0;
-    // A wavefront of the split form waits for each store before it issues the next; one that stores to every
-    // destination keeps two in flight (each measured best for its form; HCCL_AMD_COPY_PACE = 0..3 overrides).
+    // A wavefront issues a store when at most one earlier store is outstanding (measured best: 0.75 of the HBM
+    // peak against 0.72-0.74 with none or two outstanding, or without a limit); HCCL_AMD_COPY_PACE = 0..3 overrides.
     static const int paceEnv = getenv("HCCL_AMD_COPY_PACE") ? atoi(getenv("HCCL_AMD_COPY_PACE")) : -1;
-    a.pace = paceEnv >= 0 ? static_cast<uint32_t>(paceEnv) : (split ? 0u : 1u);
-    if (!split) {
-        const dim3 grid(a.nTiles);
-        switch (tileBytes) {
-            case 1024: return LaunchBcastT<64, false>(a, mode, grid, stream);
-            case 4096: return LaunchBcastT<256, false>(a, mode, grid, stream);
-            case 16384: return LaunchBcastT<1024, false>(a, mode, grid, stream);
-            default: return hipErrorInvalidValue;
-        }
-    }
-    // Destination pointers by group, kMaxSplitDst slots each; rows of eight tiles (one per XCD), every row
-    // repeated once per group along x.
-    if (a.nGroup * kMaxSplitDst > static_cast<uint32_t>(kMaxRanks)) {
-        return hipErrorInvalidValue;
-    }
-    for (uint32_t k = 0; k < static_cast<uint32_t>(kMaxRanks); ++k) {
-        a.dst[k] = nullptr;
-    }
-    for (uint32_t d = 0; d < a.nDst; ++d) {
-        a.dst[(d / dstPerGroup) * kMaxSplitDst + d % dstPerGroup] = in.dst[d];
-    }
-    const uint32_t supers = static_cast<uint32_t>((tiles + 7) / 8);
-    a.superY = supers < 32768u ? supers : 32768u;
-    const dim3 grid(8u * a.nGroup, a.superY, (supers + a.superY - 1) / a.superY);
+    a.pace = paceEnv >= 0 ? static_cast<uint32_t>(paceEnv) : 1u;
     switch (tileBytes) {
-        case 1024: return LaunchBcastT<64, true>(a, mode, grid, stream);
-        case 4096: return LaunchBcastT<256, true>(a, mode, grid, stream);
-        case 16384: return LaunchBcastT<1024, true>(a, mode, grid, stream);
+        case 1024: return LaunchBcastT<64>(a, mode, a.nTiles, stream);
+        case 4096: return LaunchBcastT<256>(a, mode, a.nTiles, stream);
+        case 16384: return LaunchBcastT<1024>(a, mode, a.nTiles, stream);
         default: return hipErrorInvalidValue;
     }
+}
+
+bool FanOutTakes(const FanOutArgs& args)
+{
+    if (args.nDst == 0 || args.nDst > static_cast<uint32_t>(kMaxRanks) || args.bytes == 0 ||
+        (args.bytes >> 10) + 2 > 0x7FFFFFFFull) {
+        return false;
+    }
+    for (uint32_t d = 0; d < args.nDst; ++d) {
+        if (((reinterpret_cast<uint64_t>(args.dst[d]) ^ reinterpret_cast<uint64_t>(args.src)) & 15u) != 0) {
+            return false;
+        }
+    }
+    return true;
+}
+
+hipError_t LaunchFanOut(const FanOutArgs& in, hipStream_t stream)
+{
+    if (!FanOutTakes(in)) {
+        return hipErrorInvalidValue;
+    }
+    FanOutArgs a = in;
+    a.dstPerWave = (a.nDst + kFanOutWaves - 1) / kFanOutWaves;
+    const uint32_t waves = (a.nDst + a.dstPerWave - 1) / a.dstPerWave;
+    // vectors of the body plus up to seven lanes skipped in front of it; at least one workgroup for the edge bytes
+    const uint64_t vecs = (a.bytes >> 4) + 7;
+    const uint32_t tiles = static_cast<uint32_t>((vecs + 63) / 64);
+    hipLaunchKernelGGL(FanOutKernel, dim3(tiles), dim3(64, waves), 0, stream, a);
+    return hipGetLastError();
 }
 
 hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, uint32_t tileBytes, hipStream_t stream)

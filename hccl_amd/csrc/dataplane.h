@@ -153,8 +153,6 @@ inline uint32_t BuildTileHints(const uint32_t* tileEnd, uint32_t nSeg, uint32_t 
 // once from src[j] and written to dst[d] + dstOff[j] for every d < nDst.  The caller fills the first six
 // members; LaunchBcastCopy derives the rest: tileEnd[j] = inclusive prefix sum of the segments' tile counts,
 // padded with 0xFFFFFFFF up to nSegPadded (a multiple of 16) entries.
-constexpr uint32_t kMaxSplitDst = 4;   // most destinations one wavefront stores to when a tile's destinations are split
-constexpr uint64_t kSplitMaxExtent = 256ull << 20;   // largest written range per destination the split form is used for
 struct BcastCopyArgs {
     const void* src[kMaxRanks];
     void* dst[kMaxRanks];
@@ -164,9 +162,6 @@ struct BcastCopyArgs {
     uint32_t nDst;
     uint32_t nSegPadded;
     uint32_t nTiles;
-    uint32_t dstPerGroup;   // destinations one wavefront stores to; nGroup = ceil(nDst / dstPerGroup) wavefronts per tile
-    uint32_t nGroup;        // when > 1, dst[] is laid out by group: group g's destinations at dst[g * kMaxSplitDst ...]
-    uint32_t superY;        // split form: rows of eight tiles along y before the grid continues along z
     uint64_t leadBase;      // address of the first destination: tiles are cut on its 128-byte lines
     uint32_t pace;          // stores of a wavefront that may be outstanding when it issues the next (3: no limit)
     uint32_t tileEnd[kMaxRanks];
@@ -218,10 +213,21 @@ inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
     // eight fp32 accumulators (half SUM) or sixteen 16-bit ones (int8) vs one 16-byte pack
     return ((half && op == HCCL_REDUCE_SUM) || dtype == HCCL_DATA_TYPE_INT8) ? 32u : 16u;
 }
-// tileBytes: 1024, 4096 or 16384; 0 lets the launcher choose.  dstPerGroup: destinations per wavefront, 0 lets
-// the launcher choose.  sourceIsHot: the source has just been written by the previous kernel on the stream.
-hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream, uint32_t dstPerGroup = 0,
-                           bool sourceIsHot = false);
+// tileBytes: 1024, 4096 or 16384; 0 lets the launcher choose.
+hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStream_t stream);
 hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, uint32_t tileBytes, hipStream_t stream);
+
+// One freshly written source range to nDst destinations that share its offset from a 16-byte boundary, a
+// workgroup of up to sixteen wavefronts per 1 KiB tile with a destination (beyond sixteen: a few) each.
+// FanOutTakes says whether the operands fit; the caller uses LaunchBcastCopy for those that do not.
+struct FanOutArgs {
+    const void* src;
+    void* dst[kMaxRanks];
+    uint64_t bytes;
+    uint32_t nDst;
+    uint32_t dstPerWave;
+};
+bool FanOutTakes(const FanOutArgs& args);
+hipError_t LaunchFanOut(const FanOutArgs& args, hipStream_t stream);
 
 }  // namespace hccl_amd

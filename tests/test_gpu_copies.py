@@ -90,19 +90,13 @@ def test_all_to_all_v(n, aligned):
         w.close()
 
 
-@pytest.mark.parametrize("per_wave", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("n", [4, 7, 17, 64])
-def test_all_gather_v_with_destinations_split_over_wavefronts(monkeypatch, n, per_wave):
-    """The copy kernel's split form (every tile copied by several wavefronts, each storing to a few
-    destinations): group sizes 1 to 4 and the launcher's own choice, destination counts that leave a short last
-    group, segments that end inside a row of eight tiles, odd element displacements, differently aligned
-    buffers, empty segments."""
-    if per_wave:
-        monkeypatch.setenv("HCCL_AMD_COPY_DST_PER_WAVE", str(per_wave))
+def test_all_gather_v_ragged_segments_many_destinations(n):
+    """AllGatherV over destination counts from 4 to 64: segments that end inside a tile, odd element
+    displacements, differently aligned buffers, empty segments."""
     w = World(n)
-    monkeypatch.delenv("HCCL_AMD_COPY_DST_PER_WAVE", raising=False)
     try:
-        rng = np.random.default_rng(5000 + 10 * n + per_wave)
+        rng = np.random.default_rng(5000 + 10 * n)
         esz = 2
         for trial in range(3):
             counts = rng.integers(0, 9_000 if n <= 17 else 1_500, n).astype(np.uint64)
@@ -122,14 +116,14 @@ def test_all_gather_v_with_destinations_split_over_wavefronts(monkeypatch, n, pe
             recvs = [dev_zeros(total * esz, pad_front=0 if trial != 1 else 2 * (r % 5), fill=FILL) for r in range(n)]
             w.all_gather_v(sends, recvs, counts, displs, DT.FP16)
             for r in range(n):
-                assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), (n, per_wave, trial, r)
+                assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), (n, trial, r)
     finally:
         w.close()
 
 
-def test_broadcast_and_all_gather_beyond_the_split_form_s_extent():
-    """Destinations written over more than 256 MiB take the plain form of the copy kernel; checked by equality
-    with the source on the device (512 MiB broadcast to 4 ranks, AllGather of 5 x 80 MiB)."""
+def test_broadcast_and_all_gather_of_half_a_gigabyte():
+    """Large one-to-many copies, checked by equality with the source on the device (512 MiB broadcast to 4 ranks,
+    AllGather of 5 x 80 MiB)."""
     import torch
     n, nbytes = 5, 512 << 20
     w = World(n)

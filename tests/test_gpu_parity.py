@@ -365,15 +365,17 @@ def test_workgroups_that_loop_over_several_positions(monkeypatch):
         w.close()
 
 
-@pytest.mark.parametrize("n", [2, 5, 16])
-def test_all_reduce_through_the_staging_slab(monkeypatch, n):
-    """The two-kernel form of the rank-order AllReduce (fold into a slab, slab to every recvBuf), forced for
-    small messages with a slab of 4 KiB so that counts span several pieces and end in a ragged one."""
-    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB", "1")
-    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB_BYTES", "4096")
+@pytest.mark.parametrize("n", [2, 5, 16, 33])
+def test_all_reduce_as_fold_and_fan_out(monkeypatch, n):
+    """The two-kernel form of AllReduce (fold into the first recvBuf, that range to the other recvBufs with a
+    wavefront per destination), forced for small messages with pieces of 4 KiB: counts that span several pieces and
+    end in a ragged one, orders with a fold program per sub-segment (pieces of whole sub-segments, and parts of a
+    sub-segment that is longer than a piece), recvBufs that share their misalignment and recvBufs that do not."""
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "1")
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_PIECE_BYTES", "4096")
     w = World(n)
-    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB")
-    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB_BYTES")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_PIECE_BYTES")
     try:
         seed = 2000 + n
         for dtype in REDUCE_TYPES:
@@ -382,10 +384,17 @@ def test_all_reduce_through_the_staging_slab(monkeypatch, n):
                 seed += 1
         run_all_reduce(w, DT.INT32, PROD, 17, "mesh", seed=seed)            # less than one piece
         run_all_reduce(w, DT.FP32, SUM, 1_024, "ring", seed=seed + 1)       # exactly one piece
-        run_all_reduce(w, DT.FP32, SUM, 65_543, "ring", seed=seed + 2, pad=4)
+        run_all_reduce(w, DT.FP32, SUM, 65_543, "ring", seed=seed + 2, pad=4)   # every buffer 4 bytes off: shared misalignment
         run_all_reduce(w, DT.BFP16, SUM, 10_007, "mesh", seed=seed + 3, pad=lambda r, which: 2 * r + (6 if which == "recv" else 0))
         run_all_reduce(w, DT.FP16, MIN, 9_001, "mesh", seed=seed + 4, in_place=True)
-        run_all_reduce(w, DT.FP32, SUM, 5_000, "rhd", seed=seed + 5)        # tree orders keep the fused kernel
+        run_all_reduce(w, DT.FP32, SUM, 5_000, "rhd", seed=seed + 5)        # sub-segments shorter than a piece
+        run_all_reduce(w, DT.FP16, SUM, 70_001, "rhd", seed=seed + 6)       # remainder frame after the whole frames
+        run_all_reduce(w, DT.BFP16, SUM, 50_003, "nhr", seed=seed + 7, pad=2)
+        run_all_reduce(w, DT.INT32, SUM, 200_003, "nhr", seed=seed + 8)     # sub-segments longer than a piece
+        run_all_reduce(w, DT.FP32, SUM, 33_333, "order_preserved", seed=seed + 9)
+        run_all_reduce(w, DT.FP32, MAX, 20_011, "mesh_symmetric", seed=seed + 11, in_place=True)
+        run_all_reduce(w, DT.INT8, SUM, 30_011, "mesh_chunk", seed=seed + 12)   # keeps the fused kernel
+        run_all_reduce(w, DT.INT8, SUM, 3, "nhr", seed=seed + 13)           # fewer elements than ranks
     finally:
         w.close()
 
@@ -393,13 +402,13 @@ def test_all_reduce_through_the_staging_slab(monkeypatch, n):
 @pytest.mark.parametrize("n,waves", [(2, 2), (5, 2), (6, 3), (8, 4), (16, 4), (3, 4)])
 def test_all_reduce_with_the_stores_of_a_tile_shared_by_wavefronts(monkeypatch, n, waves):
     """The many-destination form of the fused kernel (wavefront 0 folds a tile, `waves` wavefronts store it),
-    forced for small messages; a slab never steps in, and a small grid makes every workgroup loop over tiles."""
+    forced for small messages and with the two-kernel form off; a small grid makes every workgroup loop over tiles."""
     monkeypatch.setenv("HCCL_AMD_REDUCE_STORE_WAVES", str(waves))
-    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB", "0")
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "0")
     monkeypatch.setenv("HCCL_AMD_REDUCE_BLOCKS", "24")
     w = World(n)
     monkeypatch.delenv("HCCL_AMD_REDUCE_STORE_WAVES")
-    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS")
     monkeypatch.delenv("HCCL_AMD_REDUCE_BLOCKS")
     try:
         seed = 5200 + 10 * n + waves
@@ -417,15 +426,16 @@ def test_all_reduce_with_the_stores_of_a_tile_shared_by_wavefronts(monkeypatch, 
         w.close()
 
 
-def test_slab_all_reduce_can_be_captured_into_a_graph(monkeypatch):
-    """Once the slab exists (one eager call of that size) the two-kernel AllReduce is launches only."""
+def test_two_kernel_all_reduce_can_be_captured_into_a_graph(monkeypatch):
+    """Once its fold program is on the device (one eager call of the same kind) the fold + fan-out AllReduce is
+    kernel launches only."""
     import torch
-    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB", "1")
-    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_SLAB_BYTES", "65536")
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "1")
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_PIECE_BYTES", "65536")
     n, count = 8, 40_003
     w = World(n)
-    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB")
-    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_SLAB_BYTES")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_PIECE_BYTES")
     try:
         rng = np.random.default_rng(4343)
         host = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]

@@ -77,8 +77,12 @@ def run_ranks(nranks, body):
 
 
 def zeros(nbytes):
+    """A cleared device buffer; the fill (on torch's current stream) has finished when this returns, so that a
+    collective on another stream, possibly a peer's, cannot be overtaken by it."""
     import torch
-    return torch.zeros(max(nbytes, 1), dtype=torch.uint8, device="cuda")
+    t = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device="cuda")
+    torch.cuda.current_stream().synchronize()
+    return t
 
 
 @pytest.mark.parametrize("collective", GOLD["reduce_op_suite"]["collectives"])
