@@ -20,6 +20,21 @@ def _native_library():
     require_library_on_gpu()
 
 
+FORMS = ["by_size", "two_kernels"]
+
+
+def world_with_form(monkeypatch, n, form):
+    """A world whose one-to-many copies take the launcher's choice, or the two-kernel form (segments into the
+    first destination, then a fan-out of that range) with windows of 4 KiB whatever the size."""
+    if form == "two_kernels":
+        monkeypatch.setenv("HCCL_AMD_COPY_TWO_KERNELS", "1")
+        monkeypatch.setenv("HCCL_AMD_ALLREDUCE_PIECE_BYTES", "4096")
+    w = World(n)
+    monkeypatch.delenv("HCCL_AMD_COPY_TWO_KERNELS", raising=False)
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_PIECE_BYTES", raising=False)
+    return w
+
+
 @pytest.mark.parametrize("n", [1, 2, 3, 8, 64])
 @pytest.mark.parametrize("dtype,esz", [(DT.UINT8, 1), (DT.BFP16, 2), (DT.FP32, 4), (DT.INT64, 8)])
 def test_all_gather(n, dtype, esz):
@@ -39,9 +54,10 @@ def test_all_gather(n, dtype, esz):
         w.close()
 
 
+@pytest.mark.parametrize("form", FORMS)
 @pytest.mark.parametrize("n", [2, 6, 8, 64])
-def test_all_gather_v_unordered_holes_and_odd_offsets(n):
-    w = World(n)
+def test_all_gather_v_unordered_holes_and_odd_offsets(monkeypatch, n, form):
+    w = world_with_form(monkeypatch, n, form)
     try:
         rng = np.random.default_rng(n)
         esz = 2
@@ -90,11 +106,13 @@ def test_all_to_all_v(n, aligned):
         w.close()
 
 
+@pytest.mark.parametrize("form", FORMS)
 @pytest.mark.parametrize("n", [4, 7, 17, 64])
-def test_all_gather_v_ragged_segments_many_destinations(n):
+def test_all_gather_v_ragged_segments_many_destinations(monkeypatch, n, form):
     """AllGatherV over destination counts from 4 to 64: segments that end inside a tile, odd element
-    displacements, differently aligned buffers, empty segments."""
-    w = World(n)
+    displacements, differently aligned buffers (the two-kernel form then falls back to one kernel), empty
+    segments."""
+    w = world_with_form(monkeypatch, n, form)
     try:
         rng = np.random.default_rng(5000 + 10 * n)
         esz = 2
@@ -247,12 +265,13 @@ def test_one_host_thread_per_rank_with_own_streams():
         assert np.array_equal(results[r].view(np.uint32), want.view(np.uint32)), r
 
 
-def test_all_gather_and_broadcast_into_differently_aligned_buffers():
+@pytest.mark.parametrize("form", FORMS)
+def test_all_gather_and_broadcast_into_differently_aligned_buffers(monkeypatch, form):
     """Every rank's buffers sit at their own offset from a 16-byte boundary: the stores to all but the first
     destination are unaligned 128-bit stores."""
     import hccl_amd
     n, count = 6, 33_333
-    w = World(n)
+    w = world_with_form(monkeypatch, n, form)
     try:
         rng = np.random.default_rng(404)
         ins = [rand_bytes(rng, count * 2) for _ in range(n)]
@@ -283,12 +302,13 @@ def test_all_gather_and_broadcast_into_differently_aligned_buffers():
         w.close()
 
 
+@pytest.mark.parametrize("form", FORMS)
 @pytest.mark.parametrize("n,count", [(4, 10_001), (8, 65_536)])
-def test_all_gather_with_the_send_buffer_inside_the_receive_buffer(n, count):
+def test_all_gather_with_the_send_buffer_inside_the_receive_buffer(monkeypatch, n, count, form):
     """Every rank sends the slice of its own recvBuf where its contribution belongs (the entry point puts no
     restriction on overlapping buffers, reference all_gather.cc:118-149): the own slot is copied onto itself."""
     import torch
-    w = World(n)
+    w = world_with_form(monkeypatch, n, form)
     try:
         rng = np.random.default_rng(n + count)
         parts = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]
@@ -300,5 +320,47 @@ def test_all_gather_with_the_send_buffer_inside_the_receive_buffer(n, count):
         want = np.concatenate(parts)
         for r in range(n):
             assert np.array_equal(recvs[r].cpu().numpy().view(np.uint32), want.view(np.uint32)), r
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("n", [3, 8, 20])
+def test_one_to_many_copies_as_gather_and_fan_out(monkeypatch, n):
+    """The two-kernel form with buffers that share an offset of 4 bytes from a 16-byte boundary (the fan-out
+    moves the bytes in front of and behind its aligned body one by one): AllGather over many windows, Broadcast
+    from every kind of root, AllGatherV with adjacent and separate destination ranges."""
+    w = world_with_form(monkeypatch, n, "two_kernels")
+    try:
+        rng = np.random.default_rng(900 + n)
+        count = 3_001
+        ins = [rand_bytes(rng, count * 4) for _ in range(n)]
+        want = [np.zeros(n * count * 4, dtype=np.uint8) for _ in range(n)]
+        assert oracle.all_gather(ins, want, count, int(DT.FP32)) == 0
+        sends = [to_dev(x, 4) for x in ins]
+        recvs = [dev_zeros(n * count * 4, 4) for _ in range(n)]
+        w.all_gather(sends, recvs, count, DT.FP32)
+        for r in range(n):
+            assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), ("all_gather", r)
+        for root, nbytes in ((0, 70_001), (n - 1, 5), (n // 2, 4_096), (1, 12_288)):
+            bufs = [to_dev(rand_bytes(rng, nbytes), 4) for _ in range(n)]
+            src = to_host(bufs[root], np.uint8)
+            w.broadcast(bufs, nbytes, DT.UINT8, root)
+            for r in range(n):
+                assert np.array_equal(to_host(bufs[r], np.uint8), src), ("broadcast", root, nbytes, r)
+        counts = rng.integers(1, 3_000, n).astype(np.uint64)
+        displs = np.zeros(n, dtype=np.uint64)
+        off = 0
+        for j in range(n):                       # adjacent ranges, a gap after every third
+            displs[j] = off
+            off += int(counts[j]) + (7 if j % 3 == 2 else 0)
+        total = off + 9
+        vins = [rand_bytes(rng, int(c) * 2) for c in counts]
+        vwant = [np.full(total * 2, FILL, dtype=np.uint8) for _ in range(n)]
+        assert oracle.all_gather_v(vins, vwant, counts, displs, int(DT.BFP16)) == 0
+        sends = [to_dev(x, 2 * (r % 3)) for r, x in enumerate(vins)]
+        recvs = [dev_zeros(total * 2, 4, fill=FILL) for _ in range(n)]
+        w.all_gather_v(sends, recvs, counts, displs, DT.BFP16)
+        for r in range(n):
+            assert np.array_equal(to_host(recvs[r], np.uint8), vwant[r]), ("all_gather_v", r)
     finally:
         w.close()
