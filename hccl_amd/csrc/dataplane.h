@@ -218,14 +218,13 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& args, uint32_t tileBytes, hipStr
 hipError_t LaunchA2aCopy(const A2aArgs& args, uint32_t nTiles, uint32_t tileBytes, hipStream_t stream);
 
 // One freshly written source range to nDst destinations that share its offset from a 16-byte boundary, a
-// workgroup of up to sixteen wavefronts per 1 KiB tile with a destination (beyond sixteen: a few) each.
-// FanOutTakes says whether the operands fit; the caller uses LaunchBcastCopy for those that do not.
+// workgroup of up to sixteen wavefronts per 1 KiB tile with a destination each (more destinations: several
+// launches).  FanOutTakes says whether the operands fit; the caller uses LaunchBcastCopy for those that do not.
 struct FanOutArgs {
     const void* src;
     void* dst[kMaxRanks];
     uint64_t bytes;
     uint32_t nDst;
-    uint32_t dstPerWave;
 };
 bool FanOutTakes(const FanOutArgs& args);
 hipError_t LaunchFanOut(const FanOutArgs& args, hipStream_t stream);
