@@ -393,7 +393,9 @@ def test_all_reduce_as_fold_and_fan_out(monkeypatch, n):
         run_all_reduce(w, DT.INT32, SUM, 200_003, "nhr", seed=seed + 8)     # sub-segments longer than a piece
         run_all_reduce(w, DT.FP32, SUM, 33_333, "order_preserved", seed=seed + 9)
         run_all_reduce(w, DT.FP32, MAX, 20_011, "mesh_symmetric", seed=seed + 11, in_place=True)
-        run_all_reduce(w, DT.INT8, SUM, 30_011, "mesh_chunk", seed=seed + 12)   # keeps the fused kernel
+        run_all_reduce(w, DT.INT8, SUM, 30_011, "mesh_chunk", seed=seed + 12)   # pieces of whole slices
+        run_all_reduce(w, DT.FP32, SUM, 257, "mesh_chunk", seed=seed + 14)      # slices shorter than a piece, short last slice
+        run_all_reduce(w, DT.BFP16, SUM, 3 * n + 1, "mesh_chunk", seed=seed + 15, pad=2)
         run_all_reduce(w, DT.INT8, SUM, 3, "nhr", seed=seed + 13)           # fewer elements than ranks
     finally:
         w.close()
@@ -542,11 +544,18 @@ def test_all_reduce_follows_staging_buffer_loops(n, algo):
         w.close()
 
 
+@pytest.mark.parametrize("two_kernels", [False, True])
 @pytest.mark.parametrize("n", [2, 3, 8, 16])
-def test_mesh_chunk_order_with_aligned_segments_and_staging_loops(n):
+def test_mesh_chunk_order_with_aligned_segments_and_staging_loops(monkeypatch, n, two_kernels):
     """Slices long enough for the 4 KiB rule, odd sizes, several types; then the executor's loops, which cut
-    every loop's share into segments of its own."""
+    every loop's share into segments of its own.  Also with the AllReduce forced into fold + fan-out over pieces of
+    64 KiB (pieces of whole slices; slices longer than a piece keep the fused kernel)."""
+    if two_kernels:
+        monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "1")
+        monkeypatch.setenv("HCCL_AMD_ALLREDUCE_PIECE_BYTES", "65536")
     w = World(n)
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", raising=False)
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_PIECE_BYTES", raising=False)
     try:
         for dtype, c in ((DT.FP32, 100_000), (DT.FP32, 7 * 1024 * (n - 1) - 1), (DT.BFP16, 300_001), (DT.INT8, 77_777),
                          (DT.FP16, 65_536)):
