@@ -139,11 +139,13 @@ def test_all_gather_v_ragged_segments_many_destinations(monkeypatch, n, form):
         w.close()
 
 
-def test_broadcast_and_all_gather_of_half_a_gigabyte():
-    """Large one-to-many copies, checked by equality with the source on the device (512 MiB broadcast to 4 ranks,
-    AllGather of 5 x 80 MiB)."""
+@pytest.mark.parametrize("n", [5, 9])
+def test_broadcast_and_all_gather_of_half_a_gigabyte(n):
+    """Large one-to-many copies, checked by equality with the source on the device (512 MiB broadcast to n - 1
+    ranks, AllGather of n x 80 MiB): one kernel for five ranks, gather + fan-out over several 256 MiB windows for
+    nine."""
     import torch
-    n, nbytes = 5, 512 << 20
+    nbytes = 512 << 20
     w = World(n)
     try:
         g = torch.Generator(device="cuda")
