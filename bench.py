@@ -29,7 +29,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 SEED = 0xC0FFEE
 CONFIGS = ("c1", "c2", "c3max", "c3prod", "c4", "c5a", "c5b")
-EXTRA = ("rsv", "reduce", "bcast", "scatter", "a2a")
+EXTRA = ("rsv", "reduce", "bcast", "ag", "scatter", "a2a")
 
 
 def parse_args():
@@ -252,6 +252,25 @@ class Workloads:
                     h.broadcast(comms[r], bufs[k][r], count, h.HcclDataType.UINT8, root, stream)
 
         return step, n * count, count, 1.0, bufs, "Broadcast rankSize=8 128 MiB, 4 buffer sets in rotation", "u8", n, "mesh"
+
+    def ag(self, algo):
+        """AllGather bf16, 16 ranks, 32 Mi elements (64 MiB) from every rank: 1 GiB into every recvBuf."""
+        t, h = self.torch, self.h
+        n, count = 16, 1 << 25
+        comms = self.world(n)
+        sends = [t.randint(-32768, 32767, (count,), generator=self.gen(SEED + 6600 + r), device="cuda", dtype=t.int16)
+                 for r in range(n)]
+        recvs = [t.empty(n * count, dtype=t.int16, device="cuda") for _ in range(n)]
+        stream = self.stream
+
+        def step():
+            with h.group():
+                for r in range(n):
+                    h.all_gather(comms[r], sends[r], recvs[r], count, h.HcclDataType.BFP16, stream)
+
+        total = n * count * 2
+        return step, (1 + n) * total, total, (n - 1) / n, (sends, recvs), \
+            "AllGather bf16 rankSize=16 32Mi el/rank", "u8", n, "mesh"
 
     def scatter(self, algo):
         t, h = self.torch, self.h
