@@ -32,10 +32,30 @@ def pick_count(rng):
     return int(rng.integers(5_000, 120_000))
 
 
+FORMS = {
+    "by_size": {},
+    # AllReduce as fold + fan-out whatever the size, pieces of a few KiB
+    "two_kernels": {"HCCL_AMD_ALLREDUCE_TWO_KERNELS": "1", "HCCL_AMD_ALLREDUCE_PIECE_BYTES": None},
+    # the fused kernel with a tile's stores shared by wavefronts, on a grid so small that workgroups loop
+    "shared_stores": {"HCCL_AMD_ALLREDUCE_TWO_KERNELS": "0", "HCCL_AMD_REDUCE_STORE_WAVES": None,
+                      "HCCL_AMD_REDUCE_BLOCKS": "40"},
+}
+
+
+@pytest.mark.parametrize("form", list(FORMS))
 @pytest.mark.parametrize("n", [2, 3, 4, 6, 7, 8, 12, 16])
-def test_random_reduce_cases(n):
+def test_random_reduce_cases(monkeypatch, n, form):
     rng = np.random.default_rng(90_000 + n)
+    env = dict(FORMS[form])
+    if "HCCL_AMD_ALLREDUCE_PIECE_BYTES" in env:
+        env["HCCL_AMD_ALLREDUCE_PIECE_BYTES"] = str([4096, 20_480, 65_536][n % 3])
+    if "HCCL_AMD_REDUCE_STORE_WAVES" in env:
+        env["HCCL_AMD_REDUCE_STORE_WAVES"] = str(2 + n % 3)
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
     w = World(n)
+    for k in env:
+        monkeypatch.delenv(k)
     try:
         for case in range(28):
             dtype = TYPES[rng.integers(0, len(TYPES))]
