@@ -602,7 +602,7 @@ HcclResult PrepareNoAlloc(World* w)
 // ---------------------------------------------------------------------------------------------
 uint32_t BlocksPerSub(const World* w, uint64_t subLen, uint32_t esz, uint64_t nSubTotal, uint32_t threads)
 {
-    uint64_t vecs = (subLen * esz + 15) / 16 + 7;   // the kernel skips up to 7 lanes to start on a 128-byte line
+    uint64_t vecs = (subLen * esz + 15) / 16 + kReduceLeadMask;   // lanes the kernel may skip to start on a 1 KiB boundary
     uint64_t maxUseful = (vecs + threads - 1) / threads;
     if (maxUseful == 0) maxUseful = 1;
     uint64_t want = (w->reduceBlocks + nSubTotal - 1) / nSubTotal;

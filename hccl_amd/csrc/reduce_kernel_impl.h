@@ -638,8 +638,9 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     // body follows, and fewer than W elements remain.  Sources and further destinations only need element
     // alignment: their 128-bit accesses may be unaligned (full speed when they are congruent with the first
     // destination, up to 15 % less otherwise).  Without vecOk everything goes element by element.  The body's vectors are dealt to the lanes shifted by `lead`, so that lane 0
-    // of every wavefront starts a 128-byte line (a wavefront whose 1 KiB straddles nine lines moves two of them
-    // twice): of the destination, or with leadFromSrc of the sources.
+    // of every wavefront starts a 1 KiB boundary (a wavefront whose 1 KiB straddles nine lines moves two of them
+    // twice, and one that starts on a line but off the 1 KiB grid still loads slower): of the destination, or
+    // with leadFromSrc of the sources.
     uint64_t head = len;
     uint64_t nVec = 0;
     uint32_t lead = 0;
@@ -654,7 +655,7 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
         const uint64_t lineOf = args.leadFromSrc
                                     ? reinterpret_cast<uint64_t>(args.src[0]) + (srcOff + head) * sizeof(S)
                                     : addr + head * sizeof(S);
-        lead = static_cast<uint32_t>((lineOf >> 4) & 7u);
+        lead = static_cast<uint32_t>((lineOf >> 4) & kReduceLeadMask);
     }
     const uint64_t bodyEnd = head + nVec * W;
     const uint64_t nScalar = head + (len - bodyEnd);
