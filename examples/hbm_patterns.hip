@@ -124,17 +124,17 @@ __global__ __launch_bounds__(64) void FoldToFirst(Bufs b, size_t first)
 // `source` to the destinations firstDst, firstDst + 1, ...: wavefront w of the workgroup takes destinations
 // firstDst + w, firstDst + w + W, ... below N.  HOT: the source has just been written (plain load, non-temporal
 // stores); otherwise it comes from memory (non-temporal load, stores written through).
-template <int N, int W, bool HOT>
+template <int N, int W, int HOT>
 __global__ __launch_bounds__(64 * W) void FanOut(Bufs b, const U4* source, int firstDst, size_t first)
 {
     const unsigned wave = threadIdx.x >> 6;
     const size_t idx = first + static_cast<size_t>(blockIdx.x) * 64 + (threadIdx.x & 63u);
-    const U4 v = HOT ? LoadPlain(source + idx) : LoadNt(source + idx);
+    const U4 v = HOT ? LoadPlain(source + idx) : LoadNt(source + idx);   // HOT == 2: source from memory through the caches
 #pragma unroll
     for (int i = 0; i < (N + W - 1) / W; ++i) {
         const int d = firstDst + static_cast<int>(wave) + W * i;
         if (d < N) {
-            Store<HOT ? 0 : 1>(v, b.dst[d] + idx);
+            Store<HOT == 1 ? 0 : 1>(v, b.dst[d] + idx);
         }
     }
 }
@@ -189,7 +189,7 @@ void FoldFanRow(const Bufs& b, size_t nVec, size_t pieceMiB, bool twoStreams, hi
                 CK(hipEventRecord(folded[k % 64], 0));
                 CK(hipStreamWaitEvent(other, folded[k % 64], 0));
             }
-            hipLaunchKernelGGL((FanOut<N, W, true>), dim3(blocks), dim3(64 * W), 0, twoStreams ? other : 0, b, b.dst[0], 1, first);
+            hipLaunchKernelGGL((FanOut<N, W, 1>), dim3(blocks), dim3(64 * W), 0, twoStreams ? other : 0, b, b.dst[0], 1, first);
         }
         if (twoStreams) {
             CK(hipEventRecord(joined, other));
@@ -237,10 +237,16 @@ void Run(size_t bytesPerRank)
     int pass = 0;
     const double moved = (1.0 + N) * bytesPerRank;
     Report(N, "1 source to N destinations, one wavefront per tile", MsPerPass([&] {
-               hipLaunchKernelGGL((FanOut<N, 1, false>), dim3(blocks), dim3(64), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
+               hipLaunchKernelGGL((FanOut<N, 1, 0>), dim3(blocks), dim3(64), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
            }), moved);
     Report(N, "1 source to N destinations, two wavefronts per tile", MsPerPass([&] {
-               hipLaunchKernelGGL((FanOut<N, 2, false>), dim3(blocks), dim3(128), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
+               hipLaunchKernelGGL((FanOut<N, 2, 0>), dim3(blocks), dim3(128), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
+           }), moved);
+    Report(N, "1 source to N destinations, three wavefronts per tile, cached loads", MsPerPass([&] {
+               hipLaunchKernelGGL((FanOut<N, 3, 2>), dim3(blocks), dim3(192), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
+           }), moved);
+    Report(N, "1 source to N destinations, one wavefront per destination, cached loads", MsPerPass([&] {
+               hipLaunchKernelGGL((FanOut<N, N, 2>), dim3(blocks), dim3(64 * N), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
            }), moved);
     for (int i = 0; i < N; ++i) {
         CK(hipFree((void*)b.src[i]));
