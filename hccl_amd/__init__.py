@@ -111,7 +111,12 @@ def lib():
         return _lib
     if not os.path.exists(LIB_PATH):
         raise ImportError("%s is missing: run `make -C hccl_amd/csrc` (or hccl_amd.build()) first" % LIB_PATH)
-    L = ctypes.CDLL(LIB_PATH)
+    _lib = _bind(ctypes.CDLL(LIB_PATH))
+    return _lib
+
+
+def _bind(L):
+    """Declares the argument and result types of the library's entry points on the loaded library L."""
     vp, u64, u32, i32 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_int
     L.HcclAllReduce.argtypes = [vp, vp, u64, i32, i32, vp, vp]
     L.HcclReduceScatter.argtypes = [vp, vp, u64, i32, i32, vp, vp]
@@ -153,7 +158,6 @@ def lib():
                  "HcclAmdGetFoldProgram", "HcclAmdSetCclBufferSize", "HcclAmdGetCclBufferSize",
                  "HcclAmdAlltoAllVNoAlloc", "HcclAmdGetStuckCounters"):
         getattr(L, name).restype = ctypes.c_int
-    _lib = L
     return L
 
 

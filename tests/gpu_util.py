@@ -2,11 +2,74 @@
 allocations, driven through the C ABI exactly as a single-threaded caller would (one call per rank
 inside a group, all on one non-default stream)."""
 import ctypes
+import os
 
 import numpy as np
 
 import hccl_amd
 from hccl_amd import Algo, OpKind
+
+# HCCL_AMD_TEST_EMU=1 (set by tests/test_emulated_kernels.py for the pytest run it starts, never on the GPU box):
+# the same tests drive the CPU emulation build of the library (tests/emu) with host buffers, so that the kernels'
+# index arithmetic runs where AddressSanitizer and a debugger can see it.  conftest.py has then replaced the
+# library the Python mirror calls.
+EMU = os.environ.get("HCCL_AMD_TEST_EMU") == "1"
+_libc = ctypes.CDLL(None)
+_libc.malloc.restype = ctypes.c_void_p
+_libc.malloc.argtypes = [ctypes.c_size_t]
+_libc.free.argtypes = [ctypes.c_void_p]
+
+
+class HostBuf:
+    """A malloc'ed block of the bytes asked for, rounded up to whole 16-byte granules (so that the sanitizer's red zone
+    starts with the first granule behind the payload), or a byte range of one; stands in for a torch device tensor in
+    the emulation run.  Whole granules because the irregular copy path loads the aligned 16-byte vectors that cover
+    its source bytes: it may read, never use, the rest of the first and last granule, which on the GPU cannot leave
+    the allocation (or its page) either."""
+
+    class _Block:
+        def __init__(self, nbytes):
+            self.ptr = _libc.malloc(max((nbytes + 15) & ~15, 16))
+            assert self.ptr and self.ptr % 16 == 0, "out of memory"
+
+        def __del__(self):
+            _libc.free(self.ptr)
+
+    def __init__(self, nbytes, block=None, offset=0):
+        self.block = block if block is not None else HostBuf._Block(nbytes)
+        self.offset = offset
+        self.nbytes = nbytes
+
+    def data_ptr(self):
+        return self.block.ptr + self.offset
+
+    def numel(self):
+        return self.nbytes
+
+    def bytes(self):
+        return (ctypes.c_uint8 * self.nbytes).from_address(self.data_ptr())
+
+    def __getitem__(self, key):
+        start, stop, step = key.indices(self.nbytes)
+        assert step == 1
+        return HostBuf(max(stop - start, 0), self.block, self.offset + start)
+
+    def fill(self, value):
+        ctypes.memset(self.data_ptr(), value, self.nbytes)
+
+    def write(self, raw):
+        if raw.size:
+            ctypes.memmove(self.data_ptr(), raw.ctypes.data, raw.size)
+
+    def read(self):
+        return np.frombuffer(self.bytes(), dtype=np.uint8).copy() if self.nbytes else np.zeros(0, np.uint8)
+
+
+class _EmuStream:
+    cuda_stream = 0x1000   # any non-null handle: the emulation runs every launch to completion
+
+    def synchronize(self):
+        pass
 
 ALGO_BY_NAME = {"mesh": Algo.MESH, "ring": Algo.RING, "rhd": Algo.RHD, "nhr": Algo.NHR,
                 "order_preserved": Algo.ORDER_PRESERVED, "aiv_mesh": Algo.AIV_MESH, "mesh_symmetric": Algo.MESH_SYMMETRIC,
@@ -15,6 +78,9 @@ ALGO_BY_NAME = {"mesh": Algo.MESH, "ring": Algo.RING, "rhd": Algo.RHD, "nhr": Al
 
 def require_library_on_gpu():
     """The GPU tests are meaningless without the native library: fail, never skip."""
+    if EMU:
+        assert "emu" in os.path.basename(hccl_amd.lib()._name), "the emulation run must not load the GPU library"
+        return
     import torch
     assert torch.cuda.is_available(), "these tests need the MI355X"
     hccl_amd.lib()
@@ -22,8 +88,13 @@ def require_library_on_gpu():
 
 def to_dev(arr, pad_front=0):
     """Uploads a numpy array as raw bytes.  pad_front shifts the payload to break 16-byte alignment."""
-    import torch
     raw = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+    if EMU:
+        t = HostBuf(raw.size + pad_front)
+        view = t[pad_front:pad_front + raw.size]
+        view.write(raw)
+        return view
+    import torch
     t = torch.empty(raw.size + pad_front + 64, dtype=torch.uint8, device="cuda")
     view = t[pad_front:pad_front + raw.size]
     if raw.size:
@@ -32,25 +103,35 @@ def to_dev(arr, pad_front=0):
 
 
 def dev_zeros(nbytes, pad_front=0, fill=0xAB):
+    if EMU:
+        t = HostBuf(nbytes + pad_front)
+        t.fill(fill)
+        return t[pad_front:pad_front + nbytes]
     import torch
     t = torch.full((nbytes + pad_front + 64,), fill, dtype=torch.uint8, device="cuda")
     return t[pad_front:pad_front + nbytes]
 
 
 def to_host(t, np_dtype):
+    if EMU:
+        return t.read().view(np_dtype).copy()
     return t.cpu().numpy().view(np_dtype).copy()
 
 
 class World:
     def __init__(self, n):
-        import torch
         self.n = n
         self.comms = hccl_amd.comm_init_all(n)
-        self.stream = torch.cuda.Stream()
+        if EMU:
+            self.stream = _EmuStream()
+        else:
+            import torch
+            self.stream = torch.cuda.Stream()
 
     def close(self):
-        import torch
-        torch.cuda.synchronize()
+        if not EMU:
+            import torch
+            torch.cuda.synchronize()
         for c in self.comms:
             hccl_amd.comm_destroy(c)
 
@@ -62,6 +143,8 @@ class World:
 
     def inputs_ready(self):
         """Inputs are produced on torch's default stream; the collective runs on self.stream."""
+        if EMU:
+            return
         import torch
         torch.cuda.current_stream().synchronize()
 

@@ -1,0 +1,135 @@
+"""CPU tier: the GPU parity tests, run against the library's own sources built for the host.
+
+tests/emu compiles hccl_amd/csrc (host layer and gfx950 kernels, inline assembly replaced by its plain meaning)
+against a stand-in HIP runtime that runs every launch workgroup by workgroup and lane by lane on the CPU.  The
+parity tests of tests/test_gpu_*.py then run unchanged in a pytest process of their own with HCCL_AMD_TEST_EMU=1:
+tests/gpu_util.py hands out host buffers, tests/conftest.py points the Python mirror at the emulation library.
+
+What this checks without a GPU: the kernels' index arithmetic, fold interpreter, heads / tails, tile tables and the
+host layer's launch geometry give the oracle's bits, and, in the AddressSanitizer run, touch no byte outside the
+16-byte granules of the buffers they were given.  It is how a kernel change is tried before it goes to the GPU.
+It says nothing about timing or about what the GPU compiler makes of the code: the `-m gpu` run stays the
+parity gate.  The emulation is test infrastructure; the package never loads it.
+"""
+import glob
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "tests", "emu"))
+import build_emu  # noqa: E402
+
+FILES = ["tests/test_gpu_parity.py", "tests/test_gpu_copies.py", "tests/test_gpu_rooted_and_v_ops.py",
+         "tests/test_gpu_random_sweep.py", "tests/test_gpu_point_to_point.py", "tests/test_zz_no_alloc.py"]
+# Tests that allocate or compute with torch on the GPU themselves (graphs, own streams, device-side generators), or
+# whose size is meant for the GPU.
+DESELECT = [
+    "tests/test_gpu_parity.py::test_two_kernel_all_reduce_can_be_captured_into_a_graph",
+    "tests/test_gpu_parity.py::test_warmed_up_collectives_can_be_captured_into_a_graph_and_replayed",
+    "tests/test_gpu_parity.py::test_all_reduce_larger_than_a_million_workgroups",
+    "tests/test_gpu_parity.py::test_reduce_scatter_into_the_own_slice_of_the_send_buffer",
+    "tests/test_gpu_parity.py::test_config2_reduce_scatter_bf16_n8",
+    "tests/test_gpu_parity.py::test_config3_all_reduce_int32_n16_max_and_prod",
+    "tests/test_gpu_copies.py::test_one_host_thread_per_rank_with_own_streams",
+    "tests/test_gpu_copies.py::test_all_gather_with_the_send_buffer_inside_the_receive_buffer",
+    "tests/test_gpu_copies.py::test_broadcast_and_all_gather_of_half_a_gigabyte",
+    "tests/test_gpu_rooted_and_v_ops.py::test_rooted_ops_with_one_blocking_thread_per_rank",
+    "tests/test_gpu_point_to_point.py::test_blocking_calls_from_one_thread_per_rank_on_streams_of_their_own",
+    "tests/test_gpu_point_to_point.py::test_barrier_orders_the_streams_of_all_ranks",
+    "tests/test_zz_no_alloc.py::test_ranks_on_their_own_streams",
+    "tests/test_zz_no_alloc.py::test_it_can_be_captured_into_a_graph_and_replayed",
+]
+
+
+def asan_runtime():
+    found = glob.glob("/opt/rocm/llvm/lib/clang/*/lib/linux/libclang_rt.asan-x86_64.so")
+    assert found, "the sanitizer runtime of the ROCm clang is missing"
+    return found[0]
+
+
+def emu_env(lib, asan_log=None):
+    env = dict(os.environ)
+    env["HCCL_AMD_TEST_EMU"] = "1"
+    env["HCCL_AMD_TEST_EMU_LIB"] = lib
+    if asan_log is not None:
+        # The sanitizer's runtime has to be in the process before Python allocates; whatever is preloaded already stays.
+        env["LD_PRELOAD"] = ":".join(x for x in (env.get("LD_PRELOAD", ""), asan_runtime()) if x)
+        env["ASAN_OPTIONS"] = "detect_leaks=0:verify_asan_link_order=0:log_path=" + asan_log
+    return env
+
+
+def run_gpu_tests(env, files=FILES, workers=None):
+    workers = workers or max(2, min(8, os.cpu_count() or 2))
+    cmd = [sys.executable, "-m", "pytest", "-m", "gpu", "-q", "-x", "-p", "no:cacheprovider", "-n", str(workers),
+           "--timeout", "900"] + files
+    for name in DESELECT:
+        cmd += ["--deselect", name]
+    proc = subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    tail = proc.stdout[-6000:]
+    m = re.search(r"(\d+) passed", proc.stdout)
+    return proc.returncode, int(m.group(1)) if m else 0, tail
+
+
+def test_gpu_parity_tests_pass_on_the_emulation():
+    lib = build_emu.build()
+    rc, passed, tail = run_gpu_tests(emu_env(lib))
+    assert rc == 0, tail
+    assert passed >= 280, tail   # a shrinking selection would hide what no longer runs
+
+
+def test_gpu_parity_tests_touch_no_byte_outside_their_buffers(tmp_path):
+    lib = build_emu.build(asan=True)
+    log = str(tmp_path / "asan")
+    rc, passed, tail = run_gpu_tests(emu_env(lib, log))
+    reports = "".join(open(f).read()[:3000] for f in sorted(glob.glob(log + "*"))[:2])
+    assert rc == 0 and not reports, tail + reports
+    assert passed >= 280, tail
+
+
+OVERRUN = r"""
+import ctypes, sys
+sys.path.insert(0, %r)
+import hccl_amd
+from gpu_util import HostBuf
+comms = hccl_amd.comm_init_all(2)
+count = 1000                                   # fp32 elements per rank
+sends = [HostBuf(4 * count), HostBuf(4 * count - 64)]   # the second send buffer is 64 bytes short
+recvs = [HostBuf(8 * count), HostBuf(8 * count)]
+with hccl_amd.group():
+    for r in range(2):
+        hccl_amd.all_gather(comms[r], sends[r], recvs[r], count, hccl_amd.HcclDataType.FP32, 0x1000)
+print("not caught")
+"""
+
+
+def test_the_sanitizer_run_does_catch_a_kernel_that_leaves_its_buffer(tmp_path):
+    """The check checks: a collective over a buffer that is too short must end the process with a report."""
+    lib = build_emu.build(asan=True)
+    log = str(tmp_path / "asan")
+    script = tmp_path / "overrun.py"
+    script.write_text(OVERRUN % os.path.join(ROOT, "tests"))
+    env = emu_env(lib, log)
+    env["PYTHONPATH"] = os.pathsep.join([ROOT, os.path.join(ROOT, "tests"), env.get("PYTHONPATH", "")])
+    boot = ("import ctypes, os, hccl_amd; hccl_amd._lib = hccl_amd._bind(ctypes.CDLL(os.environ['HCCL_AMD_TEST_EMU_LIB']));"
+            "exec(open(%r).read())" % str(script))
+    proc = subprocess.run([sys.executable, "-c", boot], cwd=ROOT, env=env, stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True)
+    reports = "".join(open(f).read()[:2000] for f in glob.glob(log + "*"))
+    assert proc.returncode != 0 and "not caught" not in proc.stdout, proc.stdout[-2000:]
+    assert "heap-buffer-overflow" in reports, reports
+
+
+def test_the_package_never_loads_the_emulation():
+    """The emulation is a checker.  Nothing under hccl_amd/, bench.py or __graft_entry__.py may name it."""
+    offenders = []
+    for path in glob.glob(os.path.join(ROOT, "hccl_amd", "**", "*"), recursive=True) + [
+            os.path.join(ROOT, "bench.py"), os.path.join(ROOT, "__graft_entry__.py")]:
+        if os.path.isfile(path) and path.endswith((".py", ".cc", ".h", ".hip", "Makefile")) and "/build/" not in path:
+            text = open(path, errors="replace").read()
+            if "libhccl_amd_emu" in text or "tests/emu" in text or "TEST_EMU" in text:
+                offenders.append(path)
+    assert not offenders, offenders
