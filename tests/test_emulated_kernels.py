@@ -2,7 +2,8 @@
 
 tests/emu compiles hccl_amd/csrc (host layer and gfx950 kernels, inline assembly replaced by its plain meaning)
 against a stand-in HIP runtime that runs every launch workgroup by workgroup and lane by lane on the CPU.  The
-parity tests of tests/test_gpu_*.py then run unchanged in a pytest process of their own with HCCL_AMD_TEST_EMU=1:
+parity tests of six tests/test_gpu_*.py files then run unchanged in a pytest process of their own with
+HCCL_AMD_TEST_EMU=1:
 tests/gpu_util.py hands out host buffers, tests/conftest.py points the Python mirror at the emulation library.
 
 What this checks without a GPU: the kernels' index arithmetic, fold interpreter, heads / tails, tile tables and the
@@ -25,8 +26,9 @@ import build_emu  # noqa: E402
 
 FILES = ["tests/test_gpu_parity.py", "tests/test_gpu_copies.py", "tests/test_gpu_rooted_and_v_ops.py",
          "tests/test_gpu_random_sweep.py", "tests/test_gpu_point_to_point.py", "tests/test_zz_no_alloc.py"]
-# Tests that allocate or compute with torch on the GPU themselves (graphs, own streams, device-side generators), or
-# whose size is meant for the GPU.
+# Left out: tests that allocate or compute with torch on the GPU themselves (graphs, own streams, device-side
+# generators), tests whose size is meant for the GPU, and the thread-per-rank tests: a stream or an event is an empty
+# handle here, so nothing orders a rank's read of its buffer after a copy that a peer's call runs.
 DESELECT = [
     "tests/test_gpu_parity.py::test_two_kernel_all_reduce_can_be_captured_into_a_graph",
     "tests/test_gpu_parity.py::test_warmed_up_collectives_can_be_captured_into_a_graph_and_replayed",
@@ -78,7 +80,7 @@ def test_gpu_parity_tests_pass_on_the_emulation():
     lib = build_emu.build()
     rc, passed, tail = run_gpu_tests(emu_env(lib))
     assert rc == 0, tail
-    assert passed >= 280, tail   # a shrinking selection would hide what no longer runs
+    assert passed >= 270, tail   # a shrinking selection would hide what no longer runs
 
 
 def test_gpu_parity_tests_touch_no_byte_outside_their_buffers(tmp_path):
@@ -87,7 +89,7 @@ def test_gpu_parity_tests_touch_no_byte_outside_their_buffers(tmp_path):
     rc, passed, tail = run_gpu_tests(emu_env(lib, log))
     reports = "".join(open(f).read()[:3000] for f in sorted(glob.glob(log + "*"))[:2])
     assert rc == 0 and not reports, tail + reports
-    assert passed >= 280, tail
+    assert passed >= 270, tail
 
 
 OVERRUN = r"""
