@@ -2698,6 +2698,10 @@ HcclResult HcclSend(void* sendBuf, uint64_t count, HcclDataType dataType, uint32
     }
     World* w = c->world;
     std::unique_lock<std::mutex> lock(w->mu);
+    if (w->destroyed != 0) {
+        Log(1, "%s on rank %u: a communicator of this world has been destroyed", "HcclSend", c->rank);
+        return HCCL_E_UNAVAIL;   // the peer may be the one that left: nothing would ever complete this transfer
+    }
     std::vector<std::shared_ptr<P2pOp>> ops{
         DepositP2p(w, true, c->rank, destRank, sendBuf, count, dataType, static_cast<hipStream_t>(stream))};
     return AwaitP2p(ref, lock, ops, "HcclSend", c->rank);
@@ -2735,6 +2739,10 @@ HcclResult HcclRecv(void* recvBuf, uint64_t count, HcclDataType dataType, uint32
     }
     World* w = c->world;
     std::unique_lock<std::mutex> lock(w->mu);
+    if (w->destroyed != 0) {
+        Log(1, "%s on rank %u: a communicator of this world has been destroyed", "HcclRecv", c->rank);
+        return HCCL_E_UNAVAIL;   // the peer may be the one that left: nothing would ever complete this transfer
+    }
     std::vector<std::shared_ptr<P2pOp>> ops{
         DepositP2p(w, false, srcRank, c->rank, recvBuf, count, dataType, static_cast<hipStream_t>(stream))};
     return AwaitP2p(ref, lock, ops, "HcclRecv", c->rank);
@@ -2807,6 +2815,10 @@ HcclResult HcclBatchSendRecv(HcclSendRecvItem* sendRecvInfo, uint32_t itemNum, H
     std::stable_sort(sends.begin(), sends.end(), bigFirst);
     std::stable_sort(recvs.begin(), recvs.end(), bigFirst);
     std::unique_lock<std::mutex> lock(w->mu);
+    if (w->destroyed != 0) {
+        Log(1, "%s on rank %u: a communicator of this world has been destroyed", "HcclBatchSendRecv", c->rank);
+        return HCCL_E_UNAVAIL;   // the peer may be the one that left: nothing would ever complete this transfer
+    }
     std::vector<std::shared_ptr<P2pOp>> ops;
     for (const HcclSendRecvItem* it : sends) {
         ops.push_back(DepositP2p(w, true, c->rank, it->remoteRank, it->buf, it->count, it->dataType,

@@ -2,7 +2,7 @@
 
 tests/emu compiles hccl_amd/csrc (host layer and gfx950 kernels, inline assembly replaced by its plain meaning)
 against a stand-in HIP runtime that runs every launch workgroup by workgroup and lane by lane on the CPU.  The
-parity tests of six tests/test_gpu_*.py files then run unchanged in a pytest process of their own with
+parity tests of seven tests/test_gpu_*.py files then run unchanged in a pytest process of their own with
 HCCL_AMD_TEST_EMU=1:
 tests/gpu_util.py hands out host buffers, tests/conftest.py points the Python mirror at the emulation library.
 
@@ -25,10 +25,10 @@ sys.path.insert(0, os.path.join(ROOT, "tests", "emu"))
 import build_emu  # noqa: E402
 
 FILES = ["tests/test_gpu_parity.py", "tests/test_gpu_copies.py", "tests/test_gpu_rooted_and_v_ops.py",
-         "tests/test_gpu_random_sweep.py", "tests/test_gpu_point_to_point.py", "tests/test_zz_no_alloc.py"]
+         "tests/test_gpu_random_sweep.py", "tests/test_gpu_point_to_point.py",
+         "tests/test_gpu_reference_python_suites.py", "tests/test_zz_no_alloc.py"]
 # Left out: tests that allocate or compute with torch on the GPU themselves (graphs, own streams, device-side
-# generators), tests whose size is meant for the GPU, and the thread-per-rank tests: a stream or an event is an empty
-# handle here, so nothing orders a rank's read of its buffer after a copy that a peer's call runs.
+# generators) and tests whose size is meant for the GPU.
 DESELECT = [
     "tests/test_gpu_parity.py::test_two_kernel_all_reduce_can_be_captured_into_a_graph",
     "tests/test_gpu_parity.py::test_warmed_up_collectives_can_be_captured_into_a_graph_and_replayed",
@@ -80,7 +80,7 @@ def test_gpu_parity_tests_pass_on_the_emulation():
     lib = build_emu.build()
     rc, passed, tail = run_gpu_tests(emu_env(lib))
     assert rc == 0, tail
-    assert passed >= 270, tail   # a shrinking selection would hide what no longer runs
+    assert passed >= 310, tail   # a shrinking selection would hide what no longer runs
 
 
 def test_gpu_parity_tests_touch_no_byte_outside_their_buffers(tmp_path):
@@ -89,7 +89,7 @@ def test_gpu_parity_tests_touch_no_byte_outside_their_buffers(tmp_path):
     rc, passed, tail = run_gpu_tests(emu_env(lib, log))
     reports = "".join(open(f).read()[:3000] for f in sorted(glob.glob(log + "*"))[:2])
     assert rc == 0 and not reports, tail + reports
-    assert passed >= 270, tail
+    assert passed >= 310, tail
 
 
 OVERRUN = r"""

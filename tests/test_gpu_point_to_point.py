@@ -58,6 +58,7 @@ def test_blocking_calls_from_one_thread_per_rank_on_streams_of_their_own():
     info = hccl_amd.get_root_info()
     got = [None] * n
     errors = []
+    all_through = threading.Barrier(n)   # destroying one rank ends the world: wait until every rank has made its calls
 
     def main(rank):
         try:
@@ -79,6 +80,7 @@ def test_blocking_calls_from_one_thread_per_rank_on_streams_of_their_own():
                 total = (inbox * 2.0).sum()
             stream.synchronize()
             got[rank] = float(total.item())
+            all_through.wait(90)
             hccl_amd.comm_destroy(comm)
         except Exception as e:   # noqa: BLE001 - reported below
             errors.append((rank, repr(e)))

@@ -12,6 +12,7 @@ import hccl_amd as h
 import oracle
 from hccl_amd import HcclDataType as DT, HcclReduceOp as OP
 
+import gpu_util
 from gpu_util import require_library_on_gpu
 
 pytestmark = pytest.mark.gpu
@@ -43,14 +44,23 @@ def unpack(name, raw, n):
 
 def run_ranks(nranks, body):
     """body(rank, comm, stream, to_dev, to_host) in one thread per rank; returns the per-rank results."""
-    import torch
+    if not gpu_util.EMU:
+        import torch
     info = h.get_root_info()
     out = [None] * nranks
     errors = []
+    # A rank that is through may not destroy its communicator while a peer still has point-to-point calls to make:
+    # destroying one rank ends the world for all of them.
+    all_through = threading.Barrier(nranks)
 
     def main(rank):
         try:
             comm = h.comm_init_root_info(nranks, info, rank)
+            if gpu_util.EMU:   # the CPU emulation run: host buffers, launches run to completion
+                out[rank] = body(rank, comm, gpu_util._EmuStream(), gpu_util.to_dev, lambda t: t.read())
+                all_through.wait(90)
+                h.comm_destroy(comm)
+                return
             stream = torch.cuda.Stream()
 
             def to_dev(arr):
@@ -63,6 +73,7 @@ def run_ranks(nranks, body):
                 return t.cpu().numpy()
             out[rank] = body(rank, comm, stream, to_dev, to_host)
             stream.synchronize()
+            all_through.wait(90)
             h.comm_destroy(comm)
         except Exception as e:   # noqa: BLE001 - reported below
             errors.append((rank, repr(e)))
@@ -79,6 +90,8 @@ def run_ranks(nranks, body):
 def zeros(nbytes):
     """A cleared device buffer; the fill (on torch's current stream) has finished when this returns, so that a
     collective on another stream, possibly a peer's, cannot be overtaken by it."""
+    if gpu_util.EMU:
+        return gpu_util.dev_zeros(max(nbytes, 1), fill=0)
     import torch
     t = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device="cuda")
     torch.cuda.current_stream().synchronize()

@@ -558,6 +558,23 @@ def test_a_live_rank_learns_that_a_peer_left():
     assert code_of(hccl_amd.barrier, comms[0], FAKE_STREAM) == 1
 
 
+def test_point_to_point_calls_after_a_peer_left_return_at_once():
+    """A send, a receive or a batch towards a rank that has destroyed its communicator can never be completed: the
+    call returns HCCL_E_UNAVAIL instead of waiting for the execution time-out."""
+    import time
+    comms = hccl_amd.comm_init_all(3)
+    hccl_amd.comm_destroy(comms[2])
+    t0 = time.perf_counter()
+    assert code_of(hccl_amd.send, comms[0], 0x2000, 8, DT.FP32, 1, FAKE_STREAM) == 7
+    assert code_of(hccl_amd.recv, comms[1], 0x2000, 8, DT.FP32, 0, FAKE_STREAM) == 7
+    items = [hccl_amd.make_send_recv_item(hccl_amd.HcclSendRecvType.SEND, 0x2000, 8, DT.FP32, 1),
+             hccl_amd.make_send_recv_item(hccl_amd.HcclSendRecvType.RECV, 0x3000, 8, DT.FP32, 2)]
+    assert code_of(hccl_amd.batch_send_recv, comms[0], items, FAKE_STREAM) == 7
+    assert time.perf_counter() - t0 < 5
+    for c in comms[:2]:
+        hccl_amd.comm_destroy(c)
+
+
 def test_two_threads_each_grouping_half_of_the_ranks():
     """Every HcclGroupEnd returns only when the calls its thread queued are complete, whichever thread completed
     the set (a barrier over one stream launches nothing, so this runs without a GPU)."""
