@@ -66,6 +66,10 @@ def prepare_sources():
     return digest.hexdigest()
 
 
+SANITIZE = {"": [], "asan": ["-fsanitize=address", "-fno-omit-frame-pointer"],
+            "tsan": ["-fsanitize=thread", "-fno-omit-frame-pointer"]}
+
+
 def flags(asan):
     f = [CLANG, "-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-ffp-contract=off", "-mf16c", "-pthread",
          "-Wno-unknown-attributes", "-Wno-ignored-attributes",
@@ -73,15 +77,14 @@ def flags(asan):
          "-D__builtin_amdgcn_readfirstlane=emu::ReadFirstLane", "-D__builtin_amdgcn_update_dpp=emu::UpdateDpp",
          "-D__builtin_amdgcn_alignbyte=emu::AlignByte", "-D__builtin_amdgcn_s_waitcnt=emu::WaitCnt",
          "-Daddress_space(x)="]
-    if asan:
-        f += ["-fsanitize=address", "-fno-omit-frame-pointer"]
+    f += SANITIZE["asan" if asan is True else (asan or "")]
     return f
 
 
 def build(asan=False, jobs=8):
     """Returns the path of the emulation library (built if its sources changed)."""
     stamp = prepare_sources()
-    tag = "_asan" if asan else ""
+    tag = "_asan" if asan is True else ("_" + asan if asan else "")
     lib = os.path.join(BUILD, "libhccl_amd_emu%s.so" % tag)
     stamp_file = lib + ".stamp"
     if os.path.exists(lib) and os.path.exists(stamp_file) and open(stamp_file).read() == stamp:
@@ -104,10 +107,28 @@ def build(asan=False, jobs=8):
         _reap(running.pop(0))
     link = [CLANG, "-shared", "-pthread", "-o", lib] + [obj for _, obj, _ in jobs_list]
     if asan:
-        link += ["-fsanitize=address", "-shared-libsan"]
+        link += SANITIZE["asan" if asan is True else asan][:1] + ["-shared-libsan"]
     subprocess.check_call(link)
     open(stamp_file, "w").write(stamp)
     return lib
+
+
+def build_example(name, sanitizer=""):
+    """One of the native callers of examples/ (a .cc file) linked against the emulation library, optionally under a
+    sanitizer ("asan" or "tsan"); returns the path of the executable."""
+    lib = build(asan=sanitizer or False)
+    exe = os.path.join(BUILD, name + ("_" + sanitizer if sanitizer else ""))
+    src = os.path.join(ROOT, "examples", name + ".cc")
+    if not os.path.exists(src):
+        src = os.path.join(HERE, name + ".cc")   # a driver of the tests' own
+    if os.path.exists(exe) and os.path.getmtime(exe) >= max(os.path.getmtime(lib), os.path.getmtime(src)):
+        return exe
+    cmd = [CLANG, "-std=c++17", "-O1", "-g", "-pthread", "-I" + HERE, "-I" + os.path.join(ROOT, "include"), src, lib,
+           "-Wl,-rpath," + BUILD, "-o", exe] + SANITIZE[sanitizer]
+    if sanitizer:
+        cmd += ["-shared-libsan"]
+    subprocess.check_call(cmd)
+    return exe
 
 
 def _reap(job):

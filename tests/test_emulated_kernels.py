@@ -125,6 +125,30 @@ def test_the_sanitizer_run_does_catch_a_kernel_that_leaves_its_buffer(tmp_path):
     assert "heap-buffer-overflow" in reports, reports
 
 
+def run_native(name, sanitizer, *args):
+    exe = build_emu.build_example(name, sanitizer)
+    env = dict(os.environ)
+    env["LD_LIBRARY_PATH"] = os.pathsep.join(x for x in (os.path.dirname(asan_runtime()), env.get("LD_LIBRARY_PATH", "")) if x)
+    return subprocess.run([exe] + [str(a) for a in args], cwd=ROOT, env=env, stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True, timeout=900)
+
+
+def test_host_layer_has_no_data_race_under_thread_sanitizer():
+    """tests/emu/host_stress.cc: two worlds with a thread per rank (blocking collectives, point-to-point rings,
+    batches), a world driven through groups by one thread and a world that a rank leaves while its peers are parked,
+    all at once, against the emulation build under ThreadSanitizer."""
+    proc = run_native("host_stress", "tsan", 600)
+    assert proc.returncode == 0 and "PASS" in proc.stdout, proc.stdout[-4000:]
+    assert "ThreadSanitizer" not in proc.stdout, proc.stdout[-4000:]
+
+
+def test_native_thread_per_rank_example_runs_on_the_emulation():
+    """examples/collectives_threads.cc, the shape of the reference's own examples, under ThreadSanitizer."""
+    proc = run_native("collectives_threads", "tsan", 4, 5000)
+    assert proc.returncode == 0 and "PASS" in proc.stdout, proc.stdout[-4000:]
+    assert "ThreadSanitizer" not in proc.stdout, proc.stdout[-4000:]
+
+
 def test_the_package_never_loads_the_emulation():
     """The emulation is a checker.  Nothing under hccl_amd/, bench.py or __graft_entry__.py may name it."""
     offenders = []
