@@ -125,9 +125,9 @@ def test_the_sanitizer_run_does_catch_a_kernel_that_leaves_its_buffer(tmp_path):
     assert "heap-buffer-overflow" in reports, reports
 
 
-def run_native(name, sanitizer, *args):
+def run_native(name, sanitizer, *args, **extra_env):
     exe = build_emu.build_example(name, sanitizer)
-    env = dict(os.environ)
+    env = dict(os.environ, **extra_env)
     env["LD_LIBRARY_PATH"] = os.pathsep.join(x for x in (os.path.dirname(asan_runtime()), env.get("LD_LIBRARY_PATH", "")) if x)
     return subprocess.run([exe] + [str(a) for a in args], cwd=ROOT, env=env, stdout=subprocess.PIPE,
                           stderr=subprocess.STDOUT, text=True, timeout=900)
@@ -140,6 +140,14 @@ def test_host_layer_has_no_data_race_under_thread_sanitizer():
     proc = run_native("host_stress", "tsan", 600)
     assert proc.returncode == 0 and "PASS" in proc.stdout, proc.stdout[-4000:]
     assert "ThreadSanitizer" not in proc.stdout, proc.stdout[-4000:]
+
+
+def test_host_layer_frees_what_it_allocates():
+    """The same driver under AddressSanitizer with its leak check: worlds, pending calls, events and plans are gone
+    when their last communicator has been destroyed."""
+    proc = run_native("host_stress", "asan", 300, ASAN_OPTIONS="detect_leaks=1")
+    assert proc.returncode == 0 and "PASS" in proc.stdout, proc.stdout[-4000:]
+    assert "Sanitizer" not in proc.stdout, proc.stdout[-4000:]
 
 
 def test_native_thread_per_rank_example_runs_on_the_emulation():
