@@ -13,6 +13,12 @@
 //                                 overlapped on two streams
 //   one source, N destinations    the AllGather / Broadcast pattern, source read from memory
 //
+//   placement                     `hbm_patterns place <ranks> <MiB>`: the fused and the fold kernels over buffers carved
+//                                 out of one allocation at a stride of the buffer size + D, for a list of D: how much
+//                                 the relative position of the peers' buffers is worth
+//   small messages                `hbm_patterns small <MiB>`: eight ranks of a few MiB over buffer sets in rotation (no
+//                                 pass finds its data cached): an empty launch of the same grid, reads, writes, fused
+//
 // Build: make -C examples      Run: examples/bin/hbm_patterns [ranks=16] [MiB per rank=256]
 // Prints one line per pattern: time per pass, bytes moved per second, fraction of the 8 TB/s HBM peak.
 #include <hip/hip_runtime.h>
@@ -20,6 +26,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 
 typedef uint32_t U4 __attribute__((ext_vector_type(4)));
 #define CK(x)                                                                      \
@@ -159,7 +166,7 @@ float MsPerPass(F pass)
 
 void Report(int n, const char* what, float ms, double bytes)
 {
-    printf("N=%-2d %-72s %8.3f ms %6.0f GB/s  %.3f\n", n, what, ms, bytes / ms / 1e6, bytes / ms / 1e6 / kPeakGBs);
+    printf("N=%-2d %-72s %8.4f ms %6.0f GB/s  %.3f\n", n, what, ms, bytes / ms / 1e6, bytes / ms / 1e6 / kPeakGBs);
     fflush(stdout);
 }
 
@@ -255,8 +262,98 @@ void Run(size_t bytesPerRank)
     CK(hipStreamDestroy(other));
 }
 
+// Nothing but the launch: what a grid of that many one-wavefront workgroups costs by itself.
+__global__ __launch_bounds__(64) void Empty(Bufs b, size_t nVec)
+{
+    if (static_cast<size_t>(blockIdx.x) * 64 + threadIdx.x == nVec + 1) {   // never true
+        b.dst[0][0] = U4{1u, 2u, 3u, 4u};
+    }
+}
+
+template <int N>
+void Placement(size_t bytesPerRank)
+{
+    const size_t nVec = bytesPerRank / 16;
+    const unsigned blocks = static_cast<unsigned>(nVec / 64);
+    const size_t gaps[] = {0, 256, 1024, 4096, 65536, 1u << 20, 2u << 20, 4u << 20, 8u << 20, 32u << 20, (32u << 20) + 4096};
+    const size_t maxGap = (32u << 20) + 4096;
+    const size_t gib = size_t(1) << 30;
+    char* raw = nullptr;
+    CK(hipMalloc((void**)&raw, 2 * N * (bytesPerRank + maxGap) + gib));
+    char* pool = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(raw) + gib - 1) & ~(uintptr_t)(gib - 1));
+    CK(hipMemset(pool, 3, 2 * N * (bytesPerRank + maxGap)));
+    const double moved = 2.0 * N * bytesPerRank;
+    for (size_t gap : gaps) {
+        Bufs b{};
+        for (int i = 0; i < N; ++i) {   // source i, destination i, source i + 1, ... at a stride of the size + gap
+            b.src[i] = reinterpret_cast<const U4*>(pool + static_cast<size_t>(2 * i) * (bytesPerRank + gap));
+            b.dst[i] = reinterpret_cast<U4*>(pool + static_cast<size_t>(2 * i + 1) * (bytesPerRank + gap));
+        }
+        char what[128];
+        snprintf(what, sizeof what, "stride = size + %8zu B: fused, one wavefront per tile", gap);
+        Report(N, what, MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, true, true, 0>), dim3(blocks), dim3(64), 0, 0, b, nVec); }), moved);
+        snprintf(what, sizeof what, "stride = size + %8zu B: fused, stores shared by 3 wavefronts", gap);
+        Report(N, what, MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 3, true, true, 0>), dim3(blocks), dim3(192), 0, 0, b, nVec); }), moved);
+        snprintf(what, sizeof what, "stride = size + %8zu B: fold into the first destination", gap);
+        Report(N, what, MsPerPass([&] { hipLaunchKernelGGL((FoldToFirst<N>), dim3(blocks), dim3(64), 0, 0, b, size_t(0)); }),
+               (N + 1.0) * bytesPerRank);
+    }
+    CK(hipFree(raw));
+}
+
+void Small(size_t bytesPerRank)
+{
+    constexpr int N = 8;
+    constexpr int kSets = 6;   // 6 x 16 x 4 MiB = 384 MiB: past the last-level cache
+    const size_t nVec = bytesPerRank / 16;
+    const unsigned blocks = static_cast<unsigned>(nVec / 64);
+    Bufs sets[kSets] = {};
+    for (Bufs& b : sets) {
+        for (int i = 0; i < N; ++i) {
+            CK(hipMalloc((void**)&b.src[i], bytesPerRank));
+            CK(hipMemset((void*)b.src[i], 1 + i, bytesPerRank));
+            CK(hipMalloc((void**)&b.dst[i], bytesPerRank));
+        }
+    }
+    int pass = 0;
+    const double half = static_cast<double>(N) * bytesPerRank;
+    Report(N, "empty launch of the same grid", MsPerPass([&] { hipLaunchKernelGGL(Empty, dim3(blocks), dim3(64), 0, 0, sets[pass++ % kSets], nVec); }), 0);
+    Report(N, "reads alone", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, true, false, 0>), dim3(blocks), dim3(64), 0, 0, sets[pass++ % kSets], nVec); }), half);
+    Report(N, "writes alone, non-temporal", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, false, true, 0>), dim3(blocks), dim3(64), 0, 0, sets[pass++ % kSets], nVec); }), half);
+    Report(N, "fused N reads + N writes, non-temporal stores", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, true, true, 0>), dim3(blocks), dim3(64), 0, 0, sets[pass++ % kSets], nVec); }), 2 * half);
+    Report(N, "fused, stores shared by 2 wavefronts", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 2, true, true, 0>), dim3(blocks), dim3(128), 0, 0, sets[pass++ % kSets], nVec); }), 2 * half);
+    for (Bufs& b : sets) {
+        for (int i = 0; i < N; ++i) {
+            CK(hipFree((void*)b.src[i]));
+            CK(hipFree(b.dst[i]));
+        }
+    }
+}
+
 int main(int argc, char** argv)
 {
+    if (argc > 1 && (strcmp(argv[1], "place") == 0 || strcmp(argv[1], "small") == 0)) {
+        const bool place = argv[1][0] == 'p';
+        const int ranks = place && argc > 2 ? atoi(argv[2]) : 8;
+        const size_t mibArg = static_cast<size_t>(atoi(argc > (place ? 3 : 2) ? argv[place ? 3 : 2] : "4"));
+        if (mibArg < 1 || mibArg > 1024 || (ranks != 6 && ranks != 8 && ranks != 16)) {
+            printf("usage: hbm_patterns place <ranks: 6, 8 or 16> <MiB per rank: 1 .. 1024> | hbm_patterns small <MiB per rank>\n");
+            return 1;
+        }
+        CK(hipEventCreate(&g_start));
+        CK(hipEventCreate(&g_stop));
+        printf("pattern%68s time per pass   moved   of 8 TB/s\n", "");
+        if (!place) {
+            Small(mibArg << 20);
+        } else if (ranks == 16) {
+            Placement<16>(mibArg << 20);
+        } else if (ranks == 8) {
+            Placement<8>(mibArg << 20);
+        } else {
+            Placement<6>(mibArg << 20);
+        }
+        return 0;
+    }
     const int n = argc > 1 ? atoi(argv[1]) : 16;
     const size_t mib = argc > 2 ? static_cast<size_t>(atoi(argv[2])) : 256;
     if ((n != 6 && n != 8 && n != 16) || mib < 64 || mib > 2048) {

@@ -119,12 +119,19 @@ def build_example(name, sanitizer=""):
     lib = build(asan=sanitizer or False)
     exe = os.path.join(BUILD, name + ("_" + sanitizer if sanitizer else ""))
     src = os.path.join(ROOT, "examples", name + ".cc")
+    if not os.path.exists(src) and os.path.exists(os.path.join(ROOT, "examples", name + ".hip")):
+        # an example with kernels of its own: same treatment as the library's kernels
+        os.makedirs(SRC, exist_ok=True)
+        src = os.path.join(SRC, "example_" + name + ".cc")
+        text = transform(open(os.path.join(ROOT, "examples", name + ".hip")).read(), name + ".hip")
+        if not os.path.exists(src) or open(src).read() != text:
+            open(src, "w").write(text)
     if not os.path.exists(src):
         src = os.path.join(HERE, name + ".cc")   # a driver of the tests' own
     if os.path.exists(exe) and os.path.getmtime(exe) >= max(os.path.getmtime(lib), os.path.getmtime(src)):
         return exe
-    cmd = [CLANG, "-std=c++17", "-O1", "-g", "-pthread", "-I" + HERE, "-I" + os.path.join(ROOT, "include"), src, lib,
-           "-Wl,-rpath," + BUILD, "-o", exe] + SANITIZE[sanitizer]
+    cmd = flags(sanitizer or False)[:1] + [f for f in flags(sanitizer or False)[3:] if f != "-fPIC"] + [
+        "-D__HIPCC__=1", src, lib, "-Wl,-rpath," + BUILD, "-o", exe]
     if sanitizer:
         cmd += ["-shared-libsan"]
     subprocess.check_call(cmd)
