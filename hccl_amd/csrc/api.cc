@@ -331,6 +331,13 @@ uint32_t EnvU32(const char* name, uint32_t dflt)
     return v > 0 ? static_cast<uint32_t>(v) : dflt;
 }
 
+// An integer variable that may be 0: `dflt` when it is unset or empty.
+int EnvInt(const char* name, int dflt)
+{
+    const char* s = getenv(name);
+    return (s && *s) ? atoi(s) : dflt;
+}
+
 bool ParseAlgoName(const std::string& s, HcclAmdAlgo* algo)
 {
     static const struct { const char* name; HcclAmdAlgo algo; } table[] = {
@@ -424,11 +431,11 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     }
     w->reduceVector = EnvU32("HCCL_AMD_REDUCE_VECTOR", 1) != 0;
     w->stuckEnabled = EnvU32("HCCL_AMD_STUCK_COUNTERS", 0) != 0;
-    w->twoKernelMode = getenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS") != nullptr ? atoi(getenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS")) : 2;
+    w->twoKernelMode = EnvInt("HCCL_AMD_ALLREDUCE_TWO_KERNELS", 2);
     if (w->twoKernelMode < 0 || w->twoKernelMode > 1) {
         w->twoKernelMode = 2;
     }
-    w->copyTwoKernelMode = getenv("HCCL_AMD_COPY_TWO_KERNELS") != nullptr ? atoi(getenv("HCCL_AMD_COPY_TWO_KERNELS")) : 2;
+    w->copyTwoKernelMode = EnvInt("HCCL_AMD_COPY_TWO_KERNELS", 2);
     if (w->copyTwoKernelMode < 0 || w->copyTwoKernelMode > 1) {
         w->copyTwoKernelMode = 2;
     }
@@ -436,7 +443,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->pieceBytes == 0) {
         w->pieceBytes = 256;
     }
-    w->leadFromSrc = getenv("HCCL_AMD_LEAD_FROM_SRC") == nullptr || atoi(getenv("HCCL_AMD_LEAD_FROM_SRC")) != 0;
+    w->leadFromSrc = EnvInt("HCCL_AMD_LEAD_FROM_SRC", 1) != 0;
     w->reduceBatch = EnvU32("HCCL_AMD_REDUCE_BATCH", 0);
     if (w->reduceBatch != 8 && w->reduceBatch != 16) {
         w->reduceBatch = 0;
@@ -812,6 +819,9 @@ HcclResult LaunchToAll(World* w, const ReduceArgs& a, const DevicePlan& plan, Hc
                        hipStream_t s)
 {
     const uint32_t esz = DataTypeSize(dtype);
+    if (esz == 0) {
+        return HCCL_E_INTERNAL;   // the entry points admit known types only
+    }
     if (a.nGroup != 1 || a.dstOwn != 0 || a.varGroups != 0 || !FoldThenFanOut(w, a.nDst, a.total * esz)) {
         ReduceArgs fused = a;
         return LaunchOneReduce(w, fused, plan, dtype, op, s);
