@@ -59,9 +59,10 @@ constexpr uint8_t kCtlOpen = 0x80;
 // and writes either to every dst[d], d < nDst, at  g * dstGroupStride + c * subLen + e   (dstOwn == 0)
 // or only to dst[g] at  c * subLen + e                                                    (dstOwn == 1).
 // Its fold program is number  g * progGroupStride + c * progSubStride.
-struct ReduceArgs {
-    const void* src[kMaxRanks];
-    void* dst[kMaxRanks];
+// The scalars of a launch come first and together (ReduceHot): a workgroup fetches them with one block of scalar
+// loads before it does anything else.  Fetched one by one, where the code happens to need them, they were a
+// dozen round trips in a row in front of the first vector load of every wavefront.
+struct ReduceHot {
     const uint8_t* prog;
     uint64_t total;
     uint64_t groupLen;
@@ -74,7 +75,7 @@ struct ReduceArgs {
     uint32_t dstOwn;
     uint32_t progGroupStride;
     uint32_t progSubStride;
-    uint32_t blocksPerSub;
+    uint32_t blocksPerSub;   // workgroups per sub-segment: the grid is (blocksPerSub, nSub, nGroup), or one-dimensional with varGroups
     uint32_t vecOk;   // take the 128-bit path (0: element by element, for testing)
     uint32_t threads; // workgroup size of the launch
     uint32_t vecBatch;       // leaves per load batch of the 128-bit path: 8 or 16 (picks the kernel instantiation)
@@ -83,11 +84,16 @@ struct ReduceArgs {
     uint32_t storeWaves;     // > 1: workgroups of 64 * storeWaves threads, wavefront 0 folds and wavefront k stores to
                              // destinations k, k + storeWaves, ... (threads must be 64, dstOwn 0); 0 or 1: every wavefront
                              // folds and stores its own tile
+    uint32_t varGroups;      // groups of unequal length, see below
+};
+
+struct ReduceArgs : ReduceHot {
+    const void* src[kMaxRanks];
+    void* dst[kMaxRanks];
     // Groups of unequal length (ReduceScatterV): when varGroups is set, group g spans groupLenV[g]
     // elements starting groupOffV[g] elements into every source, instead of the uniform
     // groupLen / srcGroupStride / total geometry, and owns the workgroups
     // [groupBlockEnd[g-1], groupBlockEnd[g]) of the grid (filled by the launcher's caller).
-    uint32_t varGroups;
     uint32_t groupBlockEnd[kMaxRanks];
     uint64_t groupOffV[kMaxRanks];
     uint64_t groupLenV[kMaxRanks];

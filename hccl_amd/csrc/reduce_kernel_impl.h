@@ -295,6 +295,26 @@ struct TableBytes {
     __device__ __forceinline__ uint32_t operator[](int i) const { return (w[i / 4] >> (8 * (i % 4))) & 0xFFu; }
 };
 
+// The rank and control bytes of a program's first batch of leaves, fetched by the kernel together with the
+// program's header (one round of scalar loads) and handed to the interpreter.
+template <int kBatch>
+struct FirstBatch {
+    TableBytes<kBatch> ranks, ctls;
+    __device__ __forceinline__ void Load(ProgWords words)
+    {
+        ranks.Load(words, kDevProgRankOff);
+        ctls.Load(words, kDevProgCtlOff);
+    }
+    // every word exists before the first is used
+    __device__ __forceinline__ void Fence()
+    {
+#pragma unroll
+        for (int k = 0; k < kBatch / 4; ++k) {
+            asm volatile("" : "+s"(ranks.w[k]), "+s"(ctls.w[k]));
+        }
+    }
+};
+
 // The same for eight uniform 64-bit values (leaf addresses): all of them exist before the first is used.
 __device__ __forceinline__ void ScalarFence8(uint64_t* r)
 {
@@ -305,6 +325,19 @@ __device__ __forceinline__ void ScalarFence8(uint64_t* r)
 __device__ __forceinline__ void IssueFence8(U32x4* r)
 {
     asm volatile("" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
+}
+
+// The launch's scalars, all fetched before anything is done with one of them: the compiler then requests them as a
+// few wide scalar loads behind one wait, instead of one load and one wait wherever the code first needs a field.
+__device__ __forceinline__ void FenceHot(ReduceHot& h)
+{
+    uint64_t prog = reinterpret_cast<uint64_t>(h.prog);
+    asm volatile(""
+                 : "+s"(prog), "+s"(h.total), "+s"(h.groupLen), "+s"(h.subLen), "+s"(h.srcGroupStride),
+                   "+s"(h.dstGroupStride), "+s"(h.nGroup), "+s"(h.nSub), "+s"(h.nDst), "+s"(h.dstOwn),
+                   "+s"(h.progGroupStride), "+s"(h.progSubStride), "+s"(h.blocksPerSub), "+s"(h.vecOk), "+s"(h.threads),
+                   "+s"(h.vecBatch), "+s"(h.writeThrough), "+s"(h.leadFromSrc), "+s"(h.storeWaves), "+s"(h.varGroups));
+    h.prog = reinterpret_cast<const uint8_t*>(prog);
 }
 
 // acc <- x (+) acc for a stored element x: the traits' fused form where they have one.
@@ -460,7 +493,8 @@ struct PackOps<E, 16, typename E::Swar> {
 // kBatch leaves are taken at a time (a multiple of 8).
 template <class E, int W, int kBatch>
 __device__ __forceinline__ Pack<typename E::S, W> ReduceValue(const ProgramView& pv, uint32_t* stack,
-                                                              const ReduceArgs& args, uint64_t e)
+                                                              const ReduceArgs& args, const ReduceHot& h, uint64_t e,
+                                                              const FirstBatch<kBatch>* first = nullptr)
 {
     using S = typename E::S;
     AccPack<E, W> acc;
@@ -473,8 +507,13 @@ __device__ __forceinline__ Pack<typename E::S, W> ReduceValue(const ProgramView&
     const uint32_t nLeaves = pv.nLeaves;
     for (uint32_t b = 0; b < nLeaves; b += kBatch) {
         TableBytes<kBatch> ranks, ctls;
-        ranks.Load(pv.words, kDevProgRankOff + b);
-        ctls.Load(pv.words, kDevProgCtlOff + b);
+        if (first != nullptr && b == 0) {
+            ranks = first->ranks;
+            ctls = first->ctls;
+        } else {
+            ranks.Load(pv.words, kDevProgRankOff + b);
+            ctls.Load(pv.words, kDevProgCtlOff + b);
+        }
         // Leaf addresses first and unconditionally (table bytes past the last leaf name rank 0), so that their
         // scalar loads go out together instead of one wait per leaf.
         uint64_t leaf[kBatch];
@@ -525,7 +564,7 @@ __device__ __forceinline__ Pack<typename E::S, W> ReduceValue(const ProgramView&
             if (b + i < nLeaves) {
                 const uint32_t ctl = ctls[i];
                 if (ctl & kCtlOpen) {
-                    PushAcc<E, W>(stack, args.threads, level, acc);
+                    PushAcc<E, W>(stack, h.threads, level, acc);
                     ++level;
                     init = true;
                 }
@@ -538,7 +577,7 @@ __device__ __forceinline__ Pack<typename E::S, W> ReduceValue(const ProgramView&
                 for (uint32_t closes = ctl & 0x7Fu; closes != 0; --closes) {
                     AccPack<E, W> outer;
                     --level;
-                    PopAcc<E, W>(stack, args.threads, level, outer);
+                    PopAcc<E, W>(stack, h.threads, level, outer);
                     PackOps<E, W>::Merge(acc, outer);   // nested value is src, enclosing level is dst
                 }
             }
@@ -550,24 +589,25 @@ __device__ __forceinline__ Pack<typename E::S, W> ReduceValue(const ProgramView&
 // The value of ReduceValue written to the destinations firstDst, firstDst + dstStep, ... of the launch (all of
 // them with 0 and 1), or to the group's own destination.
 template <class S, int W>
-__device__ __forceinline__ void StoreResult(const ReduceArgs& args, const Pack<S, W>& out, uint64_t elemOff,
-                                            uint32_t group, uint32_t firstDst, uint32_t dstStep)
+__device__ __forceinline__ void StoreResult(const ReduceArgs& args, const ReduceHot& h, const Pack<S, W>& out,
+                                            uint64_t elemOff, uint32_t group, uint32_t firstDst, uint32_t dstStep)
 {
-    if (args.dstOwn) {
-        StorePack<S, W>(args.dst[group], elemOff, out, args.writeThrough != 0);
+    if (h.dstOwn) {
+        StorePack<S, W>(args.dst[group], elemOff, out, h.writeThrough != 0);
     } else {
-        for (uint32_t d = firstDst; d < args.nDst; d += dstStep) {
-            StorePack<S, W>(args.dst[d], elemOff, out, args.writeThrough != 0);
+        for (uint32_t d = firstDst; d < h.nDst; d += dstStep) {
+            StorePack<S, W>(args.dst[d], elemOff, out, h.writeThrough != 0);
         }
     }
 }
 
 template <class E, int W, int kBatch>
 __device__ __forceinline__ void ReduceOne(const ProgramView& pv, uint32_t* stack, const ReduceArgs& args,
-                                          uint64_t e, uint64_t dstOff, uint32_t group)
+                                          const ReduceHot& h, uint64_t e, uint64_t dstOff, uint32_t group,
+                                          const FirstBatch<kBatch>* first = nullptr)
 {
-    const Pack<typename E::S, W> out = ReduceValue<E, W, kBatch>(pv, stack, args, e);
-    StoreResult<typename E::S, W>(args, out, dstOff + e, group, 0, 1);
+    const Pack<typename E::S, W> out = ReduceValue<E, W, kBatch>(pv, stack, args, h, e, first);
+    StoreResult<typename E::S, W>(args, h, out, dstOff + e, group, 0, 1);
 }
 
 // Dynamic LDS: the accumulator stack, (plan depth - 1) * accumulator bytes * args.threads.
@@ -579,14 +619,16 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     using S = typename E::S;
     constexpr int W = 16 / sizeof(S);
     extern __shared__ uint32_t accStack[];
+    ReduceHot h = args;
+    FenceHot(h);
 
     uint32_t g, c, blk, blocksHere;   // group, sub-segment, this workgroup's index among the blocksHere of it
     uint64_t gLen;
     uint64_t gSrc;
-    if (args.varGroups) {
+    if (h.varGroups) {
         // Groups of unequal length own unequal shares of the grid: first group whose last block is not before us.
         uint32_t lo = 0;
-        uint32_t hi = args.nGroup - 1;
+        uint32_t hi = h.nGroup - 1;
         while (lo < hi) {
             const uint32_t mid = (lo + hi) >> 1;
             if (blockIdx.x >= args.groupBlockEnd[mid]) {
@@ -603,36 +645,53 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
         gLen = args.groupLenV[g];
         gSrc = args.groupOffV[g];
     } else {
-        const uint32_t sub = blockIdx.x / args.blocksPerSub;
-        blk = blockIdx.x - sub * args.blocksPerSub;
-        blocksHere = args.blocksPerSub;
-        g = sub / args.nSub;
-        c = sub - g * args.nSub;
-        const uint64_t gBeg = static_cast<uint64_t>(g) * args.groupLen;
-        if (gBeg >= args.total) {
+        // The grid is (workgroups per sub-segment, sub-segments, groups): no division to find one's place.
+        blk = blockIdx.x;
+        blocksHere = h.blocksPerSub;
+        c = blockIdx.y;
+        g = blockIdx.z;
+        const uint64_t gBeg = static_cast<uint64_t>(g) * h.groupLen;
+        if (gBeg >= h.total) {
             return;
         }
-        gLen = (args.total - gBeg < args.groupLen) ? args.total - gBeg : args.groupLen;
-        gSrc = static_cast<uint64_t>(g) * args.srcGroupStride;
+        gLen = (h.total - gBeg < h.groupLen) ? h.total - gBeg : h.groupLen;
+        gSrc = static_cast<uint64_t>(g) * h.srcGroupStride;
     }
-    const uint64_t sBeg = static_cast<uint64_t>(c) * args.subLen;
-    uint64_t sEnd = (c == args.nSub - 1) ? gLen : sBeg + args.subLen;
+    const uint64_t sBeg = static_cast<uint64_t>(c) * h.subLen;
+    uint64_t sEnd = (c == h.nSub - 1) ? gLen : sBeg + h.subLen;
     sEnd = sEnd < gLen ? sEnd : gLen;
     if (sBeg >= sEnd) {
         return;
     }
     const uint64_t len = sEnd - sBeg;
     const uint64_t srcOff = gSrc + sBeg;
-    const uint64_t dstOff = args.dstOwn ? sBeg : static_cast<uint64_t>(g) * args.dstGroupStride + sBeg;
+    const uint64_t dstOff = h.dstOwn ? sBeg : static_cast<uint64_t>(g) * h.dstGroupStride + sBeg;
 
     ProgramView pv;
-    pv.words = (ProgWords)(uintptr_t)(args.prog + static_cast<uint64_t>(g * args.progGroupStride + c * args.progSubStride) *
+    pv.words = (ProgWords)(uintptr_t)(h.prog + static_cast<uint64_t>(g * h.progGroupStride + c * h.progSubStride) *
                                                       kDevProgBytes);
     pv.srcByteOff = srcOff * sizeof(S);
-    pv.nLeaves = pv.words[0] & 0xFFu;
+    // Second round of scalar loads, all requested together: the program's header, and the two buffer addresses the
+    // alignment below is taken from.
+    uint32_t header = pv.words[0];
+    // (The sixteen-leaf batch keeps its tables out of this round: with sixteen leaf addresses live as well, the
+    // scalar registers would not hold them.)
+    constexpr bool kPreloadBatch = VB == 8;
+    FirstBatch<VB> firstBatch;
+    if constexpr (kPreloadBatch) {
+        firstBatch.Load(pv.words);
+    }
+    uint64_t firstDstAddr = reinterpret_cast<uint64_t>(h.dstOwn ? args.dst[g] : args.dst[0]);
+    uint64_t firstSrcAddr = reinterpret_cast<uint64_t>(args.src[0]);
+    asm volatile("" : "+s"(header), "+s"(firstDstAddr), "+s"(firstSrcAddr));
+    if constexpr (kPreloadBatch) {
+        firstBatch.Fence();
+    }
+    const FirstBatch<VB>* const preloaded = kPreloadBatch ? &firstBatch : nullptr;
+    pv.nLeaves = header & 0xFFu;
 
-    const uint64_t stride = static_cast<uint64_t>(blocksHere) * args.threads;
-    const uint64_t first = static_cast<uint64_t>(blk) * args.threads + threadIdx.x;
+    const uint64_t stride = static_cast<uint64_t>(blocksHere) * h.threads;
+    const uint64_t first = static_cast<uint64_t>(blk) * h.threads + threadIdx.x;
 
     // When vecOk, `head` elements bring the stores to the first destination onto a 16-byte boundary, a 128-bit
     // body follows, and fewer than W elements remain.  Sources and further destinations only need element
@@ -644,23 +703,23 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     uint64_t head = len;
     uint64_t nVec = 0;
     uint32_t lead = 0;
-    if (args.vecOk) {
-        const uint64_t addr = reinterpret_cast<uint64_t>(args.dstOwn ? args.dst[g] : args.dst[0]) + dstOff * sizeof(S);
+    if (h.vecOk) {
+        const uint64_t addr = firstDstAddr + dstOff * sizeof(S);
         const uint32_t mis = static_cast<uint32_t>(addr & 15u);
         head = mis ? (16u - mis) / sizeof(S) : 0;
         head = head < len ? head : len;
         nVec = (len - head) / W;
         // One result stream fed by many sources: the sources' lines count (those of the first rank stand for all;
         // peers' buffers are usually congruent), otherwise the destination's.
-        const uint64_t lineOf = args.leadFromSrc
-                                    ? reinterpret_cast<uint64_t>(args.src[0]) + (srcOff + head) * sizeof(S)
+        const uint64_t lineOf = h.leadFromSrc
+                                    ? firstSrcAddr + (srcOff + head) * sizeof(S)
                                     : addr + head * sizeof(S);
         lead = static_cast<uint32_t>((lineOf >> 4) & kReduceLeadMask);
     }
     const uint64_t bodyEnd = head + nVec * W;
     const uint64_t nScalar = head + (len - bodyEnd);
-    if (args.storeWaves > 1) {
-        // Stores split over the wavefronts of the workgroup (args.threads == 64 lanes fold, 64 * storeWaves run):
+    if (h.storeWaves > 1) {
+        // Stores split over the wavefronts of the workgroup (h.threads == 64 lanes fold, 64 * storeWaves run):
         // wavefront 0 folds the tile and parks the result in LDS, wavefront k writes it to destinations k,
         // k + storeWaves, ...  A wavefront that stores to many streams one after the other is what bounds the
         // many-destination launches; with two to four destinations per wavefront the same stores leave 5-15 %
@@ -676,7 +735,7 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
             const uint64_t e = head + (u - lead) * W;
             Pack<S, W> out;
             if (wave == 0 && active) {
-                out = ReduceValue<E, W, VB>(pv, accStack, args, e);
+                out = ReduceValue<E, W, VB>(pv, accStack, args, h, e, preloaded);
                 parked[slot][lane] = __builtin_bit_cast(U32x4, out);
             }
             __syncthreads();
@@ -684,26 +743,26 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
                 if (wave != 0) {
                     out = __builtin_bit_cast(Pack<S, W>, parked[slot][lane]);
                 }
-                StoreResult<S, W>(args, out, dstOff + e, g, wave, args.storeWaves);
+                StoreResult<S, W>(args, h, out, dstOff + e, g, wave, h.storeWaves);
             }
             slot ^= 1u;
         }
         if (wave == 0) {
             for (uint64_t i = static_cast<uint64_t>(blk) * 64 + lane; i < nScalar; i += static_cast<uint64_t>(blocksHere) * 64) {
                 const uint64_t e = i < head ? i : i - head + bodyEnd;
-                ReduceOne<E, 1, 8>(pv, accStack, args, e, dstOff, g);
+                ReduceOne<E, 1, 8>(pv, accStack, args, h, e, dstOff, g);
             }
         }
         return;
     }
     for (uint64_t u = first; u < nVec + lead; u += stride) {
         if (u >= lead) {
-            ReduceOne<E, W, VB>(pv, accStack, args, head + (u - lead) * W, dstOff, g);
+            ReduceOne<E, W, VB>(pv, accStack, args, h, head + (u - lead) * W, dstOff, g, preloaded);
         }
     }
     for (uint64_t i = first; i < nScalar; i += stride) {
         const uint64_t e = i < head ? i : i - head + bodyEnd;
-        ReduceOne<E, 1, 8>(pv, accStack, args, e, dstOff, g);
+        ReduceOne<E, 1, 8>(pv, accStack, args, h, e, dstOff, g);
     }
 }
 

@@ -31,7 +31,17 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
         }
         threads = 64 * args.storeWaves;
     }
-    hipLaunchKernelGGL(fn, dim3(nBlocks), dim3(threads), ldsBytes, stream, args);
+    // Uniform geometry: (workgroups per sub-segment, sub-segments, groups), consecutive workgroups on consecutive
+    // positions of a sub-segment as before; groups of unequal length own runs of a one-dimensional grid.
+    dim3 grid(nBlocks);
+    if (!args.varGroups) {
+        if (args.blocksPerSub == 0 || args.nSub == 0 || args.nGroup == 0 || args.nSub > 65535u || args.nGroup > 65535u ||
+            static_cast<uint64_t>(args.blocksPerSub) * args.nSub * args.nGroup != nBlocks) {
+            return hipErrorInvalidValue;
+        }
+        grid = dim3(args.blocksPerSub, args.nSub, args.nGroup);
+    }
+    hipLaunchKernelGGL(fn, grid, dim3(threads), ldsBytes, stream, args);
     return hipGetLastError();
 }
 

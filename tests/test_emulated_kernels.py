@@ -76,20 +76,15 @@ def run_gpu_tests(env, files=FILES, workers=None):
     return proc.returncode, int(m.group(1)) if m else 0, tail
 
 
-def test_gpu_parity_tests_pass_on_the_emulation():
-    lib = build_emu.build()
-    rc, passed, tail = run_gpu_tests(emu_env(lib))
-    assert rc == 0, tail
-    assert passed >= 310, tail   # a shrinking selection would hide what no longer runs
-
-
-def test_gpu_parity_tests_touch_no_byte_outside_their_buffers(tmp_path):
+def test_gpu_parity_tests_pass_on_the_emulation_and_touch_no_byte_outside_their_buffers(tmp_path):
+    """One run for both: the tests compare with the oracle, AddressSanitizer watches every access.  (Without the
+    sanitizer, for a quick look while working on a kernel: run_gpu_tests(emu_env(build_emu.build())).)"""
     lib = build_emu.build(asan=True)
     log = str(tmp_path / "asan")
     rc, passed, tail = run_gpu_tests(emu_env(lib, log))
     reports = "".join(open(f).read()[:3000] for f in sorted(glob.glob(log + "*"))[:2])
     assert rc == 0 and not reports, tail + reports
-    assert passed >= 310, tail
+    assert passed >= 310, tail   # a shrinking selection would hide what no longer runs
 
 
 OVERRUN = r"""
