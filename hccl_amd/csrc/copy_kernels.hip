@@ -313,17 +313,26 @@ template <int T, int MODE>
 __global__ __launch_bounds__(T) void A2aCopyKernel(const A2aArgs args)
 {
     constexpr uint32_t kTile = T * 16u;
-    const K32 tileEnd = (K32)(uintptr_t)args.tileEnd;
-    const K32 hint = (K32)(uintptr_t)args.hint;
+    // Rounds of scalar loads in front of the tile's vector load: the arguments; the two hints; the search steps
+    // (usually none or one); the descriptor.  Each round's values are requested together.
+    uint64_t tileEndAddr = reinterpret_cast<uint64_t>(args.tileEnd);
+    uint64_t hintAddr = reinterpret_cast<uint64_t>(args.hint);
+    uint64_t descAddr = reinterpret_cast<uint64_t>(args.desc);
+    uint32_t hintShift = args.hintShift;
+    asm volatile("" : "+s"(tileEndAddr), "+s"(hintAddr), "+s"(descAddr), "+s"(hintShift));
+    const K32 tileEnd = (K32)(uintptr_t)tileEndAddr;
+    const K32 hint = (K32)(uintptr_t)hintAddr;
     const uint32_t tile = blockIdx.x;
-    const uint32_t seg = FindSegment(tile, args.hintShift, hint, tileEnd);
-    const K64 desc = (K64)(uintptr_t)args.desc + static_cast<uint64_t>(seg) * kA2aDescWords;
-    const uint64_t srcBase = desc[0];
-    const uint64_t dstBase = desc[1];
-    const uint64_t len = desc[2];
+    const uint32_t seg = FindSegment(tile, hintShift, hint, tileEnd);
+    const K64 desc = (K64)(uintptr_t)descAddr + static_cast<uint64_t>(seg) * kA2aDescWords;
+    uint64_t srcBase = desc[0];
+    uint64_t dstBase = desc[1];
+    uint64_t len = desc[2];
+    uint64_t firstTile = desc[3];
+    asm volatile("" : "+s"(srcBase), "+s"(dstBase), "+s"(len), "+s"(firstTile));
     uint64_t off;
     uint32_t bytes;
-    TileRange<kTile>(tile - static_cast<uint32_t>(desc[3]), TileLead(dstBase), len, &off, &bytes);
+    TileRange<kTile>(tile - static_cast<uint32_t>(firstTile), TileLead(dstBase), len, &off, &bytes);
     const uint8_t* src = reinterpret_cast<const uint8_t*>(srcBase + off);
     CopyTile<T, MODE, 1, true>(src, bytes, 1u, off, 3u, [&](uint32_t) { return dstBase; });
 }
@@ -359,18 +368,24 @@ hipError_t LaunchA2aT(const A2aArgs& a, uint32_t tiles, hipStream_t stream)
 // front of the aligned body and up to 15 behind it move byte by byte, and the body's vectors are dealt to the
 // lanes shifted by `lead`, so that every wavefront covers whole 128-byte lines.
 constexpr uint32_t kFanOutWaves = 16;
+static_assert(kFanOutWaves <= static_cast<uint32_t>(kMaxRanks), "a wavefront reads dst[wave] before it knows nDst");
 __global__ __launch_bounds__(64 * kFanOutWaves) void FanOutKernel(const FanOutArgs args)
 {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.y);
-    if (wave >= args.nDst) {
+    // Everything the wavefront needs, requested in one round of scalar loads (the workgroup has at most sixteen
+    // wavefronts, so dst[wave] is an entry of the table whatever nDst is).
+    uint32_t nDst = args.nDst;
+    uint64_t dstAddr = reinterpret_cast<uint64_t>(args.dst[wave]);
+    uint64_t srcAddr = reinterpret_cast<uint64_t>(args.src);
+    uint64_t bytes = args.bytes;
+    asm volatile("" : "+s"(nDst), "+s"(dstAddr), "+s"(srcAddr), "+s"(bytes));
+    if (wave >= nDst) {
         return;
     }
-    const uint64_t dstAddr = reinterpret_cast<uint64_t>(args.dst[wave]);
-    const uint64_t srcAddr = reinterpret_cast<uint64_t>(args.src);
     const uint32_t mis = static_cast<uint32_t>(srcAddr & 15u);
     uint64_t head = mis ? 16u - mis : 0u;
-    head = head < args.bytes ? head : args.bytes;
-    const uint64_t nVec = (args.bytes - head) >> 4;
+    head = head < bytes ? head : bytes;
+    const uint64_t nVec = (bytes - head) >> 4;
     const uint32_t lead = static_cast<uint32_t>(((srcAddr + head) >> 4) & 7u);
     const uint64_t u = static_cast<uint64_t>(blockIdx.x) * 64u + threadIdx.x;
     if (u >= lead && u < nVec + lead) {
@@ -379,7 +394,7 @@ __global__ __launch_bounds__(64 * kFanOutWaves) void FanOutKernel(const FanOutAr
         __builtin_nontemporal_store(v, (__attribute__((address_space(1))) U32x4*)(dstAddr + at));
     }
     const uint64_t bodyEnd = head + (nVec << 4);
-    const uint32_t edge = static_cast<uint32_t>(head + (args.bytes - bodyEnd));   // < 32
+    const uint32_t edge = static_cast<uint32_t>(head + (bytes - bodyEnd));   // < 32
     if (blockIdx.x == 0 && threadIdx.x < edge) {
         const uint64_t at = threadIdx.x < head ? threadIdx.x : bodyEnd + (threadIdx.x - head);
         const uint8_t byte = *((const __attribute__((address_space(1))) uint8_t*)(srcAddr + at));
