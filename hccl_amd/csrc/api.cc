@@ -687,6 +687,9 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
             }
             a.groupBlockEnd[g] = static_cast<uint32_t>(blocks < 0x7FFFFFFFull ? blocks : 0x7FFFFFFFull);
         }
+        for (uint32_t g = a.nGroup; g < 16; ++g) {
+            a.groupBlockEnd[g] = 0xFFFFFFFFu;   // the kernel reads sixteen entries in one go when there are that few groups
+        }
     }
     if (blocks == 0 || blocks > 0x7FFFFFFFull) {
         return HCCL_E_INTERNAL;

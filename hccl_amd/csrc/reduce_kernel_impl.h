@@ -627,21 +627,54 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     uint64_t gSrc;
     if (h.varGroups) {
         // Groups of unequal length own unequal shares of the grid: first group whose last block is not before us.
-        uint32_t lo = 0;
-        uint32_t hi = h.nGroup - 1;
-        while (lo < hi) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (blockIdx.x >= args.groupBlockEnd[mid]) {
-                lo = mid + 1;
-            } else {
-                hi = mid;
+        uint32_t firstBlock = 0;
+        uint32_t endBlock = 0xFFFFFFFFu;
+        g = 0;
+        if (h.nGroup <= 16) {
+            // Up to sixteen groups: their ends in one round of scalar loads (the launcher pads the table with
+            // 0xFFFFFFFF up to sixteen entries), then a count without branches: the ends do not decrease, so the
+            // groups that end at or before this workgroup are the ones in front of it, the last of them ends where
+            // this workgroup's group begins, and the first of the others is its own.
+            uint32_t ends[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                ends[j] = args.groupBlockEnd[j];
             }
+            asm volatile("" : "+s"(ends[0]), "+s"(ends[1]), "+s"(ends[2]), "+s"(ends[3]), "+s"(ends[4]), "+s"(ends[5]),
+                              "+s"(ends[6]), "+s"(ends[7]), "+s"(ends[8]), "+s"(ends[9]), "+s"(ends[10]), "+s"(ends[11]),
+                              "+s"(ends[12]), "+s"(ends[13]), "+s"(ends[14]), "+s"(ends[15]));
+            const uint32_t me = blockIdx.x;
+            const int used = h.nGroup <= 8 ? 8 : 16;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                if (j < used) {
+                    const bool before = ends[j] <= me;
+                    // 1 when the group ends at or before this workgroup, in scalar arithmetic (a comparison result
+                    // added up as a number would travel through a vector register)
+                    g += (ends[j] > me + 1u ? ends[j] : me + 1u) - (ends[j] > me ? ends[j] : me);
+                    firstBlock = before ? ends[j] : firstBlock;
+                    const uint32_t behind = before ? 0xFFFFFFFFu : ends[j];
+                    endBlock = behind < endBlock ? behind : endBlock;
+                }
+            }
+        } else {
+            uint32_t lo = 0;
+            uint32_t hi = h.nGroup - 1;
+            while (lo < hi) {
+                const uint32_t mid = (lo + hi) >> 1;
+                if (blockIdx.x >= args.groupBlockEnd[mid]) {
+                    lo = mid + 1;
+                } else {
+                    hi = mid;
+                }
+            }
+            g = lo;
+            firstBlock = g == 0 ? 0u : args.groupBlockEnd[g - 1];
+            endBlock = args.groupBlockEnd[g];
         }
-        g = lo;
         c = 0;
-        const uint32_t firstBlock = g == 0 ? 0u : args.groupBlockEnd[g - 1];
         blk = blockIdx.x - firstBlock;
-        blocksHere = args.groupBlockEnd[g] - firstBlock;
+        blocksHere = endBlock - firstBlock;
         gLen = args.groupLenV[g];
         gSrc = args.groupOffV[g];
     } else {
