@@ -42,7 +42,9 @@ struct IntOps {
         if constexpr (OP == kSum) {
             return static_cast<T>(static_cast<UT>(static_cast<UT>(src) + static_cast<UT>(dst)));
         } else if constexpr (OP == kProd) {
-            return static_cast<T>(static_cast<UT>(static_cast<UT>(src) * static_cast<UT>(dst)));
+            // (16-bit operands are widened first: promoted to int, the product of two large ones would overflow)
+            using Wide = decltype(UT{} + 0u);
+            return static_cast<T>(static_cast<UT>(static_cast<Wide>(static_cast<UT>(src)) * static_cast<Wide>(static_cast<UT>(dst))));
         } else if constexpr (OP == kMax) {
             return (src < dst) ? dst : src;
         } else {
@@ -67,7 +69,9 @@ struct Int8Ops {
         if constexpr (OP == kSum) {
             return static_cast<A>(static_cast<uint16_t>(static_cast<uint16_t>(src) + static_cast<uint16_t>(dst)));
         } else if constexpr (OP == kProd) {
-            return static_cast<A>(static_cast<uint16_t>(static_cast<uint16_t>(src) * static_cast<uint16_t>(dst)));
+            // (widened to 32 bits first: promoted to int, the product of two large 16-bit values would overflow)
+            return static_cast<A>(static_cast<uint16_t>(static_cast<uint32_t>(static_cast<uint16_t>(src)) *
+                                                        static_cast<uint32_t>(static_cast<uint16_t>(dst))));
         } else if constexpr (OP == kMax) {
             return (src < dst) ? dst : src;
         } else {
