@@ -640,7 +640,7 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     // keep non-temporal stores, 2-3 % faster there.  HCCL_AMD_STORE_POLICY = 0 / 1 forces one of them.
     const bool oneStream = a.dstOwn || a.nDst == 1;
     a.writeThrough = w->storePolicy != 2 ? w->storePolicy : (oneStream ? 1u : 0u);
-    // Many sources folded into one result stream: the wavefronts start on the sources' 128-byte lines (a
+    // Many sources folded into one result stream: the wavefronts start on the sources' 1 KiB boundaries (a
     // ReduceScatterV slice begins wherever its displacement puts it; measured 0.74 -> 0.80 of peak on uneven
     // slices) and the single store stream straddles.  HCCL_AMD_LEAD_FROM_SRC=0 keeps the destination's lines.
     a.leadFromSrc = (oneStream && w->leadFromSrc) ? 1u : 0u;

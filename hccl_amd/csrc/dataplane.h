@@ -80,7 +80,7 @@ struct ReduceHot {
     uint32_t threads; // workgroup size of the launch
     uint32_t vecBatch;       // leaves per load batch of the 128-bit path: 8 or 16 (picks the kernel instantiation)
     uint32_t writeThrough;   // 16-byte results leave through StoreStream16 instead of a non-temporal store
-    uint32_t leadFromSrc;    // wavefronts start on a 128-byte line of the sources instead of the destination
+    uint32_t leadFromSrc;    // wavefronts start on a 1 KiB boundary of the sources instead of the destination's
     uint32_t storeWaves;     // > 1: workgroups of 64 * storeWaves threads, wavefront 0 folds and wavefront k stores to
                              // destinations k, k + storeWaves, ... (threads must be 64, dstOwn 0); 0 or 1: every wavefront
                              // folds and stores its own tile
