@@ -140,6 +140,7 @@ def _bind(L):
     L.HcclCommDestroy.argtypes = [vp]
     L.HcclGetRankSize.argtypes = [vp, ctypes.POINTER(u32)]
     L.HcclGetRankId.argtypes = [vp, ctypes.POINTER(u32)]
+    L.HcclGetCommName.argtypes = [vp, ctypes.c_char_p]
     L.HcclGetErrorString.argtypes = [i32]
     L.HcclGetErrorString.restype = ctypes.c_char_p
     L.HcclGroupStart.argtypes = []
@@ -154,7 +155,7 @@ def _bind(L):
                  "HcclAlltoAll", "HcclAlltoAllVC", "HcclReduceScatterV", "HcclReduce", "HcclBroadcast", "HcclScatter",
                  "HcclSend", "HcclRecv", "HcclBatchSendRecv", "HcclBarrier",
                  "HcclCommInitAll", "HcclGetRootInfo", "HcclCommInitRootInfo", "HcclCommDestroy", "HcclGetRankSize",
-                 "HcclGetRankId", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
+                 "HcclGetRankId", "HcclGetCommName", "HcclGroupStart", "HcclGroupEnd", "HcclAmdSetAlgo", "HcclAmdGetAlgo",
                  "HcclAmdGetFoldProgram", "HcclAmdSetCclBufferSize", "HcclAmdGetCclBufferSize",
                  "HcclAmdAlltoAllVNoAlloc", "HcclAmdGetStuckCounters"):
         getattr(L, name).restype = ctypes.c_int
@@ -244,6 +245,13 @@ def get_rank_id(hccl_comm):
     v = ctypes.c_uint32()
     check(lib().HcclGetRankId(hccl_comm, ctypes.byref(v)), "HcclGetRankId")
     return v.value
+
+
+def get_comm_name(hccl_comm):
+    """The world's name: the same for every rank of a world, different between worlds."""
+    buf = ctypes.create_string_buffer(128)
+    check(lib().HcclGetCommName(hccl_comm, buf), "HcclGetCommName")
+    return buf.value.decode()
 
 
 def group_start():

@@ -2645,6 +2645,18 @@ HcclResult HcclGetRankId(HcclComm comm, uint32_t* rank)
     return HCCL_SUCCESS;
 }
 
+HcclResult HcclGetCommName(HcclComm comm, char* commName)
+{
+    CHK_PTR(comm, "comm");
+    CHK_PTR(commName, "commName");
+    CommRef ref = AsComm(comm);
+    if (ref.c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    snprintf(commName, HCCL_AMD_COMM_NAME_LENGTH, "hccl_amd_world_%llu", static_cast<unsigned long long>(ref.c->world->id));
+    return HCCL_SUCCESS;
+}
+
 const char* HcclGetErrorString(HcclResult code)
 {
     switch (code) {

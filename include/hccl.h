@@ -183,6 +183,12 @@ HcclResult HcclCommInitRootInfo(uint32_t nRanks, const HcclRootInfo* rootInfo, u
 HcclResult HcclCommDestroy(HcclComm comm);
 HcclResult HcclGetRankSize(HcclComm comm, uint32_t* rankSize);
 HcclResult HcclGetRankId(HcclComm comm, uint32_t* rank);
+/* Writes the world's name, NUL-terminated, into commName, which holds at least HCCL_AMD_COMM_NAME_LENGTH bytes: the
+ * same for every rank of a world, different between worlds.  (HCOMM's call of that name; the reference's entry
+ * points and custom-operator examples key their per-communicator state by it: src/ops/all_reduce/all_reduce.cc:124,
+ * src/ops/op_common/inc/alg_param.h:75 COMM_INDENTIFIER_MAX_LENGTH = 128.) */
+#define HCCL_AMD_COMM_NAME_LENGTH 128
+HcclResult HcclGetCommName(HcclComm comm, char* commName);
 const char* HcclGetErrorString(HcclResult code);
 
 /* Calls between Start and End on the calling thread are queued without blocking. */

@@ -223,6 +223,13 @@ def code_of(fn, *a, **k):
 
 def test_lifecycle_queries(world):
     assert [hccl_amd.get_rank_id(c) for c in world] == [0, 1, 2, 3]
+    names = {hccl_amd.get_comm_name(c) for c in world}
+    assert len(names) == 1 and 0 < len(names.pop()) < 128          # one name per world
+    other = hccl_amd.comm_init_all(2)
+    assert hccl_amd.get_comm_name(other[0]) == hccl_amd.get_comm_name(other[1]) != hccl_amd.get_comm_name(world[0])
+    for c in other:
+        hccl_amd.comm_destroy(c)
+    assert code_of(hccl_amd.get_comm_name, other[0]) == 1          # a destroyed handle
     assert hccl_amd.get_rank_size(world[2]) == 4
     assert code_of(hccl_amd.comm_init_all, 0) == 1
     assert code_of(hccl_amd.comm_init_all, 65) == 1
