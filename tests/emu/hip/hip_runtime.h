@@ -88,7 +88,9 @@ inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
 inline hipError_t hipSetDevice(int d) { return d == 0 ? hipSuccess : hipErrorInvalidDevice; }
 inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
-inline hipError_t hipMalloc(void** p, size_t n) { *p = malloc(n ? n : 1); return *p ? hipSuccess : hipErrorOutOfMemory; }
+// Whole 16-byte granules, as little as the GPU's allocator guarantees: the irregular copy path loads the aligned
+// vectors that cover its source bytes and may read, never use, the rest of the last granule.
+inline hipError_t hipMalloc(void** p, size_t n) { *p = malloc(n ? (n + 15) & ~size_t(15) : 16); return *p ? hipSuccess : hipErrorOutOfMemory; }
 inline hipError_t hipFree(void* p) { free(p); return hipSuccess; }
 inline hipError_t hipHostMalloc(void** p, size_t n, unsigned) { return hipMalloc(p, n); }
 inline hipError_t hipHostFree(void* p) { free(p); return hipSuccess; }

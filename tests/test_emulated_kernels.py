@@ -145,11 +145,14 @@ def test_host_layer_frees_what_it_allocates():
     assert "Sanitizer" not in proc.stdout, proc.stdout[-4000:]
 
 
-def test_native_thread_per_rank_example_runs_on_the_emulation():
-    """examples/collectives_threads.cc, the shape of the reference's own examples, under ThreadSanitizer."""
-    proc = run_native("collectives_threads", "tsan", 4, 5000)
-    assert proc.returncode == 0 and "PASS" in proc.stdout, proc.stdout[-4000:]
-    assert "ThreadSanitizer" not in proc.stdout, proc.stdout[-4000:]
+@pytest.mark.parametrize("ranks,count", [(8, 100003), (3, 1), (16, 4096), (1, 77), (7, 1001)])
+def test_native_thread_per_rank_example_runs_on_the_emulation(ranks, count):
+    """examples/collectives_threads.cc, the thirteen operators of the reference's own examples with a thread per rank,
+    under ThreadSanitizer and under AddressSanitizer (the first four cases are the ones the GPU test runs)."""
+    for sanitizer in ("tsan", "asan"):
+        proc = run_native("collectives_threads", sanitizer, ranks, count)
+        assert proc.returncode == 0 and proc.stdout.startswith("PASS"), sanitizer + "\n" + proc.stdout[-4000:]
+        assert "Sanitizer" not in proc.stdout, proc.stdout[-4000:]
 
 
 def test_the_package_never_loads_the_emulation():
