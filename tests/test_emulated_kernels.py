@@ -137,6 +137,17 @@ def test_host_layer_has_no_data_race_under_thread_sanitizer():
     assert "ThreadSanitizer" not in proc.stdout, proc.stdout[-4000:]
 
 
+@pytest.mark.parametrize("seed,sanitizer", [(1, "tsan"), (2, "tsan"), (3, "asan")])
+def test_faulty_calls_reach_every_rank_and_leave_the_sequence_intact(seed, sanitizer):
+    """tests/emu/host_fuzz.cc: seeded scripts of collectives in which, now and then, one rank passes a different count,
+    a null buffer or a type the operator does not take.  Every rank must see the same code for such a step, the
+    clean steps must give the right values and the calls after a fault must pair up as before; with a thread per
+    rank in two worlds and through groups in a third, at once."""
+    proc = run_native("host_fuzz", sanitizer, seed, 300, HCCL_EXEC_TIMEOUT="30", HCCL_AMD_LOG_LEVEL="0")
+    assert proc.returncode == 0 and "PASS" in proc.stdout, proc.stdout[-4000:]
+    assert "Sanitizer" not in proc.stdout, proc.stdout[-4000:]
+
+
 def test_host_layer_frees_what_it_allocates():
     """The same driver under AddressSanitizer with its leak check: worlds, pending calls, events and plans are gone
     when their last communicator has been destroyed."""
