@@ -146,6 +146,33 @@ __global__ __launch_bounds__(64 * W) void FanOut(Bufs b, const U4* source, int f
     }
 }
 
+// One source from memory to N destinations, the loading done once per tile: wavefront 0 loads the tile and hands it
+// to the other W - 1 wavefronts through LDS; wavefront w stores to destinations w, w + W, ...
+template <int N, int W>
+__global__ __launch_bounds__(64 * W) void FanOutShared(Bufs b, const U4* source)
+{
+    __shared__ U4 parked[64];
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned wave = threadIdx.x >> 6;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 64 + lane;
+    U4 v = {0u, 0u, 0u, 0u};
+    if (wave == 0) {
+        v = LoadNt(source + idx);
+        parked[lane] = v;
+    }
+    __syncthreads();
+    if (wave != 0) {
+        v = parked[lane];
+    }
+#pragma unroll
+    for (int i = 0; i < (N + W - 1) / W; ++i) {
+        const int d = static_cast<int>(wave) + W * i;
+        if (d < N) {
+            Store<1>(v, b.dst[d] + idx);
+        }
+    }
+}
+
 hipEvent_t g_start, g_stop;
 template <class F>
 float MsPerPass(F pass)
@@ -254,6 +281,12 @@ void Run(size_t bytesPerRank)
            }), moved);
     Report(N, "1 source to N destinations, one wavefront per destination, cached loads", MsPerPass([&] {
                hipLaunchKernelGGL((FanOut<N, N, 2>), dim3(blocks), dim3(64 * N), 0, 0, b, b.src[pass++ % N], 0, size_t(0));
+           }), moved);
+    Report(N, "1 source to N destinations, wavefront 0 loads, 2 wavefronts store", MsPerPass([&] {
+               hipLaunchKernelGGL((FanOutShared<N, 2>), dim3(blocks), dim3(128), 0, 0, b, b.src[pass++ % N]);
+           }), moved);
+    Report(N, "1 source to N destinations, wavefront 0 loads, 3 wavefronts store", MsPerPass([&] {
+               hipLaunchKernelGGL((FanOutShared<N, 3>), dim3(blocks), dim3(192), 0, 0, b, b.src[pass++ % N]);
            }), moved);
     for (int i = 0; i < N; ++i) {
         CK(hipFree((void*)b.src[i]));
