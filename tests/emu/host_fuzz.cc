@@ -2,8 +2,9 @@
 // ThreadSanitizer / AddressSanitizer: test infrastructure only.
 //
 // A seeded script of steps is shared by the ranks of a world (one host thread per rank, blocking calls).  A step is a
-// collective; in some steps one rank passes a count that differs from its peers', a null buffer, a data type the
-// operator does not take, or a zero count together with everybody else.  What must hold whatever the interleaving:
+// collective (the V operators among them, with counts and displacements that change from step to step); in some
+// steps one rank passes a count (for a V operator: a count table) that differs from its peers', a null buffer, a data
+// type the operator does not take, or a zero count together with everybody else.  What must hold whatever the interleaving:
 // every rank gets the same return code for the step (success, or the code of the fault), the results of the clean
 // steps are right, the calls after a fault pair up as if nothing had happened, and nothing hangs.  Prints PASS.
 #include <hip/hip_runtime.h>
@@ -23,7 +24,7 @@ std::atomic<int> g_failures{0};
 hipStream_t const kStream = reinterpret_cast<hipStream_t>(0x1000);
 
 enum Fault { kNone, kWrongCount, kNullBuffer, kBadType, kZeroCount, kFaults };
-enum Op { kAllReduce, kAllGather, kReduceScatter, kBroadcast, kReduce, kBarrier, kOps };
+enum Op { kAllReduce, kAllGather, kReduceScatter, kBroadcast, kReduce, kBarrier, kAllGatherV, kReduceScatterV, kAlltoAllV, kOps };
 
 struct Step {
     Op op;
@@ -87,8 +88,44 @@ void RankMain(uint32_t n, const HcclRootInfo* info, uint32_t rank, const std::ve
             in[i] = static_cast<int32_t>(rank * 100000 + k * 7 + i);
             out[i] = -1;
         }
+        // V operators: rank r contributes / receives vcount(r) elements, slices packed back to back; AlltoAllV trades
+        // pair(i, j) elements between ranks i and j in blocks of st.count.
+        auto vcount = [&](uint32_t r) { return (st.count + r * 13) % 97 + 1; };
+        auto pair = [&](uint32_t i, uint32_t j) { return (st.count + (i + j) * 7) % (st.count + 1); };
+        std::vector<uint64_t> counts(n), displs(n), sendCounts(n), blockAt(n);
+        uint64_t packed = 0;
+        for (uint32_t r = 0; r < n; ++r) {
+            counts[r] = vcount(r);
+            displs[r] = packed;
+            packed += counts[r];
+            sendCounts[r] = pair(rank, r);
+            blockAt[r] = r * (st.count + 1);
+        }
+        const bool isV = st.op == kAllGatherV || st.op == kReduceScatterV || st.op == kAlltoAllV;
+        if (isV && st.fault == kZeroCount) {
+            continue;   // the V operators have no single count to zero
+        }
+        if (isV && bad && st.fault == kWrongCount) {
+            counts[(rank + 1) % n] += 1;        // a table that differs from the peers'
+            sendCounts[(rank + 1) % n] += 1;    // an amount the receiver does not expect
+            if (n == 1) {
+                continue;
+            }
+        }
         HcclResult rc = HCCL_SUCCESS;
         switch (st.op) {
+            case kAllGatherV:
+                rc = HcclAllGatherV(send, vcount(rank), out.data(), counts.data(), displs.data(), dtype, comm, kStream);
+                break;
+            case kReduceScatterV:
+                rc = HcclReduceScatterV(send, counts.data(), displs.data(), out.data(), vcount(rank), dtype, HCCL_REDUCE_MAX, comm, kStream);
+                break;
+            case kAlltoAllV: {
+                std::vector<uint64_t> recvCounts(n);
+                for (uint32_t r = 0; r < n; ++r) recvCounts[r] = pair(r, rank);
+                rc = HcclAlltoAllV(send, sendCounts.data(), blockAt.data(), dtype, out.data(), recvCounts.data(), blockAt.data(), dtype, comm, kStream);
+                break;
+            }
             case kAllReduce: rc = HcclAllReduce(send, out.data(), count, dtype, HCCL_REDUCE_MAX, comm, kStream); break;
             case kAllGather: rc = HcclAllGather(send, out.data(), count, dtype, comm, kStream); break;
             case kReduceScatter: rc = HcclReduceScatter(send, out.data(), count, dtype, HCCL_REDUCE_MAX, comm, kStream); break;
@@ -130,6 +167,22 @@ void RankMain(uint32_t n, const HcclRootInfo* info, uint32_t rank, const std::ve
             case kReduce:
                 if (rank == st.root && out[0] != top) Fail("reduce value", rank, static_cast<int>(k), out[0], top);
                 break;
+            case kAllGatherV:
+                for (uint32_t r = 0; r < n; ++r) {
+                    const int32_t v = static_cast<int32_t>(r * 100000 + k * 7 + counts[r] - 1);
+                    if (out[displs[r] + counts[r] - 1] != v) Fail("all_gather_v value", rank, static_cast<int>(k), out[displs[r] + counts[r] - 1], v);
+                }
+                break;
+            case kReduceScatterV:
+                if (out[0] != top + static_cast<int32_t>(displs[rank])) Fail("reduce_scatter_v value", rank, static_cast<int>(k), out[0], top);
+                break;
+            case kAlltoAllV:
+                for (uint32_t r = 0; r < n; ++r) {
+                    if (pair(r, rank) == 0) continue;
+                    const int32_t v = static_cast<int32_t>(r * 100000 + k * 7 + rank * (st.count + 1));
+                    if (out[r * (st.count + 1)] != v) Fail("all_to_all_v value", rank, static_cast<int>(k), out[r * (st.count + 1)], v);
+                }
+                break;
             default: break;
         }
     }
@@ -146,7 +199,7 @@ void Grouped(uint32_t n, const std::vector<Step>& script)
     std::vector<std::vector<int32_t>> in(n, std::vector<int32_t>(cap)), out(n, std::vector<int32_t>(cap));
     for (size_t k = 0; k < script.size(); ++k) {
         const Step& st = script[k];
-        if (st.op == kBroadcast || st.op == kBarrier || st.fault == kZeroCount) {
+        if (st.op == kBroadcast || st.op >= kBarrier || st.fault == kZeroCount) {
             continue;
         }
         for (uint32_t r = 0; r < n; ++r) {
