@@ -5,6 +5,8 @@ Reads (as text; nothing of the reference is imported or run) the test cases of
     test/st/algorithm/testcase/alltoallvc_testcase.cc     the same
     test/st/algorithm/testcase/all_gather_v_testcase.cc   counts / displs + data type per TEST_F
     test/st/algorithm/testcase/reduce_scatter_v_testcase.cc, reduce_scatter_v_testcase_a3.cc   counts / displs / type / op
+(cases whose numbers are written out; the few that build them in loops or helper functions, the 32- and 128-rank
+"pairwise" matrices among them, are left out)
 and writes tests/golden/reference_st_shapes.json: one entry per test case with its name, the file and line it starts
 on, the rank count, the data type names and the numbers; for the cases that only assert the entry point's return code,
 that code ("expect") and whether the call was in place.  The reference checks these cases with a simulated world and
@@ -58,6 +60,9 @@ def main():
             continue
         for name, line, body in cases_of(path):
             counts, displs = numbers(body, r"\.counts"), numbers(body, r"\.displs")
+            made = re.search(r"MakeVDataDes\(\s*\{([^{}]*)\}\s*,\s*\{([^{}]*)\}\s*,", body)
+            if made and not counts:   # the helper form: MakeVDataDes({counts}, {displs}, type)
+                counts, displs = ([int(v) for v in re.findall(r"\d+", made.group(k))] for k in (1, 2))
             types = re.findall(r"HCCL_DATA_TYPE_(\w+)", body)
             ops = re.findall(r"HCCL_REDUCE_(\w+)", body)
             if counts and displs and len(counts) == len(displs) and types:

@@ -16,14 +16,13 @@ import pytest
 
 import hccl_amd
 import oracle
-from hccl_amd import HcclDataType as DT
+from hccl_amd import HcclDataType as DT, HcclReduceOp as OP
 
 from gpu_util import World, dev_zeros, rand_bytes, require_library_on_gpu, to_dev, to_host
 from test_gpu_parity import NP, check, gen
 
 pytestmark = pytest.mark.gpu
 FILL = 0xAB
-SUM = 0
 CASES = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_st_shapes.json")))
 
 
@@ -58,7 +57,7 @@ def test_the_catalogue_is_whole():
     kinds = {}
     for c in CASES:
         kinds[c["kind"]] = kinds.get(c["kind"], 0) + 1
-    assert kinds == {"all_to_all_v": 36, "all_to_all_vc": 36, "all_gather_v": 13, "reduce_scatter_v": 11}
+    assert kinds == {"all_to_all_v": 36, "all_to_all_vc": 36, "all_gather_v": 13, "reduce_scatter_v": 22}
 
 
 def matrix_of(case):
@@ -171,19 +170,24 @@ def test_all_gather_v_cases(worlds, case):
 
 @pytest.mark.parametrize("case", of_kind("reduce_scatter_v"))
 def test_reduce_scatter_v_cases(worlds, case):
-    """Sum, as in every case of the catalogue (reduce_scatter_v_testcase.cc:61).  Send displacements may overlap:
-    reduce_scatter_v_testcase_a3.cc:140 hands three ranks the same slice."""
+    """Sum where the case names no operation (reduce_scatter_v_testcase.cc:61), else the one it names.  Send
+    displacements may overlap: reduce_scatter_v_testcase_a3.cc:140 hands three ranks the same slice; ranks may
+    receive nothing (:285); counts may differ by a factor of 4096 (:293)."""
     n = case["ranks"]
     w = worlds(n)
     counts, displs, total = folded_layout(case)
     dtype = DT[case["types"][0]]
+    op = int(OP[case.get("ops", ["SUM"])[0]])
     rng = np.random.default_rng(len(case["name"]) + 1)
-    ins = [gen(dtype, SUM, rng, max(total, 1)) for _ in range(n)]
+    ins = [gen(dtype, op, rng, max(total, 1)) for _ in range(n)]
     want = [np.zeros(max(int(c), 1), dtype=NP[dtype]) for c in counts]
-    assert oracle.reduce_scatter_v(ins, want, counts, displs, int(dtype), SUM, acc=oracle.ACC_FP32) == 0
+    assert oracle.reduce_scatter_v(ins, want, counts, displs, int(dtype), op, acc=oracle.ACC_FP32) == 0
     sends = [to_dev(x) for x in ins]
     recvs = [dev_zeros(x.nbytes) for x in want]
-    w.reduce_scatter_v(sends, recvs, counts, displs, dtype, SUM)
+    w.reduce_scatter_v(sends, recvs, counts, displs, dtype, op)
     for r in range(n):
         c = int(counts[r])
-        check(dtype, SUM, to_host(recvs[r], NP[dtype])[:c], want[r][:c], "%s rank %d" % (case["source"], r))
+        got = to_host(recvs[r], NP[dtype])
+        check(dtype, op, got[:c], want[r][:c], "%s rank %d" % (case["source"], r))
+        if c == 0:
+            assert np.all(got.view(np.uint8) == FILL)           # a rank that receives nothing is left alone
