@@ -1,0 +1,73 @@
+"""CPU tier: what the compiler made of the kernels, read from the built library's own code objects.
+
+Every kernel of hccl_amd/libhccl_amd.so carries a metadata note (registers, spills, private memory).  The fold
+interpreter lives on the edge of the scalar register file: a change that looks harmless in the source can push a
+few uniform values into vector registers or into private memory, and the launch then runs at a fraction of its rate
+without any test failing.  This test fails instead.  Nothing runs on a GPU here; the note is written by hipcc when
+the library is built.
+"""
+import os
+import re
+import subprocess
+
+import pytest
+
+import hccl_amd
+
+LLVM = "/opt/rocm/llvm/bin"
+MAGIC = b"__CLANG_OFFLOAD_BUNDLE__"
+
+
+def kernel_notes(tmp_path):
+    """[{name, vgpr, sgpr, sgpr_spills, vgpr_spills, private_bytes, lds_bytes}] for every kernel of the library."""
+    fat = tmp_path / "fat.bin"
+    subprocess.check_call([LLVM + "/llvm-objcopy", "--dump-section", ".hip_fatbin=%s" % fat, hccl_amd.LIB_PATH,
+                           str(tmp_path / "unused.so")])
+    data = fat.read_bytes()
+    starts = [m.start() for m in re.finditer(re.escape(MAGIC), data)]   # one bundle per translation unit
+    kernels = []
+    for i, at in enumerate(starts):
+        bundle = tmp_path / ("bundle%d.bin" % i)
+        bundle.write_bytes(data[at:starts[i + 1] if i + 1 < len(starts) else len(data)])
+        obj = tmp_path / ("code%d.o" % i)
+        subprocess.check_call([LLVM + "/clang-offload-bundler", "--unbundle", "--type=o",
+                               "--targets=hipv4-amdgcn-amd-amdhsa--gfx950", "--input=%s" % bundle, "--output=%s" % obj])
+        notes = subprocess.run([LLVM + "/llvm-readelf", "--notes", str(obj)], stdout=subprocess.PIPE, text=True,
+                               check=True).stdout
+        for block in re.split(r"\n\s+- \.agpr_count:", notes)[1:]:
+            def field(key, block=block):
+                m = re.search(r"\.%s:\s+(\S+)" % key, block)
+                return m.group(1) if m else None
+            kernels.append({"name": field("name"), "vgpr": int(field("vgpr_count")), "sgpr": int(field("sgpr_count")),
+                            "sgpr_spills": int(field("sgpr_spill_count")), "vgpr_spills": int(field("vgpr_spill_count")),
+                            "private_bytes": int(field("private_segment_fixed_size")),
+                            "lds_bytes": int(field("group_segment_fixed_size"))})
+    return kernels
+
+
+@pytest.fixture(scope="module")
+def kernels(tmp_path_factory):
+    if not os.path.exists(hccl_amd.LIB_PATH):
+        pytest.fail("%s is missing: build the library first" % hccl_amd.LIB_PATH)
+    return kernel_notes(tmp_path_factory.mktemp("notes"))
+
+
+def test_every_translation_unit_is_there(kernels):
+    reduce_kernels = [k for k in kernels if "ReduceKernel" in k["name"]]
+    # 34 combinations of element type and operation, each with the eight-leaf and the sixteen-leaf load batch
+    assert len(reduce_kernels) == 68, sorted(k["name"] for k in reduce_kernels)
+    assert len(kernels) - len(reduce_kernels) == 21            # the copy, fan-out and AlltoAllV kernels
+
+
+def test_no_kernel_spills_or_uses_private_memory(kernels):
+    bad = [k for k in kernels if k["sgpr_spills"] or k["vgpr_spills"] or k["private_bytes"]]
+    assert not bad, bad
+
+
+def test_register_budgets(kernels):
+    """Vector registers: at most 96 for a fold kernel, so that five wavefronts fit a SIMD (512 / 96) whatever the
+    type and batch; at most 24 for the copy kernels.  Scalar registers cannot exceed what the hardware has; what is
+    checked for them is that the compiler did not have to spill (above)."""
+    for k in kernels:
+        limit = 96 if "ReduceKernel" in k["name"] else 24
+        assert k["vgpr"] <= limit, k
