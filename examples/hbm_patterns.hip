@@ -18,6 +18,9 @@
 //                                 the relative position of the peers' buffers is worth
 //   small messages                `hbm_patterns small <MiB>`: eight ranks of a few MiB over buffer sets in rotation (no
 //                                 pass finds its data cached): an empty launch of the same grid, reads, writes, fused
+//   scalar preamble               `hbm_patterns chain <ranks> <MiB>` (and the last rows of `small`): the fused pattern
+//                                 behind 0 .. 14 scalar loads that each wait for the one before, with one and with
+//                                 three wavefronts per tile: what fetching launch parameters one by one costs
 //
 // Build: make -C examples      Run: examples/bin/hbm_patterns [ranks=16] [MiB per rank=256]
 // Prints one line per pattern: time per pass, bytes moved per second, fraction of the 8 TB/s HBM peak.
@@ -117,6 +120,43 @@ __global__ __launch_bounds__(64 * W) void Streams(Bufs b, size_t nVec)
         }
     } else if (acc.x == 0x12345678u && acc.y == 0x9ABCDEF0u) {
         Store<STORE>(acc, b.dst[0] + idx);   // keeps the loads alive
+    }
+}
+
+// The fused pattern behind `rounds` dependent scalar loads (the address of each comes out of the one before): what a
+// kernel pays whose wavefronts fetch their launch parameters one after the other before the first vector load.
+// Table entries are below 256, so the chain's result adds nothing to the index; the compiler cannot know that.
+template <int N, int W>
+__global__ __launch_bounds__(64 * W) void StreamsAfterChain(Bufs b, const uint32_t* chain, int rounds, size_t nVec)
+{
+    typedef const __attribute__((address_space(4))) uint32_t* K32;
+    __shared__ U4 parked[64];
+    const K32 table = (K32)(uintptr_t)chain;
+    uint32_t x = blockIdx.x & 255u;
+    for (int r = 0; r < rounds; ++r) {
+        x = table[x & 255u];
+    }
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned wave = threadIdx.x >> 6;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 64 + lane + (x >> 31);
+    U4 acc = {1u, 2u, 3u, static_cast<uint32_t>(idx)};
+    if (wave == 0) {
+        acc = Fold<N>(b, idx);
+        if (W > 1) {
+            parked[lane] = acc;
+        }
+    }
+    if (W > 1) {
+        __syncthreads();
+        if (wave != 0) {
+            acc = parked[lane];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < (N + W - 1) / W; ++i) {
+        if (wave + W * i < N) {
+            Store<0>(acc, b.dst[wave + W * i] + idx);
+        }
     }
 }
 
@@ -334,6 +374,50 @@ void Placement(size_t bytesPerRank)
     CK(hipFree(raw));
 }
 
+// Rows of the fused pattern behind 0 .. 14 dependent scalar rounds, one and three wavefronts per tile.
+template <int N>
+void ChainRows(const Bufs* sets, int nSets, size_t nVec)
+{
+    uint32_t host[256];
+    for (uint32_t i = 0; i < 256; ++i) {
+        host[i] = (i * 37u + 11u) & 255u;
+    }
+    uint32_t* chain = nullptr;
+    CK(hipMalloc((void**)&chain, sizeof host));
+    CK(hipMemcpy(chain, host, sizeof host, hipMemcpyHostToDevice));
+    const unsigned blocks = static_cast<unsigned>(nVec / 64);
+    const double moved = 2.0 * N * nVec * 16;
+    int pass = 0;
+    for (int rounds : {0, 2, 4, 8, 14}) {
+        char what[128];
+        snprintf(what, sizeof what, "fused behind %2d dependent scalar loads, one wavefront per tile", rounds);
+        Report(N, what, MsPerPass([&] {
+                   hipLaunchKernelGGL((StreamsAfterChain<N, 1>), dim3(blocks), dim3(64), 0, 0, sets[pass++ % nSets], chain, rounds, nVec);
+               }), moved);
+        snprintf(what, sizeof what, "fused behind %2d dependent scalar loads, stores shared by 3 wavefronts", rounds);
+        Report(N, what, MsPerPass([&] {
+                   hipLaunchKernelGGL((StreamsAfterChain<N, 3>), dim3(blocks), dim3(192), 0, 0, sets[pass++ % nSets], chain, rounds, nVec);
+               }), moved);
+    }
+    CK(hipFree(chain));
+}
+
+template <int N>
+void Chain(size_t bytesPerRank)
+{
+    Bufs b{};
+    for (int i = 0; i < N; ++i) {
+        CK(hipMalloc((void**)&b.src[i], bytesPerRank));
+        CK(hipMemset((void*)b.src[i], 1 + i, bytesPerRank));
+        CK(hipMalloc((void**)&b.dst[i], bytesPerRank));
+    }
+    ChainRows<N>(&b, 1, bytesPerRank / 16);
+    for (int i = 0; i < N; ++i) {
+        CK(hipFree((void*)b.src[i]));
+        CK(hipFree(b.dst[i]));
+    }
+}
+
 void Small(size_t bytesPerRank)
 {
     constexpr int N = 8;
@@ -355,6 +439,7 @@ void Small(size_t bytesPerRank)
     Report(N, "writes alone, non-temporal", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, false, true, 0>), dim3(blocks), dim3(64), 0, 0, sets[pass++ % kSets], nVec); }), half);
     Report(N, "fused N reads + N writes, non-temporal stores", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 1, true, true, 0>), dim3(blocks), dim3(64), 0, 0, sets[pass++ % kSets], nVec); }), 2 * half);
     Report(N, "fused, stores shared by 2 wavefronts", MsPerPass([&] { hipLaunchKernelGGL((Streams<N, 2, true, true, 0>), dim3(blocks), dim3(128), 0, 0, sets[pass++ % kSets], nVec); }), 2 * half);
+    ChainRows<N>(sets, kSets, nVec);
     for (Bufs& b : sets) {
         for (int i = 0; i < N; ++i) {
             CK(hipFree((void*)b.src[i]));
@@ -365,12 +450,13 @@ void Small(size_t bytesPerRank)
 
 int main(int argc, char** argv)
 {
-    if (argc > 1 && (strcmp(argv[1], "place") == 0 || strcmp(argv[1], "small") == 0)) {
-        const bool place = argv[1][0] == 'p';
+    if (argc > 1 && (strcmp(argv[1], "place") == 0 || strcmp(argv[1], "small") == 0 || strcmp(argv[1], "chain") == 0)) {
+        const bool chain = argv[1][0] == 'c';
+        const bool place = argv[1][0] == 'p' || chain;   // both take <ranks> <MiB>
         const int ranks = place && argc > 2 ? atoi(argv[2]) : 8;
         const size_t mibArg = static_cast<size_t>(atoi(argc > (place ? 3 : 2) ? argv[place ? 3 : 2] : "4"));
         if (mibArg < 1 || mibArg > 1024 || (ranks != 6 && ranks != 8 && ranks != 16)) {
-            printf("usage: hbm_patterns place <ranks: 6, 8 or 16> <MiB per rank: 1 .. 1024> | hbm_patterns small <MiB per rank>\n");
+            printf("usage: hbm_patterns place|chain <ranks: 6, 8 or 16> <MiB per rank: 1 .. 1024> | hbm_patterns small <MiB per rank>\n");
             return 1;
         }
         CK(hipEventCreate(&g_start));
@@ -378,6 +464,14 @@ int main(int argc, char** argv)
         printf("pattern%68s time per pass   moved   of 8 TB/s\n", "");
         if (!place) {
             Small(mibArg << 20);
+        } else if (chain) {
+            if (ranks == 16) {
+                Chain<16>(mibArg << 20);
+            } else if (ranks == 8) {
+                Chain<8>(mibArg << 20);
+            } else {
+                Chain<6>(mibArg << 20);
+            }
         } else if (ranks == 16) {
             Placement<16>(mibArg << 20);
         } else if (ranks == 8) {
