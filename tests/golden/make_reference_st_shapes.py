@@ -5,6 +5,8 @@ Reads (as text; nothing of the reference is imported or run) the test cases of
     test/st/algorithm/testcase/alltoallvc_testcase.cc     the same
     test/st/algorithm/testcase/all_gather_v_testcase.cc   counts / displs + data type per TEST_F
     test/st/algorithm/testcase/reduce_scatter_v_testcase.cc, reduce_scatter_v_testcase_a3.cc   counts / displs / type / op
+    test/st/algorithm/testcase/broadcast_testcase.cc      rank count, count, type, root per TEST_F
+    test/st/algorithm/testcase/scatter_testcase.cc        root, count (per rank), type per TEST_F
 (cases whose numbers are written out; the few that build them in loops or helper functions, the 32- and 128-rank
 "pairwise" matrices among them, are left out)
 and writes tests/golden/reference_st_shapes.json: one entry per test case with its name, the file and line it starts
@@ -43,6 +45,56 @@ def numbers(body, name):
     return [int(v.rstrip("uUlL")) for v in vals] if all(re.fullmatch(r"\d+[uUlL]*", v) for v in vals) else None
 
 
+def product(expr):
+    """An element count written as a number or a product of numbers, casts allowed: `(uint64_t)1024 * 1024 * 4`."""
+    expr = re.sub(r"\(\s*(uint64_t|u64)\s*\)|static_cast<\w+>", "", expr).replace("(", "").replace(")", "")
+    factors = [f.strip() for f in expr.split("*")]
+    if not all(re.fullmatch(r"\d+[uUlL]*", f) for f in factors):
+        return None
+    value = 1
+    for f in factors:
+        value *= int(f.rstrip("uUlL"))
+    return value
+
+
+def ranks_of(body):
+    """Rank count of the topology a case builds: the devices listed in `TopoMeta topoMeta{{{..}, {..}}}`, or the
+    product of the three numbers of `GenTopoMeta(topoMeta, pods, servers, devices)`."""
+    m = re.search(r"TopoMeta\s+topoMeta\s*\{(.*?)\}\s*;", body, re.S)
+    if m:
+        return len(re.findall(r"\d+", m.group(1)))
+    m = re.search(r"GenTopoMeta\(\s*topoMeta\s*,\s*(\d+)\s*,\s*(\d+)\s*,\s*(\d+)\s*\)", body)
+    return int(m.group(1)) * int(m.group(2)) * int(m.group(3)) if m else None
+
+
+def rooted_cases(out):
+    # broadcast_testcase.cc: either named locals (rankSize, count, dataType, root) or the arguments written into the call
+    fn = "broadcast_testcase.cc"
+    for name, line, body in cases_of(os.path.join(REF, fn)):
+        body = re.sub(r"//[^\n]*", "", body)
+        types = re.findall(r"HCCL_DATA_TYPE_(\w+)", body)
+        call = re.search(r"RunBroadcastTest\(\s*topoMeta\s*,\s*([^,]+),\s*([^,]+),\s*[\w:]+\s*,\s*([^,]+),", body)
+        if not (types and call):
+            continue
+        local = {k: re.search(r"\b%s\s*=\s*([^;]+);" % k, body) for k in ("rankSize", "count", "root")}
+        arg = [local[k].group(1) if local[k] and a.strip() == k else a for k, a in zip(("rankSize", "count", "root"), call.groups())]
+        ranks, count, root = (product(a) for a in arg)
+        if None in (ranks, count, root) or ranks != ranks_of(body):
+            continue
+        out.append({"kind": "broadcast", "name": name, "source": "%s:%d" % (fn, line), "ranks": ranks,
+                    "types": [types[0]], "count": count, "root": root})
+    # scatter_testcase.cc: RunScatterTest(root, topoMeta, count, type)
+    fn = "scatter_testcase.cc"
+    for name, line, body in cases_of(os.path.join(REF, fn)):
+        body = re.sub(r"//[^\n]*", "", body)
+        call = re.search(r"RunScatterTest\w*\(\s*(\d+)\s*,\s*topoMeta\s*,\s*([^,]+),\s*HcclDataType::HCCL_DATA_TYPE_(\w+)\s*\)", body)
+        ranks = ranks_of(body)
+        if not call or ranks is None or product(call.group(2)) is None:
+            continue
+        out.append({"kind": "scatter", "name": name, "source": "%s:%d" % (fn, line), "ranks": ranks,
+                    "types": [call.group(3)], "count": product(call.group(2)), "root": int(call.group(1))})
+
+
 def main():
     out = []
     for fn, kind in (("alltoallv_testcase.cc", "all_to_all_v"), ("alltoallvc_testcase.cc", "all_to_all_vc")):
@@ -76,6 +128,7 @@ def main():
                     entry["in_place"] = m.group(1) == "true"
                     entry["expect"] = m.group(2)
                 out.append(entry)
+    rooted_cases(out)
     path = os.path.join(HERE, "reference_st_shapes.json")
     with open(path, "w") as f:
         json.dump(out, f, indent=None, separators=(",", ":"))

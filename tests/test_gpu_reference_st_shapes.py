@@ -1,8 +1,9 @@
-"""GPU parity on the shapes of the reference's own system tests for the V operators.
+"""GPU parity on the shapes of the reference's own system tests for the V operators, Broadcast and Scatter.
 
 tests/golden/reference_st_shapes.json holds, as data, every case of test/st/algorithm/testcase/alltoallv_testcase.cc,
-alltoallvc_testcase.cc, all_gather_v_testcase.cc and reduce_scatter_v_testcase*.cc: rank count, data type(s), the
-send-count matrix or the counts / displacements, and for the cases that only assert a return code, that code.  The
+alltoallvc_testcase.cc, all_gather_v_testcase.cc, reduce_scatter_v_testcase*.cc, broadcast_testcase.cc and
+scatter_testcase.cc whose numbers are written out: rank count, data type(s), the send-count matrix, the counts /
+displacements or count and root, and for the cases that only assert a return code, that code.  The
 reference runs them in a simulated world and verifies the task graph; here the same shapes go through the C ABI on
 real buffers and are compared with the oracle, byte for byte.  Counts in the millions and beyond (the catalogue goes
 up to 10 Gi elements) are folded down to a few thousand elements, keeping zero at zero, small counts as they are,
@@ -57,7 +58,8 @@ def test_the_catalogue_is_whole():
     kinds = {}
     for c in CASES:
         kinds[c["kind"]] = kinds.get(c["kind"], 0) + 1
-    assert kinds == {"all_to_all_v": 36, "all_to_all_vc": 36, "all_gather_v": 13, "reduce_scatter_v": 22}
+    assert kinds == {"all_to_all_v": 36, "all_to_all_vc": 36, "all_gather_v": 13, "reduce_scatter_v": 22,
+                     "broadcast": 34, "scatter": 24}
 
 
 def matrix_of(case):
@@ -191,3 +193,38 @@ def test_reduce_scatter_v_cases(worlds, case):
         check(dtype, op, got[:c], want[r][:c], "%s rank %d" % (case["source"], r))
         if c == 0:
             assert np.all(got.view(np.uint8) == FILL)           # a rank that receives nothing is left alone
+
+
+@pytest.mark.parametrize("case", of_kind("broadcast"))
+def test_broadcast_cases(worlds, case):
+    """Up to 64 ranks, roots in every position of the reference's multi-level topologies (here one flat world)."""
+    n, root, count = case["ranks"], case["root"], fold(case["count"])
+    w = worlds(n)
+    dtype = DT[case["types"][0]]
+    esz = oracle.lib().orc_dtype_size(int(dtype))
+    rng = np.random.default_rng(len(case["name"]) + root)
+    host = [rand_bytes(rng, count * esz) for _ in range(n)]
+    want = [x.copy() for x in host]
+    assert oracle.broadcast(want, count, int(dtype), root) == 0
+    bufs = [to_dev(x) for x in host]
+    w.broadcast(bufs, count, dtype, root)
+    for r in range(n):
+        assert np.array_equal(to_host(bufs[r], np.uint8), want[r]), (case["source"], r)
+        assert np.array_equal(want[r], host[root])
+
+
+@pytest.mark.parametrize("case", of_kind("scatter"))
+def test_scatter_cases(worlds, case):
+    n, root, count = case["ranks"], case["root"], fold(case["count"])
+    w = worlds(n)
+    dtype = DT[case["types"][0]]
+    esz = oracle.lib().orc_dtype_size(int(dtype))
+    rng = np.random.default_rng(len(case["name"]) + 3 * root)
+    ins = [rand_bytes(rng, n * count * esz) for _ in range(n)]
+    want = [np.zeros(count * esz, dtype=np.uint8) for _ in range(n)]
+    assert oracle.scatter(ins, want, count, int(dtype), root) == 0
+    sends = [to_dev(ins[r]) if r == root else None for r in range(n)]      # only the root has a send buffer
+    recvs = [dev_zeros(count * esz) for _ in range(n)]
+    w.scatter(sends, recvs, count, dtype, root)
+    for r in range(n):
+        assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), (case["source"], r)
