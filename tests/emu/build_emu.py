@@ -66,12 +66,14 @@ def prepare_sources():
     return digest.hexdigest()
 
 
-SANITIZE = {"": [], "asan": ["-fsanitize=address", "-fno-omit-frame-pointer"],
+# "asan" is AddressSanitizer together with the undefined-behaviour checks (one runtime serves both); a finding of
+# either kind ends the process.
+SANITIZE = {"": [], "asan": ["-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer"],
             "tsan": ["-fsanitize=thread", "-fno-omit-frame-pointer"]}
 
 
 def flags(asan):
-    f = [CLANG, "-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-ffp-contract=off", "-mf16c", "-pthread",
+    f = [CLANG, "-x", "c++", "-std=c++17", "-O1", "-gline-tables-only", "-fPIC", "-ffp-contract=off", "-mf16c", "-pthread",
          "-Wno-unknown-attributes", "-Wno-ignored-attributes",
          "-I" + HERE, "-I" + os.path.join(ROOT, "include"), "-I" + SRC,
          "-D__builtin_amdgcn_readfirstlane=emu::ReadFirstLane", "-D__builtin_amdgcn_update_dpp=emu::UpdateDpp",

@@ -7,8 +7,9 @@ HCCL_AMD_TEST_EMU=1:
 tests/gpu_util.py hands out host buffers, tests/conftest.py points the Python mirror at the emulation library.
 
 What this checks without a GPU: the kernels' index arithmetic, fold interpreter, heads / tails, tile tables and the
-host layer's launch geometry give the oracle's bits, and, in the AddressSanitizer run, touch no byte outside the
-16-byte granules of the buffers they were given.  It is how a kernel change is tried before it goes to the GPU.
+host layer's launch geometry give the oracle's bits, touch no byte outside the 16-byte granules of the buffers
+they were given (AddressSanitizer) and do nothing the language leaves undefined, such as an overflowing signed
+product or a misaligned vector access (the undefined-behaviour checks of the same build).  It is how a kernel change is tried before it goes to the GPU.
 It says nothing about timing or about what the GPU compiler makes of the code: the `-m gpu` run stays the
 parity gate.  The emulation is test infrastructure; the package never loads it.
 """
