@@ -71,3 +71,19 @@ def test_register_budgets(kernels):
     for k in kernels:
         limit = 96 if "ReduceKernel" in k["name"] else 24
         assert k["vgpr"] <= limit, k
+
+
+def test_uniform_values_are_uniform_for_the_compiler_too(kernels, tmp_path_factory):
+    """The kernels pin launch scalars, program words and leaf addresses in scalar registers (the "+s" operands of
+    their empty assembly statements).  Had one of them been computed per lane, the compiler would satisfy the
+    constraint by taking the first lane's value, silently: a v_readfirstlane in the code.  The only one the sources
+    ask for themselves is the fan-out kernel's wavefront index."""
+    tmp = tmp_path_factory.mktemp("code")
+    kernel_notes(tmp)
+    counts = {}
+    for obj in sorted(tmp.glob("code*.o")):
+        text = subprocess.run([LLVM + "/llvm-objdump", "-d", "--mcpu=gfx950", str(obj)], stdout=subprocess.PIPE,
+                              text=True, check=True).stdout
+        assert "s_endpgm" in text                       # the listing is real
+        counts[obj.name] = text.count("v_readfirstlane")
+    assert sorted(counts.values()) == [0] * (len(counts) - 1) + [1], counts
