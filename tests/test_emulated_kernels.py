@@ -139,6 +139,15 @@ def test_host_layer_has_no_data_race_under_thread_sanitizer():
     assert "ThreadSanitizer" not in proc.stdout, proc.stdout[-4000:]
 
 
+def test_wavefronts_that_share_a_tiles_stores_do_not_race():
+    """The same driver with the reduce kernel's shared-store form forced: the folding wavefront parks a tile in one of
+    two LDS slots, one barrier per tile, the storing wavefronts read it.  Lanes are OS threads here, so
+    ThreadSanitizer sees a slot that is written again before every reader is through."""
+    proc = run_native("host_stress", "tsan", 120, HCCL_AMD_REDUCE_STORE_WAVES="3")
+    assert proc.returncode == 0 and "PASS" in proc.stdout, proc.stdout[-4000:]
+    assert "ThreadSanitizer" not in proc.stdout, proc.stdout[-4000:]
+
+
 @pytest.mark.parametrize("seed,sanitizer", [(1, "tsan"), (2, "tsan"), (3, "asan")])
 def test_faulty_calls_reach_every_rank_and_leave_the_sequence_intact(seed, sanitizer):
     """tests/emu/host_fuzz.cc: seeded scripts of collectives in which, now and then, one rank passes a different count,
