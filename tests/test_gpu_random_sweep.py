@@ -1,5 +1,7 @@
 """Seeded random sweep over (collective, type, op, algorithm, rank count, element count, buffer alignment,
 staging-buffer size): every case is compared with the oracle like the hand-picked cases of test_gpu_parity.py."""
+import os
+
 import numpy as np
 import pytest
 
@@ -10,6 +12,8 @@ from gpu_util import World, require_library_on_gpu
 from test_gpu_parity import MAX, MIN, NP, PROD, SUM, run_all_reduce, run_reduce_scatter
 
 pytestmark = pytest.mark.gpu
+# Another number here draws other cases (used for longer runs by hand, mostly on the CPU emulation).
+SWEEP_SEED = int(os.environ.get("HCCL_AMD_TEST_SWEEP_SEED", "90000"))
 
 TYPES = [DT.INT8, DT.INT16, DT.INT32, DT.INT64, DT.UINT64, DT.FP16, DT.BFP16, DT.FP32, DT.FP64]
 AR_ALGOS = ["mesh", "ring", "rhd", "nhr", "order_preserved", "mesh_symmetric", "mesh_chunk"]
@@ -45,7 +49,7 @@ FORMS = {
 @pytest.mark.parametrize("form", list(FORMS))
 @pytest.mark.parametrize("n", [2, 3, 4, 6, 7, 8, 12, 16])
 def test_random_reduce_cases(monkeypatch, n, form):
-    rng = np.random.default_rng(90_000 + n)
+    rng = np.random.default_rng(SWEEP_SEED + n)
     env = dict(FORMS[form])
     if "HCCL_AMD_ALLREDUCE_PIECE_BYTES" in env:
         env["HCCL_AMD_ALLREDUCE_PIECE_BYTES"] = str([4096, 20_480, 65_536][n % 3])
