@@ -35,6 +35,24 @@ def test_step_counts(orc):
         assert orc.lib().orc_nhr_step_num(n) == steps
 
 
+def test_nhr_steps_match_the_reference_golden_values(orc):
+    """The step tables the reference's own unit test holds for 2, 3, 4, 5, 6 and 8 ranks
+    (test/ut/reduce_scatter_nhr_dpu/test_nhr_geometry.cc:51-84), and its step counts (:226-236)."""
+    for n, want in GOLD["nhr_step_num"]:
+        assert orc.lib().orc_nhr_step_num(n) == want
+    seen = 0
+    for case in GOLD["nhr_golden_steps"]:
+        n, rank = case["rankSize"], case["rank"]
+        assert orc.lib().orc_nhr_step_num(n) == len(case["steps"])
+        for step, want in enumerate(case["steps"]):
+            rc, to, frm, tx, rx = orc.nhr_step_info(n, rank, step)
+            assert rc == 0, (n, rank, step)
+            assert (to, frm, len(tx), tx, rx) == (want["toRank"], want["fromRank"], want["nSlices"], want["tx"], want["rx"]), \
+                (n, rank, step)
+            seen += 1
+    assert seen == 25
+
+
 def test_round_up(orc):
     assert orc.lib().orc_round_up(10, 4) == 3
     assert orc.lib().orc_round_up(8, 4) == 2
