@@ -240,6 +240,7 @@ def test_rhd_tail_loop_plan(orc):
             tail = c
         processed += c
     assert processed == g["totalCount"] and tail == g["tailCount"]
+    assert sel(144, 72, 12) == 72      # test/ut/common/hostdpu_inline_reduce/all_reduce_rhd_test.cc:88-94: a full loop, no tail
     for ranks in (2, 3, 6, 12, 16, 24, 72):       # every element processed exactly once
         cap = 3 * ranks
         for total in range(0, 300):
