@@ -12,7 +12,7 @@ Reads (as text; nothing of the reference is imported or run) the test cases of
 and writes tests/golden/reference_st_shapes.json: one entry per test case with its name, the file and line it starts
 on, the rank count, the data type names and the numbers; for the cases that only assert the entry point's return code,
 that code ("expect") and whether the call was in place.  The reference checks these cases with a simulated world and
-a verifier of the data flow, not with values; here tests/test_gpu_reference_st_shapes.py replays the shapes (scaled
+a verifier of the data flow, not with values; here tests/test_wide_gpu_reference_st_shapes.py replays the shapes (scaled
 down where a count is in the millions) against the oracle.
 
 Usage (in the container that holds /root/reference):  python tests/golden/make_reference_st_shapes.py

@@ -2,7 +2,7 @@
 
 tests/emu compiles hccl_amd/csrc (host layer and gfx950 kernels, inline assembly replaced by its plain meaning)
 against a stand-in HIP runtime that runs every launch workgroup by workgroup and lane by lane on the CPU.  The
-parity tests of nine tests/test_gpu_*.py files then run unchanged in a pytest process of their own with
+parity tests of ten GPU test files then run unchanged in a pytest process of their own with
 HCCL_AMD_TEST_EMU=1:
 tests/gpu_util.py hands out host buffers, tests/conftest.py points the Python mirror at the emulation library.
 
@@ -25,10 +25,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, os.path.join(ROOT, "tests", "emu"))
 import build_emu  # noqa: E402
 
-FILES = ["tests/test_gpu_parity.py", "tests/test_gpu_copies.py", "tests/test_gpu_copy_random_sweep.py",
-         "tests/test_gpu_rooted_and_v_ops.py",
+FILES = ["tests/test_gpu_parity.py", "tests/test_gpu_copies.py", "tests/test_wide_gpu_copy_sweep.py",
+         "tests/test_wide_gpu_rooted_sweep.py", "tests/test_gpu_rooted_and_v_ops.py",
          "tests/test_gpu_random_sweep.py", "tests/test_gpu_point_to_point.py",
-         "tests/test_gpu_reference_python_suites.py", "tests/test_gpu_reference_st_shapes.py",
+         "tests/test_gpu_reference_python_suites.py", "tests/test_wide_gpu_reference_st_shapes.py",
          "tests/test_zz_no_alloc.py"]
 # Left out: tests that allocate or compute with torch on the GPU themselves (graphs, own streams, device-side
 # generators) and tests whose size is meant for the GPU.
