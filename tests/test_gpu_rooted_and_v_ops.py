@@ -135,14 +135,6 @@ def test_reduce_scatter_v_other_ops(worlds, dtype, op):
     run_rsv(worlds(5), dtype, op, 1, 3000, "gaps", 31 + int(dtype) + op)
 
 
-@pytest.mark.parametrize("n", [2, 9, 16, 17, 33])
-def test_reduce_scatter_v_rank_counts_either_side_of_the_sixteen_group_table(worlds, n):
-    """Up to sixteen slices a workgroup finds its slice by counting the slices' ends, which it reads in one go;
-    beyond that it searches.  Both with an empty slice among them."""
-    run_rsv(worlds(n), DT.INT32, SUM, 1, 3000, "gaps", 70 + n)
-    run_rsv(worlds(n), DT.FP16, MAX, 200, 2000, "prefix", 90 + n)
-
-
 def test_reduce_scatter_v_large_uneven_slices(worlds):
     run_rsv(worlds(6), DT.BFP16, SUM, 1 << 18, 1 << 21, "aligned", 5)
     run_rsv(worlds(6), DT.FP32, SUM, 1 << 16, 1 << 19, "prefix", 6, pad=4)

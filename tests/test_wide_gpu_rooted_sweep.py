@@ -9,7 +9,7 @@ import oracle
 from hccl_amd import HcclDataType as DT
 
 from gpu_util import World, dev_zeros, require_library_on_gpu, to_dev, to_host
-from test_gpu_parity import NP, PROD, SUM, check, gen
+from test_gpu_parity import MAX, NP, PROD, SUM, check, gen
 from test_gpu_random_sweep import SWEEP_SEED, TYPES, pick_count
 from test_gpu_rooted_and_v_ops import RSV_TYPES, run_rsv
 
@@ -58,4 +58,16 @@ def test_random_reduce_and_reduce_scatter_v_cases(n):
     finally:
         w.set_algo(hccl_amd.OpKind.REDUCE, "mesh")
         w.set_algo(hccl_amd.OpKind.REDUCE_SCATTER, "mesh")
+        w.close()
+
+
+@pytest.mark.parametrize("n", [2, 9, 16, 17, 33])
+def test_reduce_scatter_v_rank_counts_either_side_of_the_sixteen_group_table(n):
+    """Up to sixteen slices a workgroup finds its slice by counting the slices' ends, which it reads in one go;
+    beyond that it searches.  Both with an empty slice among them."""
+    w = World(n)
+    try:
+        run_rsv(w, DT.INT32, SUM, 1, 3000, "gaps", 70 + n)
+        run_rsv(w, DT.FP16, MAX, 200, 2000, "prefix", 90 + n)
+    finally:
         w.close()
