@@ -592,26 +592,57 @@ __device__ __forceinline__ Pack<typename E::S, W> ReduceValue(const ProgramView&
 
 // The value of ReduceValue written to the destinations firstDst, firstDst + dstStep, ... of the launch (all of
 // them with 0 and 1), or to the group's own destination.
-template <class S, int W>
+// `ownOrFirst` is the address the kernel fetched ahead with its second round of scalar loads: the group's own
+// destination, or destination 0.  A launch with one destination per result (ReduceScatter(V), Reduce, the fold of
+// the two-kernel AllReduce) then stores without another scalar load between the fold and the store.
+// kAhead: firstDst and dstStep are uniform (every wavefront stores to every destination), so the remaining
+// addresses can be fetched four at a time.
+template <class S, int W, bool kAhead>
 __device__ __forceinline__ void StoreResult(const ReduceArgs& args, const ReduceHot& h, const Pack<S, W>& out,
-                                            uint64_t elemOff, uint32_t group, uint32_t firstDst, uint32_t dstStep)
+                                            uint64_t elemOff, uint64_t ownOrFirst, uint32_t firstDst, uint32_t dstStep)
 {
+    void* const ahead = reinterpret_cast<void*>(ownOrFirst);
     if (h.dstOwn) {
-        StorePack<S, W>(args.dst[group], elemOff, out, h.writeThrough != 0);
+        StorePack<S, W>(ahead, elemOff, out, h.writeThrough != 0);
     } else {
-        for (uint32_t d = firstDst; d < h.nDst; d += dstStep) {
-            StorePack<S, W>(args.dst[d], elemOff, out, h.writeThrough != 0);
+        uint32_t d = firstDst;
+        if (d == 0) {
+            StorePack<S, W>(ahead, elemOff, out, h.writeThrough != 0);
+            d = dstStep;
+        }
+        if constexpr (!kAhead) {
+            for (; d < h.nDst; d += dstStep) {
+                StorePack<S, W>(args.dst[d], elemOff, out, h.writeThrough != 0);
+            }
+            return;
+        }
+        // The other destinations four at a time: their addresses are requested together, one round of scalar loads
+        // per four stores instead of one per store (indices past the table are never used and read entry 0).
+        for (; d < h.nDst; d += 4 * dstStep) {
+            uint64_t to[4];
+#pragma unroll
+            for (uint32_t k = 0; k < 4; ++k) {
+                const uint32_t dk = d + k * dstStep;
+                to[k] = reinterpret_cast<uint64_t>(args.dst[dk < static_cast<uint32_t>(kMaxRanks) ? dk : 0u]);
+            }
+            asm volatile("" : "+s"(to[0]), "+s"(to[1]), "+s"(to[2]), "+s"(to[3]));
+#pragma unroll
+            for (uint32_t k = 0; k < 4; ++k) {
+                if (d + k * dstStep < h.nDst) {
+                    StorePack<S, W>(reinterpret_cast<void*>(to[k]), elemOff, out, h.writeThrough != 0);
+                }
+            }
         }
     }
 }
 
 template <class E, int W, int kBatch>
 __device__ __forceinline__ void ReduceOne(const ProgramView& pv, uint32_t* stack, const ReduceArgs& args,
-                                          const ReduceHot& h, uint64_t e, uint64_t dstOff, uint32_t group,
+                                          const ReduceHot& h, uint64_t e, uint64_t dstOff, uint64_t ownOrFirst,
                                           const FirstBatch<kBatch>* first = nullptr)
 {
     const Pack<typename E::S, W> out = ReduceValue<E, W, kBatch>(pv, stack, args, h, e, first);
-    StoreResult<typename E::S, W>(args, h, out, dstOff + e, group, 0, 1);
+    StoreResult<typename E::S, W, true>(args, h, out, dstOff + e, ownOrFirst, 0, 1);
 }
 
 // Dynamic LDS: the accumulator stack, (plan depth - 1) * accumulator bytes * args.threads.
@@ -780,26 +811,26 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
                 if (wave != 0) {
                     out = __builtin_bit_cast(Pack<S, W>, parked[slot][lane]);
                 }
-                StoreResult<S, W>(args, h, out, dstOff + e, g, wave, h.storeWaves);
+                StoreResult<S, W, false>(args, h, out, dstOff + e, firstDstAddr, wave, h.storeWaves);
             }
             slot ^= 1u;
         }
         if (wave == 0) {
             for (uint64_t i = static_cast<uint64_t>(blk) * 64 + lane; i < nScalar; i += static_cast<uint64_t>(blocksHere) * 64) {
                 const uint64_t e = i < head ? i : i - head + bodyEnd;
-                ReduceOne<E, 1, 8>(pv, accStack, args, h, e, dstOff, g);
+                ReduceOne<E, 1, 8>(pv, accStack, args, h, e, dstOff, firstDstAddr);
             }
         }
         return;
     }
     for (uint64_t u = first; u < nVec + lead; u += stride) {
         if (u >= lead) {
-            ReduceOne<E, W, VB>(pv, accStack, args, h, head + (u - lead) * W, dstOff, g, preloaded);
+            ReduceOne<E, W, VB>(pv, accStack, args, h, head + (u - lead) * W, dstOff, firstDstAddr, preloaded);
         }
     }
     for (uint64_t i = first; i < nScalar; i += stride) {
         const uint64_t e = i < head ? i : i - head + bodyEnd;
-        ReduceOne<E, 1, 8>(pv, accStack, args, h, e, dstOff, g);
+        ReduceOne<E, 1, 8>(pv, accStack, args, h, e, dstOff, firstDstAddr);
     }
 }
 
