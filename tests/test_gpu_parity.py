@@ -609,6 +609,56 @@ def test_prod_and_64_bit_types_fold_in_mesh_order_under_write_reduce_algorithms(
         reduce_scatter_as_mesh(DT.FP16, PROD, 9_001, algo, 6)
 
 
+def test_fp16_prod_carries_the_payload_of_a_single_nan_operand_bit_for_bit():
+    """fp16 PROD is the one half-precision reduction whose arithmetic the reference holds itself (AicpuReduceFp16,
+    alg_data_trans_wrapper.cc:1237-1257): widen, multiply in fp32, narrow with Fp32ToFp16, whose NaN rule keeps
+    the top ten mantissa bits (:1196-1207).  With exactly one NaN among the operands of an element the result is
+    defined on every machine (the multiply returns that NaN, quieted), so it is compared bit for bit: every payload,
+    both signs, quiet and signalling, the NaN at any rank, next to finite values, zeros, subnormals and infinities."""
+    payloads = np.arange(1, 0x400, dtype=np.uint16)
+    nans = np.concatenate([0x7C00 | payloads, 0xFC00 | payloads]).astype(np.uint16)     # 2046 patterns
+    # Two pools, so that the other operands never make a NaN of their own (0 * Inf): one with infinities and nothing
+    # that can underflow to zero, one with zeros and subnormals and nothing that can overflow.
+    with_inf = np.array([0x3C00, 0xBC00, 0x7C00, 0xFC00, 0x3555, 0xC100, 0x4000], dtype=np.uint16)
+    with_zero = np.array([0x3C00, 0xBC00, 0x0000, 0x8000, 0x0001, 0x0400, 0x3555, 0x3800], dtype=np.uint16)
+    for n, algo in ((2, "mesh"), (3, "ring"), (8, "mesh"), (6, "rhd")):
+        w = World(n)
+        try:
+            rng = np.random.default_rng(900 + n)
+            count = 3 * nans.size + 5
+            even = np.arange(count) % 2 == 0
+            ins = [np.where(even, with_inf[rng.integers(0, with_inf.size, count)],
+                            with_zero[rng.integers(0, with_zero.size, count)]) for _ in range(n)]
+            holder = rng.integers(0, n, count)
+            pattern = np.resize(nans, count)
+            for r in range(n):
+                ins[r] = np.where(holder == r, pattern, ins[r]).astype(np.uint16)
+            want = [np.zeros(count, dtype=np.uint16) for _ in range(n)]
+            assert oracle.all_reduce(ins, want, count, int(DT.FP16), PROD, acc=oracle.ACC_FP32,
+                                     algo=order_of(algo, DT.FP16, PROD, False)) == 0
+            # the closed form of the reference's rule: the operand's NaN with its quiet bit set
+            assert np.array_equal(want[0], pattern | 0x0200)
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(2 * count) for _ in range(n)]
+            w.all_reduce(sends, recvs, count, DT.FP16, PROD, algo)
+            for r in range(n):
+                got = to_host(recvs[r], np.uint16)
+                bad = np.nonzero(got != want[r])[0]
+                assert bad.size == 0, "n=%d rank %d: %d differ, first %s got %s want %s" % (
+                    n, r, bad.size, bad[:4], [hex(x) for x in got[bad[:4]]], [hex(x) for x in want[r][bad[:4]]])
+            # ReduceScatter takes the element path for its ragged tail as well
+            c = count // n
+            rs_want = [np.zeros(c, dtype=np.uint16) for _ in range(n)]
+            rs_ins = [x[:n * c] for x in ins]
+            assert oracle.reduce_scatter(rs_ins, rs_want, c, int(DT.FP16), PROD, acc=oracle.ACC_FP32, algo="mesh") == 0
+            rs_recvs = [dev_zeros(2 * c) for _ in range(n)]
+            w.reduce_scatter([to_dev(x) for x in rs_ins], rs_recvs, c, DT.FP16, PROD, "mesh")
+            for r in range(n):
+                assert np.array_equal(to_host(rs_recvs[r], np.uint16), rs_want[r]), "reduce_scatter n=%d rank %d" % (n, r)
+        finally:
+            w.close()
+
+
 def test_warmed_up_collectives_can_be_captured_into_a_graph_and_replayed():
     """After one eager call (which uploads the fold programs) AllReduce, ReduceScatter and AllGather are plain kernel
     launches on the caller's stream: a captured graph of them must reproduce the eager results on every replay,
