@@ -213,6 +213,13 @@ struct DevicePlan {
 constexpr uint32_t kMagic = 0x48434C41u;   // "HCLA"
 constexpr int kStagingSlots = 4;
 
+// One (source, destination, length in bytes) copy; sources and destinations are arbitrary device addresses.
+struct CopySeg {
+    uint64_t src;
+    uint64_t dst;
+    uint64_t len;
+};
+
 struct World;
 struct Comm {
     uint32_t magic = kMagic;
@@ -263,6 +270,7 @@ struct World {
     int copyTwoKernelMode = 2;            // HCCL_AMD_COPY_TWO_KERNELS, likewise for AllGather(V) and Broadcast
     // Allocation-free AlltoAllV: host image of the tables and the device array that receives them.
     std::vector<uint64_t> a2aImage;
+    std::vector<CopySeg> a2aSegs;   // the segment list of the AlltoAllV being launched (one launch at a time per world)
     uint8_t* a2aScratch = nullptr;
     uint32_t reduceBlocks = 1u << 26;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
@@ -580,6 +588,18 @@ HcclResult EnsureA2aBuffers(World* w)
     return HCCL_SUCCESS;
 }
 
+// Every world and stream of a GPU shares that GPU's table array.  Its users are put in order: one at a time on
+// the host (the mutex is held from the wait to the record), and on the device each call's table writes wait for
+// the event recorded behind the copy kernel of the call before it, whichever world or stream that was on.  The
+// event is created with the first allocation-free call on the device; waiting and recording allocate nothing.
+struct ScratchUsers {
+    std::mutex mu;
+    hipEvent_t lastUse = nullptr;
+    bool used = false;
+};
+constexpr int kScratchDevices = 64;
+ScratchUsers g_scratchUsers[kScratchDevices];
+
 // Set-up of the allocation-free entry point, on its first call in a world (the world's device is current):
 // the address of the device-resident table array, and the events a launch over several streams takes from
 // the pool, so that later calls create nothing.
@@ -587,6 +607,16 @@ HcclResult PrepareNoAlloc(World* w)
 {
     if (w->a2aScratch != nullptr) {
         return HCCL_SUCCESS;
+    }
+    if (w->device < 0 || w->device >= kScratchDevices) {
+        return HCCL_E_NOT_SUPPORT;
+    }
+    {
+        ScratchUsers& users = g_scratchUsers[w->device];
+        std::lock_guard<std::mutex> lock(users.mu);
+        if (users.lastUse == nullptr) {
+            HIP_OK(hipEventCreateWithFlags(&users.lastUse, hipEventDisableTiming));
+        }
     }
     uint8_t* ptr = nullptr;
     HIP_OK(A2aScratchOfCurrentDevice(&ptr));
@@ -1269,13 +1299,6 @@ HcclResult RunAllGatherV(World* w, PendingOp& p, hipStream_t s)
     return RunOneToMany(w, b, s);
 }
 
-// One (source, destination, length in bytes) copy; sources and destinations are arbitrary device addresses.
-struct CopySeg {
-    uint64_t src;
-    uint64_t dst;
-    uint64_t len;
-};
-
 // Copies a list of at most n * n non-empty segments with one launch of the descriptor-driven copy kernel.
 // With `noAlloc` the tables travel in kernel arguments to the library's device-resident array instead of
 // through a pinned staging slot into allocated device memory.
@@ -1320,6 +1343,11 @@ HcclResult RunSegmentCopy(World* w, const std::vector<CopySeg>& segs, hipStream_
                 w->launchLock->lock();
             }
             HIP_OK(waited);
+            if (w->destroyed != 0) {
+                // A rank left while the lock was released: its HcclCommDestroy has settled this collective for the
+                // peers (who may free their buffers now), so nothing of it is enqueued.
+                return HCCL_E_UNAVAIL;
+            }
         }
         hDesc = w->a2aHost[slot];
         dev = w->a2aDev + slot * A2aSlotBytes(n);
@@ -1349,19 +1377,33 @@ HcclResult RunSegmentCopy(World* w, const std::vector<CopySeg>& segs, hipStream_
     a.hintShift = BuildTileHints(hEnd, nSeg, static_cast<uint32_t>(tiles), kA2aHintMax, hHint, &nHint);
     a.mode = !congruent ? COPY_GENERAL : ((misfit & 15u) == 0 ? COPY_ALIGNED : COPY_CONGRUENT);
     const size_t used = reinterpret_cast<uint8_t*>(hHint + nHint + 1) - reinterpret_cast<uint8_t*>(hDesc);
-    if (noAlloc) {
-        HIP_OK(LaunchTableWrite(dev, hDesc, static_cast<uint32_t>((used + 7) / 8), s));
-    } else {
-        HIP_OK(hipMemcpyAsync(dev, hDesc, used, hipMemcpyHostToDevice, s));
-    }
     a.desc = reinterpret_cast<const uint64_t*>(dev);
     a.tileEnd = reinterpret_cast<const uint32_t*>(a.desc + static_cast<size_t>(kA2aDescWords) * nSeg);
     a.hint = a.tileEnd + ((nSeg + 1u) & ~1u);
-    HIP_OK(LaunchA2aCopy(a, static_cast<uint32_t>(tiles), tileBytes, s));
-    if (!noAlloc) {
-        HIP_OK(hipEventRecord(w->a2aSlotFree[slot], s));
-        w->a2aSlotUsed[slot] = true;
+    if (noAlloc) {
+        // The array's users on this GPU in order: this call's table writes start when the copy kernel of the call
+        // before it, of whichever world and on whichever stream, has read its tables.  A stream under capture
+        // records launches for later: the replays of a captured call are ordered by whoever launches the graph.
+        ScratchUsers& users = g_scratchUsers[w->device];
+        std::lock_guard<std::mutex> order(users.mu);
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        HIP_OK(hipStreamIsCapturing(s, &capture));
+        const bool eager = capture == hipStreamCaptureStatusNone;
+        if (eager && users.used) {
+            HIP_OK(hipStreamWaitEvent(s, users.lastUse, 0));
+        }
+        HIP_OK(LaunchTableWrite(dev, hDesc, static_cast<uint32_t>((used + 7) / 8), s));
+        HIP_OK(LaunchA2aCopy(a, static_cast<uint32_t>(tiles), tileBytes, s));
+        if (eager) {
+            HIP_OK(hipEventRecord(users.lastUse, s));
+            users.used = true;
+        }
+        return HCCL_SUCCESS;
     }
+    HIP_OK(hipMemcpyAsync(dev, hDesc, used, hipMemcpyHostToDevice, s));
+    HIP_OK(LaunchA2aCopy(a, static_cast<uint32_t>(tiles), tileBytes, s));
+    HIP_OK(hipEventRecord(w->a2aSlotFree[slot], s));
+    w->a2aSlotUsed[slot] = true;
     return HCCL_SUCCESS;
 }
 
@@ -1384,7 +1426,8 @@ HcclResult RunAlltoAllV(World* w, PendingOp& p, hipStream_t s)
     // One descriptor per non-empty segment, destination-major so that neighbouring tiles write
     // neighbouring addresses: recv_i[rdispls_i[j] ...] = send_j[sdispls_j[i] ...]
     // (reference ins_temp_all_to_all_v_mesh_1D.cc:229-246).
-    std::vector<CopySeg> segs;
+    std::vector<CopySeg>& segs = w->a2aSegs;   // keeps its capacity from call to call
+    segs.clear();
     segs.reserve(static_cast<size_t>(n) * n);
     for (uint32_t i = 0; i < n; ++i) {
         const uint64_t* vi = p.ranks[i].var.data();
@@ -1818,7 +1861,10 @@ HcclResult Submit(const CommRef& ref, OpType type, HcclDataType dtype, HcclReduc
     if (p->result == HCCL_SUCCESS && w->destroyed == 0) {
         w->launchBusy = true;
         w->launchLock = &lock;
-        p->result = Launch(w, *p, c->rank);
+        const HcclResult launched = Launch(w, *p, c->rank);
+        if (!p->done) {   // (settled meanwhile by a rank that left while a launch waited without the lock: that verdict stands)
+            p->result = launched;
+        }
         w->launchLock = nullptr;
         w->launchBusy = false;
     } else if (p->result == HCCL_SUCCESS) {

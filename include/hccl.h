@@ -80,10 +80,14 @@ HcclResult HcclAlltoAllV(const void* sendBuf, const void* sendCounts, const void
  * HcclAlltoAllV; every rank of a collective must call the same variant (HCCL_E_PARA otherwise).  The
  * segment tables live in a device array that is part of the library (164,096 bytes per GPU, held until the
  * process ends) and reach it inside kernel arguments, so the call performs no hipMalloc / hipFree /
- * hipHostMalloc and no copy from host memory.  The first call in a world looks up the array's address and
- * creates the events a launch over several streams uses.  HCCL_E_MEMORY if the tables of the call's non-empty
- * segments exceed the array (cannot happen up to HCCL_AMD_MAX_RANKS ranks).  All calls on one GPU share the
- * array: calls that overlap in time on one GPU (different streams without ordering, different worlds) race.
+ * hipHostMalloc and no copy from host memory (its bookkeeping on the host uses the process heap like every
+ * other entry point's).  The first call in a world looks up the array's address and creates the events later
+ * calls use.  HCCL_E_MEMORY if the tables of the call's non-empty segments exceed the array (cannot happen up
+ * to HCCL_AMD_MAX_RANKS ranks).  All calls on one GPU share the array and the library puts them in order: a
+ * call's table writes wait (hipStreamWaitEvent, no allocation) for the copy kernel of the call before it on that
+ * GPU, whichever world or stream that was, so calls from different worlds or streams never see each other's
+ * tables; they do not overlap on the GPU either.  A call recorded into a HIP graph is ordered by whoever
+ * launches the graph: replays that overlap another user of the array on the same GPU race.
  */
 HcclResult HcclAmdAlltoAllVNoAlloc(const void* sendBuf, const void* sendCounts, const void* sdispls,
                                    HcclDataType sendType, const void* recvBuf, const void* recvCounts,

@@ -87,6 +87,45 @@ def test_ranks_on_their_own_streams():
         w.close()
 
 
+def test_two_worlds_on_unordered_streams_take_turns_at_the_array():
+    """Two worlds, each on a stream of its own and nothing between the streams: the second world's call is made while
+    the first world's copy kernel may still be reading its tables from the GPU's one array.  The library orders the
+    array's users itself (the table writes of a call wait for the copy kernel of the call before it), so both get
+    the oracle's bytes, several times over and in both orders."""
+    rng = np.random.default_rng(17)
+    first, second = World(8), World(5)          # a stream each (World creates its own)
+    try:
+        cases = []
+        for w, max_count in ((first, 1_500_000), (second, 4_000)):
+            n = w.n
+            sc, sd, rc, rd, in_sz, out_sz = a2a_case(rng, n, 2, max_count, False)
+            ins = [rand_bytes(rng, in_sz * 2) for _ in range(n)]
+            want = [np.full(out_sz * 2, FILL, dtype=np.uint8) for _ in range(n)]
+            assert oracle.all_to_all_v(ins, want, sc, sd, rc, rd, int(DT.BFP16)) == 0
+            cases.append((w, sc, sd, rc, rd, [to_dev(x) for x in ins], want, out_sz))
+        for order in ((0, 1), (1, 0), (0, 1)):
+            outs = {}
+            for k in (0, 1):
+                w, _, _, _, _, _, _, out_sz = cases[k]
+                outs[k] = [dev_zeros(out_sz * 2, fill=FILL) for _ in range(w.n)]
+            first.inputs_ready()
+            for k in order:                     # back to back, no synchronisation in between
+                w, sc, sd, rc, rd, sends, _, _ = cases[k]
+                with hccl_amd.group():
+                    for r in range(w.n):
+                        hccl_amd.all_to_all_v_no_alloc(w.comms[r], sends[r], sc[r], sd[r], DT.BFP16, outs[k][r], rc[r],
+                                                       rd[r], DT.BFP16, w.stream)
+            first.sync()
+            second.sync()
+            for k in (0, 1):
+                w, want = cases[k][0], cases[k][6]
+                for r in range(w.n):
+                    assert np.array_equal(to_host(outs[k][r], np.uint8), want[r]), (order, k, r)
+    finally:
+        first.close()
+        second.close()
+
+
 def test_mixing_the_two_entry_points_in_one_collective_is_rejected():
     n = 2
     w = World(n)
