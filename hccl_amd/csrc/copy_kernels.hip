@@ -141,11 +141,8 @@ __device__ __forceinline__ void PaceStores(uint32_t pace)
     }
 }
 
-// `ahead`, where not null, holds the addresses of the first kBatch destinations, fetched by the caller before the
-// tile's load was waited for: the first batch of stores then follows the load without a round of scalar loads.
 template <int kBatch, bool kStatic, class PtrFn, class StoreFn>
-__device__ __forceinline__ void ForEachDst(uint32_t nDst, uint64_t dOff, uint32_t pace, PtrFn ptrOf, StoreFn store,
-                                           const uint64_t* ahead)
+__device__ __forceinline__ void ForEachDst(uint32_t nDst, uint64_t dOff, uint32_t pace, PtrFn ptrOf, StoreFn store)
 {
     static_assert(kBatch == 1 || kBatch == 4 || kBatch == 8, "the fences below name every pointer of a batch");
     for (uint32_t base = 0; base < nDst; base += kBatch) {
@@ -154,8 +151,6 @@ __device__ __forceinline__ void ForEachDst(uint32_t nDst, uint64_t dOff, uint32_
         for (uint32_t k = 0; k < static_cast<uint32_t>(kBatch); ++k) {
             if constexpr (kStatic) {
                 ptr[k] = ptrOf(k);
-            } else if (ahead != nullptr && base == 0) {
-                ptr[k] = ahead[k];
             } else {
                 ptr[k] = ptrOf(base + k < nDst ? base + k : nDst - 1);
             }
@@ -191,7 +186,7 @@ __device__ __forceinline__ void Ready(uint32_t& v) { asm volatile("" : "+v"(v));
 // by all T threads of the workgroup.
 template <int T, int MODE, int kBatch, bool kStatic, class PtrFn>
 __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uint32_t nDst, uint64_t dOff, uint32_t pace,
-                                         PtrFn ptrOf, const uint64_t* ahead = nullptr)
+                                         PtrFn ptrOf)
 {
     const uint32_t idx = threadIdx.x;
     if (MODE == COPY_ALIGNED) {
@@ -200,11 +195,11 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
             Ready(v);
             ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
                 StoreVec<U32x4>(v, reinterpret_cast<U32x4*>(dst) + idx);
-            }, ahead);
+            });
         }
         return;
     }
-    const uint32_t dMis = static_cast<uint32_t>(((ahead != nullptr ? ahead[0] : ptrOf(0)) + dOff) & 15u);
+    const uint32_t dMis = static_cast<uint32_t>((ptrOf(0) + dOff) & 15u);
     uint32_t head = (16u - dMis) & 15u;     // bytes before the first aligned destination vector
     head = head < bytes ? head : bytes;
     const uint32_t nVec = (bytes - head) / 16u;   // <= T
@@ -251,12 +246,12 @@ __device__ __forceinline__ void CopyTile(const uint8_t* src, uint32_t bytes, uin
     if (idx < nVec) {
         ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
             StoreVec<U32x4>(out, reinterpret_cast<U32x4*>(dst + head) + idx);
-        }, ahead);
+        });
     }
     if (idx < edge) {
         ForEachDst<kBatch, kStatic>(nDst, dOff, pace, ptrOf, [&](uint8_t* dst) {
             StoreVec<uint8_t>(static_cast<uint8_t>(edgeByte), dst + edgeAt);
-        }, ahead);
+        });
     }
 }
 
@@ -279,21 +274,10 @@ __global__ __launch_bounds__(T) void BcastCopyKernel(const BcastCopyArgs args)
     for (uint32_t k = 0; k < 16; ++k) {
         ends[k] = args.tileEnd[k];
     }
-    // (The first eight destination addresses among them: entries past nDst exist in the table and are never used.
-    // Fetched where the stores need them, they were a round of scalar loads between the tile's arrival and its
-    // first store.)
-    static_assert(kMaxRanks >= 8, "dst[0 .. 7] are read whatever nDst is");
-    uint64_t firstDst[8];
-#pragma unroll
-    for (uint32_t k = 0; k < 8; ++k) {
-        firstDst[k] = reinterpret_cast<uint64_t>(args.dst[k]);
-    }
     asm volatile("" : "+s"(nDst), "+s"(nSegPadded));
     asm volatile("" : "+s"(ends[0]), "+s"(ends[1]), "+s"(ends[2]), "+s"(ends[3]), "+s"(ends[4]), "+s"(ends[5]),
                       "+s"(ends[6]), "+s"(ends[7]), "+s"(ends[8]), "+s"(ends[9]), "+s"(ends[10]), "+s"(ends[11]),
                       "+s"(ends[12]), "+s"(ends[13]), "+s"(ends[14]), "+s"(ends[15]));
-    asm volatile("" : "+s"(firstDst[0]), "+s"(firstDst[1]), "+s"(firstDst[2]), "+s"(firstDst[3]), "+s"(firstDst[4]),
-                      "+s"(firstDst[5]), "+s"(firstDst[6]), "+s"(firstDst[7]));
     const uint32_t tile = blockIdx.x;
     // Number of segments that end at or before this tile = index of the tile's segment (prefixes past the last
     // segment hold 0xFFFFFFFF; empty segments repeat their predecessor's prefix and are skipped by the count).
@@ -320,7 +304,7 @@ __global__ __launch_bounds__(T) void BcastCopyKernel(const BcastCopyArgs args)
     const uint8_t* src = reinterpret_cast<const uint8_t*>(srcBase + off);
     const uint64_t dOff = segDstOff + off;
     CopyTile<T, MODE, 8, false>(src, bytes, nDst, dOff, args.pace,
-                                [&](uint32_t d) { return reinterpret_cast<uint64_t>(args.dst[d]); }, firstDst);
+                                [&](uint32_t d) { return reinterpret_cast<uint64_t>(args.dst[d]); });
 }
 
 // ---- AlltoAllV -------------------------------------------------------------------------------------
