@@ -684,8 +684,8 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     // and where folding a tile takes long (8- and 16-bit types with their wide accumulators): measured, fp32 SUM
     // in rank order, 6 ranks 0.72 -> 0.75 / 0.74 -> 0.79 / 0.73 -> 0.78 of the HBM peak at 64 / 128 / 512 MiB per
     // rank with two wavefronts (32 MiB: 0.69 -> 0.67), 8 ranks 0.65 -> 0.72 / 0.70 -> 0.77 / 0.72 -> 0.78 at 32 / 64 /
-    // 128 MiB with three (16 MiB: 0.62 -> 0.61); four ranks lose at every size.  HCCL_AMD_REDUCE_STORE_WAVES forces
-    // a count (1 = one wavefront per tile).
+    // 128 MiB with three (16 MiB: 0.62 -> 0.61).  HCCL_AMD_REDUCE_STORE_WAVES forces a count (1 = one wavefront per
+    // tile).
     a.storeWaves = 1;
     if (!oneStream && a.threads == 64 && a.vecOk) {
         const uint64_t bytes = a.total * esz;
@@ -693,7 +693,10 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
         uint32_t waves = 1;
         if (a.nDst >= 8) {
             waves = longFold ? (bytes >= (64ull << 20) ? 2u : 1u) : (bytes >= (24ull << 20) ? 3u : 1u);
-        } else if (a.nDst >= 6) {
+        } else if (a.nDst >= 4) {
+            // (four and five destinations too, since the launch's scalars come in one round: fp32 over 4 ranks
+            // 0.72 -> 0.74 / 0.75 -> 0.79 / 0.76 -> 0.79 at 64 / 256 / 512 MiB per rank, bf16 alike; two and three
+            // ranks still lose)
             waves = bytes >= (48ull << 20) ? 2u : 1u;
         }
         if (w->storeWaves != 0) {
