@@ -148,6 +148,11 @@ def _bind(L):
     L.HcclAmdSetAlgo.argtypes = [vp, i32, i32]
     L.HcclAmdGetAlgo.argtypes = [vp, i32, ctypes.POINTER(i32)]
     L.HcclAmdGetFoldProgram.argtypes = [i32, i32, u32, u32, vp, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
+    L.HcclAmdGetFoldProgramTwoLevel.argtypes = [i32, i32, u32, u32, u32, vp, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
+    L.HcclAmdSetLevel0RankSize.argtypes = [vp, u32]
+    L.HcclAmdGetLevel0RankSize.argtypes = [vp, ctypes.POINTER(u32)]
+    L.HcclAmdSelectFromHcclAlgo.argtypes = [ctypes.c_char_p, i32, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(i32),
+                                            ctypes.POINTER(ctypes.c_int32), ctypes.c_char_p, u32]
     L.HcclAmdGetStuckCounters.argtypes = [vp, ctypes.POINTER(u64), ctypes.POINTER(u64)]
     L.HcclAmdSetCclBufferSize.argtypes = [vp, u64]
     L.HcclAmdGetCclBufferSize.argtypes = [vp, ctypes.POINTER(u64)]
@@ -303,20 +308,42 @@ def get_stuck_counters(hccl_comm):
     return head.value, tail.value
 
 
-def fold_programs(op_kind, algo, rank_size):
-    """Host-only: the byte programs (one per segment) that fix the reduction order."""
+def fold_programs(op_kind, algo, rank_size, level0=1):
+    """Host-only: the byte programs (one per segment) that fix the reduction order; level0 > 1: the two-level
+    AllReduce over groups of level0 consecutive ranks with `algo` between the groups."""
     L = lib()
     out = []
     seg, count = 0, 1
     while seg < count:
         buf = (ctypes.c_uint8 * 512)()
         ln, cnt = ctypes.c_uint32(), ctypes.c_uint32()
-        check(L.HcclAmdGetFoldProgram(int(op_kind), int(algo), rank_size, seg, buf, 512, ctypes.byref(ln),
-                                      ctypes.byref(cnt)), "HcclAmdGetFoldProgram")
+        check(L.HcclAmdGetFoldProgramTwoLevel(int(op_kind), int(algo), rank_size, level0, seg, buf, 512,
+                                              ctypes.byref(ln), ctypes.byref(cnt)), "HcclAmdGetFoldProgramTwoLevel")
         count = cnt.value
         out.append(bytes(buf[:ln.value]))
         seg += 1
     return out
+
+
+def set_level0_rank_size(hccl_comm, ranks_per_group):
+    """Groups of consecutive ranks (servers) for the two-level AllReduce of the world hccl_comm belongs to."""
+    return check(lib().HcclAmdSetLevel0RankSize(hccl_comm, ctypes.c_uint32(ranks_per_group)), "HcclAmdSetLevel0RankSize")
+
+
+def get_level0_rank_size(hccl_comm):
+    v = ctypes.c_uint32()
+    check(lib().HcclAmdGetLevel0RankSize(hccl_comm, ctypes.byref(v)), "HcclAmdGetLevel0RankSize")
+    return v.value
+
+
+def select_from_hccl_algo(config, op_kind):
+    """How the library reads an HCCL_ALGO value for op_kind: (canonical text, Algo or None, two_level).  Raises
+    HcclError(HCCL_E_PARA) for a string the reference's parser rejects."""
+    sel, algo, two = ctypes.c_int32(), ctypes.c_int(), ctypes.c_int32()
+    text = ctypes.create_string_buffer(4096)
+    check(lib().HcclAmdSelectFromHcclAlgo(config.encode(), int(op_kind), ctypes.byref(sel), ctypes.byref(algo),
+                                          ctypes.byref(two), text, 4096), "HcclAmdSelectFromHcclAlgo")
+    return text.value.decode(), (Algo(algo.value) if sel.value else None), bool(two.value)
 
 
 # ---- collectives (names and argument order of hccl4py.ops) ----------------------------------------

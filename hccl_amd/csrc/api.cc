@@ -23,6 +23,7 @@
 #include <vector>
 
 #include "dataplane.h"
+#include "algo_config.h"
 #include "fold_plan.h"
 #include "hccl.h"
 
@@ -288,6 +289,11 @@ struct World {
     // Size of the staging buffer whose loops the slice-dependent AllReduce orders (NHR, RHD) reproduce; 0 = one
     // loop.  HCCL_BUFFSIZE when set, or HcclAmdSetCclBufferSize.
     uint64_t cclBytes = 0;
+    // Ranks per level-0 group of the two-level AllReduce (HcclAmdSetLevel0RankSize, HCCL_AMD_LEVEL0_RANKS); 1 = one level.
+    uint32_t level0 = 1;
+    // HCCL_ALGO asked for a sequence executor (1), a single-level one (0), or said nothing (-1): with level-0
+    // groups, AllReduce runs in two levels unless a single-level executor was asked for.
+    int allReduceSequence = -1;
     bool envInvalid = false;      // an environment variable of the reference failed its parser
 
     ~World()
@@ -411,6 +417,32 @@ void ApplyAlgoEnv(World* w)
     }
 }
 
+// HCCL_ALGO in the reference's own syntax (algo_config.h).  A string its parser rejects is ignored with a warning,
+// as there (alg_parse.cc:803-826); clauses that select nothing for the three fold-order operators are ignored too.
+void ApplyReferenceAlgoEnv(World* w)
+{
+    const char* env = getenv("HCCL_ALGO");
+    if (!env) {
+        return;
+    }
+    std::vector<AlgoSegment> segments;
+    if (ParseHcclAlgo(env, &segments) != HCCL_SUCCESS) {
+        Log(1, "HCCL_ALGO [%s] parse failed, the config has not taken effect, standard format: "
+               "'opType:executorType{level0=algoType, level1=algoType};...'", env);
+        return;
+    }
+    const AlgoSelection sel = SelectFromHcclAlgo(segments);
+    for (int op = 0; op < HCCL_AMD_OP_COUNT; ++op) {
+        const HcclAmdOpKind kind = static_cast<HcclAmdOpKind>(op);
+        if (sel.set[op] && AlgoFitsOp(kind, sel.algo[op])) {
+            w->algo[op] = sel.algo[op];
+            if (kind == HCCL_AMD_OP_ALL_REDUCE) {
+                w->allReduceSequence = sel.twoLevel[op] ? 1 : 0;
+            }
+        }
+    }
+}
+
 std::unique_ptr<World> NewWorld(uint32_t n)
 {
     auto w = std::make_unique<World>();
@@ -456,7 +488,16 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->reduceBatch != 8 && w->reduceBatch != 16) {
         w->reduceBatch = 0;
     }
+    ApplyReferenceAlgoEnv(w.get());
     ApplyAlgoEnv(w.get());
+    {
+        const uint32_t groups = EnvU32("HCCL_AMD_LEVEL0_RANKS", 1);
+        if (groups >= 1 && groups <= n && n % groups == 0) {
+            w->level0 = groups;
+        } else {
+            Log(1, "HCCL_AMD_LEVEL0_RANKS=%u does not divide the %u ranks of the world: ignored", groups, n);
+        }
+    }
     if (const char* det = getenv("HCCL_DETERMINISTIC")) {
         std::string v(det);
         for (char& ch : v) ch = static_cast<char>(toupper(static_cast<unsigned char>(ch)));
@@ -503,16 +544,16 @@ HcclResult CheckUserRank(const Comm* c)
 // ---------------------------------------------------------------------------------------------
 // Device resources
 // ---------------------------------------------------------------------------------------------
-HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DevicePlan* out)
+HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DevicePlan* out, uint32_t level0 = 1)
 {
-    uint32_t key = static_cast<uint32_t>(kind) * 64 + static_cast<uint32_t>(algo);
+    uint32_t key = (static_cast<uint32_t>(kind) * 64 + static_cast<uint32_t>(algo)) * 128 + level0;
     auto it = w->plans.find(key);
     if (it != w->plans.end()) {
         *out = it->second;
         return HCCL_SUCCESS;
     }
     FoldPlan plan;
-    HcclResult rc = BuildFoldPlan(kind, algo, w->n, &plan);
+    HcclResult rc = BuildFoldPlan(kind, algo, w->n, &plan, level0);
     if (rc != HCCL_SUCCESS) {
         return rc;
     }
@@ -929,8 +970,19 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
     HcclAmdAlgo algo = EffectiveAlgo(w, HCCL_AMD_OP_ALL_REDUCE, p.dtype, p.op);
+    // A world with level-0 groups runs the step-driven orders in two levels: a mesh ReduceScatter inside every
+    // group, the configured template between the groups (reference
+    // ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852).  The types the reference reduces on the host take its
+    // host-reduce template between the groups, which folds the own share first (EffectiveAlgo has turned their
+    // RHD / NHR into MESH; a configured sequence{mesh, nhr_aicpu_reduce} asks for the same).
+    const uint32_t level0 = w->level0;
+    const HcclAmdAlgo configured = w->algo[HCCL_AMD_OP_ALL_REDUCE];
+    const bool stepDriven = configured == HCCL_AMD_ALGO_RHD || configured == HCCL_AMD_ALGO_NHR;
+    const bool twoLevel = level0 > 1 && level0 < n && w->allReduceSequence != 0 &&
+                          (algo == HCCL_AMD_ALGO_RHD || algo == HCCL_AMD_ALGO_NHR ||
+                           (algo == HCCL_AMD_ALGO_MESH && (stepDriven || w->allReduceSequence == 1)));
     DevicePlan plan;
-    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_ALL_REDUCE, algo, &plan);
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_ALL_REDUCE, algo, &plan, twoLevel ? level0 : 1);
     if (rc != HCCL_SUCCESS) {
         return rc;
     }
@@ -1043,7 +1095,69 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
         a.subLen = unit;
         return LaunchToAll(w, a, plan, p.dtype, p.op, s);
     };
+    if (twoLevel && algo != HCCL_AMD_ALGO_RHD) {
+        // Between the groups NHR, or the host-reduce fold: every loop is cut into level0 chunks of floor(len / level0)
+        // elements, the last chunk taking the rest, and every chunk into n / level0 sub-slices the same way (reference
+        // ins_v2_all_reduce_sequence_executor_aicpu.cc:413-415, 445-455).  The loops hold what fits half the staging
+        // buffer, floored to 128 bytes and to a multiple of n elements (:653-656).
+        const uint32_t level1 = n / level0;
+        uint64_t maxPerLoop = p.count;
+        if (w->cclBytes != 0) {
+            maxPerLoop = w->cclBytes / 2 / 128 * 128 / esz / n * n;
+            if (maxPerLoop == 0) {
+                Log(1, "AllReduce: the staging buffer of %llu bytes holds no loop of the two-level order",
+                    static_cast<unsigned long long>(w->cclBytes));
+                return HCCL_E_INTERNAL;
+            }
+        }
+        for (uint64_t done = 0; done < p.count;) {
+            const uint64_t len = std::min(p.count - done, maxPerLoop);
+            const uint64_t chunk = len / level0;
+            if (chunk * level0 == len && chunk % level1 == 0 && chunk != 0) {
+                // every sub-slice equally long: one launch over the n units of the loop, unit i * level1 + j being
+                // sub-slice j of chunk i
+                a.nSub = n;
+                a.prog = plan.dev;
+                rc = launchLoop(done, len, chunk / level1);
+                if (rc != HCCL_SUCCESS) {
+                    return rc;
+                }
+                done += len;
+                continue;
+            }
+            a.nSub = level1;
+            for (uint32_t i = 0; i < level0; ++i) {
+                const uint64_t begin = done + static_cast<uint64_t>(i) * chunk;
+                const uint64_t cur = i == level0 - 1 ? len - static_cast<uint64_t>(i) * chunk : chunk;
+                if (cur == 0) {
+                    continue;
+                }
+                for (uint32_t r = 0; r < n; ++r) {
+                    a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + begin * esz;
+                    a.dst[r] = static_cast<uint8_t*>(p.ranks[r].recv) + begin * esz;
+                }
+                a.prog = plan.dev + static_cast<uint64_t>(i) * level1 * kDevProgBytes;
+                a.total = a.groupLen = cur;
+                a.subLen = cur / level1;
+                if (a.subLen == 0) {
+                    // fewer elements than sub-slices: all of them belong to the last sub-slice
+                    a.prog = plan.dev + (static_cast<uint64_t>(i) * level1 + level1 - 1) * kDevProgBytes;
+                    a.nSub = 1;
+                    a.subLen = cur;
+                }
+                rc = LaunchToAll(w, a, plan, p.dtype, p.op, s);
+                a.nSub = level1;
+                if (rc != HCCL_SUCCESS) {
+                    return rc;
+                }
+            }
+            done += len;
+        }
+        return HCCL_SUCCESS;
+    }
     if (algo == HCCL_AMD_ALGO_RHD) {
+        // (With level-0 groups the frame is the same: unit u = i * (n / level0) + j is sub-slice j of chunk i, and
+        // the remainder shorter than n is padded to one element per unit; only the programs differ.)
         // Whole frames of n uniform units while they last, then a remainder shorter than n with one element per
         // unit (reference ins_v2_all_reduce_sequence_rhd_tail.h:94-113); a bounded staging buffer limits the
         // frames one loop holds.
@@ -3031,25 +3145,104 @@ HcclResult HcclAmdGetStuckCounters(HcclComm comm, uint64_t* head, uint64_t* tail
     return HCCL_SUCCESS;
 }
 
+HcclResult HcclAmdSetLevel0RankSize(HcclComm comm, uint32_t ranksPerGroup)
+{
+    CHK_PTR(comm, "comm");
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
+    if (c == nullptr || ranksPerGroup == 0 || ranksPerGroup > c->world->n || c->world->n % ranksPerGroup != 0) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> wl(c->world->mu);
+    c->world->level0 = ranksPerGroup;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdGetLevel0RankSize(HcclComm comm, uint32_t* ranksPerGroup)
+{
+    CHK_PTR(comm, "comm");
+    CHK_PTR(ranksPerGroup, "ranksPerGroup");
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> wl(c->world->mu);
+    *ranksPerGroup = c->world->level0;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdSelectFromHcclAlgo(const char* config, HcclAmdOpKind op, int32_t* selected, HcclAmdAlgo* algo,
+                                     int32_t* twoLevel, char* canonical, uint32_t cap)
+{
+    CHK_PTR(config, "config");
+    if (static_cast<int>(op) < 0 || op >= HCCL_AMD_OP_COUNT) {
+        return HCCL_E_PARA;
+    }
+    std::vector<AlgoSegment> segments;
+    HcclResult rc = ParseHcclAlgo(config, &segments);
+    if (rc != HCCL_SUCCESS) {
+        return rc;
+    }
+    const AlgoSelection sel = SelectFromHcclAlgo(segments);
+    if (selected != nullptr) {
+        *selected = sel.set[op] ? 1 : 0;
+    }
+    if (algo != nullptr) {
+        *algo = sel.algo[op];
+    }
+    if (twoLevel != nullptr) {
+        *twoLevel = sel.twoLevel[op] ? 1 : 0;
+    }
+    if (canonical != nullptr && cap != 0) {
+        std::string text;
+        for (const AlgoSegment& seg : segments) {
+            if (!text.empty()) {
+                text += ";";
+            }
+            std::string unit = seg.executor + "{";
+            for (size_t i = 0; i < seg.templates.size(); ++i) {
+                unit += (i ? "," : "") + (seg.templates[i].enable ? seg.templates[i].name : "not(" + seg.templates[i].name + ")");
+            }
+            unit += "}";
+            text += (seg.opType.empty() ? "" : seg.opType + ":") + (seg.enable ? unit : "not(" + unit + ")");
+        }
+        if (text.size() + 1 > cap) {
+            return HCCL_E_MEMORY;
+        }
+        memcpy(canonical, text.c_str(), text.size() + 1);
+    }
+    return HCCL_SUCCESS;
+}
+
 HcclResult HcclAmdGetFoldProgram(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t segment,
                                  uint8_t* out, uint32_t cap, uint32_t* len, uint32_t* segmentCount)
+{
+    return HcclAmdGetFoldProgramTwoLevel(op, algo, rankSize, 1, segment, out, cap, len, segmentCount);
+}
+
+HcclResult HcclAmdGetFoldProgramTwoLevel(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t level0,
+                                         uint32_t segment, uint8_t* out, uint32_t cap, uint32_t* len,
+                                         uint32_t* segmentCount)
 {
     CHK_PTR(len, "len");
     // Callers walk all segments of one plan: keep the last plan built.
     static std::mutex cacheMu;
     static FoldPlan plan;
     static int cachedOp = -1, cachedAlgo = -1;
-    static uint32_t cachedSize = 0;
+    static uint32_t cachedSize = 0, cachedLevel0 = 0;
     std::lock_guard<std::mutex> cacheLock(cacheMu);
-    if (cachedOp != static_cast<int>(op) || cachedAlgo != static_cast<int>(algo) || cachedSize != rankSize) {
+    if (cachedOp != static_cast<int>(op) || cachedAlgo != static_cast<int>(algo) || cachedSize != rankSize ||
+        cachedLevel0 != level0) {
         cachedOp = -1;
-        HcclResult rc = BuildFoldPlan(op, algo, rankSize, &plan);
+        HcclResult rc = BuildFoldPlan(op, algo, rankSize, &plan, level0);
         if (rc != HCCL_SUCCESS) {
             return rc;
         }
         cachedOp = static_cast<int>(op);
         cachedAlgo = static_cast<int>(algo);
         cachedSize = rankSize;
+        cachedLevel0 = level0;
     }
     if (segmentCount != nullptr) {
         *segmentCount = static_cast<uint32_t>(plan.programs.size());

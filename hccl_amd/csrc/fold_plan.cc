@@ -5,6 +5,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <functional>
 #include <memory>
 
 #include "dataplane.h"
@@ -101,6 +102,22 @@ ExprPtr Chain(const std::vector<uint32_t>& order)
         e = Fold(e, Leaf(order[i]));
     }
     return e;
+}
+
+// What stands for participant k of a step-driven template before its first step: rank k's input in a one-level
+// world, the value a level-0 group has folded for that participant in a two-level one.
+using LeafFn = std::function<ExprPtr(uint32_t)>;
+ExprPtr RankLeaf(uint32_t k) { return Leaf(k); }
+
+HcclResult EmitAll(const std::vector<ExprPtr>& values, FoldPlan* plan)
+{
+    for (const ExprPtr& e : values) {
+        HcclResult rc = Emit(e, plan);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    return HCCL_SUCCESS;
 }
 
 uint32_t CeilLog2(uint32_t n)
@@ -242,12 +259,12 @@ HcclResult OrderPreserved(uint32_t n, FoldPlan* plan)
 // Step s: rank m write-reduces slices {m - 2^s - i * 2^(s+1)} into the same slices of rank m - 2^s,
 // i < (N - 1 + 2^s) / 2^(s+1); the receiver's value is the accumulator (reference
 // ins_temp_reduce_scatter_nhr.cc:316-447, 458-506).  Slice k ends at rank k.
-HcclResult Nhr(uint32_t n, FoldPlan* plan)
+std::vector<ExprPtr> NhrValues(uint32_t n, const LeafFn& leaf)
 {
     std::vector<std::vector<ExprPtr>> held(n, std::vector<ExprPtr>(n));
     for (uint32_t m = 0; m < n; ++m) {
         for (uint32_t k = 0; k < n; ++k) {
-            held[m][k] = Leaf(m);
+            held[m][k] = leaf(m);
         }
     }
     uint32_t steps = CeilLog2(n);
@@ -265,14 +282,14 @@ HcclResult Nhr(uint32_t n, FoldPlan* plan)
             }
         }
     }
+    std::vector<ExprPtr> out(n);
     for (uint32_t k = 0; k < n; ++k) {
-        HcclResult rc = Emit(held[k][k], plan);
-        if (rc != HCCL_SUCCESS) {
-            return rc;
-        }
+        out[k] = held[k][k];
     }
-    return HCCL_SUCCESS;
+    return out;
 }
+
+HcclResult Nhr(uint32_t n, FoldPlan* plan) { return EmitAll(NhrValues(n, RankLeaf), plan); }
 
 // ---- RHD ---------------------------------------------------------------------------------------
 uint32_t VirtualSlotStart(uint32_t r, uint32_t a) { return a < r ? 2 * a : a + r; }
@@ -284,14 +301,14 @@ uint32_t VirtualSlotEnd(uint32_t r, uint32_t b) { return b <= r ? 2 * b : b + r;
 //       half into the partner v ^ dist (the partner's value is the accumulator).
 // Share i ends at the carrier of the virtual rank owning slot sigma(i)
 // (reference template_utils.cc:117-208, ins_temp_reduce_scatter_rhd.cc:365-564).
-HcclResult Rhd(uint32_t p, FoldPlan* plan)
+std::vector<ExprPtr> RhdValues(uint32_t p, const LeafFn& leaf)
 {
     uint32_t r = RhdPairCount(p);
     uint32_t bigP = p - r;
     std::vector<std::vector<ExprPtr>> held(p, std::vector<ExprPtr>(p));
     for (uint32_t j = 0; j < p; ++j) {
         for (uint32_t u = 0; u < p; ++u) {
-            held[j][u] = Leaf(j);
+            held[j][u] = leaf(j);
         }
     }
     for (uint32_t t = 0; t < r; ++t) {
@@ -313,10 +330,60 @@ HcclResult Rhd(uint32_t p, FoldPlan* plan)
             }
         }
     }
+    std::vector<ExprPtr> out(p);
     for (uint32_t i = 0; i < p; ++i) {
         uint32_t slot = RhdSlotOfRank(p, i);
         uint32_t v = slot < 2 * r ? slot / 2 : slot - r;
-        HcclResult rc = Emit(held[RhdCarrierOfVirtual(p, v)][slot], plan);
+        out[i] = held[RhdCarrierOfVirtual(p, v)][slot];
+    }
+    return out;
+}
+
+HcclResult Rhd(uint32_t p, FoldPlan* plan) { return EmitAll(RhdValues(p, RankLeaf), plan); }
+
+// ---- two levels --------------------------------------------------------------------------------
+// AllReduce over level-0 groups of l0 consecutive ranks ("boxes") and a level-1 template between the boxes
+// (reference ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852: step 1 mesh ReduceScatter inside the box,
+// step 2 level-1 ReduceScatter between the ranks that hold the same chunk, steps 3 and 4 the two AllGathers).
+// A loop's elements are l0 chunks of l1 sub-slices; sub-slice j of chunk i is program i * l1 + j: the level-1
+// template's value for its unit j, in which participant b stands for what box b folded for chunk i, the chunk
+// owner's input first and the other ranks of the box ascending (reference
+// ins_temp_reduce_scatter_mesh_1D.cc:203-237; the level-0 template ..._Z_axis_detour derives from it).
+// Level 1: RHD with POST skipped and the merged share bridged (:700-741), NHR (:784-789), or for the types the
+// host reduces the own-first fold of ins_temp_reduce_scatter_aicpu_reduce_nhr.cc:214-250 (`MESH`).
+HcclResult TwoLevelAllReduce(uint32_t n, uint32_t l0, HcclAmdAlgo level1, FoldPlan* plan)
+{
+    const uint32_t l1 = n / l0;
+    plan->segmentsAreSubs = true;
+    for (uint32_t i = 0; i < l0; ++i) {
+        const LeafFn box = [&](uint32_t b) {
+            std::vector<uint32_t> order{b * l0 + i};
+            for (uint32_t t = 0; t < l0; ++t) {
+                if (t != i) {
+                    order.push_back(b * l0 + t);
+                }
+            }
+            return Chain(order);
+        };
+        std::vector<ExprPtr> units;
+        if (level1 == HCCL_AMD_ALGO_RHD) {
+            units = RhdValues(l1, box);
+        } else if (level1 == HCCL_AMD_ALGO_NHR) {
+            units = NhrValues(l1, box);
+        } else if (level1 == HCCL_AMD_ALGO_MESH) {
+            for (uint32_t j = 0; j < l1; ++j) {
+                ExprPtr e = box(j);
+                for (uint32_t b = 0; b < l1; ++b) {
+                    if (b != j) {
+                        e = Fold(e, box(b));
+                    }
+                }
+                units.push_back(e);
+            }
+        } else {
+            return HCCL_E_NOT_SUPPORT;
+        }
+        HcclResult rc = EmitAll(units, plan);
         if (rc != HCCL_SUCCESS) {
             return rc;
         }
@@ -356,11 +423,20 @@ uint32_t RhdCarrierOfVirtual(uint32_t p, uint32_t v)
     return v < r ? v : v + r;
 }
 
-HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPlan* plan)
+HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPlan* plan, uint32_t level0)
 {
     *plan = FoldPlan{};
     if (n == 0 || n > static_cast<uint32_t>(kMaxRanks)) {
         return HCCL_E_PARA;
+    }
+    if (level0 > 1 && level0 < n) {
+        if (n % level0 != 0) {
+            return HCCL_E_PARA;
+        }
+        if (op != HCCL_AMD_OP_ALL_REDUCE) {
+            return HCCL_E_NOT_SUPPORT;
+        }
+        return TwoLevelAllReduce(n, level0, algo, plan);
     }
     if (op == HCCL_AMD_OP_REDUCE) {
         // One-shot: rank 0's slot is the base, the others fold ascending (reference reduce_mesh_1D.cc:268-300).

@@ -304,6 +304,42 @@ HcclResult HcclAmdGetStuckCounters(HcclComm comm, uint64_t* head, uint64_t* tail
  */
 HcclResult HcclAmdGetFoldProgram(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t segment,
                                  uint8_t* out, uint32_t cap, uint32_t* len, uint32_t* segmentCount);
+/* The same for the two-level AllReduce over groups of `level0` consecutive ranks (see HcclAmdSetLevel0RankSize):
+ * segment i * (rankSize / level0) + j is sub-slice j of chunk i; algo is the template between the groups (RHD, NHR,
+ * or MESH for the own-first fold of the host-reduce template).  level0 of 1 or rankSize: HcclAmdGetFoldProgram. */
+HcclResult HcclAmdGetFoldProgramTwoLevel(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t level0,
+                                         uint32_t segment, uint8_t* out, uint32_t cap, uint32_t* len,
+                                         uint32_t* segmentCount);
+
+/*
+ * Level-0 groups.  The reference runs AllReduce over a two-level topology (servers of several ranks) as a
+ * sequence: a mesh ReduceScatter inside every server, the configured template (RHD, NHR, or the host-reduce fold for
+ * PROD and the 64-bit types) between the ranks that hold the same chunk, and the two AllGathers back
+ * (src/ops/all_reduce/algorithm/executor/ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852, registered as
+ * Aicpu AllReduce Sequence MeshConcur RHD / MeshConcur NHR / Mesh NHRAicpuReduce, :974-1023).  Where its topology
+ * comes from a rank table, a loopback world is told: `ranksPerGroup` consecutive ranks form a group (it must
+ * divide the rank size; 1, the default, and the rank size itself mean one level).  Also HCCL_AMD_LEVEL0_RANKS at
+ * world creation.  With groups, AllReduce under RHD and NHR folds in the two-level order; the other orders and the
+ * other operators are not affected.
+ */
+HcclResult HcclAmdSetLevel0RankSize(HcclComm comm, uint32_t ranksPerGroup);
+HcclResult HcclAmdGetLevel0RankSize(HcclComm comm, uint32_t* ranksPerGroup);
+
+/*
+ * The reference's HCCL_ALGO setting ("allreduce:sequence{level0=mesh_concur,level1=rhd};reducescatter:nhr;..."; grammar
+ * and vocabulary of src/common/alg_parse.cc:27-437) is read at world creation and selects the fold order of
+ * AllReduce, ReduceScatter(V) and Reduce: sole{mesh | mesh_one_shot | mesh_two_shot} -> MESH (Reduce: mesh_two_shot ->
+ * MESH_TWO_SHOT), sole{mesh_chunk...} -> MESH_CHUNK, sole{nhr...} -> NHR, sole{nhr_aicpu_reduce} -> the host-reduce
+ * order (RING for AllReduce, MESH for ReduceScatter), sole{rhd | hd | hd_aicpu_reduce} -> RHD, strictordered{...} ->
+ * ORDER_PRESERVED, sequence{<mesh...>, <template>} -> that template between level-0 groups (AllReduce).  Clauses are
+ * taken last to first, negations select nothing, clauses for the copy operators are accepted and ignored, and a
+ * string the reference's parser rejects is ignored with a warning, as there.  HCCL_AMD_ALGO and HcclAmdSetAlgo
+ * override it.  This call is the host-only view of that reading: HCCL_E_PARA for a rejected string; otherwise
+ * *selected says whether `config` selects an order for `op`, *algo and *twoLevel which, and `canonical` (optional,
+ * `cap` bytes) receives the parsed clauses in normal form ("allreduce:sequence{meshconcur,rhd};not(sole{nhr})").
+ */
+HcclResult HcclAmdSelectFromHcclAlgo(const char* config, HcclAmdOpKind op, int32_t* selected, HcclAmdAlgo* algo,
+                                     int32_t* twoLevel, char* canonical, uint32_t cap);
 
 #ifdef __cplusplus
 }

@@ -1300,6 +1300,218 @@ int orc_all_reduce_rhd(uint32_t p, const void* const* in, void* const* out, uint
     return rc;
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * Two-level AllReduce (ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852, "executor.cc" below).
+ * l0 consecutive ranks form a level-0 group ("box"), l1 = n / l0 boxes; rank b * l0 + i is member i of box b
+ * and talks, between the boxes, to the members i of the other boxes.  Per loop:
+ *   step 1  mesh ReduceScatter inside every box: member i ends with chunk i of the loop, its own input
+ *           first, the other members ascending (reduce_scatter_mesh_1D.cc:203-237; the level-0 template
+ *           ..._Z_axis_detour derives from it)
+ *   step 2  the level-1 template between the members i of all boxes, on chunk i cut into l1 sub-slices
+ *   steps 3, 4  the two AllGathers back: every rank ends with every sub-slice.
+ * Level 1 (registrations executor.cc:974-1023):
+ *   ORC_L1_RHD   RHD with POST skipped, the merged share bridged, AllGather with PRE skipped (:684-759); the
+ *                loop is cut like the flat form with the rank alignment l0 * l1: aligned prefix in uniform
+ *                units, a remainder shorter than that staged into a padded tile (rhd_tail.h:94-165)
+ *   ORC_L1_NHR   NHR ReduceScatter (:784-789); chunks of floor(len / l0), the last member's chunk takes the rest
+ *                (:413-415); sub-slices of floor(chunk / l1), the last box's takes the rest (:445-455)
+ *   ORC_L1_MESH  the host-reduce template of PROD and the 64-bit types, own share first, the other boxes
+ *                ascending (reduce_scatter_aicpu_reduce_nhr.cc:214-250), same cuts as NHR.
+ * Everything is folded in the accumulation domain and narrowed once per output (see red_t).
+ * ------------------------------------------------------------------------------------------- */
+static void level0_fold(const red_t* r, uint32_t l0, uint32_t box, uint32_t member, const uint8_t* const* src,
+                        uint64_t elemOff, uint64_t len, void* acc, void* tmp)
+{
+    red_widen(r, src[box * l0 + member] + elemOff * r->esz, acc, len);
+    for (uint32_t t = 0; t < l0; ++t) {
+        if (t != member) {
+            red_pair_from_storage(r, acc, src[box * l0 + t] + elemOff * r->esz, len, tmp);
+        }
+    }
+}
+
+/* Level 1 over chunk `member` of one loop, cut into l1 units of `unit` elements (the last holds `last`);
+ * writes unit j of every box's view to result[box] + (chunkOff + j * unit). */
+static int level1_exchange(const red_t* r, uint32_t l0, uint32_t l1, int l1Algo, uint32_t member,
+                           const uint8_t* const* src, uint64_t chunkOff, uint64_t unit, uint64_t last,
+                           uint8_t* const* result, uint64_t resultOff)
+{
+    uint64_t slot = last > unit ? last : unit;
+    if (slot == 0) {
+        return ORC_OK;
+    }
+    scratch_t sc, grid;
+    void* tmp = malloc(slot * r->asz);
+    if (!tmp || scratch_alloc(&sc, l1, slot, r->asz) != ORC_OK) {
+        free(tmp);
+        return ORC_E_INTERNAL;
+    }
+    memset(sc.mem, 0, (uint64_t)l1 * l1 * slot * r->asz);
+    int rc = ORC_OK;
+    for (uint32_t b = 0; b < l1; ++b) {
+        for (uint32_t j = 0; j < l1; ++j) {
+            uint64_t cur = j == l1 - 1 ? last : unit;
+            uint32_t at = l1Algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l1, j) : j;
+            level0_fold(r, l0, b, member, src, chunkOff + (uint64_t)j * unit, cur, scratch_at(&sc, b, at), tmp);
+        }
+    }
+    if (l1Algo == ORC_L1_RHD) {
+        rc = rhd_rs_frame(r, &sc, 1);
+        if (rc == ORC_OK && scratch_alloc(&grid, l1, slot, r->asz) != ORC_OK) {
+            rc = ORC_E_INTERNAL;
+        }
+        if (rc == ORC_OK) {
+            size_t slotBytes = slot * r->asz;
+            memset(grid.mem, 0, (uint64_t)l1 * l1 * slotBytes);
+            for (uint32_t b = 0; b < l1; ++b) {
+                orc_rhd_part1_t info;
+                orc_rhd_part1(l1, b, ORC_INVALID_RANK, &info);
+                if (info.inPart1 && !info.isRepresentative) {
+                    continue;
+                }
+                memcpy(scratch_at(&grid, b, b), scratch_at(&sc, b, orc_rhd_unit_start_of_rank(l1, b)), slotBytes);
+                if (info.inPart1 && info.isRepresentative) {
+                    memcpy(scratch_at(&grid, b, info.pairedAlgRank), scratch_at(&sc, b, info.unitStart + 1), slotBytes);
+                }
+            }
+            rc = rhd_ag_frame(&grid);
+            for (uint32_t b = 0; b < l1 && rc == ORC_OK; ++b) {
+                for (uint32_t j = 0; j < l1; ++j) {
+                    red_narrow(r, scratch_at(&grid, b, j), result[b] + (resultOff + (uint64_t)j * unit) * r->esz, unit);
+                }
+            }
+            free(grid.mem);
+        }
+    } else {
+        if (l1Algo == ORC_L1_NHR) {
+            rc = nhr_reduce_scatter_scratch(r, &sc);
+        } else {
+            /* own share first: box j folds the other boxes' shares of unit j ascending into its own */
+            for (uint32_t j = 0; j < l1; ++j) {
+                uint64_t cur = j == l1 - 1 ? last : unit;
+                for (uint32_t b = 0; b < l1; ++b) {
+                    if (b != j) {
+                        red_pair(r, scratch_at(&sc, j, j), scratch_at(&sc, b, j), cur);
+                    }
+                }
+            }
+        }
+        for (uint32_t j = 0; j < l1 && rc == ORC_OK; ++j) {
+            uint64_t cur = j == l1 - 1 ? last : unit;
+            for (uint32_t b = 0; b < l1; ++b) {   /* AllGather: every box receives box j's unit j */
+                red_narrow(r, scratch_at(&sc, j, j), result[b] + (resultOff + (uint64_t)j * unit) * r->esz, cur);
+            }
+        }
+    }
+    free(sc.mem);
+    free(tmp);
+    return rc;
+}
+
+int orc_all_reduce_two_level(uint32_t n, uint32_t l0, int l1Algo, const void* const* in, void* const* out,
+                             uint64_t count, int dtype, int op, int accMode, uint64_t maxCountPerLoop)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (l0 == 0 || n % l0 != 0 || l1Algo < ORC_L1_RHD || l1Algo > ORC_L1_MESH) {
+        return ORC_E_PARA;
+    }
+    uint32_t l1 = n / l0;
+    if (maxCountPerLoop == 0) {
+        maxCountPerLoop = UINT64_MAX / 2;
+    }
+    maxCountPerLoop = maxCountPerLoop / n * n;   /* executor.cc:653-656 */
+    if (maxCountPerLoop == 0) {
+        return ORC_E_INTERNAL;
+    }
+    /* per-box result (the members of a box end with the same bytes), and the padded tiles of the RHD tail */
+    uint8_t** result = (uint8_t**)calloc(l1, sizeof(uint8_t*));
+    uint8_t* tiles = (uint8_t*)malloc((size_t)n * n * r.esz);
+    uint8_t* tileOut = (uint8_t*)malloc((size_t)l1 * n * r.esz);
+    const uint8_t** src = (const uint8_t**)malloc(sizeof(uint8_t*) * n);
+    uint8_t** dst = (uint8_t**)malloc(sizeof(uint8_t*) * l1);
+    if (!result || !tiles || !tileOut || !src || !dst) {
+        rc = ORC_E_INTERNAL;
+    }
+    for (uint32_t b = 0; b < l1 && rc == ORC_OK; ++b) {
+        result[b] = (uint8_t*)malloc((count ? count : 1) * r.esz);
+        if (!result[b]) {
+            rc = ORC_E_INTERNAL;
+        }
+    }
+    uint64_t processed = 0;
+    while (processed < count && rc == ORC_OK) {
+        uint64_t remaining = count - processed;
+        uint64_t valid, curr;
+        int padded = 0;
+        if (l1Algo == ORC_L1_RHD) {
+            valid = orc_rhd_select_loop_count(remaining, maxCountPerLoop, n);
+            curr = valid > n ? valid : n;
+            padded = valid != curr;
+        } else {
+            valid = curr = remaining < maxCountPerLoop ? remaining : maxCountPerLoop;
+        }
+        uint64_t srcOff = processed;
+        uint64_t dstOff = processed;
+        for (uint32_t j = 0; j < n; ++j) {
+            src[j] = cbytes(in[j]);
+        }
+        for (uint32_t b = 0; b < l1; ++b) {
+            dst[b] = result[b];
+        }
+        if (padded) {
+            /* rhd_tail.h:115-146: every rank stages its valid elements and doubles them up to the tile */
+            for (uint32_t j = 0; j < n; ++j) {
+                uint8_t* t = tiles + (size_t)j * n * r.esz;
+                memcpy(t, cbytes(in[j]) + processed * r.esz, valid * r.esz);
+                uint64_t filled = valid;
+                while (filled < n) {
+                    uint64_t c = filled < n - filled ? filled : n - filled;
+                    memcpy(t + filled * r.esz, t, c * r.esz);
+                    filled += c;
+                }
+                src[j] = t;
+            }
+            for (uint32_t b = 0; b < l1; ++b) {
+                dst[b] = tileOut + (size_t)b * n * r.esz;
+            }
+            srcOff = 0;
+            dstOff = 0;
+        }
+        uint64_t chunk = curr / l0;
+        for (uint32_t i = 0; i < l0 && rc == ORC_OK; ++i) {
+            uint64_t cur = (i == l0 - 1 && l1Algo != ORC_L1_RHD) ? curr - (uint64_t)i * chunk : chunk;
+            uint64_t unit = cur / l1;
+            uint64_t last = l1Algo == ORC_L1_RHD ? unit : cur - unit * (l1 - 1);
+            rc = level1_exchange(&r, l0, l1, l1Algo, i, src, srcOff + (uint64_t)i * chunk, unit, last, dst,
+                                 dstOff + (uint64_t)i * chunk);
+        }
+        if (padded && rc == ORC_OK) {
+            for (uint32_t b = 0; b < l1; ++b) {
+                memcpy(result[b] + processed * r.esz, tileOut + (size_t)b * n * r.esz, valid * r.esz);
+            }
+        }
+        processed += valid;
+    }
+    if (rc == ORC_OK) {
+        for (uint32_t j = 0; j < n; ++j) {
+            memcpy(out[j], result[j / l0], count * r.esz);
+        }
+    }
+    for (uint32_t b = 0; result && b < l1; ++b) {
+        free(result[b]);
+    }
+    free(result);
+    free(tiles);
+    free(tileOut);
+    free(src);
+    free(dst);
+    return rc;
+}
+
 /* a12: while blocks > 1: M = largest power of two < blocks; for src = M..blocks-1:
  * slot[src % M] = slot[src] (+) slot[src % M]; blocks = M.  Block v is rank v's contribution. */
 static uint32_t largest_pow2_less_than(uint32_t v)

@@ -155,6 +155,16 @@ int orc_all_reduce_mesh_chunk(uint32_t n, const void* const* in, void* const* ou
  * last slice takes the rest; every element follows the NHR reduce-scatter tree of its slice, then gather. */
 int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
                        int accMode);
+/* Two-level AllReduce of the reference's sequence executor
+ * (ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852): l0 consecutive ranks form a level-0 group; inside
+ * it a mesh ReduceScatter (own input first), between the groups l1Algo on every chunk, then the AllGathers.
+ * maxCountPerLoop 0 = one loop.  l0 == 1 with ORC_L1_RHD is orc_all_reduce_rhd. */
+#define ORC_L1_RHD 0
+#define ORC_L1_NHR 1
+#define ORC_L1_MESH 2
+int orc_all_reduce_two_level(uint32_t n, uint32_t l0, int l1Algo, const void* const* in, void* const* out,
+                             uint64_t count, int dtype, int op, int accMode, uint64_t maxCountPerLoop);
+
 /* The same inside the executor's loop over the staging buffer (ins_v2_all_reduce_sole_executor.cc:266-300):
  * every loop of maxCountPerLoop elements (the last one shorter) is sliced afresh; 0 = one loop. */
 int orc_all_reduce_nhr_looped(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,

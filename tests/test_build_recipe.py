@@ -11,7 +11,8 @@ CSRC = os.path.join(ROOT, "hccl_amd", "csrc")
 def test_a_failed_compile_fails_the_build_and_leaves_no_object(tmp_path):
     work = tmp_path / "csrc"
     work.mkdir()
-    for name in ("Makefile", "dataplane.h", "fold_plan.h", "fold_plan.cc", "reduce_kernel_impl.h"):
+    headers = [f for f in os.listdir(CSRC) if f.endswith(".h")]   # the rules name the headers as prerequisites
+    for name in ["Makefile", "fold_plan.cc"] + headers:
         shutil.copy(os.path.join(CSRC, name), work / name)
     env = dict(os.environ)
     # the recipe includes ../../include relative to the source directory: point it at the real headers

@@ -26,6 +26,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests", "emu"))
 import build_emu  # noqa: E402
 
 FILES = ["tests/test_gpu_parity.py", "tests/test_gpu_copies.py", "tests/test_wide_gpu_copy_sweep.py",
+         "tests/test_wide_gpu_two_level.py",
          "tests/test_wide_gpu_rooted_sweep.py", "tests/test_gpu_rooted_and_v_ops.py",
          "tests/test_gpu_random_sweep.py", "tests/test_gpu_point_to_point.py",
          "tests/test_gpu_reference_python_suites.py", "tests/test_wide_gpu_reference_st_shapes.py",

@@ -1,0 +1,291 @@
+"""CPU tier: the two-level AllReduce order (level-0 groups, reference
+ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852) and the reading of the reference's HCCL_ALGO setting.
+
+The oracle's two-level function is pinned by what does not depend on it: with one rank per group it must be the
+(already pinned) one-level RHD / NHR oracle, with one group the own-first mesh order, integer sums must equal plain
+modular sums, and on small worlds it must equal expression trees written out by hand from the reference's step
+rules.  The library's fold programs are then evaluated with numpy against it.  The parser is checked against the
+cases of the reference's own unit test (test/ut/common/alg_parse/alg_parse_test.cc), transcribed as data."""
+import numpy as np
+import pytest
+
+import hccl_amd
+from hccl_amd import Algo, OpKind
+
+from test_host_plan import f32_fold, program_ranks, run_program, same, tricky, wide
+
+F32, I32, F16 = 4, 2, 3
+SUM, PROD, MAX, MIN = range(4)
+L1 = {"rhd": Algo.RHD, "nhr": Algo.NHR, "mesh": Algo.MESH}
+SHAPES = [(2, 3), (2, 4), (4, 2), (3, 2), (2, 6), (3, 5), (8, 8), (2, 2), (5, 3)]
+
+
+# ---- the oracle against what is known without it ----------------------------------------------------
+@pytest.mark.parametrize("p", [2, 3, 5, 6, 7, 8, 12])
+def test_one_rank_per_group_is_the_one_level_order(orc, p):
+    rng = np.random.default_rng(31 * p)
+    for count in (p * 7, p * 7 + 3, 1, p - 1 if p > 1 else 1):
+        for op, gen in ((SUM, wide), (MAX, tricky)):
+            ins = gen(rng, p, count)
+            for algo in ("rhd", "nhr"):
+                want = [np.zeros(count, np.float32) for _ in range(p)]
+                got = [np.zeros(count, np.float32) for _ in range(p)]
+                assert orc.all_reduce(ins, want, count, F32, op, algo=algo) == 0
+                assert orc.all_reduce_two_level(ins, got, count, F32, op, 1, algo) == 0
+                for r in range(p):
+                    assert same(got[r], want[r]), (p, count, op, algo, r)
+
+
+@pytest.mark.parametrize("n", [2, 3, 4, 8])
+def test_one_group_is_the_own_first_mesh_order(orc, n):
+    """All ranks in one group: chunk i is folded by member i, its own input first, the others ascending; with a count
+    that is a multiple of n that is the symmetric two-shot order, slice by slice."""
+    rng = np.random.default_rng(17 * n)
+    count = n * 9
+    for op, gen in ((SUM, wide), (MIN, tricky)):
+        ins = gen(rng, n, count)
+        want = [np.zeros(count, np.float32) for _ in range(n)]
+        assert orc.all_reduce(ins, want, count, F32, op, algo="mesh_symmetric") == 0
+        for level1 in ("nhr", "mesh", "rhd"):
+            got = [np.zeros(count, np.float32) for _ in range(n)]
+            assert orc.all_reduce_two_level(ins, got, count, F32, op, n, level1) == 0
+            for r in range(n):
+                assert same(got[r], want[r]), (n, op, level1, r)
+
+
+@pytest.mark.parametrize("l0,l1", SHAPES)
+def test_every_rank_counts_exactly_once(orc, l0, l1):
+    """int32 SUM of distinct powers of two per rank (n <= 30) or plain modular sums: order does not matter, every
+    contribution must be there once, whatever the count leaves over."""
+    n = l0 * l1
+    rng = np.random.default_rng(5 * n + l0)
+    for count in (n * 4, n * 4 + 1, n * 4 + n - 1, 3, 1):
+        ins = [rng.integers(-2 ** 31, 2 ** 31, count, dtype=np.int64).astype(np.int32) for _ in range(n)]
+        want = np.zeros(count, dtype=np.int64)
+        for x in ins:
+            want += x
+        want = want.astype(np.int32)   # wraps
+        for level1 in ("rhd", "nhr", "mesh"):
+            got = [np.zeros(count, np.int32) for _ in range(n)]
+            assert orc.all_reduce_two_level(ins, got, count, I32, SUM, l0, level1) == 0
+            for r in range(n):
+                assert np.array_equal(got[r], want), (l0, l1, count, level1, r)
+
+
+def box(ins, l0, b, i, lo, hi, op):
+    """What group b folds for chunk member i over elements [lo, hi): own input first, the others ascending."""
+    acc = ins[b * l0 + i][lo:hi]
+    for t in range(l0):
+        if t != i:
+            acc = f32_fold(ins[b * l0 + t][lo:hi], acc, op)
+    return acc
+
+
+def test_two_groups_of_three_and_three_groups_of_two_by_hand(orc):
+    """Written out from the reference's step rules.
+    RHD over 3 groups (template_utils.cc:117-208): r = 1, pair (0, 1), group 0 represents; PRE: group 1 is folded into
+    group 0 on every unit; MAIN, one step: virtual rank 0 (group 0) keeps units 0 and 1 and receives group 2's, virtual
+    rank 1 (group 2) keeps unit 2 and receives the pair's.  So units 0, 1 = B2 (+) (B1 (+) B0) with the pair as
+    accumulator, unit 2 = (B1 (+) B0) (+) B2 with group 2 as accumulator.
+    NHR over 2 groups (reduce_scatter_nhr.cc:458-506): one step, unit j stays at group j, the other group's share
+    comes in: unit 0 = B1 (+) B0, unit 1 = B0 (+) B1 (accumulator written last)."""
+    rng = np.random.default_rng(99)
+    for op, gen in ((SUM, wide), (MAX, tricky), (MIN, tricky)):
+        # 3 groups of 2 ranks, RHD between them; 36 elements: chunks of 18, units of 6
+        l0, l1, count = 2, 3, 36
+        ins = gen(rng, 6, count)
+        got = [np.zeros(count, np.float32) for _ in range(6)]
+        assert orc.all_reduce_two_level(ins, got, count, F32, op, l0, "rhd") == 0
+        want = np.zeros(count, np.float32)
+        for i in range(l0):
+            for j in range(l1):
+                lo = i * 18 + j * 6
+                b = [box(ins, l0, g, i, lo, lo + 6, op) for g in range(l1)]
+                pair = f32_fold(b[1], b[0], op)
+                want[lo:lo + 6] = f32_fold(b[2], pair, op) if j < 2 else f32_fold(pair, b[2], op)
+        for r in range(6):
+            assert same(got[r], want), ("rhd", op, r)
+        # 2 groups of 3 ranks, NHR between them; 31 elements: chunks 10, 10, 11; units 5 + 5 and 5 + 6
+        l0, l1, count = 3, 2, 31
+        ins = gen(rng, 6, count)
+        got = [np.zeros(count, np.float32) for _ in range(6)]
+        assert orc.all_reduce_two_level(ins, got, count, F32, op, l0, "nhr") == 0
+        want = np.zeros(count, np.float32)
+        for i, (lo, ln) in enumerate(((0, 10), (10, 10), (20, 11))):
+            for j, (ulo, uhi) in enumerate(((lo, lo + 5), (lo + 5, lo + ln))):
+                b = [box(ins, l0, g, i, ulo, uhi, op) for g in range(l1)]
+                want[ulo:uhi] = f32_fold(b[1 - j], b[j], op)
+        for r in range(6):
+            assert same(got[r], want), ("nhr", op, r)
+        # the host-reduce fold between 3 groups of 2: unit j starts from group j, the others ascending
+        l0, l1, count = 2, 3, 13
+        ins = gen(rng, 6, count)
+        got = [np.zeros(count, np.float32) for _ in range(6)]
+        assert orc.all_reduce_two_level(ins, got, count, F32, op, l0, "mesh") == 0
+        want = np.zeros(count, np.float32)
+        for i, (lo, ln) in enumerate(((0, 6), (6, 7))):
+            unit = ln // 3
+            for j in range(3):
+                ulo, uhi = lo + j * unit, (lo + ln if j == 2 else lo + (j + 1) * unit)
+                acc = box(ins, l0, j, i, ulo, uhi, op)
+                for g in range(3):
+                    if g != j:
+                        acc = f32_fold(box(ins, l0, g, i, ulo, uhi, op), acc, op)
+                want[ulo:uhi] = acc
+        for r in range(6):
+            assert same(got[r], want), ("mesh", op, r)
+
+
+def test_loops_cut_the_count_like_the_executor(orc):
+    """A bounded staging buffer: loops of maxCountPerLoop floored to a multiple of n, each sliced afresh; equal to
+    running the collective loop by loop."""
+    rng = np.random.default_rng(7)
+    l0, l1 = 2, 3
+    n, count, per_loop = 6, 100, 40          # 36 + 36 + 28
+    ins = wide(rng, n, count)
+    for level1 in ("rhd", "nhr"):
+        got = [np.zeros(count, np.float32) for _ in range(n)]
+        assert orc.all_reduce_two_level(ins, got, count, F32, SUM, l0, level1, max_count_per_loop=per_loop) == 0
+        want = np.zeros(count, np.float32)
+        pieces = ((0, 36), (36, 72), (72, 100)) if level1 == "nhr" else ((0, 36), (36, 72), (72, 96), (96, 100))
+        for lo, hi in pieces:
+            part = [x[lo:hi].copy() for x in ins]
+            out = [np.zeros(hi - lo, np.float32) for _ in range(n)]
+            assert orc.all_reduce_two_level(part, out, hi - lo, F32, SUM, l0, level1) == 0
+            want[lo:hi] = out[0]
+        assert same(got[3], want), level1
+
+
+# ---- the library's programs against the oracle ---------------------------------------------------------
+@pytest.mark.parametrize("l0,l1", SHAPES)
+@pytest.mark.parametrize("level1", ["rhd", "nhr", "mesh"])
+def test_two_level_programs_match_oracle(orc, l0, l1, level1):
+    n = l0 * l1
+    progs = hccl_amd.fold_programs(OpKind.ALL_REDUCE, L1[level1], n, level0=l0)
+    assert len(progs) == n
+    for prog in progs:
+        assert sorted(program_ranks(prog)) == list(range(n)) and len(prog) <= 320
+    for count in (n * 3, n * 3 + 5, 2):
+        for op, gen in ((SUM, wide), (MAX, tricky)):
+            rng = np.random.default_rng(1000 * n + 10 * l0 + op)
+            ins = gen(rng, n, count)
+            outs = [np.zeros(count, np.float32) for _ in range(n)]
+            assert orc.all_reduce_two_level(ins, outs, count, F32, op, l0, level1) == 0
+            got = np.zeros(count, np.float32)
+            if level1 == "rhd":
+                unit = count // n
+                for u in range(n):
+                    lo, hi = u * unit, (u + 1) * unit
+                    if hi > lo:
+                        got[lo:hi] = run_program(progs[u], lambda r: ins[r][lo:hi], op)
+                for e in range(unit * n, count):
+                    got[e:e + 1] = run_program(progs[e - unit * n], lambda r: ins[r][e:e + 1], op)
+            else:
+                chunk = count // l0
+                for i in range(l0):
+                    clo = i * chunk
+                    chi = count if i == l0 - 1 else clo + chunk
+                    unit = (chi - clo) // l1
+                    for j in range(l1):
+                        lo, hi = clo + j * unit, (chi if j == l1 - 1 else clo + (j + 1) * unit)
+                        if hi > lo:
+                            got[lo:hi] = run_program(progs[i * l1 + j], lambda r: ins[r][lo:hi], op)
+            assert same(got, outs[0]), (l0, l1, level1, count, op)
+
+
+def test_groups_must_divide_the_world():
+    with pytest.raises(hccl_amd.HcclError) as e:
+        hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.RHD, 6, level0=4)
+    assert e.value.code == 1
+    with pytest.raises(hccl_amd.HcclError) as e:
+        hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.RHD, 6, level0=2)
+    assert e.value.code == 5
+    # one rank per group, or all ranks in one: the one-level programs
+    assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.RHD, 6, level0=1) == hccl_amd.fold_programs(
+        OpKind.ALL_REDUCE, Algo.RHD, 6)
+    assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.NHR, 6, level0=6) == hccl_amd.fold_programs(
+        OpKind.ALL_REDUCE, Algo.NHR, 6)
+
+
+# ---- HCCL_ALGO ---------------------------------------------------------------------------------------
+# (config, normal form) from test/ut/common/alg_parse/alg_parse_test.cc:29-213, 266-330
+ACCEPTED = [
+    ("allreduce:sequence{mesh2die,nhrmultilink};sole{nhr};allgather:sequence{mesh,nhr,nhr};concur{mesh,nhrmultilink}; "
+     "not(meshoneshot)",
+     "allreduce:sequence{mesh2die,nhrmultilink};sole{nhr};allgather:sequence{mesh,nhr,nhr};concur{mesh,nhrmultilink};"
+     "not(sole{meshoneshot})"),
+    ("not(parallel{mesh,nhr});allgather:sequence{mesh,nhr};allreduce:not(sequence{mesh_multi_link,nhr})",
+     "not(parallel{mesh,nhr});allgather:sequence{mesh,nhr};allreduce:not(sequence{meshmultilink,nhr})"),
+    ("allgather:not(sequence{level0=mesh2die,level1=nhrmultilink}); concur{not(mesh),meshchunktwoshot};mesh_chunk",
+     "allgather:not(sequence{mesh2die,nhrmultilink});concur{not(mesh),meshchunktwoshot};sole{meshchunk}"),
+    ("mesh_concur;sequence{meshtwoshot,not(nhrmultilink)};allgather:sequence{mesh,nhr}",
+     "sole{meshconcur};sequence{meshtwoshot,not(nhrmultilink)};allgather:sequence{mesh,nhr}"),
+    ("mesh2die; sequence{meshchunk  ,not( nhrmultilink)};allgather:sequence{mesh, nhr}",
+     "sole{mesh2die};sequence{meshchunk,not(nhrmultilink)};allgather:sequence{mesh,nhr}"),
+    ("alltoall:sole{mesh}", "alltoall:sole{mesh}"),
+    ("reducescatter:sequence{level0=meshchunkconcur,level1=nhr}", "reducescatter:sequence{meshchunkconcur,nhr}"),
+    ("", ""),
+    ("nhrmultilink;meshoneshot;mesh2die", "sole{nhrmultilink};sole{meshoneshot};sole{mesh2die}"),
+    ("allreduce:sequence{mesh2die,not(nhrmultilink),not(meshchunktwoshot)}",
+     "allreduce:sequence{mesh2die,not(nhrmultilink),not(meshchunktwoshot)}"),
+    ("reducescatter:sole{level0=hdaicpureduce}", "reducescatter:sole{hdaicpureduce}"),
+    ("reducescatter:parallel{level0=mesh,level1=hd}", "reducescatter:parallel{mesh,hd}"),
+    ("hd;reducescatter:not(parallel{level0=mesh,level1=hd});sole{level0=not(hdaicpureduce)}",
+     "sole{hd};reducescatter:not(parallel{mesh,hd});sole{not(hdaicpureduce)}"),
+    # explicit levels out of order land in level order (alg_parse.cc:156-190)
+    ("allreduce:sequence{level1=rhd,level0=mesh_concur}", "allreduce:sequence{meshconcur,rhd}"),
+]
+REJECTED = [
+    "invalid_op:sole{meshchunk}",
+    "not(parallel{mesh2die,nhrmultilink};allgather:sequence{mesh,nhr}",
+    "allgather:not(sequence{level0=mesh2die,level1=nhrmultilink}); concur{not(mesh2die),nhr;meshchunk}",
+    "allreduce:sole{invalid_algo}",
+    "allreduce:invalid_exec{meshchunktwoshot}",
+    "alltoall:sole{meshwrite}",
+    "allreduce:sole{nhr",
+    "allreduce:sole{nhr}}",
+    "level0:NA;level1:H-D_R",      # the older syntax of the other device generation is not this parser's
+]
+
+
+@pytest.mark.parametrize("config,normal", ACCEPTED)
+def test_hccl_algo_strings_the_reference_accepts(config, normal):
+    text, _, _ = hccl_amd.select_from_hccl_algo(config, OpKind.ALL_REDUCE)
+    assert text == normal
+
+
+@pytest.mark.parametrize("config", REJECTED)
+def test_hccl_algo_strings_the_reference_rejects(config):
+    with pytest.raises(hccl_amd.HcclError) as e:
+        hccl_amd.select_from_hccl_algo(config, OpKind.ALL_REDUCE)
+    assert e.value.code == 1
+
+
+def test_what_hccl_algo_selects():
+    sel = hccl_amd.select_from_hccl_algo
+    AR, RS, RD = OpKind.ALL_REDUCE, OpKind.REDUCE_SCATTER, OpKind.REDUCE
+    assert sel("allreduce:sequence{level0=mesh_concur,level1=rhd}", AR)[1:] == (Algo.RHD, True)
+    assert sel("allreduce:sequence{mesh_concur,nhr}", AR)[1:] == (Algo.NHR, True)
+    assert sel("allreduce:sequence{mesh,nhr_aicpu_reduce}", AR)[1:] == (Algo.MESH, True)
+    assert sel("allreduce:sequence{mesh_concur,rhd}", RS)[1] is None          # names another operator
+    assert sel("allreduce:sole{mesh_one_shot}", AR)[1:] == (Algo.MESH, False)
+    assert sel("allreduce:mesh_two_shot", AR)[1:] == (Algo.MESH, False)
+    assert sel("allreduce:sole{mesh_chunk_two_shot}", AR)[1] == Algo.MESH_CHUNK
+    assert sel("allreduce:nhr_aicpu_reduce", AR)[1] == Algo.RING
+    assert sel("reducescatter:nhr_aicpu_reduce", RS)[1] == Algo.MESH
+    assert sel("reducescatter:sole{hd_aicpu_reduce}", RS)[1] == Algo.RHD
+    assert sel("reducescatterv:sole{mesh_chunk}", RS)[1] == Algo.MESH_CHUNK
+    assert sel("reduce:mesh_two_shot", RD)[1] == Algo.MESH_TWO_SHOT
+    assert sel("reduce:sole{nhr}", RD)[1] is None                              # no such Reduce order here
+    assert sel("strictordered{mesh}", AR)[1] == Algo.ORDER_PRESERVED
+    assert sel("strictordered{mesh}", RD)[1] is None
+    # a clause without an operator applies to all of them; later clauses are read first
+    assert sel("nhr", AR)[1] == Algo.NHR and sel("nhr", RS)[1] == Algo.NHR and sel("nhr", RD)[1] is None
+    assert sel("allreduce:sole{nhr};sole{mesh}", AR)[1] == Algo.MESH
+    assert sel("sole{mesh};allreduce:sole{nhr}", AR)[1] == Algo.NHR
+    assert sel("sole{mesh};allreduce:sole{nhr}", RS)[1] == Algo.MESH
+    # negations exclude in the reference and select nothing here; copies have no order
+    assert sel("allreduce:not(sole{nhr})", AR)[1] is None
+    assert sel("allreduce:sole{not(nhr)}", AR)[1] is None
+    assert sel("allgather:sole{mesh};alltoall:pairwise", AR)[1] is None
+    assert sel("allreduce:sequence{mesh,nhr,nhr}", AR)[1] is None              # three levels are not built
