@@ -369,6 +369,9 @@ hipError_t LaunchA2aT(const A2aArgs& a, uint32_t tiles, hipStream_t stream)
 // lanes shifted by `lead`, so that every wavefront covers whole 128-byte lines.
 constexpr uint32_t kFanOutWaves = 16;
 static_assert(kFanOutWaves <= static_cast<uint32_t>(kMaxRanks), "a wavefront reads dst[wave] before it knows nDst");
+// kStreamLoad: the source is loaded non-temporally (the caller says when, see launch_policy.h); a kernel of its own, since the
+// compiler merges the two flavours of the load into a plain one when they sit in the branches of one kernel.
+template <bool kStreamLoad>
 __global__ __launch_bounds__(64 * kFanOutWaves) void FanOutKernel(const FanOutArgs args)
 {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.y);
@@ -390,7 +393,12 @@ __global__ __launch_bounds__(64 * kFanOutWaves) void FanOutKernel(const FanOutAr
     const uint64_t u = static_cast<uint64_t>(blockIdx.x) * 64u + threadIdx.x;
     if (u >= lead && u < nVec + lead) {
         const uint64_t at = head + ((u - lead) << 4);
-        const U32x4 v = *((const __attribute__((address_space(1))) U32x4*)(srcAddr + at));
+        U32x4 v;
+        if constexpr (kStreamLoad) {
+            v = __builtin_nontemporal_load((const __attribute__((address_space(1))) U32x4*)(srcAddr + at));
+        } else {
+            v = *((const __attribute__((address_space(1))) U32x4*)(srcAddr + at));
+        }
         __builtin_nontemporal_store(v, (__attribute__((address_space(1))) U32x4*)(dstAddr + at));
     }
     const uint64_t bodyEnd = head + (nVec << 4);
@@ -548,7 +556,7 @@ bool FanOutTakes(const FanOutArgs& args)
     return true;
 }
 
-hipError_t LaunchFanOut(const FanOutArgs& in, hipStream_t stream)
+hipError_t LaunchFanOut(const FanOutArgs& in, bool streamLoad, hipStream_t stream)
 {
     if (!FanOutTakes(in)) {
         return hipErrorInvalidValue;
@@ -570,7 +578,11 @@ hipError_t LaunchFanOut(const FanOutArgs& in, hipStream_t stream)
         for (uint32_t d = 0; d < a.nDst; ++d) {
             a.dst[d] = in.dst[first + d];
         }
-        hipLaunchKernelGGL(FanOutKernel, dim3(tiles), dim3(64, a.nDst), 0, stream, a);
+        if (streamLoad) {
+            hipLaunchKernelGGL(FanOutKernel<true>, dim3(tiles), dim3(64, a.nDst), 0, stream, a);
+        } else {
+            hipLaunchKernelGGL(FanOutKernel<false>, dim3(tiles), dim3(64, a.nDst), 0, stream, a);
+        }
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) {
             return e;

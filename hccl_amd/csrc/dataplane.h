@@ -238,6 +238,7 @@ struct FanOutArgs {
     uint32_t nDst;
 };
 bool FanOutTakes(const FanOutArgs& args);
-hipError_t LaunchFanOut(const FanOutArgs& args, hipStream_t stream);
+// streamLoad: the source is read with non-temporal loads, which leave it out of the caches it passes.
+hipError_t LaunchFanOut(const FanOutArgs& args, bool streamLoad, hipStream_t stream);
 
 }  // namespace hccl_amd

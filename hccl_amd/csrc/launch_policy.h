@@ -1,0 +1,100 @@
+// The form a collective is launched in: every threshold the launch planners use, in one place, each with the
+// measurement it came from.  All figures are fractions of the 8 TB/s HBM peak on one MI355X, timed in one process
+// on the same buffers (buffer sets in rotation where a set would fit the 256 MB last-level cache); boxes of the
+// pool differ by a few per cent, crossovers move little.  `python -m hccl_amd.tune` times both sides of every
+// threshold on the GPU at hand.
+//
+// Environment overrides (read at world creation) are named with each entry.
+#pragma once
+
+#include <stdint.h>
+
+namespace hccl_amd {
+namespace policy {
+
+constexpr uint64_t kMiB = 1ull << 20;
+
+// ---- AllReduce, Reduce, ReduceScatter(V): the fused reduce kernel ----------------------------------------
+// Workgroups of one wavefront (64 lanes, one 16-byte vector each): small workgroups retire sooner and keep the
+// window of addresses in flight compact; measured best for flat and nested programs alike (128: -9 %, 256: -3 %
+// on 8 ranks x 4 MiB).  HCCL_AMD_REDUCE_THREADS.
+constexpr uint32_t kReduceThreads = 64;
+
+// Leaves whose loads are issued together.  Up to eight ranks folded into one result stream run best with
+// eight-load batches (fewer registers, more wavefronts in flight: +1-2 %); a result that goes to many destinations
+// and larger worlds with sixteen (+5 %).  8 ranks x 4 MiB: equal.  HCCL_AMD_REDUCE_BATCH.
+inline uint32_t VecBatch(uint32_t ranks, bool oneResultStream, bool unequalGroups)
+{
+    return (ranks <= 8 && !unequalGroups && oneResultStream) ? 8u : 16u;
+}
+
+// A result written once (ReduceScatter(V), Reduce, the fold of the two-kernel AllReduce) leaves through
+// write-through stores, 3-4 % faster than non-temporal ones next to eight read streams; a result written to many
+// destinations keeps non-temporal stores, 2-3 % faster there.  HCCL_AMD_STORE_POLICY.
+inline bool WriteThrough(bool oneResultStream) { return oneResultStream; }
+
+// Wavefronts that share the stores of a fused tile (wavefront 0 folds, every wavefront stores to its share of the
+// destinations): `bytes` per rank, `elemSize` of the type.
+//   4-7 destinations, from 48 MiB: two.  fp32 over 4 ranks 0.72 -> 0.74 / 0.75 -> 0.79 / 0.76 -> 0.79 at 64 / 256 /
+//     512 MiB; over 6 ranks 0.70 -> 0.75 / 0.74 -> 0.79 / 0.70 -> 0.77; three wavefronts 0.77 / 0.78 / 0.76; at
+//     16-32 MiB one wavefront wins by a point; two and three ranks lose at every size (0.83 -> 0.61, 0.80 -> 0.76).
+//   8 and more destinations: three from 24 MiB for 4- and 8-byte types (8 ranks 0.70 -> 0.78 at 64 MiB), two from
+//     64 MiB for the 1- and 2-byte types, whose folds take longer (the waiting wavefronts hold slots).
+// HCCL_AMD_REDUCE_STORE_WAVES.
+inline uint32_t StoreWaves(uint32_t nDst, uint64_t bytes, uint32_t elemSize)
+{
+    const bool longFold = elemSize < 4;
+    if (nDst >= 8) {
+        return longFold ? (bytes >= 64 * kMiB ? 2u : 1u) : (bytes >= 24 * kMiB ? 3u : 1u);
+    }
+    if (nDst >= 4) {
+        return bytes >= 48 * kMiB ? 2u : 1u;
+    }
+    return 1u;
+}
+// With the stores elsewhere the folding wavefront is better off with the eight-load batch where that holds every
+// leaf (fp16 RHD over 6 ranks 0.71 -> 0.75, fp16 NHR over 8 ranks 0.71 -> 0.77).
+inline uint32_t VecBatchWithSharedStores(uint32_t ranks, uint32_t batch) { return ranks <= 8 ? 8u : batch; }
+
+// ---- AllReduce as fold + fan-out ------------------------------------------------------------------------
+// All ranks folded into the first recvBuf, then that range to the other recvBufs with one wavefront per
+// destination.  Two kernels / fused, fp32 SUM in rank order:
+//   ranks    8 MiB         16 MiB        32 MiB        64 MiB        256 MiB per rank
+//     4                  0.63 / 0.62   0.69 / 0.67   0.74 / 0.74   0.77 / 0.79
+//     5                  0.65 / 0.62                 0.76 / 0.72   0.79 / 0.78
+//     6    0.57 / 0.58   0.66 / 0.63   0.73 / 0.69   0.78 / 0.75   0.82 / 0.79
+//     8    0.60 / 0.60   0.67 / 0.62   0.75 / 0.71   0.79 / 0.78   0.82 / 0.76
+//    16    0.65 / 0.57   0.74 / 0.58   0.79 / 0.73   0.82 / 0.76   0.83 / 0.74
+// (2 and 3 ranks lose: 0.69 / 0.83, 0.74 / 0.80.)  HCCL_AMD_ALLREDUCE_TWO_KERNELS = 0 / 1 forces a form.
+inline bool FoldThenFanOut(uint32_t nDst, uint64_t bytes)
+{
+    return nDst >= 12 ? bytes >= 8 * kMiB : (nDst >= 5 && bytes >= 16 * kMiB);
+}
+// Mesh-chunk launches write one strip per slice, so their pieces are whole slices, which pays from eight ranks on
+// (8 ranks of 256 MiB 0.74 -> 0.81, 16 ranks of 64 MiB 0.71 -> 0.79; six ranks lose, 0.74 -> 0.71).
+constexpr uint32_t kMeshChunkFanOutMinRanks = 8;
+// A piece must still be cached when it is read back: 1 GiB per rank over 6 ranks 0.76 / 0.78 / 0.78 with pieces of
+// 64 / 128 / 256 MiB, 0.64 with 512 MiB; 512 MiB per rank fp16: 0.76 / 0.74 / 0.77 / 0.67 with 96 / 176 / 256 / 352 MiB.
+// HCCL_AMD_ALLREDUCE_PIECE_BYTES.
+constexpr uint64_t kPieceBytes = 256 * kMiB;
+
+// The fan-out kernel's load of the range the kernel before it wrote.  A plain load lets the wavefronts behind the
+// first find the tile cached, but what it leaves in the caches slows the fold of the next piece down; a
+// non-temporal load leaves nothing behind and costs where many wavefronts share a tile.  AllReduce fp32, plain /
+// non-temporal: 512 MiB per rank (two pieces) over 5 / 6 / 7 / 8 / 10 / 12 ranks 0.77 / 0.79, 0.77 / 0.80, 0.78 / 0.80,
+// 0.78 / 0.79, 0.77 / 0.78, 0.76 / 0.77 (fp16 RHD over 6 ranks 0.79 / 0.81); one piece of 256 MiB over 5-7 ranks
+// equal, over 8 / 10 / 12 / 16 ranks 0.83 / 0.82, 0.83 / 0.82, 0.82 / 0.80, 0.81 / 0.78; 16 ranks in pieces of
+// 128 MiB 0.83 / 0.79; Broadcast to 7 ranks equal.  So: up to six destinations always, up to eleven where another
+// piece follows.
+inline bool FanOutStreamLoad(uint32_t nDst, bool severalPieces) { return nDst <= 6 || (severalPieces && nDst <= 11); }
+
+// ---- AllGather(V), Broadcast: gather + fan-out ----------------------------------------------------------
+// The segments into the first destination with the plain copy, then that range to the other destinations.  Two
+// kernels / one, `bytes` per destination: AllGather of 16 x 64 MiB 0.84 / 0.69, 16 x 16 MiB 0.76 / 0.68, 8 x 128 MiB
+// 0.77 / 0.71, 8 x 8 MiB 0.76 / 0.69, 6 x 32 MiB 0.72 / 0.74, 6 ranks of 2-64 MiB at odd displacements 0.74 / 0.76,
+// 4 x 64 MiB 0.67 / 0.77; Broadcast of 128 MiB to 15 ranks 0.78 / 0.68, to 7 ranks 0.81 / 0.73 (16 MiB: 0.61 / 0.65),
+// to 5 ranks 0.72 / 0.77.  HCCL_AMD_COPY_TWO_KERNELS = 0 / 1 forces a form.
+inline bool GatherThenFanOut(uint32_t nDst, uint64_t bytes) { return nDst >= 7 && bytes >= 48 * kMiB; }
+
+}  // namespace policy
+}  // namespace hccl_amd

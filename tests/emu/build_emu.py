@@ -25,7 +25,7 @@ CLANG = "/opt/rocm/llvm/bin/clang++"
 
 KERNEL_UNITS = ["reduce_i8", "reduce_i16", "reduce_i32", "reduce_i64", "reduce_u64", "reduce_f16", "reduce_bf16",
                 "reduce_f32", "reduce_f64", "reduce_launch", "copy_kernels"]
-HOST_UNITS = ["api", "fold_plan", "algo_config"]
+HOST_UNITS = ["api", "host_world", "launch_reduce", "launch_copy", "rendezvous", "fold_plan", "algo_config"]
 
 # inline assembly with a meaning -> that meaning
 ASM_RULES = [
