@@ -174,7 +174,7 @@ class Workloads:
 
         hbm = (1 + n) * total * 2
         return step, hbm, total * 2, (n - 1) / n, (sends, recvs), \
-            "AllGatherV fp16 rankSize=6 counts U[1Mi,32Mi], 4 buffer sets in rotation", "u8", n, "mesh"
+            "AllGatherV fp16 rankSize=6 counts U[1Mi,32Mi], 4 buffer sets in rotation", "f16", n, "mesh"
 
     def copycal(self, algo):
         """Plain copy of known size (the rankSize == 1 shortcut): calibrates the HBM byte counters."""
@@ -270,7 +270,7 @@ class Workloads:
 
         total = n * count * 2
         return step, (1 + n) * total, total, (n - 1) / n, (sends, recvs), \
-            "AllGather bf16 rankSize=16 32Mi el/rank", "u8", n, "mesh"
+            "AllGather bf16 rankSize=16 32Mi el/rank", "bf16", n, "mesh"
 
     def scatter(self, algo):
         t, h = self.torch, self.h
@@ -306,7 +306,7 @@ class Workloads:
 
         total = n * n * count * 2
         return step, 2 * total, total // n, (n - 1) / n, (sends, recvs), \
-            "AlltoAll bf16 rankSize=16 4Mi el per pair", "u8", n, "mesh"
+            "AlltoAll bf16 rankSize=16 4Mi el per pair", "bf16", n, "mesh"
 
     def c4(self, algo):
         import numpy as np
@@ -332,7 +332,7 @@ class Workloads:
 
         total = int(sc.sum()) * 2
         return step, 2 * total, total // n, (n - 1) / n, (sends, recvs), \
-            "AlltoAllV bf16 rankSize=64 16384 tokens x 7168 per rank, Zipf(1.1) routing", "u8", n, "mesh"
+            "AlltoAllV bf16 rankSize=64 16384 tokens x 7168 per rank, Zipf(1.1) routing", "bf16", n, "mesh"
 
 
 def time_steps(torch, stream, step, steps, warmup):
@@ -560,9 +560,12 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(hbm / t / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(hbm / t / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": traffic,
-                     "traffic_source": (TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier run, "
-                                        "calibrated against a plain copy; not measured in this run)") if traffic else None,
-                     "algorithmic_bytes_per_launch": hbm, "kernel_ms": main_res["ms_per_step"]},
+                     "traffic_source": (TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of this kernel in a "
+                                        "profiling run of this command, calibrated against a plain copy; the "
+                                        "counters cannot be read while timing)") if traffic else None,
+                     "algorithmic_bytes_per_launch": hbm, "launch_ms": main_res["ms_per_step"],
+                     "timing": "HIP events on the launch stream around the timed steps, one kernel launch per step "
+                               "(the rocprofv3 kernel duration of the same command is in profiles/)"},
         "cpu_baseline": cpu,
     }
     if others:

@@ -92,7 +92,7 @@ HcclResult RunBcast(World* w, BcastCopyArgs& b, hipStream_t s)
 // the other is what bounds the one-kernel form.  Taken when the destinations share their offset from a 16-byte
 // boundary and the segments' destination ranges do not overlap; runs of adjacent ranges fan out in one launch.
 // `bytes` is what every destination receives (launch_policy.h has the measurements).
-bool GatherThenFanOut(const World* w, uint32_t nDst, uint64_t bytes)
+bool GatherThenFanOut(const World* w, uint32_t nDst, uint64_t bytes, bool congruent)
 {
     if (nDst < 3) {
         return false;
@@ -100,7 +100,7 @@ bool GatherThenFanOut(const World* w, uint32_t nDst, uint64_t bytes)
     if (w->copyTwoKernelMode != 2) {
         return w->copyTwoKernelMode == 1;
     }
-    return policy::GatherThenFanOut(nDst, bytes);
+    return policy::GatherThenFanOut(nDst, bytes, congruent);
 }
 
 HcclResult RunOneToMany(World* w, BcastCopyArgs& b, hipStream_t s)
@@ -113,13 +113,21 @@ HcclResult RunOneToMany(World* w, BcastCopyArgs& b, hipStream_t s)
             order.push_back(j);
         }
     }
-    if (!GatherThenFanOut(w, b.nDst, total)) {
+    bool congruent = true;   // every source shares the offset of its place in the first destination from a 16-byte boundary
+    for (uint32_t j : order) {
+        congruent = congruent && ((reinterpret_cast<uint64_t>(b.src[j]) ^
+                                   (reinterpret_cast<uint64_t>(b.dst[0]) + b.dstOff[j])) & 15u) == 0;
+    }
+    bool dstCongruent = true;
+    for (uint32_t d = 1; d < b.nDst; ++d) {
+        dstCongruent = dstCongruent &&
+                       ((reinterpret_cast<uint64_t>(b.dst[d]) ^ reinterpret_cast<uint64_t>(b.dst[0])) & 15u) == 0;
+    }
+    if (!GatherThenFanOut(w, b.nDst, total, congruent)) {
         return RunBcast(w, b, s);
     }
-    for (uint32_t d = 1; d < b.nDst; ++d) {
-        if (((reinterpret_cast<uint64_t>(b.dst[d]) ^ reinterpret_cast<uint64_t>(b.dst[0])) & 15u) != 0) {
-            return RunBcast(w, b, s);
-        }
+    if (!dstCongruent) {
+        return RunBcast(w, b, s);
     }
     std::sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { return b.dstOff[x] < b.dstOff[y]; });
     for (size_t i = 1; i < order.size(); ++i) {

@@ -93,8 +93,15 @@ inline bool FanOutStreamLoad(uint32_t nDst, bool severalPieces) { return nDst <=
 // kernels / one, `bytes` per destination: AllGather of 16 x 64 MiB 0.84 / 0.69, 16 x 16 MiB 0.76 / 0.68, 8 x 128 MiB
 // 0.77 / 0.71, 8 x 8 MiB 0.76 / 0.69, 6 x 32 MiB 0.72 / 0.74, 6 ranks of 2-64 MiB at odd displacements 0.74 / 0.76,
 // 4 x 64 MiB 0.67 / 0.77; Broadcast of 128 MiB to 15 ranks 0.78 / 0.68, to 7 ranks 0.81 / 0.73 (16 MiB: 0.61 / 0.65),
-// to 5 ranks 0.72 / 0.77.  HCCL_AMD_COPY_TWO_KERNELS = 0 / 1 forces a form.
-inline bool GatherThenFanOut(uint32_t nDst, uint64_t bytes) { return nDst >= 7 && bytes >= 48 * kMiB; }
+// to 5 ranks 0.72 / 0.77.  Six destinations: from 160 MiB per destination where every source shares its
+// destination's offset from a 16-byte boundary (6 x 16 MiB 0.74 / 0.74, 6 x 32 MiB 0.77 / 0.73, 6 x 64 MiB 0.77 / 0.72,
+// 6 x 128 MiB 0.76 / 0.73; with lanes realigning the bytes the first kernel is the slower one and the one-kernel
+// form stays ahead, 0.74 / 0.76); five destinations never (0.72-0.74 / 0.75-0.77 from 16 to 128 MiB per rank).
+// HCCL_AMD_COPY_TWO_KERNELS = 0 / 1 forces a form.
+inline bool GatherThenFanOut(uint32_t nDst, uint64_t bytes, bool congruent)
+{
+    return (nDst >= 7 && bytes >= 48 * kMiB) || (nDst == 6 && congruent && bytes >= 160 * kMiB);
+}
 
 }  // namespace policy
 }  // namespace hccl_amd
