@@ -97,10 +97,19 @@ inline bool FanOutStreamLoad(uint32_t nDst, bool severalPieces) { return nDst <=
 // destination's offset from a 16-byte boundary (6 x 16 MiB 0.74 / 0.74, 6 x 32 MiB 0.77 / 0.73, 6 x 64 MiB 0.77 / 0.72,
 // 6 x 128 MiB 0.76 / 0.73; with lanes realigning the bytes the first kernel is the slower one and the one-kernel
 // form stays ahead, 0.74 / 0.76); five destinations never (0.72-0.74 / 0.75-0.77 from 16 to 128 MiB per rank).
-// HCCL_AMD_COPY_TWO_KERNELS = 0 / 1 forces a form.
+// Where the forms cross, per destination: 16 ranks 16 MiB 0.74 / 0.60, 32 MiB 0.82 / 0.59; 12 ranks 12 MiB 0.66 / 0.66,
+// 24 MiB 0.68 / 0.65, 36 MiB 0.74 / 0.65; 10 ranks 20 MiB 0.69 / 0.67, 30 MiB 0.72 / 0.69, 40 MiB 0.77 / 0.72; 8 ranks
+// 16 MiB 0.65 / 0.66, 24 MiB 0.70 / 0.69, 32 MiB 0.71 / 0.69, 40 MiB 0.73 / 0.71; 7 ranks 21-42 MiB 0.65-0.69 / 0.69-0.72,
+// 49 MiB 0.72 / 0.71.  HCCL_AMD_COPY_TWO_KERNELS = 0 / 1 forces a form.
 inline bool GatherThenFanOut(uint32_t nDst, uint64_t bytes, bool congruent)
 {
-    return (nDst >= 7 && bytes >= 48 * kMiB) || (nDst == 6 && congruent && bytes >= 160 * kMiB);
+    if (nDst >= 14) {
+        return bytes >= 16 * kMiB;
+    }
+    if (nDst >= 8) {
+        return bytes >= 24 * kMiB;
+    }
+    return (nDst == 7 && bytes >= 48 * kMiB) || (nDst == 6 && congruent && bytes >= 160 * kMiB);
 }
 
 }  // namespace policy

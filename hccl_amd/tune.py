@@ -126,6 +126,37 @@ def all_gather_rows(torch, h, ranks, mibs, rounds):
             torch.cuda.empty_cache()
 
 
+def broadcast_rows(torch, h, ranks, mibs, rounds):
+    print("# Broadcast from rank 0: one kernel, copy + fan-out, the library's own choice")
+    for n in ranks:
+        for mib in mibs:
+            nbytes = mib << 20
+            per_set = n * nbytes
+            sets = max(1, min(8, -(-(600 << 20) // per_set)))
+            bufs = [[torch.randint(0, 255, (nbytes,), device="cuda", dtype=torch.uint8) for _ in range(n)]
+                    for _ in range(sets)]
+            torch.cuda.synchronize()
+
+            def make_step(stream):
+                comms = h.comm_init_all(n)
+                turn = [0]
+
+                def step():
+                    k = turn[0]
+                    turn[0] = (k + 1) % sets
+                    with h.group():
+                        for r in range(n):
+                            h.broadcast(comms[r], bufs[k][r], nbytes, h.HcclDataType.UINT8, 0, stream)
+                return comms, step
+
+            forms = [("one", {"HCCL_AMD_COPY_TWO_KERNELS": "0"}), ("two", {"HCCL_AMD_COPY_TWO_KERNELS": "1"}),
+                     ("auto", {})]
+            steps = 10 if per_set > (200 << 20) else 50
+            _row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps))
+            del bufs
+            torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--quick", action="store_true", help="a third of the grid, one round")
@@ -140,6 +171,7 @@ def main():
     all_reduce_rows(torch, h, [3, 4, 6, 8, 16] if not args.quick else [4, 8], [16, 64, 256] if not args.quick else [64],
                     rounds)
     all_gather_rows(torch, h, [4, 6, 8, 16] if not args.quick else [8], [8, 64] if not args.quick else [64], rounds)
+    broadcast_rows(torch, h, [6, 8, 16] if not args.quick else [8], [16, 64] if not args.quick else [64], rounds)
 
 
 if __name__ == "__main__":
