@@ -93,9 +93,9 @@ inline bool FanOutStreamLoad(uint32_t nDst, bool severalPieces) { return nDst <=
 // kernels / one, `bytes` per destination: AllGather of 16 x 64 MiB 0.84 / 0.69, 16 x 16 MiB 0.76 / 0.68, 8 x 128 MiB
 // 0.77 / 0.71, 8 x 8 MiB 0.76 / 0.69, 6 x 32 MiB 0.72 / 0.74, 6 ranks of 2-64 MiB at odd displacements 0.74 / 0.76,
 // 4 x 64 MiB 0.67 / 0.77; Broadcast of 128 MiB to 15 ranks 0.78 / 0.68, to 7 ranks 0.81 / 0.73 (16 MiB: 0.61 / 0.65),
-// to 5 ranks 0.72 / 0.77.  Six destinations: from 160 MiB per destination where every source shares its
+// to 5 ranks 0.72 / 0.77.  Six destinations: from 128 MiB per destination where every source shares its
 // destination's offset from a 16-byte boundary (6 x 16 MiB 0.74 / 0.74, 6 x 32 MiB 0.77 / 0.73, 6 x 64 MiB 0.77 / 0.72,
-// 6 x 128 MiB 0.76 / 0.73; with lanes realigning the bytes the first kernel is the slower one and the one-kernel
+// 6 x 128 MiB 0.76 / 0.73, Broadcast of 64 / 128 / 192 MiB 0.73 / 0.73, 0.76 / 0.72, 0.77 / 0.73; with lanes realigning the bytes the first kernel is the slower one and the one-kernel
 // form stays ahead, 0.74 / 0.76); five destinations never (0.72-0.74 / 0.75-0.77 from 16 to 128 MiB per rank).
 // Where the forms cross, per destination: 16 ranks 16 MiB 0.74 / 0.60, 32 MiB 0.82 / 0.59; 12 ranks 12 MiB 0.66 / 0.66,
 // 24 MiB 0.68 / 0.65, 36 MiB 0.74 / 0.65; 10 ranks 20 MiB 0.69 / 0.67, 30 MiB 0.72 / 0.69, 40 MiB 0.77 / 0.72; 8 ranks
@@ -109,7 +109,7 @@ inline bool GatherThenFanOut(uint32_t nDst, uint64_t bytes, bool congruent)
     if (nDst >= 8) {
         return bytes >= 24 * kMiB;
     }
-    return (nDst == 7 && bytes >= 48 * kMiB) || (nDst == 6 && congruent && bytes >= 160 * kMiB);
+    return (nDst == 7 && bytes >= 48 * kMiB) || (nDst == 6 && congruent && bytes >= 128 * kMiB);
 }
 
 }  // namespace policy

@@ -1,6 +1,7 @@
 """Times both sides of the launch-form thresholds of hccl_amd/csrc/launch_policy.h on the GPU at hand.
 
     python -m hccl_amd.tune [--quick]
+    python -m hccl_amd.tune --all-gather 16:1,2 8:2,4,6 --broadcast 9:16,24,32     (ranks:MiB per rank,... per table)
 
 For every shape of a small grid the forms the policy chooses between are run on the same buffers, interleaved
 (worlds created with the overriding environment variable set), and the table shows each form's fraction of the 8 TB/s
@@ -160,6 +161,9 @@ def broadcast_rows(torch, h, ranks, mibs, rounds):
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--quick", action="store_true", help="a third of the grid, one round")
+    ap.add_argument("--all-reduce", nargs="*", metavar="RANKS:MIB,..", help="AllReduce rows of these shapes only")
+    ap.add_argument("--all-gather", nargs="*", metavar="RANKS:MIB,..", help="AllGather rows of these shapes only")
+    ap.add_argument("--broadcast", nargs="*", metavar="RANKS:MIB,..", help="Broadcast rows of these shapes only")
     args = ap.parse_args()
     import torch
     import hccl_amd as h
@@ -168,6 +172,13 @@ def main():
     torch.cuda.set_device(0)
     h.lib()
     rounds = 1 if args.quick else 3
+    chosen = [(args.all_reduce, all_reduce_rows), (args.all_gather, all_gather_rows), (args.broadcast, broadcast_rows)]
+    if any(specs is not None for specs, _ in chosen):
+        for specs, rows in chosen:
+            for spec in specs or []:
+                ranks, mibs = spec.split(":")
+                rows(torch, h, [int(ranks)], [int(m) for m in mibs.split(",")], rounds)
+        return
     all_reduce_rows(torch, h, [3, 4, 6, 8, 16] if not args.quick else [4, 8], [16, 64, 256] if not args.quick else [64],
                     rounds)
     all_gather_rows(torch, h, [4, 6, 8, 16] if not args.quick else [8], [8, 64] if not args.quick else [64], rounds)
