@@ -53,15 +53,18 @@ def _forms(torch, h, make_step, forms, moved, rounds, steps):
 
 
 def _row(label, fracs, own="auto"):
+    """Prints one row and returns (label, fracs)."""
     best = max((v, k) for k, v in fracs.items() if k != own)
     flag = "   <-- %s is %.1f %% ahead of the library's choice" % (best[1], 100 * (best[0] / fracs[own] - 1)) \
         if best[0] > 1.02 * fracs[own] else ""
     print("%-34s %s%s" % (label, "  ".join("%s %.3f" % (k, v) for k, v in fracs.items()), flag), flush=True)
+    return label, fracs
 
 
 def all_reduce_rows(torch, h, ranks, mibs, rounds):
     print("# AllReduce fp32 SUM in rank order: fused kernel with 1 / 2 / 3 wavefronts sharing a tile's stores, fold + "
           "fan-out, the library's own choice")
+    rows = []
     for n in ranks:
         for mib in mibs:
             count = (mib << 20) // 4
@@ -90,13 +93,15 @@ def all_reduce_rows(torch, h, ranks, mibs, rounds):
                      ("w3", dict(fused, HCCL_AMD_REDUCE_STORE_WAVES="3")),
                      ("two", {"HCCL_AMD_ALLREDUCE_TWO_KERNELS": "1"}), ("auto", {})]
             steps = 10 if per_set > (200 << 20) else 50
-            _row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps))
+            rows.append(_row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps)))
             del sends, recvs
             torch.cuda.empty_cache()
+    return rows
 
 
 def all_gather_rows(torch, h, ranks, mibs, rounds):
     print("# AllGather: one kernel, gather + fan-out, the library's own choice")
+    rows = []
     for n in ranks:
         for mib in mibs:
             nbytes = mib << 20
@@ -122,13 +127,15 @@ def all_gather_rows(torch, h, ranks, mibs, rounds):
             forms = [("one", {"HCCL_AMD_COPY_TWO_KERNELS": "0"}), ("two", {"HCCL_AMD_COPY_TWO_KERNELS": "1"}),
                      ("auto", {})]
             steps = 10 if per_set > (200 << 20) else 50
-            _row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps))
+            rows.append(_row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps)))
             del sends, recvs
             torch.cuda.empty_cache()
+    return rows
 
 
 def broadcast_rows(torch, h, ranks, mibs, rounds):
     print("# Broadcast from rank 0: one kernel, copy + fan-out, the library's own choice")
+    rows = []
     for n in ranks:
         for mib in mibs:
             nbytes = mib << 20
@@ -153,9 +160,10 @@ def broadcast_rows(torch, h, ranks, mibs, rounds):
             forms = [("one", {"HCCL_AMD_COPY_TWO_KERNELS": "0"}), ("two", {"HCCL_AMD_COPY_TWO_KERNELS": "1"}),
                      ("auto", {})]
             steps = 10 if per_set > (200 << 20) else 50
-            _row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps))
+            rows.append(_row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps)))
             del bufs
             torch.cuda.empty_cache()
+    return rows
 
 
 def main():
