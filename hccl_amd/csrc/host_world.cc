@@ -284,6 +284,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->twoKernelMode < 0 || w->twoKernelMode > 1) {
         w->twoKernelMode = 2;
     }
+    w->fanOutLoadMode = EnvInt("HCCL_AMD_FANOUT_STREAM_LOAD", 2);
+    if (w->fanOutLoadMode < 0 || w->fanOutLoadMode > 1) {
+        w->fanOutLoadMode = 2;
+    }
     w->copyTwoKernelMode = EnvInt("HCCL_AMD_COPY_TWO_KERNELS", 2);
     if (w->copyTwoKernelMode < 0 || w->copyTwoKernelMode > 1) {
         w->copyTwoKernelMode = 2;

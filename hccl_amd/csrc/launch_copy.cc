@@ -184,7 +184,7 @@ HcclResult RunOneToMany(World* w, BcastCopyArgs& b, hipStream_t s)
             }
             // (a copy in front of it, not a fold: a non-temporal load only loses here, AllGather over 16 ranks
             // 0.84 -> 0.81)
-            HIP_OK(LaunchFanOut(f, policy::FanOutStreamLoad(f.nDst, false), s));
+            HIP_OK(LaunchFanOut(f, w->fanOutLoadMode != 2 ? w->fanOutLoadMode == 1 : policy::FanOutStreamLoad(f.nDst, false), s));
         }
     }
     return HCCL_SUCCESS;

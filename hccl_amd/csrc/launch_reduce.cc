@@ -178,7 +178,7 @@ HcclResult FanOutFromFirst(World* w, void* const* dst, uint32_t nDst, uint64_t o
         f.dst[k - 1] = static_cast<uint8_t*>(dst[k]) + off;
     }
     if (FanOutTakes(f)) {
-        HIP_OK(LaunchFanOut(f, policy::FanOutStreamLoad(f.nDst, severalPieces), s));
+        HIP_OK(LaunchFanOut(f, w->fanOutLoadMode != 2 ? w->fanOutLoadMode == 1 : policy::FanOutStreamLoad(f.nDst, severalPieces), s));
         return HCCL_SUCCESS;
     }
     BcastCopyArgs b{};

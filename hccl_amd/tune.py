@@ -99,6 +99,9 @@ def all_reduce_rows(torch, h, ranks, mibs, rounds):
     return rows
 
 
+COPY_FORMS = [("one", {"HCCL_AMD_COPY_TWO_KERNELS": "0"}), ("two", {"HCCL_AMD_COPY_TWO_KERNELS": "1"}), ("auto", {})]
+
+
 def all_gather_rows(torch, h, ranks, mibs, rounds):
     print("# AllGather: one kernel, gather + fan-out, the library's own choice")
     rows = []
@@ -124,8 +127,7 @@ def all_gather_rows(torch, h, ranks, mibs, rounds):
                             h.all_gather(comms[r], sends[k][r], recvs[k][r], nbytes, h.HcclDataType.UINT8, stream)
                 return comms, step
 
-            forms = [("one", {"HCCL_AMD_COPY_TWO_KERNELS": "0"}), ("two", {"HCCL_AMD_COPY_TWO_KERNELS": "1"}),
-                     ("auto", {})]
+            forms = COPY_FORMS
             steps = 10 if per_set > (200 << 20) else 50
             rows.append(_row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps)))
             del sends, recvs
@@ -157,8 +159,7 @@ def broadcast_rows(torch, h, ranks, mibs, rounds):
                             h.broadcast(comms[r], bufs[k][r], nbytes, h.HcclDataType.UINT8, 0, stream)
                 return comms, step
 
-            forms = [("one", {"HCCL_AMD_COPY_TWO_KERNELS": "0"}), ("two", {"HCCL_AMD_COPY_TWO_KERNELS": "1"}),
-                     ("auto", {})]
+            forms = COPY_FORMS
             steps = 10 if per_set > (200 << 20) else 50
             rows.append(_row("%2d ranks x %4d MiB" % (n, mib), _forms(torch, h, make_step, forms, per_set, rounds, steps)))
             del bufs
