@@ -90,16 +90,18 @@ class Workloads:
         recvs = [[t.empty(count, dtype=tdtype, device="cuda") for _ in range(n)] for _ in range(sets)]
         opk = h.OpKind.REDUCE_SCATTER if kind == "rs" else h.OpKind.ALL_REDUCE
         h.set_algo(comms[0], opk, h.Algo[algo.upper()])
-        fn = h.reduce_scatter if kind == "rs" else h.all_reduce
+        entry = "HcclReduceScatter" if kind == "rs" else "HcclAllReduce"
         stream = self.stream
         turn = [0]
+        # one collective = the n per-rank calls of the C ABI inside a group; their arguments are converted to C types
+        # once per buffer set (a collective of 15 us would otherwise wait for Python's conversions)
+        groups = [h.prepared_group([(entry, (sends[k][r], recvs[k][r], count, hdtype, op, comms[r], stream))
+                                    for r in range(n)]) for k in range(sets)]
 
         def step():
             k = turn[0]
             turn[0] = (k + 1) % sets
-            with h.group():
-                for r in range(n):
-                    fn(comms[r], sends[k][r], recvs[k][r], count, hdtype, op, stream)
+            groups[k]()
 
         esz = sends[0][0].element_size()
         if kind == "rs":

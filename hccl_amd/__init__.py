@@ -354,6 +354,40 @@ def all_reduce(hccl_comm, send_buf, recv_buf, count, data_type=HcclDataType.FP32
     return check(code, "HcclAllReduce")
 
 
+def prepared_group(calls):
+    """One collective of a host thread that drives all ranks, for loops that repeat it: `calls` is a list of
+    (entry point name, argument tuple) with the arguments as the mirror functions would pass them (buffers, counts,
+    enums, communicator, stream); they are converted to their C types once, and the function returned issues
+    HcclGroupStart, the calls and HcclGroupEnd.  Saves the per-call conversions, which cost more than the library's
+    own host work when a collective runs for a few microseconds."""
+    library = lib()
+    start, end = library.HcclGroupStart, library.HcclGroupEnd
+    bound = []
+    for name, args in calls:
+        fn = getattr(library, name)
+        conv = []
+        for a, ctype in zip(args, fn.argtypes):
+            if ctype is ctypes.c_void_p:
+                conv.append(_as_ptr(a) if not hasattr(a, "cuda_stream") else _as_stream(a))
+            elif isinstance(a, enum.IntEnum):
+                conv.append(int(a))
+            elif isinstance(a, int):
+                conv.append(ctype(a))
+            else:
+                conv.append(a)
+        bound.append((fn, tuple(conv), name))
+
+    def run():
+        start()
+        for fn, conv, name in bound:
+            code = fn(*conv)
+            if code:
+                end()
+                check(code, name)
+        return check(end(), "HcclGroupEnd")
+    return run
+
+
 def reduce_scatter(hccl_comm, send_buf, recv_buf, recv_count, data_type=HcclDataType.FP32,
                    reduce_op=HcclReduceOp.SUM, stream=None):
     code = lib().HcclReduceScatter(_as_ptr(send_buf), _as_ptr(recv_buf), ctypes.c_uint64(recv_count), int(data_type),

@@ -78,7 +78,7 @@ struct ReduceHot {
     uint32_t blocksPerSub;   // workgroups per sub-segment: the grid is (blocksPerSub, nSub, nGroup), or one-dimensional with varGroups
     uint32_t vecOk;   // take the 128-bit path (0: element by element, for testing)
     uint32_t threads; // workgroup size of the launch
-    uint32_t vecBatch;       // leaves per load batch of the 128-bit path: 8 or 16 (picks the kernel instantiation)
+    uint32_t vecBatch;       // leaves per load batch of the 128-bit path: 8 or 16, or kVecBatchPair (picks the kernel instantiation)
     uint32_t writeThrough;   // 16-byte results leave through StoreStream16 instead of a non-temporal store
     uint32_t leadFromSrc;    // wavefronts start on a 1 KiB boundary of the sources instead of the destination's
     uint32_t storeWaves;     // > 1: workgroups of 64 * storeWaves threads, wavefront 0 folds and wavefront k stores to
@@ -86,6 +86,10 @@ struct ReduceHot {
                              // folds and stores its own tile
     uint32_t varGroups;      // groups of unequal length, see below
 };
+
+// vecBatch of the form for short launches: eight-leaf batches, two adjacent tiles per wavefront (threads 64, no shared
+// stores, uniform groups; blocksPerSub counts pairs of tiles).
+constexpr uint32_t kVecBatchPair = 0x108;
 
 struct ReduceArgs : ReduceHot {
     const void* src[kMaxRanks];

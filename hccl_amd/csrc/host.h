@@ -91,6 +91,7 @@ struct DevicePlan {
     uint8_t* dev = nullptr;
     uint32_t nProg = 0;
     uint32_t maxDepth = 1;
+    uint32_t maxLeaves = 0;   // most leaves of any program of the plan
     bool segmentsAreSubs = false;
 };
 
@@ -151,6 +152,7 @@ struct World {
     // AllReduce as fold + fan-out (two kernels per piece of at most pieceBytes of results).
     uint64_t pieceBytes = 256ull << 20;   // HCCL_AMD_ALLREDUCE_PIECE_BYTES
     int twoKernelMode = 2;                // HCCL_AMD_ALLREDUCE_TWO_KERNELS: 0 never, 1 always, unset: by rank count and size
+    int reducePair = 2;                   // HCCL_AMD_REDUCE_PAIR: 0 never, 1 wherever the form fits, else launch_policy.h decides
     int fanOutLoadMode = 2;               // HCCL_AMD_FANOUT_STREAM_LOAD: 0 plain, 1 non-temporal, else launch_policy.h decides
     int copyTwoKernelMode = 2;            // HCCL_AMD_COPY_TWO_KERNELS, likewise for AllGather(V) and Broadcast
     // Allocation-free AlltoAllV: host image of the tables and the device array that receives them.

@@ -284,6 +284,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->twoKernelMode < 0 || w->twoKernelMode > 1) {
         w->twoKernelMode = 2;
     }
+    w->reducePair = EnvInt("HCCL_AMD_REDUCE_PAIR", 2);
+    if (w->reducePair < 0 || w->reducePair > 1) {
+        w->reducePair = 2;
+    }
     w->fanOutLoadMode = EnvInt("HCCL_AMD_FANOUT_STREAM_LOAD", 2);
     if (w->fanOutLoadMode < 0 || w->fanOutLoadMode > 1) {
         w->fanOutLoadMode = 2;
@@ -372,6 +376,7 @@ HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DeviceP
     }
     // Flatten every token program to the kernel's leaf table.
     std::vector<uint8_t> image(plan.programs.size() * kDevProgBytes, 0);
+    uint32_t maxLeaves = 0;
     for (size_t s = 0; s < plan.programs.size(); ++s) {
         uint8_t* img = image.data() + s * kDevProgBytes;
         uint32_t leaves = 0;
@@ -398,11 +403,13 @@ HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DeviceP
             }
         }
         img[0] = static_cast<uint8_t>(leaves);
+        maxLeaves = leaves > maxLeaves ? leaves : maxLeaves;
     }
     DevicePlan dp;
     dp.nProg = static_cast<uint32_t>(plan.programs.size());
     dp.segmentsAreSubs = plan.segmentsAreSubs;
     dp.maxDepth = plan.maxDepth;
+    dp.maxLeaves = maxLeaves;
     HIP_OK(hipMalloc(reinterpret_cast<void**>(&dp.dev), image.size()));
     HIP_OK(hipMemcpy(dp.dev, image.data(), image.size(), hipMemcpyHostToDevice));
     w->plans[key] = dp;

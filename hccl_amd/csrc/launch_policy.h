@@ -28,6 +28,24 @@ inline uint32_t VecBatch(uint32_t ranks, bool oneResultStream, bool unequalGroup
     return (ranks <= 8 && !unequalGroups && oneResultStream) ? 8u : 16u;
 }
 
+// Two adjacent tiles per wavefront, all sixteen loads issued before the first fold and both folds before the first
+// store (kVecBatchPair; flat programs of up to eight leaves).  A launch of a few thousand tiles is one generation of
+// wavefronts: all of them load, then all of them store, and the two phases add up; with pairs the second tile's
+// loads travel while the first tile's arrive.  AllReduce fp32 SUM in rank order, us per collective, one tile / two:
+//   ranks   1 MiB       2 MiB       3 MiB        4 MiB         6 MiB         8 MiB         12-16 MiB per rank
+//     8   6.4 / 6.6   8.4 / 7.4   10.4 / 9.7   15.3 / 14.0   20.0 / 19.6   26.5 / 27.1   37.8 / 39.7, 46.8 / 47.2
+//     6               6.4 / 6.3                11.8 / 10.3                 21.0 / 21.6
+//     4               5.2 / 5.1                 7.6 / 7.6                  14.9 / 15.0   26.0 / 26.3
+//     3                                         6.8 / 6.4                  11.3 / 11.4
+//     2                                         5.7 / 4.8                   8.5 / 8.0    13.7 / 14.4
+// (kernel time of 8 ranks x 4 MiB under rocprofv3: 15.7 / 14.5 us.)  A result written once does not gain: ReduceScatter
+// over 8 ranks, 512 KiB / 1 / 2 / 4 MiB out per rank 9.7 / 9.3, 16.2 / 16.2, 27.6 / 28.6, 50.0 / 52.3.
+// HCCL_AMD_REDUCE_PAIR = 0 / 1 forces.
+inline bool PairTiles(uint32_t ranks, bool oneResultStream, uint64_t bytesPerRank)
+{
+    return !oneResultStream && 2 * bytesPerRank >= 3 * kMiB && bytesPerRank <= (ranks <= 3 ? 8 : 6) * kMiB;
+}
+
 // A result written once (ReduceScatter(V), Reduce, the fold of the two-kernel AllReduce) leaves through
 // write-through stores, 3-4 % faster than non-temporal ones next to eight read streams; a result written to many
 // destinations keeps non-temporal stores, 2-3 % faster there.  HCCL_AMD_STORE_POLICY.

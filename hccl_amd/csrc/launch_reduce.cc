@@ -64,6 +64,12 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
         }
     }
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
+    if (a.vecOk && a.threads == 64 && a.storeWaves <= 1 && !a.varGroups && plan.maxLeaves <= 8 && plan.maxDepth == 1 &&
+        (w->reduceBatch == 0 || w->reducePair == 1) &&
+        (w->reducePair != 2 ? w->reducePair == 1 : policy::PairTiles(w->n, oneStream, a.total * esz))) {
+        a.vecBatch = kVecBatchPair;
+        a.blocksPerSub = (a.blocksPerSub + 1) / 2;   // a workgroup takes two tiles
+    }
     uint64_t blocks = subs * a.blocksPerSub;
     if (a.varGroups) {
         // every group gets the workgroups its own length needs (an empty group gets none)

@@ -645,12 +645,90 @@ __device__ __forceinline__ void ReduceOne(const ProgramView& pv, uint32_t* stack
     StoreResult<typename E::S, W, true>(args, h, out, dstOff + e, ownOrFirst, 0, 1);
 }
 
+// Two adjacent tiles per wavefront for flat programs (no nested levels) of up to eight leaves (one batch): the sixteen loads of both tiles
+// are issued before the first fold and both folds before the first store.
+// A launch that is a single generation of wavefronts (a few MiB per rank) otherwise reads, then writes, and pays
+// the ramp of each phase in full.  `on0` / `on1`: this lane has a vector in the first / second tile.
+template <class E, int W>
+__device__ __forceinline__ void ReducePair(const ProgramView& pv, uint32_t* stack, const ReduceArgs& args,
+                                           const ReduceHot& h, uint64_t e0, bool on0, bool on1, uint64_t dstOff,
+                                           uint64_t ownOrFirst, const FirstBatch<8>& first)
+{
+    (void)stack;
+    using S = typename E::S;
+    static_assert(sizeof(S) * W == 16, "the pair form exists for the 128-bit path only");
+    constexpr int kBatch = 8;
+    const uint64_t e1 = e0 + 64u * W;
+    const uint32_t nLeaves = pv.nLeaves;
+    float one = 1.0f;
+    if constexpr (HasAccumulate<E>::value) {
+        one = OpaqueOne();
+    }
+    uint64_t leaf[kBatch];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+        leaf[i] = reinterpret_cast<uint64_t>(args.src[first.ranks[i]]);
+    }
+    ScalarFence8(leaf);
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+        leaf[i] += pv.srcByteOff;
+    }
+    U32x4 raw0[kBatch];
+    U32x4 raw1[kBatch];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+        if (static_cast<uint32_t>(i) < nLeaves && on0) {
+            const S* p = reinterpret_cast<const S*>(leaf[i]) + e0;
+            raw0[i] = __builtin_nontemporal_load((const HCCL_AMD_GLOBAL U32x4Unaligned*)p);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+        if (static_cast<uint32_t>(i) < nLeaves && on1) {
+            const S* p = reinterpret_cast<const S*>(leaf[i]) + e1;
+            raw1[i] = __builtin_nontemporal_load((const HCCL_AMD_GLOBAL U32x4Unaligned*)p);
+        }
+    }
+    // (a flat program: leaf 0 starts the value, every other leaf is folded into it)
+    const auto fold = [&](U32x4* raw) {
+        IssueFence8(raw);
+        AccPack<E, W> acc;
+        PackOps<E, W>::Init(acc, __builtin_bit_cast(Pack<S, W>, raw[0]));
+#pragma unroll
+        for (int i = 1; i < kBatch; ++i) {
+            if (static_cast<uint32_t>(i) < nLeaves) {
+                PackOps<E, W>::Accumulate(acc, __builtin_bit_cast(Pack<S, W>, raw[i]), one);
+            }
+        }
+        return PackOps<E, W>::Narrow(acc);
+    };
+    // Both folds in front of the first store: whatever waits for the second tile's loads would otherwise also wait
+    // for the first tile's stores to be acknowledged (loads and stores leave one counter in issue order).
+    Pack<S, W> out0;
+    Pack<S, W> out1;
+    if (on0) {
+        out0 = fold(raw0);
+    }
+    if (on1) {
+        out1 = fold(raw1);
+    }
+    if (on0) {
+        StoreResult<S, W, true>(args, h, out0, dstOff + e0, ownOrFirst, 0, 1);
+    }
+    if (on1) {
+        StoreResult<S, W, true>(args, h, out1, dstOff + e1, ownOrFirst, 0, 1);
+    }
+}
+
 // Dynamic LDS: the accumulator stack, (plan depth - 1) * accumulator bytes * args.threads.
 // VB = leaves per batch of the 128-bit path: 8 keeps the register count low (more wavefronts in flight), 16 has
 // every load of up to sixteen ranks in flight at once; the launcher picks per launch.
-template <class E, int VB>
+// kPair: workgroups of 64 lanes take two adjacent tiles each (ReducePair) where the program has at most eight leaves.
+template <class E, int VB, bool kPair = false>
 __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
 {
+    static_assert(!kPair || VB == 8, "the pair form is built on the eight-leaf batch");
     using S = typename E::S;
     constexpr int W = 16 / sizeof(S);
     extern __shared__ uint32_t accStack[];
@@ -786,7 +864,7 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     }
     const uint64_t bodyEnd = head + nVec * W;
     const uint64_t nScalar = head + (len - bodyEnd);
-    if (h.storeWaves > 1) {
+    if (!kPair && h.storeWaves > 1) {
         // Stores split over the wavefronts of the workgroup (h.threads == 64 lanes fold, 64 * storeWaves run):
         // wavefront 0 folds the tile and parks the result in LDS, wavefront k writes it to destinations k,
         // k + storeWaves, ...  A wavefront that stores to many streams one after the other is what bounds the
@@ -823,9 +901,19 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
         }
         return;
     }
-    for (uint64_t u = first; u < nVec + lead; u += stride) {
-        if (u >= lead) {
-            ReduceOne<E, W, VB>(pv, accStack, args, h, head + (u - lead) * W, dstOff, firstDstAddr, preloaded);
+    if constexpr (kPair && sizeof(S) * W == 16) {
+        // (h.threads == 64, and the launcher's caller has checked that every program is flat and has at most eight leaves)
+        // workgroup blk takes tiles 2 blk and 2 blk + 1, then strides on by pairs
+        for (uint64_t u = first + static_cast<uint64_t>(blk) * 64; u < nVec + lead; u += 2 * stride) {
+            const bool on0 = u >= lead;
+            const bool on1 = u + 64 < nVec + lead;
+            ReducePair<E, W>(pv, accStack, args, h, head + (u - lead) * W, on0, on1, dstOff, firstDstAddr, firstBatch);
+        }
+    } else {
+        for (uint64_t u = first; u < nVec + lead; u += stride) {
+            if (u >= lead) {
+                ReduceOne<E, W, VB>(pv, accStack, args, h, head + (u - lead) * W, dstOff, firstDstAddr, preloaded);
+            }
         }
     }
     for (uint64_t i = first; i < nScalar; i += stride) {
@@ -849,7 +937,9 @@ detail::ReduceKernelFn SelectReduceBf16(int op, int batch);
 detail::ReduceKernelFn SelectReduceF32(int op, int batch);
 detail::ReduceKernelFn SelectReduceF64(int op, int batch);
 
-#define HCCL_AMD_PICK(T, batch) ((batch) == 8 ? detail::ReduceKernel<T, 8> : detail::ReduceKernel<T, 16>)
+#define HCCL_AMD_PICK(T, batch)                                                                \
+    ((batch) == 8 ? detail::ReduceKernel<T, 8>                                                 \
+                  : (batch) == 16 ? detail::ReduceKernel<T, 16> : detail::ReduceKernel<T, 8, true>)
 
 #define HCCL_AMD_DEFINE_SELECT4(NAME, SUM_T, PROD_T, MAX_T, MIN_T)                 \
     detail::ReduceKernelFn NAME(int op, int batch)                                \

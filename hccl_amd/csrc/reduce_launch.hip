@@ -8,7 +8,8 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
 {
     detail::ReduceKernelFn fn = nullptr;
     const int o = static_cast<int>(op);
-    const int batch = args.vecBatch == 8 ? 8 : 16;
+    const bool pair = args.vecBatch == kVecBatchPair;
+    const int batch = pair ? 0 : (args.vecBatch == 8 ? 8 : 16);
     switch (dtype) {
         case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8(o, batch); break;
         case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16(o, batch); break;
@@ -22,6 +23,9 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
         default: break;
     }
     if (fn == nullptr || nBlocks == 0 || (args.threads != 64 && args.threads != 128 && args.threads != 256)) {
+        return hipErrorInvalidValue;
+    }
+    if (pair && (args.threads != 64 || args.storeWaves > 1 || args.varGroups != 0)) {
         return hipErrorInvalidValue;
     }
     uint32_t threads = args.threads;

@@ -428,6 +428,43 @@ def test_all_reduce_with_the_stores_of_a_tile_shared_by_wavefronts(monkeypatch, 
         w.close()
 
 
+@pytest.mark.parametrize("n,blocks", [(2, 0), (3, 24), (5, 0), (8, 0), (8, 7)])
+def test_all_reduce_and_reduce_scatter_with_two_tiles_per_wavefront(monkeypatch, n, blocks):
+    """The form for launches of about one generation of wavefronts (a wavefront takes two adjacent tiles and issues
+    the loads of both before it folds either), forced for every size: even and odd numbers of tiles, less than one
+    tile, heads and tails off the 16-byte grid, every element type; with a small grid every workgroup strides over
+    pairs.  Orders whose programs nest keep the one-tile kernel."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_PAIR", "1")
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "0")
+    if blocks:
+        monkeypatch.setenv("HCCL_AMD_REDUCE_BLOCKS", str(blocks))
+    w = World(n)
+    monkeypatch.delenv("HCCL_AMD_REDUCE_PAIR")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS")
+    if blocks:
+        monkeypatch.delenv("HCCL_AMD_REDUCE_BLOCKS")
+    try:
+        seed = 6100 + 10 * n + blocks
+        for dtype in REDUCE_TYPES:
+            run_all_reduce(w, dtype, SUM, 20_011, "mesh", seed=seed)
+            seed += 1
+        for count in (1, 255, 256, 257, 511, 512, 513, 768, 4096 * 3, 4096 * 4 + 1, 100_003):
+            run_all_reduce(w, DT.FP32, SUM, count, "ring", seed=seed)            # 256 fp32 = one tile
+            seed += 1
+        run_all_reduce(w, DT.FP16, MAX, 33_333, "mesh", seed=seed, pad=2)        # unaligned: head and tail elements
+        run_all_reduce(w, DT.BFP16, SUM, 50_003, "mesh", seed=seed + 1, pad=lambda r, which: 2 * r + (6 if which == "recv" else 0))
+        run_all_reduce(w, DT.INT8, MIN, 9, "mesh", seed=seed + 2)                # less than one vector
+        run_all_reduce(w, DT.INT32, PROD, 4_099, "mesh", seed=seed + 3, in_place=True)
+        run_all_reduce(w, DT.FP64, SUM, 12_345, "mesh", seed=seed + 4, pad=lambda r, which: r + (3 if which == "recv" else 0))
+        run_all_reduce(w, DT.FP32, SUM, 70_001, "nhr", seed=seed + 5)            # nested program: form not taken
+        run_all_reduce(w, DT.FP32, SUM, 70_001, "mesh_symmetric", seed=seed + 6)
+        run_reduce_scatter(w, DT.FP32, SUM, 5_001, "mesh", seed=seed + 7)        # one result stream, own rank first
+        run_reduce_scatter(w, DT.BFP16, SUM, 10_007, "mesh", seed=seed + 8)
+        run_reduce_scatter(w, DT.INT16, MAX, 513, "aiv_mesh", seed=seed + 9)
+    finally:
+        w.close()
+
+
 def test_two_kernel_all_reduce_can_be_captured_into_a_graph(monkeypatch):
     """Once its fold program is on the device (one eager call of the same kind) the fold + fan-out AllReduce is
     kernel launches only."""

@@ -54,8 +54,9 @@ def kernels(tmp_path_factory):
 
 def test_every_translation_unit_is_there(kernels):
     reduce_kernels = [k for k in kernels if "ReduceKernel" in k["name"]]
-    # 34 combinations of element type and operation, each with the eight-leaf and the sixteen-leaf load batch
-    assert len(reduce_kernels) == 68, sorted(k["name"] for k in reduce_kernels)
+    # 34 combinations of element type and operation, each with the eight-leaf and the sixteen-leaf load batch and
+    # with the eight-leaf batch over two tiles per wavefront
+    assert len(reduce_kernels) == 102, sorted(k["name"] for k in reduce_kernels)
     assert len(kernels) - len(reduce_kernels) == 22            # the copy, fan-out (two load flavours) and AlltoAllV kernels
 
 
