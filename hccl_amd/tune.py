@@ -2,6 +2,7 @@
 
     python -m hccl_amd.tune [--quick]
     python -m hccl_amd.tune --all-gather 16:1,2 8:2,4,6 --broadcast 9:16,24,32     (ranks:MiB per rank,... per table)
+    python -m hccl_amd.tune --all-reduce-small 8:2048,4096                          (ranks:KiB per rank,...)
 
 For every shape of a small grid the forms the policy chooses between are run on the same buffers, interleaved
 (worlds created with the overriding environment variable set), and the table shows each form's fraction of the 8 TB/s
@@ -99,6 +100,41 @@ def all_reduce_rows(torch, h, ranks, mibs, rounds):
     return rows
 
 
+def all_reduce_small_rows(torch, h, ranks, kibs, rounds):
+    print("# AllReduce fp32 SUM in rank order, a few MiB per rank: one tile per wavefront, two, the library's own choice "
+          "(collectives issued with their arguments converted once)")
+    rows = []
+    for n in ranks:
+        for kib in kibs:
+            count = (kib << 10) // 4
+            per_set = 2 * n * count * 4
+            sets = max(1, min(12, -(-(600 << 20) // per_set)))
+            sends = [[torch.randn(count, device="cuda") for _ in range(n)] for _ in range(sets)]
+            recvs = [[torch.empty(count, device="cuda") for _ in range(n)] for _ in range(sets)]
+            torch.cuda.synchronize()
+
+            def make_step(stream):
+                comms = h.comm_init_all(n)
+                groups = [h.prepared_group([("HcclAllReduce", (sends[k][r], recvs[k][r], count, h.HcclDataType.FP32,
+                                                               h.HcclReduceOp.SUM, comms[r], stream))
+                                            for r in range(n)]) for k in range(sets)]
+                turn = [0]
+
+                def step():
+                    k = turn[0]
+                    turn[0] = (k + 1) % sets
+                    groups[k]()
+                return comms, step
+
+            forms = [("one", {"HCCL_AMD_REDUCE_PAIR": "0"}), ("pair", {"HCCL_AMD_REDUCE_PAIR": "1"}), ("auto", {})]
+            fracs = _forms(torch, h, make_step, forms, per_set, rounds, 200)
+            us = "/".join("%.1f" % (per_set / (v * HBM_PEAK) * 1e6) for v in fracs.values())
+            rows.append(_row("%2d ranks x %5d KiB  %s us" % (n, kib, us), fracs))
+            del sends, recvs
+            torch.cuda.empty_cache()
+    return rows
+
+
 COPY_FORMS = [("one", {"HCCL_AMD_COPY_TWO_KERNELS": "0"}), ("two", {"HCCL_AMD_COPY_TWO_KERNELS": "1"}), ("auto", {})]
 
 
@@ -171,6 +207,7 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--quick", action="store_true", help="a third of the grid, one round")
     ap.add_argument("--all-reduce", nargs="*", metavar="RANKS:MIB,..", help="AllReduce rows of these shapes only")
+    ap.add_argument("--all-reduce-small", nargs="*", metavar="RANKS:KIB,..", help="small AllReduce rows of these shapes only")
     ap.add_argument("--all-gather", nargs="*", metavar="RANKS:MIB,..", help="AllGather rows of these shapes only")
     ap.add_argument("--broadcast", nargs="*", metavar="RANKS:MIB,..", help="Broadcast rows of these shapes only")
     args = ap.parse_args()
@@ -181,7 +218,8 @@ def main():
     torch.cuda.set_device(0)
     h.lib()
     rounds = 1 if args.quick else 3
-    chosen = [(args.all_reduce, all_reduce_rows), (args.all_gather, all_gather_rows), (args.broadcast, broadcast_rows)]
+    chosen = [(args.all_reduce, all_reduce_rows), (args.all_reduce_small, all_reduce_small_rows),
+              (args.all_gather, all_gather_rows), (args.broadcast, broadcast_rows)]
     if any(specs is not None for specs, _ in chosen):
         for specs, rows in chosen:
             for spec in specs or []:
@@ -190,6 +228,7 @@ def main():
         return
     all_reduce_rows(torch, h, [3, 4, 6, 8, 16] if not args.quick else [4, 8], [16, 64, 256] if not args.quick else [64],
                     rounds)
+    all_reduce_small_rows(torch, h, [2, 8] if not args.quick else [8], [2048, 4096, 8192] if not args.quick else [4096], rounds)
     all_gather_rows(torch, h, [4, 6, 8, 16] if not args.quick else [8], [8, 64] if not args.quick else [64], rounds)
     broadcast_rows(torch, h, [6, 8, 16] if not args.quick else [8], [16, 64] if not args.quick else [64], rounds)
 

@@ -34,6 +34,14 @@ def test_all_reduce_form(ranks, mib):
     assert behind_best(tune.all_reduce_rows(torch, hccl_amd, [ranks], [mib], 2)) == []
 
 
+@pytest.mark.parametrize("ranks,kib", [(8, 4096), (8, 16384), (2, 4096)])
+def test_small_all_reduce_form(ranks, kib):
+    import torch
+    import hccl_amd
+    from hccl_amd import tune
+    assert behind_best(tune.all_reduce_small_rows(torch, hccl_amd, [ranks], [kib], 2)) == []
+
+
 @pytest.mark.parametrize("ranks,mib", [(4, 64), (16, 8)])
 def test_all_gather_form(ranks, mib):
     import torch
