@@ -465,6 +465,35 @@ def test_all_reduce_and_reduce_scatter_with_two_tiles_per_wavefront(monkeypatch,
         w.close()
 
 
+def test_prepared_group_issues_the_same_collective():
+    """hccl_amd.prepared_group converts the arguments of a group's calls once; what it runs is the plain sequence
+    HcclGroupStart, the entry points, HcclGroupEnd, and a bad argument still raises with the entry point's code."""
+    n, count = 4, 10_007
+    w = World(n)
+    try:
+        rng = np.random.default_rng(808)
+        host = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]
+        want = [np.zeros(count, dtype=np.float32) for _ in range(n)]
+        assert oracle.all_reduce(host, want, count, int(DT.FP32), SUM, algo="mesh") == 0
+        ins = [to_dev(x) for x in host]
+        w.set_algo(OpKind.ALL_REDUCE, "mesh")
+        w.inputs_ready()
+        for _ in range(3):
+            outs = [dev_zeros(count * 4) for _ in range(n)]
+            w.inputs_ready()
+            run = hccl_amd.prepared_group([("HcclAllReduce", (ins[r], outs[r], count, DT.FP32, SUM, w.comms[r], w.stream))
+                                           for r in range(n)])
+            run()
+            w.sync()
+            for r in range(n):
+                assert np.array_equal(to_host(outs[r], np.uint32), want[r].view(np.uint32)), r
+        bad = hccl_amd.prepared_group([("HcclAllReduce", (ins[0], None, count, DT.FP32, SUM, w.comms[0], w.stream))])
+        with pytest.raises(hccl_amd.HcclError):
+            bad()
+    finally:
+        w.close()
+
+
 def test_two_kernel_all_reduce_can_be_captured_into_a_graph(monkeypatch):
     """Once its fold program is on the device (one eager call of the same kind) the fold + fan-out AllReduce is
     kernel launches only."""
