@@ -537,7 +537,7 @@ def main():
             names += [n for n in EXTRA if n != args.workload]
         for name in names:
             # the tiny configuration needs many steps for a stable figure, the large ones few
-            steps = max(args.steps, 60) if name == "c1" else max(3, args.steps // 2)
+            steps = max(args.steps, 200) if name == "c1" else max(3, args.steps // 2)
             others[name] = measure(torch, wl, name, None, steps, 3)
     del wl
     torch.cuda.empty_cache()
