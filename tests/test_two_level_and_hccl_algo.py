@@ -261,6 +261,41 @@ def test_hccl_algo_strings_the_reference_rejects(config):
     assert e.value.code == 1
 
 
+def st_strings():
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_st_hccl_algo_strings.json")
+    return [e["config"] for e in json.load(open(path))]
+
+
+@pytest.mark.parametrize("config", st_strings())
+def test_every_hccl_algo_string_of_the_reference_system_tests_parses(config):
+    """The configurations the reference's own system tests run with (test/st/algorithm/testcase/*.cc, collected as
+    data by tests/golden/make_reference_st_hccl_algo_strings.py) are valid for its parser; they are for this one, and
+    their normal form names the same operator, executor and templates."""
+    text, _, _ = hccl_amd.select_from_hccl_algo(config, OpKind.ALL_REDUCE)
+    strip = lambda t: t.replace("level0=", "").replace("level1=", "").replace("level2=", "").replace("_", "")
+    assert text == strip(config)
+
+
+def test_what_the_system_tests_two_level_strings_select():
+    sel = hccl_amd.select_from_hccl_algo
+    AR, RS, RD = OpKind.ALL_REDUCE, OpKind.REDUCE_SCATTER, OpKind.REDUCE
+    # all_reduce_testcase.cc:317-345, all_reduce_dpu_testcase.cc: level-0 mesh inside a server, RHD / NHR between them
+    assert sel("allreduce:sequence{level0=meshconcur,level1=rhd}", AR)[1:] == (Algo.RHD, True)
+    assert sel("allreduce:sequence{mesh,nhr}", AR)[1:] == (Algo.NHR, True)
+    # three levels, pipelines and parallel executors are orders this library does not build: nothing is selected
+    assert sel("allreduce:sequence{meshconcur,nhr,mesh}", AR)[1] is None
+    assert sel("allreduce:pipeline{mesh,nhr,nhr}", AR)[1] is None
+    assert sel("reducescatter:parallel{level0=mesh,level1=hd}", RS)[1] is None
+    assert sel("reduce:parallel{nhr,nhr}", RD)[1] is None
+    # one level
+    assert sel("reducescatter:sole{level0=hdaicpureduce}", RS)[1] == Algo.RHD
+    assert sel("reduce:sole{meshtwoshot}", RD)[1] == Algo.MESH_TWO_SHOT
+    assert sel("reduce:sole{mesh}", RD)[1] == Algo.MESH
+    assert sel("reducescatter:sole{level0=not(nhr)}", RS)[1] is None
+
+
 def test_what_hccl_algo_selects():
     sel = hccl_amd.select_from_hccl_algo
     AR, RS, RD = OpKind.ALL_REDUCE, OpKind.REDUCE_SCATTER, OpKind.REDUCE
