@@ -310,7 +310,7 @@ def get_stuck_counters(hccl_comm):
 
 def fold_programs(op_kind, algo, rank_size, level0=1):
     """Host-only: the byte programs (one per segment) that fix the reduction order; level0 > 1: the two-level
-    AllReduce over groups of level0 consecutive ranks with `algo` between the groups."""
+    AllReduce or ReduceScatter over groups of level0 consecutive ranks with `algo` between the groups."""
     L = lib()
     out = []
     seg, count = 0, 1

@@ -399,14 +399,20 @@ AlgoSelection SelectFromHcclAlgo(const std::vector<AlgoSegment>& segments)
                 if (!OrderOf(kind, seg.templates[0].name, &algo)) {
                     continue;
                 }
-            } else if (seg.templates.size() == 2 && kind == HCCL_AMD_OP_ALL_REDUCE &&
-                       IsMeshFamily(seg.templates[0].name)) {
-                // a mesh inside the level-0 groups, the second template between them
-                if (!OrderOf(kind, seg.templates[1].name, &algo) || algo == HCCL_AMD_ALGO_MESH_CHUNK) {
+            } else if (seg.templates.size() == 2 && seg.executor == "sequence" &&
+                       (kind == HCCL_AMD_OP_ALL_REDUCE || kind == HCCL_AMD_OP_REDUCE_SCATTER) &&
+                       IsMeshFamily(seg.templates[0].name) && seg.templates[0].name.compare(0, 9, "meshchunk") != 0) {
+                // a mesh inside the level-0 groups (the mesh-chunk templates fold in another order there, which is
+                // not built), the second template between them
+                if (!OrderOf(kind, seg.templates[1].name, &algo) ||
+                    (algo != HCCL_AMD_ALGO_RHD && algo != HCCL_AMD_ALGO_NHR && algo != HCCL_AMD_ALGO_MESH &&
+                     algo != HCCL_AMD_ALGO_RING)) {
                     continue;
                 }
                 if (seg.templates[1].name == "nhraicpureduce") {
                     algo = HCCL_AMD_ALGO_MESH;   // between the groups: the own-first fold of the host-reduce template
+                } else if (algo == HCCL_AMD_ALGO_MESH || algo == HCCL_AMD_ALGO_RING) {
+                    continue;                    // a mesh between the groups: another executor family
                 }
                 twoLevel = true;
             } else {

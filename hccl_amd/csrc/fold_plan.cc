@@ -351,39 +351,78 @@ HcclResult Rhd(uint32_t p, FoldPlan* plan) { return EmitAll(RhdValues(p, RankLea
 // ins_temp_reduce_scatter_mesh_1D.cc:203-237; the level-0 template ..._Z_axis_detour derives from it).
 // Level 1: RHD with POST skipped and the merged share bridged (:700-741), NHR (:784-789), or for the types the
 // host reduces the own-first fold of ins_temp_reduce_scatter_aicpu_reduce_nhr.cc:214-250 (`MESH`).
+// The level-1 template's values for the units of level-0 member i: unit j is what the boxes end with for the share
+// of box j, participant b standing for what box b has folded for that unit.
+HcclResult TwoLevelUnits(uint32_t l0, uint32_t l1, HcclAmdAlgo level1, uint32_t i, std::vector<ExprPtr>* units)
+{
+    const LeafFn box = [&](uint32_t b) {
+        std::vector<uint32_t> order{b * l0 + i};
+        for (uint32_t t = 0; t < l0; ++t) {
+            if (t != i) {
+                order.push_back(b * l0 + t);
+            }
+        }
+        return Chain(order);
+    };
+    units->clear();
+    if (level1 == HCCL_AMD_ALGO_RHD) {
+        *units = RhdValues(l1, box);
+    } else if (level1 == HCCL_AMD_ALGO_NHR) {
+        *units = NhrValues(l1, box);
+    } else if (level1 == HCCL_AMD_ALGO_MESH) {
+        for (uint32_t j = 0; j < l1; ++j) {
+            ExprPtr e = box(j);
+            for (uint32_t b = 0; b < l1; ++b) {
+                if (b != j) {
+                    e = Fold(e, box(b));
+                }
+            }
+            units->push_back(e);
+        }
+    } else {
+        return HCCL_E_NOT_SUPPORT;
+    }
+    return HCCL_SUCCESS;
+}
+
 HcclResult TwoLevelAllReduce(uint32_t n, uint32_t l0, HcclAmdAlgo level1, FoldPlan* plan)
 {
     const uint32_t l1 = n / l0;
     plan->segmentsAreSubs = true;
     for (uint32_t i = 0; i < l0; ++i) {
-        const LeafFn box = [&](uint32_t b) {
-            std::vector<uint32_t> order{b * l0 + i};
-            for (uint32_t t = 0; t < l0; ++t) {
-                if (t != i) {
-                    order.push_back(b * l0 + t);
-                }
-            }
-            return Chain(order);
-        };
         std::vector<ExprPtr> units;
-        if (level1 == HCCL_AMD_ALGO_RHD) {
-            units = RhdValues(l1, box);
-        } else if (level1 == HCCL_AMD_ALGO_NHR) {
-            units = NhrValues(l1, box);
-        } else if (level1 == HCCL_AMD_ALGO_MESH) {
-            for (uint32_t j = 0; j < l1; ++j) {
-                ExprPtr e = box(j);
-                for (uint32_t b = 0; b < l1; ++b) {
-                    if (b != j) {
-                        e = Fold(e, box(b));
-                    }
-                }
-                units.push_back(e);
-            }
-        } else {
-            return HCCL_E_NOT_SUPPORT;
+        HcclResult rc = TwoLevelUnits(l0, l1, level1, i, &units);
+        if (rc == HCCL_SUCCESS) {
+            rc = EmitAll(units, plan);
         }
-        HcclResult rc = EmitAll(units, plan);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// ReduceScatter over the same boxes (reference ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-372, 388-500):
+// step 1 is the mesh ReduceScatter inside the box once per box of the world (in repeat q member i folds slice
+// q * l0 + i of its box, its own input first), step 2 the level-1 ReduceScatter between the members i, whose unit q
+// is that slice; box j ends with unit j, the output of rank j * l0 + i.  Program r is therefore the level-1
+// template's value for unit r / l0 among the members r % l0: the tree of sub-slice r / l0 of chunk r % l0 of the
+// two-level AllReduce.  Level 1: RHD (reduce_scatter_rhd with its POST, which moves shares and folds nothing),
+// NHR, or the own-first fold of reduce_scatter_aicpu_reduce_nhr_pcie.cc:212-280 (`MESH`).  A loop covers the same
+// range of every slice, so loop boundaries do not show in the result.
+HcclResult TwoLevelReduceScatter(uint32_t n, uint32_t l0, HcclAmdAlgo level1, FoldPlan* plan)
+{
+    const uint32_t l1 = n / l0;
+    plan->segmentsAreSubs = false;
+    std::vector<std::vector<ExprPtr>> units(l0);
+    for (uint32_t i = 0; i < l0; ++i) {
+        HcclResult rc = TwoLevelUnits(l0, l1, level1, i, &units[i]);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    for (uint32_t r = 0; r < n; ++r) {
+        HcclResult rc = Emit(units[r % l0][r / l0], plan);
         if (rc != HCCL_SUCCESS) {
             return rc;
         }
@@ -433,10 +472,13 @@ HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPla
         if (n % level0 != 0) {
             return HCCL_E_PARA;
         }
-        if (op != HCCL_AMD_OP_ALL_REDUCE) {
-            return HCCL_E_NOT_SUPPORT;
+        if (op == HCCL_AMD_OP_ALL_REDUCE) {
+            return TwoLevelAllReduce(n, level0, algo, plan);
         }
-        return TwoLevelAllReduce(n, level0, algo, plan);
+        if (op == HCCL_AMD_OP_REDUCE_SCATTER) {
+            return TwoLevelReduceScatter(n, level0, algo, plan);
+        }
+        return HCCL_E_NOT_SUPPORT;
     }
     if (op == HCCL_AMD_OP_REDUCE) {
         // One-shot: rank 0's slot is the base, the others fold ascending (reference reduce_mesh_1D.cc:268-300).

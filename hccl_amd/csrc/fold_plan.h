@@ -22,7 +22,8 @@ struct FoldPlan {
 // Returns HCCL_E_NOT_SUPPORT for combinations that do not exist (e.g. AIV_MESH AllReduce).
 // level0 in (1, rankSize): the two-level AllReduce of the reference's sequence executor over groups of level0
 // consecutive ranks, `algo` (RHD, NHR, or MESH for the host-reduce fold) being the template between the groups;
-// program i * (rankSize / level0) + j is sub-slice j of chunk i.  level0 of 1 or rankSize: one level.
+// program i * (rankSize / level0) + j is sub-slice j of chunk i; for ReduceScatter the two-level order of the same
+// executor family, program r being rank r's output.  level0 of 1 or rankSize: one level.
 HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, FoldPlan* plan, uint32_t level0 = 1);
 
 // Geometry helpers of the recursive halving-doubling family (reference template_utils.cc:42-168).

@@ -180,6 +180,7 @@ struct World {
     // HCCL_ALGO asked for a sequence executor (1), a single-level one (0), or said nothing (-1): with level-0
     // groups, AllReduce runs in two levels unless a single-level executor was asked for.
     int allReduceSequence = -1;
+    int reduceScatterSequence = -1;       // the same for ReduceScatter (reducescatter:sequence{mesh..., rhd | nhr | nhr_aicpu_reduce})
     bool envInvalid = false;      // an environment variable of the reference failed its parser
 
     ~World()

@@ -247,6 +247,8 @@ void ApplyReferenceAlgoEnv(World* w)
             w->algo[op] = sel.algo[op];
             if (kind == HCCL_AMD_OP_ALL_REDUCE) {
                 w->allReduceSequence = sel.twoLevel[op] ? 1 : 0;
+            } else if (kind == HCCL_AMD_OP_REDUCE_SCATTER) {
+                w->reduceScatterSequence = sel.twoLevel[op] ? 1 : 0;
             }
         }
     }

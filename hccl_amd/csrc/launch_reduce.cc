@@ -524,8 +524,18 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
     HcclAmdAlgo algo = EffectiveAlgo(w, HCCL_AMD_OP_REDUCE_SCATTER, p.dtype, p.op);
+    // A world with level-0 groups runs the step-driven orders in two levels, as AllReduce does (reference
+    // ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-372): the mesh ReduceScatter inside every group, the
+    // configured template between the groups, the own-first host-reduce fold there for the types the reference
+    // reduces on the host.  Every rank's output keeps one program, so the launch is the one-level one.
+    const uint32_t level0 = w->level0;
+    const HcclAmdAlgo configured = w->algo[HCCL_AMD_OP_REDUCE_SCATTER];
+    const bool stepDriven = configured == HCCL_AMD_ALGO_RHD || configured == HCCL_AMD_ALGO_NHR;
+    const bool twoLevel = level0 > 1 && level0 < n && w->reduceScatterSequence != 0 &&
+                          (algo == HCCL_AMD_ALGO_RHD || algo == HCCL_AMD_ALGO_NHR ||
+                           (algo == HCCL_AMD_ALGO_MESH && (stepDriven || w->reduceScatterSequence == 1)));
     DevicePlan plan;
-    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, algo, &plan);
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, algo, &plan, twoLevel ? level0 : 1);
     if (rc != HCCL_SUCCESS) {
         return rc;
     }

@@ -304,9 +304,10 @@ HcclResult HcclAmdGetStuckCounters(HcclComm comm, uint64_t* head, uint64_t* tail
  */
 HcclResult HcclAmdGetFoldProgram(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t segment,
                                  uint8_t* out, uint32_t cap, uint32_t* len, uint32_t* segmentCount);
-/* The same for the two-level AllReduce over groups of `level0` consecutive ranks (see HcclAmdSetLevel0RankSize):
- * segment i * (rankSize / level0) + j is sub-slice j of chunk i; algo is the template between the groups (RHD, NHR,
- * or MESH for the own-first fold of the host-reduce template).  level0 of 1 or rankSize: HcclAmdGetFoldProgram. */
+/* The same for the two-level orders over groups of `level0` consecutive ranks (see HcclAmdSetLevel0RankSize).
+ * AllReduce: segment i * (rankSize / level0) + j is sub-slice j of chunk i; ReduceScatter: segment r is rank r's
+ * output.  algo is the template between the groups (RHD, NHR, or MESH for the own-first fold of the host-reduce
+ * template).  level0 of 1 or rankSize: HcclAmdGetFoldProgram. */
 HcclResult HcclAmdGetFoldProgramTwoLevel(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t level0,
                                          uint32_t segment, uint8_t* out, uint32_t cap, uint32_t* len,
                                          uint32_t* segmentCount);
@@ -316,11 +317,13 @@ HcclResult HcclAmdGetFoldProgramTwoLevel(HcclAmdOpKind op, HcclAmdAlgo algo, uin
  * sequence: a mesh ReduceScatter inside every server, the configured template (RHD, NHR, or the host-reduce fold for
  * PROD and the 64-bit types) between the ranks that hold the same chunk, and the two AllGathers back
  * (src/ops/all_reduce/algorithm/executor/ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852, registered as
- * Aicpu AllReduce Sequence MeshConcur RHD / MeshConcur NHR / Mesh NHRAicpuReduce, :974-1023).  Where its topology
+ * Aicpu AllReduce Sequence MeshConcur RHD / MeshConcur NHR / Mesh NHRAicpuReduce, :974-1023), and ReduceScatter
+ * as the first two of those steps (src/ops/reduce_scatter/algorithm/executor/
+ * ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-500, registrations :567-640).  Where its topology
  * comes from a rank table, a loopback world is told: `ranksPerGroup` consecutive ranks form a group (it must
  * divide the rank size; 1, the default, and the rank size itself mean one level).  Also HCCL_AMD_LEVEL0_RANKS at
- * world creation.  With groups, AllReduce under RHD and NHR folds in the two-level order; the other orders and the
- * other operators are not affected.
+ * world creation.  With groups, AllReduce and ReduceScatter under RHD and NHR fold in the two-level order; the other
+ * orders and the other operators (ReduceScatterV included) are not affected.
  */
 HcclResult HcclAmdSetLevel0RankSize(HcclComm comm, uint32_t ranksPerGroup);
 HcclResult HcclAmdGetLevel0RankSize(HcclComm comm, uint32_t* ranksPerGroup);
@@ -331,7 +334,8 @@ HcclResult HcclAmdGetLevel0RankSize(HcclComm comm, uint32_t* ranksPerGroup);
  * AllReduce, ReduceScatter(V) and Reduce: sole{mesh | mesh_one_shot | mesh_two_shot} -> MESH (Reduce: mesh_two_shot ->
  * MESH_TWO_SHOT), sole{mesh_chunk...} -> MESH_CHUNK, sole{nhr...} -> NHR, sole{nhr_aicpu_reduce} -> the host-reduce
  * order (RING for AllReduce, MESH for ReduceScatter), sole{rhd | hd | hd_aicpu_reduce} -> RHD, strictordered{...} ->
- * ORDER_PRESERVED, sequence{<mesh...>, <template>} -> that template between level-0 groups (AllReduce).  Clauses are
+ * ORDER_PRESERVED, sequence{<mesh...>, <template>} -> that template between level-0 groups (AllReduce,
+ * ReduceScatter; a mesh-chunk template inside the groups is another order and selects nothing).  Clauses are
  * taken last to first, negations select nothing, clauses for the copy operators are accepted and ignored, and a
  * string the reference's parser rejects is ignored with a warning, as there.  HCCL_AMD_ALGO and HcclAmdSetAlgo
  * override it.  This call is the host-only view of that reading: HCCL_E_PARA for a rejected string; otherwise

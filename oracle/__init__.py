@@ -282,6 +282,13 @@ def all_reduce_two_level(ins, outs, count, dtype, op, level0, level1_algo, acc=A
                                           ctypes.c_uint64(max_count_per_loop))
 
 
+def reduce_scatter_two_level(ins, outs, recv_count, dtype, op, level0, level1_algo, acc=ACC_FP32):
+    """ReduceScatter over groups of `level0` consecutive ranks; level1_algo as for all_reduce_two_level."""
+    code = {"rhd": L1_RHD, "nhr": L1_NHR, "mesh": L1_MESH}[level1_algo]
+    return lib().orc_reduce_scatter_two_level(ctypes.c_uint32(len(ins)), ctypes.c_uint32(level0), code, _ptr_array(ins),
+                                              _ptr_array(outs), ctypes.c_uint64(recv_count), dtype, op, acc)
+
+
 def reduce_scatter(ins, outs, recv_count, dtype, op, acc=ACC_FP32, algo="mesh", max_count_per_loop=0):
     if algo == "mesh_chunk":
         return _reduce_call("orc_reduce_scatter_mesh_chunk", ins, outs, recv_count, dtype, op, acc,

@@ -1408,6 +1408,75 @@ static int level1_exchange(const red_t* r, uint32_t l0, uint32_t l1, int l1Algo,
     return rc;
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * Two-level ReduceScatter (ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-372, 388-500).  Boxes as
+ * above; the input of every rank holds n slices of recvCount elements, slice b * l0 + i belongs to member i
+ * of box b.  Per loop (a loop covers the same range of every slice, so the loops do not show in the result):
+ *   step 1  l1 repeats of the mesh ReduceScatter inside every box (:311-319, repeatNum = l1, input stride
+ *           l0 slices): in repeat q member i folds slice q * l0 + i of its box, its own input first
+ *   step 2  the level-1 ReduceScatter between the members i of all boxes (:338-353): unit q of member i is
+ *           what step 1 left for slice q * l0 + i; box j ends with unit j, which is rank j * l0 + i's output.
+ * Level 1 (registrations :567-640): ORC_L1_RHD (reduce_scatter_rhd with its POST), ORC_L1_NHR, and ORC_L1_MESH
+ * for the host-reduce template of PROD and the 64-bit types, own share first and the other boxes ascending
+ * (reduce_scatter_aicpu_reduce_nhr_pcie.cc:212-280).
+ * ------------------------------------------------------------------------------------------- */
+int orc_reduce_scatter_two_level(uint32_t n, uint32_t l0, int l1Algo, const void* const* in, void* const* out,
+                                 uint64_t recvCount, int dtype, int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (l0 == 0 || n % l0 != 0 || l1Algo < ORC_L1_RHD || l1Algo > ORC_L1_MESH) {
+        return ORC_E_PARA;
+    }
+    if (recvCount == 0) {
+        return ORC_OK;
+    }
+    uint32_t l1 = n / l0;
+    const uint8_t** src = (const uint8_t**)malloc(sizeof(uint8_t*) * n);
+    void* tmp = malloc(recvCount * r.asz);
+    scratch_t sc;
+    if (!src || !tmp || scratch_alloc(&sc, l1, recvCount, r.asz) != ORC_OK) {
+        free(src);
+        free(tmp);
+        return ORC_E_INTERNAL;
+    }
+    for (uint32_t j = 0; j < n; ++j) {
+        src[j] = cbytes(in[j]);
+    }
+    for (uint32_t i = 0; i < l0 && rc == ORC_OK; ++i) {
+        for (uint32_t b = 0; b < l1; ++b) {
+            for (uint32_t q = 0; q < l1; ++q) {
+                uint32_t at = l1Algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l1, q) : q;
+                level0_fold(&r, l0, b, i, src, (uint64_t)(q * l0 + i) * recvCount, recvCount, scratch_at(&sc, b, at), tmp);
+            }
+        }
+        if (l1Algo == ORC_L1_RHD) {
+            rc = rhd_rs_frame(&r, &sc, 0);
+        } else if (l1Algo == ORC_L1_NHR) {
+            rc = nhr_reduce_scatter_scratch(&r, &sc);
+        } else {
+            for (uint32_t j = 0; j < l1; ++j) {
+                for (uint32_t b = 0; b < l1; ++b) {
+                    if (b != j) {
+                        red_pair(&r, scratch_at(&sc, j, j), scratch_at(&sc, b, j), recvCount);
+                    }
+                }
+            }
+        }
+        for (uint32_t j = 0; j < l1 && rc == ORC_OK; ++j) {
+            uint32_t at = l1Algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l1, j) : j;
+            red_narrow(&r, scratch_at(&sc, j, at), out[j * l0 + i], recvCount);
+        }
+    }
+    free(sc.mem);
+    free(src);
+    free(tmp);
+    return rc;
+}
+
 int orc_all_reduce_two_level(uint32_t n, uint32_t l0, int l1Algo, const void* const* in, void* const* out,
                              uint64_t count, int dtype, int op, int accMode, uint64_t maxCountPerLoop)
 {

@@ -162,6 +162,10 @@ int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint
 #define ORC_L1_RHD 0
 #define ORC_L1_NHR 1
 #define ORC_L1_MESH 2
+/* Two-level ReduceScatter of the reference's sequence executor (ins_v2_reduce_scatter_sequence_executor_aicpu.cc):
+ * mesh ReduceScatter inside boxes of l0 consecutive ranks, then the level-1 template (ORC_L1_*) between the boxes. */
+int orc_reduce_scatter_two_level(uint32_t n, uint32_t l0, int l1Algo, const void* const* in, void* const* out,
+                                 uint64_t recvCount, int dtype, int op, int accMode);
 int orc_all_reduce_two_level(uint32_t n, uint32_t l0, int l1Algo, const void* const* in, void* const* out,
                              uint64_t count, int dtype, int op, int accMode, uint64_t maxCountPerLoop);
 

@@ -1,5 +1,5 @@
-"""CPU tier: the two-level AllReduce order (level-0 groups, reference
-ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852) and the reading of the reference's HCCL_ALGO setting.
+"""CPU tier: the two-level AllReduce and ReduceScatter orders (level-0 groups, reference
+ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852, ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-500) and the reading of the reference's HCCL_ALGO setting.
 
 The oracle's two-level function is pinned by what does not depend on it: with one rank per group it must be the
 (already pinned) one-level RHD / NHR oracle, with one group the own-first mesh order, integer sums must equal plain
@@ -198,13 +198,121 @@ def test_groups_must_divide_the_world():
         hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.RHD, 6, level0=4)
     assert e.value.code == 1
     with pytest.raises(hccl_amd.HcclError) as e:
-        hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.RHD, 6, level0=2)
+        hccl_amd.fold_programs(OpKind.REDUCE, Algo.MESH, 6, level0=2)
+    assert e.value.code == 5
+    with pytest.raises(hccl_amd.HcclError) as e:
+        hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.ORDER_PRESERVED, 6, level0=2)
     assert e.value.code == 5
     # one rank per group, or all ranks in one: the one-level programs
     assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.RHD, 6, level0=1) == hccl_amd.fold_programs(
         OpKind.ALL_REDUCE, Algo.RHD, 6)
     assert hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.NHR, 6, level0=6) == hccl_amd.fold_programs(
         OpKind.ALL_REDUCE, Algo.NHR, 6)
+
+
+# ---- two-level ReduceScatter (reference ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-500) ---------------
+@pytest.mark.parametrize("p", [2, 3, 5, 6, 7, 8, 12])
+def test_reduce_scatter_with_one_rank_per_group_is_the_one_level_order(orc, p):
+    rng = np.random.default_rng(41 * p)
+    for c in (7, 1):
+        for op, gen in ((SUM, wide), (MAX, tricky)):
+            ins = gen(rng, p, p * c)
+            for algo in ("rhd", "nhr"):
+                want = [np.zeros(c, np.float32) for _ in range(p)]
+                got = [np.zeros(c, np.float32) for _ in range(p)]
+                assert orc.reduce_scatter(ins, want, c, F32, op, algo=algo) == 0
+                assert orc.reduce_scatter_two_level(ins, got, c, F32, op, 1, algo) == 0
+                for r in range(p):
+                    assert same(got[r], want[r]), (p, c, op, algo, r)
+
+
+@pytest.mark.parametrize("n", [2, 3, 4, 8])
+def test_reduce_scatter_with_one_group_is_the_own_first_mesh_order(orc, n):
+    rng = np.random.default_rng(19 * n)
+    c = 9
+    for op, gen in ((SUM, wide), (MIN, tricky)):
+        ins = gen(rng, n, n * c)
+        want = [np.zeros(c, np.float32) for _ in range(n)]
+        assert orc.reduce_scatter(ins, want, c, F32, op, algo="mesh") == 0
+        for level1 in ("nhr", "mesh", "rhd"):
+            got = [np.zeros(c, np.float32) for _ in range(n)]
+            assert orc.reduce_scatter_two_level(ins, got, c, F32, op, n, level1) == 0
+            for r in range(n):
+                assert same(got[r], want[r]), (n, op, level1, r)
+
+
+@pytest.mark.parametrize("l0,l1", SHAPES)
+def test_reduce_scatter_counts_every_rank_exactly_once(orc, l0, l1):
+    n = l0 * l1
+    rng = np.random.default_rng(7 * n + l0)
+    for c in (5, 1):
+        ins = [rng.integers(-2 ** 31, 2 ** 31, n * c, dtype=np.int64).astype(np.int32) for _ in range(n)]
+        want = np.zeros(n * c, dtype=np.int64)
+        for x in ins:
+            want += x
+        want = want.astype(np.int32)   # wraps
+        for level1 in ("rhd", "nhr", "mesh"):
+            got = [np.zeros(c, np.int32) for _ in range(n)]
+            assert orc.reduce_scatter_two_level(ins, got, c, I32, SUM, l0, level1) == 0
+            for r in range(n):
+                assert np.array_equal(got[r], want[r * c:(r + 1) * c]), (l0, l1, c, level1, r)
+
+
+def test_two_level_reduce_scatter_by_hand(orc):
+    """The trees of test_two_groups_of_three_and_three_groups_of_two_by_hand, slice by slice: rank j * l0 + i receives
+    slice j * l0 + i, folded inside every group with member i's input first and between the groups by the level-1
+    template's tree for unit j."""
+    rng = np.random.default_rng(98)
+    c = 6
+    for op, gen in ((SUM, wide), (MAX, tricky), (MIN, tricky)):
+        l0, l1 = 2, 3
+        ins = gen(rng, 6, 6 * c)
+        got = [np.zeros(c, np.float32) for _ in range(6)]
+        assert orc.reduce_scatter_two_level(ins, got, c, F32, op, l0, "rhd") == 0
+        for r in range(6):
+            j, i = divmod(r, l0)
+            b = [box(ins, l0, g, i, r * c, (r + 1) * c, op) for g in range(l1)]
+            pair = f32_fold(b[1], b[0], op)
+            want = f32_fold(b[2], pair, op) if j < 2 else f32_fold(pair, b[2], op)
+            assert same(got[r], want), ("rhd", op, r)
+        l0, l1 = 3, 2
+        got = [np.zeros(c, np.float32) for _ in range(6)]
+        assert orc.reduce_scatter_two_level(ins, got, c, F32, op, l0, "nhr") == 0
+        for r in range(6):
+            j, i = divmod(r, l0)
+            b = [box(ins, l0, g, i, r * c, (r + 1) * c, op) for g in range(l1)]
+            assert same(got[r], f32_fold(b[1 - j], b[j], op)), ("nhr", op, r)
+        l0, l1 = 2, 3
+        got = [np.zeros(c, np.float32) for _ in range(6)]
+        assert orc.reduce_scatter_two_level(ins, got, c, F32, op, l0, "mesh") == 0
+        for r in range(6):
+            j, i = divmod(r, l0)
+            acc = box(ins, l0, j, i, r * c, (r + 1) * c, op)
+            for g in range(3):
+                if g != j:
+                    acc = f32_fold(box(ins, l0, g, i, r * c, (r + 1) * c, op), acc, op)
+            assert same(got[r], acc), ("mesh", op, r)
+
+
+@pytest.mark.parametrize("l0,l1", SHAPES)
+@pytest.mark.parametrize("level1", ["rhd", "nhr", "mesh"])
+def test_two_level_reduce_scatter_programs_match_oracle(orc, l0, l1, level1):
+    n = l0 * l1
+    progs = hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, L1[level1], n, level0=l0)
+    assert len(progs) == n
+    all_reduce = hccl_amd.fold_programs(OpKind.ALL_REDUCE, L1[level1], n, level0=l0)
+    for r, prog in enumerate(progs):
+        assert sorted(program_ranks(prog)) == list(range(n)) and len(prog) <= 320
+        assert prog == all_reduce[(r % l0) * l1 + r // l0]      # sub-slice r / l0 of chunk r % l0 of the AllReduce
+    for c in (3, 1):
+        for op, gen in ((SUM, wide), (MAX, tricky)):
+            rng = np.random.default_rng(2000 * n + 10 * l0 + op)
+            ins = gen(rng, n, n * c)
+            outs = [np.zeros(c, np.float32) for _ in range(n)]
+            assert orc.reduce_scatter_two_level(ins, outs, c, F32, op, l0, level1) == 0
+            for r in range(n):
+                got = run_program(progs[r], lambda k: ins[k][r * c:(r + 1) * c], op)
+                assert same(got, outs[r]), (l0, l1, level1, c, op, r)
 
 
 # ---- HCCL_ALGO ---------------------------------------------------------------------------------------
@@ -324,3 +432,11 @@ def test_what_hccl_algo_selects():
     assert sel("allreduce:sole{not(nhr)}", AR)[1] is None
     assert sel("allgather:sole{mesh};alltoall:pairwise", AR)[1] is None
     assert sel("allreduce:sequence{mesh,nhr,nhr}", AR)[1] is None              # three levels are not built
+    # ReduceScatter in two levels: the same executor family (ins_v2_reduce_scatter_sequence_executor_aicpu.cc:567-640)
+    assert sel("reducescatter:sequence{level0=meshconcur,level1=rhd}", RS)[1:] == (Algo.RHD, True)
+    assert sel("reducescatter:sequence{mesh_concur,nhr}", RS)[1:] == (Algo.NHR, True)
+    assert sel("reducescatter:sequence{mesh,nhr_aicpu_reduce}", RS)[1:] == (Algo.MESH, True)
+    assert sel("reducescatter:sequence{level0=meshchunkconcur,level1=nhr}", RS)[1] is None   # mesh chunk inside the groups
+    assert sel("reducescatter:sequence{mesh,mesh}", RS)[1] is None
+    assert sel("allreduce:parallel{mesh,nhr}", AR)[1] is None                  # another executor, another order
+    assert sel("allreduce:pipeline{mesh,nhr}", AR)[1] is None

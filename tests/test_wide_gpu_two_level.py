@@ -1,5 +1,6 @@
-"""GPU parity of the two-level AllReduce (level-0 groups of consecutive ranks, the configured template between the
-groups; reference ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852) against the CPU oracle, through the C ABI:
+"""GPU parity of the two-level AllReduce and ReduceScatter (level-0 groups of consecutive ranks, the configured
+template between the groups; reference ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852,
+ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-500) against the CPU oracle, through the C ABI:
 bit-exact for fp32 / integers / MAX, fp16 and bf16 SUM against the oracle's fp32-accumulate mode.  Also the reading
 of HCCL_ALGO at world creation."""
 import os
@@ -70,6 +71,56 @@ def test_two_level_all_reduce_matches_the_oracle(l0, l1):
         w.all_reduce([to_dev(x) for x in ins], recvs, 1234, DT.FP32, SUM, "mesh")
         check(DT.FP32, SUM, to_host(recvs[0], np.float32), want[0], "mesh with groups")
     finally:
+        w.close()
+
+
+def run_rs(world, l0, algo, dtype, op, c, seed, pad=0):
+    n = world.n
+    rng = np.random.default_rng(seed)
+    ins = [gen(dtype, op, rng, n * c) for _ in range(n)]
+    want = [np.zeros(c, dtype=NP[dtype]) for _ in range(n)]
+    assert oracle.reduce_scatter_two_level(ins, want, c, int(dtype), op, l0, level1_of(algo, dtype, op),
+                                           acc=oracle.ACC_FP32) == 0
+    sends = [to_dev(x, (pad * (r + 1)) % 16 if pad else 0) for r, x in enumerate(ins)]
+    recvs = [dev_zeros(x.nbytes, pad) for x in want]
+    world.reduce_scatter(sends, recvs, c, dtype, op, algo)
+    for r in range(n):
+        check(dtype, op, to_host(recvs[r], NP[dtype]), want[r],
+              "two-level reduce_scatter %s %s %dx%d count=%d algo=%s rank=%d" % (dtype.name, op, l0, n // l0, c, algo, r))
+
+
+@pytest.mark.parametrize("l0,l1", [(2, 3), (2, 4), (4, 2), (3, 2), (2, 6), (8, 8), (4, 4)])
+def test_two_level_reduce_scatter_matches_the_oracle(l0, l1):
+    """The reference's two-level ReduceScatter (ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-500): mesh inside
+    the groups, RHD / NHR / the host-reduce fold between them; loops cover the same range of every slice and do not
+    show, so a bounded staging buffer changes nothing."""
+    n = l0 * l1
+    w = World(n)
+    try:
+        hccl_amd.set_level0_rank_size(w.comms[0], l0)
+        seed = 300 * l0 + l1
+        for algo in ("rhd", "nhr"):
+            for c in (1, 7, 256, 4093, 20011):
+                run_rs(w, l0, algo, DT.FP32, SUM, c, seed + c)
+            run_rs(w, l0, algo, DT.FP32, MAX, 3 * n + 1, seed + 1)
+            run_rs(w, l0, algo, DT.FP16, SUM, 4093, seed + 2, pad=2)
+            run_rs(w, l0, algo, DT.BFP16, SUM, 5000, seed + 3)
+            run_rs(w, l0, algo, DT.INT8, MIN, 7001, seed + 4, pad=1)
+            run_rs(w, l0, algo, DT.INT32, PROD, 1021, seed + 5)        # host-reduce fold between the groups
+            run_rs(w, l0, algo, DT.FP64, SUM, 100 + n, seed + 6)
+        w.set_ccl_buffer_size(64 * 1024)
+        run_rs(w, l0, "rhd", DT.FP32, SUM, 30011, seed + 7)
+        w.set_ccl_buffer_size(0)
+        # the other orders do not look at the groups
+        rng = np.random.default_rng(seed)
+        ins = [gen(DT.FP32, SUM, rng, n * 321) for _ in range(n)]
+        want = [np.zeros(321, dtype=np.float32) for _ in range(n)]
+        assert oracle.reduce_scatter(ins, want, 321, int(DT.FP32), SUM, algo="mesh") == 0
+        recvs = [dev_zeros(x.nbytes) for x in want]
+        w.reduce_scatter([to_dev(x) for x in ins], recvs, 321, DT.FP32, SUM, "mesh")
+        check(DT.FP32, SUM, to_host(recvs[n - 1], np.float32), want[n - 1], "mesh with groups")
+    finally:
+        w.set_ccl_buffer_size(0)
         w.close()
 
 
@@ -148,6 +199,46 @@ def test_hccl_algo_is_read_when_a_world_is_created():
                     hccl_amd.all_reduce(w.comms[r], sends[r], recvs[r], count, DT.FP32, SUM, w.stream)
             w.sync()
             check(DT.FP32, SUM, to_host(recvs[2], np.float32), want[2], "HCCL_ALGO sole{nhr} with groups")
+        finally:
+            w.close()
+        # ReduceScatter: the strings of the reference's own system tests (reduce_scatter_aicpu_testcase*.cc)
+        os.environ["HCCL_ALGO"] = "reducescatter:sequence{level0=meshconcur,level1=rhd}"
+        w = World(6)
+        try:
+            assert hccl_amd.get_algo(w.comms[0], OpKind.REDUCE_SCATTER) == Algo.RHD
+            n, c = 6, 1003
+            rng = np.random.default_rng(8)
+            ins = [gen(DT.FP32, SUM, rng, n * c) for _ in range(n)]
+            want = [np.zeros(c, dtype=np.float32) for _ in range(n)]
+            assert oracle.reduce_scatter_two_level(ins, want, c, int(DT.FP32), SUM, 2, "rhd") == 0
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(x.nbytes) for x in want]
+            w.inputs_ready()
+            with hccl_amd.group():
+                for r in range(n):
+                    hccl_amd.reduce_scatter(w.comms[r], sends[r], recvs[r], c, DT.FP32, SUM, w.stream)
+            w.sync()
+            for r in range(n):
+                check(DT.FP32, SUM, to_host(recvs[r], np.float32), want[r], "HCCL_ALGO reducescatter sequence rank %d" % r)
+        finally:
+            w.close()
+        os.environ["HCCL_ALGO"] = "reducescatter:sole{level0=hdaicpureduce}"
+        w = World(6)
+        try:
+            assert hccl_amd.get_algo(w.comms[0], OpKind.REDUCE_SCATTER) == Algo.RHD
+            n, c = 6, 501
+            rng = np.random.default_rng(9)
+            ins = [gen(DT.FP32, SUM, rng, n * c) for _ in range(n)]
+            want = [np.zeros(c, dtype=np.float32) for _ in range(n)]
+            assert oracle.reduce_scatter(ins, want, c, int(DT.FP32), SUM, algo="rhd") == 0
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(x.nbytes) for x in want]
+            w.inputs_ready()
+            with hccl_amd.group():
+                for r in range(n):
+                    hccl_amd.reduce_scatter(w.comms[r], sends[r], recvs[r], c, DT.FP32, SUM, w.stream)
+            w.sync()
+            check(DT.FP32, SUM, to_host(recvs[4], np.float32), want[4], "HCCL_ALGO reducescatter sole{hd} with groups")
         finally:
             w.close()
         os.environ["HCCL_ALGO"] = "allreduce:sole{no_such_template}"
