@@ -30,7 +30,7 @@ FILES = ["tests/test_gpu_parity.py", "tests/test_gpu_copies.py", "tests/test_wid
          "tests/test_wide_gpu_rooted_sweep.py", "tests/test_gpu_rooted_and_v_ops.py",
          "tests/test_gpu_random_sweep.py", "tests/test_gpu_point_to_point.py",
          "tests/test_gpu_reference_python_suites.py", "tests/test_wide_gpu_reference_st_shapes.py",
-         "tests/test_zz_no_alloc.py"]
+         "tests/test_wide_gpu_reference_st_reduce_shapes.py", "tests/test_zz_no_alloc.py"]
 # Left out: tests that allocate or compute with torch on the GPU themselves (graphs, own streams, device-side
 # generators) and tests whose size is meant for the GPU.
 DESELECT = [
@@ -88,7 +88,7 @@ def test_gpu_parity_tests_pass_on_the_emulation_and_touch_no_byte_outside_their_
     rc, passed, tail = run_gpu_tests(emu_env(lib, log))
     reports = "".join(open(f).read()[:3000] for f in sorted(glob.glob(log + "*"))[:2])
     assert rc == 0 and not reports, tail + reports
-    assert passed >= 506, tail   # a shrinking selection would hide what no longer runs
+    assert passed >= 600, tail   # a shrinking selection would hide what no longer runs
 
 
 OVERRUN = r"""
