@@ -1,9 +1,11 @@
-"""Collects the shapes the reference's own system tests drive through AllReduce, ReduceScatter and Reduce, as data.
+"""Collects the shapes the reference's own system tests drive through AllReduce, ReduceScatter, Reduce, AllGather and
+AlltoAll, as data.
 
 Reads (as text; nothing of the reference is imported or run) the TEST_F cases of
     test/st/algorithm/testcase/all_reduce_testcase.cc
     test/st/algorithm/testcase/reduce_scatter_testcase.cc, reduce_scatter_aicpu_testcase.cc, ..._testcase2.cc, ..._testcase3.cc
     test/st/algorithm/testcase/reduce_testcase.cc, reduce_aicpu_testcase.cc
+    test/st/algorithm/testcase/all_gather_aicpu_testcase.cc, alltoall_testcase.cc
 and writes tests/golden/reference_st_reduce_shapes.json: one entry per case whose numbers are written out, with its
 name, the file and line it starts on, the servers of its topology (ranks per server), the element count (the
 file's constants folded in), the data type, the reduce operation, the root (Reduce) and the HCCL_ALGO string the case
@@ -23,9 +25,11 @@ FILES = {
     "reduce_scatter": ["reduce_scatter_testcase.cc", "reduce_scatter_aicpu_testcase.cc", "reduce_scatter_aicpu_testcase2.cc",
                        "reduce_scatter_aicpu_testcase3.cc"],
     "reduce": ["reduce_testcase.cc", "reduce_aicpu_testcase.cc"],
+    "all_gather": ["all_gather_aicpu_testcase.cc"],
+    "all_to_all": ["alltoall_testcase.cc"],
 }
 SIZES = {"INT8": 1, "UINT8": 1, "INT16": 2, "UINT16": 2, "FP16": 2, "BFP16": 2, "INT32": 4, "UINT32": 4, "FP32": 4,
-         "INT64": 8, "UINT64": 8, "FP64": 8}
+         "INT64": 8, "UINT64": 8, "FP64": 8, "HIF8": 1, "FP8E4M3": 1, "FP8E5M2": 1, "FP8E8M0": 1}
 
 
 def cases_of(text):
@@ -44,7 +48,8 @@ def strip_comments(body):
 
 def value_of(expr, names):
     """An element count written with numbers, the file's constants, + - * /, std::max / std::min and casts."""
-    e = re.sub(r"static_cast<\s*\w+\s*>", "", expr)
+    e = re.sub(r"sizeof\(\s*HcclDataType::\w+\s*\)", "4", expr)   # the size of the enumeration, as the case writes it
+    e = re.sub(r"static_cast<\s*\w+\s*>", "", e)
     e = re.sub(r"\(\s*(u64|uint64_t|u32)\s*\)", "", e)
     e = e.replace("std::max", "max").replace("std::min", "min")
     e = re.sub(r"(\d+)[uUlL]+\b", r"\1", e)
@@ -94,7 +99,7 @@ def main():
                 if dtype and dtype.group(1) in SIZES:
                     names["dataTypeSize"] = SIZES[dtype.group(1)]
                 count = None
-                m = re.search(r"\b(?:dataCount|recvCount|count)\s*=\s*([^;]+);", body)
+                m = re.search(r"\b(?:dataCount|recvCount|sendCount|sendDataCount|count)\s*=\s*([^;]+);", body)
                 call = re.search(r"\bRun\w+\(\s*(\w+)\s*,(.*?)\)\s*;", body, re.S)
                 args = [a.strip() for a in re.split(r",(?![^()]*\))", call.group(2))] if call else []
                 if m:

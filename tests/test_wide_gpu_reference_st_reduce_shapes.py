@@ -1,7 +1,8 @@
-"""Replays the shapes of the reference's own system tests for AllReduce, ReduceScatter and Reduce
+"""Replays the shapes of the reference's own system tests for AllReduce, ReduceScatter, Reduce, AllGather and AlltoAll
 (test/st/algorithm/testcase/all_reduce_testcase.cc, reduce_scatter_testcase.cc, reduce_scatter_aicpu_testcase*.cc,
-reduce_testcase.cc, reduce_aicpu_testcase.cc; transcribed as data into tests/golden/reference_st_reduce_shapes.json by
-tests/golden/make_reference_st_reduce_shapes.py) through the C ABI against the oracle: the servers of the case's
+reduce_testcase.cc, reduce_aicpu_testcase.cc, all_gather_aicpu_testcase.cc, alltoall_testcase.cc; transcribed as
+data into tests/golden/reference_st_reduce_shapes.json by tests/golden/make_reference_st_reduce_shapes.py) through
+the C ABI against the oracle: the servers of the case's
 topology become the level-0 groups of a loopback world, the HCCL_ALGO string the case sets is in the environment when
 the world is created, and the expected bits come from the oracle in the order that string selects here (the two-level
 orders where it names a sequence executor this library builds, the one-level order otherwise).  The reference checks
@@ -17,7 +18,7 @@ import hccl_amd
 import oracle
 from hccl_amd import Algo, HcclDataType as DT, OpKind
 
-from gpu_util import World, dev_zeros, require_library_on_gpu, to_dev, to_host
+from gpu_util import World, dev_zeros, rand_bytes, require_library_on_gpu, to_dev, to_host
 from test_gpu_parity import NP, check, gen, order_of
 
 pytestmark = pytest.mark.gpu
@@ -28,6 +29,10 @@ TYPES = {"INT8": DT.INT8, "INT16": DT.INT16, "INT32": DT.INT32, "INT64": DT.INT6
          "BFP16": DT.BFP16, "FP32": DT.FP32, "FP64": DT.FP64}
 OPS = {"SUM": 0, "PROD": 1, "MAX": 2, "MIN": 3}
 KINDS = {"all_reduce": OpKind.ALL_REDUCE, "reduce_scatter": OpKind.REDUCE_SCATTER, "reduce": OpKind.REDUCE}
+COPIES = ("all_gather", "all_to_all")
+SIZES = {"INT8": 1, "UINT8": 1, "INT16": 2, "UINT16": 2, "FP16": 2, "BFP16": 2, "INT32": 4, "UINT32": 4, "FP32": 4,
+         "INT64": 8, "UINT64": 8, "FP64": 8, "HIF8": 1, "FP8E4M3": 1, "FP8E5M2": 1, "FP8E8M0": 1}
+FILL = 0xAB
 NAMES = {Algo.MESH: "mesh", Algo.RING: "ring", Algo.RHD: "rhd", Algo.NHR: "nhr", Algo.MESH_CHUNK: "mesh_chunk",
          Algo.ORDER_PRESERVED: "order_preserved", Algo.MESH_TWO_SHOT: "mesh_two_shot", Algo.AIV_MESH: "aiv_mesh",
          Algo.MESH_SYMMETRIC: "mesh_symmetric"}
@@ -45,18 +50,51 @@ def scaled(count, n):
     return base + n * ((count // n) % 7) + count % n
 
 
+def copy_shape(case, n):
+    dtype, esz = DT[case["type"]], SIZES[case["type"]]
+    count = scaled(case["count"], n)
+    rng = np.random.default_rng(len(case["name"]) * 17 + count)
+    w = World(n)
+    try:
+        if case["kind"] == "all_gather":
+            ins = [rand_bytes(rng, max(count, 1) * esz) for _ in range(n)]
+            want = [np.full(n * count * esz, FILL, dtype=np.uint8) for _ in range(n)]
+            assert oracle.all_gather(ins, want, count, int(dtype)) == 0
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(max(x.nbytes, 1), fill=FILL) for x in want]
+            w.all_gather(sends, recvs, count, dtype)
+        else:
+            ins = [rand_bytes(rng, max(n * count, 1) * esz) for _ in range(n)]
+            want = [np.full(n * count * esz, FILL, dtype=np.uint8) for _ in range(n)]
+            assert oracle.all_to_all(ins, want, count, int(dtype)) == 0
+            sends = [to_dev(x) for x in ins]
+            recvs = [dev_zeros(max(x.nbytes, 1), fill=FILL) for x in want]
+            w.inputs_ready()
+            with hccl_amd.group():
+                for r in range(n):
+                    hccl_amd.all_to_all(w.comms[r], sends[r], count, dtype, recvs[r], count, dtype, w.stream)
+            w.sync()
+        for r in range(n):
+            assert np.array_equal(to_host(recvs[r], np.uint8)[:want[r].nbytes], want[r]), (case["name"], case["source"], r)
+    finally:
+        w.close()
+
+
 def test_the_catalogue_is_what_the_generator_wrote():
-    assert len(CASES) == 78
-    assert {c["kind"] for c in CASES} == set(KINDS)
-    assert all(c["type"] in TYPES and c["op"] in OPS and sum(c["servers"]) <= 64 for c in CASES)
+    assert len(CASES) == 126
+    assert {c["kind"] for c in CASES} == set(KINDS) | set(COPIES)
+    assert all(c["type"] in (SIZES if c["kind"] in COPIES else TYPES) and c["op"] in OPS and sum(c["servers"]) <= 64
+               for c in CASES)
     assert scaled(262148, 12) % 12 == 8 and scaled(5, 3) == 5 and scaled(0, 4) == 0 and scaled(419430400, 8) % 8 == 0
 
 
 @pytest.mark.parametrize("case", CASES, ids=[c["name"] for c in CASES])
 def test_reference_system_test_shape(case):
-    kind, dtype, op = case["kind"], TYPES[case["type"]], OPS[case["op"]]
     servers = case["servers"]
     n = sum(servers)
+    if case["kind"] in COPIES:
+        return copy_shape(case, n)
+    kind, dtype, op = case["kind"], TYPES[case["type"]], OPS[case["op"]]
     level0 = servers[0] if len(servers) > 1 and len(set(servers)) == 1 and servers[0] > 1 else 1
     count = scaled(case["count"], n)
     env = {"HCCL_AMD_LEVEL0_RANKS": str(level0)}
