@@ -2,14 +2,14 @@
 picked, timed on the same buffers in one process with hccl_amd.tune: on shapes that lie well inside a form's territory
 the library's choice has to be within a few per cent of the fastest forced form.  A kernel change that moves a
 crossover far enough shows up here; the rows next to the thresholds themselves are what `python -m hccl_amd.tune`
-prints.  Timing only: what the forms compute is compared with the oracle elsewhere."""
+prints.  Timing only: what the forms compute is compared with the oracle elsewhere; collected behind the parity tests."""
 import pytest
 
 from gpu_util import require_library_on_gpu
 
 pytestmark = pytest.mark.gpu
 
-TOLERANCE = 0.94    # forms of a row repeat within 1 %; between the forms of these shapes lie 5 to 25 %
+TOLERANCE = 0.92    # forms of a row repeat within 1 %; between the forms of these shapes lie 5 to 25 %
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -31,7 +31,7 @@ def test_all_reduce_form(ranks, mib):
     import torch
     import hccl_amd
     from hccl_amd import tune
-    assert behind_best(tune.all_reduce_rows(torch, hccl_amd, [ranks], [mib], 2)) == []
+    assert behind_best(tune.all_reduce_rows(torch, hccl_amd, [ranks], [mib], 3)) == []
 
 
 @pytest.mark.parametrize("ranks,kib", [(8, 4096), (8, 16384), (2, 4096)])
@@ -39,7 +39,7 @@ def test_small_all_reduce_form(ranks, kib):
     import torch
     import hccl_amd
     from hccl_amd import tune
-    assert behind_best(tune.all_reduce_small_rows(torch, hccl_amd, [ranks], [kib], 2)) == []
+    assert behind_best(tune.all_reduce_small_rows(torch, hccl_amd, [ranks], [kib], 3)) == []
 
 
 @pytest.mark.parametrize("ranks,mib", [(4, 64), (16, 8)])
@@ -47,7 +47,7 @@ def test_all_gather_form(ranks, mib):
     import torch
     import hccl_amd
     from hccl_amd import tune
-    assert behind_best(tune.all_gather_rows(torch, hccl_amd, [ranks], [mib], 2)) == []
+    assert behind_best(tune.all_gather_rows(torch, hccl_amd, [ranks], [mib], 3)) == []
 
 
 @pytest.mark.parametrize("ranks,mib", [(6, 16), (16, 64)])
@@ -55,4 +55,4 @@ def test_broadcast_form(ranks, mib):
     import torch
     import hccl_amd
     from hccl_amd import tune
-    assert behind_best(tune.broadcast_rows(torch, hccl_amd, [ranks], [mib], 2)) == []
+    assert behind_best(tune.broadcast_rows(torch, hccl_amd, [ranks], [mib], 3)) == []
