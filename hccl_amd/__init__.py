@@ -149,7 +149,11 @@ def _bind(L):
     L.HcclAmdGetAlgo.argtypes = [vp, i32, ctypes.POINTER(i32)]
     L.HcclAmdGetFoldProgram.argtypes = [i32, i32, u32, u32, vp, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
     L.HcclAmdGetFoldProgramTwoLevel.argtypes = [i32, i32, u32, u32, u32, vp, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
+    L.HcclAmdGetFoldProgramLevels.argtypes = [i32, i32, u32, u32, u32, u32, vp, u32, ctypes.POINTER(u32),
+                                              ctypes.POINTER(u32)]
     L.HcclAmdSetLevel0RankSize.argtypes = [vp, u32]
+    L.HcclAmdSetLevel1GroupSize.argtypes = [vp, u32]
+    L.HcclAmdGetLevel1GroupSize.argtypes = [vp, ctypes.POINTER(u32)]
     L.HcclAmdGetLevel0RankSize.argtypes = [vp, ctypes.POINTER(u32)]
     L.HcclAmdSelectFromHcclAlgo.argtypes = [ctypes.c_char_p, i32, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(i32),
                                             ctypes.POINTER(ctypes.c_int32), ctypes.c_char_p, u32]
@@ -308,17 +312,18 @@ def get_stuck_counters(hccl_comm):
     return head.value, tail.value
 
 
-def fold_programs(op_kind, algo, rank_size, level0=1):
+def fold_programs(op_kind, algo, rank_size, level0=1, level1=0):
     """Host-only: the byte programs (one per segment) that fix the reduction order; level0 > 1: the two-level
-    AllReduce or ReduceScatter over groups of level0 consecutive ranks with `algo` between the groups."""
+    AllReduce, ReduceScatter or Reduce over groups of level0 consecutive ranks with `algo` between the groups;
+    level1 > 0: the three-level one, level1 consecutive groups forming a level-1 group."""
     L = lib()
     out = []
     seg, count = 0, 1
     while seg < count:
         buf = (ctypes.c_uint8 * 512)()
         ln, cnt = ctypes.c_uint32(), ctypes.c_uint32()
-        check(L.HcclAmdGetFoldProgramTwoLevel(int(op_kind), int(algo), rank_size, level0, seg, buf, 512,
-                                              ctypes.byref(ln), ctypes.byref(cnt)), "HcclAmdGetFoldProgramTwoLevel")
+        check(L.HcclAmdGetFoldProgramLevels(int(op_kind), int(algo), rank_size, level0, level1, seg, buf, 512,
+                                            ctypes.byref(ln), ctypes.byref(cnt)), "HcclAmdGetFoldProgramLevels")
         count = cnt.value
         out.append(bytes(buf[:ln.value]))
         seg += 1
@@ -333,6 +338,19 @@ def set_level0_rank_size(hccl_comm, ranks_per_group):
 def get_level0_rank_size(hccl_comm):
     v = ctypes.c_uint32()
     check(lib().HcclAmdGetLevel0RankSize(hccl_comm, ctypes.byref(v)), "HcclAmdGetLevel0RankSize")
+    return v.value
+
+
+def set_level1_group_size(hccl_comm, groups_per_level1_group):
+    """How many consecutive level-0 groups form a level-1 group (a pod of servers) in the world hccl_comm belongs
+    to; 0: all of them, which leaves two levels."""
+    return check(lib().HcclAmdSetLevel1GroupSize(hccl_comm, ctypes.c_uint32(groups_per_level1_group)),
+                 "HcclAmdSetLevel1GroupSize")
+
+
+def get_level1_group_size(hccl_comm):
+    v = ctypes.c_uint32()
+    check(lib().HcclAmdGetLevel1GroupSize(hccl_comm, ctypes.byref(v)), "HcclAmdGetLevel1GroupSize")
     return v.value
 
 

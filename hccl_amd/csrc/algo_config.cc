@@ -311,13 +311,13 @@ bool OrderOf(HcclAmdOpKind op, const std::string& t, HcclAmdAlgo* algo)
         return op != HCCL_AMD_OP_REDUCE;
     }
     if (t == "nhraicpureduce") {
-        // host-reduce NHR: AllReduce gathers and folds in rank order, ReduceScatter folds the own slice first
+        // host-reduce NHR: AllReduce and Reduce gather and fold in rank order, ReduceScatter folds the own slice first
         *algo = op == HCCL_AMD_OP_ALL_REDUCE ? HCCL_AMD_ALGO_RING : HCCL_AMD_ALGO_MESH;
-        return op != HCCL_AMD_OP_REDUCE;
+        return true;
     }
-    if (op == HCCL_AMD_OP_REDUCE) {
+    if (op == HCCL_AMD_OP_REDUCE && IsMeshFamily(t)) {
         *algo = t == "meshtwoshot" ? HCCL_AMD_ALGO_MESH_TWO_SHOT : HCCL_AMD_ALGO_MESH;
-        return IsMeshFamily(t);
+        return true;
     }
     if (IsMeshFamily(t)) {
         *algo = HCCL_AMD_ALGO_MESH;
@@ -399,24 +399,32 @@ AlgoSelection SelectFromHcclAlgo(const std::vector<AlgoSegment>& segments)
                 if (!OrderOf(kind, seg.templates[0].name, &algo)) {
                     continue;
                 }
-            } else if (seg.templates.size() == 2 && seg.executor == "sequence" &&
-                       (kind == HCCL_AMD_OP_ALL_REDUCE || kind == HCCL_AMD_OP_REDUCE_SCATTER) &&
+            } else if ((seg.templates.size() == 2 || seg.templates.size() == 3) && seg.executor == "sequence" &&
                        IsMeshFamily(seg.templates[0].name) && seg.templates[0].name.compare(0, 9, "meshchunk") != 0) {
                 // a mesh inside the level-0 groups (the mesh-chunk templates fold in another order there, which is
-                // not built), the second template between them
+                // not built), the second template between them and, with a third level, the same one once more
+                // (the reference registers Sequence MeshConcur NHR NHR and ... RHD RHD, no mixed forms)
                 if (!OrderOf(kind, seg.templates[1].name, &algo) ||
                     (algo != HCCL_AMD_ALGO_RHD && algo != HCCL_AMD_ALGO_NHR && algo != HCCL_AMD_ALGO_MESH &&
                      algo != HCCL_AMD_ALGO_RING)) {
                     continue;
                 }
                 if (seg.templates[1].name == "nhraicpureduce") {
+                    if (seg.templates.size() == 3) {
+                        continue;                // the host-reduce executors know two levels
+                    }
                     algo = HCCL_AMD_ALGO_MESH;   // between the groups: the own-first fold of the host-reduce template
                 } else if (algo == HCCL_AMD_ALGO_MESH || algo == HCCL_AMD_ALGO_RING) {
                     continue;                    // a mesh between the groups: another executor family
                 }
+                HcclAmdAlgo third;
+                if (seg.templates.size() == 3 && (!OrderOf(kind, seg.templates[2].name, &third) || third != algo ||
+                                                  seg.templates[2].name == "nhraicpureduce")) {
+                    continue;
+                }
                 twoLevel = true;
             } else {
-                continue;   // deeper hierarchies and two-level forms of the other operators are not built
+                continue;   // the other executors over several levels (parallel, pipeline, concur) are not built
             }
             sel.set[op] = true;
             sel.algo[op] = algo;

@@ -1021,6 +1021,9 @@ HcclResult HcclAmdSetLevel0RankSize(HcclComm comm, uint32_t ranksPerGroup)
     }
     std::lock_guard<std::mutex> wl(c->world->mu);
     c->world->level0 = ranksPerGroup;
+    if (c->world->level1 != 0 && (c->world->n / ranksPerGroup) % c->world->level1 != 0) {
+        c->world->level1 = 0;   // the level-1 groups no longer divide the level-0 groups: back to two levels
+    }
     return HCCL_SUCCESS;
 }
 
@@ -1035,6 +1038,37 @@ HcclResult HcclAmdGetLevel0RankSize(HcclComm comm, uint32_t* ranksPerGroup)
     }
     std::lock_guard<std::mutex> wl(c->world->mu);
     *ranksPerGroup = c->world->level0;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdSetLevel1GroupSize(HcclComm comm, uint32_t groupsPerLevel1Group)
+{
+    CHK_PTR(comm, "comm");
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> wl(c->world->mu);
+    const uint32_t groups = c->world->n / c->world->level0;
+    if (groupsPerLevel1Group != 0 && (groupsPerLevel1Group > groups || groups % groupsPerLevel1Group != 0)) {
+        return HCCL_E_PARA;
+    }
+    c->world->level1 = groupsPerLevel1Group;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdGetLevel1GroupSize(HcclComm comm, uint32_t* groupsPerLevel1Group)
+{
+    CHK_PTR(comm, "comm");
+    CHK_PTR(groupsPerLevel1Group, "groupsPerLevel1Group");
+    CommRef ref = AsComm(comm);
+    Comm* c = ref.c;
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> wl(c->world->mu);
+    *groupsPerLevel1Group = c->world->level1;
     return HCCL_SUCCESS;
 }
 
@@ -1084,24 +1118,31 @@ HcclResult HcclAmdSelectFromHcclAlgo(const char* config, HcclAmdOpKind op, int32
 HcclResult HcclAmdGetFoldProgram(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t segment,
                                  uint8_t* out, uint32_t cap, uint32_t* len, uint32_t* segmentCount)
 {
-    return HcclAmdGetFoldProgramTwoLevel(op, algo, rankSize, 1, segment, out, cap, len, segmentCount);
+    return HcclAmdGetFoldProgramLevels(op, algo, rankSize, 1, 0, segment, out, cap, len, segmentCount);
 }
 
 HcclResult HcclAmdGetFoldProgramTwoLevel(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t level0,
                                          uint32_t segment, uint8_t* out, uint32_t cap, uint32_t* len,
                                          uint32_t* segmentCount)
 {
+    return HcclAmdGetFoldProgramLevels(op, algo, rankSize, level0, 0, segment, out, cap, len, segmentCount);
+}
+
+HcclResult HcclAmdGetFoldProgramLevels(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t level0,
+                                       uint32_t level1, uint32_t segment, uint8_t* out, uint32_t cap, uint32_t* len,
+                                       uint32_t* segmentCount)
+{
     CHK_PTR(len, "len");
     // Callers walk all segments of one plan: keep the last plan built.
     static std::mutex cacheMu;
     static FoldPlan plan;
     static int cachedOp = -1, cachedAlgo = -1;
-    static uint32_t cachedSize = 0, cachedLevel0 = 0;
+    static uint32_t cachedSize = 0, cachedLevel0 = 0, cachedLevel1 = 0;
     std::lock_guard<std::mutex> cacheLock(cacheMu);
     if (cachedOp != static_cast<int>(op) || cachedAlgo != static_cast<int>(algo) || cachedSize != rankSize ||
-        cachedLevel0 != level0) {
+        cachedLevel0 != level0 || cachedLevel1 != level1) {
         cachedOp = -1;
-        HcclResult rc = BuildFoldPlan(op, algo, rankSize, &plan, level0);
+        HcclResult rc = BuildFoldPlan(op, algo, rankSize, &plan, level0, level1);
         if (rc != HCCL_SUCCESS) {
             return rc;
         }
@@ -1109,6 +1150,7 @@ HcclResult HcclAmdGetFoldProgramTwoLevel(HcclAmdOpKind op, HcclAmdAlgo algo, uin
         cachedAlgo = static_cast<int>(algo);
         cachedSize = rankSize;
         cachedLevel0 = level0;
+        cachedLevel1 = level1;
     }
     if (segmentCount != nullptr) {
         *segmentCount = static_cast<uint32_t>(plan.programs.size());

@@ -341,43 +341,37 @@ std::vector<ExprPtr> RhdValues(uint32_t p, const LeafFn& leaf)
 
 HcclResult Rhd(uint32_t p, FoldPlan* plan) { return EmitAll(RhdValues(p, RankLeaf), plan); }
 
-// ---- two levels --------------------------------------------------------------------------------
-// AllReduce over level-0 groups of l0 consecutive ranks ("boxes") and a level-1 template between the boxes
-// (reference ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852: step 1 mesh ReduceScatter inside the box,
-// step 2 level-1 ReduceScatter between the ranks that hold the same chunk, steps 3 and 4 the two AllGathers).
-// A loop's elements are l0 chunks of l1 sub-slices; sub-slice j of chunk i is program i * l1 + j: the level-1
-// template's value for its unit j, in which participant b stands for what box b folded for chunk i, the chunk
-// owner's input first and the other ranks of the box ascending (reference
-// ins_temp_reduce_scatter_mesh_1D.cc:203-237; the level-0 template ..._Z_axis_detour derives from it).
-// Level 1: RHD with POST skipped and the merged share bridged (:700-741), NHR (:784-789), or for the types the
-// host reduces the own-first fold of ins_temp_reduce_scatter_aicpu_reduce_nhr.cc:214-250 (`MESH`).
-// The level-1 template's values for the units of level-0 member i: unit j is what the boxes end with for the share
-// of box j, participant b standing for what box b has folded for that unit.
-HcclResult TwoLevelUnits(uint32_t l0, uint32_t l1, HcclAmdAlgo level1, uint32_t i, std::vector<ExprPtr>* units)
+// ---- two and three levels ----------------------------------------------------------------------
+// AllReduce over level-0 groups of l0 consecutive ranks ("boxes") and a template between the boxes (reference
+// ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852: step 1 mesh ReduceScatter inside the box, step 2 the
+// ReduceScatter between the ranks that hold the same chunk, steps 3 and 4 the two AllGathers).  A loop's elements
+// are l0 chunks of l1 sub-slices; sub-slice j of chunk i is the template's value for its unit j, in which
+// participant b stands for what box b folded for chunk i, the chunk owner's input first and the other ranks of the
+// box ascending (reference ins_temp_reduce_scatter_mesh_1D.cc:203-237; the level-0 template ..._Z_axis_detour
+// derives from it).  The template: RHD with POST skipped and the merged share bridged (:700-741), NHR (:784-789),
+// or for the types the host reduces the own-first fold of ins_temp_reduce_scatter_aicpu_reduce_nhr.cc:214-250
+// (`MESH`).
+// With three levels (reference ins_v2_all_reduce_sequence_executor_aicpu_3level.cc:536-800) l1 consecutive boxes
+// form a level-1 group, the template runs between the boxes of a group on the sub-slices and once more between
+// the l2 groups on the parts of a sub-slice: part k of sub-slice j is the template's value for unit k among the
+// groups, participant g standing for the value of unit j among the boxes of group g.  Rank (g * l1 + b) * l0 + i
+// is member i of box b of group g.
+HcclResult TemplateValues(HcclAmdAlgo algo, uint32_t count, const LeafFn& leaf, std::vector<ExprPtr>* out)
 {
-    const LeafFn box = [&](uint32_t b) {
-        std::vector<uint32_t> order{b * l0 + i};
-        for (uint32_t t = 0; t < l0; ++t) {
-            if (t != i) {
-                order.push_back(b * l0 + t);
-            }
-        }
-        return Chain(order);
-    };
-    units->clear();
-    if (level1 == HCCL_AMD_ALGO_RHD) {
-        *units = RhdValues(l1, box);
-    } else if (level1 == HCCL_AMD_ALGO_NHR) {
-        *units = NhrValues(l1, box);
-    } else if (level1 == HCCL_AMD_ALGO_MESH) {
-        for (uint32_t j = 0; j < l1; ++j) {
-            ExprPtr e = box(j);
-            for (uint32_t b = 0; b < l1; ++b) {
+    out->clear();
+    if (algo == HCCL_AMD_ALGO_RHD) {
+        *out = RhdValues(count, leaf);
+    } else if (algo == HCCL_AMD_ALGO_NHR) {
+        *out = NhrValues(count, leaf);
+    } else if (algo == HCCL_AMD_ALGO_MESH) {
+        for (uint32_t j = 0; j < count; ++j) {
+            ExprPtr e = leaf(j);
+            for (uint32_t b = 0; b < count; ++b) {
                 if (b != j) {
-                    e = Fold(e, box(b));
+                    e = Fold(e, leaf(b));
                 }
             }
-            units->push_back(e);
+            out->push_back(e);
         }
     } else {
         return HCCL_E_NOT_SUPPORT;
@@ -385,13 +379,52 @@ HcclResult TwoLevelUnits(uint32_t l0, uint32_t l1, HcclAmdAlgo level1, uint32_t 
     return HCCL_SUCCESS;
 }
 
-HcclResult TwoLevelAllReduce(uint32_t n, uint32_t l0, HcclAmdAlgo level1, FoldPlan* plan)
+// The values of level-0 member i: unit j * l2 + k is part k of sub-slice j of its chunk.
+HcclResult LevelUnits(const Levels& lv, HcclAmdAlgo algo, uint32_t i, std::vector<ExprPtr>* units)
 {
-    const uint32_t l1 = n / l0;
+    std::vector<std::vector<ExprPtr>> group(lv.l2);
+    for (uint32_t g = 0; g < lv.l2; ++g) {
+        const LeafFn box = [&](uint32_t b) {
+            const uint32_t first = (g * lv.l1 + b) * lv.l0;
+            std::vector<uint32_t> order{first + i};
+            for (uint32_t t = 0; t < lv.l0; ++t) {
+                if (t != i) {
+                    order.push_back(first + t);
+                }
+            }
+            return Chain(order);
+        };
+        HcclResult rc = TemplateValues(algo, lv.l1, box, &group[g]);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    if (lv.l2 == 1) {
+        *units = group[0];
+        return HCCL_SUCCESS;
+    }
+    units->assign(static_cast<size_t>(lv.l1) * lv.l2, nullptr);
+    for (uint32_t j = 0; j < lv.l1; ++j) {
+        std::vector<ExprPtr> parts;
+        HcclResult rc = TemplateValues(algo, lv.l2, [&](uint32_t g) { return group[g][j]; }, &parts);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+        for (uint32_t k = 0; k < lv.l2; ++k) {
+            (*units)[static_cast<size_t>(j) * lv.l2 + k] = parts[k];
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// AllReduce, and Reduce, whose sequence executors run the same steps and hand the result to the root only
+// (reference reduce_sequence_executor_aicpu_3level.cc:744-990).
+HcclResult LevelsAllReduce(const Levels& lv, HcclAmdAlgo algo, FoldPlan* plan)
+{
     plan->segmentsAreSubs = true;
-    for (uint32_t i = 0; i < l0; ++i) {
+    for (uint32_t i = 0; i < lv.l0; ++i) {
         std::vector<ExprPtr> units;
-        HcclResult rc = TwoLevelUnits(l0, l1, level1, i, &units);
+        HcclResult rc = LevelUnits(lv, algo, i, &units);
         if (rc == HCCL_SUCCESS) {
             rc = EmitAll(units, plan);
         }
@@ -404,25 +437,28 @@ HcclResult TwoLevelAllReduce(uint32_t n, uint32_t l0, HcclAmdAlgo level1, FoldPl
 
 // ReduceScatter over the same boxes (reference ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-372, 388-500):
 // step 1 is the mesh ReduceScatter inside the box once per box of the world (in repeat q member i folds slice
-// q * l0 + i of its box, its own input first), step 2 the level-1 ReduceScatter between the members i, whose unit q
-// is that slice; box j ends with unit j, the output of rank j * l0 + i.  Program r is therefore the level-1
-// template's value for unit r / l0 among the members r % l0: the tree of sub-slice r / l0 of chunk r % l0 of the
-// two-level AllReduce.  Level 1: RHD (reduce_scatter_rhd with its POST, which moves shares and folds nothing),
-// NHR, or the own-first fold of reduce_scatter_aicpu_reduce_nhr_pcie.cc:212-280 (`MESH`).  A loop covers the same
-// range of every slice, so loop boundaries do not show in the result.
-HcclResult TwoLevelReduceScatter(uint32_t n, uint32_t l0, HcclAmdAlgo level1, FoldPlan* plan)
+// q * l0 + i of its box, its own input first), step 2 the ReduceScatter between the members i, whose unit q is that
+// slice; box j ends with unit j, the output of rank j * l0 + i.  With three levels
+// (ins_v2_reduce_scatter_sequence_executor_3level.cc:243-256) the boxes of a group do that for the slices of every
+// group, and the groups reduce-scatter what they hold for each other.  Program r is therefore the tree of part
+// r / (l0 * l1) of sub-slice r / l0 % l1 of chunk r % l0 of the AllReduce over the same levels.  The template: RHD
+// (reduce_scatter_rhd with its POST, which moves shares and folds nothing), NHR, or the own-first fold of
+// reduce_scatter_aicpu_reduce_nhr_pcie.cc:212-280 (`MESH`).  A loop covers the same range of every slice, so loop
+// boundaries do not show in the result.
+HcclResult LevelsReduceScatter(const Levels& lv, HcclAmdAlgo algo, FoldPlan* plan)
 {
-    const uint32_t l1 = n / l0;
     plan->segmentsAreSubs = false;
-    std::vector<std::vector<ExprPtr>> units(l0);
-    for (uint32_t i = 0; i < l0; ++i) {
-        HcclResult rc = TwoLevelUnits(l0, l1, level1, i, &units[i]);
+    std::vector<std::vector<ExprPtr>> units(lv.l0);
+    for (uint32_t i = 0; i < lv.l0; ++i) {
+        HcclResult rc = LevelUnits(lv, algo, i, &units[i]);
         if (rc != HCCL_SUCCESS) {
             return rc;
         }
     }
+    const uint32_t n = lv.l0 * lv.l1 * lv.l2;
     for (uint32_t r = 0; r < n; ++r) {
-        HcclResult rc = Emit(units[r % l0][r / l0], plan);
+        const uint32_t box = r / lv.l0;
+        HcclResult rc = Emit(units[r % lv.l0][static_cast<size_t>(box % lv.l1) * lv.l2 + box / lv.l1], plan);
         if (rc != HCCL_SUCCESS) {
             return rc;
         }
@@ -462,33 +498,62 @@ uint32_t RhdCarrierOfVirtual(uint32_t p, uint32_t v)
     return v < r ? v : v + r;
 }
 
-HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPlan* plan, uint32_t level0)
+bool ResolveLevels(uint32_t n, uint32_t level0, uint32_t level1, Levels* out)
+{
+    if (level0 <= 1 || level0 >= n || n % level0 != 0) {
+        return false;
+    }
+    const uint32_t boxes = n / level0;
+    out->l0 = level0;
+    if (level1 == 0 || level1 >= boxes) {
+        out->l1 = boxes;
+        out->l2 = 1;
+        return true;
+    }
+    if (boxes % level1 != 0) {
+        return false;
+    }
+    out->l1 = level1;
+    out->l2 = boxes / level1;
+    return true;
+}
+
+HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPlan* plan, uint32_t level0,
+                         uint32_t level1)
 {
     *plan = FoldPlan{};
     if (n == 0 || n > static_cast<uint32_t>(kMaxRanks)) {
         return HCCL_E_PARA;
     }
     if (level0 > 1 && level0 < n) {
-        if (n % level0 != 0) {
+        Levels lv;
+        // the host-reduce fold knows two levels only: every box of the world is its peer
+        if (!ResolveLevels(n, level0, algo == HCCL_AMD_ALGO_MESH ? 0 : level1, &lv)) {
             return HCCL_E_PARA;
         }
-        if (op == HCCL_AMD_OP_ALL_REDUCE) {
-            return TwoLevelAllReduce(n, level0, algo, plan);
+        if (op == HCCL_AMD_OP_ALL_REDUCE || op == HCCL_AMD_OP_REDUCE) {
+            return LevelsAllReduce(lv, algo, plan);
         }
         if (op == HCCL_AMD_OP_REDUCE_SCATTER) {
-            return TwoLevelReduceScatter(n, level0, algo, plan);
+            return LevelsReduceScatter(lv, algo, plan);
         }
         return HCCL_E_NOT_SUPPORT;
     }
     if (op == HCCL_AMD_OP_REDUCE) {
         // One-shot: rank 0's slot is the base, the others fold ascending (reference reduce_mesh_1D.cc:268-300).
         // Two-shot: slice k is folded at rank k, own input first (reference reduce_mesh_1D_two_shot.cc:228-265).
+        // NHR: the step tree of the NHR ReduceScatter on n slices, gathered at the root (reference
+        // reduce_nhr.cc:263-339, 481-519).
         if (algo == HCCL_AMD_ALGO_MESH || algo == HCCL_AMD_ALGO_RING) {
             return MeshAllReduce(n, plan);
         }
         if (algo == HCCL_AMD_ALGO_MESH_TWO_SHOT) {
             plan->segmentsAreSubs = true;
             return MeshReduceScatter(n, plan);
+        }
+        if (algo == HCCL_AMD_ALGO_NHR) {
+            plan->segmentsAreSubs = true;
+            return Nhr(n, plan);
         }
         return HCCL_E_NOT_SUPPORT;
     }
@@ -604,6 +669,52 @@ uint64_t RhdSelectLoopCount(uint64_t remaining, uint64_t maxCountPerLoop, uint64
 {
     const uint64_t count = std::min(remaining, maxCountPerLoop);
     return count >= p ? count / p * p : count;
+}
+
+HcclResult SequenceMaxCountPerLoop(uint64_t cclBytes, uint64_t count, uint32_t l0, uint32_t total, uint64_t elemSize,
+                                   uint64_t align, bool rhdTail, uint64_t* maxCount, uint64_t* resultElems)
+{
+    if (l0 == 0 || total == 0 || elemSize == 0 || align == 0) {
+        return HCCL_E_PARA;
+    }
+    uint64_t workspace = cclBytes;
+    if (rhdTail && count % total != 0) {
+        if (total > workspace / elemSize / 2) {
+            return HCCL_E_INTERNAL;
+        }
+        const uint64_t slot = (total * elemSize + 127) / 128 * 128;
+        if (slot >= workspace / 2) {
+            return HCCL_E_INTERNAL;
+        }
+        workspace -= 2 * slot;
+    }
+    const uint64_t slice = workspace / (l0 + 1ull) / elemSize * elemSize;
+    *resultElems = slice / elemSize;
+    *maxCount = slice * l0 / align * align / elemSize / total * total;
+    return *maxCount == 0 ? HCCL_E_INTERNAL : HCCL_SUCCESS;
+}
+
+uint64_t SequenceSelectLoopCount(uint64_t remaining, uint64_t maxCountPerLoop, uint32_t l0, uint64_t resultElems)
+{
+    if (remaining > maxCountPerLoop) {
+        return maxCountPerLoop;
+    }
+    const uint64_t q = remaining / l0;
+    const uint64_t r = remaining % l0;
+    if (q + r <= resultElems || q == 0) {
+        return remaining;
+    }
+    if (resultElems == 0) {
+        return 0;
+    }
+    uint64_t newQ = q - 1;
+    uint64_t newR = 0;
+    if (newQ >= resultElems) {
+        newQ = resultElems;
+    } else {
+        newR = std::min<uint64_t>(l0 - 1, resultElems - newQ);
+    }
+    return newQ * l0 + newR;
 }
 
 }  // namespace hccl_amd

@@ -20,11 +20,21 @@ struct FoldPlan {
 };
 
 // Returns HCCL_E_NOT_SUPPORT for combinations that do not exist (e.g. AIV_MESH AllReduce).
-// level0 in (1, rankSize): the two-level AllReduce of the reference's sequence executor over groups of level0
-// consecutive ranks, `algo` (RHD, NHR, or MESH for the host-reduce fold) being the template between the groups;
-// program i * (rankSize / level0) + j is sub-slice j of chunk i; for ReduceScatter the two-level order of the same
-// executor family, program r being rank r's output.  level0 of 1 or rankSize: one level.
-HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, FoldPlan* plan, uint32_t level0 = 1);
+// level0 in (1, rankSize): the orders of the reference's sequence executors over level-0 groups of level0 consecutive
+// ranks, `algo` (RHD, NHR, or MESH for the host-reduce fold) being the template between the groups.  level1 in
+// [1, rankSize / level0): level1 consecutive groups form a level-1 group and the template runs a second time between
+// those (three levels; 0: all groups are one level-1 group, two levels).  With l1 groups per level-1 group and l2
+// level-1 groups, AllReduce and Reduce: program (i * l1 + j) * l2 + k is part k of sub-slice j of chunk i;
+// ReduceScatter: program r is rank r's output.  level0 of 1 or rankSize: one level.
+HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, FoldPlan* plan, uint32_t level0 = 1,
+                         uint32_t level1 = 0);
+
+// The sizes of the levels a world of rankSize ranks has under (level0, level1) as above: false when it has one
+// level or the sizes do not divide.  l1 * l2 = rankSize / l0; l2 is 1 in a two-level world.
+struct Levels {
+    uint32_t l0 = 1, l1 = 1, l2 = 1;
+};
+bool ResolveLevels(uint32_t rankSize, uint32_t level0, uint32_t level1, Levels* out);
 
 // Geometry helpers of the recursive halving-doubling family (reference template_utils.cc:42-168).
 uint32_t RhdPairCount(uint32_t p);                    // r = p - 2^floor(log2 p)
@@ -62,5 +72,17 @@ HcclResult RhdMaxCountPerLoop(uint64_t cclBytes, uint64_t count, uint32_t p, uin
 // Elements the next RHD loop takes: whole frames of p while they last, then the remainder below p alone
 // (reference ins_v2_all_reduce_sequence_rhd_tail.h:94-99).
 uint64_t RhdSelectLoopCount(uint64_t remaining, uint64_t maxCountPerLoop, uint64_t p);
+// Loops of the three-level sequence executors (reference ins_v2_all_reduce_sequence_executor_aicpu_3level.cc:524-534,
+// reduce_sequence_executor_aicpu_3level.cc:877-889): the buffer is cut into l0 + 1 slices of whole elements, the
+// first receives the level-0 result, the other l0 the peers' data; a loop holds what those l0 slices take, floored
+// to `align` bytes (128 for AllReduce, 4096 for Reduce), whole elements and a multiple of `total` ranks.  With
+// rhdTail the two tail tiles of RhdMaxCountPerLoop leave the buffer first (count not a multiple of total).
+// resultElems: the elements of the first slice.  HCCL_E_INTERNAL when nothing fits.
+HcclResult SequenceMaxCountPerLoop(uint64_t cclBytes, uint64_t count, uint32_t l0, uint32_t total, uint64_t elemSize,
+                                   uint64_t align, bool rhdTail, uint64_t* maxCount, uint64_t* resultElems);
+// Elements the next loop of those executors takes when the chunks are floor(len / l0) with the rest in the last:
+// a last loop whose last chunk would not fit the result slice gives some elements up to one more loop
+// (reference ins_v2_all_reduce_sequence_executor_aicpu_3level.cc:704-731).  0 when the slice holds no element.
+uint64_t SequenceSelectLoopCount(uint64_t remaining, uint64_t maxCountPerLoop, uint32_t l0, uint64_t resultElems);
 
 }  // namespace hccl_amd

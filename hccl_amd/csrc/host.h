@@ -177,10 +177,13 @@ struct World {
     uint64_t cclBytes = 0;
     // Ranks per level-0 group of the two-level AllReduce (HcclAmdSetLevel0RankSize, HCCL_AMD_LEVEL0_RANKS); 1 = one level.
     uint32_t level0 = 1;
+    // Level-0 groups per level-1 group (HcclAmdSetLevel1GroupSize, HCCL_AMD_LEVEL1_GROUPS); 0 = all of them, two levels.
+    uint32_t level1 = 0;
     // HCCL_ALGO asked for a sequence executor (1), a single-level one (0), or said nothing (-1): with level-0
     // groups, AllReduce runs in two levels unless a single-level executor was asked for.
     int allReduceSequence = -1;
     int reduceScatterSequence = -1;       // the same for ReduceScatter (reducescatter:sequence{mesh..., rhd | nhr | nhr_aicpu_reduce})
+    int reduceSequence = -1;              // and for Reduce (reduce:sequence{mesh..., rhd | nhr | nhr_aicpu_reduce})
     bool envInvalid = false;      // an environment variable of the reference failed its parser
 
     ~World()
@@ -231,7 +234,8 @@ CommRef AsComm(HcclComm h);
 HcclResult CheckUserRank(const Comm* c);
 // The fold programs of (kind, algo) for this world's rank size, uploaded on first use; level0 > 1: the two-level
 // AllReduce over groups of that many ranks.
-HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DevicePlan* out, uint32_t level0 = 1);
+HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DevicePlan* out, uint32_t level0 = 1,
+                         uint32_t level1 = 0);
 HcclResult TakeEvent(World* w, hipEvent_t* ev);
 
 // ---- launch_reduce.cc: `s` is the stream the kernels run on -----------------------------------------

@@ -186,7 +186,8 @@ bool AlgoFitsOp(HcclAmdOpKind kind, HcclAmdAlgo algo)
         case HCCL_AMD_OP_REDUCE_SCATTER:
             return algo != HCCL_AMD_ALGO_MESH_TWO_SHOT;
         case HCCL_AMD_OP_REDUCE:
-            return algo == HCCL_AMD_ALGO_MESH || algo == HCCL_AMD_ALGO_RING || algo == HCCL_AMD_ALGO_MESH_TWO_SHOT;
+            return algo == HCCL_AMD_ALGO_MESH || algo == HCCL_AMD_ALGO_RING || algo == HCCL_AMD_ALGO_MESH_TWO_SHOT ||
+                   algo == HCCL_AMD_ALGO_NHR || algo == HCCL_AMD_ALGO_RHD;
         default:
             return false;
     }
@@ -249,6 +250,8 @@ void ApplyReferenceAlgoEnv(World* w)
                 w->allReduceSequence = sel.twoLevel[op] ? 1 : 0;
             } else if (kind == HCCL_AMD_OP_REDUCE_SCATTER) {
                 w->reduceScatterSequence = sel.twoLevel[op] ? 1 : 0;
+            } else if (kind == HCCL_AMD_OP_REDUCE) {
+                w->reduceSequence = sel.twoLevel[op] ? 1 : 0;
             }
         }
     }
@@ -316,6 +319,13 @@ std::unique_ptr<World> NewWorld(uint32_t n)
         } else {
             Log(1, "HCCL_AMD_LEVEL0_RANKS=%u does not divide the %u ranks of the world: ignored", groups, n);
         }
+        const uint32_t perGroup = EnvU32("HCCL_AMD_LEVEL1_GROUPS", 0);
+        if (perGroup == 0 || (n / w->level0) % perGroup == 0) {
+            w->level1 = perGroup;
+        } else {
+            Log(1, "HCCL_AMD_LEVEL1_GROUPS=%u does not divide the %u level-0 groups of the world: ignored", perGroup,
+                n / w->level0);
+        }
     }
     if (const char* det = getenv("HCCL_DETERMINISTIC")) {
         std::string v(det);
@@ -363,16 +373,17 @@ HcclResult CheckUserRank(const Comm* c)
 // ---------------------------------------------------------------------------------------------
 // Device resources
 // ---------------------------------------------------------------------------------------------
-HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DevicePlan* out, uint32_t level0)
+HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DevicePlan* out, uint32_t level0,
+                         uint32_t level1)
 {
-    uint32_t key = (static_cast<uint32_t>(kind) * 64 + static_cast<uint32_t>(algo)) * 128 + level0;
+    uint32_t key = ((static_cast<uint32_t>(kind) * 64 + static_cast<uint32_t>(algo)) * 128 + level0) * 128 + level1;
     auto it = w->plans.find(key);
     if (it != w->plans.end()) {
         *out = it->second;
         return HCCL_SUCCESS;
     }
     FoldPlan plan;
-    HcclResult rc = BuildFoldPlan(kind, algo, w->n, &plan, level0);
+    HcclResult rc = BuildFoldPlan(kind, algo, w->n, &plan, level0, level1);
     if (rc != HCCL_SUCCESS) {
         return rc;
     }

@@ -276,23 +276,77 @@ HcclResult LaunchToAll(World* w, const ReduceArgs& a, const DevicePlan& plan, Hc
     return HCCL_SUCCESS;
 }
 
+// The cut of the sequence executors whose chunks are floor(len / d) elements with the rest in the last one, level
+// after level (reference ins_v2_all_reduce_sequence_3level_utils.h:124-126, 150-160,
+// ins_v2_all_reduce_sequence_executor_aicpu_3level.cc:361-370): `dims` are the level sizes from level 0 on, program
+// progBase + ((i * d1 + j) * d2 + k) belongs to part k of sub-slice j of chunk i.  launch(program, nSub, begin, len,
+// subLen) receives runs of nSub neighbouring units of subLen elements, the last one longer by what is left of len.
+template <class Launch>
+HcclResult CutByLevels(const uint32_t* dims, uint32_t nDims, uint32_t progBase, uint64_t begin, uint64_t len,
+                       Launch&& launch)
+{
+    if (len == 0) {
+        return HCCL_SUCCESS;
+    }
+    const uint32_t d = dims[0];
+    if (nDims == 1) {
+        const uint64_t sub = len / d;
+        // fewer elements than units: all of them belong to the last unit
+        return sub == 0 ? launch(progBase + d - 1, 1u, begin, len, len) : launch(progBase, d, begin, len, sub);
+    }
+    uint32_t below = 1;
+    for (uint32_t k = 1; k < nDims; ++k) {
+        below *= dims[k];
+    }
+    const uint64_t chunk = len / d;
+    if (chunk != 0 && chunk * d == len && chunk % below == 0) {
+        return launch(progBase, d * below, begin, len, chunk / below);   // every unit equally long: one run
+    }
+    for (uint32_t i = 0; i < d; ++i) {
+        const uint64_t cur = i == d - 1 ? len - static_cast<uint64_t>(i) * chunk : chunk;
+        HcclResult rc = CutByLevels(dims + 1, nDims - 1, progBase + i * below, begin + static_cast<uint64_t>(i) * chunk, cur,
+                                    launch);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// The levels of a world as CutByLevels takes them (a level of one participant cuts nothing and is left out).
+uint32_t LevelDims(const Levels& lv, uint32_t* dims)
+{
+    uint32_t nDims = 0;
+    dims[nDims++] = lv.l0;
+    if (lv.l1 > 1) {
+        dims[nDims++] = lv.l1;
+    }
+    if (lv.l2 > 1) {
+        dims[nDims++] = lv.l2;
+    }
+    return nDims;
+}
+
 HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
     HcclAmdAlgo algo = EffectiveAlgo(w, HCCL_AMD_OP_ALL_REDUCE, p.dtype, p.op);
     // A world with level-0 groups runs the step-driven orders in two levels: a mesh ReduceScatter inside every
     // group, the configured template between the groups (reference
-    // ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852).  The types the reference reduces on the host take its
+    // ins_v2_all_reduce_sequence_executor_aicpu.cc:592-852), and in three when the groups form level-1 groups
+    // (ins_v2_all_reduce_sequence_executor_aicpu_3level.cc).  The types the reference reduces on the host take its
     // host-reduce template between the groups, which folds the own share first (EffectiveAlgo has turned their
-    // RHD / NHR into MESH; a configured sequence{mesh, nhr_aicpu_reduce} asks for the same).
-    const uint32_t level0 = w->level0;
+    // RHD / NHR into MESH; a configured sequence{mesh, nhr_aicpu_reduce} asks for the same); that executor knows
+    // two levels only.
     const HcclAmdAlgo configured = w->algo[HCCL_AMD_OP_ALL_REDUCE];
     const bool stepDriven = configured == HCCL_AMD_ALGO_RHD || configured == HCCL_AMD_ALGO_NHR;
-    const bool twoLevel = level0 > 1 && level0 < n && w->allReduceSequence != 0 &&
+    Levels lv;
+    const bool twoLevel = ResolveLevels(n, w->level0, algo == HCCL_AMD_ALGO_MESH ? 0 : w->level1, &lv) &&
+                          w->allReduceSequence != 0 &&
                           (algo == HCCL_AMD_ALGO_RHD || algo == HCCL_AMD_ALGO_NHR ||
                            (algo == HCCL_AMD_ALGO_MESH && (stepDriven || w->allReduceSequence == 1)));
     DevicePlan plan;
-    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_ALL_REDUCE, algo, &plan, twoLevel ? level0 : 1);
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_ALL_REDUCE, algo, &plan, twoLevel ? lv.l0 : 1, twoLevel ? w->level1 : 0);
     if (rc != HCCL_SUCCESS) {
         return rc;
     }
@@ -408,73 +462,65 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
     };
     if (twoLevel && algo != HCCL_AMD_ALGO_RHD) {
         // Between the groups NHR, or the host-reduce fold: every loop is cut into level0 chunks of floor(len / level0)
-        // elements, the last chunk taking the rest, and every chunk into n / level0 sub-slices the same way (reference
-        // ins_v2_all_reduce_sequence_executor_aicpu.cc:413-415, 445-455).  The loops hold what fits half the staging
-        // buffer, floored to 128 bytes and to a multiple of n elements (:653-656).
-        const uint32_t level1 = n / level0;
+        // elements, the last chunk taking the rest, every chunk into sub-slices the same way and, with three levels,
+        // every sub-slice into parts (reference ins_v2_all_reduce_sequence_executor_aicpu.cc:413-415, 445-455).
+        // Two levels: the loops hold what fits half the staging buffer, floored to 128 bytes and to a multiple of n
+        // elements (:653-656); three: SequenceMaxCountPerLoop.
         uint64_t maxPerLoop = p.count;
+        uint64_t resultElems = ~0ull;
         if (w->cclBytes != 0) {
-            maxPerLoop = w->cclBytes / 2 / 128 * 128 / esz / n * n;
-            if (maxPerLoop == 0) {
-                Log(1, "AllReduce: the staging buffer of %llu bytes holds no loop of the two-level order",
-                    static_cast<unsigned long long>(w->cclBytes));
+            if (lv.l2 > 1) {
+                rc = SequenceMaxCountPerLoop(w->cclBytes, p.count, lv.l0, n, esz, 128, false, &maxPerLoop, &resultElems);
+            } else {
+                maxPerLoop = w->cclBytes / 2 / 128 * 128 / esz / n * n;
+                rc = maxPerLoop == 0 ? HCCL_E_INTERNAL : HCCL_SUCCESS;
+            }
+            if (rc != HCCL_SUCCESS) {
+                Log(1, "AllReduce: the staging buffer of %llu bytes holds no loop of the %s-level order",
+                    static_cast<unsigned long long>(w->cclBytes), lv.l2 > 1 ? "three" : "two");
                 return HCCL_E_INTERNAL;
             }
         }
-        for (uint64_t done = 0; done < p.count;) {
-            const uint64_t len = std::min(p.count - done, maxPerLoop);
-            const uint64_t chunk = len / level0;
-            if (chunk * level0 == len && chunk % level1 == 0 && chunk != 0) {
-                // every sub-slice equally long: one launch over the n units of the loop, unit i * level1 + j being
-                // sub-slice j of chunk i
-                a.nSub = n;
-                a.prog = plan.dev;
-                rc = launchLoop(done, len, chunk / level1);
-                if (rc != HCCL_SUCCESS) {
-                    return rc;
-                }
-                done += len;
-                continue;
+        uint32_t dims[3];
+        const uint32_t nDims = LevelDims(lv, dims);
+        auto launch = [&](uint32_t prog, uint32_t nSub, uint64_t begin, uint64_t len, uint64_t subLen) {
+            for (uint32_t r = 0; r < n; ++r) {
+                a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + begin * esz;
+                a.dst[r] = static_cast<uint8_t*>(p.ranks[r].recv) + begin * esz;
             }
-            a.nSub = level1;
-            for (uint32_t i = 0; i < level0; ++i) {
-                const uint64_t begin = done + static_cast<uint64_t>(i) * chunk;
-                const uint64_t cur = i == level0 - 1 ? len - static_cast<uint64_t>(i) * chunk : chunk;
-                if (cur == 0) {
-                    continue;
-                }
-                for (uint32_t r = 0; r < n; ++r) {
-                    a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + begin * esz;
-                    a.dst[r] = static_cast<uint8_t*>(p.ranks[r].recv) + begin * esz;
-                }
-                a.prog = plan.dev + static_cast<uint64_t>(i) * level1 * kDevProgBytes;
-                a.total = a.groupLen = cur;
-                a.subLen = cur / level1;
-                if (a.subLen == 0) {
-                    // fewer elements than sub-slices: all of them belong to the last sub-slice
-                    a.prog = plan.dev + (static_cast<uint64_t>(i) * level1 + level1 - 1) * kDevProgBytes;
-                    a.nSub = 1;
-                    a.subLen = cur;
-                }
-                rc = LaunchToAll(w, a, plan, p.dtype, p.op, s);
-                a.nSub = level1;
-                if (rc != HCCL_SUCCESS) {
-                    return rc;
-                }
+            a.prog = plan.dev + static_cast<uint64_t>(prog) * kDevProgBytes;
+            a.nSub = nSub;
+            a.total = a.groupLen = len;
+            a.subLen = subLen;
+            return LaunchToAll(w, a, plan, p.dtype, p.op, s);
+        };
+        for (uint64_t done = 0; done < p.count;) {
+            const uint64_t len = lv.l2 > 1 ? SequenceSelectLoopCount(p.count - done, maxPerLoop, lv.l0, resultElems)
+                                           : std::min(p.count - done, maxPerLoop);
+            if (len == 0) {
+                return HCCL_E_INTERNAL;
+            }
+            rc = CutByLevels(dims, nDims, 0, done, len, launch);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
             }
             done += len;
         }
         return HCCL_SUCCESS;
     }
     if (algo == HCCL_AMD_ALGO_RHD) {
-        // (With level-0 groups the frame is the same: unit u = i * (n / level0) + j is sub-slice j of chunk i, and
-        // the remainder shorter than n is padded to one element per unit; only the programs differ.)
+        // (With level-0 groups the frame is the same: unit u = i * (n / level0) + j is sub-slice j of chunk i, with
+        // three levels unit (i * l1 + j) * l2 + k part k of it, and the remainder shorter than n is padded to one
+        // element per unit; only the programs differ, and the share of the buffer a three-level loop may fill.)
         // Whole frames of n uniform units while they last, then a remainder shorter than n with one element per
         // unit (reference ins_v2_all_reduce_sequence_rhd_tail.h:94-113); a bounded staging buffer limits the
         // frames one loop holds.
         uint64_t maxPerLoop = ~0ull / 2 / n * n;
         if (w->cclBytes != 0) {
-            rc = RhdMaxCountPerLoop(w->cclBytes, p.count, n, esz, &maxPerLoop);
+            uint64_t resultElems = 0;
+            rc = twoLevel && lv.l2 > 1
+                     ? SequenceMaxCountPerLoop(w->cclBytes, p.count, lv.l0, n, esz, 128, true, &maxPerLoop, &resultElems)
+                     : RhdMaxCountPerLoop(w->cclBytes, p.count, n, esz, &maxPerLoop);
             if (rc != HCCL_SUCCESS) {
                 Log(1, "AllReduce: the staging buffer of %llu bytes holds no loop of the RHD order",
                     static_cast<unsigned long long>(w->cclBytes));
@@ -524,18 +570,21 @@ HcclResult RunReduceScatter(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
     HcclAmdAlgo algo = EffectiveAlgo(w, HCCL_AMD_OP_REDUCE_SCATTER, p.dtype, p.op);
-    // A world with level-0 groups runs the step-driven orders in two levels, as AllReduce does (reference
-    // ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-372): the mesh ReduceScatter inside every group, the
-    // configured template between the groups, the own-first host-reduce fold there for the types the reference
-    // reduces on the host.  Every rank's output keeps one program, so the launch is the one-level one.
-    const uint32_t level0 = w->level0;
+    // A world with level-0 groups runs the step-driven orders in two or three levels, as AllReduce does (reference
+    // ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-372, ins_v2_reduce_scatter_sequence_executor_3level.cc):
+    // the mesh ReduceScatter inside every group, the configured template between the groups, the own-first host-reduce
+    // fold there for the types the reference reduces on the host.  Every rank's output keeps one program, so the
+    // launch is the one-level one.
     const HcclAmdAlgo configured = w->algo[HCCL_AMD_OP_REDUCE_SCATTER];
     const bool stepDriven = configured == HCCL_AMD_ALGO_RHD || configured == HCCL_AMD_ALGO_NHR;
-    const bool twoLevel = level0 > 1 && level0 < n && w->reduceScatterSequence != 0 &&
+    Levels lv;
+    const bool twoLevel = ResolveLevels(n, w->level0, algo == HCCL_AMD_ALGO_MESH ? 0 : w->level1, &lv) &&
+                          w->reduceScatterSequence != 0 &&
                           (algo == HCCL_AMD_ALGO_RHD || algo == HCCL_AMD_ALGO_NHR ||
                            (algo == HCCL_AMD_ALGO_MESH && (stepDriven || w->reduceScatterSequence == 1)));
     DevicePlan plan;
-    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, algo, &plan, twoLevel ? level0 : 1);
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE_SCATTER, algo, &plan, twoLevel ? lv.l0 : 1,
+                                  twoLevel ? w->level1 : 0);
     if (rc != HCCL_SUCCESS) {
         return rc;
     }
@@ -672,17 +721,81 @@ HcclResult RunReduceScatterV(World* w, PendingOp& p, hipStream_t s)
 // the AllReduce rank-order program with the root's recvBuf as only destination.  MESH_TWO_SHOT: every loop of the
 // executor deals its elements into N slices, the first len mod N one element longer, and slice k folds rank k's
 // input first (reference reduce_mesh_1D_two_shot.cc:138-162, 228-265; N staging slots, :79-84,
-// reduce_sole_executor.cc:178-232).
+// reduce_sole_executor.cc:178-232).  NHR: slices of ceil(len / N) elements, short or empty towards the end, each
+// folded along the NHR step tree (reference reduce_nhr.cc:202-226, 263-339; one staging slot, :131-136).  A world
+// with level-0 groups runs RHD, NHR and, for the types the reference reduces on the host, the host-reduce fold as the
+// AllReduce sequence does, with the root as only destination (reference reduce_sequence_executor_aicpu_3level.cc:
+// 744-990): chunks, sub-slices and parts of floor(len / d) elements with the rest in the last, for RHD too.
 HcclResult RunReduce(World* w, PendingOp& p, hipStream_t s)
 {
     const uint32_t n = w->n;
     if (p.ranks[p.root].recv == nullptr) {
         return HCCL_E_PTR;
     }
-    const bool twoShot = w->algo[HCCL_AMD_OP_REDUCE] == HCCL_AMD_ALGO_MESH_TWO_SHOT;
+    const uint32_t esz = DataTypeSize(p.dtype);
+    const HcclAmdAlgo configured = w->algo[HCCL_AMD_OP_REDUCE];
+    const bool stepDriven = configured == HCCL_AMD_ALGO_RHD || configured == HCCL_AMD_ALGO_NHR;
+    HcclAmdAlgo algo = EffectiveAlgo(w, HCCL_AMD_OP_REDUCE, p.dtype, p.op);
+    Levels lv;
+    const bool levels = ResolveLevels(n, w->level0, algo == HCCL_AMD_ALGO_MESH ? 0 : w->level1, &lv) &&
+                        w->reduceSequence != 0 &&
+                        (algo == HCCL_AMD_ALGO_RHD || algo == HCCL_AMD_ALGO_NHR ||
+                         (algo == HCCL_AMD_ALGO_MESH && (stepDriven || w->reduceSequence == 1)));
+    if (levels) {
+        DevicePlan plan;
+        HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE, algo, &plan, lv.l0, w->level1);
+        if (rc != HCCL_SUCCESS) {
+            return rc;
+        }
+        uint64_t maxPerLoop = p.count;
+        uint64_t resultElems = ~0ull;
+        if (w->cclBytes != 0) {
+            rc = SequenceMaxCountPerLoop(w->cclBytes, p.count, lv.l0, n, esz, 4096, false, &maxPerLoop, &resultElems);
+            if (rc != HCCL_SUCCESS) {
+                Log(1, "Reduce: the staging buffer of %llu bytes holds no loop of the sequence order",
+                    static_cast<unsigned long long>(w->cclBytes));
+                return rc;
+            }
+        }
+        ReduceArgs a{};
+        a.nDst = 1;
+        a.dstOwn = 0;
+        a.nGroup = 1;
+        a.progSubStride = 1;
+        uint32_t dims[3];
+        const uint32_t nDims = LevelDims(lv, dims);
+        auto launch = [&](uint32_t prog, uint32_t nSub, uint64_t begin, uint64_t len, uint64_t subLen) {
+            for (uint32_t r = 0; r < n; ++r) {
+                a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + begin * esz;
+            }
+            a.dst[0] = static_cast<uint8_t*>(p.ranks[p.root].recv) + begin * esz;
+            a.prog = plan.dev + static_cast<uint64_t>(prog) * kDevProgBytes;
+            a.nSub = nSub;
+            a.total = a.groupLen = len;
+            a.subLen = subLen;
+            return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+        };
+        for (uint64_t done = 0; done < p.count;) {
+            const uint64_t len = SequenceSelectLoopCount(p.count - done, maxPerLoop, lv.l0, resultElems);
+            if (len == 0) {
+                return HCCL_E_INTERNAL;
+            }
+            rc = CutByLevels(dims, nDims, 0, done, len, launch);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+            done += len;
+        }
+        return HCCL_SUCCESS;
+    }
+    if (algo == HCCL_AMD_ALGO_RHD) {
+        algo = HCCL_AMD_ALGO_MESH;   // the reference has no single-level RHD Reduce: its selection falls back
+    }
+    const bool twoShot = algo == HCCL_AMD_ALGO_MESH_TWO_SHOT;
+    const bool nhr = algo == HCCL_AMD_ALGO_NHR;
     DevicePlan plan;
-    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE, twoShot ? HCCL_AMD_ALGO_MESH_TWO_SHOT : HCCL_AMD_ALGO_MESH,
-                                  &plan);
+    HcclResult rc = GetDevicePlan(w, HCCL_AMD_OP_REDUCE,
+                                  twoShot ? HCCL_AMD_ALGO_MESH_TWO_SHOT : nhr ? HCCL_AMD_ALGO_NHR : HCCL_AMD_ALGO_MESH, &plan);
     if (rc != HCCL_SUCCESS) {
         return rc;
     }
@@ -695,15 +808,14 @@ HcclResult RunReduce(World* w, PendingOp& p, hipStream_t s)
     a.nDst = 1;
     a.dstOwn = 0;
     a.nGroup = 1;
-    if (!twoShot) {
+    if (!twoShot && !nhr) {
         a.nSub = 1;
         a.total = a.groupLen = a.subLen = p.count;
         return LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
     }
-    const uint32_t esz = DataTypeSize(p.dtype);
     uint64_t maxPerLoop = p.count;
     if (w->cclBytes != 0) {
-        maxPerLoop = SoleMaxCountPerLoop(w->cclBytes, n, esz);
+        maxPerLoop = SoleMaxCountPerLoop(w->cclBytes, nhr ? 1 : n, esz);
         if (maxPerLoop == 0) {
             return HCCL_E_INTERNAL;
         }
@@ -711,6 +823,33 @@ HcclResult RunReduce(World* w, PendingOp& p, hipStream_t s)
     a.progSubStride = 1;
     for (uint64_t done = 0; done < p.count;) {
         const uint64_t len = std::min(p.count - done, maxPerLoop);
+        if (nhr) {
+            // nFull slices of ceil(len / n) elements, then one shorter slice if elements are left
+            const uint64_t slice = (len + n - 1) / n;
+            const uint32_t nFull = static_cast<uint32_t>(len / slice);
+            const uint64_t rest = len - static_cast<uint64_t>(nFull) * slice;
+            for (int run = 0; run < 2; ++run) {
+                const uint32_t slices = run == 0 ? nFull : (rest != 0 ? 1u : 0u);
+                if (slices == 0) {
+                    continue;
+                }
+                const uint64_t at = (done + (run == 0 ? 0 : static_cast<uint64_t>(nFull) * slice)) * esz;
+                for (uint32_t r = 0; r < n; ++r) {
+                    a.src[r] = static_cast<const uint8_t*>(p.ranks[r].send) + at;
+                }
+                a.dst[0] = static_cast<uint8_t*>(p.ranks[p.root].recv) + at;
+                a.prog = plan.dev + static_cast<uint64_t>(run == 0 ? 0 : nFull) * kDevProgBytes;
+                a.nSub = slices;
+                a.subLen = run == 0 ? slice : rest;
+                a.total = a.groupLen = run == 0 ? slice * nFull : rest;
+                rc = LaunchOneReduce(w, a, plan, p.dtype, p.op, s);
+                if (rc != HCCL_SUCCESS) {
+                    return rc;
+                }
+            }
+            done += len;
+            continue;
+        }
         const uint64_t base = len / n;
         const uint32_t nBig = static_cast<uint32_t>(len % n);
         // two runs of equally long slices: nBig of base + 1 elements, then n - nBig of base

@@ -305,12 +305,18 @@ HcclResult HcclAmdGetStuckCounters(HcclComm comm, uint64_t* head, uint64_t* tail
 HcclResult HcclAmdGetFoldProgram(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t segment,
                                  uint8_t* out, uint32_t cap, uint32_t* len, uint32_t* segmentCount);
 /* The same for the two-level orders over groups of `level0` consecutive ranks (see HcclAmdSetLevel0RankSize).
- * AllReduce: segment i * (rankSize / level0) + j is sub-slice j of chunk i; ReduceScatter: segment r is rank r's
- * output.  algo is the template between the groups (RHD, NHR, or MESH for the own-first fold of the host-reduce
- * template).  level0 of 1 or rankSize: HcclAmdGetFoldProgram. */
+ * AllReduce and Reduce: segment i * (rankSize / level0) + j is sub-slice j of chunk i; ReduceScatter: segment r is
+ * rank r's output.  algo is the template between the groups (RHD, NHR, or MESH for the own-first fold of the
+ * host-reduce template).  level0 of 1 or rankSize: HcclAmdGetFoldProgram. */
 HcclResult HcclAmdGetFoldProgramTwoLevel(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t level0,
                                          uint32_t segment, uint8_t* out, uint32_t cap, uint32_t* len,
                                          uint32_t* segmentCount);
+/* And for three levels: `level1` consecutive groups form a level-1 group (see HcclAmdSetLevel1GroupSize), l2 =
+ * rankSize / level0 / level1 of them.  AllReduce and Reduce: segment (i * level1 + j) * l2 + k is part k of
+ * sub-slice j of chunk i; ReduceScatter: segment r is rank r's output.  level1 of 0: the two-level orders. */
+HcclResult HcclAmdGetFoldProgramLevels(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t rankSize, uint32_t level0,
+                                       uint32_t level1, uint32_t segment, uint8_t* out, uint32_t cap, uint32_t* len,
+                                       uint32_t* segmentCount);
 
 /*
  * Level-0 groups.  The reference runs AllReduce over a two-level topology (servers of several ranks) as a
@@ -322,11 +328,23 @@ HcclResult HcclAmdGetFoldProgramTwoLevel(HcclAmdOpKind op, HcclAmdAlgo algo, uin
  * ins_v2_reduce_scatter_sequence_executor_aicpu.cc:298-500, registrations :567-640).  Where its topology
  * comes from a rank table, a loopback world is told: `ranksPerGroup` consecutive ranks form a group (it must
  * divide the rank size; 1, the default, and the rank size itself mean one level).  Also HCCL_AMD_LEVEL0_RANKS at
- * world creation.  With groups, AllReduce and ReduceScatter under RHD and NHR fold in the two-level order; the other
- * orders and the other operators (ReduceScatterV included) are not affected.
+ * world creation.  With groups, AllReduce, ReduceScatter and Reduce under RHD and NHR fold in the two-level order
+ * (Reduce: src/ops/reduce/algorithm/executor/reduce_sequence_executor_aicpu_3level.cc:744-990, registrations
+ * :995-1048); the other orders and the other operators (ReduceScatterV included) are not affected.
  */
 HcclResult HcclAmdSetLevel0RankSize(HcclComm comm, uint32_t ranksPerGroup);
 HcclResult HcclAmdGetLevel0RankSize(HcclComm comm, uint32_t* ranksPerGroup);
+/*
+ * Level-1 groups.  Over a three-level topology (servers in pods) the reference adds a step: the template runs
+ * between the servers of a pod and once more between the pods (ins_v2_all_reduce_sequence_executor_aicpu_3level.cc:
+ * 536-800, ins_v2_reduce_scatter_sequence_executor_3level.cc:243-256, reduce_sequence_executor_aicpu_3level.cc;
+ * registered as Sequence MeshConcur NHR NHR and ... RHD RHD).  `groupsPerLevel1Group` consecutive level-0 groups
+ * form a level-1 group; it must divide the number of level-0 groups; 0, the default, and that number itself mean
+ * two levels.  Also HCCL_AMD_LEVEL1_GROUPS at world creation.  The host-reduce fold of PROD and the 64-bit types
+ * knows two levels in the reference and keeps them here: every level-0 group of the world is its peer.
+ */
+HcclResult HcclAmdSetLevel1GroupSize(HcclComm comm, uint32_t groupsPerLevel1Group);
+HcclResult HcclAmdGetLevel1GroupSize(HcclComm comm, uint32_t* groupsPerLevel1Group);
 
 /*
  * The reference's HCCL_ALGO setting ("allreduce:sequence{level0=mesh_concur,level1=rhd};reducescatter:nhr;..."; grammar

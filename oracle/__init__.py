@@ -289,6 +289,47 @@ def reduce_scatter_two_level(ins, outs, recv_count, dtype, op, level0, level1_al
                                               _ptr_array(outs), ctypes.c_uint64(recv_count), dtype, op, acc)
 
 
+def all_reduce_three_level(ins, outs, count, dtype, op, level0, level1, algo, acc=ACC_FP32, ccl_bytes=0):
+    """AllReduce over boxes of `level0` consecutive ranks and pods of `level1` consecutive boxes; algo "rhd" or "nhr"
+    between the boxes of a pod and between the pods; ccl_bytes: the staging buffer whose loops show, 0 = one loop."""
+    code = {"rhd": L1_RHD, "nhr": L1_NHR}[algo]
+    return lib().orc_all_reduce_three_level(ctypes.c_uint32(len(ins)), ctypes.c_uint32(level0), ctypes.c_uint32(level1),
+                                            code, _ptr_array(ins), _ptr_array(outs), ctypes.c_uint64(count), dtype, op,
+                                            acc, ctypes.c_uint64(ccl_bytes))
+
+
+def reduce_scatter_three_level(ins, outs, recv_count, dtype, op, level0, level1, algo, acc=ACC_FP32):
+    code = {"rhd": L1_RHD, "nhr": L1_NHR}[algo]
+    return lib().orc_reduce_scatter_three_level(ctypes.c_uint32(len(ins)), ctypes.c_uint32(level0),
+                                                ctypes.c_uint32(level1), code, _ptr_array(ins), _ptr_array(outs),
+                                                ctypes.c_uint64(recv_count), dtype, op, acc)
+
+
+def reduce_levels(ins, outs, count, dtype, op, root, level0, level1, algo, acc=ACC_FP32, ccl_bytes=0):
+    """Reduce over two (level1 = number of boxes) or three levels; algo "rhd", "nhr", or with two levels "mesh" (the
+    host-reduce fold).  Only outs[root] is written."""
+    code = {"rhd": L1_RHD, "nhr": L1_NHR, "mesh": L1_MESH}[algo]
+    return lib().orc_reduce_levels(ctypes.c_uint32(len(ins)), ctypes.c_uint32(level0), ctypes.c_uint32(level1), code,
+                                   _ptr_array(ins), _ptr_array(outs), ctypes.c_uint64(count), dtype, op,
+                                   ctypes.c_uint32(root), acc, ctypes.c_uint64(ccl_bytes))
+
+
+def sequence_max_count_per_loop(ccl_bytes, count, level0, total, esz, align, rhd_tail):
+    """(elements per loop, elements of the result slice) of the three-level sequence executors; None when nothing fits."""
+    m, e = ctypes.c_uint64(), ctypes.c_uint64()
+    rc = lib().orc_sequence_max_count_per_loop(ctypes.c_uint64(ccl_bytes), ctypes.c_uint64(count),
+                                               ctypes.c_uint32(level0), ctypes.c_uint32(total), ctypes.c_uint64(esz),
+                                               ctypes.c_uint64(align), int(rhd_tail), ctypes.byref(m), ctypes.byref(e))
+    return (m.value, e.value) if rc == 0 else None
+
+
+def sequence_select_loop_count(remaining, max_count_per_loop, level0, result_elems):
+    f = lib().orc_sequence_select_loop_count
+    f.restype = ctypes.c_uint64
+    return f(ctypes.c_uint64(remaining), ctypes.c_uint64(max_count_per_loop), ctypes.c_uint32(level0),
+             ctypes.c_uint64(result_elems))
+
+
 def reduce_scatter(ins, outs, recv_count, dtype, op, acc=ACC_FP32, algo="mesh", max_count_per_loop=0):
     if algo == "mesh_chunk":
         return _reduce_call("orc_reduce_scatter_mesh_chunk", ins, outs, recv_count, dtype, op, acc,
@@ -361,6 +402,10 @@ def reduce(ins, outs, count, dtype, op, root, acc=ACC_FP32, algo="mesh", max_cou
         return lib().orc_reduce_two_shot(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs),
                                          ctypes.c_uint64(count), dtype, op, acc, ctypes.c_uint32(root),
                                          ctypes.c_uint64(max_count_per_loop))
+    if algo == "nhr":
+        return lib().orc_reduce_nhr(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs),
+                                    ctypes.c_uint64(count), dtype, op, acc, ctypes.c_uint32(root),
+                                    ctypes.c_uint64(max_count_per_loop))
     return lib().orc_reduce_mesh(ctypes.c_uint32(len(ins)), _ptr_array(ins), _ptr_array(outs),
                                  ctypes.c_uint64(count), dtype, op, acc, ctypes.c_uint32(root))
 

@@ -991,6 +991,54 @@ int orc_all_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint
     return orc_all_reduce_nhr_looped(n, in, out, count, dtype, op, accMode, 0);
 }
 
+/* Reduce under ReduceNHR (src/ops/reduce/algorithm/template/aicpu/reduce_nhr.cc): slices of ceil(len / n)
+ * elements, short or empty towards the end (CalcSlice :202-226), each folded along the NHR ReduceScatter step tree
+ * (GetStepInfoList :481-519, RunReduce :263-339) and gathered at the root (:341-414); one staging slot
+ * (CalcScratchMultiple :131-136), so the executor's loops hold maxCountPerLoop elements (reduce_sole_executor.cc:
+ * 178-232; 0 = one loop).  Only out[root] is written. */
+int orc_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op, int accMode,
+                   uint32_t root, uint64_t maxCountPerLoop)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (root >= n) {
+        return ORC_E_PARA;
+    }
+    if (maxCountPerLoop == 0) {
+        maxCountPerLoop = count;
+    }
+    for (uint64_t done = 0; done < count && rc == ORC_OK;) {
+        uint64_t len = count - done < maxCountPerLoop ? count - done : maxCountPerLoop;
+        uint64_t slice = (len + n - 1) / n;
+        scratch_t sc;
+        if (scratch_alloc(&sc, n, slice, r.asz) != ORC_OK) {
+            return ORC_E_INTERNAL;
+        }
+        memset(sc.mem, 0, (uint64_t)n * n * slice * r.asz);
+        for (uint32_t m = 0; m < n; ++m) {
+            uint64_t off = 0;
+            for (uint32_t i = 0; i < n; ++i) {
+                uint64_t cur = len - off < slice ? len - off : slice;
+                red_widen(&r, cbytes(in[m]) + (done + off) * r.esz, scratch_at(&sc, m, i), cur);
+                off += cur;
+            }
+        }
+        rc = nhr_reduce_scatter_scratch(&r, &sc);
+        uint64_t off = 0;
+        for (uint32_t i = 0; i < n && rc == ORC_OK; ++i) {
+            uint64_t cur = len - off < slice ? len - off : slice;
+            red_narrow(&r, scratch_at(&sc, i, i), bytes(out[root]) + (done + off) * r.esz, cur);
+            off += cur;
+        }
+        free(sc.mem);
+        done += len;
+    }
+    return rc;
+}
+
 /* ---- staging-buffer loop limits ----------------------------------------------------------------
  * hccl_op_utils.cc:204-225: HCCL_BUFFSIZE in MB (default 200, at least 2, at most UINT32_MAX, digits only),
  * less 1 MiB that is kept back. */
@@ -1579,6 +1627,431 @@ int orc_all_reduce_two_level(uint32_t n, uint32_t l0, int l1Algo, const void* co
     free(src);
     free(dst);
     return rc;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Three levels (ins_v2_all_reduce_sequence_executor_aicpu_3level.cc, "3level.cc" below;
+ * ins_v2_reduce_scatter_sequence_executor_3level.cc; reduce_sequence_executor_aicpu_3level.cc).  l0 consecutive
+ * ranks form a box, l1 consecutive boxes a pod, l2 = n / (l0 * l1) pods: rank (g * l1 + b) * l0 + i is member i
+ * of box b of pod g; between the boxes it talks to the members i of the boxes of its pod (3level.cc:209-216,
+ * infos[1]), between the pods to the members i of the boxes b of the other pods (infos[2]).  Per loop of AllReduce
+ * (3level.cc:586-693, 733-795):
+ *   RSL0  mesh ReduceScatter inside every box: member i ends with chunk i, its own input first
+ *   RSL1  the template between the boxes of a pod on chunk i cut into l1 sub-slices: box b ends with sub-slice b
+ *   RSL2  the template between the pods on that sub-slice cut into l2 parts: pod g ends with part g
+ *   AGL2, AGL1, AGL0  the AllGathers back.
+ * Templates (registrations 3level.cc:806-838): NHR at both levels, or RHD at both; RSL1 keeps its POST (which
+ * moves shares and folds nothing), RSL2 skips it and the representative's merged share is bridged (:622-660).
+ * Cuts: NHR floor(len / d) with the rest in the last chunk / sub-slice / part (3level_utils.h:124-126, 150-160,
+ * 3level.cc:361-370); RHD uniform units on the prefix aligned to n, the remainder staged into a padded tile
+ * (rhd_tail.h:94-165).
+ * The folds of a level run in the accumulation domain; a value is narrowed once, at the end.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+    const red_t* r;
+    uint32_t l0, l1, l2;
+    int algo;                  /* ORC_L1_RHD or ORC_L1_NHR; ORC_L1_MESH with one pod */
+    const uint8_t* const* src; /* n inputs (or staged tiles) */
+    void* tmp;
+} levels_t;
+
+/* RSL0 + RSL1 for member i inside pod g on elements [off, off + (l1 - 1) * unit + last): vals[b] receives the
+ * value box b ends with for sub-slice b (unit elements, `last` for the last box), in the accumulation domain. */
+static int pod_reduce_scatter(const levels_t* lv, uint32_t g, uint32_t i, uint64_t off, uint64_t unit,
+                              uint64_t last, uint8_t* const* vals)
+{
+    const red_t* r = lv->r;
+    uint32_t l1 = lv->l1;
+    uint64_t slot = last > unit ? last : unit;
+    if (slot == 0) {
+        return ORC_OK;
+    }
+    scratch_t sc;
+    if (scratch_alloc(&sc, l1, slot, r->asz) != ORC_OK) {
+        return ORC_E_INTERNAL;
+    }
+    memset(sc.mem, 0, (uint64_t)l1 * l1 * slot * r->asz);
+    for (uint32_t b = 0; b < l1; ++b) {
+        for (uint32_t j = 0; j < l1; ++j) {
+            uint64_t cur = j == l1 - 1 ? last : unit;
+            uint32_t at = lv->algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l1, j) : j;
+            level0_fold(r, lv->l0, g * l1 + b, i, lv->src, off + (uint64_t)j * unit, cur, scratch_at(&sc, b, at), lv->tmp);
+        }
+    }
+    int rc = ORC_OK;
+    if (lv->algo == ORC_L1_MESH) {
+        /* the host-reduce template: box j folds the other boxes' shares of unit j ascending into its own
+         * (reduce_scatter_aicpu_reduce_nhr_pcie.cc:212-280) */
+        for (uint32_t j = 0; j < l1; ++j) {
+            for (uint32_t b = 0; b < l1; ++b) {
+                if (b != j) {
+                    red_pair(r, scratch_at(&sc, j, j), scratch_at(&sc, b, j), j == l1 - 1 ? last : unit);
+                }
+            }
+        }
+    } else {
+        rc = lv->algo == ORC_L1_RHD ? rhd_rs_frame(r, &sc, 0) : nhr_reduce_scatter_scratch(r, &sc);
+    }
+    for (uint32_t j = 0; j < l1 && rc == ORC_OK; ++j) {
+        uint64_t cur = j == l1 - 1 ? last : unit;
+        uint32_t at = lv->algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l1, j) : j;
+        memcpy(vals[j], scratch_at(&sc, j, at), cur * r->asz);
+    }
+    free(sc.mem);
+    return rc;
+}
+
+/* RSL2 between the pods on one sub-slice: share[g] is what pod g holds for it (accumulation domain), cut into
+ * l2 parts of `unit` elements (`last` for the last pod's); part k's final value goes, narrowed, to out + k * unit. */
+static int pods_reduce_scatter(const levels_t* lv, uint8_t* const* share, uint64_t unit, uint64_t last, uint8_t* out)
+{
+    const red_t* r = lv->r;
+    uint32_t l2 = lv->l2;
+    uint64_t slot = last > unit ? last : unit;
+    if (slot == 0) {
+        return ORC_OK;
+    }
+    scratch_t sc;
+    if (scratch_alloc(&sc, l2, slot, r->asz) != ORC_OK) {
+        return ORC_E_INTERNAL;
+    }
+    memset(sc.mem, 0, (uint64_t)l2 * l2 * slot * r->asz);
+    for (uint32_t g = 0; g < l2; ++g) {
+        for (uint32_t k = 0; k < l2; ++k) {
+            uint64_t cur = k == l2 - 1 ? last : unit;
+            uint32_t at = lv->algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l2, k) : k;
+            memcpy(scratch_at(&sc, g, at), share[g] + (uint64_t)k * unit * r->asz, cur * r->asz);
+        }
+    }
+    int rc;
+    if (lv->algo == ORC_L1_RHD) {
+        /* POST skipped: a merged pod's share stays in its representative's slot 2t + 1 and is bridged to the
+         * owner slot of the AllGather grid (rhd_tail.h:33-53); the AllGather only moves data */
+        rc = rhd_rs_frame(r, &sc, 1);
+        for (uint32_t k = 0; k < l2 && rc == ORC_OK; ++k) {
+            orc_rhd_part1_t info;
+            orc_rhd_part1(l2, k, ORC_INVALID_RANK, &info);
+            const uint8_t* from;
+            if (info.inPart1 && !info.isRepresentative) {
+                orc_rhd_part1_t rep;
+                orc_rhd_part1(l2, info.pairedAlgRank, ORC_INVALID_RANK, &rep);
+                from = scratch_at(&sc, info.pairedAlgRank, rep.unitStart + 1);
+            } else {
+                from = scratch_at(&sc, k, orc_rhd_unit_start_of_rank(l2, k));
+            }
+            red_narrow(r, from, out + (uint64_t)k * unit * r->esz, k == l2 - 1 ? last : unit);
+        }
+    } else {
+        rc = nhr_reduce_scatter_scratch(r, &sc);
+        for (uint32_t k = 0; k < l2 && rc == ORC_OK; ++k) {
+            red_narrow(r, scratch_at(&sc, k, k), out + (uint64_t)k * unit * r->esz, k == l2 - 1 ? last : unit);
+        }
+    }
+    free(sc.mem);
+    return rc;
+}
+
+/* One loop of `cur` elements from element `off` of lv->src into out + off (every rank ends with the same bytes);
+ * uniform: every cut is exact (RHD), else floor with the rest in the last. */
+static int levels_all_reduce_loop(const levels_t* lv, uint64_t off, uint64_t cur, int uniform, uint8_t* out,
+                                  uint64_t outOff)
+{
+    const red_t* r = lv->r;
+    uint32_t l0 = lv->l0, l1 = lv->l1, l2 = lv->l2;
+    uint64_t chunk = cur / l0;
+    uint64_t longest = cur - chunk * (l0 - 1);
+    uint8_t** vals = (uint8_t**)calloc((size_t)l1 * l2, sizeof(uint8_t*));
+    uint8_t** share = (uint8_t**)calloc(l2, sizeof(uint8_t*));
+    int rc = vals && share ? ORC_OK : ORC_E_INTERNAL;
+    for (uint32_t x = 0; x < l1 * l2 && rc == ORC_OK; ++x) {
+        vals[x] = (uint8_t*)malloc((longest ? longest : 1) * r->asz);
+        if (!vals[x]) {
+            rc = ORC_E_INTERNAL;
+        }
+    }
+    for (uint32_t i = 0; i < l0 && rc == ORC_OK; ++i) {
+        uint64_t cLen = (i == l0 - 1 && !uniform) ? cur - (uint64_t)i * chunk : chunk;
+        uint64_t cOff = (uint64_t)i * chunk;
+        uint64_t sub = cLen / l1;
+        uint64_t subLast = uniform ? sub : cLen - sub * (l1 - 1);
+        for (uint32_t g = 0; g < l2 && rc == ORC_OK; ++g) {
+            rc = pod_reduce_scatter(lv, g, i, off + cOff, sub, subLast, vals + (size_t)g * l1);
+        }
+        for (uint32_t j = 0; j < l1 && rc == ORC_OK; ++j) {
+            uint64_t sLen = j == l1 - 1 ? subLast : sub;
+            uint64_t part = sLen / l2;
+            uint64_t partLast = uniform ? part : sLen - part * (l2 - 1);
+            for (uint32_t g = 0; g < l2; ++g) {
+                share[g] = vals[(size_t)g * l1 + j];
+            }
+            rc = pods_reduce_scatter(lv, share, part, partLast, out + (outOff + cOff + (uint64_t)j * sub) * r->esz);
+        }
+    }
+    for (uint32_t x = 0; vals && x < l1 * l2; ++x) {
+        free(vals[x]);
+    }
+    free(vals);
+    free(share);
+    return rc;
+}
+
+static int levels_check(uint32_t n, uint32_t l0, uint32_t l1, int algo)
+{
+    if (l0 == 0 || l1 == 0 || n % l0 != 0 || (n / l0) % l1 != 0 || algo < ORC_L1_RHD || algo > ORC_L1_MESH) {
+        return ORC_E_PARA;
+    }
+    /* the host-reduce executors know two levels */
+    return algo == ORC_L1_MESH && l1 != n / l0 ? ORC_E_PARA : ORC_OK;
+}
+
+int orc_all_reduce_three_level(uint32_t n, uint32_t l0, uint32_t l1, int algo, const void* const* in,
+                               void* const* out, uint64_t count, int dtype, int op, int accMode, uint64_t cclBytes)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (levels_check(n, l0, l1, algo) != ORC_OK || algo == ORC_L1_MESH) {
+        return ORC_E_PARA;
+    }
+    if (count == 0) {
+        return ORC_OK;
+    }
+    uint64_t maxPerLoop = UINT64_MAX / 2 / n * n, resultElems = UINT64_MAX;
+    if (cclBytes != 0) {
+        rc = orc_sequence_max_count_per_loop(cclBytes, count, l0, n, r.esz, 128, algo == ORC_L1_RHD, &maxPerLoop,
+                                             &resultElems);
+        if (rc != ORC_OK) {
+            return rc;
+        }
+    }
+    levels_t lv = {&r, l0, l1, n / l0 / l1, algo, NULL, NULL};
+    const uint8_t** src = (const uint8_t**)malloc(sizeof(uint8_t*) * n);
+    uint8_t* tiles = (uint8_t*)malloc((size_t)n * n * r.esz);
+    uint8_t* tileOut = (uint8_t*)malloc((size_t)n * r.esz);
+    uint8_t* result = (uint8_t*)malloc(count * r.esz);
+    lv.tmp = malloc(count * r.asz);
+    lv.src = src;
+    if (!src || !tiles || !tileOut || !result || !lv.tmp) {
+        rc = ORC_E_INTERNAL;
+    }
+    uint64_t processed = 0;
+    while (processed < count && rc == ORC_OK) {
+        uint64_t remaining = count - processed;
+        for (uint32_t j = 0; j < n; ++j) {
+            src[j] = cbytes(in[j]);
+        }
+        if (algo == ORC_L1_RHD) {
+            uint64_t valid = orc_rhd_select_loop_count(remaining, maxPerLoop, n);
+            if (valid >= n) {
+                rc = levels_all_reduce_loop(&lv, processed, valid, 1, result, processed);
+            } else {
+                /* rhd_tail.h:115-146: the valid elements staged and doubled up to a tile of n; only they come back */
+                for (uint32_t j = 0; j < n; ++j) {
+                    uint8_t* t = tiles + (size_t)j * n * r.esz;
+                    memcpy(t, cbytes(in[j]) + processed * r.esz, valid * r.esz);
+                    uint64_t filled = valid;
+                    while (filled < n) {
+                        uint64_t c = filled < n - filled ? filled : n - filled;
+                        memcpy(t + filled * r.esz, t, c * r.esz);
+                        filled += c;
+                    }
+                    src[j] = t;
+                }
+                rc = levels_all_reduce_loop(&lv, 0, n, 1, tileOut, 0);
+                memcpy(result + processed * r.esz, tileOut, valid * r.esz);
+            }
+            processed += valid;
+        } else {
+            uint64_t cur = orc_sequence_select_loop_count(remaining, maxPerLoop, l0, resultElems);
+            if (cur == 0) {
+                rc = ORC_E_INTERNAL;
+                break;
+            }
+            rc = levels_all_reduce_loop(&lv, processed, cur, 0, result, processed);
+            processed += cur;
+        }
+    }
+    for (uint32_t j = 0; j < n && rc == ORC_OK; ++j) {
+        memcpy(out[j], result, count * r.esz);
+    }
+    free(src);
+    free(tiles);
+    free(tileOut);
+    free(result);
+    free(lv.tmp);
+    return rc;
+}
+
+/* Reduce over two or three levels (reduce_sequence_executor_aicpu_3level.cc:744-990): the steps of the AllReduce
+ * with the root's output as the only destination of the last AllGather, the cuts floor(len / d) with the rest in
+ * the last for both templates (GenTempAlgParamsRSL0 / RSL1 / RSL2, :444-560), loops of
+ * orc_sequence_max_count_per_loop with 4096-byte alignment (:877-889).  l1 = n / l0 makes it the two-level form. */
+int orc_reduce_levels(uint32_t n, uint32_t l0, uint32_t l1, int algo, const void* const* in, void* const* out,
+                      uint64_t count, int dtype, int op, uint32_t root, int accMode, uint64_t cclBytes)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (levels_check(n, l0, l1, algo) != ORC_OK || root >= n) {
+        return ORC_E_PARA;
+    }
+    if (count == 0) {
+        return ORC_OK;
+    }
+    uint64_t maxPerLoop = UINT64_MAX / 2 / n * n, resultElems = UINT64_MAX;
+    if (cclBytes != 0) {
+        rc = orc_sequence_max_count_per_loop(cclBytes, count, l0, n, r.esz, 4096, 0, &maxPerLoop, &resultElems);
+        if (rc != ORC_OK) {
+            return rc;
+        }
+    }
+    levels_t lv = {&r, l0, l1, n / l0 / l1, algo, NULL, NULL};
+    const uint8_t** src = (const uint8_t**)malloc(sizeof(uint8_t*) * n);
+    lv.tmp = malloc(count * r.asz);
+    lv.src = src;
+    if (!src || !lv.tmp) {
+        rc = ORC_E_INTERNAL;
+    }
+    for (uint32_t j = 0; j < n && rc == ORC_OK; ++j) {
+        src[j] = cbytes(in[j]);
+    }
+    uint64_t processed = 0;
+    while (processed < count && rc == ORC_OK) {
+        uint64_t cur = orc_sequence_select_loop_count(count - processed, maxPerLoop, l0, resultElems);
+        if (cur == 0) {
+            rc = ORC_E_INTERNAL;
+            break;
+        }
+        rc = levels_all_reduce_loop(&lv, processed, cur, 0, bytes(out[root]), processed);
+        processed += cur;
+    }
+    free(src);
+    free(lv.tmp);
+    return rc;
+}
+
+/* ReduceScatter over three levels (ins_v2_reduce_scatter_sequence_executor_3level.cc:243-256): the mesh
+ * ReduceScatter inside every box for the slices of every box of the world, the template between the boxes of a
+ * pod for the slices of every pod, the template between the pods; rank (g * l1 + b) * l0 + i ends with its slice. */
+int orc_reduce_scatter_three_level(uint32_t n, uint32_t l0, uint32_t l1, int algo, const void* const* in,
+                                   void* const* out, uint64_t recvCount, int dtype, int op, int accMode)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (levels_check(n, l0, l1, algo) != ORC_OK || algo == ORC_L1_MESH) {
+        return ORC_E_PARA;
+    }
+    if (recvCount == 0) {
+        return ORC_OK;
+    }
+    uint32_t l2 = n / l0 / l1;
+    const uint8_t** src = (const uint8_t**)malloc(sizeof(uint8_t*) * n);
+    void* tmp = malloc(recvCount * r.asz);
+    scratch_t sc1, sc2;
+    sc1.mem = sc2.mem = NULL;
+    if (!src || !tmp || scratch_alloc(&sc1, l1, recvCount, r.asz) != ORC_OK ||
+        scratch_alloc(&sc2, l2, recvCount, r.asz) != ORC_OK) {
+        rc = ORC_E_INTERNAL;
+    }
+    for (uint32_t j = 0; j < n && rc == ORC_OK; ++j) {
+        src[j] = cbytes(in[j]);
+    }
+    for (uint32_t i = 0; i < l0 && rc == ORC_OK; ++i) {
+        for (uint32_t b = 0; b < l1 && rc == ORC_OK; ++b) {
+            /* the slices (q, b, i) of all pods q, as the pods hold them after RSL1: pod g's boxes fold their
+             * level-0 results for the slices (q, b', i); box b ends with the units b */
+            for (uint32_t q = 0; q < l2 && rc == ORC_OK; ++q) {
+                for (uint32_t g = 0; g < l2 && rc == ORC_OK; ++g) {
+                    for (uint32_t bb = 0; bb < l1; ++bb) {
+                        for (uint32_t u = 0; u < l1; ++u) {
+                            uint32_t at = algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l1, u) : u;
+                            level0_fold(&r, l0, g * l1 + bb, i, src, (uint64_t)((q * l1 + u) * l0 + i) * recvCount,
+                                        recvCount, scratch_at(&sc1, bb, at), tmp);
+                        }
+                    }
+                    rc = algo == ORC_L1_RHD ? rhd_rs_frame(&r, &sc1, 0) : nhr_reduce_scatter_scratch(&r, &sc1);
+                    uint32_t at1 = algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l1, b) : b;
+                    uint32_t at2 = algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l2, q) : q;
+                    memcpy(scratch_at(&sc2, g, at2), scratch_at(&sc1, b, at1), recvCount * r.asz);
+                }
+            }
+            if (rc == ORC_OK) {
+                rc = algo == ORC_L1_RHD ? rhd_rs_frame(&r, &sc2, 0) : nhr_reduce_scatter_scratch(&r, &sc2);
+            }
+            for (uint32_t g = 0; g < l2 && rc == ORC_OK; ++g) {
+                uint32_t at2 = algo == ORC_L1_RHD ? orc_rhd_unit_start_of_rank(l2, g) : g;
+                red_narrow(&r, scratch_at(&sc2, g, at2), out[(g * l1 + b) * l0 + i], recvCount);
+            }
+        }
+    }
+    free(sc1.mem);
+    free(sc2.mem);
+    free(src);
+    free(tmp);
+    return rc;
+}
+
+/* Loop rule of the three-level sequence executors (3level.cc:524-534; reduce_sequence_executor_aicpu_3level.cc:
+ * 877-889): the buffer, less the two tail tiles of rhd_tail.h:64-92 when they are needed, is cut into l0 + 1
+ * slices of whole elements; a loop holds what l0 of them take, floored to `align` bytes, whole elements and a
+ * multiple of `total`.  resultElems: the elements of one slice. */
+int orc_sequence_max_count_per_loop(uint64_t cclBytes, uint64_t count, uint32_t l0, uint32_t total, uint64_t esz,
+                                    uint64_t align, int rhdTail, uint64_t* maxCount, uint64_t* resultElems)
+{
+    if (l0 == 0 || total == 0 || esz == 0 || align == 0) {
+        return ORC_E_PARA;
+    }
+    uint64_t ws = cclBytes;
+    if (rhdTail && count % total != 0) {
+        if (total > ws / esz / 2) {
+            return ORC_E_INTERNAL;
+        }
+        uint64_t tile = (uint64_t)total * esz;
+        uint64_t slot = (tile / 128 + (tile % 128 != 0)) * 128;
+        if (slot >= ws / 2) {
+            return ORC_E_INTERNAL;
+        }
+        ws -= 2 * slot;
+    }
+    uint64_t slice = ws / (l0 + 1) / esz * esz;
+    uint64_t comm = (uint64_t)l0 * slice;
+    *resultElems = slice / esz;
+    *maxCount = comm / align * align / esz / total * total;
+    return *maxCount == 0 ? ORC_E_INTERNAL : ORC_OK;
+}
+
+/* 3level.cc:704-731: a last loop whose last chunk, floor(cur / l0) + cur mod l0 elements, would not fit the
+ * result slice is shortened; what it leaves runs as one more loop. */
+uint64_t orc_sequence_select_loop_count(uint64_t remaining, uint64_t maxCountPerLoop, uint32_t l0, uint64_t resultElems)
+{
+    if (remaining > maxCountPerLoop) {
+        return maxCountPerLoop;
+    }
+    uint64_t cur = remaining;
+    uint64_t q = cur / l0;
+    uint64_t rem = cur % l0;
+    if (q + rem > resultElems && q > 0) {
+        if (resultElems == 0) {
+            return 0;
+        }
+        uint64_t newQ = q - 1;
+        uint64_t newR;
+        if (newQ >= resultElems) {
+            newQ = resultElems;
+            newR = 0;
+        } else {
+            newR = l0 - 1 < resultElems - newQ ? l0 - 1 : resultElems - newQ;
+        }
+        cur = newQ * l0 + newR;
+    }
+    return cur;
 }
 
 /* a12: while blocks > 1: M = largest power of two < blocks; for src = M..blocks-1:

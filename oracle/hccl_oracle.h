@@ -168,6 +168,24 @@ int orc_reduce_scatter_two_level(uint32_t n, uint32_t l0, int l1Algo, const void
                                  uint64_t recvCount, int dtype, int op, int accMode);
 int orc_all_reduce_two_level(uint32_t n, uint32_t l0, int l1Algo, const void* const* in, void* const* out,
                              uint64_t count, int dtype, int op, int accMode, uint64_t maxCountPerLoop);
+/* Three levels (ins_v2_all_reduce_sequence_executor_aicpu_3level.cc, ins_v2_reduce_scatter_sequence_executor_3level.cc,
+ * reduce_sequence_executor_aicpu_3level.cc): l0 consecutive ranks form a box, l1 consecutive boxes a pod; the mesh
+ * ReduceScatter inside the boxes, `algo` (ORC_L1_RHD or ORC_L1_NHR) between the boxes of a pod and once more between
+ * the pods.  cclBytes: the staging buffer whose loops show in the cuts of AllReduce and Reduce, 0 = one loop.
+ * orc_reduce_levels also is the two-level Reduce (l1 = n / l0; ORC_L1_MESH allowed there: the host-reduce fold). */
+int orc_all_reduce_three_level(uint32_t n, uint32_t l0, uint32_t l1, int algo, const void* const* in,
+                               void* const* out, uint64_t count, int dtype, int op, int accMode, uint64_t cclBytes);
+int orc_reduce_scatter_three_level(uint32_t n, uint32_t l0, uint32_t l1, int algo, const void* const* in,
+                                   void* const* out, uint64_t recvCount, int dtype, int op, int accMode);
+int orc_reduce_levels(uint32_t n, uint32_t l0, uint32_t l1, int algo, const void* const* in, void* const* out,
+                      uint64_t count, int dtype, int op, uint32_t root, int accMode, uint64_t cclBytes);
+int orc_sequence_max_count_per_loop(uint64_t cclBytes, uint64_t count, uint32_t l0, uint32_t total, uint64_t esz,
+                                    uint64_t align, int rhdTail, uint64_t* maxCount, uint64_t* resultElems);
+uint64_t orc_sequence_select_loop_count(uint64_t remaining, uint64_t maxCountPerLoop, uint32_t l0,
+                                        uint64_t resultElems);
+/* Reduce along the NHR step tree on slices of ceil(len / n) elements (reduce_nhr.cc); only out[root] is written. */
+int orc_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op, int accMode,
+                   uint32_t root, uint64_t maxCountPerLoop);
 
 /* The same inside the executor's loop over the staging buffer (ins_v2_all_reduce_sole_executor.cc:266-300):
  * every loop of maxCountPerLoop elements (the last one shorter) is sliced afresh; 0 = one loop. */

@@ -2,14 +2,15 @@
 AlltoAll, as data.
 
 Reads (as text; nothing of the reference is imported or run) the TEST_F cases of
-    test/st/algorithm/testcase/all_reduce_testcase.cc
-    test/st/algorithm/testcase/reduce_scatter_testcase.cc, reduce_scatter_aicpu_testcase.cc, ..._testcase2.cc, ..._testcase3.cc
-    test/st/algorithm/testcase/reduce_testcase.cc, reduce_aicpu_testcase.cc
-    test/st/algorithm/testcase/all_gather_aicpu_testcase.cc, alltoall_testcase.cc
-and writes tests/golden/reference_st_reduce_shapes.json: one entry per case whose numbers are written out, with its
-name, the file and line it starts on, the servers of its topology (ranks per server), the element count (the
-file's constants folded in), the data type, the reduce operation, the root (Reduce) and the HCCL_ALGO string the case
-sets, if any.  The reference checks these cases on a simulated task graph; tests/test_wide_gpu_reference_st_reduce_shapes.py
+    test/st/algorithm/testcase/all_reduce_testcase.cc, all_reduce_multilevel_testcase.cc, all_reduce_parallel_testcase.cc
+    test/st/algorithm/testcase/reduce_scatter_testcase.cc, reduce_scatter_aicpu_testcase.cc, ..._testcase2.cc, ..._testcase3.cc,
+        reduce_scatter_3level_testcase.cc, reduce_scatter_meshchunk_concur_testcase.cc
+    test/st/algorithm/testcase/reduce_testcase.cc, reduce_aicpu_testcase.cc, reduce_3level_testcase.cc, reduce_sequence_testcase.cc
+    test/st/algorithm/testcase/all_gather_aicpu_testcase.cc, all_gather_3level_testcase.cc, alltoall_testcase.cc
+and writes tests/golden/reference_st_reduce_shapes.json: one entry per case whose numbers are written out and whose
+world has at most 64 ranks, with its name, the file and line it starts on, the servers of its topology (ranks per
+server) and its pods (servers per pod), the element count (the file's constants folded in), the data type, the reduce
+operation, the root (Reduce) and the HCCL_ALGO string the case, or its fixture's SetUp, sets, if any.  The reference checks these cases on a simulated task graph; tests/test_wide_gpu_reference_st_reduce_shapes.py
 replays the shapes (counts scaled down, remainders kept) against the oracle.
 
 Usage (in the container that holds /root/reference):  python tests/golden/make_reference_st_reduce_shapes.py
@@ -21,11 +22,12 @@ import re
 REF = "/root/reference/test/st/algorithm/testcase"
 HERE = os.path.dirname(os.path.abspath(__file__))
 FILES = {
-    "all_reduce": ["all_reduce_testcase.cc"],
+    "all_reduce": ["all_reduce_testcase.cc", "all_reduce_multilevel_testcase.cc", "all_reduce_parallel_testcase.cc"],
     "reduce_scatter": ["reduce_scatter_testcase.cc", "reduce_scatter_aicpu_testcase.cc", "reduce_scatter_aicpu_testcase2.cc",
-                       "reduce_scatter_aicpu_testcase3.cc"],
-    "reduce": ["reduce_testcase.cc", "reduce_aicpu_testcase.cc"],
-    "all_gather": ["all_gather_aicpu_testcase.cc"],
+                       "reduce_scatter_aicpu_testcase3.cc", "reduce_scatter_3level_testcase.cc",
+                       "reduce_scatter_meshchunk_concur_testcase.cc"],
+    "reduce": ["reduce_testcase.cc", "reduce_aicpu_testcase.cc", "reduce_3level_testcase.cc", "reduce_sequence_testcase.cc"],
+    "all_gather": ["all_gather_aicpu_testcase.cc", "all_gather_3level_testcase.cc"],
     "all_to_all": ["alltoall_testcase.cc"],
 }
 SIZES = {"INT8": 1, "UINT8": 1, "INT16": 2, "UINT16": 2, "FP16": 2, "BFP16": 2, "INT32": 4, "UINT32": 4, "FP32": 4,
@@ -67,20 +69,38 @@ def value_of(expr, names):
 
 
 def topology(body):
+    """(ranks per server, servers per pod) of a case: TopoMeta is a list of pods of servers of device ids."""
     m = re.search(r"TopoMeta\s+\w+\s*\{(.*?)\}\s*;", body, re.S)
     if m:
-        servers = re.findall(r"\{([\d\s,]*)\}", m.group(1))
-        sizes = [len([x for x in s.split(",") if x.strip()]) for s in servers]
-        return [s for s in sizes if s] or None
+        text = m.group(1)
+        servers, pods, depth, inPod = [], [], 0, 0
+        for k, ch in enumerate(text):
+            if ch == "{":
+                depth += 1
+                if depth == 1:
+                    inPod = 0
+                elif depth == 2:
+                    end = text.index("}", k)
+                    size = len([x for x in text[k + 1:end].split(",") if x.strip()])
+                    if size:
+                        servers.append(size)
+                        inPod += 1
+            elif ch == "}":
+                if depth == 1 and inPod:
+                    pods.append(inPod)
+                depth -= 1
+        return (servers, pods) if servers else None
     m = re.search(r"GenTopoMeta\(\s*\w+\s*,\s*(\d+)\s*,\s*(\d+)\s*,\s*(\d+)\s*\)", body)
-    if m and int(m.group(1)) == 1:
-        return [int(m.group(3))] * int(m.group(2))
+    if m:
+        pods, servers, ranks = int(m.group(1)), int(m.group(2)), int(m.group(3))
+        return [ranks] * (pods * servers), [servers] * pods
     return None
 
 
 def main():
     out = []
     skipped = 0
+    large = 0
     for kind, files in FILES.items():
         for name in files:
             text = open(os.path.join(REF, name), encoding="utf-8", errors="replace").read()
@@ -90,9 +110,13 @@ def main():
                 if v is not None:
                     consts[m.group(1)] = v
             tokens = dict(re.findall(r'constexpr\s+char\s+(\w+)\[\]\s*=\s*"([^"]+)"\s*;', text))
+            tokens.update(re.findall(r'constexpr\s+const\s+char\s*\*\s*(\w+)\s*=\s*"([^"]+)"\s*;', text))
+            # a string the fixture's SetUp puts into HCCL_ALGO holds for every case of the file
+            fixture = re.search(r'void\s+SetUp\(\)[^{]*\{[^}]*setenv\(\s*"HCCL_ALGO"\s*,\s*"([^"]+)"', text, re.S)
             for case, line, raw in cases_of(text):
                 body = strip_comments(raw)
-                servers = topology(body)
+                topo = topology(body)
+                servers, pods = topo if topo else (None, None)
                 dtype = re.search(r"HCCL_DATA_TYPE_(\w+)", body)
                 op = re.search(r"HCCL_REDUCE_(\w+)", body)
                 names = dict(consts)
@@ -114,6 +138,8 @@ def main():
                     m = re.search(r'setenv\(\s*"HCCL_ALGO"\s*,\s*(\w+)\s*,', body)
                     if m and m.group(1) in tokens:
                         config = tokens[m.group(1)]
+                    elif fixture:
+                        config = fixture.group(1)
                 root = None
                 if kind == "reduce":
                     m = re.search(r"\broot\s*=\s*(\d+)\s*;", body)
@@ -124,13 +150,17 @@ def main():
                 if not servers or not dtype or count is None or (kind == "reduce" and root is None):
                     skipped += 1
                     continue
+                if sum(servers) > 64:
+                    large += 1
+                    continue
                 out.append({"kind": kind, "name": case, "source": "%s:%d" % (name, line), "servers": servers,
-                            "count": count, "type": dtype.group(1), "op": op.group(1) if op else "SUM",
+                            "pods": pods, "count": count, "type": dtype.group(1), "op": op.group(1) if op else "SUM",
                             "root": root, "hccl_algo": config})
     with open(os.path.join(HERE, "reference_st_reduce_shapes.json"), "w") as f:
         json.dump(out, f, indent=0)
         f.write("\n")
-    print(len(out), "cases written,", skipped, "left out (numbers built by helpers or loops, or deeper topologies)")
+    print(len(out), "cases written,", skipped, "left out (numbers built by helpers or loops),", large,
+          "for worlds of more than 64 ranks")
 
 
 if __name__ == "__main__":

@@ -251,13 +251,15 @@ def test_algo_knob(world):
     assert hccl_amd.get_algo(world[3], OpKind.ALL_REDUCE) == Algo.RHD   # per world, not per rank
     assert code_of(hccl_amd.set_algo, world[0], OpKind.ALL_REDUCE, Algo.AIV_MESH) == 5
     hccl_amd.set_algo(world[0], OpKind.ALL_REDUCE, Algo.MESH)
-    # Reduce knows its one-shot and two-shot orders only; the two-shot order exists for Reduce only
+    # Reduce knows its one-shot and two-shot orders, NHR, and RHD for worlds with levels; the two-shot order exists
+    # for Reduce only
     assert hccl_amd.get_algo(world[0], OpKind.REDUCE) == Algo.MESH
-    hccl_amd.set_algo(world[0], OpKind.REDUCE, Algo.MESH_TWO_SHOT)
-    assert hccl_amd.get_algo(world[2], OpKind.REDUCE) == Algo.MESH_TWO_SHOT
+    for algo in (Algo.MESH_TWO_SHOT, Algo.NHR, Algo.RHD):
+        hccl_amd.set_algo(world[0], OpKind.REDUCE, algo)
+        assert hccl_amd.get_algo(world[2], OpKind.REDUCE) == algo
     hccl_amd.set_algo(world[0], OpKind.REDUCE, Algo.MESH)
-    for kind, algo in ((OpKind.REDUCE, Algo.NHR), (OpKind.REDUCE, Algo.MESH_CHUNK), (OpKind.ALL_REDUCE, Algo.MESH_TWO_SHOT),
-                       (OpKind.REDUCE_SCATTER, Algo.MESH_TWO_SHOT)):
+    for kind, algo in ((OpKind.REDUCE, Algo.ORDER_PRESERVED), (OpKind.REDUCE, Algo.MESH_CHUNK),
+                       (OpKind.ALL_REDUCE, Algo.MESH_TWO_SHOT), (OpKind.REDUCE_SCATTER, Algo.MESH_TWO_SHOT)):
         assert code_of(hccl_amd.set_algo, world[0], kind, algo) == 5
 
 

@@ -197,9 +197,9 @@ def test_groups_must_divide_the_world():
     with pytest.raises(hccl_amd.HcclError) as e:
         hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.RHD, 6, level0=4)
     assert e.value.code == 1
-    with pytest.raises(hccl_amd.HcclError) as e:
-        hccl_amd.fold_programs(OpKind.REDUCE, Algo.MESH, 6, level0=2)
-    assert e.value.code == 5
+    # Reduce over groups runs the AllReduce's steps and hands the root the result
+    assert hccl_amd.fold_programs(OpKind.REDUCE, Algo.MESH, 6, level0=2) == hccl_amd.fold_programs(
+        OpKind.ALL_REDUCE, Algo.MESH, 6, level0=2)
     with pytest.raises(hccl_amd.HcclError) as e:
         hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.ORDER_PRESERVED, 6, level0=2)
     assert e.value.code == 5
@@ -392,7 +392,8 @@ def test_what_the_system_tests_two_level_strings_select():
     # all_reduce_testcase.cc:317-345, all_reduce_dpu_testcase.cc: level-0 mesh inside a server, RHD / NHR between them
     assert sel("allreduce:sequence{level0=meshconcur,level1=rhd}", AR)[1:] == (Algo.RHD, True)
     assert sel("allreduce:sequence{mesh,nhr}", AR)[1:] == (Algo.NHR, True)
-    # three levels, pipelines and parallel executors are orders this library does not build: nothing is selected
+    # mixed templates above level 0, pipelines and parallel executors are orders this library does not build:
+    # nothing is selected
     assert sel("allreduce:sequence{meshconcur,nhr,mesh}", AR)[1] is None
     assert sel("allreduce:pipeline{mesh,nhr,nhr}", AR)[1] is None
     assert sel("reducescatter:parallel{level0=mesh,level1=hd}", RS)[1] is None
@@ -419,11 +420,12 @@ def test_what_hccl_algo_selects():
     assert sel("reducescatter:sole{hd_aicpu_reduce}", RS)[1] == Algo.RHD
     assert sel("reducescatterv:sole{mesh_chunk}", RS)[1] == Algo.MESH_CHUNK
     assert sel("reduce:mesh_two_shot", RD)[1] == Algo.MESH_TWO_SHOT
-    assert sel("reduce:sole{nhr}", RD)[1] is None                              # no such Reduce order here
+    assert sel("reduce:sole{nhr}", RD)[1:] == (Algo.NHR, False)                # reduce_nhr.cc
     assert sel("strictordered{mesh}", AR)[1] == Algo.ORDER_PRESERVED
     assert sel("strictordered{mesh}", RD)[1] is None
     # a clause without an operator applies to all of them; later clauses are read first
-    assert sel("nhr", AR)[1] == Algo.NHR and sel("nhr", RS)[1] == Algo.NHR and sel("nhr", RD)[1] is None
+    assert sel("nhr", AR)[1] == Algo.NHR and sel("nhr", RS)[1] == Algo.NHR and sel("nhr", RD)[1] == Algo.NHR
+    assert sel("mesh_chunk", AR)[1] == Algo.MESH_CHUNK and sel("mesh_chunk", RD)[1] is None
     assert sel("allreduce:sole{nhr};sole{mesh}", AR)[1] == Algo.MESH
     assert sel("sole{mesh};allreduce:sole{nhr}", AR)[1] == Algo.NHR
     assert sel("sole{mesh};allreduce:sole{nhr}", RS)[1] == Algo.MESH
@@ -431,7 +433,7 @@ def test_what_hccl_algo_selects():
     assert sel("allreduce:not(sole{nhr})", AR)[1] is None
     assert sel("allreduce:sole{not(nhr)}", AR)[1] is None
     assert sel("allgather:sole{mesh};alltoall:pairwise", AR)[1] is None
-    assert sel("allreduce:sequence{mesh,nhr,nhr}", AR)[1] is None              # three levels are not built
+    assert sel("allreduce:sequence{mesh,nhr,nhr}", AR)[1:] == (Algo.NHR, True)  # the same template at both upper levels
     # ReduceScatter in two levels: the same executor family (ins_v2_reduce_scatter_sequence_executor_aicpu.cc:567-640)
     assert sel("reducescatter:sequence{level0=meshconcur,level1=rhd}", RS)[1:] == (Algo.RHD, True)
     assert sel("reducescatter:sequence{mesh_concur,nhr}", RS)[1:] == (Algo.NHR, True)

@@ -1,11 +1,14 @@
 """Replays the shapes of the reference's own system tests for AllReduce, ReduceScatter, Reduce, AllGather and AlltoAll
-(test/st/algorithm/testcase/all_reduce_testcase.cc, reduce_scatter_testcase.cc, reduce_scatter_aicpu_testcase*.cc,
-reduce_testcase.cc, reduce_aicpu_testcase.cc, all_gather_aicpu_testcase.cc, alltoall_testcase.cc; transcribed as
-data into tests/golden/reference_st_reduce_shapes.json by tests/golden/make_reference_st_reduce_shapes.py) through
-the C ABI against the oracle: the servers of the case's
-topology become the level-0 groups of a loopback world, the HCCL_ALGO string the case sets is in the environment when
-the world is created, and the expected bits come from the oracle in the order that string selects here (the two-level
-orders where it names a sequence executor this library builds, the one-level order otherwise).  The reference checks
+(test/st/algorithm/testcase/all_reduce_testcase.cc, all_reduce_multilevel_testcase.cc, all_reduce_parallel_testcase.cc,
+reduce_scatter_testcase.cc, reduce_scatter_aicpu_testcase*.cc, reduce_scatter_3level_testcase.cc,
+reduce_scatter_meshchunk_concur_testcase.cc, reduce_testcase.cc, reduce_aicpu_testcase.cc, reduce_3level_testcase.cc,
+reduce_sequence_testcase.cc, all_gather_aicpu_testcase.cc, all_gather_3level_testcase.cc, alltoall_testcase.cc;
+transcribed as data into tests/golden/reference_st_reduce_shapes.json by
+tests/golden/make_reference_st_reduce_shapes.py) through the C ABI against the oracle: the servers of the case's
+topology become the level-0 groups of a loopback world and its pods the level-1 groups, the HCCL_ALGO string the case
+sets is in the environment when the world is created, and the expected bits come from the oracle in the order that
+string selects here (the two- and three-level orders where it names a sequence executor this library builds, the
+one-level order otherwise).  The reference checks
 these cases on a simulated task graph, not with values.  Counts above 6000 elements (the catalogue goes to 400 Mi) are
 scaled down to about 3000; what they leave over after division by the rank count is kept, zero stays zero."""
 import json
@@ -81,7 +84,7 @@ def copy_shape(case, n):
 
 
 def test_the_catalogue_is_what_the_generator_wrote():
-    assert len(CASES) == 126
+    assert len(CASES) == 241
     assert {c["kind"] for c in CASES} == set(KINDS) | set(COPIES)
     assert all(c["type"] in (SIZES if c["kind"] in COPIES else TYPES) and c["op"] in OPS and sum(c["servers"]) <= 64
                for c in CASES)
@@ -96,11 +99,13 @@ def test_reference_system_test_shape(case):
         return copy_shape(case, n)
     kind, dtype, op = case["kind"], TYPES[case["type"]], OPS[case["op"]]
     level0 = servers[0] if len(servers) > 1 and len(set(servers)) == 1 and servers[0] > 1 else 1
+    pods = case["pods"]
+    level1 = pods[0] if level0 > 1 and len(pods) > 1 and len(set(pods)) == 1 else 0
     count = scaled(case["count"], n)
-    env = {"HCCL_AMD_LEVEL0_RANKS": str(level0)}
+    env = {"HCCL_AMD_LEVEL0_RANKS": str(level0), "HCCL_AMD_LEVEL1_GROUPS": str(level1)}
     if case["hccl_algo"]:
         env["HCCL_ALGO"] = case["hccl_algo"]
-    saved = {k: os.environ.get(k) for k in ("HCCL_ALGO", "HCCL_AMD_LEVEL0_RANKS")}
+    saved = {k: os.environ.get(k) for k in ("HCCL_ALGO", "HCCL_AMD_LEVEL0_RANKS", "HCCL_AMD_LEVEL1_GROUPS")}
     os.environ.pop("HCCL_ALGO", None)
     os.environ.update(env)
     try:
@@ -117,11 +122,18 @@ def test_reference_system_test_shape(case):
         host_only = op == OPS["PROD"] or dtype in (DT.INT64, DT.UINT64, DT.FP64)
         rng = np.random.default_rng(len(case["name"]) * 131 + count)
         what = "%s %s" % (case["name"], case["source"])
+        two_level = level0 > 1 and (sequence or not case["hccl_algo"]) and algo in ("rhd", "nhr")
         if kind == "reduce":
             root = case["root"]
             ins = [gen(dtype, op, rng, count) for _ in range(n)]
             want = [np.zeros(count, dtype=NP[dtype]) for _ in range(n)]
-            assert oracle.reduce(ins, want, count, int(dtype), op, root, algo=algo) == 0
+            if two_level:
+                assert oracle.reduce_levels(ins, want, count, int(dtype), op, root, level0,
+                                            n // level0 if host_only or not level1 else level1,
+                                            "mesh" if host_only else algo) == 0
+            else:   # one level: NHR, or the rank order (which the host-reduced types and a lone RHD fall back to)
+                order = algo if algo in ("mesh", "ring", "mesh_two_shot") or (algo == "nhr" and not host_only) else "mesh"
+                assert oracle.reduce(ins, want, count, int(dtype), op, root, algo=order) == 0
             sends = [to_dev(x) for x in ins]
             recvs = [dev_zeros(max(x.nbytes, 1)) for x in ins]
             w.inputs_ready()
@@ -132,13 +144,14 @@ def test_reference_system_test_shape(case):
             if count:
                 check(dtype, op, to_host(recvs[root], NP[dtype])[:count], want[root], what)
             return
-        two_level = level0 > 1 and (sequence or not case["hccl_algo"]) and algo in ("rhd", "nhr")
-        level1 = "mesh" if host_only else algo
+        between = "mesh" if host_only else algo
         if kind == "all_reduce":
             ins = [gen(dtype, op, rng, count) for _ in range(n)]
             want = [np.zeros(count, dtype=NP[dtype]) for _ in range(n)]
-            if two_level:
-                assert oracle.all_reduce_two_level(ins, want, count, int(dtype), op, level0, level1) == 0
+            if two_level and level1 and not host_only:
+                assert oracle.all_reduce_three_level(ins, want, count, int(dtype), op, level0, level1, algo) == 0
+            elif two_level:
+                assert oracle.all_reduce_two_level(ins, want, count, int(dtype), op, level0, between) == 0
             else:
                 assert oracle.all_reduce(ins, want, count, int(dtype), op, algo=order_of(algo, dtype, op, False)) == 0
             sends = [to_dev(x) for x in ins]
@@ -150,8 +163,10 @@ def test_reference_system_test_shape(case):
         else:
             ins = [gen(dtype, op, rng, n * count) for _ in range(n)]
             want = [np.zeros(count, dtype=NP[dtype]) for _ in range(n)]
-            if two_level:
-                assert oracle.reduce_scatter_two_level(ins, want, count, int(dtype), op, level0, level1) == 0
+            if two_level and level1 and not host_only:
+                assert oracle.reduce_scatter_three_level(ins, want, count, int(dtype), op, level0, level1, algo) == 0
+            elif two_level:
+                assert oracle.reduce_scatter_two_level(ins, want, count, int(dtype), op, level0, between) == 0
             else:
                 assert oracle.reduce_scatter(ins, want, count, int(dtype), op, algo=order_of(algo, dtype, op, True)) == 0
             sends = [to_dev(x) for x in ins]
