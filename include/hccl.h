@@ -207,7 +207,7 @@ HcclResult HcclGroupEnd(void);
 typedef enum {
     HCCL_AMD_OP_ALL_REDUCE = 0,
     HCCL_AMD_OP_REDUCE_SCATTER = 1,   /* also ReduceScatterV */
-    HCCL_AMD_OP_REDUCE = 2,           /* MESH (alias RING) or MESH_TWO_SHOT */
+    HCCL_AMD_OP_REDUCE = 2,           /* MESH (alias RING), MESH_TWO_SHOT, NHR; RHD in worlds with level-0 groups */
     HCCL_AMD_OP_COUNT
 } HcclAmdOpKind;
 
@@ -222,11 +222,13 @@ typedef enum {
      * in rank order like MESH; "ring" ReduceScatter uses the NHR step tree. */
     HCCL_AMD_ALGO_RING = 1,
     /* Recursive halving-doubling with pre-fold of non-power-of-two ranks
-     * (reference template_utils.cc:117-307, ins_temp_reduce_scatter_rhd.cc). */
+     * (reference template_utils.cc:117-307, ins_temp_reduce_scatter_rhd.cc).  Reduce knows it between level-0
+     * groups only (reduce_sequence_executor_aicpu_3level.cc:1024-1048) and folds in the MESH order without them. */
     HCCL_AMD_ALGO_RHD = 2,
     /* Non-uniform hierarchical ring step tree (reference ins_temp_reduce_scatter_nhr.cc:458-506).  AllReduce
      * cuts the count into N slices of floor(count / N) elements, the last slice taking the rest, and folds
-     * slice k by rank k's tree (reference ins_temp_all_reduce_nhr.cc:214-216, 646-687). */
+     * slice k by rank k's tree (reference ins_temp_all_reduce_nhr.cc:214-216, 646-687).  Reduce cuts slices of
+     * ceil(count / N) elements, short or empty towards the end (reference reduce_nhr.cc:202-226). */
     HCCL_AMD_ALGO_NHR = 3,
     /* Power-of-two block fold used when results must not depend on arrival order
      * (reference ins_temp_reduce_scatter_order_preserved_group.cc:306-409). */
@@ -351,9 +353,10 @@ HcclResult HcclAmdGetLevel1GroupSize(HcclComm comm, uint32_t* groupsPerLevel1Gro
  * and vocabulary of src/common/alg_parse.cc:27-437) is read at world creation and selects the fold order of
  * AllReduce, ReduceScatter(V) and Reduce: sole{mesh | mesh_one_shot | mesh_two_shot} -> MESH (Reduce: mesh_two_shot ->
  * MESH_TWO_SHOT), sole{mesh_chunk...} -> MESH_CHUNK, sole{nhr...} -> NHR, sole{nhr_aicpu_reduce} -> the host-reduce
- * order (RING for AllReduce, MESH for ReduceScatter), sole{rhd | hd | hd_aicpu_reduce} -> RHD, strictordered{...} ->
- * ORDER_PRESERVED, sequence{<mesh...>, <template>} -> that template between level-0 groups (AllReduce,
- * ReduceScatter; a mesh-chunk template inside the groups is another order and selects nothing).  Clauses are
+ * order (RING for AllReduce, MESH for ReduceScatter and Reduce), sole{rhd | hd | hd_aicpu_reduce} -> RHD, strictordered{...} ->
+ * ORDER_PRESERVED, sequence{<mesh...>, <template>[, <the same template>]} -> that template between level-0 groups
+ * and, where the world has them, between level-1 groups (AllReduce, ReduceScatter, Reduce; a mesh-chunk template
+ * inside the groups and different templates at the upper levels are other orders and select nothing).  Clauses are
  * taken last to first, negations select nothing, clauses for the copy operators are accepted and ignored, and a
  * string the reference's parser rejects is ignored with a warning, as there.  HCCL_AMD_ALGO and HcclAmdSetAlgo
  * override it.  This call is the host-only view of that reading: HCCL_E_PARA for a rejected string; otherwise
