@@ -405,3 +405,22 @@ def test_what_hccl_algo_selects_for_three_levels_and_for_reduce():
     assert sel("reduce:sole{nhr_aicpu_reduce}", OpKind.REDUCE)[1:] == (Algo.MESH, False)
     assert sel("reduce:sole{mesh_two_shot}", OpKind.REDUCE)[1:] == (Algo.MESH_TWO_SHOT, False)
     assert sel("reduce:sole{mesh_chunk}", OpKind.REDUCE)[1] is None
+
+
+def test_every_division_of_up_to_64_ranks_into_levels_has_programs_the_kernel_can_run():
+    """Nesting depth and program length stay within what the kernel's interpreter takes (8 levels, 320 bytes) for every
+    way of cutting 2 .. 64 ranks into boxes and pods, under both templates."""
+    longest = 0
+    for n in range(2, 65):
+        for l0 in range(2, n):
+            if n % l0:
+                continue
+            boxes = n // l0
+            for l1 in range(1, boxes + 1):
+                if boxes % l1:
+                    continue
+                for algo in (Algo.NHR, Algo.RHD):
+                    progs = hccl_amd.fold_programs(OpKind.ALL_REDUCE, algo, n, level0=l0, level1=l1)
+                    assert len(progs) == n
+                    longest = max(longest, max(len(p) for p in progs))
+    assert longest <= 320
