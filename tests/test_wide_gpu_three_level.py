@@ -252,3 +252,63 @@ def test_levels_and_orders_from_the_environment():
         check(DT.FP32, SUM, to_host(recvs[3], np.float32), want[3], "reduce:sole{nhr} in a world with levels")
     finally:
         w.close()
+
+
+# Another number here draws other cases (used for longer runs by hand, mostly on the CPU emulation).
+SWEEP_SEED = int(os.environ.get("HCCL_AMD_TEST_SWEEP_SEED", "91000"))
+TYPES = [DT.INT8, DT.INT16, DT.INT32, DT.INT64, DT.UINT64, DT.FP16, DT.BFP16, DT.FP32, DT.FP64]
+LEVELS = [(2, 2, 2), (2, 2, 3), (3, 2, 2), (2, 3, 2), (2, 1, 4), (3, 3, 2), (2, 5, 2), (4, 2, 2), (2, 2, 5), (5, 2, 3),
+          (2, 4, 4), (6, 2, 2)]
+
+
+def pick_count(rng, n):
+    kind = rng.integers(0, 4)
+    if kind == 0:
+        return int(rng.integers(1, 3 * n))                       # around one element per unit
+    if kind == 1:
+        return int(rng.integers(70, 5_000))
+    if kind == 2:
+        return int(rng.choice([4096, 8192, 65536]) + rng.integers(-3, 4))
+    return n * int(rng.integers(1, 2_000))                       # everything divides
+
+
+@pytest.mark.parametrize("l0,l1,l2", LEVELS)
+def test_random_cases_over_levels(l0, l1, l2):
+    """Seeded random sweep over (operator, type, operation, template, count, root, buffer alignment, staging-buffer
+    size) in worlds of three levels."""
+    n = l0 * l1 * l2
+    rng = np.random.default_rng(SWEEP_SEED + 100 * l0 + 10 * l1 + l2)
+    w = levels_world(l0, l1, l2)
+    try:
+        for case in range(24):
+            dtype = TYPES[rng.integers(0, len(TYPES))]
+            op = int(rng.integers(0, 4))
+            if op == PROD and dtype in (DT.INT16, DT.BFP16):
+                op = SUM
+            algo = ("rhd", "nhr")[rng.integers(0, 2)]
+            count = pick_count(rng, n)
+            esz = np.dtype(NP[dtype]).itemsize
+            pad = int(rng.integers(0, 16 // esz)) if rng.random() < 0.5 else 0
+            which = rng.integers(0, 3)
+            ccl = 0
+            if which != 1 and rng.random() < 0.4:
+                ccl = int(rng.choice([24_000, 1 << 16, 200_000]))
+                host = host_only(dtype, op)
+                if which == 0:      # AllReduce
+                    fits = (ccl // 2 // 128 * 128 // esz // n * n > 0 if host
+                            else oracle.sequence_max_count_per_loop(ccl, count, l0, n, esz, 128, algo == "rhd") is not None)
+                else:               # Reduce
+                    fits = oracle.sequence_max_count_per_loop(ccl, count, l0, n, esz, 4096, False) is not None
+                if not fits:
+                    ccl = 0
+            w.set_ccl_buffer_size(ccl)
+            seed = SWEEP_SEED + case * 139 + n
+            if which == 0:
+                run_ar(w, l0, l1, algo, dtype, op, count, seed, pad=pad, ccl=ccl)
+            elif which == 1:
+                run_rs(w, l0, l1, algo, dtype, op, max(1, count // n), seed, pad=pad)
+            else:
+                run_reduce(w, l0, l1, algo, dtype, op, count, int(rng.integers(0, n)), seed, ccl=ccl, pad=pad)
+    finally:
+        w.set_ccl_buffer_size(0)
+        w.close()
