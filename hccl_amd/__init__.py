@@ -66,6 +66,7 @@ class Algo(enum.IntEnum):
     MESH_SYMMETRIC = 6
     MESH_CHUNK = 7
     MESH_TWO_SHOT = 8
+    MESH_CONCUR = 9
 
 
 class HcclSendRecvType(enum.IntEnum):

@@ -315,6 +315,10 @@ bool OrderOf(HcclAmdOpKind op, const std::string& t, HcclAmdAlgo* algo)
         *algo = op == HCCL_AMD_OP_ALL_REDUCE ? HCCL_AMD_ALGO_RING : HCCL_AMD_ALGO_MESH;
         return true;
     }
+    if (t == "meshconcur" && op == HCCL_AMD_OP_ALL_REDUCE) {
+        *algo = HCCL_AMD_ALGO_MESH_CONCUR;   // Aicpu AllReduce Sole MeshConcur: mesh ReduceScatter + AllGather
+        return true;
+    }
     if (op == HCCL_AMD_OP_REDUCE && IsMeshFamily(t)) {
         *algo = t == "meshtwoshot" ? HCCL_AMD_ALGO_MESH_TWO_SHOT : HCCL_AMD_ALGO_MESH;
         return true;

@@ -586,6 +586,14 @@ HcclResult BuildFoldPlan(HcclAmdOpKind op, HcclAmdAlgo algo, uint32_t n, FoldPla
         case HCCL_AMD_ALGO_MESH_CHUNK:
             plan->segmentsAreSubs = true;
             return MeshChunk(n, plan);
+        case HCCL_AMD_ALGO_MESH_CONCUR:
+            // AllReduce only: slice k of a loop is folded like rank k's ReduceScatter output (reference
+            // ins_v2_all_reduce_two_shot_sole_executor.cc:395-398: mesh ReduceScatter + AllGather).
+            if (!ar) {
+                return HCCL_E_NOT_SUPPORT;
+            }
+            plan->segmentsAreSubs = true;
+            return MeshReduceScatter(n, plan);
         case HCCL_AMD_ALGO_MESH_TWO_SHOT:
             return HCCL_E_NOT_SUPPORT;   // Reduce only; AllReduce's two-shot folds in the MESH order
         default:

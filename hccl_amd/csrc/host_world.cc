@@ -167,7 +167,8 @@ bool ParseAlgoName(const std::string& s, HcclAmdAlgo* algo)
         {"mesh", HCCL_AMD_ALGO_MESH}, {"ring", HCCL_AMD_ALGO_RING}, {"rhd", HCCL_AMD_ALGO_RHD},
         {"nhr", HCCL_AMD_ALGO_NHR}, {"order_preserved", HCCL_AMD_ALGO_ORDER_PRESERVED},
         {"aiv_mesh", HCCL_AMD_ALGO_AIV_MESH}, {"mesh_symmetric", HCCL_AMD_ALGO_MESH_SYMMETRIC},
-        {"mesh_chunk", HCCL_AMD_ALGO_MESH_CHUNK}, {"mesh_two_shot", HCCL_AMD_ALGO_MESH_TWO_SHOT}};
+        {"mesh_chunk", HCCL_AMD_ALGO_MESH_CHUNK}, {"mesh_two_shot", HCCL_AMD_ALGO_MESH_TWO_SHOT},
+        {"mesh_concur", HCCL_AMD_ALGO_MESH_CONCUR}};
     for (const auto& e : table) {
         if (s == e.name) {
             *algo = e.algo;
@@ -184,7 +185,7 @@ bool AlgoFitsOp(HcclAmdOpKind kind, HcclAmdAlgo algo)
         case HCCL_AMD_OP_ALL_REDUCE:
             return algo != HCCL_AMD_ALGO_AIV_MESH && algo != HCCL_AMD_ALGO_MESH_TWO_SHOT;
         case HCCL_AMD_OP_REDUCE_SCATTER:
-            return algo != HCCL_AMD_ALGO_MESH_TWO_SHOT;
+            return algo != HCCL_AMD_ALGO_MESH_TWO_SHOT && algo != HCCL_AMD_ALGO_MESH_CONCUR;
         case HCCL_AMD_OP_REDUCE:
             return algo == HCCL_AMD_ALGO_MESH || algo == HCCL_AMD_ALGO_RING || algo == HCCL_AMD_ALGO_MESH_TWO_SHOT ||
                    algo == HCCL_AMD_ALGO_NHR || algo == HCCL_AMD_ALGO_RHD;

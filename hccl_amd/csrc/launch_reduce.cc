@@ -109,7 +109,7 @@ HcclAmdAlgo EffectiveAlgo(const World* w, HcclAmdOpKind kind, HcclDataType dtype
     const bool hostOnly = op == HCCL_REDUCE_PROD || dtype == HCCL_DATA_TYPE_INT64 || dtype == HCCL_DATA_TYPE_UINT64 ||
                           dtype == HCCL_DATA_TYPE_FP64;
     if (hostOnly && (algo == HCCL_AMD_ALGO_NHR || algo == HCCL_AMD_ALGO_RHD || algo == HCCL_AMD_ALGO_MESH_CHUNK ||
-                     algo == HCCL_AMD_ALGO_AIV_MESH ||
+                     algo == HCCL_AMD_ALGO_AIV_MESH || algo == HCCL_AMD_ALGO_MESH_CONCUR ||
                      (algo == HCCL_AMD_ALGO_RING && kind == HCCL_AMD_OP_REDUCE_SCATTER))) {
         return HCCL_AMD_ALGO_MESH;
     }
@@ -547,6 +547,29 @@ HcclResult RunAllReduce(World* w, PendingOp& p, hipStream_t s)
             maxPerLoop = SoleMaxCountPerLoop(w->cclBytes, 1, esz);
             if (maxPerLoop == 0) {
                 Log(1, "AllReduce: the staging buffer of %llu bytes holds no element",
+                    static_cast<unsigned long long>(w->cclBytes));
+                return HCCL_E_INTERNAL;
+            }
+        }
+        for (uint64_t done = 0; done < p.count;) {
+            const uint64_t len = std::min(p.count - done, maxPerLoop);
+            rc = launchLoop(done, len, len / n);
+            if (rc != HCCL_SUCCESS) {
+                return rc;
+            }
+            done += len;
+        }
+        return HCCL_SUCCESS;
+    }
+    if (algo == HCCL_AMD_ALGO_MESH_CONCUR) {
+        // Slices of floor(len / n) elements, the last slice takes the rest; loops of half the staging buffer,
+        // floored to 128 bytes and a multiple of n elements (reference
+        // ins_v2_all_reduce_two_shot_sole_executor.cc:236-237, 328-340).
+        uint64_t maxPerLoop = p.count;
+        if (w->cclBytes != 0) {
+            maxPerLoop = w->cclBytes / 2 / 128 * 128 / esz / n * n;
+            if (maxPerLoop == 0) {
+                Log(1, "AllReduce: the staging buffer of %llu bytes holds no loop of the mesh two-shot executor",
                     static_cast<unsigned long long>(w->cclBytes));
                 return HCCL_E_INTERNAL;
             }

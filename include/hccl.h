@@ -256,12 +256,18 @@ typedef enum {
      * reduce_auto_selector.cc:346-351).  Reduce under MESH folds rank 0's input first and the others ascending
      * (reduce_mesh_1D.cc:268-300). */
     HCCL_AMD_ALGO_MESH_TWO_SHOT = 8,
+    /* AllReduce only: the reference's two-shot executor over one mesh (Aicpu AllReduce Sole MeshConcur, reference
+     * ins_v2_all_reduce_two_shot_sole_executor.cc:228-250, 328-392): a mesh ReduceScatter, then an AllGather.  Every
+     * loop is cut into N slices of floor(len / N) elements, the last slice taking the rest, and slice k starts from
+     * rank k's input and adds the other ranks ascending (ins_temp_reduce_scatter_mesh_1D.cc:203-237); loops hold half
+     * of the staging buffer, floored to 128 bytes and a multiple of N elements. */
+    HCCL_AMD_ALGO_MESH_CONCUR = 9,
     HCCL_AMD_ALGO_COUNT
 } HcclAmdAlgo;
 
 /* Sets the algorithm every later call of `op` on comm's world uses.  Also settable before
  * world creation through HCCL_AMD_ALGO="allreduce=rhd;reducescatter=nhr;reduce=mesh_two_shot".  Calls with PROD or a 64-bit type
- * fold in the MESH order under NHR, RHD, MESH_CHUNK, AIV_MESH and (ReduceScatter) RING: the reference does not
+ * fold in the MESH order under NHR, RHD, MESH_CHUNK, MESH_CONCUR, AIV_MESH and (ReduceScatter) RING: the reference does not
  * offer those templates for them and falls back to its host-reduce mesh templates
  * (op_common/selector/cost_table.cc:104-131). */
 HcclResult HcclAmdSetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo algo);
@@ -271,7 +277,7 @@ HcclResult HcclAmdGetAlgo(HcclComm comm, HcclAmdOpKind op, HcclAmdAlgo* algo);
  * Staging-buffer loops.  The reference's executors move every AllReduce through a bounded buffer: the count is
  * cut into loops and each loop is sliced afresh (ins_v2_all_reduce_sole_executor.cc:241-300,
  * ins_v2_all_reduce_sequence_executor_aicpu.cc:645-760), so under the orders whose fold depends on the slice
- * (NHR, RHD, MESH_CHUNK) the association order of an element depends on the loop it falls in.  No staging exists here;
+ * (NHR, RHD, MESH_CHUNK, MESH_CONCUR) the association order of an element depends on the loop it falls in.  No staging exists here;
  * `bytes` only tells the library which loop boundaries to reproduce: 0 (default) = one loop.  The environment
  * variable HCCL_BUFFSIZE (MB), when set at world creation, gives MB * 2^20 - 2^20 bytes
  * (src/common/op_graph/hccl_op_utils.cc:204-225); a value its parser rejects makes every collective return
@@ -352,7 +358,7 @@ HcclResult HcclAmdGetLevel1GroupSize(HcclComm comm, uint32_t* groupsPerLevel1Gro
  * The reference's HCCL_ALGO setting ("allreduce:sequence{level0=mesh_concur,level1=rhd};reducescatter:nhr;..."; grammar
  * and vocabulary of src/common/alg_parse.cc:27-437) is read at world creation and selects the fold order of
  * AllReduce, ReduceScatter(V) and Reduce: sole{mesh | mesh_one_shot | mesh_two_shot} -> MESH (Reduce: mesh_two_shot ->
- * MESH_TWO_SHOT), sole{mesh_chunk...} -> MESH_CHUNK, sole{nhr...} -> NHR, sole{nhr_aicpu_reduce} -> the host-reduce
+ * MESH_TWO_SHOT), sole{mesh_concur} for AllReduce -> MESH_CONCUR, sole{mesh_chunk...} -> MESH_CHUNK, sole{nhr...} -> NHR, sole{nhr_aicpu_reduce} -> the host-reduce
  * order (RING for AllReduce, MESH for ReduceScatter and Reduce), sole{rhd | hd | hd_aicpu_reduce} -> RHD, strictordered{...} ->
  * ORDER_PRESERVED, sequence{<mesh...>, <template>[, <the same template>]} -> that template between level-0 groups
  * and, where the world has them, between level-1 groups (AllReduce, ReduceScatter, Reduce; a mesh-chunk template

@@ -267,6 +267,9 @@ def all_reduce(ins, outs, count, dtype, op, acc=ACC_FP32, algo="mesh", max_count
     if algo == "mesh_chunk":
         return _reduce_call("orc_all_reduce_mesh_chunk", ins, outs, count, dtype, op, acc,
                             ctypes.c_uint64(max_count_per_loop))
+    if algo == "mesh_concur":
+        return _reduce_call("orc_all_reduce_mesh_concur", ins, outs, count, dtype, op, acc,
+                            ctypes.c_uint64(max_count_per_loop))
     raise ValueError(algo)
 
 

@@ -755,6 +755,66 @@ int orc_all_reduce_two_shot(uint32_t n, const void* const* in, void* const* out,
     return ORC_OK;
 }
 
+/* AllReduce of the two-shot executor over one mesh (ins_v2_all_reduce_two_shot_sole_executor.cc; registered as
+ * Aicpu AllReduce Sole MeshConcur, :395-398): per loop a mesh ReduceScatter on n slices of floor(len / n) elements,
+ * the last slice taking the rest (:236-237), slice k folded by rank k, its own input first and the other ranks
+ * ascending (reduce_scatter_mesh_1D.cc:203-237), then the AllGather.  Loops of maxCountPerLoop elements floored to
+ * a multiple of n (:335-336), the last one taking what is left (:354); 0 = one loop. */
+int orc_all_reduce_mesh_concur(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                               int accMode, uint64_t maxCountPerLoop)
+{
+    red_t r;
+    int rc = red_init(&r, dtype, op, accMode);
+    if (rc != ORC_OK) {
+        return rc;
+    }
+    if (count == 0) {
+        return ORC_OK;
+    }
+    if (maxCountPerLoop == 0) {
+        maxCountPerLoop = UINT64_MAX / 2;
+    }
+    maxCountPerLoop = maxCountPerLoop / n * n;
+    if (maxCountPerLoop == 0) {
+        return ORC_E_INTERNAL;
+    }
+    void* acc = malloc(count * r.asz);
+    void* tmp = malloc(count * r.asz);
+    uint8_t* res = (uint8_t*)malloc(count * r.esz);
+    if (!acc || !tmp || !res) {
+        free(acc);
+        free(tmp);
+        free(res);
+        return ORC_E_INTERNAL;
+    }
+    for (uint64_t done = 0; done < count;) {
+        uint64_t len = count - done < maxCountPerLoop ? count - done : maxCountPerLoop;
+        uint64_t slice = len / n;
+        for (uint32_t k = 0; k < n; ++k) {
+            uint64_t off = done + (uint64_t)k * slice;
+            uint64_t cur = k == n - 1 ? len - slice * (n - 1) : slice;
+            if (cur == 0) {
+                continue;
+            }
+            red_widen(&r, cbytes(in[k]) + off * r.esz, acc, cur);
+            for (uint32_t t = 0; t < n; ++t) {
+                if (t != k) {
+                    red_pair_from_storage(&r, acc, cbytes(in[t]) + off * r.esz, cur, tmp);
+                }
+            }
+            red_narrow(&r, acc, res + off * r.esz, cur);
+        }
+        done += len;
+    }
+    for (uint32_t d = 0; d < n; ++d) {
+        memcpy(out[d], res, count * r.esz);
+    }
+    free(acc);
+    free(tmp);
+    free(res);
+    return ORC_OK;
+}
+
 /* Two-shot, symmetric-memory variant (two_shot.cc:341-357 with supportSymmetricMemAccess_): slice k starts
  * from rank k's own input slice, then the other ranks ascending; every rank gets every slice. */
 int orc_all_reduce_two_shot_symmetric(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype,

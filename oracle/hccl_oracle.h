@@ -183,6 +183,10 @@ int orc_sequence_max_count_per_loop(uint64_t cclBytes, uint64_t count, uint32_t 
                                     uint64_t align, int rhdTail, uint64_t* maxCount, uint64_t* resultElems);
 uint64_t orc_sequence_select_loop_count(uint64_t remaining, uint64_t maxCountPerLoop, uint32_t l0,
                                         uint64_t resultElems);
+/* AllReduce of the two-shot executor over one mesh (ins_v2_all_reduce_two_shot_sole_executor.cc): slices of
+ * floor(len / n) elements, the last taking the rest, slice k folded own input first; maxCountPerLoop 0 = one loop. */
+int orc_all_reduce_mesh_concur(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op,
+                               int accMode, uint64_t maxCountPerLoop);
 /* Reduce along the NHR step tree on slices of ceil(len / n) elements (reduce_nhr.cc); only out[root] is written. */
 int orc_reduce_nhr(uint32_t n, const void* const* in, void* const* out, uint64_t count, int dtype, int op, int accMode,
                    uint32_t root, uint64_t maxCountPerLoop);

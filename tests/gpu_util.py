@@ -73,7 +73,7 @@ class _EmuStream:
 
 ALGO_BY_NAME = {"mesh": Algo.MESH, "ring": Algo.RING, "rhd": Algo.RHD, "nhr": Algo.NHR,
                 "order_preserved": Algo.ORDER_PRESERVED, "aiv_mesh": Algo.AIV_MESH, "mesh_symmetric": Algo.MESH_SYMMETRIC,
-                "mesh_chunk": Algo.MESH_CHUNK, "mesh_two_shot": Algo.MESH_TWO_SHOT}
+                "mesh_chunk": Algo.MESH_CHUNK, "mesh_two_shot": Algo.MESH_TWO_SHOT, "mesh_concur": Algo.MESH_CONCUR}
 
 
 def require_library_on_gpu():

@@ -97,7 +97,7 @@ def pad_of(pad, r, which):
 def order_of(algo, dtype, op, reduce_scatter):
     """PROD and the 64-bit types are not offered by the reference's write-reduce templates: mesh order."""
     host_only = op == PROD or dtype in (DT.INT64, DT.UINT64, DT.FP64)
-    if host_only and (algo in ("nhr", "rhd", "mesh_chunk", "aiv_mesh") or (algo == "ring" and reduce_scatter)):
+    if host_only and (algo in ("nhr", "rhd", "mesh_chunk", "mesh_concur", "aiv_mesh") or (algo == "ring" and reduce_scatter)):
         return "mesh"
     return algo
 
@@ -165,7 +165,7 @@ def test_reduce_scatter_type_matrix(world8, dtype, op):
 def test_all_reduce_algorithms_and_ragged_counts(n):
     w = World(n)
     try:
-        for algo in ("mesh", "ring", "rhd", "nhr", "order_preserved", "mesh_symmetric", "mesh_chunk"):
+        for algo in ("mesh", "ring", "rhd", "nhr", "order_preserved", "mesh_symmetric", "mesh_chunk", "mesh_concur"):
             for count in (1, 3, 17, 129, 1023, 4093, 65_543):
                 run_all_reduce(w, DT.FP32, SUM, count, algo, seed=n * 1000 + count)
             run_all_reduce(w, DT.FP32, MAX, 2_051, algo, seed=n)
@@ -393,6 +393,7 @@ def test_all_reduce_as_fold_and_fan_out(monkeypatch, n):
         run_all_reduce(w, DT.INT32, SUM, 200_003, "nhr", seed=seed + 8)     # sub-segments longer than a piece
         run_all_reduce(w, DT.FP32, SUM, 33_333, "order_preserved", seed=seed + 9)
         run_all_reduce(w, DT.FP32, MAX, 20_011, "mesh_symmetric", seed=seed + 11, in_place=True)
+        run_all_reduce(w, DT.FP16, SUM, 40_009, "mesh_concur", seed=seed + 16, pad=2)   # uneven last slice
         run_all_reduce(w, DT.INT8, SUM, 30_011, "mesh_chunk", seed=seed + 12)   # pieces of whole slices
         run_all_reduce(w, DT.FP32, SUM, 257, "mesh_chunk", seed=seed + 14)      # slices shorter than a piece, short last slice
         run_all_reduce(w, DT.BFP16, SUM, 3 * n + 1, "mesh_chunk", seed=seed + 15, pad=2)

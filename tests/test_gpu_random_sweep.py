@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 SWEEP_SEED = int(os.environ.get("HCCL_AMD_TEST_SWEEP_SEED", "90000"))
 
 TYPES = [DT.INT8, DT.INT16, DT.INT32, DT.INT64, DT.UINT64, DT.FP16, DT.BFP16, DT.FP32, DT.FP64]
-AR_ALGOS = ["mesh", "ring", "rhd", "nhr", "order_preserved", "mesh_symmetric", "mesh_chunk"]
+AR_ALGOS = ["mesh", "ring", "rhd", "nhr", "order_preserved", "mesh_symmetric", "mesh_chunk", "mesh_concur"]
 RS_ALGOS = ["mesh", "ring", "nhr", "rhd", "order_preserved", "aiv_mesh", "mesh_symmetric", "mesh_chunk"]
 
 
@@ -73,12 +73,16 @@ def test_random_reduce_cases(monkeypatch, n, form):
             if rng.random() < 0.5:
                 algo = AR_ALGOS[rng.integers(0, len(AR_ALGOS))]
                 loop, ccl = 0, 0
-                if algo in ("nhr", "rhd", "mesh_chunk") and rng.random() < 0.4 and op != PROD and esz < 8:
+                if algo in ("nhr", "rhd", "mesh_chunk", "mesh_concur") and rng.random() < 0.4 and op != PROD and esz < 8:
                     ccl = int(rng.choice([4096, 20_000, 1 << 16]))
                     if algo == "nhr":
                         loop = oracle.sole_max_count_per_loop(ccl, 1, esz)
                     elif algo == "mesh_chunk":
                         loop = oracle.sole_max_count_per_loop(ccl, 2, esz)
+                    elif algo == "mesh_concur":
+                        loop = ccl // 2 // 128 * 128 // esz // n * n
+                        if loop == 0:
+                            ccl = 0
                     else:
                         rc, loop = oracle.rhd_max_count_per_loop(ccl, count, n, esz)
                         if rc != 0:

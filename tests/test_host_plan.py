@@ -104,8 +104,10 @@ def test_every_program_uses_every_rank_once(n):
         for algo in Algo:
             if kind == OpKind.ALL_REDUCE and algo == Algo.AIV_MESH:
                 continue
+            if kind != OpKind.ALL_REDUCE and algo == Algo.MESH_CONCUR:
+                continue
             if (kind == OpKind.REDUCE) != (algo == Algo.MESH_TWO_SHOT) and not (
-                    kind == OpKind.REDUCE and algo in (Algo.MESH, Algo.RING)):
+                    kind == OpKind.REDUCE and algo in (Algo.MESH, Algo.RING, Algo.NHR)):
                 continue
             for prog in hccl_amd.fold_programs(kind, algo, n):
                 assert sorted(program_ranks(prog)) == list(range(n)), (kind, algo, n)

@@ -424,3 +424,55 @@ def test_every_division_of_up_to_64_ranks_into_levels_has_programs_the_kernel_ca
                     assert len(progs) == n
                     longest = max(longest, max(len(p) for p in progs))
     assert longest <= 320
+
+
+@pytest.mark.parametrize("n", [2, 3, 5, 6, 8, 12, 33])
+def test_all_reduce_of_the_two_shot_executor_over_one_mesh(orc, n):
+    """Aicpu AllReduce Sole MeshConcur (ins_v2_all_reduce_two_shot_sole_executor.cc): a mesh ReduceScatter on slices
+    of floor(len / n) elements with the rest in the last, slice k folded own input first, then the AllGather.  Where
+    n divides the count the slices are those of the symmetric two-shot order (pinned elsewhere); all ranks in one
+    level-0 group is the same executor seen from the two-level one; uneven counts by hand."""
+    rng = np.random.default_rng(23 * n)
+    for count in (n * 6, n * 6 + 1, n * 6 + n - 1, n - 1, 1):
+        for op, gen in ((SUM, wide), (MIN, tricky)):
+            ins = gen(rng, n, count)
+            got = [np.zeros(count, np.float32) for _ in range(n)]
+            assert orc.all_reduce(ins, got, count, F32, op, algo="mesh_concur") == 0
+            if count % n == 0:
+                want = [np.zeros(count, np.float32) for _ in range(n)]
+                assert orc.all_reduce(ins, want, count, F32, op, algo="mesh_symmetric") == 0
+                assert same(got[0], want[0]), (n, count, op)
+            want = [np.zeros(count, np.float32) for _ in range(n)]
+            assert orc.all_reduce_two_level(ins, want, count, F32, op, n, "nhr") == 0
+            assert same(got[n - 1], want[n - 1]), (n, count, op)
+            by_hand = np.zeros(count, np.float32)
+            slice_len = count // n
+            for k in range(n):
+                lo = k * slice_len
+                hi = count if k == n - 1 else lo + slice_len
+                by_hand[lo:hi] = box(ins, n, 0, k, lo, hi, op)
+            for r in range(n):
+                assert same(got[r], by_hand), (n, count, op, r)
+    # loops: floored to a multiple of n, each cut afresh
+    count, per_loop = 11 * n + 3, 4 * n + n - 1
+    ins = wide(rng, n, count)
+    got = [np.zeros(count, np.float32) for _ in range(n)]
+    assert orc.all_reduce(ins, got, count, F32, SUM, algo="mesh_concur", max_count_per_loop=per_loop) == 0
+    want = np.zeros(count, np.float32)
+    for lo in range(0, count, 4 * n):
+        hi = min(count, lo + 4 * n)
+        part = [x[lo:hi].copy() for x in ins]
+        out = [np.zeros(hi - lo, np.float32) for _ in range(n)]
+        assert orc.all_reduce(part, out, hi - lo, F32, SUM, algo="mesh_concur") == 0
+        want[lo:hi] = out[0]
+    assert same(got[0], want)
+    # the library's programs: those of the mesh ReduceScatter, one per slice
+    progs = hccl_amd.fold_programs(OpKind.ALL_REDUCE, Algo.MESH_CONCUR, n)
+    assert progs == hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.MESH, n)
+    with pytest.raises(hccl_amd.HcclError) as e:
+        hccl_amd.fold_programs(OpKind.REDUCE_SCATTER, Algo.MESH_CONCUR, n)
+    assert e.value.code == 5
+    sel = hccl_amd.select_from_hccl_algo
+    assert sel("allreduce:sole{mesh_concur}", OpKind.ALL_REDUCE)[1:] == (Algo.MESH_CONCUR, False)
+    assert sel("mesh_concur", OpKind.REDUCE_SCATTER)[1:] == (Algo.MESH, False)
+    assert sel("allreduce:sequence{mesh,mesh_concur}", OpKind.ALL_REDUCE)[1] is None

@@ -38,7 +38,7 @@ SIZES = {"INT8": 1, "UINT8": 1, "INT16": 2, "UINT16": 2, "FP16": 2, "BFP16": 2, 
 FILL = 0xAB
 NAMES = {Algo.MESH: "mesh", Algo.RING: "ring", Algo.RHD: "rhd", Algo.NHR: "nhr", Algo.MESH_CHUNK: "mesh_chunk",
          Algo.ORDER_PRESERVED: "order_preserved", Algo.MESH_TWO_SHOT: "mesh_two_shot", Algo.AIV_MESH: "aiv_mesh",
-         Algo.MESH_SYMMETRIC: "mesh_symmetric"}
+         Algo.MESH_SYMMETRIC: "mesh_symmetric", Algo.MESH_CONCUR: "mesh_concur"}
 
 
 @pytest.fixture(scope="module", autouse=True)
