@@ -405,6 +405,9 @@ def test_what_hccl_algo_selects_for_three_levels_and_for_reduce():
     assert sel("reduce:sole{nhr_aicpu_reduce}", OpKind.REDUCE)[1:] == (Algo.MESH, False)
     assert sel("reduce:sole{mesh_two_shot}", OpKind.REDUCE)[1:] == (Algo.MESH_TWO_SHOT, False)
     assert sel("reduce:sole{mesh_chunk}", OpKind.REDUCE)[1] is None
+    # Aicpu Reduce Sequence NHRAicpuReduce NHR: mesh inside the groups, the host-reduce fold between them
+    assert sel("reduce:sequence{nhr_aicpu_reduce,nhr}", OpKind.REDUCE)[1:] == (Algo.MESH, True)
+    assert sel("sequence{nhr_aicpu_reduce,nhr}", OpKind.ALL_REDUCE)[1] is None
 
 
 def test_every_division_of_up_to_64_ranks_into_levels_has_programs_the_kernel_can_run():
