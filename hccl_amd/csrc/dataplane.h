@@ -83,13 +83,18 @@ struct ReduceHot {
     uint32_t leadFromSrc;    // wavefronts start on a 1 KiB boundary of the sources instead of the destination's
     uint32_t storeWaves;     // > 1: workgroups of 64 * storeWaves threads, wavefront 0 folds and wavefront k stores to
                              // destinations k, k + storeWaves, ... (threads must be 64, dstOwn 0); 0 or 1: every wavefront
-                             // folds and stores its own tile
+                             // folds and stores its own tile.  With kStoreWavesAllFold added: every wavefront folds a
+                             // tile of its own and stores the tiles of all to its destinations (flat programs only)
     uint32_t varGroups;      // groups of unequal length, see below
 };
 
 // vecBatch of the form for short launches: eight-leaf batches, two adjacent tiles per wavefront (threads 64, no shared
 // stores, uniform groups; blocksPerSub counts pairs of tiles).
 constexpr uint32_t kVecBatchPair = 0x108;
+// Flag in storeWaves: the workgroup's wavefronts fold one tile each and exchange the results through LDS (2 KiB of
+// dynamic LDS per wavefront), so that wavefront k writes storeWaves neighbouring tiles to destinations k,
+// k + storeWaves, ...: one or two long store streams per wavefront instead of a short piece of every stream.
+constexpr uint32_t kStoreWavesAllFold = 0x100;
 
 struct ReduceArgs : ReduceHot {
     const void* src[kMaxRanks];

@@ -290,6 +290,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->twoKernelMode < 0 || w->twoKernelMode > 1) {
         w->twoKernelMode = 2;
     }
+    w->reduceAllFold = EnvInt("HCCL_AMD_REDUCE_ALL_FOLD", -1);
+    if (w->reduceAllFold != 0 && (w->reduceAllFold < 2 || w->reduceAllFold > static_cast<int>(kMaxReduceThreads / 64))) {
+        w->reduceAllFold = -1;
+    }
     w->reducePair = EnvInt("HCCL_AMD_REDUCE_PAIR", 2);
     if (w->reducePair < 0 || w->reducePair > 1) {
         w->reducePair = 2;

@@ -64,6 +64,21 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
         }
     }
     a.blocksPerSub = BlocksPerSub(w, longest, a.vecOk ? esz : 16 /* one element per lane */, subs, a.threads);
+    uint32_t exchangeLds = 0;
+    if (a.vecOk && a.threads == 64 && a.storeWaves <= 1 && !oneStream && !a.varGroups && plan.maxDepth == 1 &&
+        w->reduceAllFold != 0 && w->storeWaves == 0) {
+        // every wavefront folds a tile and stores the tiles of its workgroup to its own destinations (forced: wherever
+        // the form fits; by itself: where it was measured, a result that is one sub-segment)
+        const uint32_t waves = w->reduceAllFold > 0 ? static_cast<uint32_t>(w->reduceAllFold)
+                               : (subs == 1 && w->reduceBatch == 0 && w->reducePair != 1)
+                                     ? policy::AllFoldWaves(a.nDst, a.total * esz) : 0u;
+        if (waves > 1) {
+            a.vecBatch = 8;   // the form exists in the eight-leaf kernels
+            a.storeWaves = waves | kStoreWavesAllFold;
+            a.blocksPerSub = (a.blocksPerSub + waves - 1) / waves;   // a workgroup takes `waves` tiles
+            exchangeLds = 2u * waves * 1024u;
+        }
+    }
     if (a.vecOk && a.threads == 64 && a.storeWaves <= 1 && !a.varGroups && plan.maxLeaves <= 8 && plan.maxDepth == 1 &&
         (w->reduceBatch == 0 || w->reducePair == 1) &&
         (w->reducePair != 2 ? w->reducePair == 1 : policy::PairTiles(w->n, oneStream, a.total * esz))) {
@@ -87,7 +102,7 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     if (blocks == 0 || blocks > 0x7FFFFFFFull) {
         return HCCL_E_INTERNAL;
     }
-    const uint32_t lds = (plan.maxDepth - 1) * ReduceAccBytes(dtype, op) * a.threads;
+    const uint32_t lds = exchangeLds != 0 ? exchangeLds : (plan.maxDepth - 1) * ReduceAccBytes(dtype, op) * a.threads;
     HIP_OK(LaunchReduce(a, dtype, op, static_cast<uint32_t>(blocks), lds, s));
     return HCCL_SUCCESS;
 }

@@ -864,6 +864,45 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
     }
     const uint64_t bodyEnd = head + nVec * W;
     const uint64_t nScalar = head + (len - bodyEnd);
+    if (!kPair && VB == 8 && (h.storeWaves & kStoreWavesAllFold) != 0) {
+        // (Built into the eight-leaf batch only: the sixteen-leaf kernels have no scalar registers to spare.)
+        // Every wavefront of the workgroup folds a tile of its own, parks the result in LDS, and after the barrier
+        // writes the tiles of all wavefronts to its destinations: wavefront k owns destinations k, k + waves, ...
+        // A launch that is a single generation of wavefronts (a few MiB per rank, many destinations) otherwise ends
+        // with every wavefront writing 1 KiB to every stream at the same moment; this way a wavefront writes
+        // `waves` KiB in a row to one or two of them.  The programs are flat (the launcher's caller has checked), so
+        // the dynamic LDS holds no accumulator stack and is the exchange area: two rounds of `waves` tiles, which
+        // makes one barrier per round enough.  The trip count is the same for every wavefront.
+        const uint32_t waves = h.storeWaves & 0xFFu;
+        U32x4* const parked = reinterpret_cast<U32x4*>(accStack);
+        const uint32_t wave = threadIdx.x >> 6;
+        const uint32_t lane = threadIdx.x & 63u;
+        const uint64_t span = static_cast<uint64_t>(waves) * 64;
+        uint32_t slot = 0;
+        for (uint64_t base = static_cast<uint64_t>(blk) * span; base < nVec + lead; base += static_cast<uint64_t>(blocksHere) * span) {
+            const uint64_t u = base + wave * 64 + lane;
+            if (u >= lead && u < nVec + lead) {
+                const Pack<S, W> out = ReduceValue<E, W, VB>(pv, accStack, args, h, head + (u - lead) * W, preloaded);
+                parked[(slot * waves + wave) * 64 + lane] = __builtin_bit_cast(U32x4, out);
+            }
+            __syncthreads();
+            for (uint32_t t = 0; t < waves; ++t) {
+                const uint64_t ut = base + t * 64 + lane;
+                if (ut >= lead && ut < nVec + lead) {
+                    const Pack<S, W> out = __builtin_bit_cast(Pack<S, W>, parked[(slot * waves + t) * 64 + lane]);
+                    StoreResult<S, W, false>(args, h, out, dstOff + head + (ut - lead) * W, firstDstAddr, wave, waves);
+                }
+            }
+            slot ^= 1u;
+        }
+        if (wave == 0) {
+            for (uint64_t i = static_cast<uint64_t>(blk) * 64 + lane; i < nScalar; i += static_cast<uint64_t>(blocksHere) * 64) {
+                const uint64_t e = i < head ? i : i - head + bodyEnd;
+                ReduceOne<E, 1, 8>(pv, accStack, args, h, e, dstOff, firstDstAddr);
+            }
+        }
+        return;
+    }
     if (!kPair && h.storeWaves > 1) {
         // Stores split over the wavefronts of the workgroup (h.threads == 64 lanes fold, 64 * storeWaves run):
         // wavefront 0 folds the tile and parks the result in LDS, wavefront k writes it to destinations k,

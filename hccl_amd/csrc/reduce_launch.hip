@@ -30,10 +30,17 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
     }
     uint32_t threads = args.threads;
     if (args.storeWaves > 1) {
-        if (args.threads != 64 || args.dstOwn != 0 || args.storeWaves * 64 > kMaxReduceThreads) {
+        const uint32_t waves = args.storeWaves & 0xFFu;
+        const bool allFold = (args.storeWaves & kStoreWavesAllFold) != 0;
+        if ((args.storeWaves & ~(kStoreWavesAllFold | 0xFFu)) != 0 || waves < 2 || args.threads != 64 ||
+            args.dstOwn != 0 || waves * 64 > kMaxReduceThreads) {
             return hipErrorInvalidValue;
         }
-        threads = 64 * args.storeWaves;
+        // the wavefronts that all fold exchange their tiles through the dynamic LDS: two rounds of `waves` KiB
+        if (allFold && (args.varGroups != 0 || batch != 8 || ldsBytes < 2u * waves * 1024u)) {
+            return hipErrorInvalidValue;
+        }
+        threads = 64 * waves;
     }
     // Uniform geometry: (workgroups per sub-segment, sub-segments, groups), consecutive workgroups on consecutive
     // positions of a sub-segment as before; groups of unequal length own runs of a one-dimensional grid.

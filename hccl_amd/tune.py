@@ -101,7 +101,8 @@ def all_reduce_rows(torch, h, ranks, mibs, rounds):
 
 
 def all_reduce_small_rows(torch, h, ranks, kibs, rounds):
-    print("# AllReduce fp32 SUM in rank order, a few MiB per rank: one tile per wavefront, two, the library's own choice "
+    print("# AllReduce fp32 SUM in rank order, a few MiB per rank: one tile per wavefront, two, workgroups of 2 / 3 / 4 "
+          "wavefronts that exchange their tiles and store one or two streams each, the library's own choice "
           "(collectives issued with their arguments converted once)")
     rows = []
     for n in ranks:
@@ -126,7 +127,10 @@ def all_reduce_small_rows(torch, h, ranks, kibs, rounds):
                     groups[k]()
                 return comms, step
 
-            forms = [("one", {"HCCL_AMD_REDUCE_PAIR": "0"}), ("pair", {"HCCL_AMD_REDUCE_PAIR": "1"}), ("auto", {})]
+            forms = [("one", {"HCCL_AMD_REDUCE_PAIR": "0", "HCCL_AMD_REDUCE_ALL_FOLD": "0"}),
+                     ("pair", {"HCCL_AMD_REDUCE_PAIR": "1", "HCCL_AMD_REDUCE_ALL_FOLD": "0"}),
+                     ("fold2", {"HCCL_AMD_REDUCE_ALL_FOLD": "2"}), ("fold3", {"HCCL_AMD_REDUCE_ALL_FOLD": "3"}),
+                     ("fold4", {"HCCL_AMD_REDUCE_ALL_FOLD": "4"}), ("auto", {})]
             fracs = _forms(torch, h, make_step, forms, per_set, rounds, 200)
             us = "/".join("%.1f" % (per_set / (v * HBM_PEAK) * 1e6) for v in fracs.values())
             rows.append(_row("%2d ranks x %5d KiB  %s us" % (n, kib, us), fracs))

@@ -466,6 +466,46 @@ def test_all_reduce_and_reduce_scatter_with_two_tiles_per_wavefront(monkeypatch,
         w.close()
 
 
+@pytest.mark.parametrize("n,waves,blocks", [(2, 2, 0), (3, 4, 24), (5, 3, 0), (8, 3, 0), (8, 4, 7), (16, 2, 0), (12, 3, 5)])
+def test_all_reduce_with_wavefronts_that_exchange_their_tiles_and_store_their_own_destinations(monkeypatch, n, waves, blocks):
+    """The form for many destinations and a few MiB per rank (every wavefront of a workgroup folds a tile, the results
+    change hands through LDS, wavefront k stores all of them to destinations k, k + waves, ...), forced for every size:
+    tile counts that the workgroup's wavefronts divide and do not, less than one tile, heads and tails off the 16-byte
+    grid, every element type, more wavefronts than destinations and fewer; with a small grid every workgroup strides
+    on.  Results cut into sub-segments with programs of their own take it too; orders whose programs nest and results
+    with one destination keep the plain kernel."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_ALL_FOLD", str(waves))
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "0")
+    if blocks:
+        monkeypatch.setenv("HCCL_AMD_REDUCE_BLOCKS", str(blocks))
+    w = World(n)
+    monkeypatch.delenv("HCCL_AMD_REDUCE_ALL_FOLD")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS")
+    if blocks:
+        monkeypatch.delenv("HCCL_AMD_REDUCE_BLOCKS")
+    try:
+        seed = 6500 + 10 * n + waves
+        for dtype in REDUCE_TYPES:
+            run_all_reduce(w, dtype, SUM, 20_011, "mesh", seed=seed)
+            seed += 1
+        for count in (1, 255, 256, 257, 256 * waves - 1, 256 * waves, 256 * waves + 1, 256 * (2 * waves + 1), 4096 * 3,
+                      4096 * 4 + 1, 100_003):
+            run_all_reduce(w, DT.FP32, SUM, count, "ring", seed=seed)            # 256 fp32 = one tile
+            seed += 1
+        run_all_reduce(w, DT.FP16, MAX, 33_333, "mesh", seed=seed, pad=2)        # unaligned: head and tail elements
+        run_all_reduce(w, DT.BFP16, SUM, 50_003, "mesh", seed=seed + 1, pad=lambda r, which: 2 * r + (6 if which == "recv" else 0))
+        run_all_reduce(w, DT.INT8, MIN, 9, "mesh", seed=seed + 2)                # less than one vector
+        run_all_reduce(w, DT.INT32, PROD, 4_099, "mesh", seed=seed + 3, in_place=True)
+        run_all_reduce(w, DT.FP64, SUM, 12_345, "mesh", seed=seed + 4, pad=lambda r, which: r + (3 if which == "recv" else 0))
+        run_all_reduce(w, DT.FP32, SUM, 70_001, "nhr", seed=seed + 5)            # nested program: form not taken
+        run_all_reduce(w, DT.FP32, SUM, 70_001, "mesh_symmetric", seed=seed + 6)     # n sub-segments, flat programs
+        run_all_reduce(w, DT.BFP16, SUM, 30_011, "mesh_concur", seed=seed + 7, pad=2)
+        run_all_reduce(w, DT.FP32, MIN, 9_973, "mesh_chunk", seed=seed + 8)
+        run_reduce_scatter(w, DT.FP32, SUM, 5_001, "mesh", seed=seed + 9)        # one result stream: form not taken
+    finally:
+        w.close()
+
+
 def test_prepared_group_issues_the_same_collective():
     """hccl_amd.prepared_group converts the arguments of a group's calls once; what it runs is the plain sequence
     HcclGroupStart, the entry points, HcclGroupEnd, and a bad argument still raises with the entry point's code."""

@@ -15,15 +15,15 @@ PROBE = r"""
 using namespace hccl_amd::policy;
 int main()
 {
-    const unsigned long long sizes[] = {1ull << 10, 1ull << 16, 1ull << 20, 3ull << 19, 2ull << 20, 4ull << 20, 6ull << 20,
-        (6ull << 20) + 1, 8ull << 20, (8ull << 20) + 1, 16ull << 20, 24ull << 20, 48ull << 20, 64ull << 20, 128ull << 20,
+    const unsigned long long sizes[] = {1ull << 10, 1ull << 16, 1ull << 20, 3ull << 19, 2ull << 20, 5ull << 19, 3ull << 20,
+        4ull << 20, 5ull << 20, 6ull << 20, (6ull << 20) + 1, 7ull << 20, (7ull << 20) + 1, 8ull << 20, (8ull << 20) + 1, 16ull << 20, 24ull << 20, 48ull << 20, 64ull << 20, 128ull << 20,
         160ull << 20, 256ull << 20, 1ull << 30, 8ull << 30};
     for (unsigned n = 1; n <= 64; ++n) {
         for (unsigned long long b : sizes) {
-            std::printf("%u %llu %d %d %d %d %u %u %u %u %d %d\n", n, b, (int)FoldThenFanOut(n, b),
+            std::printf("%u %llu %d %d %d %d %u %u %u %u %d %d %u\n", n, b, (int)FoldThenFanOut(n, b),
                         (int)GatherThenFanOut(n, b, true), (int)GatherThenFanOut(n, b, false), (int)PairTiles(n, false, b),
                         StoreWaves(n, b, 4), StoreWaves(n, b, 2), VecBatch(n, false, false), VecBatch(n, true, false),
-                        (int)FanOutStreamLoad(n, false), (int)FanOutStreamLoad(n, true));
+                        (int)FanOutStreamLoad(n, false), (int)FanOutStreamLoad(n, true), AllFoldWaves(n, b));
         }
     }
     return 0;
@@ -42,7 +42,7 @@ def table(tmp_path_factory):
     for line in subprocess.check_output([str(exe)], text=True).splitlines():
         v = [int(x) for x in line.split()]
         rows[(v[0], v[1])] = dict(fold=v[2], gather=v[3], gather_general=v[4], pair=v[5], waves4=v[6], waves2=v[7],
-                                  batch_many=v[8], batch_one=v[9], nt_single=v[10], nt_several=v[11])
+                                  batch_many=v[8], batch_one=v[9], nt_single=v[10], nt_several=v[11], all_fold=v[12])
     return rows
 
 
@@ -70,6 +70,21 @@ def test_small_worlds_never_split_into_two_kernels(table):
             assert not row["gather"] and not row["gather_general"], (n, b)
         if row["gather_general"]:
             assert row["gather"], (n, b)         # sources that share the destinations' alignment never fare worse
+
+
+def test_the_all_fold_form_has_one_window_of_sizes_and_fits_the_workgroup(table):
+    for n, rows in by_world(table).items():
+        flags = [row["all_fold"] for _, row in rows]
+        assert all(f in (0, 2, 3, 4) for f in flags), (n, flags)
+        on = [bool(f) for f in flags]
+        assert not on[0] and not on[-1], n
+        assert sum(1 for a, b in zip(on, on[1:]) if a != b) in (0, 2), (n, flags)
+        if n < 5 or n > 32:
+            assert not any(on), n
+    assert table[(8, 4 << 20)]["all_fold"] == 3 and table[(8, 7 << 20)]["all_fold"] == 2
+    assert table[(8, 3 << 20)]["all_fold"] == 0 and table[(8, (7 << 20) + 1)]["all_fold"] == 0
+    assert table[(16, 5 << 19)]["all_fold"] == 3 and table[(16, 2 << 20)]["all_fold"] == 0
+    assert table[(6, 4 << 20)]["all_fold"] == 0 and table[(6, 5 << 20)]["all_fold"] == 3
 
 
 def test_the_pair_form_has_one_window_of_sizes(table):

@@ -122,7 +122,11 @@ def test_reference_system_test_shape(case):
         host_only = op == OPS["PROD"] or dtype in (DT.INT64, DT.UINT64, DT.FP64)
         rng = np.random.default_rng(len(case["name"]) * 131 + count)
         what = "%s %s" % (case["name"], case["source"])
-        two_level = level0 > 1 and (sequence or not case["hccl_algo"]) and algo in ("rhd", "nhr")
+        # over levels: RHD / NHR unless a single-level executor was named, and the host-reduce fold where a sequence
+        # executor with it was named (the order is then MESH for every type)
+        two_level = level0 > 1 and ((sequence or not case["hccl_algo"]) and algo in ("rhd", "nhr") or
+                                    (sequence and algo == "mesh"))
+        host_only = host_only or (two_level and algo == "mesh")
         if kind == "reduce":
             root = case["root"]
             ins = [gen(dtype, op, rng, count) for _ in range(n)]
