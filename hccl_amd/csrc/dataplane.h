@@ -108,6 +108,23 @@ struct ReduceArgs : ReduceHot {
     uint64_t groupLenV[kMaxRanks];
 };
 
+// A fold of a few MiB per rank with everything the kernel needs in its arguments: up to eight leaves in fold order
+// (src[i] is leaf i's buffer) and up to eight destinations, all 16-byte aligned, `nVec` whole 16-byte vectors and
+// `tail` (< 16 / element size) elements behind them.  No program image, no tables: the one block of scalar loads that
+// fetches the arguments is all that stands in front of a wavefront's first vector load.
+constexpr uint32_t kDirectFoldMaxLeaves = 8;
+constexpr uint32_t kDirectFoldMaxDst = 8;
+constexpr uint32_t kDirectFoldMaxWaves = 8;    // wavefronts per workgroup, 1 KiB of dynamic LDS each
+struct DirectFoldArgs {
+    const void* src[kDirectFoldMaxLeaves];
+    void* dst[kDirectFoldMaxDst];
+    uint64_t nVec;
+    uint32_t nSrc;
+    uint32_t nDst;
+    uint32_t tail;
+    uint32_t waves;      // wavefronts per workgroup (filled by the launcher)
+};
+
 #if defined(__HIPCC__)
 // 16-byte streaming store to global memory, written through at system scope.  On this part that cache
 // policy sustains about 5 % more bandwidth than a non-temporal store when the stores are mixed with a
@@ -227,6 +244,9 @@ hipError_t LaunchMark(uint64_t* word, uint64_t value, hipStream_t stream);
 // ldsBytes = (plan depth - 1) * ReduceAccBytes(dtype, op) * args.threads: the accumulator stack of nested levels.
 hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t nBlocks,
                         uint32_t ldsBytes, hipStream_t stream);
+// Workgroups of `waves` wavefronts (2 .. kDirectFoldMaxWaves), one 1 KiB tile per wavefront.
+hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t waves,
+                            hipStream_t stream);
 inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)
 {
     bool half = dtype == HCCL_DATA_TYPE_FP16 || dtype == HCCL_DATA_TYPE_BFP16;

@@ -93,6 +93,7 @@ struct DevicePlan {
     uint32_t maxDepth = 1;
     uint32_t maxLeaves = 0;   // most leaves of any program of the plan
     bool segmentsAreSubs = false;
+    std::shared_ptr<const std::vector<uint8_t>> host;   // the image at `dev`, for launches that resolve a program's leaves on the host
 };
 
 constexpr uint32_t kMagic = 0x48434C41u;   // "HCLA"
@@ -112,6 +113,8 @@ struct Comm {
     uint32_t rank = 0;
     bool destroyed = false;
 };
+
+constexpr uint32_t kReduceBlocksDefault = 1u << 26;   // HCCL_AMD_REDUCE_BLOCKS unset: as many workgroups as there are tiles
 
 struct World {
     std::mutex mu;
@@ -153,6 +156,7 @@ struct World {
     uint64_t pieceBytes = 256ull << 20;   // HCCL_AMD_ALLREDUCE_PIECE_BYTES
     int twoKernelMode = 2;                // HCCL_AMD_ALLREDUCE_TWO_KERNELS: 0 never, 1 always, unset: by rank count and size
     int reducePair = 2;                   // HCCL_AMD_REDUCE_PAIR: 0 never, 1 wherever the form fits, else launch_policy.h decides
+    int reduceDirect = -1;                // HCCL_AMD_REDUCE_DIRECT: 0 never, 2 .. 8 wavefronts wherever the form fits, else launch_policy.h decides
     int reduceAllFold = -1;               // HCCL_AMD_REDUCE_ALL_FOLD: 0 never, 2 .. 4 wavefronts wherever the form fits, else launch_policy.h decides
     int fanOutLoadMode = 2;               // HCCL_AMD_FANOUT_STREAM_LOAD: 0 plain, 1 non-temporal, else launch_policy.h decides
     int copyTwoKernelMode = 2;            // HCCL_AMD_COPY_TWO_KERNELS, likewise for AllGather(V) and Broadcast
@@ -160,7 +164,7 @@ struct World {
     std::vector<uint64_t> a2aImage;
     std::vector<CopySeg> a2aSegs;   // the segment list of the AlltoAllV being launched (one launch at a time per world)
     uint8_t* a2aScratch = nullptr;
-    uint32_t reduceBlocks = 1u << 26;
+    uint32_t reduceBlocks = kReduceBlocksDefault;
     uint32_t reduceThreads = 0;   // 0: chosen per launch
     uint32_t storeWaves = 0;      // wavefronts sharing the stores of a many-destination reduce tile; 0: chosen per launch
     uint32_t copyTileBytes = 0;

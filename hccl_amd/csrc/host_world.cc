@@ -266,7 +266,7 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (hipGetDevice(&w->device) != hipSuccess) {
         w->device = 0;
     }
-    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", 1u << 26);
+    w->reduceBlocks = EnvU32("HCCL_AMD_REDUCE_BLOCKS", kReduceBlocksDefault);
     w->storeWaves = EnvU32("HCCL_AMD_REDUCE_STORE_WAVES", 0);
     if (w->storeWaves > kMaxReduceThreads / 64) {
         w->storeWaves = 0;
@@ -293,6 +293,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     w->reduceAllFold = EnvInt("HCCL_AMD_REDUCE_ALL_FOLD", -1);
     if (w->reduceAllFold != 0 && (w->reduceAllFold < 2 || w->reduceAllFold > static_cast<int>(kMaxReduceThreads / 64))) {
         w->reduceAllFold = -1;
+    }
+    w->reduceDirect = EnvInt("HCCL_AMD_REDUCE_DIRECT", -1);
+    if (w->reduceDirect != 0 && (w->reduceDirect < 2 || w->reduceDirect > static_cast<int>(kDirectFoldMaxWaves))) {
+        w->reduceDirect = -1;
     }
     w->reducePair = EnvInt("HCCL_AMD_REDUCE_PAIR", 2);
     if (w->reducePair < 0 || w->reducePair > 1) {
@@ -430,6 +434,7 @@ HcclResult GetDevicePlan(World* w, HcclAmdOpKind kind, HcclAmdAlgo algo, DeviceP
     dp.maxLeaves = maxLeaves;
     HIP_OK(hipMalloc(reinterpret_cast<void**>(&dp.dev), image.size()));
     HIP_OK(hipMemcpy(dp.dev, image.data(), image.size(), hipMemcpyHostToDevice));
+    dp.host = std::make_shared<const std::vector<uint8_t>>(std::move(image));
     w->plans[key] = dp;
     *out = dp;
     return HCCL_SUCCESS;

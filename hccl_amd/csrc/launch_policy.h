@@ -9,6 +9,8 @@
 
 #include <stdint.h>
 
+#include <initializer_list>
+
 namespace hccl_amd {
 namespace policy {
 
@@ -66,6 +68,58 @@ inline bool PairTiles(uint32_t ranks, bool oneResultStream, uint64_t bytesPerRan
 // are the best (8 ranks x 4 MiB: 14.8 one tile per wavefront, 12.7 three wavefronts, 12.2 eight); inside the library
 // eight measured 13.9 against 13.8 for three, so the workgroup limit stays at 256 lanes.
 // HCCL_AMD_REDUCE_ALL_FOLD = 0 / 2 .. 4 forces.
+// A flat fold of up to eight leaves to two to eight destinations launched from its arguments alone
+// (DirectFoldKernel; every operand on a 16-byte boundary, the first destination on a 1 KiB boundary): wavefronts per
+// workgroup, 0 = not this form.  Nothing but one block of scalar loads stands in front of a wavefront's first vector
+// load, the code is a few hundred instructions, and the wavefronts of a workgroup exchange their tiles so that each
+// writes `waves` KiB in a row to its own destinations.  AllReduce fp32 SUM in rank order, us per collective: the
+// general kernel with one tile per wavefront / two / wavefronts that exchange (kStoreWavesAllFold, 3) / this kernel
+// with 2 / 3 / 4 / 6 / 8 wavefronts:
+//   ranks   1 MiB                                   2 MiB                                   3 MiB                                    4 MiB                                            6 MiB                                            8 MiB                                            12 MiB per rank
+//     8   6.9/6.8/7.1/ 6.3/6.5/6.6/6.6/6.6   8.4/7.4/8.2/ 6.6/6.7/6.5/7.5/6.5   10.1/9.6/10.3/ 9.2/9.1/10.1/8.6/10.2   15.7/14.4/13.6/ 15.0/14.0/14.4/13.7/13.0   20.7/20.0/18.8/ 19.1/18.9/19.9/18.6/18.6   26.6/26.6/28.4/ 26.3/25.2/26.1/26.4/26.0   37.3/39.6/40.0/ 39.2/36.8/38.8/38.3/37.8
+//     6   6.2/6.2/6.1/ 5.5/5.8/5.8/5.8/5.8   6.8/6.3/7.0/ 5.8/6.0/6.0/6.0/6.1    7.7/7.9/8.2/ 7.1/6.6/6.9/6.7/7.3      12.1/10.5/10.4/ 11.1/10.7/11.3/11.0/9.5    16.4/15.2/14.4/ 14.6/14.4/14.6/13.8/14.3   20.7/20.9/21.4/ 20.8/19.1/20.5/19.8/18.9   28.7/29.4/30.2/ 29.2/27.7/28.6/28.4/28.3
+//     4   5.3/5.3/5.2/ 4.7/5.0/5.0/5.0/5.0   5.4/5.3/5.7/ 4.7/5.0/5.0/5.1/5.0    6.1/6.2/6.3/ 5.5/5.6/5.3/5.6/5.7       7.7/7.6/8.0/ 7.5/7.5/7.3/7.0/6.5         11.7/10.5/9.9/ 10.6/10.5/10.5/9.9/10.1     14.6/14.7/15.4/ 14.0/13.1/13.6/13.5/13.3   20.1/20.6/20.6/ 20.7/18.8/19.3/19.1/19.4
+//     2   4.3/4.4/4.5/ 3.8/4.0/4.1/4.0/4.1   4.3/4.4/4.6/ 3.8/4.1/4.0/4.0/4.1                                             5.7/4.8/6.4/ 4.7/4.6/4.4/4.8/4.4          7.4/6.0/7.6/ 5.4/5.3/5.3/5.4/5.4           8.7/7.9/9.0/ 8.0/7.5/7.6/7.6/7.2          (16 MiB: 13.6/14.3/14.4/ 13.7/13.0/13.0/13.0/13.3)
+// (8 ranks x 256 / 512 KiB: 6.9 against 6.3 / 6.4; 8 ranks x 2.5 / 3.5 / 5 / 7 / 10 MiB: 8.3 -> 7.3 with 2, 12.5 -> 11.6
+// with 8, 15.4 -> 15.6 with 4, 22.4 -> 23.1 with 4, 32.0 -> 31.1 with 3; 5 ranks x 4 MiB 9.1 -> 7.9, 7 ranks x 4 MiB
+// 12.0 -> 11.7; 4 ranks x 16 MiB 26.0 -> 24.5 with 3, 3 ranks x 16 MiB 19.7 -> 18.8, 2 ranks x 32 MiB 23.4 -> 23.3; at
+// 8 ranks x 16 MiB every form takes 46.6.)  Up to 2 MiB the launch is bound by its latency and two wavefronts are
+// ahead; up to 8 MiB the whole launch is one generation of wavefronts and the longer store runs of many wavefronts
+// pay, as long as the workgroups deal out evenly over the 256 CUs (8 ranks x 3 MiB = 3072 tiles: 384 workgroups of
+// eight wavefronts 10.2, 512 of six 8.6; 5 MiB: 640 of eight 17.1, 1280 of four 15.6); above, three wavefronts.
+// HCCL_AMD_REDUCE_DIRECT = 0 / 2 .. 8 forces.
+inline uint32_t DirectFoldWaves(uint32_t nLeaves, uint32_t nDst, uint64_t bytesPerRank)
+{
+    (void)nLeaves;
+    if (bytesPerRank > (nDst <= 4 ? 16 : 12) * kMiB) {
+        return 0;
+    }
+    if (bytesPerRank <= 2 * kMiB) {
+        return 2;
+    }
+    if (bytesPerRank > 8 * kMiB) {
+        return 3;
+    }
+    // the most wavefronts whose workgroups fill whole rounds of the CUs to 95 %, else the count that fills them best
+    constexpr uint64_t kCus = 256;
+    const uint64_t tiles = (bytesPerRank + 1023) / 1024;
+    uint32_t best = 2;
+    uint64_t bestFill = 0;   // per mille
+    for (uint32_t waves : {8u, 6u, 4u, 3u, 2u}) {
+        const uint64_t groups = (tiles + waves - 1) / waves;
+        const uint64_t rounds = (groups + kCus - 1) / kCus;
+        const uint64_t fill = groups * 1000 / (rounds * kCus);
+        if (fill >= 950) {
+            return waves;
+        }
+        if (fill > bestFill) {
+            bestFill = fill;
+            best = waves;
+        }
+    }
+    return best;
+}
+
 inline uint32_t AllFoldWaves(uint32_t nDst, uint64_t bytesPerRank)
 {
     if (nDst < 5 || nDst > 32 || bytesPerRank > 7 * kMiB) {

@@ -27,10 +27,75 @@ uint32_t BlocksPerSub(const World* w, uint64_t subLen, uint32_t esz, uint64_t nS
     return static_cast<uint32_t>(want < maxUseful ? want : maxUseful);
 }
 
+// The launch described by its arguments alone (DirectFoldKernel): one result of one flat program of up to eight
+// leaves that goes to two to eight destinations, every operand on a 16-byte boundary.  Returns the wavefronts per
+// workgroup and fills `d`, or 0 where the launch is not of that shape or another form is asked for.
+static uint32_t DirectFoldWaves(const World* w, const ReduceArgs& a, const DevicePlan& plan, uint32_t esz,
+                                DirectFoldArgs* d)
+{
+    if (w->reduceDirect == 0 || !w->reduceVector || a.varGroups != 0 || a.dstOwn != 0 || a.nGroup != 1 || a.nSub != 1 ||
+        a.nDst < 2 || a.nDst > kDirectFoldMaxDst || a.total == 0 || plan.host == nullptr || plan.maxDepth != 1) {
+        return 0;
+    }
+    const bool forced = w->reduceDirect > 0;
+    if (!forced && (w->reduceThreads != 0 || w->storeWaves != 0 || w->reduceBatch != 0 || w->reducePair == 1 ||
+                    w->reduceAllFold > 0 || w->storePolicy == 1 || w->reduceBlocks != kReduceBlocksDefault)) {
+        return 0;   // a setting names another form
+    }
+    const uint64_t progOff = static_cast<uint64_t>(a.prog - plan.dev);
+    if (a.prog < plan.dev || progOff % kDevProgBytes != 0 || progOff + kDevProgBytes > plan.host->size()) {
+        return 0;
+    }
+    const uint8_t* img = plan.host->data() + progOff;
+    const uint32_t leaves = img[0];
+    if (leaves == 0 || leaves > kDirectFoldMaxLeaves) {
+        return 0;
+    }
+    *d = DirectFoldArgs{};
+    for (uint32_t i = 0; i < leaves; ++i) {
+        const uint32_t rank = img[kDevProgRankOff + i];
+        if (img[kDevProgCtlOff + i] != 0 || rank >= w->n || a.src[rank] == nullptr ||
+            (reinterpret_cast<uintptr_t>(a.src[rank]) & 15u) != 0) {
+            return 0;
+        }
+        d->src[i] = a.src[rank];
+    }
+    for (uint32_t k = 0; k < a.nDst; ++k) {
+        if (a.dst[k] == nullptr || (reinterpret_cast<uintptr_t>(a.dst[k]) & 15u) != 0) {
+            return 0;
+        }
+        d->dst[k] = a.dst[k];
+    }
+    const uint32_t perVec = 16 / esz;
+    d->nVec = a.total / perVec;
+    d->tail = static_cast<uint32_t>(a.total % perVec);
+    d->nSrc = leaves;
+    d->nDst = a.nDst;
+    if (forced) {
+        return static_cast<uint32_t>(w->reduceDirect);
+    }
+    // by itself: where it was measured, and with tiles that start on the destination's 1 KiB boundaries
+    if ((reinterpret_cast<uintptr_t>(a.dst[0]) & 1023u) != 0) {
+        return 0;
+    }
+    return policy::DirectFoldWaves(leaves, a.nDst, a.total * esz);
+}
+
 HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, HcclDataType dtype, HcclReduceOp op,
                            hipStream_t s)
 {
     uint32_t esz = DataTypeSize(dtype);
+    if (esz == 0) {
+        return HCCL_E_INTERNAL;
+    }
+    {
+        DirectFoldArgs d;
+        const uint32_t waves = DirectFoldWaves(w, a, plan, esz, &d);
+        if (waves != 0) {
+            HIP_OK(LaunchDirectFold(d, dtype, op, waves, s));
+            return HCCL_SUCCESS;
+        }
+    }
     // 128-bit loads and stores may start on any element (the head is peeled for the first destination, which
     // makes every store aligned in the usual case of equally aligned recvBufs).  HCCL_AMD_REDUCE_VECTOR=0
     // forces the element-by-element path.

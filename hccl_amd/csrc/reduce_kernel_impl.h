@@ -963,6 +963,110 @@ __global__ __launch_bounds__(kThreads) void ReduceKernel(const ReduceArgs args)
 
 using ReduceKernelFn = void (*)(const ReduceArgs);
 
+// A flat fold of up to eight leaves to up to eight destinations, described by its arguments alone (DirectFoldArgs):
+// for the launch that is a single generation of wavefronts (a few MiB per rank), where the time in front of the first
+// vector load and the length of the code count.  Workgroup b takes the blockDim.x / 64 tiles from tile
+// b * (blockDim.x / 64) on: every wavefront folds one tile (all leaves' loads issued before the first fold, leaves in
+// the order of src[]), parks the result in LDS, and behind the barrier wavefront k writes the tiles of all wavefronts
+// to destinations k, k + waves, ...: `waves` KiB in a row to one or two streams instead of 1 KiB to each.  The
+// elements behind the last whole vector are folded one by one by the first lanes of workgroup 0.  Same folds in the
+// same order as ReduceValue on a flat program, hence the same bits.
+template <class E>
+__global__ __launch_bounds__(64 * kDirectFoldMaxWaves) void DirectFoldKernel(const DirectFoldArgs a)
+{
+    using S = typename E::S;
+    constexpr int W = 16 / sizeof(S);
+    constexpr int kLeaves = static_cast<int>(kDirectFoldMaxLeaves);
+    constexpr uint32_t kPerWave = kDirectFoldMaxDst / 2;   // destinations of one wavefront at most (two wavefronts or more)
+    static_assert(kLeaves == 8, "one batch of eight loads");
+    extern __shared__ uint32_t accStack[];
+    U32x4* const parked = reinterpret_cast<U32x4*>(accStack);
+    const uint32_t wave = Uniform(threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63u;
+    // all leaf addresses and the counts exist before the first is used: one block of scalar loads, one wait
+    uint64_t leaf[kLeaves];
+#pragma unroll
+    for (int i = 0; i < kLeaves; ++i) {
+        leaf[i] = reinterpret_cast<uint64_t>(a.src[i]);
+    }
+    uint64_t nVec = a.nVec;
+    uint32_t nSrc = a.nSrc;
+    uint32_t nDst = a.nDst;
+    uint32_t waves = a.waves;   // == blockDim.x / 64, which would be a scalar load of its own in front of these
+    ScalarFence8(leaf);
+    asm volatile("" : "+s"(nVec), "+s"(nSrc), "+s"(nDst), "+s"(waves));
+    // this wavefront's destination addresses, requested before the vector loads and first used behind the barrier
+    // (indices past the table read entry 0 and are never used)
+    uint64_t to[kPerWave];
+#pragma unroll
+    for (uint32_t k = 0; k < kPerWave; ++k) {
+        const uint32_t d = wave + k * waves;
+        to[k] = reinterpret_cast<uint64_t>(a.dst[d < kDirectFoldMaxDst ? d : 0u]);
+    }
+    float one = 1.0f;
+    if constexpr (HasAccumulate<E>::value) {
+        one = OpaqueOne();
+    }
+    const uint64_t tile0 = static_cast<uint64_t>(blockIdx.x) * waves;
+    const uint64_t u = (tile0 + wave) * 64 + lane;
+    if (u < nVec) {
+        U32x4 raw[kLeaves];
+#pragma unroll
+        for (int i = 0; i < kLeaves; ++i) {
+            if (static_cast<uint32_t>(i) < nSrc) {
+                raw[i] = __builtin_nontemporal_load(reinterpret_cast<const HCCL_AMD_GLOBAL U32x4*>(leaf[i]) + u);
+            }
+        }
+        IssueFence8(raw);
+        AccPack<E, W> acc;
+        PackOps<E, W>::Init(acc, __builtin_bit_cast(Pack<S, W>, raw[0]));
+#pragma unroll
+        for (int i = 1; i < kLeaves; ++i) {
+            if (static_cast<uint32_t>(i) < nSrc) {
+                PackOps<E, W>::Accumulate(acc, __builtin_bit_cast(Pack<S, W>, raw[i]), one);
+            }
+        }
+        parked[wave * 64 + lane] = __builtin_bit_cast(U32x4, PackOps<E, W>::Narrow(acc));
+    }
+    __syncthreads();
+    // (a workgroup whose tiles are all whole, every one but the last, stores without a bounds check per tile)
+    const bool whole = (tile0 + waves) * 64 <= nVec;
+#pragma unroll
+    for (uint32_t k = 0; k < kPerWave; ++k) {
+        if (wave + k * waves < nDst) {
+            HCCL_AMD_GLOBAL U32x4* const out = reinterpret_cast<HCCL_AMD_GLOBAL U32x4*>(to[k]) + tile0 * 64 + lane;
+            if (whole) {
+                for (uint32_t t = 0; t < waves; ++t) {
+                    __builtin_nontemporal_store(parked[t * 64 + lane], out + t * 64);
+                }
+            } else {
+                for (uint32_t t = 0; t < waves; ++t) {
+                    if ((tile0 + t) * 64 + lane < nVec) {
+                        __builtin_nontemporal_store(parked[t * 64 + lane], out + t * 64);
+                    }
+                }
+            }
+        }
+    }
+    if (blockIdx.x == 0 && wave == 0 && lane < a.tail) {
+        const uint64_t e = nVec * W + lane;
+        AccPack<E, 1> acc;
+        PackOps<E, 1>::Init(acc, LoadPack<S, 1>(reinterpret_cast<const void*>(leaf[0]), e));
+#pragma unroll
+        for (int i = 1; i < kLeaves; ++i) {
+            if (static_cast<uint32_t>(i) < nSrc) {
+                PackOps<E, 1>::Accumulate(acc, LoadPack<S, 1>(reinterpret_cast<const void*>(leaf[i]), e), one);
+            }
+        }
+        const Pack<S, 1> out = PackOps<E, 1>::Narrow(acc);
+        for (uint32_t d = 0; d < nDst; ++d) {
+            StorePack<S, 1>(a.dst[d], e, out, false);
+        }
+    }
+}
+
+using DirectFoldFn = void (*)(const DirectFoldArgs);
+
 }  // namespace detail
 
 // One translation unit per data type defines its selector (nullptr = combination not offered).
@@ -975,6 +1079,15 @@ detail::ReduceKernelFn SelectReduceF16(int op, int batch);
 detail::ReduceKernelFn SelectReduceBf16(int op, int batch);
 detail::ReduceKernelFn SelectReduceF32(int op, int batch);
 detail::ReduceKernelFn SelectReduceF64(int op, int batch);
+detail::DirectFoldFn SelectReduceI8Direct(int op);
+detail::DirectFoldFn SelectReduceI16Direct(int op);
+detail::DirectFoldFn SelectReduceI32Direct(int op);
+detail::DirectFoldFn SelectReduceI64Direct(int op);
+detail::DirectFoldFn SelectReduceU64Direct(int op);
+detail::DirectFoldFn SelectReduceF16Direct(int op);
+detail::DirectFoldFn SelectReduceBf16Direct(int op);
+detail::DirectFoldFn SelectReduceF32Direct(int op);
+detail::DirectFoldFn SelectReduceF64Direct(int op);
 
 #define HCCL_AMD_PICK(T, batch)                                                                \
     ((batch) == 8 ? detail::ReduceKernel<T, 8>                                                 \
@@ -990,6 +1103,16 @@ detail::ReduceKernelFn SelectReduceF64(int op, int batch);
             case detail::kMin: return HCCL_AMD_PICK(MIN_T, batch);                \
             default: return nullptr;                                              \
         }                                                                         \
+    }                                                                             \
+    detail::DirectFoldFn NAME##Direct(int op)                                     \
+    {                                                                             \
+        switch (op) {                                                             \
+            case detail::kSum: return detail::DirectFoldKernel<SUM_T>;            \
+            case detail::kProd: return detail::DirectFoldKernel<PROD_T>;          \
+            case detail::kMax: return detail::DirectFoldKernel<MAX_T>;            \
+            case detail::kMin: return detail::DirectFoldKernel<MIN_T>;            \
+            default: return nullptr;                                              \
+        }                                                                         \
     }
 
 #define HCCL_AMD_DEFINE_SELECT3(NAME, SUM_T, MAX_T, MIN_T)                         \
@@ -999,6 +1122,15 @@ detail::ReduceKernelFn SelectReduceF64(int op, int batch);
             case detail::kSum: return HCCL_AMD_PICK(SUM_T, batch);                \
             case detail::kMax: return HCCL_AMD_PICK(MAX_T, batch);                \
             case detail::kMin: return HCCL_AMD_PICK(MIN_T, batch);                \
+            default: return nullptr;                                              \
+        }                                                                         \
+    }                                                                             \
+    detail::DirectFoldFn NAME##Direct(int op)                                     \
+    {                                                                             \
+        switch (op) {                                                             \
+            case detail::kSum: return detail::DirectFoldKernel<SUM_T>;            \
+            case detail::kMax: return detail::DirectFoldKernel<MAX_T>;            \
+            case detail::kMin: return detail::DirectFoldKernel<MIN_T>;            \
             default: return nullptr;                                              \
         }                                                                         \
     }

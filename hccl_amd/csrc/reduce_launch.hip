@@ -56,4 +56,59 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
     return hipGetLastError();
 }
 
+hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t waves,
+                            hipStream_t stream)
+{
+    detail::DirectFoldFn fn = nullptr;
+    const int o = static_cast<int>(op);
+    switch (dtype) {
+        case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8Direct(o); break;
+        case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16Direct(o); break;
+        case HCCL_DATA_TYPE_INT32: fn = SelectReduceI32Direct(o); break;
+        case HCCL_DATA_TYPE_INT64: fn = SelectReduceI64Direct(o); break;
+        case HCCL_DATA_TYPE_UINT64: fn = SelectReduceU64Direct(o); break;
+        case HCCL_DATA_TYPE_FP16: fn = SelectReduceF16Direct(o); break;
+        case HCCL_DATA_TYPE_BFP16: fn = SelectReduceBf16Direct(o); break;
+        case HCCL_DATA_TYPE_FP32: fn = SelectReduceF32Direct(o); break;
+        case HCCL_DATA_TYPE_FP64: fn = SelectReduceF64Direct(o); break;
+        default: break;
+    }
+    uint32_t esz = 0;
+    switch (dtype) {
+        case HCCL_DATA_TYPE_INT8: esz = 1; break;
+        case HCCL_DATA_TYPE_INT16: case HCCL_DATA_TYPE_FP16: case HCCL_DATA_TYPE_BFP16: esz = 2; break;
+        case HCCL_DATA_TYPE_INT32: case HCCL_DATA_TYPE_FP32: esz = 4; break;
+        case HCCL_DATA_TYPE_INT64: case HCCL_DATA_TYPE_UINT64: case HCCL_DATA_TYPE_FP64: esz = 8; break;
+        default: break;
+    }
+    if (fn == nullptr || esz == 0 || waves < 2 || waves > kDirectFoldMaxWaves || args.nSrc == 0 ||
+        args.nSrc > kDirectFoldMaxLeaves || args.nDst == 0 || args.nDst > kDirectFoldMaxDst || args.tail >= 16 / esz ||
+        (args.nVec == 0 && args.tail == 0)) {
+        return hipErrorInvalidValue;
+    }
+    // a wavefront holds the addresses of at most half the destination table
+    if ((args.nDst + waves - 1) / waves > kDirectFoldMaxDst / 2) {
+        return hipErrorInvalidValue;
+    }
+    for (uint32_t i = 0; i < args.nSrc; ++i) {
+        if (args.src[i] == nullptr || (reinterpret_cast<uintptr_t>(args.src[i]) & 15u) != 0) {
+            return hipErrorInvalidValue;
+        }
+    }
+    for (uint32_t d = 0; d < args.nDst; ++d) {
+        if (args.dst[d] == nullptr || (reinterpret_cast<uintptr_t>(args.dst[d]) & 15u) != 0) {
+            return hipErrorInvalidValue;
+        }
+    }
+    const uint64_t tiles = (args.nVec + 63) / 64;
+    const uint64_t blocks = tiles == 0 ? 1 : (tiles + waves - 1) / waves;
+    if (blocks > 0x7FFFFFFFull) {
+        return hipErrorInvalidValue;
+    }
+    DirectFoldArgs a = args;
+    a.waves = waves;
+    hipLaunchKernelGGL(fn, dim3(static_cast<uint32_t>(blocks)), dim3(64 * waves), waves * 1024u, stream, a);
+    return hipGetLastError();
+}
+
 }  // namespace hccl_amd

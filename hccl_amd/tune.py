@@ -127,10 +127,14 @@ def all_reduce_small_rows(torch, h, ranks, kibs, rounds):
                     groups[k]()
                 return comms, step
 
-            forms = [("one", {"HCCL_AMD_REDUCE_PAIR": "0", "HCCL_AMD_REDUCE_ALL_FOLD": "0"}),
-                     ("pair", {"HCCL_AMD_REDUCE_PAIR": "1", "HCCL_AMD_REDUCE_ALL_FOLD": "0"}),
-                     ("fold2", {"HCCL_AMD_REDUCE_ALL_FOLD": "2"}), ("fold3", {"HCCL_AMD_REDUCE_ALL_FOLD": "3"}),
-                     ("fold4", {"HCCL_AMD_REDUCE_ALL_FOLD": "4"}), ("auto", {})]
+            off = {"HCCL_AMD_REDUCE_DIRECT": "0"}
+            forms = [("one", dict(off, HCCL_AMD_REDUCE_PAIR="0", HCCL_AMD_REDUCE_ALL_FOLD="0")),
+                     ("pair", dict(off, HCCL_AMD_REDUCE_PAIR="1", HCCL_AMD_REDUCE_ALL_FOLD="0")),
+                     ("fold2", dict(off, HCCL_AMD_REDUCE_ALL_FOLD="2")), ("fold3", dict(off, HCCL_AMD_REDUCE_ALL_FOLD="3")),
+                     ("fold4", dict(off, HCCL_AMD_REDUCE_ALL_FOLD="4"))]
+            if n <= 8:
+                forms += [("direct%d" % k, {"HCCL_AMD_REDUCE_DIRECT": str(k)}) for k in (2, 3, 4, 6, 8)]
+            forms.append(("auto", {}))
             fracs = _forms(torch, h, make_step, forms, per_set, rounds, 200)
             us = "/".join("%.1f" % (per_set / (v * HBM_PEAK) * 1e6) for v in fracs.values())
             rows.append(_row("%2d ranks x %5d KiB  %s us" % (n, kib, us), fracs))

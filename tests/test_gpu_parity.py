@@ -506,6 +506,44 @@ def test_all_reduce_with_wavefronts_that_exchange_their_tiles_and_store_their_ow
         w.close()
 
 
+@pytest.mark.parametrize("n,waves", [(2, 2), (3, 8), (5, 3), (6, 4), (8, 2), (8, 3), (8, 8)])
+def test_all_reduce_launched_from_its_arguments_alone(monkeypatch, n, waves):
+    """The kernel for a flat fold of up to eight ranks to up to eight destinations that finds everything in its
+    arguments (no program image), forced for every size: tile counts that the workgroup's wavefronts divide and do
+    not, less than one tile and less than one vector, elements behind the last whole vector, every element type and
+    operator, in place, more wavefronts than destinations and fewer.  Operands off the 16-byte grid, nested programs,
+    results cut into sub-segments and results with one destination keep the general kernel."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_DIRECT", str(waves))
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "0")
+    w = World(n)
+    monkeypatch.delenv("HCCL_AMD_REDUCE_DIRECT")
+    monkeypatch.delenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS")
+    try:
+        seed = 6900 + 10 * n + waves
+        for dtype in REDUCE_TYPES:
+            for op in (SUM, PROD, MAX, MIN):
+                if op == PROD and dtype in (DT.INT16, DT.BFP16):
+                    continue   # not defined for these types
+                run_all_reduce(w, dtype, op, 20_011, "mesh", seed=seed)
+                seed += 1
+        for count in (1, 3, 4, 5, 255, 256, 257, 256 * waves - 1, 256 * waves, 256 * waves + 1, 256 * (2 * waves + 1),
+                      4096 * 3, 4096 * 4 + 1, 100_003):
+            run_all_reduce(w, DT.FP32, SUM, count, "ring", seed=seed)            # 256 fp32 = one tile
+            seed += 1
+        run_all_reduce(w, DT.INT8, MIN, 9, "mesh", seed=seed)                    # less than one vector
+        run_all_reduce(w, DT.INT8, SUM, 16 * 64 * 3 + 15, "mesh", seed=seed + 1)  # fifteen elements behind the vectors
+        run_all_reduce(w, DT.INT32, PROD, 4_099, "mesh", seed=seed + 2, in_place=True)
+        run_all_reduce(w, DT.BFP16, SUM, 30_011, "mesh", seed=seed + 3, in_place=True)
+        run_all_reduce(w, DT.FP16, MAX, 33_333, "mesh", seed=seed + 4, pad=2)    # off the 16-byte grid: general kernel
+        run_all_reduce(w, DT.FP64, SUM, 12_345, "mesh", seed=seed + 5, pad=lambda r, which: r + (3 if which == "recv" else 0))
+        run_all_reduce(w, DT.FP32, SUM, 70_001, "nhr", seed=seed + 6)            # nested program: general kernel
+        run_all_reduce(w, DT.FP32, SUM, 70_001, "mesh_symmetric", seed=seed + 7)   # n sub-segments: general kernel
+        run_all_reduce(w, DT.FP32, MIN, 9_973, "mesh_chunk", seed=seed + 8)
+        run_reduce_scatter(w, DT.FP32, SUM, 5_001, "mesh", seed=seed + 9)        # one result stream: general kernel
+    finally:
+        w.close()
+
+
 def test_prepared_group_issues_the_same_collective():
     """hccl_amd.prepared_group converts the arguments of a group's calls once; what it runs is the plain sequence
     HcclGroupStart, the entry points, HcclGroupEnd, and a bad argument still raises with the entry point's code."""

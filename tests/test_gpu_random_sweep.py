@@ -38,6 +38,8 @@ def pick_count(rng):
 
 FORMS = {
     "by_size": {},
+    # without the kernel that is launched from its arguments alone: the general kernel on the short messages too
+    "general_kernel": {"HCCL_AMD_REDUCE_DIRECT": "0"},
     # AllReduce as fold + fan-out whatever the size, pieces of a few KiB
     "two_kernels": {"HCCL_AMD_ALLREDUCE_TWO_KERNELS": "1", "HCCL_AMD_ALLREDUCE_PIECE_BYTES": None},
     # the fused kernel with a tile's stores shared by wavefronts, on a grid so small that workgroups loop

@@ -57,7 +57,11 @@ def test_every_translation_unit_is_there(kernels):
     # 34 combinations of element type and operation, each with the eight-leaf and the sixteen-leaf load batch and
     # with the eight-leaf batch over two tiles per wavefront
     assert len(reduce_kernels) == 102, sorted(k["name"] for k in reduce_kernels)
-    assert len(kernels) - len(reduce_kernels) == 22            # the copy, fan-out (two load flavours) and AlltoAllV kernels
+    # and once as the kernel that is launched from its arguments alone
+    direct_kernels = [k for k in kernels if "DirectFoldKernel" in k["name"]]
+    assert len(direct_kernels) == 34, sorted(k["name"] for k in direct_kernels)
+    # the copy, fan-out (two load flavours) and AlltoAllV kernels
+    assert len(kernels) - len(reduce_kernels) - len(direct_kernels) == 22
 
 
 def test_no_kernel_spills_or_uses_private_memory(kernels):
@@ -70,7 +74,9 @@ def test_register_budgets(kernels):
     type and batch; at most 24 for the copy kernels.  Scalar registers cannot exceed what the hardware has; what is
     checked for them is that the compiler did not have to spill (above)."""
     for k in kernels:
-        limit = 96 if "ReduceKernel" in k["name"] else 24
+        # (the kernel launched from its arguments: at most 64, so that the eight
+        # wavefronts a SIMD can hold all fit)
+        limit = 96 if "ReduceKernel" in k["name"] else 64 if "DirectFoldKernel" in k["name"] else 24
         assert k["vgpr"] <= limit, k
 
 
@@ -78,7 +84,8 @@ def test_uniform_values_are_uniform_for_the_compiler_too(kernels, tmp_path_facto
     """The kernels pin launch scalars, program words and leaf addresses in scalar registers (the "+s" operands of
     their empty assembly statements).  Had one of them been computed per lane, the compiler would satisfy the
     constraint by taking the first lane's value, silently: a v_readfirstlane in the code.  The only one the sources
-    ask for themselves is the fan-out kernel's wavefront index (two instantiations of that kernel)."""
+    ask for themselves are the wavefront index of the fan-out kernel (two instantiations of that kernel) and of the
+    fold kernel that is launched from its arguments alone (one per instantiation)."""
     tmp = tmp_path_factory.mktemp("code")
     kernel_notes(tmp)
     counts = {}
@@ -86,5 +93,6 @@ def test_uniform_values_are_uniform_for_the_compiler_too(kernels, tmp_path_facto
         text = subprocess.run([LLVM + "/llvm-objdump", "-d", "--mcpu=gfx950", str(obj)], stdout=subprocess.PIPE,
                               text=True, check=True).stdout
         assert "s_endpgm" in text                       # the listing is real
-        counts[obj.name] = text.count("v_readfirstlane")
+        direct = len(re.findall(r"^[0-9a-f]+ <[^>+]*DirectFoldKernel[^>+]*>:$", text, re.M))
+        counts[obj.name] = text.count("v_readfirstlane") - direct
     assert sorted(counts.values()) == [0] * (len(counts) - 1) + [2], counts   # the fan-out kernel's two load flavours

@@ -20,10 +20,11 @@ int main()
         160ull << 20, 256ull << 20, 1ull << 30, 8ull << 30};
     for (unsigned n = 1; n <= 64; ++n) {
         for (unsigned long long b : sizes) {
-            std::printf("%u %llu %d %d %d %d %u %u %u %u %d %d %u\n", n, b, (int)FoldThenFanOut(n, b),
+            std::printf("%u %llu %d %d %d %d %u %u %u %u %d %d %u %u\n", n, b, (int)FoldThenFanOut(n, b),
                         (int)GatherThenFanOut(n, b, true), (int)GatherThenFanOut(n, b, false), (int)PairTiles(n, false, b),
                         StoreWaves(n, b, 4), StoreWaves(n, b, 2), VecBatch(n, false, false), VecBatch(n, true, false),
-                        (int)FanOutStreamLoad(n, false), (int)FanOutStreamLoad(n, true), AllFoldWaves(n, b));
+                        (int)FanOutStreamLoad(n, false), (int)FanOutStreamLoad(n, true), AllFoldWaves(n, b),
+                        DirectFoldWaves(n < 8 ? n : 8, n < 8 ? n : 8, b));
         }
     }
     return 0;
@@ -42,7 +43,8 @@ def table(tmp_path_factory):
     for line in subprocess.check_output([str(exe)], text=True).splitlines():
         v = [int(x) for x in line.split()]
         rows[(v[0], v[1])] = dict(fold=v[2], gather=v[3], gather_general=v[4], pair=v[5], waves4=v[6], waves2=v[7],
-                                  batch_many=v[8], batch_one=v[9], nt_single=v[10], nt_several=v[11], all_fold=v[12])
+                                  batch_many=v[8], batch_one=v[9], nt_single=v[10], nt_several=v[11], all_fold=v[12],
+                                  direct=v[13])
     return rows
 
 
@@ -85,6 +87,24 @@ def test_the_all_fold_form_has_one_window_of_sizes_and_fits_the_workgroup(table)
     assert table[(8, 3 << 20)]["all_fold"] == 0 and table[(8, (7 << 20) + 1)]["all_fold"] == 0
     assert table[(16, 5 << 19)]["all_fold"] == 3 and table[(16, 2 << 20)]["all_fold"] == 0
     assert table[(6, 4 << 20)]["all_fold"] == 0 and table[(6, 5 << 20)]["all_fold"] == 3
+
+
+def test_the_kernel_launched_from_its_arguments_covers_everything_up_to_its_limit(table):
+    """From the shortest message up to 12 MiB per rank (16 MiB for up to four destinations), with a count of
+    wavefronts the launcher takes for up to eight destinations; two where the launch is latency-bound, the count whose
+    workgroups deal out evenly over the CUs in between (3 MiB = 3072 tiles: six, 4 MiB: eight, 5 MiB: four)."""
+    for n, rows in by_world(table).items():
+        if n < 2 or n > 8:
+            continue
+        limit = (16 if n <= 4 else 12) << 20
+        for b, row in rows:
+            assert (row["direct"] != 0) == (b <= limit), (n, b)
+            assert row["direct"] in (0, 2, 3, 4, 6, 8), (n, b)
+    assert table[(8, 1 << 20)]["direct"] == 2 and table[(8, 2 << 20)]["direct"] == 2
+    assert table[(8, 3 << 20)]["direct"] == 6 and table[(8, 4 << 20)]["direct"] == 8
+    assert table[(8, 5 << 20)]["direct"] == 4 and table[(8, 6 << 20)]["direct"] == 8
+    assert table[(8, 8 << 20)]["direct"] == 8 and table[(8, (8 << 20) + 1)]["direct"] == 3
+    assert table[(8, 16 << 20)]["direct"] == 0 and table[(4, 16 << 20)]["direct"] == 3
 
 
 def test_the_pair_form_has_one_window_of_sizes(table):
