@@ -992,9 +992,10 @@ __global__ __launch_bounds__(64 * kDirectFoldMaxWaves) void DirectFoldKernel(con
     uint64_t nVec = a.nVec;
     uint32_t nSrc = a.nSrc;
     uint32_t nDst = a.nDst;
+    uint32_t tail = a.tail;
     uint32_t waves = a.waves;   // == blockDim.x / 64, which would be a scalar load of its own in front of these
     ScalarFence8(leaf);
-    asm volatile("" : "+s"(nVec), "+s"(nSrc), "+s"(nDst), "+s"(waves));
+    asm volatile("" : "+s"(nVec), "+s"(nSrc), "+s"(nDst), "+s"(tail), "+s"(waves));
     // this wavefront's destination addresses, requested before the vector loads and first used behind the barrier
     // (indices past the table read entry 0 and are never used)
     uint64_t to[kPerWave];
@@ -1048,7 +1049,7 @@ __global__ __launch_bounds__(64 * kDirectFoldMaxWaves) void DirectFoldKernel(con
             }
         }
     }
-    if (blockIdx.x == 0 && wave == 0 && lane < a.tail) {
+    if (blockIdx.x == 0 && wave == 0 && lane < tail) {
         const uint64_t e = nVec * W + lane;
         AccPack<E, 1> acc;
         PackOps<E, 1>::Init(acc, LoadPack<S, 1>(reinterpret_cast<const void*>(leaf[0]), e));
