@@ -61,16 +61,19 @@ hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, Hccl
 {
     detail::DirectFoldFn fn = nullptr;
     const int o = static_cast<int>(op);
+    // eight of everything and only whole workgroups: the straight-line kernel
+    const bool exact = waves == 8 && args.nSrc == 8 && args.nDst == 8 && args.tail == 0 && args.nVec != 0 &&
+                       args.nVec % (8 * 64) == 0;
     switch (dtype) {
-        case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8Direct(o); break;
-        case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16Direct(o); break;
-        case HCCL_DATA_TYPE_INT32: fn = SelectReduceI32Direct(o); break;
-        case HCCL_DATA_TYPE_INT64: fn = SelectReduceI64Direct(o); break;
-        case HCCL_DATA_TYPE_UINT64: fn = SelectReduceU64Direct(o); break;
-        case HCCL_DATA_TYPE_FP16: fn = SelectReduceF16Direct(o); break;
-        case HCCL_DATA_TYPE_BFP16: fn = SelectReduceBf16Direct(o); break;
-        case HCCL_DATA_TYPE_FP32: fn = SelectReduceF32Direct(o); break;
-        case HCCL_DATA_TYPE_FP64: fn = SelectReduceF64Direct(o); break;
+        case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8Direct(o, exact); break;
+        case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16Direct(o, exact); break;
+        case HCCL_DATA_TYPE_INT32: fn = SelectReduceI32Direct(o, exact); break;
+        case HCCL_DATA_TYPE_INT64: fn = SelectReduceI64Direct(o, exact); break;
+        case HCCL_DATA_TYPE_UINT64: fn = SelectReduceU64Direct(o, exact); break;
+        case HCCL_DATA_TYPE_FP16: fn = SelectReduceF16Direct(o, exact); break;
+        case HCCL_DATA_TYPE_BFP16: fn = SelectReduceBf16Direct(o, exact); break;
+        case HCCL_DATA_TYPE_FP32: fn = SelectReduceF32Direct(o, exact); break;
+        case HCCL_DATA_TYPE_FP64: fn = SelectReduceF64Direct(o, exact); break;
         default: break;
     }
     uint32_t esz = 0;

@@ -530,6 +530,14 @@ def test_all_reduce_launched_from_its_arguments_alone(monkeypatch, n, waves):
                       4096 * 3, 4096 * 4 + 1, 100_003):
             run_all_reduce(w, DT.FP32, SUM, count, "ring", seed=seed)            # 256 fp32 = one tile
             seed += 1
+        # whole workgroups of eight tiles only (eight ranks and eight wavefronts: the straight-line instantiation)
+        for dtype in REDUCE_TYPES:
+            esz = np.dtype(NP[dtype]).itemsize
+            for op in (SUM, PROD, MAX, MIN):
+                if op == PROD and dtype in (DT.INT16, DT.BFP16):
+                    continue
+                run_all_reduce(w, dtype, op, 3 * 8192 // esz, "mesh", seed=seed, in_place=(op == MAX))
+                seed += 1
         run_all_reduce(w, DT.INT8, MIN, 9, "mesh", seed=seed)                    # less than one vector
         run_all_reduce(w, DT.INT8, SUM, 16 * 64 * 3 + 15, "mesh", seed=seed + 1)  # fifteen elements behind the vectors
         run_all_reduce(w, DT.INT32, PROD, 4_099, "mesh", seed=seed + 2, in_place=True)
