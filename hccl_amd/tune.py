@@ -100,10 +100,11 @@ def all_reduce_rows(torch, h, ranks, mibs, rounds):
     return rows
 
 
-def all_reduce_small_rows(torch, h, ranks, kibs, rounds):
-    print("# AllReduce fp32 SUM in rank order, a few MiB per rank: one tile per wavefront, two, workgroups of 2 / 3 / 4 "
-          "wavefronts that exchange their tiles and store one or two streams each, the library's own choice "
-          "(collectives issued with their arguments converted once)")
+def all_reduce_small_rows(torch, h, ranks, kibs, rounds, only=None):
+    print("# AllReduce fp32 SUM in rank order, a few MiB per rank: the general kernel with one tile per wavefront, two, "
+          "workgroups of 2 / 3 / 4 wavefronts that exchange their tiles and store one or two streams each; up to eight "
+          "ranks also the kernel launched from its arguments alone with 2 / 3 / 4 / 6 / 8 wavefronts; the library's own "
+          "choice (collectives issued with their arguments converted once)")
     rows = []
     for n in ranks:
         for kib in kibs:
@@ -134,6 +135,8 @@ def all_reduce_small_rows(torch, h, ranks, kibs, rounds):
                      ("fold4", dict(off, HCCL_AMD_REDUCE_ALL_FOLD="4"))]
             if n <= 8:
                 forms += [("direct%d" % k, {"HCCL_AMD_REDUCE_DIRECT": str(k)}) for k in (2, 3, 4, 6, 8)]
+            if only is not None:
+                forms = [f for f in forms if f[0] in only]
             forms.append(("auto", {}))
             fracs = _forms(torch, h, make_step, forms, per_set, rounds, 200)
             us = "/".join("%.1f" % (per_set / (v * HBM_PEAK) * 1e6) for v in fracs.values())

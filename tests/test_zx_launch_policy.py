@@ -39,7 +39,9 @@ def test_small_all_reduce_form(ranks, kib):
     import torch
     import hccl_amd
     from hccl_amd import tune
-    assert behind_best(tune.all_reduce_small_rows(torch, hccl_amd, [ranks], [kib], 3)) == []
+    # (one form of each kind: the more forms are timed, the further the luckiest of them lies ahead of its own mean)
+    forms = ("one", "pair", "fold3", "direct3", "direct8")
+    assert behind_best(tune.all_reduce_small_rows(torch, hccl_amd, [ranks], [kib], 3, only=forms)) == []
 
 
 @pytest.mark.parametrize("ranks,mib", [(4, 64), (16, 8)])
