@@ -69,7 +69,7 @@ inline bool PairTiles(uint32_t ranks, bool oneResultStream, uint64_t bytesPerRan
 // eight measured 13.9 against 13.8 for three, so the workgroup limit stays at 256 lanes.
 // HCCL_AMD_REDUCE_ALL_FOLD = 0 / 2 .. 4 forces.
 // A flat fold of up to eight leaves to two to eight destinations launched from its arguments alone
-// (DirectFoldKernel; every operand on a 16-byte boundary, the first destination on a 1 KiB boundary): wavefronts per
+// (DirectFoldKernel; every operand on a 16-byte boundary, the first destination on a 128-byte line): wavefronts per
 // workgroup, 0 = not this form.  Nothing but one block of scalar loads stands in front of a wavefront's first vector
 // load, the code is a few hundred instructions, and the wavefronts of a workgroup exchange their tiles so that each
 // writes `waves` KiB in a row to its own destinations.  AllReduce fp32 SUM in rank order, us per collective: the

@@ -74,8 +74,9 @@ static uint32_t DirectFoldWaves(const World* w, const ReduceArgs& a, const Devic
     if (forced) {
         return static_cast<uint32_t>(w->reduceDirect);
     }
-    // by itself: where it was measured, and with tiles that start on the destination's 1 KiB boundaries
-    if ((reinterpret_cast<uintptr_t>(a.dst[0]) & 1023u) != 0) {
+    // by itself: where it was measured, and with tiles that are whole 128-byte lines of the first destination (the
+    // general kernel deals its vectors to the lanes shifted so that they are; this one starts at the buffer's start)
+    if ((reinterpret_cast<uintptr_t>(a.dst[0]) & 127u) != 0) {
         return 0;
     }
     return policy::DirectFoldWaves(leaves, a.nDst, a.total * esz);
