@@ -157,6 +157,7 @@ struct World {
     int twoKernelMode = 2;                // HCCL_AMD_ALLREDUCE_TWO_KERNELS: 0 never, 1 always, unset: by rank count and size
     int reducePair = 2;                   // HCCL_AMD_REDUCE_PAIR: 0 never, 1 wherever the form fits, else launch_policy.h decides
     int reduceDirect = -1;                // HCCL_AMD_REDUCE_DIRECT: 0 never, 2 .. 8 wavefronts wherever the form fits, else launch_policy.h decides
+    int reduceDirectTiles = 0;            // HCCL_AMD_REDUCE_DIRECT_TILES: 1 / 2 tiles per wavefront of its straight-line instantiation, else launch_policy.h decides
     int reduceAllFold = -1;               // HCCL_AMD_REDUCE_ALL_FOLD: 0 never, 2 .. 4 wavefronts wherever the form fits, else launch_policy.h decides
     int fanOutLoadMode = 2;               // HCCL_AMD_FANOUT_STREAM_LOAD: 0 plain, 1 non-temporal, else launch_policy.h decides
     int copyTwoKernelMode = 2;            // HCCL_AMD_COPY_TWO_KERNELS, likewise for AllGather(V) and Broadcast

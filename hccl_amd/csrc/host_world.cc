@@ -298,6 +298,10 @@ std::unique_ptr<World> NewWorld(uint32_t n)
     if (w->reduceDirect != 0 && (w->reduceDirect < 2 || w->reduceDirect > static_cast<int>(kDirectFoldMaxWaves))) {
         w->reduceDirect = -1;
     }
+    w->reduceDirectTiles = EnvInt("HCCL_AMD_REDUCE_DIRECT_TILES", 0);
+    if (w->reduceDirectTiles < 1 || w->reduceDirectTiles > 2) {
+        w->reduceDirectTiles = 0;
+    }
     w->reducePair = EnvInt("HCCL_AMD_REDUCE_PAIR", 2);
     if (w->reducePair < 0 || w->reducePair > 1) {
         w->reducePair = 2;

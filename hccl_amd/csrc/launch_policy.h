@@ -48,26 +48,6 @@ inline bool PairTiles(uint32_t ranks, bool oneResultStream, uint64_t bytesPerRan
     return !oneResultStream && 2 * bytesPerRank >= 3 * kMiB && bytesPerRank <= (ranks <= 3 ? 8 : 6) * kMiB;
 }
 
-// Every wavefront of a workgroup folds a tile of its own and, after an exchange through LDS, stores the tiles of all
-// to its own destinations (kStoreWavesAllFold; flat programs, one sub-segment): the number of wavefronts per
-// workgroup, 0 = not this form.  Between the launch that is one generation of wavefronts and the one that reaches a
-// steady state, a fused launch to many destinations ends with every wavefront writing 1 KiB to every stream; with
-// three wavefronts exchanging their tiles each writes 3 KiB in a row to a third of the streams.  AllReduce fp32 SUM in
-// rank order, us per collective: one tile per wavefront / two / this form with 2 / 3 / 4 wavefronts:
-//   ranks    3 MiB                 4 MiB                      5 MiB                 6 MiB                      7 MiB              7.5 - 8 MiB per rank
-//     5                   10.4/ 9.3/ 9.8/ 9.3/ 9.5   12.0/10.7/10.5/10.4/10.7   13.9/13.1/12.0/12.1/12.6   15.6/15.5/14.3/16.3/14.5
-//     6                   12.1/10.7/11.3/10.5/11.1   13.9/13.3/12.5/11.9/12.7   16.0/15.2/14.4/14.2/15.4   18.0/17.8/16.7/18.7/17.1   19.9/20.1/21.1/20.5/21.4
-//     8   9.9/9.6/10.4/10.2/10.7   15.8/14.3/14.2/13.8/14.1   17.3/16.8/15.8/15.4/16.1   20.7/20.0/18.8/19.0/19.5   23.6/23.8/22.2/24.9/22.9   26.3/27.4/30.6/28.4/30.4
-//    12   15.3/15.3/14.7/14.3/15.0   21.4/21.3/19.8/19.0/20.3                       31.2/31.3/27.3/27.8/29.4   35.6/35.6/34.6/36.1/35.2
-//    16   20.3/20.2/18.2/18.3/19.2   28.8/28.7/26.2/25.1/27.0                       39.5/39.5/36.6/36.9/39.4   47.6/47.5/44.1/48.5/46.0   (8 MiB: two kernels)
-//    24   28.0/27.9/26.8/26.8/28.3   42.0/41.8/39.2/38.1/41.3
-//    32   37.9/37.7/35.8/35.0/37.6   54.9/54.7/51.8/50.0/58.0          (2 MiB: 25.5/25.3/24.1/25.4/27.1)
-// Below the window the form loses (16 ranks x 2 MiB 12.5/12.4/13.5/14.0/14.3, 2.5 MiB 17.5/17.4/15.5/16.2/16.5; 12 ranks x
-// 2 MiB 10.0/10.0/10.5/10.9/10.6; 24 ranks x 2 MiB 18.9/18.9/19.0/19.6/20.4; 2 to 4 ranks never gain; 64 ranks x 1 MiB
-// 28.6/28.5/34.5/33.5/37.6).  Three wavefronts lose at 7 MiB where two still gain.  As a bare kernel eight wavefronts
-// are the best (8 ranks x 4 MiB: 14.8 one tile per wavefront, 12.7 three wavefronts, 12.2 eight); inside the library
-// eight measured 13.9 against 13.8 for three, so the workgroup limit stays at 256 lanes.
-// HCCL_AMD_REDUCE_ALL_FOLD = 0 / 2 .. 4 forces.
 // A flat fold of up to eight leaves to two to eight destinations launched from its arguments alone
 // (DirectFoldKernel; every operand on a 16-byte boundary, the first destination on a 128-byte line): wavefronts per
 // workgroup, 0 = not this form.  Nothing but one block of scalar loads stands in front of a wavefront's first vector
@@ -120,6 +100,45 @@ inline uint32_t DirectFoldWaves(uint32_t nLeaves, uint32_t nDst, uint64_t bytesP
     return best;
 }
 
+// The straight-line instantiation of that kernel (eight leaves, eight destinations, eight wavefronts) with two tiles
+// per wavefront, for a multiple of 16 KiB per rank: sixteen loads in flight per lane, and 16 KiB in a row to every
+// destination.  True where it is taken, and then with eight wavefronts whatever DirectFoldWaves says.  AllReduce
+// fp32 SUM over 8 ranks, us per collective, DirectFoldWaves' count with one tile per wavefront / eight wavefronts
+// with two:  2 MiB 6.6 / 6.8, 3 MiB 8.6 / 8.8, 4 MiB 12.9 / 11.2, 5 MiB 15.6 / 17.0 (320 workgroups on 256 CUs),
+// 6 MiB 18.5 / 18.0, 7 MiB 22.9 / 20.9, 8 MiB 25.4 / 23.5, 10 MiB 31.1 / 31.2, 12 MiB 36.6 / 35.5.
+// HCCL_AMD_REDUCE_DIRECT_TILES = 1 / 2 forces.
+inline bool DirectFoldTwoTiles(uint32_t nLeaves, uint32_t nDst, uint64_t bytesPerRank)
+{
+    if (nLeaves != 8 || nDst != 8 || bytesPerRank % (16 * 1024) != 0 || 2 * bytesPerRank < 7 * kMiB ||
+        bytesPerRank > 12 * kMiB) {
+        return false;
+    }
+    constexpr uint64_t kCus = 256;
+    const uint64_t groups = bytesPerRank / (16 * 1024);
+    const uint64_t rounds = (groups + kCus - 1) / kCus;
+    return groups * 100 >= 70 * rounds * kCus;   // the workgroups fill whole rounds of the CUs to 70 %
+}
+
+// Every wavefront of a workgroup folds a tile of its own and, after an exchange through LDS, stores the tiles of all
+// to its own destinations (kStoreWavesAllFold; flat programs, one sub-segment): the number of wavefronts per
+// workgroup, 0 = not this form.  Between the launch that is one generation of wavefronts and the one that reaches a
+// steady state, a fused launch to many destinations ends with every wavefront writing 1 KiB to every stream; with
+// three wavefronts exchanging their tiles each writes 3 KiB in a row to a third of the streams.  AllReduce fp32 SUM in
+// rank order, us per collective: one tile per wavefront / two / this form with 2 / 3 / 4 wavefronts:
+//   ranks    3 MiB                 4 MiB                      5 MiB                 6 MiB                      7 MiB              7.5 - 8 MiB per rank
+//     5                   10.4/ 9.3/ 9.8/ 9.3/ 9.5   12.0/10.7/10.5/10.4/10.7   13.9/13.1/12.0/12.1/12.6   15.6/15.5/14.3/16.3/14.5
+//     6                   12.1/10.7/11.3/10.5/11.1   13.9/13.3/12.5/11.9/12.7   16.0/15.2/14.4/14.2/15.4   18.0/17.8/16.7/18.7/17.1   19.9/20.1/21.1/20.5/21.4
+//     8   9.9/9.6/10.4/10.2/10.7   15.8/14.3/14.2/13.8/14.1   17.3/16.8/15.8/15.4/16.1   20.7/20.0/18.8/19.0/19.5   23.6/23.8/22.2/24.9/22.9   26.3/27.4/30.6/28.4/30.4
+//    12   15.3/15.3/14.7/14.3/15.0   21.4/21.3/19.8/19.0/20.3                       31.2/31.3/27.3/27.8/29.4   35.6/35.6/34.6/36.1/35.2
+//    16   20.3/20.2/18.2/18.3/19.2   28.8/28.7/26.2/25.1/27.0                       39.5/39.5/36.6/36.9/39.4   47.6/47.5/44.1/48.5/46.0   (8 MiB: two kernels)
+//    24   28.0/27.9/26.8/26.8/28.3   42.0/41.8/39.2/38.1/41.3
+//    32   37.9/37.7/35.8/35.0/37.6   54.9/54.7/51.8/50.0/58.0          (2 MiB: 25.5/25.3/24.1/25.4/27.1)
+// Below the window the form loses (16 ranks x 2 MiB 12.5/12.4/13.5/14.0/14.3, 2.5 MiB 17.5/17.4/15.5/16.2/16.5; 12 ranks x
+// 2 MiB 10.0/10.0/10.5/10.9/10.6; 24 ranks x 2 MiB 18.9/18.9/19.0/19.6/20.4; 2 to 4 ranks never gain; 64 ranks x 1 MiB
+// 28.6/28.5/34.5/33.5/37.6).  Three wavefronts lose at 7 MiB where two still gain.  As a bare kernel eight wavefronts
+// are the best (8 ranks x 4 MiB: 14.8 one tile per wavefront, 12.7 three wavefronts, 12.2 eight); inside the library
+// eight measured 13.9 against 13.8 for three, so the workgroup limit stays at 256 lanes.
+// HCCL_AMD_REDUCE_ALL_FOLD = 0 / 2 .. 4 forces.
 inline uint32_t AllFoldWaves(uint32_t nDst, uint64_t bytesPerRank)
 {
     if (nDst < 5 || nDst > 32 || bytesPerRank > 7 * kMiB) {

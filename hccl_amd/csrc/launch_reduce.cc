@@ -91,9 +91,14 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
     }
     {
         DirectFoldArgs d;
-        const uint32_t waves = DirectFoldWaves(w, a, plan, esz, &d);
+        uint32_t waves = DirectFoldWaves(w, a, plan, esz, &d);
         if (waves != 0) {
-            HIP_OK(LaunchDirectFold(d, dtype, op, waves, s));
+            uint32_t tiles = w->reduceDirectTiles != 0 ? static_cast<uint32_t>(w->reduceDirectTiles) : 1u;
+            if (w->reduceDirectTiles == 0 && w->reduceDirect < 0 && policy::DirectFoldTwoTiles(d.nSrc, d.nDst, a.total * esz)) {
+                waves = 8;
+                tiles = 2;
+            }
+            HIP_OK(LaunchDirectFold(d, dtype, op, waves, tiles, s));
             return HCCL_SUCCESS;
         }
     }

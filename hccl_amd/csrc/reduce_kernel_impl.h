@@ -1067,18 +1067,20 @@ __global__ __launch_bounds__(64 * kDirectFoldMaxWaves) void DirectFoldKernel(con
 }
 
 // The same for exactly eight leaves, eight destinations, eight wavefronts per workgroup and a vector count that
-// fills every workgroup (a multiple of 512; no elements behind the last vector): straight-line code without a count
-// or bounds check.  At a few MiB per rank every wavefront of the launch is resident at once and shares its SIMD's
+// fills every workgroup (a multiple of 512, or of 1024 with K = 2 tiles per wavefront; no elements behind the last
+// vector): straight-line code without a count or bounds check.  At a few MiB per rank every wavefront of the launch is resident at once and shares its SIMD's
 // issue slots with three others, so the instructions between a wavefront's start and its first load, and between
 // the barrier and its stores, are latency that nothing hides.
-template <class E>
+template <class E, int K>
 __global__ __launch_bounds__(64 * 8) void DirectFoldExactKernel(const DirectFoldArgs a)
 {
     using S = typename E::S;
     constexpr int W = 16 / sizeof(S);
     constexpr int kLeaves = 8;
     constexpr uint32_t kWaves = 8;
+    constexpr uint32_t kLanes = kWaves * 64;
     static_assert(kDirectFoldMaxLeaves == 8 && kDirectFoldMaxDst == 8 && kDirectFoldMaxWaves == 8, "eight of each");
+    static_assert(K == 1 || K == 2, "one or two tiles per wavefront");
     extern __shared__ uint32_t accStack[];
     U32x4* const parked = reinterpret_cast<U32x4*>(accStack);
     const uint32_t wave = Uniform(threadIdx.x >> 6);
@@ -1094,24 +1096,35 @@ __global__ __launch_bounds__(64 * 8) void DirectFoldExactKernel(const DirectFold
     if constexpr (HasAccumulate<E>::value) {
         one = OpaqueOne();
     }
-    const uint64_t first = static_cast<uint64_t>(blockIdx.x) * (kWaves * 64);   // the workgroup's first vector
-    U32x4 raw[kLeaves];
+    // the workgroup's first vector; with two tiles per wavefront the second round of eight tiles follows the first
+    const uint64_t first = static_cast<uint64_t>(blockIdx.x) * (K * kLanes);
+    U32x4 raw[K][kLeaves];
 #pragma unroll
-    for (int i = 0; i < kLeaves; ++i) {
-        raw[i] = __builtin_nontemporal_load(reinterpret_cast<const HCCL_AMD_GLOBAL U32x4*>(leaf[i]) + first + threadIdx.x);
-    }
-    IssueFence8(raw);
-    AccPack<E, W> acc;
-    PackOps<E, W>::Init(acc, __builtin_bit_cast(Pack<S, W>, raw[0]));
+    for (int k = 0; k < K; ++k) {
 #pragma unroll
-    for (int i = 1; i < kLeaves; ++i) {
-        PackOps<E, W>::Accumulate(acc, __builtin_bit_cast(Pack<S, W>, raw[i]), one);
+        for (int i = 0; i < kLeaves; ++i) {
+            raw[k][i] = __builtin_nontemporal_load(reinterpret_cast<const HCCL_AMD_GLOBAL U32x4*>(leaf[i]) + first +
+                                                   k * kLanes + threadIdx.x);
+        }
     }
-    parked[threadIdx.x] = __builtin_bit_cast(U32x4, PackOps<E, W>::Narrow(acc));
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        IssueFence8(raw[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        AccPack<E, W> acc;
+        PackOps<E, W>::Init(acc, __builtin_bit_cast(Pack<S, W>, raw[k][0]));
+#pragma unroll
+        for (int i = 1; i < kLeaves; ++i) {
+            PackOps<E, W>::Accumulate(acc, __builtin_bit_cast(Pack<S, W>, raw[k][i]), one);
+        }
+        parked[k * kLanes + threadIdx.x] = __builtin_bit_cast(U32x4, PackOps<E, W>::Narrow(acc));
+    }
     __syncthreads();
     HCCL_AMD_GLOBAL U32x4* const out = reinterpret_cast<HCCL_AMD_GLOBAL U32x4*>(to) + first + lane;
 #pragma unroll
-    for (uint32_t t = 0; t < kWaves; ++t) {
+    for (uint32_t t = 0; t < K * kWaves; ++t) {
         __builtin_nontemporal_store(parked[t * 64 + lane], out + t * 64);
     }
 }
@@ -1130,21 +1143,23 @@ detail::ReduceKernelFn SelectReduceF16(int op, int batch);
 detail::ReduceKernelFn SelectReduceBf16(int op, int batch);
 detail::ReduceKernelFn SelectReduceF32(int op, int batch);
 detail::ReduceKernelFn SelectReduceF64(int op, int batch);
-detail::DirectFoldFn SelectReduceI8Direct(int op, bool exact);
-detail::DirectFoldFn SelectReduceI16Direct(int op, bool exact);
-detail::DirectFoldFn SelectReduceI32Direct(int op, bool exact);
-detail::DirectFoldFn SelectReduceI64Direct(int op, bool exact);
-detail::DirectFoldFn SelectReduceU64Direct(int op, bool exact);
-detail::DirectFoldFn SelectReduceF16Direct(int op, bool exact);
-detail::DirectFoldFn SelectReduceBf16Direct(int op, bool exact);
-detail::DirectFoldFn SelectReduceF32Direct(int op, bool exact);
-detail::DirectFoldFn SelectReduceF64Direct(int op, bool exact);
+detail::DirectFoldFn SelectReduceI8Direct(int op, int exact);
+detail::DirectFoldFn SelectReduceI16Direct(int op, int exact);
+detail::DirectFoldFn SelectReduceI32Direct(int op, int exact);
+detail::DirectFoldFn SelectReduceI64Direct(int op, int exact);
+detail::DirectFoldFn SelectReduceU64Direct(int op, int exact);
+detail::DirectFoldFn SelectReduceF16Direct(int op, int exact);
+detail::DirectFoldFn SelectReduceBf16Direct(int op, int exact);
+detail::DirectFoldFn SelectReduceF32Direct(int op, int exact);
+detail::DirectFoldFn SelectReduceF64Direct(int op, int exact);
 
 #define HCCL_AMD_PICK(T, batch)                                                                \
     ((batch) == 8 ? detail::ReduceKernel<T, 8>                                                 \
                   : (batch) == 16 ? detail::ReduceKernel<T, 16> : detail::ReduceKernel<T, 8, true>)
 
-#define HCCL_AMD_PICK_DIRECT(T, exact) ((exact) ? detail::DirectFoldExactKernel<T> : detail::DirectFoldKernel<T>)
+#define HCCL_AMD_PICK_DIRECT(T, exact)                                                              \
+    ((exact) == 1 ? detail::DirectFoldExactKernel<T, 1>                                             \
+                  : (exact) == 2 ? detail::DirectFoldExactKernel<T, 2> : detail::DirectFoldKernel<T>)
 
 #define HCCL_AMD_DEFINE_SELECT4(NAME, SUM_T, PROD_T, MAX_T, MIN_T)                 \
     detail::ReduceKernelFn NAME(int op, int batch)                                \
@@ -1157,7 +1172,7 @@ detail::DirectFoldFn SelectReduceF64Direct(int op, bool exact);
             default: return nullptr;                                              \
         }                                                                         \
     }                                                                             \
-    detail::DirectFoldFn NAME##Direct(int op, bool exact)                         \
+    detail::DirectFoldFn NAME##Direct(int op, int exact)                         \
     {                                                                             \
         switch (op) {                                                             \
             case detail::kSum: return HCCL_AMD_PICK_DIRECT(SUM_T, exact);         \
@@ -1178,7 +1193,7 @@ detail::DirectFoldFn SelectReduceF64Direct(int op, bool exact);
             default: return nullptr;                                              \
         }                                                                         \
     }                                                                             \
-    detail::DirectFoldFn NAME##Direct(int op, bool exact)                         \
+    detail::DirectFoldFn NAME##Direct(int op, int exact)                         \
     {                                                                             \
         switch (op) {                                                             \
             case detail::kSum: return HCCL_AMD_PICK_DIRECT(SUM_T, exact);         \

@@ -57,13 +57,13 @@ hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp
 }
 
 hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t waves,
-                            hipStream_t stream)
+                            uint32_t tilesPerWave, hipStream_t stream)
 {
     detail::DirectFoldFn fn = nullptr;
     const int o = static_cast<int>(op);
     // eight of everything and only whole workgroups: the straight-line kernel
-    const bool exact = waves == 8 && args.nSrc == 8 && args.nDst == 8 && args.tail == 0 && args.nVec != 0 &&
-                       args.nVec % (8 * 64) == 0;
+    const bool eights = waves == 8 && args.nSrc == 8 && args.nDst == 8 && args.tail == 0 && args.nVec != 0;
+    const int exact = !eights ? 0 : (tilesPerWave == 2 && args.nVec % (2 * 8 * 64) == 0) ? 2 : args.nVec % (8 * 64) == 0 ? 1 : 0;
     switch (dtype) {
         case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8Direct(o, exact); break;
         case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16Direct(o, exact); break;
@@ -104,13 +104,14 @@ hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, Hccl
         }
     }
     const uint64_t tiles = (args.nVec + 63) / 64;
-    const uint64_t blocks = tiles == 0 ? 1 : (tiles + waves - 1) / waves;
+    const uint32_t perGroup = waves * (exact == 2 ? 2u : 1u);
+    const uint64_t blocks = tiles == 0 ? 1 : (tiles + perGroup - 1) / perGroup;
     if (blocks > 0x7FFFFFFFull) {
         return hipErrorInvalidValue;
     }
     DirectFoldArgs a = args;
     a.waves = waves;
-    hipLaunchKernelGGL(fn, dim3(static_cast<uint32_t>(blocks)), dim3(64 * waves), waves * 1024u, stream, a);
+    hipLaunchKernelGGL(fn, dim3(static_cast<uint32_t>(blocks)), dim3(64 * waves), perGroup * 1024u, stream, a);
     return hipGetLastError();
 }
 

@@ -134,7 +134,10 @@ def all_reduce_small_rows(torch, h, ranks, kibs, rounds, only=None):
                      ("fold2", dict(off, HCCL_AMD_REDUCE_ALL_FOLD="2")), ("fold3", dict(off, HCCL_AMD_REDUCE_ALL_FOLD="3")),
                      ("fold4", dict(off, HCCL_AMD_REDUCE_ALL_FOLD="4"))]
             if n <= 8:
-                forms += [("direct%d" % k, {"HCCL_AMD_REDUCE_DIRECT": str(k)}) for k in (2, 3, 4, 6, 8)]
+                forms += [("direct%d" % k, {"HCCL_AMD_REDUCE_DIRECT": str(k), "HCCL_AMD_REDUCE_DIRECT_TILES": "1"})
+                          for k in (2, 3, 4, 6, 8)]
+            if n == 8:
+                forms.append(("direct8x2", {"HCCL_AMD_REDUCE_DIRECT": "8", "HCCL_AMD_REDUCE_DIRECT_TILES": "2"}))
             if only is not None:
                 forms = [f for f in forms if f[0] in only]
             forms.append(("auto", {}))

@@ -552,6 +552,33 @@ def test_all_reduce_launched_from_its_arguments_alone(monkeypatch, n, waves):
         w.close()
 
 
+def test_all_reduce_launched_from_its_arguments_with_two_tiles_per_wavefront(monkeypatch):
+    """The straight-line instantiation that takes two tiles per wavefront (eight ranks, eight wavefronts, a multiple of
+    16 KiB per rank), asked for by name: every type and operator at sizes it takes, and sizes that only the one-tile
+    instantiation (a multiple of 8 KiB) or the kernel with counts takes."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_DIRECT", "8")
+    monkeypatch.setenv("HCCL_AMD_REDUCE_DIRECT_TILES", "2")
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "0")
+    w = World(8)
+    for k in ("HCCL_AMD_REDUCE_DIRECT", "HCCL_AMD_REDUCE_DIRECT_TILES", "HCCL_AMD_ALLREDUCE_TWO_KERNELS"):
+        monkeypatch.delenv(k)
+    try:
+        seed = 7300
+        for dtype in REDUCE_TYPES:
+            esz = np.dtype(NP[dtype]).itemsize
+            for op in (SUM, PROD, MAX, MIN):
+                if op == PROD and dtype in (DT.INT16, DT.BFP16):
+                    continue
+                run_all_reduce(w, dtype, op, 3 * 16384 // esz, "mesh", seed=seed, in_place=(op == MIN))
+                seed += 1
+        for kib in (16, 8, 24, 40, 64):
+            run_all_reduce(w, DT.FP32, SUM, kib * 256, "mesh", seed=seed + kib)
+        run_all_reduce(w, DT.FP32, SUM, 16 * 256 + 4, "mesh", seed=seed + 1)
+        run_all_reduce(w, DT.BFP16, SUM, 32 * 512 - 8, "mesh", seed=seed + 2)
+    finally:
+        w.close()
+
+
 def test_prepared_group_issues_the_same_collective():
     """hccl_amd.prepared_group converts the arguments of a group's calls once; what it runs is the plain sequence
     HcclGroupStart, the entry points, HcclGroupEnd, and a bad argument still raises with the entry point's code."""

@@ -20,11 +20,11 @@ int main()
         160ull << 20, 256ull << 20, 1ull << 30, 8ull << 30};
     for (unsigned n = 1; n <= 64; ++n) {
         for (unsigned long long b : sizes) {
-            std::printf("%u %llu %d %d %d %d %u %u %u %u %d %d %u %u\n", n, b, (int)FoldThenFanOut(n, b),
+            std::printf("%u %llu %d %d %d %d %u %u %u %u %d %d %u %u %d\n", n, b, (int)FoldThenFanOut(n, b),
                         (int)GatherThenFanOut(n, b, true), (int)GatherThenFanOut(n, b, false), (int)PairTiles(n, false, b),
                         StoreWaves(n, b, 4), StoreWaves(n, b, 2), VecBatch(n, false, false), VecBatch(n, true, false),
                         (int)FanOutStreamLoad(n, false), (int)FanOutStreamLoad(n, true), AllFoldWaves(n, b),
-                        DirectFoldWaves(n < 8 ? n : 8, n < 8 ? n : 8, b));
+                        DirectFoldWaves(n < 8 ? n : 8, n < 8 ? n : 8, b), (int)DirectFoldTwoTiles(n, n, b));
         }
     }
     return 0;
@@ -44,7 +44,7 @@ def table(tmp_path_factory):
         v = [int(x) for x in line.split()]
         rows[(v[0], v[1])] = dict(fold=v[2], gather=v[3], gather_general=v[4], pair=v[5], waves4=v[6], waves2=v[7],
                                   batch_many=v[8], batch_one=v[9], nt_single=v[10], nt_several=v[11], all_fold=v[12],
-                                  direct=v[13])
+                                  direct=v[13], two_tiles=v[14])
     return rows
 
 
@@ -105,6 +105,18 @@ def test_the_kernel_launched_from_its_arguments_covers_everything_up_to_its_limi
     assert table[(8, 5 << 20)]["direct"] == 4 and table[(8, 6 << 20)]["direct"] == 8
     assert table[(8, 8 << 20)]["direct"] == 8 and table[(8, (8 << 20) + 1)]["direct"] == 3
     assert table[(8, 16 << 20)]["direct"] == 0 and table[(4, 16 << 20)]["direct"] == 3
+
+
+def test_two_tiles_per_wavefront_only_for_eight_ranks_and_whole_workgroups(table):
+    """Eight leaves and destinations, a multiple of 16 KiB between 3.5 and 12 MiB per rank whose workgroups of sixteen
+    tiles fill the CUs (4 MiB: 256 workgroups; 5 MiB: 320, left to the one-tile forms)."""
+    for (n, b), row in table.items():
+        if row["two_tiles"]:
+            assert n == 8 and b % (16 << 10) == 0 and (7 << 19) <= b <= (12 << 20), (n, b)
+    assert table[(8, 4 << 20)]["two_tiles"] and table[(8, 7 << 20)]["two_tiles"] and table[(8, 8 << 20)]["two_tiles"]
+    assert table[(8, 6 << 20)]["two_tiles"]
+    assert not table[(8, 5 << 20)]["two_tiles"] and not table[(8, 3 << 20)]["two_tiles"]
+    assert not table[(8, (8 << 20) + 1)]["two_tiles"] and not table[(8, 16 << 20)]["two_tiles"]
 
 
 def test_the_pair_form_has_one_window_of_sizes(table):
