@@ -245,7 +245,7 @@ hipError_t LaunchMark(uint64_t* word, uint64_t value, hipStream_t stream);
 hipError_t LaunchReduce(const ReduceArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t nBlocks,
                         uint32_t ldsBytes, hipStream_t stream);
 // Workgroups of `waves` wavefronts (2 .. kDirectFoldMaxWaves), one 1 KiB tile per wavefront; tilesPerWave = 2: two
-// where the straight-line instantiation fits (eight leaves, destinations and wavefronts, a multiple of 16 KiB).
+// where the launch is whole workgroups of 2 * waves tiles.
 hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, HcclReduceOp op, uint32_t waves,
                             uint32_t tilesPerWave, hipStream_t stream);
 inline uint32_t ReduceAccBytes(HcclDataType dtype, HcclReduceOp op)

@@ -100,17 +100,26 @@ inline uint32_t DirectFoldWaves(uint32_t nLeaves, uint32_t nDst, uint64_t bytesP
     return best;
 }
 
-// The straight-line instantiation of that kernel (eight leaves, eight destinations, eight wavefronts) with two tiles
-// per wavefront, for a multiple of 16 KiB per rank: sixteen loads in flight per lane, and 16 KiB in a row to every
-// destination.  True where it is taken, and then with eight wavefronts whatever DirectFoldWaves says.  AllReduce
-// fp32 SUM over 8 ranks, us per collective, DirectFoldWaves' count with one tile per wavefront / eight wavefronts
-// with two:  2 MiB 6.6 / 6.8, 3 MiB 8.6 / 8.8, 4 MiB 12.9 / 11.2, 5 MiB 15.6 / 17.0 (320 workgroups on 256 CUs),
-// 6 MiB 18.5 / 18.0, 7 MiB 22.9 / 20.9, 8 MiB 25.4 / 23.5, 10 MiB 31.1 / 31.2, 12 MiB 36.6 / 35.5.
+// That kernel with eight wavefronts and two tiles per wavefront, for a multiple of 16 KiB per rank: sixteen loads in
+// flight per lane, half as many workgroups, and 16 KiB in a row to every destination.  True where it is taken, and
+// then with eight wavefronts whatever DirectFoldWaves says.  AllReduce fp32 SUM, us per collective, DirectFoldWaves'
+// count with one tile per wavefront / eight wavefronts with two:
+//   ranks   3 MiB        4 MiB         6 MiB         8 MiB         12 MiB        16 MiB per rank
+//     8   8.6 / 8.8   12.9 / 11.2   18.5 / 18.0   25.4 / 23.5   36.6 / 35.5                 (2 MiB 6.6 / 6.8, 7 MiB 22.9 / 20.9)
+//     7               11.9 / 10.2   16.8 / 16.2   22.6 / 19.5   32.1 / 29.9
+//     6   6.7 / 7.2    9.4 / 9.0    14.3 / 14.6   19.1 / 16.9   27.5 / 25.0
+//     5                7.9 / 7.8                  15.9 / 14.5
+//     4   5.5 / 5.5    6.6 / 6.6    10.1 / 10.1   13.3 / 12.3   18.7 / 18.4   24.3 / 24.9
+//     3                5.7 / 5.4                  10.4 / 8.3                  18.7 / 18.3
+//     2                4.4 / 4.4                   7.2 / 6.3                  12.8 / 13.9
+// It pays where the workgroups of sixteen tiles come out even over the 256 CUs (4 MiB: 256 of them, 8 MiB: 512) and
+// not where they do not (8 ranks x 5 MiB: 320 workgroups, 15.6 / 16.8; 10 MiB: 640, 31.1 / 31.5).
 // HCCL_AMD_REDUCE_DIRECT_TILES = 1 / 2 forces.
 inline bool DirectFoldTwoTiles(uint32_t nLeaves, uint32_t nDst, uint64_t bytesPerRank)
 {
-    if (nLeaves != 8 || nDst != 8 || bytesPerRank % (16 * 1024) != 0 || 2 * bytesPerRank < 7 * kMiB ||
-        bytesPerRank > 12 * kMiB) {
+    (void)nLeaves;
+    (void)nDst;
+    if (bytesPerRank % (16 * 1024) != 0 || 2 * bytesPerRank < 7 * kMiB || bytesPerRank > 12 * kMiB) {
         return false;
     }
     constexpr uint64_t kCus = 256;

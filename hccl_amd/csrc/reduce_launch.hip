@@ -63,7 +63,9 @@ hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, Hccl
     const int o = static_cast<int>(op);
     // eight of everything and only whole workgroups: the straight-line kernel
     const bool eights = waves == 8 && args.nSrc == 8 && args.nDst == 8 && args.tail == 0 && args.nVec != 0;
-    const int exact = !eights ? 0 : (tilesPerWave == 2 && args.nVec % (2 * 8 * 64) == 0) ? 2 : args.nVec % (8 * 64) == 0 ? 1 : 0;
+    const bool twoTiles = tilesPerWave == 2 && args.tail == 0 && args.nVec != 0 && waves != 0 &&
+                          args.nVec % (2 * 64 * static_cast<uint64_t>(waves)) == 0;
+    const int exact = eights ? (twoTiles ? 2 : args.nVec % (8 * 64) == 0 ? 1 : 0) : (twoTiles ? 3 : 0);
     switch (dtype) {
         case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8Direct(o, exact); break;
         case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16Direct(o, exact); break;
@@ -104,7 +106,7 @@ hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, Hccl
         }
     }
     const uint64_t tiles = (args.nVec + 63) / 64;
-    const uint32_t perGroup = waves * (exact == 2 ? 2u : 1u);
+    const uint32_t perGroup = waves * (exact >= 2 ? 2u : 1u);
     const uint64_t blocks = tiles == 0 ? 1 : (tiles + perGroup - 1) / perGroup;
     if (blocks > 0x7FFFFFFFull) {
         return hipErrorInvalidValue;

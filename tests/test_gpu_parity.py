@@ -552,29 +552,32 @@ def test_all_reduce_launched_from_its_arguments_alone(monkeypatch, n, waves):
         w.close()
 
 
-def test_all_reduce_launched_from_its_arguments_with_two_tiles_per_wavefront(monkeypatch):
-    """The straight-line instantiation that takes two tiles per wavefront (eight ranks, eight wavefronts, a multiple of
-    16 KiB per rank), asked for by name: every type and operator at sizes it takes, and sizes that only the one-tile
-    instantiation (a multiple of 8 KiB) or the kernel with counts takes."""
-    monkeypatch.setenv("HCCL_AMD_REDUCE_DIRECT", "8")
+@pytest.mark.parametrize("n,waves", [(8, 8), (8, 4), (2, 4), (3, 8), (4, 8), (5, 2), (6, 8), (7, 3)])
+def test_all_reduce_launched_from_its_arguments_with_two_tiles_per_wavefront(monkeypatch, n, waves):
+    """The instantiations that take two tiles per wavefront (whole workgroups of 2 * waves tiles only; straight-line
+    code for eight ranks and eight wavefronts), asked for by name: every type and operator at sizes they take, and
+    sizes that only the one-tile kernels take (half a workgroup more, elements behind the last vector)."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_DIRECT", str(waves))
     monkeypatch.setenv("HCCL_AMD_REDUCE_DIRECT_TILES", "2")
     monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "0")
-    w = World(8)
+    w = World(n)
     for k in ("HCCL_AMD_REDUCE_DIRECT", "HCCL_AMD_REDUCE_DIRECT_TILES", "HCCL_AMD_ALLREDUCE_TWO_KERNELS"):
         monkeypatch.delenv(k)
     try:
-        seed = 7300
+        seed = 7300 + 100 * n + waves
+        group = 2 * waves * 1024           # bytes of one workgroup
         for dtype in REDUCE_TYPES:
             esz = np.dtype(NP[dtype]).itemsize
             for op in (SUM, PROD, MAX, MIN):
                 if op == PROD and dtype in (DT.INT16, DT.BFP16):
                     continue
-                run_all_reduce(w, dtype, op, 3 * 16384 // esz, "mesh", seed=seed, in_place=(op == MIN))
+                run_all_reduce(w, dtype, op, 3 * group // esz, "mesh", seed=seed, in_place=(op == MIN))
                 seed += 1
-        for kib in (16, 8, 24, 40, 64):
-            run_all_reduce(w, DT.FP32, SUM, kib * 256, "mesh", seed=seed + kib)
-        run_all_reduce(w, DT.FP32, SUM, 16 * 256 + 4, "mesh", seed=seed + 1)
-        run_all_reduce(w, DT.BFP16, SUM, 32 * 512 - 8, "mesh", seed=seed + 2)
+        for groups2 in (2, 1, 3, 5, 8):    # halves of a workgroup
+            run_all_reduce(w, DT.FP32, SUM, groups2 * group // 8, "mesh", seed=seed + groups2)
+        run_all_reduce(w, DT.FP32, SUM, group // 4 + 4, "mesh", seed=seed + 11)
+        run_all_reduce(w, DT.BFP16, SUM, 2 * group // 2 - 8, "mesh", seed=seed + 12)
+        run_all_reduce(w, DT.INT8, MAX, group + 5, "mesh", seed=seed + 13)
     finally:
         w.close()
 

@@ -107,12 +107,13 @@ def test_the_kernel_launched_from_its_arguments_covers_everything_up_to_its_limi
     assert table[(8, 16 << 20)]["direct"] == 0 and table[(4, 16 << 20)]["direct"] == 3
 
 
-def test_two_tiles_per_wavefront_only_for_eight_ranks_and_whole_workgroups(table):
-    """Eight leaves and destinations, a multiple of 16 KiB between 3.5 and 12 MiB per rank whose workgroups of sixteen
-    tiles fill the CUs (4 MiB: 256 workgroups; 5 MiB: 320, left to the one-tile forms)."""
+def test_two_tiles_per_wavefront_only_for_whole_workgroups_that_fill_the_cus(table):
+    """A multiple of 16 KiB between 3.5 and 12 MiB per rank whose workgroups of sixteen tiles fill the CUs (4 MiB: 256
+    workgroups; 5 MiB: 320, left to the one-tile forms)."""
     for (n, b), row in table.items():
         if row["two_tiles"]:
-            assert n == 8 and b % (16 << 10) == 0 and (7 << 19) <= b <= (12 << 20), (n, b)
+            assert b % (16 << 10) == 0 and (7 << 19) <= b <= (12 << 20), (n, b)
+    assert table[(4, 8 << 20)]["two_tiles"] and table[(2, 4 << 20)]["two_tiles"]
     assert table[(8, 4 << 20)]["two_tiles"] and table[(8, 7 << 20)]["two_tiles"] and table[(8, 8 << 20)]["two_tiles"]
     assert table[(8, 6 << 20)]["two_tiles"]
     assert not table[(8, 5 << 20)]["two_tiles"] and not table[(8, 3 << 20)]["two_tiles"]
