@@ -115,9 +115,12 @@ struct ReduceArgs : ReduceHot {
 constexpr uint32_t kDirectFoldMaxLeaves = 8;
 constexpr uint32_t kDirectFoldMaxDst = 8;
 constexpr uint32_t kDirectFoldMaxWaves = 8;    // wavefronts per workgroup, 1 KiB of dynamic LDS each
+// One instantiation takes up to sixteen leaves and destinations (whole workgroups only, one tile per wavefront).
+constexpr uint32_t kDirectFoldWideLeaves = 16;
+constexpr uint32_t kDirectFoldWideDst = 16;
 struct DirectFoldArgs {
-    const void* src[kDirectFoldMaxLeaves];
-    void* dst[kDirectFoldMaxDst];
+    const void* src[kDirectFoldWideLeaves];
+    void* dst[kDirectFoldWideDst];
     uint64_t nVec;
     uint32_t nSrc;
     uint32_t nDst;

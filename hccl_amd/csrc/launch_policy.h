@@ -100,6 +100,30 @@ inline uint32_t DirectFoldWaves(uint32_t nLeaves, uint32_t nDst, uint64_t bytesP
     return best;
 }
 
+// That kernel's instantiation for nine to sixteen leaves or destinations (whole workgroups only, one tile per
+// wavefront): wavefronts per workgroup, 0 = not this form.  AllReduce fp32 SUM in rank order, us per collective, the
+// general kernel's best form (one tile per wavefront or wavefronts that exchange their tiles) / this kernel with
+// 2 / 4 / 8 wavefronts:
+//   ranks   512 KiB             1 MiB                2 MiB                  3 MiB                  4 MiB                  6 MiB per rank
+//    16   9.8 / 9.5 9.8 9.7   10.0 / 9.5 9.6 9.7   13.4 / 11.9 12.5 11.3   18.2 / 18.6 18.7 17.7   24.9 / 27.5 25.7 26.4   36.4 / 37.0 38.1 36.8
+//    12                        8.6 / 8.0 8.3 8.3   10.6 /  8.7  9.3  8.9   14.4 / 14.7 14.4 14.4   19.0 / 21.4 19.9 20.3   27.3 / 27.8 28.7 27.7
+//    10                                             8.6 /  7.6  8.0  7.9                          16.0 / 16.9 16.9 16.1
+//     9                                             8.7 /  7.1  7.2  7.3                          14.9 / 17.0 16.2 14.4
+// (16 ranks x 8 MiB, where fold + fan-out takes over: 48.6 for every form.)  The short launches gain what the
+// kernels for up to eight ranks gain; from 4 MiB the general kernel's exchange form is level or ahead.
+// HCCL_AMD_REDUCE_DIRECT = 0 / 2 .. 8 forces.
+inline uint32_t DirectFoldWideWaves(uint32_t nLeaves, uint32_t nDst, uint64_t bytesPerRank)
+{
+    (void)nLeaves;
+    if (bytesPerRank > 3 * kMiB) {
+        return 0;
+    }
+    if (bytesPerRank <= kMiB) {
+        return 2;
+    }
+    return (nDst >= 14 || 2 * bytesPerRank > 5 * kMiB) ? 8 : 2;
+}
+
 // That kernel with eight wavefronts and two tiles per wavefront, for a multiple of 16 KiB per rank: sixteen loads in
 // flight per lane, half as many workgroups, and 16 KiB in a row to every destination.  True where it is taken, and
 // then with eight wavefronts whatever DirectFoldWaves says.  AllReduce fp32 SUM, us per collective, DirectFoldWaves'

@@ -34,7 +34,7 @@ static uint32_t DirectFoldWaves(const World* w, const ReduceArgs& a, const Devic
                                 DirectFoldArgs* d)
 {
     if (w->reduceDirect == 0 || !w->reduceVector || a.varGroups != 0 || a.dstOwn != 0 || a.nGroup != 1 || a.nSub != 1 ||
-        a.nDst < 2 || a.nDst > kDirectFoldMaxDst || a.total == 0 || plan.host == nullptr || plan.maxDepth != 1) {
+        a.nDst < 2 || a.nDst > kDirectFoldWideDst || a.total == 0 || plan.host == nullptr || plan.maxDepth != 1) {
         return 0;
     }
     const bool forced = w->reduceDirect > 0;
@@ -48,9 +48,10 @@ static uint32_t DirectFoldWaves(const World* w, const ReduceArgs& a, const Devic
     }
     const uint8_t* img = plan.host->data() + progOff;
     const uint32_t leaves = img[0];
-    if (leaves == 0 || leaves > kDirectFoldMaxLeaves) {
+    if (leaves == 0 || leaves > kDirectFoldWideLeaves) {
         return 0;
     }
+    const bool wide = leaves > kDirectFoldMaxLeaves || a.nDst > kDirectFoldMaxDst;
     *d = DirectFoldArgs{};
     for (uint32_t i = 0; i < leaves; ++i) {
         const uint32_t rank = img[kDevProgRankOff + i];
@@ -71,6 +72,13 @@ static uint32_t DirectFoldWaves(const World* w, const ReduceArgs& a, const Devic
     d->tail = static_cast<uint32_t>(a.total % perVec);
     d->nSrc = leaves;
     d->nDst = a.nDst;
+    if (wide) {
+        // the kernel for nine to sixteen leaves or destinations takes whole workgroups only
+        const uint32_t waves = forced ? static_cast<uint32_t>(w->reduceDirect)
+                               : (reinterpret_cast<uintptr_t>(a.dst[0]) & 127u) != 0 ? 0u
+                               : policy::DirectFoldWideWaves(leaves, a.nDst, a.total * esz);
+        return waves != 0 && d->tail == 0 && d->nVec % (64ull * waves) == 0 ? waves : 0u;
+    }
     if (forced) {
         return static_cast<uint32_t>(w->reduceDirect);
     }
@@ -94,7 +102,8 @@ HcclResult LaunchOneReduce(World* w, ReduceArgs& a, const DevicePlan& plan, Hccl
         uint32_t waves = DirectFoldWaves(w, a, plan, esz, &d);
         if (waves != 0) {
             uint32_t tiles = w->reduceDirectTiles != 0 ? static_cast<uint32_t>(w->reduceDirectTiles) : 1u;
-            if (w->reduceDirectTiles == 0 && w->reduceDirect < 0 && policy::DirectFoldTwoTiles(d.nSrc, d.nDst, a.total * esz)) {
+            const bool wide = d.nSrc > kDirectFoldMaxLeaves || d.nDst > kDirectFoldMaxDst;
+            if (!wide && w->reduceDirectTiles == 0 && w->reduceDirect < 0 && policy::DirectFoldTwoTiles(d.nSrc, d.nDst, a.total * esz)) {
                 waves = 8;
                 tiles = 2;
             }

@@ -1139,6 +1139,73 @@ __global__ __launch_bounds__(64 * kDirectFoldMaxWaves) void DirectFoldTwoTileKer
     }
 }
 
+// The same for nine to sixteen leaves or destinations: one tile per wavefront, both batches of eight loads issued
+// before the first fold, whole workgroups only (a vector count that is a multiple of 64 * waves, no elements behind
+// the last vector; no bounds checks).  With two wavefronts a wavefront stores to up to eight destinations.
+template <class E>
+__global__ __launch_bounds__(64 * kDirectFoldMaxWaves) void DirectFoldWideKernel(const DirectFoldArgs a)
+{
+    using S = typename E::S;
+    constexpr int W = 16 / sizeof(S);
+    constexpr int kLeaves = static_cast<int>(kDirectFoldWideLeaves);
+    constexpr uint32_t kPerWave = kDirectFoldWideDst / 2;
+    static_assert(kLeaves == 16, "two batches of eight loads");
+    extern __shared__ uint32_t accStack[];
+    U32x4* const parked = reinterpret_cast<U32x4*>(accStack);
+    const uint32_t wave = Uniform(threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63u;
+    uint64_t leaf[kLeaves];
+#pragma unroll
+    for (int i = 0; i < kLeaves; ++i) {
+        leaf[i] = reinterpret_cast<uint64_t>(a.src[i]);
+    }
+    uint32_t nSrc = a.nSrc;
+    uint32_t nDst = a.nDst;
+    uint32_t waves = a.waves;
+    ScalarFence8(leaf);
+    ScalarFence8(leaf + 8);
+    asm volatile("" : "+s"(nSrc), "+s"(nDst), "+s"(waves));
+    uint64_t to[kPerWave];
+#pragma unroll
+    for (uint32_t k = 0; k < kPerWave; ++k) {
+        const uint32_t d = wave + k * waves;
+        to[k] = reinterpret_cast<uint64_t>(a.dst[d < kDirectFoldWideDst ? d : 0u]);
+    }
+    float one = 1.0f;
+    if constexpr (HasAccumulate<E>::value) {
+        one = OpaqueOne();
+    }
+    const uint64_t first = static_cast<uint64_t>(blockIdx.x) * (waves * 64);   // the workgroup's first vector
+    U32x4 raw[kLeaves];
+#pragma unroll
+    for (int i = 0; i < kLeaves; ++i) {
+        if (static_cast<uint32_t>(i) < nSrc) {
+            raw[i] = __builtin_nontemporal_load(reinterpret_cast<const HCCL_AMD_GLOBAL U32x4*>(leaf[i]) + first + threadIdx.x);
+        }
+    }
+    IssueFence8(raw);
+    IssueFence8(raw + 8);
+    AccPack<E, W> acc;
+    PackOps<E, W>::Init(acc, __builtin_bit_cast(Pack<S, W>, raw[0]));
+#pragma unroll
+    for (int i = 1; i < kLeaves; ++i) {
+        if (static_cast<uint32_t>(i) < nSrc) {
+            PackOps<E, W>::Accumulate(acc, __builtin_bit_cast(Pack<S, W>, raw[i]), one);
+        }
+    }
+    parked[threadIdx.x] = __builtin_bit_cast(U32x4, PackOps<E, W>::Narrow(acc));
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < kPerWave; ++k) {
+        if (wave + k * waves < nDst) {
+            HCCL_AMD_GLOBAL U32x4* const out = reinterpret_cast<HCCL_AMD_GLOBAL U32x4*>(to[k]) + first + lane;
+            for (uint32_t t = 0; t < waves; ++t) {
+                __builtin_nontemporal_store(parked[t * 64 + lane], out + t * 64);
+            }
+        }
+    }
+}
+
 // The same for exactly eight leaves, eight destinations, eight wavefronts per workgroup and a vector count that
 // fills every workgroup (a multiple of 512, or of 1024 with K = 2 tiles per wavefront; no elements behind the last
 // vector): straight-line code without a count or bounds check.  At a few MiB per rank every wavefront of the launch is resident at once and shares its SIMD's
@@ -1230,11 +1297,13 @@ detail::DirectFoldFn SelectReduceF64Direct(int op, int exact);
     ((batch) == 8 ? detail::ReduceKernel<T, 8>                                                 \
                   : (batch) == 16 ? detail::ReduceKernel<T, 16> : detail::ReduceKernel<T, 8, true>)
 
-// 0: any counts; 1 / 2: eight of everything, one / two tiles per wavefront; 3: any counts, two tiles per wavefront
+// 0: any counts; 1 / 2: eight of everything, one / two tiles per wavefront; 3: any counts, two tiles per wavefront;
+// 4: up to sixteen leaves and destinations
 #define HCCL_AMD_PICK_DIRECT(T, exact)                                                              \
     ((exact) == 1 ? detail::DirectFoldExactKernel<T, 1>                                             \
      : (exact) == 2 ? detail::DirectFoldExactKernel<T, 2>                                           \
-     : (exact) == 3 ? detail::DirectFoldTwoTileKernel<T> : detail::DirectFoldKernel<T>)
+     : (exact) == 3 ? detail::DirectFoldTwoTileKernel<T>                                            \
+     : (exact) == 4 ? detail::DirectFoldWideKernel<T> : detail::DirectFoldKernel<T>)
 
 #define HCCL_AMD_DEFINE_SELECT4(NAME, SUM_T, PROD_T, MAX_T, MIN_T)                 \
     detail::ReduceKernelFn NAME(int op, int batch)                                \

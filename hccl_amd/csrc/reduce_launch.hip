@@ -65,7 +65,8 @@ hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, Hccl
     const bool eights = waves == 8 && args.nSrc == 8 && args.nDst == 8 && args.tail == 0 && args.nVec != 0;
     const bool twoTiles = tilesPerWave == 2 && args.tail == 0 && args.nVec != 0 && waves != 0 &&
                           args.nVec % (2 * 64 * static_cast<uint64_t>(waves)) == 0;
-    const int exact = eights ? (twoTiles ? 2 : args.nVec % (8 * 64) == 0 ? 1 : 0) : (twoTiles ? 3 : 0);
+    const bool wide = args.nSrc > kDirectFoldMaxLeaves || args.nDst > kDirectFoldMaxDst;
+    const int exact = wide ? 4 : eights ? (twoTiles ? 2 : args.nVec % (8 * 64) == 0 ? 1 : 0) : (twoTiles ? 3 : 0);
     switch (dtype) {
         case HCCL_DATA_TYPE_INT8: fn = SelectReduceI8Direct(o, exact); break;
         case HCCL_DATA_TYPE_INT16: fn = SelectReduceI16Direct(o, exact); break;
@@ -87,12 +88,16 @@ hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, Hccl
         default: break;
     }
     if (fn == nullptr || esz == 0 || waves < 2 || waves > kDirectFoldMaxWaves || args.nSrc == 0 ||
-        args.nSrc > kDirectFoldMaxLeaves || args.nDst == 0 || args.nDst > kDirectFoldMaxDst || args.tail >= 16 / esz ||
+        args.nSrc > kDirectFoldWideLeaves || args.nDst == 0 || args.nDst > kDirectFoldWideDst || args.tail >= 16 / esz ||
         (args.nVec == 0 && args.tail == 0)) {
         return hipErrorInvalidValue;
     }
+    // the kernel for more than eight leaves or destinations takes whole workgroups only
+    if (wide && (args.tail != 0 || args.nVec % (64 * static_cast<uint64_t>(waves)) != 0)) {
+        return hipErrorInvalidValue;
+    }
     // a wavefront holds the addresses of at most half the destination table
-    if ((args.nDst + waves - 1) / waves > kDirectFoldMaxDst / 2) {
+    if ((args.nDst + waves - 1) / waves > (wide ? kDirectFoldWideDst : kDirectFoldMaxDst) / 2) {
         return hipErrorInvalidValue;
     }
     for (uint32_t i = 0; i < args.nSrc; ++i) {
@@ -106,7 +111,7 @@ hipError_t LaunchDirectFold(const DirectFoldArgs& args, HcclDataType dtype, Hccl
         }
     }
     const uint64_t tiles = (args.nVec + 63) / 64;
-    const uint32_t perGroup = waves * (exact >= 2 ? 2u : 1u);
+    const uint32_t perGroup = waves * (exact == 2 || exact == 3 ? 2u : 1u);   // tiles of one workgroup
     const uint64_t blocks = tiles == 0 ? 1 : (tiles + perGroup - 1) / perGroup;
     if (blocks > 0x7FFFFFFFull) {
         return hipErrorInvalidValue;

@@ -138,6 +138,8 @@ def all_reduce_small_rows(torch, h, ranks, kibs, rounds, only=None):
                           for k in (2, 3, 4, 6, 8)]
                 forms += [("direct%dx2" % k, {"HCCL_AMD_REDUCE_DIRECT": str(k), "HCCL_AMD_REDUCE_DIRECT_TILES": "2"})
                           for k in (4, 8)]
+            elif n <= 16:
+                forms += [("direct%d" % k, {"HCCL_AMD_REDUCE_DIRECT": str(k)}) for k in (2, 4, 8)]
             if only is not None:
                 forms = [f for f in forms if f[0] in only]
             forms.append(("auto", {}))

@@ -582,6 +582,35 @@ def test_all_reduce_launched_from_its_arguments_with_two_tiles_per_wavefront(mon
         w.close()
 
 
+@pytest.mark.parametrize("n,waves", [(9, 2), (12, 8), (13, 4), (16, 8), (16, 2)])
+def test_all_reduce_of_nine_to_sixteen_ranks_launched_from_its_arguments(monkeypatch, n, waves):
+    """The instantiation for nine to sixteen leaves and destinations (whole workgroups of `waves` tiles only), asked
+    for by name: every type and operator at sizes it takes, and sizes that fall to the general kernel (half a
+    workgroup more, elements behind the last vector, operands off the 16-byte grid)."""
+    monkeypatch.setenv("HCCL_AMD_REDUCE_DIRECT", str(waves))
+    monkeypatch.setenv("HCCL_AMD_ALLREDUCE_TWO_KERNELS", "0")
+    w = World(n)
+    for k in ("HCCL_AMD_REDUCE_DIRECT", "HCCL_AMD_ALLREDUCE_TWO_KERNELS"):
+        monkeypatch.delenv(k)
+    try:
+        seed = 7700 + 100 * n + waves
+        group = waves * 1024               # bytes of one workgroup
+        for dtype in REDUCE_TYPES:
+            esz = np.dtype(NP[dtype]).itemsize
+            for op in (SUM, PROD, MAX, MIN):
+                if op == PROD and dtype in (DT.INT16, DT.BFP16):
+                    continue
+                run_all_reduce(w, dtype, op, 5 * group // esz, "mesh", seed=seed, in_place=(op == MIN))
+                seed += 1
+        for halves in (2, 1, 3, 7, 16):
+            run_all_reduce(w, DT.FP32, SUM, halves * group // 8, "mesh", seed=seed + halves)
+        run_all_reduce(w, DT.FP32, SUM, group // 4 + 4, "mesh", seed=seed + 21)
+        run_all_reduce(w, DT.BFP16, SUM, 3 * group // 2, "mesh", seed=seed + 22, pad=2)
+        run_all_reduce(w, DT.FP32, SUM, 3 * group // 4, "nhr", seed=seed + 23)      # nested program: general kernel
+    finally:
+        w.close()
+
+
 def test_prepared_group_issues_the_same_collective():
     """hccl_amd.prepared_group converts the arguments of a group's calls once; what it runs is the plain sequence
     HcclGroupStart, the entry points, HcclGroupEnd, and a bad argument still raises with the entry point's code."""

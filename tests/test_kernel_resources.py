@@ -57,10 +57,10 @@ def test_every_translation_unit_is_there(kernels):
     # 34 combinations of element type and operation, each with the eight-leaf and the sixteen-leaf load batch and
     # with the eight-leaf batch over two tiles per wavefront
     assert len(reduce_kernels) == 102, sorted(k["name"] for k in reduce_kernels)
-    # and four times as the kernel that is launched from its arguments alone (any counts and eight of everything,
-    # each with one and with two tiles per wavefront)
+    # and five times as the kernel that is launched from its arguments alone (any counts and eight of everything,
+    # each with one and with two tiles per wavefront; up to sixteen leaves and destinations)
     direct_kernels = [k for k in kernels if "DirectFold" in k["name"]]
-    assert len(direct_kernels) == 136, sorted(k["name"] for k in direct_kernels)
+    assert len(direct_kernels) == 170, sorted(k["name"] for k in direct_kernels)
     # the copy, fan-out (two load flavours) and AlltoAllV kernels
     assert len(kernels) - len(reduce_kernels) - len(direct_kernels) == 22
 
@@ -76,8 +76,8 @@ def test_register_budgets(kernels):
     checked for them is that the compiler did not have to spill (above)."""
     for k in kernels:
         # (the kernel launched from its arguments: at most 64, so that the eight wavefronts a SIMD can hold all fit;
-        # with two tiles per wavefront, sixteen loaded vectors, 96 like the fold kernels)
-        two_tiles = re.search(r"DirectFoldExactKernel.*Li2EEEv|DirectFoldTwoTileKernel", k["name"]) is not None
+        # with sixteen loaded vectors, two tiles per wavefront or sixteen leaves, 96 like the fold kernels)
+        two_tiles = re.search(r"DirectFoldExactKernel.*Li2EEEv|DirectFoldTwoTileKernel|DirectFoldWideKernel", k["name"]) is not None
         limit = (96 if "ReduceKernel" in k["name"] or two_tiles else 64 if "DirectFold" in k["name"] else 24)
         assert k["vgpr"] <= limit, k
 
@@ -95,6 +95,6 @@ def test_uniform_values_are_uniform_for_the_compiler_too(kernels, tmp_path_facto
         text = subprocess.run([LLVM + "/llvm-objdump", "-d", "--mcpu=gfx950", str(obj)], stdout=subprocess.PIPE,
                               text=True, check=True).stdout
         assert "s_endpgm" in text                       # the listing is real
-        direct = len(re.findall(r"^[0-9a-f]+ <[^>+]*DirectFold(Exact|TwoTile)?Kernel[^>+]*>:$", text, re.M))
+        direct = len(re.findall(r"^[0-9a-f]+ <[^>+]*DirectFold(Exact|TwoTile|Wide)?Kernel[^>+]*>:$", text, re.M))
         counts[obj.name] = text.count("v_readfirstlane") - direct
     assert sorted(counts.values()) == [0] * (len(counts) - 1) + [2], counts   # the fan-out kernel's two load flavours

@@ -20,11 +20,12 @@ int main()
         160ull << 20, 256ull << 20, 1ull << 30, 8ull << 30};
     for (unsigned n = 1; n <= 64; ++n) {
         for (unsigned long long b : sizes) {
-            std::printf("%u %llu %d %d %d %d %u %u %u %u %d %d %u %u %d\n", n, b, (int)FoldThenFanOut(n, b),
+            std::printf("%u %llu %d %d %d %d %u %u %u %u %d %d %u %u %d %u\n", n, b, (int)FoldThenFanOut(n, b),
                         (int)GatherThenFanOut(n, b, true), (int)GatherThenFanOut(n, b, false), (int)PairTiles(n, false, b),
                         StoreWaves(n, b, 4), StoreWaves(n, b, 2), VecBatch(n, false, false), VecBatch(n, true, false),
                         (int)FanOutStreamLoad(n, false), (int)FanOutStreamLoad(n, true), AllFoldWaves(n, b),
-                        DirectFoldWaves(n < 8 ? n : 8, n < 8 ? n : 8, b), (int)DirectFoldTwoTiles(n, n, b));
+                        DirectFoldWaves(n < 8 ? n : 8, n < 8 ? n : 8, b), (int)DirectFoldTwoTiles(n, n, b),
+                        DirectFoldWideWaves(n, n, b));
         }
     }
     return 0;
@@ -44,7 +45,7 @@ def table(tmp_path_factory):
         v = [int(x) for x in line.split()]
         rows[(v[0], v[1])] = dict(fold=v[2], gather=v[3], gather_general=v[4], pair=v[5], waves4=v[6], waves2=v[7],
                                   batch_many=v[8], batch_one=v[9], nt_single=v[10], nt_several=v[11], all_fold=v[12],
-                                  direct=v[13], two_tiles=v[14])
+                                  direct=v[13], two_tiles=v[14], wide=v[15])
     return rows
 
 
@@ -118,6 +119,17 @@ def test_two_tiles_per_wavefront_only_for_whole_workgroups_that_fill_the_cus(tab
     assert table[(8, 6 << 20)]["two_tiles"]
     assert not table[(8, 5 << 20)]["two_tiles"] and not table[(8, 3 << 20)]["two_tiles"]
     assert not table[(8, (8 << 20) + 1)]["two_tiles"] and not table[(8, 16 << 20)]["two_tiles"]
+
+
+def test_the_kernel_for_nine_to_sixteen_ranks_takes_the_short_messages(table):
+    for n, rows in by_world(table).items():
+        if n < 9 or n > 16:
+            continue
+        for b, row in rows:
+            assert (row["wide"] != 0) == (b <= (3 << 20)), (n, b)
+            assert row["wide"] in (0, 2, 8), (n, b)
+    assert table[(16, 1 << 20)]["wide"] == 2 and table[(16, 2 << 20)]["wide"] == 8 and table[(12, 2 << 20)]["wide"] == 2
+    assert table[(12, 3 << 20)]["wide"] == 8 and table[(16, 4 << 20)]["wide"] == 0
 
 
 def test_the_pair_form_has_one_window_of_sizes(table):
