@@ -362,8 +362,8 @@ def measure(torch, wl, name, algo, steps, warmup):
     step, hbm, alg, bus, keep, desc, dtype, n, algo_used = getattr(wl, name)(algo)
     dev_ms, wall_ms = time_steps(torch, wl.stream, step, steps, warmup)
     t = dev_ms * 1e-3
-    out = {"workload": desc, "algorithm": algo_used, "n_ranks": n, "steps": steps, "ms_per_step": round(dev_ms, 4),
-           "wall_ms_per_step": round(wall_ms, 4),
+    out = {"workload": desc, "algorithm": algo_used, "n_ranks": n, "steps": steps, "ms_per_step": round(dev_ms, 5 if dev_ms < 0.1 else 4),
+           "wall_ms_per_step": round(wall_ms, 5 if wall_ms < 0.1 else 4),
            "algbw_GBs": round(alg / t / 1e9, 2), "busbw_GBs": round(alg / t / 1e9 * bus, 2),
            "hbm_GBs": round(hbm / t / 1e9, 2), "hbm_frac": round(hbm / t / 1e9 / HBM_PEAK_GBS, 4),
            "algorithmic_bytes": hbm, "dtype": dtype}
