@@ -434,6 +434,29 @@ __global__ __launch_bounds__(64) void MarkKernel(uint64_t* word, uint64_t value)
     }
 }
 
+// Up to eight equally long segments into one destination, everything on 16-byte boundaries and every segment's place
+// in the destination on a 128-byte line, described by the arguments alone: segment blockIdx.y, 1 KiB per wavefront.
+// A copy with one read and one write stream moves its kilobyte in two memory instructions; the general kernel's way
+// to a tile (tile prefixes, hints, alignment cases) is a few hundred instructions per wavefront, which at 128 MiB is
+// a quarter of the launch (128 MiB: 52 us against 40 us; 256 MiB: 95 against 80).
+constexpr uint32_t kDirectCopyMaxSeg = 8;
+struct DirectCopyArgs {
+    const void* src[kDirectCopyMaxSeg];
+    void* dst[kDirectCopyMaxSeg];   // the segment's place in the destination
+    uint64_t nVec;                  // 16-byte vectors per segment
+};
+
+__global__ __launch_bounds__(64) void DirectCopyKernel(const DirectCopyArgs a)
+{
+    const uint32_t j = blockIdx.y;
+    const uint64_t u = static_cast<uint64_t>(blockIdx.x) * 64 + threadIdx.x;
+    if (u >= a.nVec) {
+        return;
+    }
+    const U32x4 v = LoadVec<U32x4>(static_cast<const U32x4*>(a.src[j]) + u);
+    StoreVec<U32x4>(v, static_cast<U32x4*>(a.dst[j]) + u);
+}
+
 constexpr int kMaxDevices = 64;
 std::mutex g_scratchMu;
 uint8_t* g_scratchPtr[kMaxDevices] = {};
@@ -508,6 +531,36 @@ hipError_t LaunchBcastCopy(const BcastCopyArgs& in, uint32_t tileBytes, hipStrea
         }
     }
     const uint32_t mode = !congruent ? COPY_GENERAL : ((misfit & 15u) == 0 ? COPY_ALIGNED : COPY_CONGRUENT);
+    // One destination, up to eight equally long aligned segments: the kernel that needs nothing but its arguments.
+    // HCCL_AMD_COPY_DIRECT=0 keeps the general kernel (read once per process).
+    static const bool directEnv = getenv("HCCL_AMD_COPY_DIRECT") == nullptr || atoi(getenv("HCCL_AMD_COPY_DIRECT")) != 0;
+    if (directEnv && tileBytes == 0 && mode == COPY_ALIGNED && a.nDst == 1) {
+        DirectCopyArgs d{};
+        uint32_t nSeg = 0;
+        uint64_t len = 0;
+        bool fits = true;
+        for (uint32_t j = 0; j < a.nSeg && fits; ++j) {
+            if (a.len[j] == 0) {
+                continue;
+            }
+            fits = nSeg < kDirectCopyMaxSeg && (len == 0 || a.len[j] == len) && ((dst0 + a.dstOff[j]) & 127u) == 0;
+            if (fits) {
+                len = a.len[j];
+                d.src[nSeg] = a.src[j];
+                d.dst[nSeg] = reinterpret_cast<void*>(dst0 + a.dstOff[j]);
+                ++nSeg;
+            }
+        }
+        if (fits && nSeg == 0) {
+            return hipSuccess;   // nothing but empty segments
+        }
+        const uint64_t tiles = ((len >> 4) + 63) / 64;
+        if (fits && tiles <= 0x7FFFFFFFull) {
+            d.nVec = len >> 4;
+            hipLaunchKernelGGL(DirectCopyKernel, dim3(static_cast<uint32_t>(tiles), nSeg), dim3(64), 0, stream, d);
+            return hipGetLastError();
+        }
+    }
     if (tileBytes == 0) {
         // One wavefront per tile, except where lanes realign their source for several destinations: there the
         // larger workgroup measured 1-2 % faster.

@@ -366,3 +366,35 @@ def test_one_to_many_copies_as_gather_and_fan_out(monkeypatch, n):
             assert np.array_equal(to_host(recvs[r], np.uint8), vwant[r]), ("all_gather_v", r)
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("n", [2, 8, 12])
+def test_gather_step_as_the_copy_launched_from_its_arguments(monkeypatch, n):
+    """One destination and up to eight equally long segments on 16-byte boundaries whose places in the destination
+    start on 128-byte lines go through the copy kernel that finds everything in its arguments: the gather step of a
+    two-kernel AllGather (128-byte multiples per rank; more than eight ranks and other lengths keep the general
+    kernel) and the root's copy of a two-kernel Broadcast, lengths from one vector to many tiles and a tile and a
+    half."""
+    w = world_with_form(monkeypatch, n, "two_kernels")
+    try:
+        rng = np.random.default_rng(1300 + n)
+        cases = [(nbytes, 0) for nbytes in (128, 16, 1_024, 1_536, 4_096 + 128, 65_536 + 16, 1_000_000 - 1_000_000 % 128)]
+        # destinations on a 16-byte boundary that is no 128-byte line: everything aligned, yet the general kernel's
+        cases += [(nbytes, 48) for nbytes in (16, 128, 4_096 + 128)]
+        for nbytes, pad in cases:
+            ins = [rand_bytes(rng, nbytes) for _ in range(n)]
+            want = [np.zeros(n * nbytes, dtype=np.uint8) for _ in range(n)]
+            assert oracle.all_gather(ins, want, nbytes, int(DT.UINT8)) == 0
+            sends = [to_dev(x, 0) for x in ins]
+            recvs = [dev_zeros(n * nbytes, pad) for _ in range(n)]
+            w.all_gather(sends, recvs, nbytes, DT.UINT8)
+            for r in range(n):
+                assert np.array_equal(to_host(recvs[r], np.uint8), want[r]), ("all_gather", nbytes, pad, r)
+            bufs = [to_dev(rand_bytes(rng, nbytes), pad) for _ in range(n)]
+            root = int(rng.integers(0, n))
+            src = to_host(bufs[root], np.uint8)
+            w.broadcast(bufs, nbytes, DT.UINT8, root)
+            for r in range(n):
+                assert np.array_equal(to_host(bufs[r], np.uint8), src), ("broadcast", root, nbytes, r)
+    finally:
+        w.close()
