@@ -260,7 +260,13 @@ inline bool FanOutStreamLoad(uint32_t nDst, bool severalPieces) { return nDst <=
 // Where the forms cross, per destination: 16 ranks 16 MiB 0.74 / 0.60, 32 MiB 0.82 / 0.59; 12 ranks 12 MiB 0.66 / 0.66,
 // 24 MiB 0.68 / 0.65, 36 MiB 0.74 / 0.65; 10 ranks 20 MiB 0.69 / 0.67, 30 MiB 0.72 / 0.69, 40 MiB 0.77 / 0.72; 8 ranks
 // 16 MiB 0.65 / 0.66, 24 MiB 0.70 / 0.69, 32 MiB 0.71 / 0.69, 40 MiB 0.73 / 0.71; 7 ranks 21-42 MiB 0.65-0.69 / 0.69-0.72,
-// 49 MiB 0.72 / 0.71.  HCCL_AMD_COPY_TWO_KERNELS = 0 / 1 forces a form.
+// 49 MiB 0.72 / 0.71.  Since the gather step runs through the copy kernel that is launched from its arguments alone
+// (a quarter faster), with aligned operands: AllGather of 16 x 16 MiB 0.85 / 0.68, 12 x 8 MiB 0.81 / 0.68, 8 x 8 MiB
+// 0.81 / 0.72, 8 x 24 MiB 0.85 / 0.70, 7 x 8 MiB 0.79 / 0.74, 7 x 32 MiB 0.84 / 0.74, 6 x 16 MiB 0.80 / 0.76, 6 x 32 MiB
+// 0.82 / 0.74, 5 x 16 MiB 0.75 / 0.77, 5 x 64 MiB 0.77 / 0.76, 4 x 64 MiB 0.76 / 0.77; Broadcast to 15 ranks of 16 / 64 MiB
+// 0.76 / 0.64, 0.86 / 0.66, to 6 ranks of 32 / 64 / 128 MiB 0.70 / 0.72, 0.75 / 0.73, 0.82 / 0.73, to 5 ranks of 64 /
+// 128 MiB 0.74 / 0.76, 0.78 / 0.78, to 4 ranks 0.71-0.73 / 0.76-0.78: six destinations now from 64 MiB.
+// HCCL_AMD_COPY_TWO_KERNELS = 0 / 1 forces a form.
 inline bool GatherThenFanOut(uint32_t nDst, uint64_t bytes, bool congruent)
 {
     if (nDst >= 14) {
@@ -269,7 +275,7 @@ inline bool GatherThenFanOut(uint32_t nDst, uint64_t bytes, bool congruent)
     if (nDst >= 8) {
         return bytes >= 24 * kMiB;
     }
-    return (nDst == 7 && bytes >= 48 * kMiB) || (nDst == 6 && congruent && bytes >= 128 * kMiB);
+    return (nDst == 7 && bytes >= 48 * kMiB) || (nDst == 6 && congruent && bytes >= 64 * kMiB);
 }
 
 }  // namespace policy
