@@ -1108,7 +1108,8 @@ __global__ __launch_bounds__(64 * kDirectFoldMaxWaves) void DirectFoldTwoTileKer
 #pragma unroll
     for (int i = 0; i < kLeaves; ++i) {
         if (static_cast<uint32_t>(i) < nSrc) {
-            const HCCL_AMD_GLOBAL U32x4* const p = reinterpret_cast<const HCCL_AMD_GLOBAL U32x4*>(leaf[i]) + first + threadIdx.x;
+            const HCCL_AMD_GLOBAL U32x4* const p =
+                reinterpret_cast<const HCCL_AMD_GLOBAL U32x4*>(leaf[i]) + first + threadIdx.x;
             raw[0][i] = __builtin_nontemporal_load(p);
             raw[1][i] = __builtin_nontemporal_load(p + lanes);
         }
@@ -1208,9 +1209,9 @@ __global__ __launch_bounds__(64 * kDirectFoldMaxWaves) void DirectFoldWideKernel
 
 // The same for exactly eight leaves, eight destinations, eight wavefronts per workgroup and a vector count that
 // fills every workgroup (a multiple of 512, or of 1024 with K = 2 tiles per wavefront; no elements behind the last
-// vector): straight-line code without a count or bounds check.  At a few MiB per rank every wavefront of the launch is resident at once and shares its SIMD's
-// issue slots with three others, so the instructions between a wavefront's start and its first load, and between
-// the barrier and its stores, are latency that nothing hides.
+// vector): straight-line code without a count or bounds check.  At a few MiB per rank every wavefront of the launch
+// is resident at once and shares its SIMD's issue slots with three others, so the instructions between a
+// wavefront's start and its first load, and between the barrier and its stores, are latency that nothing hides.
 template <class E, int K>
 __global__ __launch_bounds__(64 * 8) void DirectFoldExactKernel(const DirectFoldArgs a)
 {
