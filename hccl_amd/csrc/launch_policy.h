@@ -265,15 +265,19 @@ inline bool FanOutStreamLoad(uint32_t nDst, bool severalPieces) { return nDst <=
 // 0.81 / 0.72, 8 x 24 MiB 0.85 / 0.70, 7 x 8 MiB 0.79 / 0.74, 7 x 32 MiB 0.84 / 0.74, 6 x 16 MiB 0.80 / 0.76, 6 x 32 MiB
 // 0.82 / 0.74, 5 x 16 MiB 0.75 / 0.77, 5 x 64 MiB 0.77 / 0.76, 4 x 64 MiB 0.76 / 0.77; Broadcast to 15 ranks of 16 / 64 MiB
 // 0.76 / 0.64, 0.86 / 0.66, to 6 ranks of 32 / 64 / 128 MiB 0.70 / 0.72, 0.75 / 0.73, 0.82 / 0.73, to 5 ranks of 64 /
-// 128 MiB 0.74 / 0.76, 0.78 / 0.78, to 4 ranks 0.71-0.73 / 0.76-0.78: six destinations now from 64 MiB.
+// 128 MiB 0.74 / 0.76, 0.78 / 0.78, to 4 ranks 0.71-0.73 / 0.76-0.78: six destinations now from 64 MiB.  And per
+// destination: 8 ranks 8 MiB 0.61 / 0.67, 16 MiB 0.69 / 0.66, 24 MiB 0.74 / 0.67; 10 ranks 10 MiB 0.63 / 0.65, 20 MiB
+// 0.70 / 0.67; 12 ranks 12 MiB 0.67 / 0.66; Broadcast to 8 ranks of 8 / 16 / 24 MiB 0.59 / 0.62, 0.70 / 0.67, 0.74 / 0.67,
+// to 11 ranks 0.63 / 0.64, 0.71 / 0.66, 0.75 / 0.68, to 14 ranks of 4 / 8 / 16 MiB 0.36 / 0.40, 0.70 / 0.66, 0.75 / 0.63:
+// eight to thirteen destinations from 16 MiB, fourteen and more from 8 MiB.
 // HCCL_AMD_COPY_TWO_KERNELS = 0 / 1 forces a form.
 inline bool GatherThenFanOut(uint32_t nDst, uint64_t bytes, bool congruent)
 {
     if (nDst >= 14) {
-        return bytes >= 16 * kMiB;
+        return bytes >= 8 * kMiB;
     }
     if (nDst >= 8) {
-        return bytes >= 24 * kMiB;
+        return bytes >= 16 * kMiB;
     }
     return (nDst == 7 && bytes >= 48 * kMiB) || (nDst == 6 && congruent && bytes >= 64 * kMiB);
 }
